@@ -1,0 +1,179 @@
+/* lten_hip.h — C ABI of the MI355X (gfx950) GEMM hot path for light-tensor ("l-ten").
+ *
+ * Every entry point takes plain pointers and sizes.  Device pointers are raw HIP
+ * device addresses (what lten_hip_alloc returns, or any hipMalloc'ed memory); the
+ * caller owns every buffer and no call retains a pointer after it returns.  All work
+ * is issued on one stream per process (the null stream unless lten_hip_set_stream is
+ * called) and is stream ordered: kernels are asynchronous, lten_hip_copy_from_gpu and
+ * lten_hip_sync are the synchronisation points — the model l-ten's GPU branches
+ * already assume (l-ten/utils.cu:73-94 synchronous copies, default stream elsewhere).
+ *
+ * Return value: 0 on success, non-zero on failure with a message available from
+ * lten_hip_last_error().  A C ABI cannot throw; the C++ glue turns a non-zero status
+ * into LTEN_ERR, which is how l-ten reports failures (l-ten/error.h:78-93).
+ *
+ * Matrices are row-major, as every l-ten tensor is.
+ */
+#ifndef LTEN_HIP_H
+#define LTEN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Layout-identical to l-ten's QuantizationParams (l-ten/math_fns.h:12-16). */
+typedef struct lten_hip_qparams {
+	float   scale;
+	uint8_t zero_point;
+} lten_hip_qparams;
+
+/* ------------------------------------------------------------------ context / errors */
+
+/* Replaces the lazy cuBLAS/cuDNN handle creation of CUDA_globlas (l-ten/globals.h:89-123).
+ * Selects `device`, checks that it is a gfx950 part. Idempotent. */
+int lten_hip_init(int device);
+/* Message of the last failing call on this thread ("" if none). */
+const char* lten_hip_last_error(void);
+/* Replaces GetDevice (l-ten/utils.h:41, l-ten/utils.cu:110-116). */
+int lten_hip_get_device(int* device);
+/* Routes all later work to `hip_stream` (a hipStream_t; NULL = the null stream).
+ * No counterpart in l-ten, which only ever uses the default stream. */
+int lten_hip_set_stream(void* hip_stream);
+/* Blocks until the stream is idle. l-ten's equivalent is the implicit sync of cudaMemcpy. */
+int lten_hip_sync(void);
+
+/* ------------------------------------------------------------------------- memory */
+
+/* Replaces AllocateMemoryOnGPU / gpu_alloc (l-ten/utils.h:29,33; l-ten/utils.cu:8-28,30-58). */
+int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory);
+/* Replaces FreeMemoryOnGPU / gpu_free (l-ten/utils.h:30,35; l-ten/utils.cu:60-71). */
+int lten_hip_free(void* device_ptr);
+/* Replaces ZeroMemoryOnGPU (l-ten/utils.h:34; l-ten/utils.cu:49-52). */
+int lten_hip_zero(void* device_ptr, size_t size);
+/* Replace CopyDataToGPU / CopyDataFromGPU / GPUToGPUCopy (l-ten/utils.h:36-38; l-ten/utils.cu:73-108).
+ * Host <-> device copies return after the data has arrived, as cudaMemcpy does. */
+int lten_hip_copy_to_gpu(void* device_dst, const void* host_src, size_t size);
+int lten_hip_copy_from_gpu(void* host_dst, const void* device_src, size_t size);
+int lten_hip_copy_gpu_to_gpu(void* device_dst, const void* device_src, size_t size);
+
+/* Replace gpu_fill<T> (l-ten/math_fns.h:180-181; l-ten/math_fns.cu:729-775). */
+int lten_hip_fill_f32(float* device_ptr, uint64_t count, float value);
+int lten_hip_fill_i32(int32_t* device_ptr, uint64_t count, int32_t value);
+int lten_hip_fill_u8(uint8_t* device_ptr, uint64_t count, uint8_t value);
+
+/* ----------------------------------------------------------------------- fp32 GEMM */
+
+/* C[M x N] = alpha * op(A) * op(B) + beta * C, row-major with leading dimensions.
+ * The contract of cpu_gemm<float> (l-ten/math_fns.h:18-19, l-ten/math_fns.cpp:1258) plus
+ * lda/ldb/ldc; replaces every cublasSgemm site of l-ten's GPU branches
+ * (l-ten/fully_connected.cpp:150,165; l-ten/conv2d.cpp:169; l-ten/md_array_cuda.h:513;
+ * l-ten/backprop.cpp:562,580,2003,2024,2228,2252,2267).  beta == 0 overwrites C
+ * (NaN/Inf in C are not propagated); A and B are never modified.  The K == 1
+ * (bias rank-1 update) and M == 1 (bias-gradient column sum) shapes those sites use
+ * are served by dedicated kernels. */
+int lten_hip_sgemm(int trans_a, int trans_b, uint64_t M, uint64_t N, uint64_t K, float alpha,
+                   const float* A, uint64_t lda, const float* B, uint64_t ldb, float beta,
+                   float* C, uint64_t ldc);
+
+/* `batch` GEMMs with element strides between consecutive problems; a stride of 0
+ * re-uses (broadcasts) that operand.  Serves the per-leading-index loop of
+ * CUDA_MultiDimArray::matmul (l-ten/md_array_cuda.h:450-525) and matmul_backward
+ * (l-ten/backprop.cpp:533-585) in one launch.  With stride_c == 0 and beta == 1 the
+ * batch accumulates into one C (the broadcast-operand gradient); that case is
+ * serialised internally so the sum is deterministic. */
+int lten_hip_sgemm_strided_batched(int trans_a, int trans_b, uint64_t M, uint64_t N, uint64_t K, float alpha,
+                                   const float* A, uint64_t lda, int64_t stride_a,
+                                   const float* B, uint64_t ldb, int64_t stride_b, float beta,
+                                   float* C, uint64_t ldc, int64_t stride_c, uint64_t batch);
+
+/* FullyConnected forward in one launch: Y[M x out] = X[M x in] * W[out x in]^T (+ bias[out]),
+ * i.e. the two cublasSgemm calls of l-ten/fully_connected.cpp:150,165 with the bias
+ * rank-1 update folded into the epilogue.  bias may be NULL. */
+int lten_hip_fc_forward_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X,
+                            const float* W, const float* bias, float* Y);
+/* The three GEMMs of fc_backward (l-ten/backprop.cpp:2228,2252,2267).  Any output may be
+ * NULL.  dX and dW are overwritten (beta = 0); db accumulates (beta = 1), as in l-ten. */
+int lten_hip_fc_backward_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X,
+                             const float* W, const float* dY, float* dX, float* dW, float* db);
+
+/* ------------------------------------------------------------------ quantized GEMM */
+
+/* GPU counterpart of quantized_matmul (l-ten/math_fns.h:104, l-ten/math_fns.cpp:1311-1478),
+ * same argument list: C_u8[M x N] from A_u8, B_u8 (all four transpose modes), qparams[3] =
+ * {A, B, C} (host memory), optional int32 bias[N] (device), int32 workspace[M + N]
+ * (device scratch for the zero-point row/column terms; contents unspecified on return).
+ * alpha != 1 or beta != 0 fail, as in l-ten (:1331-1334).  Outputs are bit-exact with the
+ * CPU function wherever that function does not overflow int32 (K * 255^2 < 2^31) and
+ * |real_multiplier * acc + zero_point| stays representable as a float. */
+int lten_hip_quantized_matmul(int transpose_a, int transpose_b, uint64_t M, uint64_t N, uint64_t K,
+                              uint8_t alpha, const uint8_t* A, const uint8_t* B, uint8_t beta, uint8_t* C,
+                              const lten_hip_qparams* qparams, const int32_t* bias, int32_t* workspace);
+/* Same computation, stopping before the requantize: acc[M x N] receives the corrected
+ * int32 `element` of l-ten/math_fns.cpp:1469-1473.  For parity checks. */
+int lten_hip_quantized_matmul_acc(int transpose_a, int transpose_b, uint64_t M, uint64_t N, uint64_t K,
+                                  const uint8_t* A, const uint8_t* B, int32_t* acc,
+                                  const lten_hip_qparams* qparams, const int32_t* bias, int32_t* workspace);
+/* FullyConnected_q::forward's loop over leading dims (l-ten/fully_connected.cpp:373-396) as
+ * one call: `batch` independent [M x in] inputs against one W[out x in]. workspace holds
+ * batch * M + out ints. */
+int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features,
+                         const uint8_t* X, const uint8_t* W, const int32_t* bias,
+                         const lten_hip_qparams* qparams_in_wt_out, uint8_t* Y, int32_t* workspace);
+
+/* ------------------------------------------------------------------ im2col / conv */
+
+/* Replace im2col_gpu / col2im_gpu (l-ten/im_col.h:60-73, l-ten/im_col.cu:98-118,164-184).
+ * col is [C*kh*kw, Hout*Wout]; col2im overwrites im with the gathered sums, as the
+ * CUDA kernel does (l-ten/im_col.cu:123-162). */
+int lten_hip_im2col_f32(const float* im, int channels, int height, int width, int kernel_h, int kernel_w,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                        float* col);
+int lten_hip_im2col_u8(const uint8_t* im, int channels, int height, int width, int kernel_h, int kernel_w,
+                       int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                       uint8_t* col);
+int lten_hip_col2im_f32(const float* col, int channels, int height, int width, int kernel_h, int kernel_w,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                        float* im);
+
+/* Conv2d::forward's per-image im2col + cublasSgemm loop (l-ten/conv2d.cpp:164-171) as one
+ * implicit-GEMM launch over the whole batch; no col buffer is materialised.
+ * x[N,Cin,H,W], w[Cout,Cin*kh*kw], y[N,Cout,Hout,Wout]; bias[Cout] may be NULL
+ * (l-ten adds it afterwards as a broadcast tensor add, l-ten/conv2d.cpp:189-192). */
+int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                                int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                                const float* x, const float* w, const float* bias, float* y);
+/* conv2_backward's weight branch (l-ten/backprop.cpp:1941-1954, the CPU semantics: the sum
+ * over all images; the CUDA branch at :1989-2005 keeps only the last image and is not
+ * followed).  dw[Cout, Cin*kh*kw] is overwritten.  workspace: device scratch of at least
+ * lten_hip_conv2d_wgrad_workspace_bytes(...) bytes. */
+int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                              int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                              const float* x, const float* dy, float* dw, void* workspace);
+uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                                               int kernel_h, int kernel_w, int pad_h, int pad_w,
+                                               int stride_h, int stride_w);
+
+/* ----------------------------------------------------------------------- measurement */
+
+/* HIP events on the library's stream; no counterpart in l-ten (its benchmarks use
+ * steady_clock around synchronous calls). */
+int lten_hip_event_create(void** event);
+int lten_hip_event_record(void* event);
+int lten_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* synchronises on `stop` */
+int lten_hip_event_destroy(void* event);
+
+/* Kernel-selection override for tests and tuning sweeps; 0 restores the built-in heuristic.
+ * Options: "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant".  No counterpart in l-ten. */
+int lten_hip_set_option(const char* name, int value);
+
+/* Name of the kernel variant the last GEMM-type call on this thread dispatched to
+ * (e.g. "qgemm_nt_256x256x64"); for reports and tests. */
+const char* lten_hip_last_kernel(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LTEN_HIP_H */

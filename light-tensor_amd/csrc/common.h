@@ -1,0 +1,46 @@
+// Shared plumbing of the C-ABI library: error reporting, the per-process stream and
+// small launch helpers.  Everything here is host side.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "../../include/lten_hip.h"
+
+namespace lten_hip {
+
+// Thread-local message behind lten_hip_last_error(); l-ten itself prints and throws
+// (l-ten/error.h:78-93), which a C ABI cannot do.
+void set_error(const char* fmt, ...);
+void set_kernel_name(const char* name);
+hipStream_t stream();
+
+// Tuning / test switches behind lten_hip_set_option.
+enum Option { OPT_QGEMM_TILE = 0, OPT_SGEMM_TILE, OPT_QSKINNY, OPT_CONV_VARIANT, OPT_COUNT };
+int get_option(Option o);
+
+inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
+
+}  // namespace lten_hip
+
+#define LTEN_HIP_CHECK(expr)                                                                     \
+	do {                                                                                     \
+		hipError_t e_ = (expr);                                                          \
+		if (e_ != hipSuccess) {                                                          \
+			lten_hip::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, __LINE__); \
+			return 1;                                                                \
+		}                                                                                \
+	} while (0)
+
+#define LTEN_HIP_REQUIRE(cond, ...)                                                              \
+	do {                                                                                     \
+		if (!(cond)) {                                                                   \
+			lten_hip::set_error(__VA_ARGS__);                                        \
+			return 2;                                                                \
+		}                                                                                \
+	} while (0)
+
+// After a kernel launch: surface launch-configuration errors immediately.
+#define LTEN_HIP_LAUNCH_CHECK() LTEN_HIP_CHECK(hipGetLastError())

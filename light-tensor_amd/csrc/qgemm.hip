@@ -1,0 +1,484 @@
+// int8 GEMM for gfx950: the GPU counterpart of l-ten's quantized_matmul
+// (l-ten/math_fns.cpp:1311-1478), which has no GPU implementation in l-ten
+// (l-ten/fully_connected.cpp:399).
+//
+// Arithmetic.  l-ten multiplies two uint8 matrices with uint8 zero points.  The matrix
+// cores multiply signed bytes, so every operand byte is mapped to a' = a XOR 0x80
+// (= a - 128 as int8) on its way into LDS, and the exact integer identity
+//
+//   sum_k (A-zpA)(B-zpB) = sum_k a'b' + (128-zpB) * SA_m + (128-zpA) * SB_n + K (zpA zpB - 16384)
+//
+// (SA_m, SB_n = plain byte sums of row m of A / row n of B) restores l-ten's value
+// `element` of :1469 in the epilogue, which then requantizes exactly as :1474 does.
+// All integer arithmetic wraps modulo 2^32, which equals l-ten's int arithmetic wherever
+// that does not overflow.
+//
+// Tiling.  One workgroup computes a BM x BN tile of C with WM x WN wavefronts; each
+// wavefront owns a (BM/WM) x (BN/WN) sub-tile built from 32x32x32 int8 MFMA blocks.  The
+// MFMA "A" operand is fed from the weight tile and the "B" operand from the activation
+// tile, so that the four consecutive accumulator registers of a lane are four consecutive
+// output columns n and are stored as one packed dword.  A and B tiles are staged through
+// LDS in two buffers (global -> registers -> XOR -> LDS while the MFMAs of the current
+// buffer run), rows of BK bytes with a 16-byte-chunk XOR swizzle that keeps the
+// ds_read_b128 operand fetches bank-conflict free.
+#include "common.h"
+
+namespace lten_hip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+enum QOut { Q_OUT_U8_FAST = 0, Q_OUT_U8_EXACT = 1, Q_OUT_ACC = 2 };
+
+struct QProblem {
+	const uint8_t* A;  // element (m, k) at A[m * a_rs + k * a_ks]
+	const uint8_t* B;  // element (n, k) at B[n * b_rs + k * b_ks]
+	void* C;           // uint8 [M x N] or int32 [M x N], row-major, ld = N
+	int64_t a_rs, a_ks, b_rs, b_ks;
+	int M, N, K;
+	const int32_t* rterm;  // [M] (128 - zpB) * SA_m, or null
+	const int32_t* cterm;  // [N] (128 - zpA) * SB_n + bias_n, or null
+	int32_t konst;         // K (zpA zpB - 16384)
+	float mult;            // real_multiplier
+	float zp_c;            // (float) output zero point
+	int vec_ok;            // operand bases and row strides are multiples of 16 bytes
+};
+
+// 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).
+// Chosen so that any aligned group of 8 or of 16 consecutive rows, read at one logical
+// chunk, touches every LDS bank group once (both for 32 and for 64 four-byte banks).
+template <int CPR>
+__device__ __forceinline__ int swz(int row)
+{
+	if (CPR == 2) return ((row >> 2) ^ (row >> 3)) & 1;
+	if (CPR == 4) return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1);
+	if (CPR == 8) return ((row ^ (row >> 3)) & 1) | (row & 6);
+	return 0;
+}
+
+__device__ __forceinline__ v4i flip_sign_bits(v4i v)
+{
+	v.x ^= 0x80808080;
+	v.y ^= 0x80808080;
+	v.z ^= 0x80808080;
+	v.w ^= 0x80808080;
+	return v;
+}
+
+// One 16-byte chunk of an operand tile, raw bytes (before the XOR), as four dwords.
+// Out-of-range bytes read as 0x80, which becomes 0 after the XOR.
+template <bool GUARD>
+__device__ __forceinline__ v4i load_chunk(const uint8_t* base, int64_t rs, int64_t ks, int row, int rows, int k, int K, int vec_ok)
+{
+	if (!GUARD) {
+		return *reinterpret_cast<const v4i*>(base + (int64_t)row * rs + k);
+	} else {
+		if (ks == 1 && vec_ok && row < rows && k + 16 <= K)
+			return *reinterpret_cast<const v4i*>(base + (int64_t)row * rs + k);
+		v4i v;
+		int* vp = reinterpret_cast<int*>(&v);
+#pragma unroll
+		for (int d = 0; d < 4; d++) {
+			unsigned w = 0;
+#pragma unroll
+			for (int b = 0; b < 4; b++) {
+				int kk = k + d * 4 + b;
+				unsigned byte = 0x80u;
+				if (row < rows && kk < K) byte = base[(int64_t)row * rs + (int64_t)kk * ks];
+				w |= byte << (8 * b);
+			}
+			vp[d] = (int)w;
+		}
+		return v;
+	}
+}
+
+// Exact image of l-ten/math_fns.cpp:1474 for one accumulator.
+template <int OUT>
+__device__ __forceinline__ unsigned requant(int acc, float mult, float zp)
+{
+	// Two separately rounded operations: a fused multiply-add rounds once and differs in the last bit.
+#pragma clang fp contract(off)
+	float prod = (float)acc * mult;
+	float s = prod + zp;
+	if (OUT == Q_OUT_U8_EXACT) {
+		// x86 cvttss2si: NaN and anything outside [-2^31, 2^31) give 0x80000000.
+		int i = (s >= -2147483648.0f && s < 2147483648.0f) ? (int)s : (int)0x80000000;
+		return (unsigned)i & 0xFFu;
+	}
+	return (unsigned)(int)s & 0xFFu;  // caller guarantees |s| < 2^31
+}
+
+template <int BM, int BN, int BK, int WM, int WN, bool GUARD, int OUT>
+__global__ __launch_bounds__(WM* WN * 64) void qgemm_kernel(QProblem p)
+{
+	constexpr int T = WM * WN * 64;
+	constexpr int CPR = BK / 16;  // 16-byte chunks per tile row
+	constexpr int TM = BM / WM, TN = BN / WN;
+	constexpr int FM = TM / 32, FN = TN / 32;
+	constexpr int A_CHUNKS = BM * CPR, B_CHUNKS = BN * CPR;
+	constexpr int A_PER_T = (A_CHUNKS + T - 1) / T, B_PER_T = (B_CHUNKS + T - 1) / T;
+	constexpr int STAGE = (BM + BN) * BK;
+	static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA block");
+	static_assert(BK % 32 == 0, "BK must hold whole MFMA k-slices");
+
+	__shared__ __attribute__((aligned(16))) uint8_t smem[2 * STAGE];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = tid >> 6;
+	const int wm = wave / WN, wn = wave % WN;
+
+	// Workgroup -> tile.  Consecutive workgroup ids go round-robin to the 8 XCDs, each
+	// with its own L2; give every XCD one compact block of tiles so that the A rows and
+	// B rows it streams are shared by its CUs.
+	const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+	int bid = blockIdx.x;
+	int tm, tn;
+	{
+		const int nb = tiles_m * tiles_n;
+		int lid = bid;
+		if ((nb & 7) == 0) lid = (bid & 7) * (nb >> 3) + (bid >> 3);
+		constexpr int GM = 4, GN = 8;
+		if (tiles_m % GM == 0 && tiles_n % GN == 0) {
+			int group = lid / (GM * GN), within = lid % (GM * GN);
+			int groups_n = tiles_n / GN;
+			tm = (group / groups_n) * GM + within / GN;
+			tn = (group % groups_n) * GN + within % GN;
+		} else {
+			tm = lid / tiles_n;
+			tn = lid % tiles_n;
+		}
+	}
+	const int m0 = tm * BM, n0 = tn * BN;
+
+	const bool a_kmajor = (p.a_ks == 1), b_kmajor = (p.b_ks == 1);
+
+	v4i stage_a[A_PER_T], stage_b[B_PER_T];
+
+	auto load_global = [&](int k0) {
+#pragma unroll
+		for (int i = 0; i < A_PER_T; i++) {
+			int c = tid + i * T;
+			if (A_CHUNKS % T != 0 && c >= A_CHUNKS) break;
+			// K-contiguous operands: neighbouring threads take neighbouring chunks of a row.
+			// K-strided operands: neighbouring threads take neighbouring rows.
+			int row = (!GUARD || a_kmajor) ? c / CPR : c % BM;
+			int kc = (!GUARD || a_kmajor) ? c % CPR : c / BM;
+			stage_a[i] = load_chunk<GUARD>(p.A, p.a_rs, p.a_ks, m0 + row, p.M, k0 + kc * 16, p.K, p.vec_ok);
+		}
+#pragma unroll
+		for (int i = 0; i < B_PER_T; i++) {
+			int c = tid + i * T;
+			if (B_CHUNKS % T != 0 && c >= B_CHUNKS) break;
+			int row = (!GUARD || b_kmajor) ? c / CPR : c % BN;
+			int kc = (!GUARD || b_kmajor) ? c % CPR : c / BN;
+			stage_b[i] = load_chunk<GUARD>(p.B, p.b_rs, p.b_ks, n0 + row, p.N, k0 + kc * 16, p.K, p.vec_ok);
+		}
+	};
+
+	auto store_lds = [&](int buf) {
+		uint8_t* sa = smem + buf * STAGE;
+		uint8_t* sb = sa + BM * BK;
+#pragma unroll
+		for (int i = 0; i < A_PER_T; i++) {
+			int c = tid + i * T;
+			if (A_CHUNKS % T != 0 && c >= A_CHUNKS) break;
+			int row = (!GUARD || a_kmajor) ? c / CPR : c % BM;
+			int kc = (!GUARD || a_kmajor) ? c % CPR : c / BM;
+			*reinterpret_cast<v4i*>(sa + row * BK + ((kc ^ swz<CPR>(row)) << 4)) = flip_sign_bits(stage_a[i]);
+		}
+#pragma unroll
+		for (int i = 0; i < B_PER_T; i++) {
+			int c = tid + i * T;
+			if (B_CHUNKS % T != 0 && c >= B_CHUNKS) break;
+			int row = (!GUARD || b_kmajor) ? c / CPR : c % BN;
+			int kc = (!GUARD || b_kmajor) ? c % CPR : c / BN;
+			*reinterpret_cast<v4i*>(sb + row * BK + ((kc ^ swz<CPR>(row)) << 4)) = flip_sign_bits(stage_b[i]);
+		}
+	};
+
+	v16i acc[FN][FM];
+#pragma unroll
+	for (int i = 0; i < FN; i++)
+#pragma unroll
+		for (int j = 0; j < FM; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+
+	const int KT = (p.K + BK - 1) / BK;
+	const int lrow = lane & 31;  // row of the 32-row MFMA operand block this lane feeds
+	const int lgrp = lane >> 5;  // which 16-byte half of the 32-byte k-slice
+
+	load_global(0);
+	store_lds(0);
+	__syncthreads();
+
+	for (int kt = 0; kt < KT; kt++) {
+		const int cur = kt & 1;
+		if (kt + 1 < KT) load_global((kt + 1) * BK);
+
+		const uint8_t* sa = smem + cur * STAGE;
+		const uint8_t* sb = sa + BM * BK;
+#pragma unroll
+		for (int s = 0; s < BK / 32; s++) {
+			v4i fw[FN], fx[FM];
+			const int kc = s * 2 + lgrp;
+#pragma unroll
+			for (int i = 0; i < FN; i++) {
+				int row = wn * TN + i * 32 + lrow;
+				fw[i] = *reinterpret_cast<const v4i*>(sb + row * BK + ((kc ^ swz<CPR>(row)) << 4));
+			}
+#pragma unroll
+			for (int j = 0; j < FM; j++) {
+				int row = wm * TM + j * 32 + lrow;
+				fx[j] = *reinterpret_cast<const v4i*>(sa + row * BK + ((kc ^ swz<CPR>(row)) << 4));
+			}
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int j = 0; j < FM; j++)
+					acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[i], fx[j], acc[i][j], 0, 0, 0);
+		}
+
+		if (kt + 1 < KT) store_lds(cur ^ 1);
+		__syncthreads();
+	}
+
+	// Epilogue.  Lane (lrow, lgrp) of block (i, j) holds, in register 4q + e, the output
+	// at m = m0 + wm*TM + j*32 + lrow, n = n0 + wn*TN + i*32 + 8q + 4*lgrp + e.
+#pragma unroll
+	for (int j = 0; j < FM; j++) {
+		const int m = m0 + wm * TM + j * 32 + lrow;
+		if (GUARD && m >= p.M) continue;
+		const int rt = (p.rterm ? p.rterm[m] : 0) + p.konst;
+#pragma unroll
+		for (int i = 0; i < FN; i++) {
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				const int n = n0 + wn * TN + i * 32 + q * 8 + lgrp * 4;
+				int v[4];
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					v[e] = acc[i][j][q * 4 + e] + rt;
+					if (p.cterm && (!GUARD || n + e < p.N)) v[e] += p.cterm[n + e];
+				}
+				if (OUT == Q_OUT_ACC) {
+					int* out = static_cast<int*>(p.C) + (int64_t)m * p.N + n;
+					if (!GUARD) {
+						*reinterpret_cast<v4i*>(out) = v4i{ v[0], v[1], v[2], v[3] };
+					} else {
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							if (n + e < p.N) out[e] = v[e];
+					}
+				} else {
+					unsigned b0 = requant<OUT>(v[0], p.mult, p.zp_c);
+					unsigned b1 = requant<OUT>(v[1], p.mult, p.zp_c);
+					unsigned b2 = requant<OUT>(v[2], p.mult, p.zp_c);
+					unsigned b3 = requant<OUT>(v[3], p.mult, p.zp_c);
+					uint8_t* out = static_cast<uint8_t*>(p.C) + (int64_t)m * p.N + n;
+					if (!GUARD) {
+						*reinterpret_cast<unsigned*>(out) = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+					} else {
+						if (n + 0 < p.N) out[0] = (uint8_t)b0;
+						if (n + 1 < p.N) out[1] = (uint8_t)b1;
+						if (n + 2 < p.N) out[2] = (uint8_t)b2;
+						if (n + 3 < p.N) out[3] = (uint8_t)b3;
+					}
+				}
+			}
+		}
+	}
+}
+
+// Byte sums of the rows of A and of B, turned into the epilogue's correction vectors:
+//   rterm[m] = (128 - zpB) * sum_k A[m,k]
+//   cterm[n] = (128 - zpA) * sum_k B[n,k] + bias[n]
+// One wavefront per row; a zero coefficient skips the read of that matrix.
+__global__ __launch_bounds__(256) void qgemm_terms_kernel(QProblem p, int coef_a, int coef_b, const int32_t* bias,
+                                                          int32_t* rterm, int32_t* cterm)
+{
+	const int lane = threadIdx.x & 63;
+	const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	const bool is_a = wave < p.M;
+	const int64_t row = is_a ? wave : wave - p.M;
+	if (!is_a && row >= p.N) return;
+	const uint8_t* base = is_a ? p.A : p.B;
+	const int64_t rs = is_a ? p.a_rs : p.b_rs, ks = is_a ? p.a_ks : p.b_ks;
+	const int coef = is_a ? coef_a : coef_b;
+	unsigned sum = 0;
+	if (coef != 0) {
+		const uint8_t* r = base + row * rs;
+		if (ks == 1 && p.vec_ok) {
+			int k = lane * 16;
+			for (; k + 16 <= p.K; k += 64 * 16) {
+				v4i v = *reinterpret_cast<const v4i*>(r + k);
+				const unsigned one = 0x01010101u;
+				sum = __builtin_amdgcn_udot4((unsigned)v.x, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.y, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.z, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.w, one, sum, false);
+			}
+			// tail shorter than 16 bytes: the lane whose chunk straddles K finishes it
+			if (k < p.K)
+				for (int kk = k; kk < p.K && kk < k + 16; kk++) sum += r[kk];
+		} else {
+			for (int k = lane; k < p.K; k += 64) sum += r[(int64_t)k * ks];
+		}
+#pragma unroll
+		for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+	}
+	if (lane == 0) {
+		if (is_a)
+			rterm[row] = (int)(sum * (unsigned)coef);
+		else
+			cterm[row] = (int)(sum * (unsigned)coef) + (bias ? bias[row] : 0);
+	}
+}
+
+// -------------------------------------------------------------------------- dispatch
+
+template <int BM, int BN, int BK, int WM, int WN, bool GUARD>
+static int launch_tile(const QProblem& p, int out, const char* name)
+{
+	const unsigned grid = (unsigned)(ceil_div(p.M, BM) * ceil_div(p.N, BN));
+	const dim3 block(WM * WN * 64);
+	set_kernel_name(name);
+	switch (out) {
+	case Q_OUT_U8_FAST:
+		qgemm_kernel<BM, BN, BK, WM, WN, GUARD, Q_OUT_U8_FAST><<<dim3(grid), block, 0, stream()>>>(p);
+		break;
+	case Q_OUT_U8_EXACT:
+		qgemm_kernel<BM, BN, BK, WM, WN, GUARD, Q_OUT_U8_EXACT><<<dim3(grid), block, 0, stream()>>>(p);
+		break;
+	default:
+		qgemm_kernel<BM, BN, BK, WM, WN, GUARD, Q_OUT_ACC><<<dim3(grid), block, 0, stream()>>>(p);
+		break;
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+static int qgemm_dispatch(const QProblem& p, int out)
+{
+	const bool kmajor = p.a_ks == 1 && p.b_ks == 1;
+	const bool c_ok = (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+	auto fits = [&](int bm, int bn, int bk) {
+		return kmajor && p.vec_ok && c_ok && p.M % bm == 0 && p.N % bn == 0 && p.K % bk == 0;
+	};
+	const uint64_t out_elems = (uint64_t)p.M * p.N;
+	int choice = get_option(OPT_QGEMM_TILE);  // 0 = heuristic
+	if (choice == 0) {
+		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
+			choice = 1;
+		else if (fits(128, 128, 64) && out_elems >= 128ull * 128 * 128)
+			choice = 2;
+		else if (out_elems >= 64ull * 64 * 256)
+			choice = 3;
+		else
+			choice = 4;
+	}
+	switch (choice) {
+	case 1:
+		LTEN_HIP_REQUIRE(fits(256, 256, 64), "qgemm: forced 256x256x64 tile does not fit this problem");
+		return launch_tile<256, 256, 64, 2, 2, false>(p, out, "qgemm_nt_256x256x64");
+	case 2:
+		LTEN_HIP_REQUIRE(fits(128, 128, 64), "qgemm: forced 128x128x64 tile does not fit this problem");
+		return launch_tile<128, 128, 64, 2, 2, false>(p, out, "qgemm_nt_128x128x64");
+	case 3:
+		return launch_tile<64, 64, 64, 2, 2, true>(p, out, "qgemm_guard_64x64x64");
+	default:
+		return launch_tile<32, 32, 64, 1, 1, true>(p, out, "qgemm_guard_32x32x64");
+	}
+}
+
+static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A, const uint8_t* B, void* C,
+                     int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace)
+{
+	LTEN_HIP_REQUIRE(qp != nullptr, "quantized_matmul: qparams is null");
+	if (M == 0 || N == 0) return 0;
+	LTEN_HIP_REQUIRE(A && B && C, "quantized_matmul: null matrix pointer");
+	LTEN_HIP_REQUIRE(M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31), "quantized_matmul: dimension too large");
+	// The reference accumulates u8*u8 products in int (l-ten/math_fns.cpp:1442-1467): beyond this K
+	// it overflows and there is nothing defined to match.
+	LTEN_HIP_REQUIRE(K * 65025ull < (1ull << 31), "quantized_matmul: K=%llu overflows the reference's int accumulator",
+	                 (unsigned long long)K);
+
+	const int zpA = qp[0].zero_point, zpB = qp[1].zero_point;
+	QProblem p;
+	p.A = A;
+	p.B = B;
+	p.C = C;
+	// l-ten/math_fns.cpp:1445-1465: A is [M x K] or, transposed, [K x M]; B is [K x N] or, transposed, [N x K].
+	p.a_rs = tA ? 1 : (int64_t)K;
+	p.a_ks = tA ? (int64_t)M : 1;
+	p.b_rs = tB ? (int64_t)K : 1;
+	p.b_ks = tB ? 1 : (int64_t)N;
+	p.M = (int)M;
+	p.N = (int)N;
+	p.K = (int)K;
+	p.konst = (int32_t)((uint32_t)K * (uint32_t)(zpA * zpB - 16384));
+	// l-ten/math_fns.cpp:1436, left to right in fp32
+	volatile float ab = qp[0].scale * qp[1].scale;
+	p.mult = ab / qp[2].scale;
+	p.zp_c = (float)qp[2].zero_point;
+	p.vec_ok = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (K & 15) == 0 &&
+	           p.a_ks == 1 && p.b_ks == 1;
+
+	const int coef_a = 128 - zpB, coef_b = 128 - zpA;
+	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {
+		LTEN_HIP_REQUIRE(workspace != nullptr, "quantized_matmul: workspace is null");
+		p.cterm = workspace;      // N ints, where l-ten keeps row_vector (:1325)
+		p.rterm = workspace + N;  // M ints, where l-ten keeps col_vector (:1326)
+		const unsigned blocks = (unsigned)ceil_div(M + N, 4);
+		qgemm_terms_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(p, coef_a, coef_b, bias, workspace + N, workspace);
+		LTEN_HIP_LAUNCH_CHECK();
+	} else {
+		p.cterm = nullptr;
+		p.rterm = nullptr;
+	}
+
+	int out = Q_OUT_ACC;
+	if (!out_acc) {
+		// |mult * acc + zp| < 2^31 for every int32 acc  <=>  the saturating GPU convert and the
+		// x86 convert agree; otherwise take the epilogue that spells out the x86 behaviour.
+		const float m = p.mult;
+		out = (m == m && (m < 0 ? -m : m) <= 0.99f) ? Q_OUT_U8_FAST : Q_OUT_U8_EXACT;
+	}
+	return qgemm_dispatch(p, out);
+}
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+int lten_hip_quantized_matmul(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, uint8_t alpha, const uint8_t* A,
+                              const uint8_t* B, uint8_t beta, uint8_t* C, const lten_hip_qparams* qparams,
+                              const int32_t* bias, int32_t* workspace)
+{
+	// l-ten/math_fns.cpp:1331-1334
+	LTEN_HIP_REQUIRE(alpha == 1 && beta == 0, "Support for alpha != 1 and beta != 0 not implemented");
+	return qgemm_run(tA, tB, M, N, K, A, B, C, 0, qparams, bias, workspace);
+}
+
+int lten_hip_quantized_matmul_acc(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A,
+                                  const uint8_t* B, int32_t* acc, const lten_hip_qparams* qparams,
+                                  const int32_t* bias, int32_t* workspace)
+{
+	return qgemm_run(tA, tB, M, N, K, A, B, acc, 1, qparams, bias, workspace);
+}
+
+int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features, const uint8_t* X,
+                         const uint8_t* W, const int32_t* bias, const lten_hip_qparams* qparams, uint8_t* Y,
+                         int32_t* workspace)
+{
+	// l-ten/fully_connected.cpp:373-396 runs one quantized_matmul(false, true, M, out, in) per leading
+	// index against the same weights.  Rows of the output are independent of each other, so the loop is
+	// one GEMM with batch * M rows.
+	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, workspace);
+}
+
+}  // extern "C"

@@ -1,0 +1,189 @@
+// Context, memory, fill and event entry points of the C ABI (the HIP counterparts of
+// l-ten/utils.cu and of gpu_fill in l-ten/math_fns.cu).
+#include "common.h"
+
+#include <cstring>
+
+namespace lten_hip {
+
+static thread_local char g_error[512] = "";
+static thread_local char g_kernel[96] = "";
+static hipStream_t g_stream = nullptr;
+static int g_device = -1;
+
+void set_error(const char* fmt, ...)
+{
+	va_list ap;
+	va_start(ap, fmt);
+	vsnprintf(g_error, sizeof(g_error), fmt, ap);
+	va_end(ap);
+}
+
+void set_kernel_name(const char* name)
+{
+	strncpy(g_kernel, name, sizeof(g_kernel) - 1);
+	g_kernel[sizeof(g_kernel) - 1] = 0;
+}
+
+hipStream_t stream() { return g_stream; }
+
+static int g_options[OPT_COUNT] = { 0 };
+static const char* const g_option_names[OPT_COUNT] = { "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant" };
+int get_option(Option o) { return g_options[o]; }
+
+template <typename T>
+__global__ void fill_kernel(T* p, uint64_t n, T v)
+{
+	uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+	uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+	for (; i < n; i += step) p[i] = v;
+}
+
+template <typename T>
+static int fill(T* p, uint64_t n, T v)
+{
+	if (n == 0) return 0;
+	LTEN_HIP_REQUIRE(p != nullptr, "fill: null pointer");
+	uint64_t blocks = ceil_div(n, 256);
+	if (blocks > 4096) blocks = 4096;
+	fill_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream()>>>(p, n, v);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+int lten_hip_init(int device)
+{
+	int count = 0;
+	LTEN_HIP_CHECK(hipGetDeviceCount(&count));
+	LTEN_HIP_REQUIRE(device >= 0 && device < count, "lten_hip_init: device %d out of range (%d devices)", device, count);
+	LTEN_HIP_CHECK(hipSetDevice(device));
+	hipDeviceProp_t prop;
+	LTEN_HIP_CHECK(hipGetDeviceProperties(&prop, device));
+	LTEN_HIP_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
+	                 "lten_hip_init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
+	g_device = device;
+	return 0;
+}
+
+const char* lten_hip_last_error(void) { return g_error; }
+const char* lten_hip_last_kernel(void) { return g_kernel; }
+
+int lten_hip_get_device(int* device)
+{
+	LTEN_HIP_REQUIRE(device != nullptr, "lten_hip_get_device: null pointer");
+	LTEN_HIP_CHECK(hipGetDevice(device));
+	return 0;
+}
+
+int lten_hip_set_stream(void* hip_stream)
+{
+	g_stream = static_cast<hipStream_t>(hip_stream);
+	return 0;
+}
+
+int lten_hip_sync(void)
+{
+	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
+	return 0;
+}
+
+int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
+{
+	LTEN_HIP_REQUIRE(device_ptr != nullptr, "lten_hip_alloc: null pointer");
+	*device_ptr = nullptr;
+	LTEN_HIP_CHECK(hipMalloc(device_ptr, size ? size : 1));
+	if (zero_memory && size) LTEN_HIP_CHECK(hipMemsetAsync(*device_ptr, 0, size, stream()));
+	return 0;
+}
+
+int lten_hip_free(void* device_ptr)
+{
+	if (device_ptr) LTEN_HIP_CHECK(hipFree(device_ptr));
+	return 0;
+}
+
+int lten_hip_zero(void* device_ptr, size_t size)
+{
+	if (size == 0) return 0;
+	LTEN_HIP_REQUIRE(device_ptr != nullptr, "lten_hip_zero: null pointer");
+	// A fill kernel rather than hipMemsetAsync, so that callers may capture this call
+	// into a HIP graph.
+	if ((reinterpret_cast<uintptr_t>(device_ptr) & 3) == 0 && (size & 3) == 0)
+		return fill<int32_t>(static_cast<int32_t*>(device_ptr), size / 4, 0);
+	return fill<uint8_t>(static_cast<uint8_t*>(device_ptr), size, 0);
+}
+
+int lten_hip_copy_to_gpu(void* device_dst, const void* host_src, size_t size)
+{
+	if (size == 0) return 0;
+	LTEN_HIP_CHECK(hipMemcpyAsync(device_dst, host_src, size, hipMemcpyHostToDevice, stream()));
+	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
+	return 0;
+}
+
+int lten_hip_copy_from_gpu(void* host_dst, const void* device_src, size_t size)
+{
+	if (size == 0) return 0;
+	LTEN_HIP_CHECK(hipMemcpyAsync(host_dst, device_src, size, hipMemcpyDeviceToHost, stream()));
+	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
+	return 0;
+}
+
+int lten_hip_copy_gpu_to_gpu(void* device_dst, const void* device_src, size_t size)
+{
+	if (size == 0) return 0;
+	LTEN_HIP_CHECK(hipMemcpyAsync(device_dst, device_src, size, hipMemcpyDeviceToDevice, stream()));
+	return 0;
+}
+
+int lten_hip_fill_f32(float* p, uint64_t n, float v) { return fill<float>(p, n, v); }
+int lten_hip_fill_i32(int32_t* p, uint64_t n, int32_t v) { return fill<int32_t>(p, n, v); }
+int lten_hip_fill_u8(uint8_t* p, uint64_t n, uint8_t v) { return fill<uint8_t>(p, n, v); }
+
+int lten_hip_set_option(const char* name, int value)
+{
+	LTEN_HIP_REQUIRE(name != nullptr, "lten_hip_set_option: null name");
+	for (int i = 0; i < OPT_COUNT; i++)
+		if (strcmp(name, g_option_names[i]) == 0) {
+			g_options[i] = value;
+			return 0;
+		}
+	set_error("lten_hip_set_option: unknown option '%s'", name);
+	return 2;
+}
+
+int lten_hip_event_create(void** event)
+{
+	LTEN_HIP_REQUIRE(event != nullptr, "lten_hip_event_create: null pointer");
+	hipEvent_t e;
+	LTEN_HIP_CHECK(hipEventCreate(&e));
+	*event = e;
+	return 0;
+}
+
+int lten_hip_event_record(void* event)
+{
+	LTEN_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), stream()));
+	return 0;
+}
+
+int lten_hip_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+	LTEN_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+	LTEN_HIP_CHECK(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+	return 0;
+}
+
+int lten_hip_event_destroy(void* event)
+{
+	LTEN_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+	return 0;
+}
+
+}  // extern "C"

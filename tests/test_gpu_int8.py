@@ -1,0 +1,147 @@
+"""GPU parity tests of the int8 path, through the C ABI, against the oracle and the golden vectors.
+Bar: bit-exact int32 accumulators and bit-exact requantized uint8 outputs."""
+import numpy as np
+import pytest
+
+from conftest import exact_acc, golden_path, requant_numpy
+
+pytestmark = pytest.mark.gpu
+
+TILES = {0: "heuristic", 1: "256x256", 2: "128x128", 3: "guard 64x64", 4: "guard 32x32"}
+
+
+def run_case(gpu, ob, A, B, sc, zp, tA=False, tB=True, bias=None, M=None, N=None, K=None, tile=0):
+    gpu.set_option("qgemm_tile", tile)
+    try:
+        Cg, accg = gpu.qgemm_host(A, B, sc, zp, tA=tA, tB=tB, bias=bias, want_acc=True, M=M, N=N, K=K)
+    finally:
+        gpu.set_option("qgemm_tile", 0)
+    Co, acco = ob.quantized_matmul(A, B, sc, zp, tA=tA, tB=tB, bias=bias, M=M, N=N, K=K)
+    assert np.array_equal(accg, acco), "int32 accumulators differ"
+    assert np.array_equal(Cg, Co), "requantized outputs differ"
+    return Cg
+
+
+def test_cfg1_bit_exact_and_golden(gpu, ob, wl):
+    X, W, sc, zp = wl.cfg1()
+    want = np.load(golden_path("cfg1_expected.npz"))["C"]
+    for tile in (0, 3, 4):
+        Cg = run_case(gpu, ob, X, W, sc, zp, tile=tile)
+        assert np.array_equal(Cg, want)
+
+
+def test_golden_cases_all_transpose_modes(gpu):
+    g = np.load(golden_path("qmm_cases.npz"))
+    for i in range(int(g["count"])):
+        pre = f"c{i}_"
+        M, N, K, tA, tB = (int(v) for v in g[pre + "dims"])
+        bias = g[pre + "bias"] if pre + "bias" in g.files else None
+        Cg, _ = gpu.qgemm_host(g[pre + "A"], g[pre + "B"], g[pre + "sc"], g[pre + "zp"], tA=bool(tA), tB=bool(tB),
+                               bias=bias, M=M, N=N, K=K)
+        assert np.array_equal(Cg, g[pre + "C"]), (i, M, N, K, tA, tB)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 5, 7), (33, 65, 100), (64, 64, 64), (100, 200, 300), (17, 512, 784),
+                                   (300, 257, 1000), (1, 300, 33), (130, 1, 2000)])
+def test_ragged_shapes_random_zero_points(gpu, ob, shape):
+    M, N, K = shape
+    rng = np.random.default_rng(M * 1000003 + N * 1009 + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    zp = rng.integers(0, 256, 3).astype(np.uint8)
+    sc = np.array([0.02, 0.01, 0.7], np.float32)
+    bias = rng.integers(-100000, 100000, N).astype(np.int32)
+    for tile in (0, 3, 4):
+        run_case(gpu, ob, A, B, sc, zp, bias=bias, tile=tile)
+
+
+@pytest.mark.parametrize("tile,shape", [(1, (256, 256, 64)), (1, (512, 768, 320)), (2, (128, 128, 64)),
+                                        (2, (384, 256, 448)), (1, (256, 512, 1024))])
+def test_fast_tiles(gpu, ob, tile, shape):
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + tile)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    for zp in ([128, 128, 128], [0, 128, 3], [255, 1, 200]):
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array(zp, np.uint8),
+                 bias=rng.integers(-5000, 5000, N).astype(np.int32) if zp[0] else None, tile=tile)
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (1, 1)])
+def test_other_transpose_modes(gpu, ob, tA, tB):
+    rng = np.random.default_rng(77 + tA * 2 + tB)
+    M, N, K = 70, 130, 150
+    A = rng.integers(0, 256, M * K, dtype=np.uint8)
+    B = rng.integers(0, 256, N * K, dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.01, 0.5], np.array([7, 99, 128], np.uint8), tA=bool(tA), tB=bool(tB), M=M, N=N, K=K)
+
+
+def test_extreme_values_and_zero_point_invariants(gpu, ob):
+    M, N, K = 64, 96, 2048
+    for a, b in ((255, 255), (0, 0), (255, 0)):
+        A = np.full((M, K), a, np.uint8)
+        B = np.full((N, K), b, np.uint8)
+        run_case(gpu, ob, A, B, [0.001, 0.001, 1.0], np.array([0, 0, 0], np.uint8))       # largest accumulators
+        run_case(gpu, ob, A, B, [0.001, 0.001, 1.0], np.array([255, 255, 9], np.uint8))   # most negative terms
+    rng = np.random.default_rng(0)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    Bc = np.full((N, K), 77, np.uint8)
+    Cg = run_case(gpu, ob, A, Bc, [0.3, 0.2, 0.1], np.array([5, 77, 200], np.uint8))
+    assert (Cg == 200).all()   # B == zpB: accumulator 0, output = output zero point
+
+
+def test_requantize_sweep_on_gpu(gpu):
+    """Arbitrary int32 accumulators through the GPU epilogue: A = 0, zero points 0 make `element`
+    equal to bias[n] (l-ten/math_fns.cpp:1469-1473).  Expected bytes come from l-ten's own code."""
+    g = np.load(golden_path("requant_sweep.npz"))
+    acc, mults, zps, expected = g["acc"], g["mults"], g["zps"], g["expected"]
+    n = len(acc)
+    A = np.zeros((1, 1), np.uint8)
+    B = np.zeros((n, 1), np.uint8)
+    for i, m in enumerate(mults):
+        for j, z in enumerate(zps):
+            Cg, _ = gpu.qgemm_host(A, B, [m, 1.0, 1.0], [0, 0, z], bias=acc)
+            assert np.array_equal(Cg.reshape(-1), expected[i, j]), (float(m), int(z))
+
+
+def test_fcq_forward_leading_dims(gpu, ob, wl):
+    """FullyConnected_q on a {2, 32, 784} input (l-ten/fully_connected.cpp:364-396) in one call."""
+    X, W, sc, zp = wl.cfg1()
+    dX, dW = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(W)
+    dY = gpu.DeviceBuffer(64 * 512)
+    ws = gpu.DeviceBuffer(4 * (64 + 512))
+    gpu.check(gpu.lib().lten_hip_fcq_forward(2, 32, 784, 512, dX.ptr, dW.ptr, None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
+    assert np.array_equal(dY.numpy(np.uint8, (64, 512)), np.load(golden_path("cfg1_expected.npz"))["C"])
+
+
+def test_cfg3_full_size_properties(gpu, wl):
+    """4096^3: exact closed form of every accumulator (fp64 BLAS holds these integers exactly),
+    then the requantize rule on top; plus linearity in the bias."""
+    X, W, sc, zp = wl.cfg3()
+    M = N = K = 4096
+    dA, dB = gpu.DeviceBuffer.from_numpy(X), gpu.DeviceBuffer.from_numpy(W)
+    dC, dacc = gpu.DeviceBuffer(M * N), gpu.DeviceBuffer(4 * M * N)
+    ws = gpu.DeviceBuffer(4 * (M + N))
+    qp = gpu.qparams3(sc, zp)
+    gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
+    assert gpu.last_kernel() == "qgemm_nt_256x256x64"
+    gpu.quantized_matmul_acc(False, True, M, N, K, dA, dB, dacc, qp, None, ws)
+    acc = dacc.numpy(np.int32, (M, N))
+    want = exact_acc(X, W, int(zp[0]), int(zp[1]))
+    assert np.array_equal(acc, want)
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    out = dC.numpy(np.uint8, (M, N))
+    assert np.array_equal(out, requant_numpy(want, mult, int(zp[2])))
+    s = want * float(mult) + float(zp[2])
+    assert 0.03 < ((s < 0) | (s >= 256)).mean() < 0.25   # some outputs wrap, most do not
+
+
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_cfg4_skinny(gpu, wl, M):
+    X, W, sc, zp = wl.cfg4(M)
+    N = K = 8192
+    Cg, accg = gpu.qgemm_host(X, W, sc, zp, want_acc=True)
+    want = exact_acc(X, W, int(zp[0]), int(zp[1]))
+    assert np.array_equal(accg, want)
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    assert np.array_equal(Cg, requant_numpy(want, mult, int(zp[2])))
