@@ -1,0 +1,298 @@
+// im2col / col2im and the fused (implicit-GEMM) Conv2d forward and weight gradient for gfx950.
+//
+// l-ten lowers Conv2d to one im2col + one GEMM per image (l-ten/conv2d.cpp:164-171 forward,
+// l-ten/backprop.cpp:1949-1953 weight gradient), writing and re-reading a [Cin*kh*kw, Hout*Wout] column
+// buffer each time.  Here the column matrix is never stored: the GEMM operand fetch computes the im2col
+// address on the fly (col[k][hw] = x[ci][ho*sh - ph + i][wo*sw - pw + j], zero outside the image), and one
+// launch covers the whole batch.  The standalone im2col / col2im kernels keep the semantics of l-ten's
+// CUDA ones (l-ten/im_col.cu:65-96, 123-162) for callers that still want the buffer.
+#include "common.h"
+#include "gemm_f32_core.h"
+
+#include <algorithm>
+
+namespace lten_hip {
+
+struct ConvGeo {
+	int N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, dh, dw, Ho, Wo;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void im2col_kernel(const T* im, ConvGeo g, T* col)
+{
+	// one thread per element of col, consecutive threads along Hout*Wout
+	const int64_t total = (int64_t)g.Cin * g.kh * g.kw * g.Ho * g.Wo;
+	for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+		const int wo = (int)(idx % g.Wo);
+		const int ho = (int)((idx / g.Wo) % g.Ho);
+		const int r = (int)(idx / ((int64_t)g.Wo * g.Ho));
+		const int j = r % g.kw, i = (r / g.kw) % g.kh, c = r / (g.kw * g.kh);
+		const int y = ho * g.sh - g.ph + i * g.dh, x = wo * g.sw - g.pw + j * g.dw;
+		col[idx] = (y >= 0 && y < g.H && x >= 0 && x < g.W) ? im[((int64_t)c * g.H + y) * g.W + x] : (T)0;
+	}
+}
+
+__global__ __launch_bounds__(256) void col2im_kernel(const float* col, ConvGeo g, float* im)
+{
+	// one thread per image element gathers every column entry that maps to it, kernel taps in increasing
+	// (i, j) order — the order in which l-ten's CPU scatter-add reaches that element (l-ten/im_col.h:41-55)
+	const int64_t total = (int64_t)g.Cin * g.H * g.W;
+	for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+		const int x = (int)(idx % g.W), y = (int)((idx / g.W) % g.H), c = (int)(idx / ((int64_t)g.W * g.H));
+		float s = 0.0f;
+		for (int i = 0; i < g.kh; i++) {
+			const int yy = y + g.ph - i * g.dh;
+			if (yy < 0 || yy % g.sh != 0 || yy / g.sh >= g.Ho) continue;
+			for (int j = 0; j < g.kw; j++) {
+				const int xx = x + g.pw - j * g.dw;
+				if (xx < 0 || xx % g.sw != 0 || xx / g.sw >= g.Wo) continue;
+				s += col[(((int64_t)c * g.kh + i) * g.kw + j) * g.Ho * g.Wo + (int64_t)(yy / g.sh) * g.Wo + xx / g.sw];
+			}
+		}
+		im[idx] = s;
+	}
+}
+
+// Per reduction index k = (ci, i, j): offset of the tap inside one image and the tap coordinates.
+struct KTap {
+	int off;  // (ci*H + i*dh)*W + j*dw
+	int ij;   // i*dh | (j*dw) << 16
+};
+constexpr int MAX_KTAB = 2304;  // Cin*kh*kw up to 2304 (e.g. 256 channels of 3x3) use the LDS table
+
+__device__ __forceinline__ KTap make_tap(const ConvGeo& g, int k)
+{
+	const int j = k % g.kw, i = (k / g.kw) % g.kh, ci = k / (g.kw * g.kh);
+	KTap t;
+	t.off = (ci * g.H + i * g.dh) * g.W + j * g.dw;
+	t.ij = (i * g.dh) | ((j * g.dw) << 16);
+	return t;
+}
+
+// Forward: y[n][co][hw] = sum_k w[co][k] * col_n[k][hw]  (+ bias[co]).  GEMM rows = co, columns = hw.
+template <int BM, int BN, int BK, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, const float* x, const float* w, const float* bias, float* y)
+{
+	typedef GemmCore<BM, BN, BK, WM, WN, false, true> Core;
+	__shared__ float lds[Core::LDS_FLOATS];
+	__shared__ KTap ktab[MAX_KTAB];
+
+	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	const int tiles_n = (HW + BN - 1) / BN;
+	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+	const float* xi = x + (int64_t)blockIdx.z * g.Cin * g.H * g.W;
+	float* yi = y + (int64_t)blockIdx.z * g.Cout * HW;
+	const bool use_tab = Kc <= MAX_KTAB;
+	if (use_tab) {
+		for (int k = threadIdx.x; k < Kc; k += WM * WN * 64) ktab[k] = make_tap(g, k);
+		__syncthreads();
+	}
+
+	auto fetch_a = [&](int row, int k) -> float {
+		const int co = m0 + row;
+		return (co < g.Cout && k < Kc) ? w[(int64_t)co * Kc + k] : 0.0f;
+	};
+	auto fetch_b = [&](int row, int k) -> float {
+		const int n = n0 + row;
+		if (n >= HW || k >= Kc) return 0.0f;
+		const int ho = n / g.Wo, wo = n - ho * g.Wo;
+		const KTap t = use_tab ? ktab[k] : make_tap(g, k);
+		const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
+		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
+		if ((unsigned)ty >= (unsigned)g.H || (unsigned)tx >= (unsigned)g.W) return 0.0f;
+		return xi[t.off + yy * g.W + xx];
+	};
+
+	v16f acc[Core::FM][Core::FN];
+	Core::run(lds, 0, Kc, fetch_a, fetch_b, acc);
+	Core::for_each(acc, [&](int row, int col, float v) {
+		const int co = m0 + row, n = n0 + col;
+		if (co < g.Cout && n < HW) yi[(int64_t)co * HW + n] = bias ? v + bias[co] : v;
+	});
+}
+
+// Weight gradient: dw[co][k] = sum_n sum_hw dy[n][co][hw] * col_n[k][hw].  GEMM rows = co, columns = k,
+// reduction over hw.  Workgroup (tile, image, slice) reduces one slice of one image's hw range and writes
+// a partial [Cout x Kc] matrix; conv2d_wgrad_reduce_kernel adds the partials in a fixed order.
+template <int BM, int BN, int BK, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, const float* x, const float* dy, float* partial, int slices, int slice_len)
+{
+	typedef GemmCore<BM, BN, BK, WM, WN, false, false> Core;
+	__shared__ float lds[Core::LDS_FLOATS];
+
+	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	const int tiles_n = (Kc + BN - 1) / BN;
+	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+	const int img = blockIdx.z / slices, slice = blockIdx.z % slices;
+	const int r0 = slice * slice_len, r1 = min(HW, r0 + slice_len);
+	const float* xi = x + (int64_t)img * g.Cin * g.H * g.W;
+	const float* dyi = dy + (int64_t)img * g.Cout * HW;
+	float* out = partial + (int64_t)blockIdx.z * g.Cout * Kc;
+
+	auto fetch_a = [&](int row, int r) -> float {
+		const int co = m0 + row;
+		return (co < g.Cout && r < r1) ? dyi[(int64_t)co * HW + r] : 0.0f;
+	};
+	auto fetch_b = [&](int row, int r) -> float {
+		const int k = n0 + row;
+		if (k >= Kc || r >= r1) return 0.0f;
+		const KTap t = make_tap(g, k);
+		const int ho = r / g.Wo, wo = r - ho * g.Wo;
+		const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
+		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
+		if ((unsigned)ty >= (unsigned)g.H || (unsigned)tx >= (unsigned)g.W) return 0.0f;
+		return xi[t.off + yy * g.W + xx];
+	};
+
+	v16f acc[Core::FM][Core::FN];
+	Core::run(lds, r0, r1, fetch_a, fetch_b, acc);
+	Core::for_each(acc, [&](int row, int col, float v) {
+		const int co = m0 + row, k = n0 + col;
+		if (co < g.Cout && k < Kc) out[(int64_t)co * Kc + k] = v;
+	});
+}
+
+__global__ __launch_bounds__(256) void conv2d_wgrad_reduce_kernel(const float* partial, int parts, int64_t count, float* dw)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= count) return;
+	float s = 0.0f;
+	for (int p = 0; p < parts; p++) s += partial[(int64_t)p * count + idx];
+	dw[idx] = s;
+}
+
+static int make_geo(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
+                    int pw, int sh, int sw, int dh, int dw)
+{
+	LTEN_HIP_REQUIRE(kh > 0 && kw > 0 && sh > 0 && sw > 0 && dh > 0 && dw > 0 && ph >= 0 && pw >= 0, "conv: bad kernel geometry");
+	LTEN_HIP_REQUIRE(N < 65536 && Cin < (1u << 20) && Cout < (1u << 20) && H < (1u << 15) && W < (1u << 15), "conv: dimension too large");
+	LTEN_HIP_REQUIRE(Cin * H * W < (1ull << 31) && Cout * H * W < (1ull << 31), "conv: one image must stay below 2^31 elements");
+	const int64_t eh = (int64_t)H + 2 * ph - ((int64_t)dh * (kh - 1) + 1), ew = (int64_t)W + 2 * pw - ((int64_t)dw * (kw - 1) + 1);
+	LTEN_HIP_REQUIRE(eh >= 0 && ew >= 0, "conv: kernel larger than the padded image");
+	g.N = (int)N; g.Cin = (int)Cin; g.H = (int)H; g.W = (int)W; g.Cout = (int)Cout;
+	g.kh = kh; g.kw = kw; g.ph = ph; g.pw = pw; g.sh = sh; g.sw = sw; g.dh = dh; g.dw = dw;
+	// l-ten/conv2d.cpp:102-103 (dilation 1) and l-ten/im_col.cu:104-107
+	g.Ho = (int)(eh / sh + 1);
+	g.Wo = (int)(ew / sw + 1);
+	return 0;
+}
+
+static void wgrad_split(const ConvGeo& g, int& slices, int& slice_len)
+{
+	// enough (image, slice) pairs to fill 256 CUs a few times over, slices a multiple of the k-step
+	const int HW = g.Ho * g.Wo;
+	int want = (int)ceil_div(256, (uint64_t)g.N);
+	if (want < 1) want = 1;
+	slice_len = (int)ceil_div((uint64_t)HW, (uint64_t)want);
+	slice_len = (int)(ceil_div((uint64_t)slice_len, 64) * 64);
+	if (slice_len < 256) slice_len = 256;
+	slices = (int)ceil_div((uint64_t)HW, (uint64_t)slice_len);
+}
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+int lten_hip_im2col_f32(const float* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
+                        int dw, float* col)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
+	const int64_t total = (int64_t)C * kh * kw * g.Ho * g.Wo;
+	if (total == 0) return 0;
+	LTEN_HIP_REQUIRE(im && col, "im2col: null pointer");
+	im2col_kernel<float><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(im, g, col);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_im2col_u8(const uint8_t* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
+                       int dw, uint8_t* col)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
+	const int64_t total = (int64_t)C * kh * kw * g.Ho * g.Wo;
+	if (total == 0) return 0;
+	LTEN_HIP_REQUIRE(im && col, "im2col: null pointer");
+	im2col_kernel<uint8_t><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(im, g, col);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_col2im_f32(const float* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
+                        int dw, float* im)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
+	const int64_t total = (int64_t)C * H * W;
+	if (total == 0) return 0;
+	LTEN_HIP_REQUIRE(im && col, "col2im: null pointer");
+	col2im_kernel<<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(col, g, im);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
+                                int pw, int sh, int sw, const float* x, const float* w, const float* bias, float* y)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return rc;
+	if (N == 0 || Cout == 0 || g.Ho * g.Wo == 0) return 0;
+	LTEN_HIP_REQUIRE(x && w && y, "conv2d_forward: null pointer");
+	const int HW = g.Ho * g.Wo;
+	if (Cout > 32) {
+		set_kernel_name("conv2d_forward_64x64x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
+		conv2d_forward_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	} else {
+		set_kernel_name("conv2d_forward_32x128x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(HW, 128)), 1, (unsigned)N);
+		conv2d_forward_kernel<32, 128, 32, 1, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh,
+                                               int kw, int ph, int pw, int sh, int sw)
+{
+	ConvGeo g;
+	if (make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return 0;
+	int slices, slice_len;
+	wgrad_split(g, slices, slice_len);
+	return (uint64_t)N * slices * Cout * Cin * kh * kw * sizeof(float);
+}
+
+int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
+                              int pw, int sh, int sw, const float* x, const float* dy, float* dw, void* workspace)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return rc;
+	const int64_t Kc = (int64_t)Cin * kh * kw, count = (int64_t)Cout * Kc;
+	if (count == 0) return 0;
+	LTEN_HIP_REQUIRE(dw != nullptr, "conv2d_wgrad: dw is null");
+	if (N == 0 || g.Ho * g.Wo == 0) return lten_hip_zero(dw, count * sizeof(float));
+	LTEN_HIP_REQUIRE(x && dy && workspace, "conv2d_wgrad: null pointer");
+	int slices, slice_len;
+	wgrad_split(g, slices, slice_len);
+	const int parts = (int)N * slices;
+	LTEN_HIP_REQUIRE(parts < 65536, "conv2d_wgrad: too many partial sums");
+	float* partial = static_cast<float*>(workspace);
+	if (Cout > 32) {
+		set_kernel_name("conv2d_wgrad_64x64x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(Kc, 64)), 1, (unsigned)parts);
+		conv2d_wgrad_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, slices, slice_len);
+	} else {
+		set_kernel_name("conv2d_wgrad_32x32x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(Kc, 32)), 1, (unsigned)parts);
+		conv2d_wgrad_kernel<32, 32, 32, 1, 1><<<grid, dim3(64), 0, stream()>>>(g, x, dy, partial, slices, slice_len);
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	conv2d_wgrad_reduce_kernel<<<dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, stream()>>>(partial, parts, count, dw);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+// fp32 GEMM for gfx950: the row-major sgemm that stands in for every cublasSgemm call of l-ten's GPU
+// branches (l-ten/fully_connected.cpp:150,165; l-ten/md_array_cuda.h:513; l-ten/backprop.cpp:562,580,
+// 2228,2252,2267) with the contract of cpu_gemm<float> (l-ten/math_fns.cpp:1258) plus leading dimensions.
+//
+// The tile loop lives in gemm_f32_core.h (32x32x2 fp32 MFMA blocks, LDS double buffer); this file adds
+// the strided operand fetch, the alpha/beta/bias epilogue, the two degenerate shapes l-ten uses (K == 1
+// rank-1 bias update, M == 1 column sum) and the dispatch.
+#include "common.h"
+#include "gemm_f32_core.h"
+
+namespace lten_hip {
+
+struct SProblem {
+	const float* A;
+	const float* B;
+	float* C;
+	const float* bias;  // optional, added per output column n (FullyConnected bias), or null
+	int64_t lda, ldb, ldc;
+	int64_t stride_a, stride_b, stride_c;  // per blockIdx.z
+	int M, N, K;
+	float alpha, beta;
+};
+
+template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
+__global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
+{
+	// A[m][k] is at A[m*lda + k] (not transposed, contiguous in k) or A[k*lda + m] (transposed).
+	// B[k][n] is at B[k*ldb + n] (not transposed, contiguous in n) or B[n*ldb + k] (transposed).
+	typedef GemmCore<BM, BN, BK, WM, WN, TA, !TB> Core;
+	__shared__ float lds[Core::LDS_FLOATS];
+
+	const int tiles_n = (p.N + BN - 1) / BN;
+	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
+	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
+	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+
+	auto fetch_a = [&](int row, int k) -> float {
+		const int m = m0 + row;
+		if (m >= p.M || k >= p.K) return 0.0f;
+		return TA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+	};
+	auto fetch_b = [&](int row, int k) -> float {
+		const int n = n0 + row;
+		if (n >= p.N || k >= p.K) return 0.0f;
+		return TB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
+	};
+
+	v16f acc[Core::FM][Core::FN];
+	Core::run(lds, 0, p.K, fetch_a, fetch_b, acc);
+
+	Core::for_each(acc, [&](int row, int col, float v) {
+		const int m = m0 + row, n = n0 + col;
+		if (m >= p.M || n >= p.N) return;
+		float* c = C + (int64_t)m * p.ldc + n;
+		float out = p.alpha * v;
+		if (p.beta != 0.0f) out += p.beta * *c;  // beta == 0 overwrites: NaN/Inf in C must not survive
+		if (p.bias) out += p.bias[n];
+		*c = out;
+	});
+}
+
+// K == 1: the rank-1 update C = alpha * a b^T + beta * C that l-ten uses to add the FC bias
+// (l-ten/fully_connected.cpp:165).
+__global__ __launch_bounds__(256) void sgemm_rank1_kernel(SProblem p, int tA, int tB)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= (int64_t)p.M * p.N) return;
+	const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+	const float a = tA ? p.A[m] : p.A[(int64_t)m * p.lda];
+	const float b = tB ? p.B[(int64_t)n * p.ldb] : p.B[n];
+	float* c = p.C + (int64_t)m * p.ldc + n;
+	float v = p.alpha * (a * b);
+	if (p.beta != 0.0f) v += p.beta * *c;
+	*c = v;
+}
+
+// M == 1 with B not transposed: c[n] = alpha * sum_k a[k] B[k][n] + beta * c[n] — the column sum that
+// l-ten uses for the bias gradient with a = ones (l-ten/backprop.cpp:2267).  256 threads = 64 columns x
+// 4 k-slices; the slices are combined in a fixed order.  A null A stands for a vector of ones, so the
+// bias_multiplier tensor of l-ten's FullyConnected is never needed on the device.
+__global__ __launch_bounds__(256) void sgemm_rowvec_kernel(SProblem p, int tA)
+{
+	__shared__ float part[4][64];
+	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+	const int n = blockIdx.x * 64 + tx;
+	float s = 0.0f;
+	if (n < p.N)
+		for (int k = ty; k < p.K; k += 4) {
+			const float a = p.A == nullptr ? 1.0f : (tA ? p.A[(int64_t)k * p.lda] : p.A[k]);
+			s = fmaf(a, p.B[(int64_t)k * p.ldb + n], s);
+		}
+	part[ty][tx] = s;
+	__syncthreads();
+	if (ty == 0 && n < p.N) {
+		float v = p.alpha * (((part[0][tx] + part[1][tx]) + part[2][tx]) + part[3][tx]);
+		if (p.beta != 0.0f) v += p.beta * p.C[n];
+		p.C[n] = v;
+	}
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+static int launch_sgemm(const SProblem& p, int tA, int tB, uint64_t batch, const char* name)
+{
+	const dim3 grid((unsigned)(ceil_div(p.M, BM) * ceil_div(p.N, BN)), 1, (unsigned)batch);
+	const dim3 block(WM * WN * 64);
+	set_kernel_name(name);
+	if (!tA && !tB) sgemm_kernel<BM, BN, BK, WM, WN, false, false><<<grid, block, 0, stream()>>>(p);
+	if (!tA && tB) sgemm_kernel<BM, BN, BK, WM, WN, false, true><<<grid, block, 0, stream()>>>(p);
+	if (tA && !tB) sgemm_kernel<BM, BN, BK, WM, WN, true, false><<<grid, block, 0, stream()>>>(p);
+	if (tA && tB) sgemm_kernel<BM, BN, BK, WM, WN, true, true><<<grid, block, 0, stream()>>>(p);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
+              int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
+              int64_t stride_c, uint64_t batch, const float* bias)
+{
+	if (M == 0 || N == 0 || batch == 0) return 0;
+	LTEN_HIP_REQUIRE(C != nullptr, "sgemm: C is null");
+	LTEN_HIP_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "sgemm: null operand");
+	LTEN_HIP_REQUIRE(M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) && batch < 65536, "sgemm: dimension too large");
+	LTEN_HIP_REQUIRE(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N, "sgemm: leading dimension smaller than the row");
+	if (batch > 1 && stride_c == 0) {
+		// every problem writes the same C: run them one after another so the sum has one fixed order
+		for (uint64_t b = 0; b < batch; b++) {
+			int rc = sgemm_run(tA, tB, M, N, K, alpha, A + b * stride_a, lda, 0, B + b * stride_b, ldb, 0,
+			                   (b == 0) ? beta : 1.0f, C, ldc, 0, 1, bias && b == 0 ? bias : nullptr);
+			if (rc) return rc;
+		}
+		return 0;
+	}
+	SProblem p;
+	p.A = A; p.B = B; p.C = C; p.bias = bias;
+	p.lda = (int64_t)lda; p.ldb = (int64_t)ldb; p.ldc = (int64_t)ldc;
+	p.stride_a = stride_a; p.stride_b = stride_b; p.stride_c = stride_c;
+	p.M = (int)M; p.N = (int)N; p.K = (int)K;
+	p.alpha = alpha; p.beta = beta;
+
+	const int force = get_option(OPT_SGEMM_TILE);
+	if (force == 0 && batch == 1 && bias == nullptr && K == 1) {
+		set_kernel_name("sgemm_rank1");
+		sgemm_rank1_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(p, tA, tB);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+	if (force == 0 && batch == 1 && bias == nullptr && M == 1 && !tB) {
+		set_kernel_name("sgemm_rowvec");
+		sgemm_rowvec_kernel<<<dim3((unsigned)ceil_div(N, 64)), dim3(256), 0, stream()>>>(p, tA);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+	const uint64_t tiles64 = ceil_div(M, 64) * ceil_div(N, 64) * batch;
+	const uint64_t tiles128 = ceil_div(M, 128) * ceil_div(N, 128) * batch;
+	int choice = force;
+	if (choice == 0) choice = tiles128 >= 512 ? 1 : (tiles64 >= 256 ? 2 : 3);
+	switch (choice) {
+	case 1: return launch_sgemm<128, 128, 16, 2, 2>(p, tA, tB, batch, "sgemm_128x128x16");
+	case 2: return launch_sgemm<64, 64, 32, 2, 2>(p, tA, tB, batch, "sgemm_64x64x32");
+	default: return launch_sgemm<32, 32, 32, 1, 1>(p, tA, tB, batch, "sgemm_32x32x32");
+	}
+}
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+int lten_hip_sgemm(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
+                   const float* B, uint64_t ldb, float beta, float* C, uint64_t ldc)
+{
+	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, nullptr);
+}
+
+int lten_hip_sgemm_strided_batched(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A,
+                                   uint64_t lda, int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b,
+                                   float beta, float* C, uint64_t ldc, int64_t stride_c, uint64_t batch)
+{
+	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, batch, nullptr);
+}
+
+int lten_hip_fc_forward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* bias,
+                            float* Y)
+{
+	// l-ten/fully_connected.cpp:150 (NT GEMM) and :165 (ones x bias, beta = 1) in one launch
+	return sgemm_run(0, 1, M, out, in, 1.0f, X, in, 0, W, in, 0, 0.0f, Y, out, 0, 1, bias);
+}
+
+int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
+                             float* dX, float* dW, float* db)
+{
+	int rc = 0;
+	// l-ten/backprop.cpp:2228  dX[M x in] = dY[M x out] W[out x in]
+	if (dX) rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr);
+	// :2252  dW[out x in] = dY[M x out]^T X[M x in]
+	if (!rc && dW) rc = sgemm_run(1, 0, out, in, M, 1.0f, dY, out, 0, X, in, 0, 0.0f, dW, in, 0, 1, nullptr);
+	// :2267  db[1 x out] += ones[1 x M] dY[M x out]; the ones vector is never materialised: a = 1 for every k
+	if (!rc && db && M != 0 && out != 0) {
+		SProblem p = {};
+		p.A = nullptr;  // a[k] = 1
+		p.B = dY; p.C = db;
+		p.ldb = (int64_t)out; p.ldc = (int64_t)out;
+		p.M = 1; p.N = (int)out; p.K = (int)M;
+		p.alpha = 1.0f; p.beta = 1.0f;
+		set_kernel_name("sgemm_rowvec");
+		sgemm_rowvec_kernel<<<dim3((unsigned)ceil_div(out, 64)), dim3(256), 0, stream()>>>(p, 0);
+		LTEN_HIP_LAUNCH_CHECK();
+	}
+	return rc;
+}
+
+}  // extern "C"

@@ -1,0 +1,124 @@
+"""GPU parity tests of im2col / col2im and the fused Conv2d forward + weight gradient (C ABI).
+im2col and col2im are data movement / fixed-order sums: bit-exact.  Convolutions: max relative error 1e-4
+(conftest.rel_err)."""
+import numpy as np
+import pytest
+
+from conftest import golden_path, rel_err
+from test_oracle_conv import GEOS, direct_conv
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+@pytest.mark.parametrize("geo", GEOS + [(3, 33, 47, 3, 3, 1, 1, 1, 1), (2, 64, 64, 5, 3, 2, 1, 2, 2)])
+def test_im2col_col2im_bit_exact(gpu, ob, geo):
+    C, H, W, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    im = rng.standard_normal((C, H, W)).astype(np.float32)
+    col = np.empty((C * kh * kw, Ho * Wo), np.float32)
+    ob.oracle().oracle_im2col_f32(im.reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, col.reshape(-1))
+    D = gpu.DeviceBuffer
+    dIm, dCol = D.from_numpy(im), D(col.nbytes)
+    gpu.check(gpu.lib().lten_hip_im2col_f32(dIm.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dCol.ptr))
+    assert np.array_equal(dCol.numpy(np.float32, col.shape), col)
+    # uint8 flavour (Conv2d_q's operand)
+    imu = rng.integers(0, 256, (C, H, W), dtype=np.uint8)
+    colu = np.empty((C * kh * kw, Ho * Wo), np.uint8)
+    ob.oracle().oracle_im2col_u8(imu.reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, colu.reshape(-1))
+    dImu, dColu = D.from_numpy(imu), D(colu.nbytes)
+    gpu.check(gpu.lib().lten_hip_im2col_u8(dImu.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dColu.ptr))
+    assert np.array_equal(dColu.numpy(np.uint8, colu.shape), colu)
+    # col2im: same taps in the same order as the CPU scatter-add -> identical floats
+    c = rng.standard_normal(col.shape).astype(np.float32)
+    back = np.zeros_like(im)
+    ob.oracle().oracle_col2im_f32(c.reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, back.reshape(-1))
+    dC, dBack = D.from_numpy(c), D(im.nbytes)
+    gpu.check(gpu.lib().lten_hip_col2im_f32(dC.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dBack.ptr))
+    assert np.array_equal(dBack.numpy(np.float32, im.shape), back)
+
+
+def gpu_conv(gpu, geo, x, w, dy=None, bias=None):
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    Ho, Wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    D = gpu.DeviceBuffer
+    dX, dW = D.from_numpy(x), D.from_numpy(w)
+    dB = D.from_numpy(bias) if bias is not None else None
+    dY = D(4 * N * Cout * Ho * Wo)
+    l = gpu.lib()
+    gpu.check(l.lten_hip_conv2d_forward_f32(*geo, dX.ptr, dW.ptr, dB.ptr if dB else None, dY.ptr))
+    fk = gpu.last_kernel()
+    y = dY.numpy(np.float32, (N, Cout, Ho, Wo))
+    dw = None
+    if dy is not None:
+        dDY = D.from_numpy(dy)
+        ws = D(max(int(l.lten_hip_conv2d_wgrad_workspace_bytes(*geo)), 4))
+        dDW = D(w.nbytes)
+        gpu.check(l.lten_hip_conv2d_wgrad_f32(*geo, dX.ptr, dDY.ptr, dDW.ptr, ws.ptr))
+        dw = dDW.numpy(np.float32, w.shape)
+    return y, dw, fk
+
+
+def test_conv_layer_golden(gpu):
+    g = np.load(golden_path("layer_cases.npz"))
+    for i in range(int(g["conv_count"])):
+        pre = f"cv{i}_"
+        geo = tuple(int(v) for v in g[pre + "geo"])
+        y, dw, _ = gpu_conv(gpu, geo, g[pre + "x"], g[pre + "w"], g[pre + "dy"])
+        assert rel_err(y.reshape(-1), g[pre + "y"]) < TOL, i
+        assert rel_err(dw.reshape(-1), g[pre + "dw"]) < TOL, i
+
+
+@pytest.mark.parametrize("geo", [(2, 3, 9, 8, 4, 3, 3, 1, 1, 1, 1), (1, 2, 10, 7, 3, 3, 2, 0, 1, 2, 1),
+                                 (2, 4, 6, 6, 5, 5, 5, 2, 2, 1, 1), (3, 16, 33, 29, 40, 3, 3, 1, 1, 1, 1),
+                                 (2, 8, 40, 40, 70, 3, 3, 1, 1, 2, 2), (2, 1, 64, 64, 32, 3, 3, 1, 1, 1, 1)])
+def test_conv_vs_oracle(gpu, ob, geo):
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_y = np.empty((N, Cout, Ho, Wo), np.float32)
+    ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
+    want_dw = np.empty_like(w)
+    ob.oracle().oracle_conv2d_wgrad(*geo, x.reshape(-1), dy.reshape(-1), want_dw.reshape(-1), col)
+    y, dw, fk = gpu_conv(gpu, geo, x, w, dy, bias)
+    assert rel_err(y, want_y + bias[None, :, None, None]) < TOL, fk
+    assert rel_err(dw, want_dw) < TOL
+    assert rel_err(y, direct_conv(x, w, ph, pw, sh, sw) + bias[None, :, None, None]) < TOL
+
+
+def test_cfg5_full_size(gpu, wl):
+    """32x1x128x128 -> 32 channels -> 64 channels, 3x3 s1 p1: forward of both layers and both weight gradients,
+    checked in fp64 on sampled outputs (forward) and in full (weight gradients are only 288 / 18432 numbers)."""
+    x, ws, dyshapes = wl.cfg5()
+    rng = np.random.default_rng(0)
+    inp = x
+    for layer, w in enumerate(ws):
+        N, Cin, H, W = inp.shape
+        Cout = w.shape[0]
+        geo = (N, Cin, H, W, Cout, 3, 3, 1, 1, 1, 1)
+        dy = wl.cfg5_dy(dyshapes[layer], layer=layer)
+        y, dw, fk = gpu_conv(gpu, geo, inp, w, dy)
+        # forward: sampled output positions against a direct fp64 sum
+        xp = np.pad(inp.astype(np.float64), ((0, 0), (0, 0), (1, 1), (1, 1)))
+        idx = [(int(rng.integers(0, N)), int(rng.integers(0, Cout)), int(rng.integers(0, H)), int(rng.integers(0, W)))
+               for _ in range(400)] + [(0, 0, 0, 0), (N - 1, Cout - 1, H - 1, W - 1), (1, 1, 0, W - 1), (2, 0, H - 1, 0)]
+        want = np.array([(xp[n, :, h:h + 3, ww:ww + 3] * w[c].astype(np.float64)).sum() for (n, c, h, ww) in idx])
+        got = np.array([y[i] for i in idx])
+        scale = float(np.sqrt((y.astype(np.float64) ** 2).mean()))
+        assert (np.abs(got - want) / np.maximum(np.abs(want), scale)).max() < TOL, fk
+        # weight gradient in full: dw[c, ci, i, j] = sum_{n,h,w} dy[n,c,h,w] * xpad[n,ci,h+i,w+j]
+        want_dw = np.empty(w.shape, np.float64)
+        dy64 = dy.astype(np.float64)
+        for i in range(3):
+            for j in range(3):
+                want_dw[:, :, i, j] = np.einsum("nchw,ndhw->cd", dy64, xp[:, :, i:i + H, j:j + W], optimize=True)
+        assert rel_err(dw, want_dw) < TOL
+        print(f"  layer {layer + 1}: forward via {fk}, wgrad via {gpu.last_kernel()}, "
+              f"dw max rel err {rel_err(dw, want_dw):.2e}")
+        inp = y

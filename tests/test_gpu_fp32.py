@@ -1,0 +1,183 @@
+"""GPU parity tests of the fp32 GEMM path through the C ABI.  Tolerance (north star): max relative
+error 1e-4, measured as max |got - want| / max(|want|, rms(want)) (conftest.rel_err); integer-valued
+inputs must come out exactly (any summation order is exact), which checks layouts and transposes bit for bit."""
+import json
+
+import numpy as np
+import pytest
+
+from conftest import golden_path, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def gpu_sgemm(gpu, tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, C0, ldc, tile=0):
+    dA, dB, dC = gpu.DeviceBuffer.from_numpy(A), gpu.DeviceBuffer.from_numpy(B), gpu.DeviceBuffer.from_numpy(C0)
+    gpu.set_option("sgemm_tile", tile)
+    try:
+        gpu.sgemm(tA, tB, M, N, K, alpha, dA, lda, dB, ldb, beta, dC, ldc)
+    finally:
+        gpu.set_option("sgemm_tile", 0)
+    return dC.numpy(np.float32, C0.shape)
+
+
+def test_sgemm_golden_cases(gpu):
+    g = np.load(golden_path("sgemm_cases.npz"))
+    for i in range(int(g["count"])):
+        pre = f"c{i}_"
+        M, N, K, tA, tB = (int(v) for v in g[pre + "dims"])
+        alpha, beta = (float(v) for v in g[pre + "ab"])
+        got = gpu_sgemm(gpu, tA, tB, M, N, K, alpha, g[pre + "A"], M if tA else K, g[pre + "B"], K if tB else N, beta,
+                        g[pre + "C0"], N)
+        assert rel_err(got, g[pre + "C"]) < TOL, (i, M, N, K, tA, tB, alpha, beta, gpu.last_kernel())
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_integer_valued_exact_with_leading_dims(gpu, tile, tA, tB):
+    rng = np.random.default_rng(40 + 2 * tA + tB + 10 * tile)
+    M, N, K = 77, 139, 101
+    A = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, (K, N)).astype(np.float32)
+    want = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    lda, ldb, ldc = (M if tA else K) + 3, (K if tB else N) + 5, N + 2
+    As = np.zeros(((K if tA else M), lda), np.float32)
+    As[:, :(M if tA else K)] = A.T if tA else A
+    Bs = np.zeros(((N if tB else K), ldb), np.float32)
+    Bs[:, :(K if tB else N)] = B.T if tB else B
+    C0 = np.full((M, ldc), 7.0, np.float32)
+    got = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, C0, ldc, tile)
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, tA, tB, M, N, K, 2.0, As, lda, Bs, ldb, -1.0, got, ldc, tile)
+    assert np.array_equal(got2[:, :N], want)
+
+
+def test_beta_zero_overwrites_nan(gpu):
+    A = np.ones((5, 3), np.float32)
+    B = np.ones((3, 6), np.float32)
+    got = gpu_sgemm(gpu, 0, 0, 5, 6, 3, 1.0, A, 3, B, 6, 0.0, np.full((5, 6), np.nan, np.float32), 6)
+    assert np.array_equal(got, np.full((5, 6), 3.0, np.float32))
+
+
+@pytest.mark.parametrize("shape", [(128, 1024, 784), (128, 1024, 1024), (128, 10, 1024)])
+def test_cfg2_gemm_shapes_all_layouts(gpu, ob, shape):
+    """The nine GEMMs of the MLP step: forward NT, data gradient NN, weight gradient TN."""
+    M, N, K = shape  # forward: Y[M x N] = X[M x K] W[N x K]^T
+    rng = np.random.default_rng(M + N + K)
+    X = rng.uniform(0, 1, (M, K)).astype(np.float32)
+    W = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    dY = rng.standard_normal((M, N)).astype(np.float32)
+    for (tA, tB, m, n, k, A, B) in [(0, 1, M, N, K, X, W), (0, 0, M, K, N, dY, W), (1, 0, N, K, M, dY, X)]:
+        lda, ldb = A.shape[1], B.shape[1]
+        want = np.zeros((m, n), np.float32)
+        ob.sgemm(tA, tB, m, n, k, 1.0, A, lda, B, ldb, 0.0, want, n, f64=True)
+        got = gpu_sgemm(gpu, tA, tB, m, n, k, 1.0, A, lda, B, ldb, 0.0, np.zeros((m, n), np.float32), n)
+        err = rel_err(got, want)
+        print(f"  {'TN'[tA]}{'NT'[tB]} {m}x{n}x{k} via {gpu.last_kernel()}: max rel err {err:.2e}")
+        assert err < TOL
+
+
+def test_rank1_and_rowvec_shapes(gpu, ob):
+    rng = np.random.default_rng(9)
+    M, N = 128, 1024
+    ones = np.ones((M, 1), np.float32)
+    bias = rng.standard_normal((1, N)).astype(np.float32)
+    Y0 = rng.standard_normal((M, N)).astype(np.float32)
+    # l-ten/fully_connected.cpp:165: Y += ones[M x 1] bias[1 x N]
+    got = gpu_sgemm(gpu, 0, 0, M, N, 1, 1.0, ones, 1, bias, N, 1.0, Y0, N)
+    assert gpu.last_kernel() == "sgemm_rank1"
+    assert np.array_equal(got, Y0 + bias)
+    # l-ten/backprop.cpp:2267: db[1 x N] += ones[1 x M] dY[M x N]
+    db0 = rng.standard_normal((1, N)).astype(np.float32)
+    got = gpu_sgemm(gpu, 0, 0, 1, N, M, 1.0, np.ones((1, M), np.float32), M, Y0, N, 1.0, db0, N)
+    assert gpu.last_kernel() == "sgemm_rowvec"
+    assert rel_err(got, db0 + Y0.astype(np.float64).sum(0, keepdims=True)) < TOL
+
+
+def test_strided_batched_and_broadcast(gpu, ob):
+    g = np.load(golden_path("layer_cases.npz"))
+    # case 0: a{2,1,4,8} x b{1,1,8,15}: b broadcast over the leading index (stride 0)
+    a, b, c = g["mm0_a"], g["mm0_b"], g["mm0_c"]
+    dA, dB, dC = gpu.DeviceBuffer.from_numpy(a), gpu.DeviceBuffer.from_numpy(b), gpu.DeviceBuffer(c.nbytes)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(0, 0, 4, 15, 8, 1.0, dA.ptr, 8, 32, dB.ptr, 15, 0, 0.0, dC.ptr, 15,
+                                                       60, 2))
+    assert rel_err(dC.numpy(np.float32, c.shape), c) < TOL
+    # its weight gradient: dB += A_i^T dC_i over the batch, all into one dB (stride_c = 0, beta = 1)
+    dc, db = g["mm0_dc"], g["mm0_db"]
+    dDC, dDB = gpu.DeviceBuffer.from_numpy(dc), gpu.DeviceBuffer(db.nbytes, zero=True)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(1, 0, 8, 15, 4, 1.0, dA.ptr, 8, 32, dDC.ptr, 15, 60, 1.0, dDB.ptr,
+                                                       15, 0, 2))
+    assert rel_err(dDB.numpy(np.float32, db.shape), db) < TOL
+
+
+def test_fc_forward_backward_golden_and_lten_vectors(gpu):
+    g = np.load(golden_path("layer_cases.npz"))
+    cases = []
+    for i in range(int(g["fc_count"])):
+        pre = f"fc{i}_"
+        M, fin, fout, use_bias = (int(v) for v in g[pre + "dims"])
+        cases.append((M, fin, fout, g[pre + "x"], g[pre + "w"], g[pre + "b"] if use_bias else None, g[pre + "dy"],
+                      g[pre + "y"], g[pre + "dx"], g[pre + "dw"], g[pre + "db"] if use_bias else None, TOL, True))
+    v = json.load(open(golden_path("lten_unit_test_vectors.json")))["fc_test"]   # tests/unit_tests.cpp fc_test
+    dy = np.zeros((2, 1, 4, 8), np.float32)
+    dy[tuple(v["backward_from"])] = 1.0
+    cases.append((8, 3, 8, np.array(v["x"], np.float32), np.array(v["weights"], np.float32), None, dy.reshape(-1),
+                  np.array(v["z"], np.float32), np.array(v["x_grad"], np.float32), np.array(v["w_grad"], np.float32),
+                  None, v["tolerance"], False))
+    for (M, fin, fout, x, w, b, dy, y, dx, dw, db, tol, relative) in cases:
+        D = gpu.DeviceBuffer
+        dX, dW, dDY = D.from_numpy(x), D.from_numpy(w), D.from_numpy(dy)
+        dB = D.from_numpy(b) if b is not None else None
+        dYo, dDX, dDW = D(4 * M * fout), D(4 * M * fin), D(4 * fout * fin)
+        dDB = D(4 * fout, zero=True) if b is not None else None
+        gpu.check(gpu.lib().lten_hip_fc_forward_f32(M, fin, fout, dX.ptr, dW.ptr, dB.ptr if dB else None, dYo.ptr))
+        gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, dDX.ptr, dDW.ptr,
+                                                     dDB.ptr if dDB else None))
+        for got, want in ((dYo.numpy(np.float32, y.shape), y), (dDX.numpy(np.float32, dx.shape), dx),
+                          (dDW.numpy(np.float32, dw.shape), dw)) + (((dDB.numpy(np.float32, db.shape), db),) if b is not None else ()):
+            if relative:
+                assert rel_err(got, want) < tol
+            else:
+                assert np.abs(got - want).max() <= tol   # l-ten's own abs tolerance for fc_test
+
+
+def test_lten_matmul_test_vectors(gpu):
+    """tests/unit_tests.cpp matmul_test through the strided-batched entry point: exact values."""
+    v = json.load(open(golden_path("lten_unit_test_vectors.json")))["matmul_test"]
+    a, b = np.array(v["x"], np.float32), np.array(v["w"], np.float32)
+    D = gpu.DeviceBuffer
+    dA, dB, dC = D.from_numpy(a), D.from_numpy(b), D(4 * 32)
+    l = gpu.lib()
+    gpu.check(l.lten_hip_sgemm_strided_batched(0, 0, 4, 4, 3, 1.0, dA.ptr, 3, 12, dB.ptr, 4, 0, 0.0, dC.ptr, 4, 16, 2))
+    assert np.array_equal(dC.numpy(np.float32, (32,)), np.array(v["z"], np.float32))
+    dc = np.zeros((2, 1, 4, 4), np.float32)
+    dc[tuple(v["backward_from"])] = 1.0
+    dDC, dDA, dDB = D.from_numpy(dc), D(4 * 24, zero=True), D(4 * 12, zero=True)
+    # l-ten/backprop.cpp:562  dA_i += dC_i B^T ; :580  dB += A_i^T dC_i (B broadcast: one dB for both i)
+    gpu.check(l.lten_hip_sgemm_strided_batched(0, 1, 4, 3, 4, 1.0, dDC.ptr, 4, 16, dB.ptr, 4, 0, 1.0, dDA.ptr, 3, 12, 2))
+    gpu.check(l.lten_hip_sgemm_strided_batched(1, 0, 3, 4, 4, 1.0, dA.ptr, 3, 12, dDC.ptr, 4, 16, 1.0, dDB.ptr, 4, 0, 2))
+    assert np.array_equal(dDA.numpy(np.float32, (24,)), np.array(v["x_grad"], np.float32))
+    assert np.array_equal(dDB.numpy(np.float32, (12,)), np.array(v["w_grad"], np.float32))
+
+
+def test_large_gemm_linearity_property(gpu):
+    """2048^3: too large for the scalar oracle; check (A1 + A2) B == A1 B + A2 B on integer-valued data
+    (exact in fp32 at these magnitudes) and a sampled fp64 comparison on random data."""
+    n = 2048
+    rng = np.random.default_rng(1)
+    A1 = rng.integers(-4, 5, (n, n)).astype(np.float32)
+    A2 = rng.integers(-4, 5, (n, n)).astype(np.float32)
+    B = rng.integers(-4, 5, (n, n)).astype(np.float32)
+    z = np.zeros((n, n), np.float32)
+    c1 = gpu_sgemm(gpu, 0, 0, n, n, n, 1.0, A1, n, B, n, 0.0, z, n)
+    c12 = gpu_sgemm(gpu, 0, 0, n, n, n, 1.0, A2, n, B, n, 1.0, c1, n)
+    cs = gpu_sgemm(gpu, 0, 0, n, n, n, 1.0, A1 + A2, n, B, n, 0.0, z, n)
+    assert np.array_equal(c12, cs)
+    R = rng.standard_normal((n, n)).astype(np.float32)
+    S = rng.standard_normal((n, n)).astype(np.float32)
+    got = gpu_sgemm(gpu, 0, 1, n, n, n, 1.0, R, n, S, n, 0.0, z, n)
+    rows = rng.integers(0, n, 64)
+    want = R[rows].astype(np.float64) @ S.astype(np.float64).T
+    assert rel_err(got[rows], want) < TOL
