@@ -64,6 +64,9 @@ _SIGNATURES = {
     "lten_hip_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "lten_hip_event_destroy": (C.c_int, [vp]),
     "lten_hip_set_option": (C.c_int, [C.c_char_p, C.c_int]),
+    "lten_hip_measure_mfma_peak": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "lten_hip_measure_last_clocks": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "lten_hip_copy_kernel": (C.c_int, [vp, vp, u64]),
 }
 
 _lib = None
@@ -113,6 +116,18 @@ def last_kernel():
 
 def set_option(name, value):
     check(lib().lten_hip_set_option(name.encode(), int(value)))
+
+
+def measure_mfma_peak(kind=0, waves_per_simd=1):
+    out = C.c_float()
+    check(lib().lten_hip_measure_mfma_peak(kind, waves_per_simd, C.byref(out)))
+    return out.value
+
+
+def measure_last_clocks():
+    a, b = C.c_double(), C.c_double()
+    check(lib().lten_hip_measure_last_clocks(C.byref(a), C.byref(b)))
+    return a.value, b.value
 
 
 def qparams3(scales, zps):

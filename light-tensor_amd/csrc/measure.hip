@@ -1,0 +1,127 @@
+// Calibration kernels for the roofline figures: the MFMA issue rate this part actually sustains with no
+// memory traffic at all, and the HBM rate of a plain copy.  l-ten has no counterpart; these exist so that
+// reported fractions can be stated against measured ceilings as well as against the published peaks, and so
+// that profiler byte counters can be scaled by a kernel whose traffic is known.
+#include "common.h"
+
+#include <algorithm>
+
+namespace lten_hip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma_i8_peak_kernel(int iters, int* sink, long long* clocks)
+{
+	v16i acc0 = {}, acc1 = {}, acc2 = {}, acc3 = {};
+	v4i a = { (int)threadIdx.x, 1, 2, 3 }, b = { 4, 5, (int)blockIdx.x, 7 };
+	const long long c0 = clock64(), w0 = wall_clock64();
+	for (int i = 0; i < iters; i++) {
+		acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc0, 0, 0, 0);
+		acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc1, 0, 0, 0);
+		acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc2, 0, 0, 0);
+		acc3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc3, 0, 0, 0);
+	}
+	int s = 0;
+	for (int r = 0; r < 16; r++) s += acc0[r] + acc1[r] + acc2[r] + acc3[r];
+	if (clocks && blockIdx.x == 0 && threadIdx.x == 0) {
+		clocks[0] = clock64() - c0;       // shader clocks spent in the loop
+		clocks[1] = wall_clock64() - w0;  // same span in the 100 MHz wall clock
+	}
+	if (s == 0x7fffffff) *sink = s;  // keeps the loop alive without a store in practice
+}
+
+__global__ __launch_bounds__(256) void mfma_f32_peak_kernel(int iters, float* sink)
+{
+	v16f acc0 = {}, acc1 = {}, acc2 = {}, acc3 = {};
+	float a = (float)threadIdx.x, b = (float)blockIdx.x;
+	for (int i = 0; i < iters; i++) {
+		acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc0, 0, 0, 0);
+		acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc1, 0, 0, 0);
+		acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc2, 0, 0, 0);
+		acc3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc3, 0, 0, 0);
+	}
+	float s = 0;
+	for (int r = 0; r < 16; r++) s += acc0[r] + acc1[r] + acc2[r] + acc3[r];
+	if (s == 12345.678f) *sink = s;
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, uint64_t n16)
+{
+	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256) dst[i] = src[i];
+}
+
+static double g_last_cycles_per_mfma = 0.0, g_last_shader_mhz = 0.0;
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+// kind 0: int8 32x32x32 MFMA, result in tera-ops/s.  kind 1: fp32 32x32x2 MFMA, result in TFLOP/s.
+int lten_hip_measure_mfma_peak(int kind, int waves_per_simd, float* tera_per_s)
+{
+	LTEN_HIP_REQUIRE(tera_per_s != nullptr && (kind == 0 || kind == 1) && waves_per_simd >= 1 && waves_per_simd <= 8, "measure_mfma_peak: bad argument");
+	hipDeviceProp_t prop;
+	int dev = 0;
+	LTEN_HIP_CHECK(hipGetDevice(&dev));
+	LTEN_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+	const int blocks = prop.multiProcessorCount * waves_per_simd;  // 4 waves per block = 1 per SIMD
+	const int iters = kind == 0 ? 4096 : 2048;
+	void* sink = nullptr;
+	LTEN_HIP_CHECK(hipMalloc(&sink, 64));
+	hipEvent_t e0, e1;
+	LTEN_HIP_CHECK(hipEventCreate(&e0));
+	LTEN_HIP_CHECK(hipEventCreate(&e1));
+	float best = 1e30f;
+	for (int rep = 0; rep < 4; rep++) {
+		LTEN_HIP_CHECK(hipEventRecord(e0, stream()));
+		if (kind == 0)
+			mfma_i8_peak_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<int*>(sink), static_cast<long long*>(sink) + 1);
+		else
+			mfma_f32_peak_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<float*>(sink));
+		LTEN_HIP_CHECK(hipEventRecord(e1, stream()));
+		LTEN_HIP_CHECK(hipEventSynchronize(e1));
+		float ms = 0;
+		LTEN_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+		if (rep > 0 && ms < best) best = ms;
+	}
+	const double ops_per_mfma = kind == 0 ? 2.0 * 32 * 32 * 32 : 2.0 * 32 * 32 * 2;
+	*tera_per_s = (float)(ops_per_mfma * 4.0 * iters * 4.0 * blocks / (best * 1e-3) / 1e12);
+	if (kind == 0) {
+		long long clk[2] = { 0, 0 };
+		LTEN_HIP_CHECK(hipMemcpy(clk, static_cast<long long*>(sink) + 1, sizeof(clk), hipMemcpyDeviceToHost));
+		g_last_cycles_per_mfma = (double)clk[0] / (4.0 * iters);
+		g_last_shader_mhz = clk[1] > 0 ? (double)clk[0] / ((double)clk[1] / 100.0) : 0.0;
+	}
+	hipEventDestroy(e0);
+	hipEventDestroy(e1);
+	LTEN_HIP_CHECK(hipFree(sink));
+	return 0;
+}
+
+// After lten_hip_measure_mfma_peak(0, ...): shader clocks per int8 32x32x32 MFMA as seen by one wavefront,
+// and the shader clock rate in MHz over that loop (shader clock counter against the 100 MHz wall clock).
+int lten_hip_measure_last_clocks(double* cycles_per_mfma, double* shader_mhz)
+{
+	if (cycles_per_mfma) *cycles_per_mfma = g_last_cycles_per_mfma;
+	if (shader_mhz) *shader_mhz = g_last_shader_mhz;
+	return 0;
+}
+
+// Copies `bytes` (a multiple of 16) from src to dst with 16-byte accesses: 2 * bytes of HBM traffic.
+int lten_hip_copy_kernel(const void* src, void* dst, uint64_t bytes)
+{
+	LTEN_HIP_REQUIRE((bytes & 15) == 0 && ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) == 0,
+	                 "copy_kernel: size and pointers must be multiples of 16");
+	if (bytes == 0) return 0;
+	const uint64_t n16 = bytes / 16;
+	const unsigned blocks = (unsigned)std::min<uint64_t>(ceil_div(n16, 256), 256 * 32);
+	copy_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(static_cast<const v4i*>(src), static_cast<v4i*>(dst), n16);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+}  // extern "C"

@@ -22,48 +22,9 @@
 // buffer run), rows of BK bytes with a 16-byte-chunk XOR swizzle that keeps the
 // ds_read_b128 operand fetches bank-conflict free.
 #include "common.h"
+#include "qgemm_common.h"
 
 namespace lten_hip {
-
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef int v16i __attribute__((ext_vector_type(16)));
-
-enum QOut { Q_OUT_U8_FAST = 0, Q_OUT_U8_EXACT = 1, Q_OUT_ACC = 2 };
-
-struct QProblem {
-	const uint8_t* A;  // element (m, k) at A[m * a_rs + k * a_ks]
-	const uint8_t* B;  // element (n, k) at B[n * b_rs + k * b_ks]
-	void* C;           // uint8 [M x N] or int32 [M x N], row-major, ld = N
-	int64_t a_rs, a_ks, b_rs, b_ks;
-	int M, N, K;
-	const int32_t* rterm;  // [M] (128 - zpB) * SA_m, or null
-	const int32_t* cterm;  // [N] (128 - zpA) * SB_n + bias_n, or null
-	int32_t konst;         // K (zpA zpB - 16384)
-	float mult;            // real_multiplier
-	float zp_c;            // (float) output zero point
-	int vec_ok;            // operand bases and row strides are multiples of 16 bytes
-};
-
-// 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).
-// Chosen so that any aligned group of 8 or of 16 consecutive rows, read at one logical
-// chunk, touches every LDS bank group once (both for 32 and for 64 four-byte banks).
-template <int CPR>
-__device__ __forceinline__ int swz(int row)
-{
-	if (CPR == 2) return ((row >> 2) ^ (row >> 3)) & 1;
-	if (CPR == 4) return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1);
-	if (CPR == 8) return ((row ^ (row >> 3)) & 1) | (row & 6);
-	return 0;
-}
-
-__device__ __forceinline__ v4i flip_sign_bits(v4i v)
-{
-	v.x ^= 0x80808080;
-	v.y ^= 0x80808080;
-	v.z ^= 0x80808080;
-	v.w ^= 0x80808080;
-	return v;
-}
 
 // One 16-byte chunk of an operand tile, raw bytes (before the XOR), as four dwords.
 // Out-of-range bytes read as 0x80, which becomes 0 after the XOR.
@@ -91,22 +52,6 @@ __device__ __forceinline__ v4i load_chunk(const uint8_t* base, int64_t rs, int64
 		}
 		return v;
 	}
-}
-
-// Exact image of l-ten/math_fns.cpp:1474 for one accumulator.
-template <int OUT>
-__device__ __forceinline__ unsigned requant(int acc, float mult, float zp)
-{
-	// Two separately rounded operations: a fused multiply-add rounds once and differs in the last bit.
-#pragma clang fp contract(off)
-	float prod = (float)acc * mult;
-	float s = prod + zp;
-	if (OUT == Q_OUT_U8_EXACT) {
-		// x86 cvttss2si: NaN and anything outside [-2^31, 2^31) give 0x80000000.
-		int i = (s >= -2147483648.0f && s < 2147483648.0f) ? (int)s : (int)0x80000000;
-		return (unsigned)i & 0xFFu;
-	}
-	return (unsigned)(int)s & 0xFFu;  // caller guarantees |s| < 2^31
 }
 
 template <int BM, int BN, int BK, int WM, int WN, bool GUARD, int OUT>
@@ -370,6 +315,9 @@ static int qgemm_dispatch(const QProblem& p, int out)
 	const uint64_t out_elems = (uint64_t)p.M * p.N;
 	int choice = get_option(OPT_QGEMM_TILE);  // 0 = heuristic
 	if (choice == 0) {
+		// Large problems that tile exactly go to the direct-to-LDS 256x256x128 kernel; it wants enough tiles
+		// to occupy most CUs and a K long enough to amortise its prologue and epilogue.
+		if (out_elems >= 256ull * 256 * 128 && p.K >= 512 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
 		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
 			choice = 1;
 		else if (fits(128, 128, 64) && out_elems >= 128ull * 128 * 128)
@@ -378,6 +326,11 @@ static int qgemm_dispatch(const QProblem& p, int out)
 			choice = 3;
 		else
 			choice = 4;
+	}
+	if (choice >= 20) {
+		const int rc = qgemm_fast_dispatch(p, out, choice);
+		LTEN_HIP_REQUIRE(rc >= 0, "qgemm: forced fast variant %d does not fit this problem", choice);
+		return rc;
 	}
 	switch (choice) {
 	case 1:
@@ -388,6 +341,16 @@ static int qgemm_dispatch(const QProblem& p, int out)
 		return launch_tile<128, 128, 64, 2, 2, false>(p, out, "qgemm_nt_128x128x64");
 	case 3:
 		return launch_tile<64, 64, 64, 2, 2, true>(p, out, "qgemm_guard_64x64x64");
+#ifdef LTEN_HIP_TUNING_VARIANTS
+	case 11: return launch_tile<256, 256, 64, 2, 4, false>(p, out, "x_256x256x64_w2x4");
+	case 12: return launch_tile<256, 256, 64, 4, 2, false>(p, out, "x_256x256x64_w4x2");
+	case 13: return launch_tile<256, 256, 128, 2, 2, false>(p, out, "x_256x256x128_w2x2");
+	case 14: return launch_tile<256, 256, 128, 2, 4, false>(p, out, "x_256x256x128_w2x4");
+	case 15: return launch_tile<256, 128, 64, 2, 2, false>(p, out, "x_256x128x64_w2x2");
+	case 16: return launch_tile<128, 256, 64, 2, 2, false>(p, out, "x_128x256x64_w2x2");
+	case 17: return launch_tile<256, 128, 128, 2, 2, false>(p, out, "x_256x128x128_w2x2");
+	case 18: return launch_tile<256, 256, 32, 2, 2, false>(p, out, "x_256x256x32_w2x2");
+#endif
 	default:
 		return launch_tile<32, 32, 64, 1, 1, true>(p, out, "qgemm_guard_32x32x64");
 	}
@@ -423,6 +386,10 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	volatile float ab = qp[0].scale * qp[1].scale;
 	p.mult = ab / qp[2].scale;
 	p.zp_c = (float)qp[2].zero_point;
+	p.stamps = nullptr;
+#ifdef LTEN_HIP_STAMPS
+	if (workspace) p.stamps = reinterpret_cast<long long*>(workspace + ((M + N + 3) & ~3ull));
+#endif
 	p.vec_ok = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (K & 15) == 0 &&
 	           p.a_ks == 1 && p.b_ks == 1;
 

@@ -1,0 +1,71 @@
+// Definitions shared by the int8 GEMM kernels: the problem descriptor handed to every kernel, the LDS
+// chunk swizzle and the requantize step.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <cstdint>
+
+namespace lten_hip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+enum QOut { Q_OUT_U8_FAST = 0, Q_OUT_U8_EXACT = 1, Q_OUT_ACC = 2 };
+
+struct QProblem {
+	const uint8_t* A;  // element (m, k) at A[m * a_rs + k * a_ks]
+	const uint8_t* B;  // element (n, k) at B[n * b_rs + k * b_ks]
+	void* C;           // uint8 [M x N] or int32 [M x N], row-major, ld = N
+	int64_t a_rs, a_ks, b_rs, b_ks;
+	int M, N, K;
+	const int32_t* rterm;  // [M] (128 - zpB) * SA_m, or null
+	const int32_t* cterm;  // [N] (128 - zpA) * SB_n + bias_n, or null
+	int32_t konst;         // K (zpA zpB - 16384)
+	float mult;            // real_multiplier
+	float zp_c;            // (float) output zero point
+	int vec_ok;            // operand bases and row strides are multiples of 16 bytes
+	long long* stamps;     // tuning builds only: per-workgroup phase timestamps, else null
+};
+
+// 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).
+// Chosen so that any aligned group of 8 or of 16 consecutive rows, read at one logical
+// chunk, touches every LDS bank group once (both for 32 and for 64 four-byte banks).
+template <int CPR>
+__device__ __forceinline__ int swz(int row)
+{
+	if (CPR == 2) return ((row >> 2) ^ (row >> 3)) & 1;
+	if (CPR == 4) return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1);
+	if (CPR == 8) return ((row ^ (row >> 3)) & 1) | (row & 6);
+	return 0;
+}
+
+__device__ __forceinline__ v4i flip_sign_bits(v4i v)
+{
+	v.x ^= 0x80808080;
+	v.y ^= 0x80808080;
+	v.z ^= 0x80808080;
+	v.w ^= 0x80808080;
+	return v;
+}
+
+// Exact image of l-ten/math_fns.cpp:1474 for one accumulator.
+template <int OUT>
+__device__ __forceinline__ unsigned requant(int acc, float mult, float zp)
+{
+	// Two separately rounded operations: a fused multiply-add rounds once and differs in the last bit.
+#pragma clang fp contract(off)
+	float prod = (float)acc * mult;
+	float s = prod + zp;
+	if (OUT == Q_OUT_U8_EXACT) {
+		// x86 cvttss2si: NaN and anything outside [-2^31, 2^31) give 0x80000000.
+		int i = (s >= -2147483648.0f && s < 2147483648.0f) ? (int)s : (int)0x80000000;
+		return (unsigned)i & 0xFFu;
+	}
+	return (unsigned)(int)s & 0xFFu;  // caller guarantees |s| < 2^31
+}
+
+
+// Dispatch of the tuned square-ish kernels (qgemm_fast.hip).  Returns -1 when no fast variant fits.
+int qgemm_fast_dispatch(const QProblem& p, int out, int variant);
+
+}  // namespace lten_hip

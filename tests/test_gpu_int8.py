@@ -67,6 +67,30 @@ def test_fast_tiles(gpu, ob, tile, shape):
                  bias=rng.integers(-5000, 5000, N).astype(np.int32) if zp[0] else None, tile=tile)
 
 
+@pytest.mark.parametrize("variant", [21, 23, 24, 26, 28, 31, 33, 34])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 640), (256, 1024, 2048)])
+def test_direct_to_lds_tiles(gpu, ob, variant, shape):
+    """The tuned 256x256 tiles (LDS stage ring filled by direct global->LDS loads): every wave layout, both
+    k-step sizes, with and without zero-point terms and bias, short and long K (prologue/drain paths)."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + variant)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=variant)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8),
+             bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
+
+
+def test_requantize_exact_epilogue_in_tiled_kernels(gpu, ob):
+    """Multipliers above 1 select the epilogue that spells out the x86 conversion (out-of-range -> 0x80000000)."""
+    rng = np.random.default_rng(4)
+    A = rng.integers(0, 256, (256, 256), dtype=np.uint8)
+    B = rng.integers(0, 256, (256, 256), dtype=np.uint8)
+    for scales in ([300.0, 500.0, 1.0], [1.0, 1.0, 1e-6]):
+        for tile in (0, 1, 3, 31):
+            run_case(gpu, ob, A, B, scales, np.array([128, 128, 9], np.uint8), tile=tile)
+
+
 @pytest.mark.parametrize("tA,tB", [(0, 0), (1, 0), (1, 1)])
 def test_other_transpose_modes(gpu, ob, tA, tB):
     rng = np.random.default_rng(77 + tA * 2 + tB)
@@ -124,7 +148,7 @@ def test_cfg3_full_size_properties(gpu, wl):
     ws = gpu.DeviceBuffer(4 * (M + N))
     qp = gpu.qparams3(sc, zp)
     gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
-    assert gpu.last_kernel() == "qgemm_nt_256x256x64"
+    assert gpu.last_kernel().startswith("qgemm_fast_256x256x128")
     gpu.quantized_matmul_acc(False, True, M, N, K, dA, dB, dacc, qp, None, ws)
     acc = dacc.numpy(np.int32, (M, N))
     want = exact_acc(X, W, int(zp[0]), int(zp[1]))
