@@ -3,11 +3,14 @@
 
 A step is one lten_hip_quantized_matmul call (the whole FC forward: MFMA GEMM with the
 zero-point correction and the requantize fused in) over one synthetic batch whose operands
-are already resident in HBM.  Prints ONE JSON line.
+are already resident in HBM.  Prints ONE JSON line.  The headline fields describe config 3;
+"configs" adds one record per other benchmark configuration (1, 2, 4, 5), each with its own
+roofline figure and the CPU path timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra]
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -22,38 +25,217 @@ if ROOT not in sys.path:
 from __graft_entry__ import load_package  # noqa: E402
 
 INT8_MFMA_PEAK_TOPS = 5000.0   # MI355X dense int8 MFMA, published: 5.0 POP/s
+FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 MFMA, published
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published: 8 TB/s
 
-# HBM bytes per launch of the dominant kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs,
-# scaled by the same counters on a plain copy kernel; None until such a run is on file under profiles/.
-TRAFFIC_BYTES = {"qgemm_nt_256x256x64": None}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the
+# same counters on the plain copy kernel (profiles/qgemm_fast_cfg3_4096.md): FETCH_SIZE reads half the bytes
+# the copy kernel is known to fetch (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
+TRAFFIC_BYTES = {"qgemm_fast_256x256x128_w2x4_s2": 49250 * 1024 * 2.0 + 16384 * 1024 * 1.0}
+
+
+def timed(lt, fn, iters, warmup=3):
+    """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on the library's stream)."""
+    for _ in range(warmup):
+        fn()
+    lt.sync()
+    t = lt.Timer()
+    t.start()
+    for _ in range(iters):
+        fn()
+    return t.stop_ms() / iters
+
+
+def best_of(fn, reps):
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def cpu_int8(ob, X, W, sc, zp, rows=None):
+    ref = ob.ref()
+    A = np.ascontiguousarray(X if rows is None else X[:rows])
+    t0 = time.perf_counter()
+    if ref is not None:
+        ob.ref_quantized_matmul(A, W, sc, zp)
+    else:
+        ob.quantized_matmul(A, W, sc, zp, want_acc=False)
+    return time.perf_counter() - t0, ("reference" if ref is not None else "port")
 
 
 def cpu_baseline(X, W, sc, zp, budget_s=15.0):
     """l-ten's own quantized_matmul (compiled reference) or, where that library is absent, the C port,
     on the first rows of the same workload, single thread as in l-ten."""
     from oracle import bindings as ob
-    ref = ob.ref()
     N, K = W.shape
-
-    def run(rows):
-        A = np.ascontiguousarray(X[:rows])
-        t0 = time.perf_counter()
-        if ref is not None:
-            ob.ref_quantized_matmul(A, W, sc, zp)
-        else:
-            ob.quantized_matmul(A, W, sc, zp, want_acc=False)
-        return time.perf_counter() - t0
-
     probe_rows = 16
-    t_probe = run(probe_rows)
+    t_probe, kind = cpu_int8(ob, X, W, sc, zp, probe_rows)
     rows = int(min(X.shape[0], max(probe_rows, budget_s / max(t_probe, 1e-6) * probe_rows)))
     rows = max(16, rows // 16 * 16)
-    t = run(rows)
+    t, kind = cpu_int8(ob, X, W, sc, zp, rows)
     tops = 2.0 * rows * N * K / t / 1e12
-    return {"value": tops, "unit": "TOPS", "cores": 1, "kind": "reference" if ref is not None else "port",
+    return {"value": tops, "unit": "TOPS", "cores": 1, "kind": kind,
             "sample": f"first {rows} of {X.shape[0]} activation rows against the full {N}x{K} weight matrix "
                       f"({t:.1f} s single-threaded quantized_matmul)"}
+
+
+def cpu_sgemm(ob, tA, tB, M, N, K, A, B, Cm, beta, threads):
+    """One fp32 GEMM on the CPU path: l-ten's cpu_gemm<float> (threadpool + AVX build) where compiled, else the port."""
+    ref = ob.ref()
+    if ref is not None and (N < 16 or N % 8 == 0):
+        rc = ref.ref_cpu_gemm_f32(int(tA), int(tB), M, N, K, 1.0, A.reshape(-1), B.reshape(-1), beta, Cm.reshape(-1))
+        assert rc == 0
+        return "reference"
+    ob.oracle().oracle_sgemm_mt(int(tA), int(tB), M, N, K, 1.0, A.reshape(-1), M if tA else K, B.reshape(-1),
+                                K if tB else N, beta, Cm.reshape(-1), N, threads)
+    return "port"
+
+
+def extra_configs(lt, wl, with_cpu):
+    """Configs 1, 2, 4, 5: GPU time per pass (HIP events), rate against the bound that applies, CPU path beside it."""
+    from oracle import bindings as ob
+    D = lt.DeviceBuffer
+    l = lt.lib()
+    threads = os.cpu_count() or 1
+    if ob.ref() is not None:
+        threads = int(ob.ref().ref_hardware_threads())
+    out = []
+
+    # ---- config 1: int8 FC 64x512x784 (latency bound)
+    X, W, sc, zp = wl.cfg1()
+    M, K = X.shape
+    N = W.shape[0]
+    dA, dB, dC, ws, qp = D.from_numpy(X), D.from_numpy(W), D(M * N), D(4 * (M + N)), lt.qparams3(sc, zp)
+    ms = timed(lt, lambda: lt.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws), 200)
+    rec = {"config": "cfg1 int8 FC 64x512x784 (zero point 0, zero-point row-sum correction active)", "gpu_us": round(ms * 1e3, 2),
+           "kernel": lt.last_kernel(), "gops": round(2.0 * M * N * K / ms / 1e6, 1), "bound": "launch latency",
+           "algorithmic_bytes": M * K + N * K + M * N}
+    if with_cpu:
+        t = min(cpu_int8(ob, X, W, sc, zp)[0] for _ in range(5))
+        rec.update(cpu_ms=round(t * 1e3, 3), cpu_cores=1, cpu_kind=cpu_int8(ob, X, W, sc, zp)[1], speedup=round(t * 1e3 / ms, 1))
+    out.append(rec)
+
+    # ---- config 4: skinny weight streaming, M in {1, 4, 16}, K = N = 8192 (HBM bound)
+    for M in (1, 4, 16):
+        X, W, sc, zp = wl.cfg4(M)
+        N, K = W.shape
+        dA, dB, dC, ws, qp = D.from_numpy(X), D.from_numpy(W), D(M * N), D(4 * (M + N)), lt.qparams3(sc, zp)
+        ms = timed(lt, lambda: lt.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws), 100)
+        nbytes = N * K + M * K + M * N
+        gbs = nbytes / ms / 1e6
+        rec = {"config": f"cfg4 int8 FC skinny M={M} K=N=8192", "gpu_us": round(ms * 1e3, 2), "kernel": lt.last_kernel(),
+               "algorithmic_bytes": nbytes,
+               "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                            "frac": round(gbs / HBM_PEAK_GBS, 4)}}
+        if with_cpu:
+            t, kind = cpu_int8(ob, X, W, sc, zp)
+            rec.update(cpu_ms=round(t * 1e3, 2), cpu_cores=1, cpu_kind=kind, speedup=round(t * 1e3 / ms, 1))
+        out.append(rec)
+        del dA, dB, dC, ws
+
+    # ---- config 2: fp32 MLP 784-1024-1024-10, batch 128: 3 forward GEMMs with bias, 3 data-gradient GEMMs,
+    # 3 weight-gradient GEMMs, 3 bias-gradient column sums.  The element-wise pieces between them (ReLU, loss) are
+    # outside this path, so the timed chain feeds each GEMM from resident buffers of the right shape.
+    X, Ws, bs, labels = wl.cfg2()
+    B_ = X.shape[0]
+    sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
+    acts = [D.from_numpy(X)] + [D(4 * B_ * n) for n in sizes[1:]]
+    grads = [D(4 * B_ * n, zero=True) for n in sizes]
+    dWs, dbs = [D.from_numpy(w) for w in Ws], [D.from_numpy(b) for b in bs]
+    gWs, gbs_ = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
+    lt.check(l.lten_hip_fill_f32(grads[-1].ptr, B_ * sizes[-1], 0.01))
+
+    def mlp_step():
+        for i in range(3):
+            lt.check(l.lten_hip_fc_forward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, dbs[i].ptr, acts[i + 1].ptr))
+        for i in (2, 1, 0):
+            lt.check(l.lten_hip_fc_backward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, grads[i + 1].ptr,
+                                                grads[i].ptr, gWs[i].ptr, gbs_[i].ptr))
+    ms = timed(lt, mlp_step, 100)
+    flops = sum(3 * 2.0 * B_ * sizes[i] * sizes[i + 1] for i in range(3))
+    tf = flops / ms / 1e9
+    rec = {"config": "cfg2 fp32 MLP 784-1024-1024-10 batch 128, forward + backward GEMMs (9 GEMMs, 3 bias adds fused, 3 column sums)",
+           "gpu_us": round(ms * 1e3, 2), "gflop_per_step": round(flops / 1e9, 3),
+           "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)},
+           "note": "twelve small launches; launch latency, not the MFMA rate, sets this time"}
+    if with_cpu:
+        hA = [np.random.default_rng(i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
+        hG = [np.random.default_rng(9 + i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
+        kinds = set()
+
+        def cpu_step():
+            for i in range(3):
+                kinds.add(cpu_sgemm(ob, 0, 1, B_, sizes[i + 1], sizes[i], hA[i], Ws[i], hA[i + 1], 0.0, threads))
+            for i in (2, 1, 0):
+                kinds.add(cpu_sgemm(ob, 0, 0, B_, sizes[i], sizes[i + 1], hG[i + 1], Ws[i], hG[i], 0.0, threads))
+                dw = np.empty_like(Ws[i])
+                kinds.add(cpu_sgemm(ob, 1, 0, sizes[i + 1], sizes[i], B_, hG[i + 1], hA[i], dw, 0.0, threads))
+        cpu_step()
+        t = best_of(cpu_step, 5)
+        rec.update(cpu_ms=round(t * 1e3, 2), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)), speedup=round(t * 1e3 / ms, 1),
+                   cpu_note="l-ten's own threadpool + AVX cpu_gemm (its non-OpenBLAS build); bias rank-1 and column-sum GEMMs left out of the CPU leg")
+    out.append(rec)
+    del acts, grads, dWs, dbs, gWs, gbs_
+
+    # ---- config 5: Conv2d 3x3 s1 p1, 32x1x128x128 -> 32 ch -> 64 ch: forward + weight gradient of both layers
+    x, cws, dyshapes = wl.cfg5()
+    Nimg, H, Wd = x.shape[0], x.shape[2], x.shape[3]
+    chans = [x.shape[1]] + [w.shape[0] for w in cws]
+    dx = [D.from_numpy(x)] + [D(4 * Nimg * c * H * Wd) for c in chans[1:]]
+    dw_ = [D.from_numpy(w) for w in cws]
+    ddy = [D.from_numpy(wl.cfg5_dy(s, layer=i)) for i, s in enumerate(dyshapes)]
+    ddw = [D(w.nbytes) for w in cws]
+    geos = [(Nimg, chans[i], H, Wd, chans[i + 1], 3, 3, 1, 1, 1, 1) for i in range(2)]
+    wss = [D(max(int(l.lten_hip_conv2d_wgrad_workspace_bytes(*g)), 4)) for g in geos]
+    for i, g in enumerate(geos):
+        Cin, Cout = g[1], g[4]
+        fl = 2.0 * Nimg * Cout * H * Wd * Cin * 9
+        ms_f = timed(lt, lambda: lt.check(l.lten_hip_conv2d_forward_f32(*g, dx[i].ptr, dw_[i].ptr, None, dx[i + 1].ptr)), 30)
+        kf = lt.last_kernel()
+        ms_w = timed(lt, lambda: lt.check(l.lten_hip_conv2d_wgrad_f32(*g, dx[i].ptr, ddy[i].ptr, ddw[i].ptr, wss[i].ptr)), 30)
+        kw = lt.last_kernel()
+        in_b, out_b = 4 * Nimg * Cin * H * Wd, 4 * Nimg * Cout * H * Wd
+        rec = {"config": f"cfg5 Conv2d layer {i + 1}: {Cin}->{Cout} ch 3x3 s1 p1 on 32x{Cin}x128x128, forward + weight gradient",
+               "forward_us": round(ms_f * 1e3, 1), "wgrad_us": round(ms_w * 1e3, 1), "kernels": [kf, kw],
+               "gflop": round(2 * fl / 1e9, 2)}
+        if Cin * 9 >= 64:
+            tf = 2 * fl / (ms_f + ms_w) / 1e9
+            rec["roofline"] = {"bound": "mfma", "achieved": round(tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                               "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}
+        else:
+            gbs = 2.0 * (in_b + out_b) / (ms_f + ms_w) / 1e6
+            rec["roofline"] = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                               "frac": round(gbs / HBM_PEAK_GBS, 4), "algorithmic_bytes": 2 * (in_b + out_b)}
+        if with_cpu:
+            # l-ten's own loop (im2col + cpu_gemm per image) on the first 2 images, scaled to 32
+            sample = 2
+            Kc, HW = Cin * 9, H * Wd
+            xin = x if i == 0 else np.random.default_rng(3).standard_normal((sample, Cin, H, Wd)).astype(np.float32)
+            wmat = np.ascontiguousarray(cws[i].reshape(Cout, Kc))
+            dyh = wl.cfg5_dy((sample, Cout, H, Wd), layer=i)
+            col = np.empty((Kc, HW), np.float32)
+            yimg = np.empty((Cout, HW), np.float32)
+            dwh = np.zeros((Cout, Kc), np.float32)
+            kinds = set()
+            im2col = ob.ref().ref_im2col_f32 if ob.ref() is not None else ob.oracle().oracle_im2col_f32
+
+            def cpu_pass():
+                for n in range(sample):
+                    im2col(xin[n].reshape(-1), Cin, H, Wd, 3, 3, 1, 1, 1, 1, col.reshape(-1))
+                    kinds.add(cpu_sgemm(ob, 0, 0, Cout, HW, Kc, wmat, col, yimg, 0.0, threads))
+                for n in range(sample):
+                    im2col(xin[n].reshape(-1), Cin, H, Wd, 3, 3, 1, 1, 1, 1, col.reshape(-1))
+                    kinds.add(cpu_sgemm(ob, 0, 1, Cout, Kc, HW, np.ascontiguousarray(dyh[n].reshape(Cout, HW)), col, dwh, 1.0, threads))
+            cpu_pass()
+            t = best_of(cpu_pass, 2) * (Nimg / sample)
+            rec.update(cpu_ms=round(t * 1e3, 1), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)),
+                       cpu_sample=f"{sample} of {Nimg} images, scaled", speedup=round(t * 1e3 / (ms_f + ms_w), 1))
+        out.append(rec)
+    return out
 
 
 def main():
@@ -61,8 +243,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run output check")
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-config records for configs 1, 2, 4, 5")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (the path has no collective to scale); use --gpus 1")
@@ -107,6 +290,9 @@ def main():
         want = (np.trunc(s).astype(np.int64) & 0xFF).astype(np.uint8)
         verified = bool(np.array_equal(dC.numpy(np.uint8, (M, N)), want))
 
+    measured_peak = lt.measure_mfma_peak(0, 1)
+    _, shader_mhz = lt.measure_last_clocks()
+
     out = {
         "metric": "int8_fc_forward_tops_4096",
         "value": round(value, 2),
@@ -125,12 +311,18 @@ def main():
                    "M": M, "N": N, "K": K, "input_digest": wl.digest(X, W)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": TRAFFIC_BYTES.get(kernel),
-                     "kernel": kernel, "kernel_us": round(kernel_ms * 1e3, 2),
-                     "note": "int8 multiply-add counted as 2 ops; achieved/peak in tera-ops per second"},
+                     "kernel": kernel, "kernel_us": round(kernel_ms * 1e3, 2), "algorithmic_bytes": 3 * M * N,
+                     "measured_mfma_only_tops": round(measured_peak, 1), "measured_mfma_only_shader_mhz": round(shader_mhz),
+                     "frac_of_measured_mfma_only": round(achieved / measured_peak, 4),
+                     "note": "int8 multiply-add counted as 2 ops; achieved/peak in tera-ops per second; "
+                             "measured_mfma_only = a kernel that issues nothing but 32x32x32 int8 MFMAs"},
         "verified_bit_exact": verified,
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, W, sc, zp)
+    del dA, dB, dC, ws
+    if not args.no_extra:
+        out["configs"] = extra_configs(lt, wl, not args.no_cpu)
     print(json.dumps(out), flush=True)
 
 

@@ -393,6 +393,22 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	p.vec_ok = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (K & 15) == 0 &&
 	           p.a_ks == 1 && p.b_ks == 1;
 
+	int out = Q_OUT_ACC;
+	if (!out_acc) {
+		// |mult * acc + zp| < 2^31 for every int32 acc  <=>  the saturating GPU convert and the
+		// x86 convert agree; otherwise take the epilogue that spells out the x86 behaviour.
+		const float m = p.mult;
+		out = (m == m && (m < 0 ? -m : m) <= 0.99f) ? Q_OUT_U8_FAST : Q_OUT_U8_EXACT;
+	}
+
+	// skinny activations: one streaming pass over the weights (option "qskinny": 0 = auto, 2 = off)
+	p.cterm = nullptr;
+	p.rterm = nullptr;
+	if (M <= 16 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
+		if (rc >= 0) return rc;
+	}
+
 	const int coef_a = 128 - zpB, coef_b = 128 - zpA;
 	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {
 		LTEN_HIP_REQUIRE(workspace != nullptr, "quantized_matmul: workspace is null");
@@ -401,17 +417,6 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		const unsigned blocks = (unsigned)ceil_div(M + N, 4);
 		qgemm_terms_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(p, coef_a, coef_b, bias, workspace + N, workspace);
 		LTEN_HIP_LAUNCH_CHECK();
-	} else {
-		p.cterm = nullptr;
-		p.rterm = nullptr;
-	}
-
-	int out = Q_OUT_ACC;
-	if (!out_acc) {
-		// |mult * acc + zp| < 2^31 for every int32 acc  <=>  the saturating GPU convert and the
-		// x86 convert agree; otherwise take the epilogue that spells out the x86 behaviour.
-		const float m = p.mult;
-		out = (m == m && (m < 0 ? -m : m) <= 0.99f) ? Q_OUT_U8_FAST : Q_OUT_U8_EXACT;
 	}
 	return qgemm_dispatch(p, out);
 }

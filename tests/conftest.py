@@ -53,6 +53,7 @@ def gpu(lt):
     lt.init(0)
     yield lt
     lt.set_option("qgemm_tile", 0)
+    lt.set_option("qskinny", 0)
 
 
 @pytest.fixture(autouse=True)

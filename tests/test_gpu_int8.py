@@ -160,11 +160,33 @@ def test_cfg3_full_size_properties(gpu, wl):
     assert 0.03 < ((s < 0) | (s >= 256)).mean() < 0.25   # some outputs wrap, most do not
 
 
+@pytest.mark.parametrize("shape", [(1, 16, 2048), (4, 48, 4096), (7, 160, 8192), (16, 64, 8192), (13, 32, 2048)])
+def test_weight_streaming_kernel(gpu, ob, shape):
+    """M <= 16: the streaming kernel with in-kernel zero-point sums, every combination of needed terms,
+    checked against the oracle and against the tiled kernels (option qskinny = 2 switches it off)."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    for zp in ([128, 128, 128], [3, 128, 9], [128, 200, 0], [17, 250, 100]):
+        bias = rng.integers(-9999, 9999, N).astype(np.int32) if zp[0] != 128 else None
+        Cg = run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array(zp, np.uint8), bias=bias)
+        assert gpu.last_kernel().startswith("qskinny_mfma")
+        gpu.set_option("qskinny", 2)
+        try:
+            Ct = run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array(zp, np.uint8), bias=bias)
+            assert not gpu.last_kernel().startswith("qskinny")
+        finally:
+            gpu.set_option("qskinny", 0)
+        assert np.array_equal(Cg, Ct)
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_cfg4_skinny(gpu, wl, M):
     X, W, sc, zp = wl.cfg4(M)
     N = K = 8192
     Cg, accg = gpu.qgemm_host(X, W, sc, zp, want_acc=True)
+    assert gpu.last_kernel() == "qskinny_mfma_w8_k1024"
     want = exact_acc(X, W, int(zp[0]), int(zp[1]))
     assert np.array_equal(accg, want)
     mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
