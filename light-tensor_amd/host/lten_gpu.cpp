@@ -1,0 +1,602 @@
+// See lten_gpu.h.  Every GPU branch is a call through the C ABI of liblten_hip (include/lten_hip.h);
+// the l-ten source line each one stands in for is cited beside it.
+#include "lten_gpu.h"
+
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <random>
+
+#include "../../include/lten_hip.h"
+
+namespace lten {
+
+// ------------------------------------------------------------------------------ errors
+
+ExceptionInfo::ExceptionInfo(const char* msg, const char* file, const char* func, int line)
+{
+	char buf[1024];
+	snprintf(buf, sizeof(buf), "%s [%s %s:%d]", msg, func, file, line);
+	text_ = buf;
+}
+
+void ltenFail(const char* msg, const char* file, const char* func, int line)
+{
+	// l-ten prints, then throws (l-ten/error.h:91-93, l-ten/utils.cpp:303-321)
+	fprintf(stderr, "[Error] File: %s Function: %s Line:%d Msg: %s\n", file, func, line, msg);
+	throw ExceptionInfo(msg, file, func, line);
+}
+
+// a non-zero status of the C ABI becomes an l-ten error, message included
+#define LTEN_HIP_CALL(expr)                                  \
+	do {                                                 \
+		if ((expr) != 0) LTEN_ERR(lten_hip_last_error()); \
+	} while (0)
+
+// ------------------------------------------------------------------------------ TensorImpl
+
+static size_t elem_size(dtype t) { return t == UINT8 ? 1 : 4; }
+
+struct TensorImpl {
+	uint64_t dims[MAX_DIMS] = { 0 };
+	int ndims = 0;
+	uint64_t numels = 0;
+	dtype data_type = FLOAT32;
+	device dev = CPU;
+	int dev_index = 0;
+	void* data = nullptr;
+	bool own_data = false;
+	void* grad = nullptr;
+	bool autograd = false;
+	std::vector<std::shared_ptr<TensorImpl>> children;
+	grad_fn_t grad_fn;
+
+	size_t nbytes() const { return numels * elem_size(data_type); }
+
+	static void* alloc(device d, size_t bytes, bool zero)
+	{
+		if (d == CPU) return zero ? calloc(bytes ? bytes : 1, 1) : malloc(bytes ? bytes : 1);
+		void* p = nullptr;
+		LTEN_HIP_CALL(lten_hip_alloc(&p, bytes, zero ? 1 : 0));  // l-ten/utils.cu:30-58 AllocateMemoryOnGPU
+		return p;
+	}
+	static void release(device d, void* p)
+	{
+		if (!p) return;
+		if (d == CPU) free(p);
+		else lten_hip_free(p);  // l-ten/utils.cu:60-71
+	}
+	void ensure_grad()
+	{
+		if (!grad) grad = alloc(dev, nbytes(), true);
+	}
+	~TensorImpl()
+	{
+		if (own_data) release(dev, data);
+		release(dev, grad);
+	}
+};
+
+static std::shared_ptr<TensorImpl> make_impl(const uint64_t* dims, int ndims, void* data, bool own, const TensorOps* ops)
+{
+	if (ndims < 1 || ndims > MAX_DIMS) LTEN_ERR("Invalid number of dimensions");
+	auto t = std::make_shared<TensorImpl>();
+	TensorOps def;
+	if (!ops) ops = &def;
+	t->ndims = ndims;
+	t->numels = 1;
+	for (int i = 0; i < ndims; i++) {
+		t->dims[i] = dims[i];
+		t->numels *= dims[i];
+	}
+	t->data_type = ops->data_type;
+	t->dev = ops->device_type;
+	t->dev_index = ops->device_index;
+	if (t->dev == GPU) LTEN_HIP_CALL(lten_hip_init(t->dev_index));
+	if (data) {
+		t->data = data;
+		t->own_data = own;
+	} else {
+		t->data = TensorImpl::alloc(t->dev, t->nbytes(), false);
+		t->own_data = true;
+	}
+	if (ops->alloc_gradient_buffer) t->ensure_grad();
+	return t;
+}
+
+// ------------------------------------------------------------------------------ Tensor
+
+void* Tensor::get_data_ptr() { return impl_->data; }
+void* Tensor::get_grad_ptr() { return impl_->grad; }
+uint64_t Tensor::get_numels() const { return impl_->numels; }
+const uint64_t* Tensor::get_sizes() const { return impl_->dims; }
+int Tensor::get_ndims() const { return impl_->ndims; }
+dtype Tensor::get_data_type() const { return impl_->data_type; }
+device Tensor::get_device() const { return impl_->dev; }
+int Tensor::get_device_index() const { return impl_->dev_index; }
+void Tensor::set_autograd(bool setting) { impl_->autograd = setting; }
+
+void Tensor::clear_gradients()
+{
+	if (!impl_->grad) return;
+	if (impl_->dev == CPU) memset(impl_->grad, 0, impl_->nbytes());
+	else LTEN_HIP_CALL(lten_hip_zero(impl_->grad, impl_->nbytes()));  // l-ten/utils.cu:49-52 ZeroMemoryOnGPU
+}
+
+Tensor TensorFromBuffer(const uint64_t* dims_ptr, int ndims, void* data_ptr, bool own_memory, TensorOps* options_ptr)
+{
+	return Tensor(make_impl(dims_ptr, ndims, data_ptr, own_memory, options_ptr));
+}
+Tensor TensorFromBuffer(const std::initializer_list<uint64_t>& dims, void* data_ptr, bool own_memory, TensorOps* options_ptr)
+{
+	return TensorFromBuffer(dims.begin(), (int)dims.size(), data_ptr, own_memory, options_ptr);
+}
+Tensor AllocateTensor(const uint64_t* dims_ptr, int ndims, TensorOps* options_ptr)
+{
+	return TensorFromBuffer(dims_ptr, ndims, nullptr, true, options_ptr);
+}
+Tensor AllocateTensor(const std::initializer_list<uint64_t>& dims, TensorOps* options_ptr)
+{
+	return TensorFromBuffer(dims.begin(), (int)dims.size(), nullptr, true, options_ptr);
+}
+
+static void copy_between(device dst_dev, void* dst, device src_dev, const void* src, size_t bytes)
+{
+	if (bytes == 0) return;
+	if (dst_dev == CPU && src_dev == CPU) memcpy(dst, src, bytes);
+	else if (dst_dev == GPU && src_dev == CPU) LTEN_HIP_CALL(lten_hip_copy_to_gpu(dst, src, bytes));        // l-ten/utils.cu:73-80
+	else if (dst_dev == CPU && src_dev == GPU) LTEN_HIP_CALL(lten_hip_copy_from_gpu(dst, src, bytes));      // l-ten/utils.cu:82-94
+	else LTEN_HIP_CALL(lten_hip_copy_gpu_to_gpu(dst, src, bytes));                                         // l-ten/utils.cu:96-108
+}
+
+Tensor Tensor::to(device target_device, int target_device_index)
+{
+	// l-ten/tensorimpl.cpp:311-412: data and, when present, the gradient buffer move together
+	TensorOps ops;
+	ops.data_type = impl_->data_type;
+	ops.device_type = target_device;
+	ops.device_index = target_device_index;
+	Tensor out = AllocateTensor(impl_->dims, impl_->ndims, &ops);
+	copy_between(target_device, out.impl_->data, impl_->dev, impl_->data, impl_->nbytes());
+	if (impl_->grad) {
+		out.impl_->ensure_grad();
+		copy_between(target_device, out.impl_->grad, impl_->dev, impl_->grad, impl_->nbytes());
+	}
+	out.impl_->autograd = impl_->autograd;
+	return out;
+}
+
+// Where a child's gradient goes: straight into its own (zero-initialised, accumulating) gradient buffer when
+// it is a leaf, into a fresh zeroed buffer when it is an intermediate result that has to be propagated further.
+struct Bottom {
+	std::shared_ptr<TensorImpl> child;
+	float* ptr = nullptr;
+	bool temporary = false;
+	explicit Bottom(const std::shared_ptr<TensorImpl>& c) : child(c)
+	{
+		if (c->grad_fn) {
+			ptr = static_cast<float*>(TensorImpl::alloc(c->dev, c->nbytes(), true));
+			temporary = true;
+		} else {
+			c->ensure_grad();
+			ptr = static_cast<float*>(c->grad);
+		}
+	}
+	void propagate()
+	{
+		if (temporary) {
+			child->grad_fn(*child, ptr);
+			if (child->dev == GPU) LTEN_HIP_CALL(lten_hip_sync());
+			TensorImpl::release(child->dev, ptr);
+			temporary = false;
+		}
+	}
+};
+static bool wants_gradient(const std::shared_ptr<TensorImpl>& c) { return c->autograd || (bool)c->grad_fn; }
+
+void Tensor::backward(const Tensor* top_gradient)
+{
+	if (impl_->data_type != FLOAT32) LTEN_ERR("backward is only supported for FLOAT32 tensors");
+	if (!impl_->grad_fn) return;
+	if (top_gradient) {
+		if (top_gradient->get_numels() != impl_->numels || top_gradient->get_device() != impl_->dev)
+			LTEN_ERR("top gradient must have the shape and device of the tensor");
+		impl_->grad_fn(*impl_, static_cast<const float*>(top_gradient->impl_->data));
+		return;
+	}
+	if (impl_->numels != 1) LTEN_ERR("backward without a top gradient needs a one-element tensor");
+	float one = 1.0f;
+	TensorOps ops;
+	Tensor seed = TensorFromBuffer({ 1 }, &one, false, &ops).to(impl_->dev, impl_->dev_index);
+	impl_->grad_fn(*impl_, static_cast<const float*>(seed.impl_->data));
+}
+
+// ------------------------------------------------------------------------------ matmul
+
+struct BatchPlan {
+	uint64_t count = 1;
+	int64_t stride_a = 0, stride_b = 0, stride_c = 0;
+	bool uniform = true;  // one strided call covers it
+};
+
+static void leading_offsets(const TensorImpl& a, const TensorImpl& b, const uint64_t* cdims, int ndims, std::vector<uint64_t>& oa,
+                            std::vector<uint64_t>& ob)
+{
+	// l-ten/md_array.h:1252-1282: broadcast = coordinate clamped to dim - 1
+	uint64_t count = 1;
+	for (int i = 0; i < ndims - 2; i++) count *= cdims[i];
+	oa.resize(count);
+	ob.resize(count);
+	const uint64_t ma = a.dims[ndims - 2] * a.dims[ndims - 1], mb = b.dims[ndims - 2] * b.dims[ndims - 1];
+	for (uint64_t idx = 0; idx < count; idx++) {
+		uint64_t rem = idx, offa = 0, offb = 0, sa = 1, sb = 1;
+		for (int i = ndims - 3; i >= 0; i--) {
+			const uint64_t c = rem % cdims[i];
+			rem /= cdims[i];
+			offa += (c < a.dims[i] ? c : a.dims[i] - 1) * sa;
+			offb += (c < b.dims[i] ? c : b.dims[i] - 1) * sb;
+			sa *= a.dims[i];
+			sb *= b.dims[i];
+		}
+		oa[idx] = offa * ma;
+		ob[idx] = offb * mb;
+	}
+}
+
+Tensor Tensor::matmul(const Tensor& other)
+{
+	TensorImpl& a = *impl_;
+	TensorImpl& b = *other.impl_;
+	if (a.data_type != b.data_type) LTEN_ERR("Tensor data types must match");                       // l-ten/tensor.h:87-90
+	if (a.data_type != FLOAT32) LTEN_ERR("Not yet implemented");                                    // l-ten/math_fns.cpp:1295-1305
+	if (a.ndims != b.ndims) LTEN_ERR("MultiDimArrays must have the same number of dimensions");    // l-ten/md_array.h:971-974
+	if (a.dev != b.dev || a.dev_index != b.dev_index) LTEN_ERR("Tensors must be on the same device");
+	if (a.ndims < 2) LTEN_ERR("matmul requires at least 2 dimensions");
+	const int nd = a.ndims;
+	if (a.dims[nd - 1] != b.dims[nd - 2]) LTEN_ERR("MultiDimArrays must have compatiple dimensions");  // l-ten/md_array.h:985-988
+	uint64_t cdims[MAX_DIMS];
+	for (int i = 0; i < nd - 2; i++) {
+		if (a.dims[i] != b.dims[i] && a.dims[i] != 1 && b.dims[i] != 1) LTEN_ERR("MultiDimArrays must have compatiple dimensions");
+		cdims[i] = a.dims[i] > b.dims[i] ? a.dims[i] : b.dims[i];
+	}
+	const uint64_t M = a.dims[nd - 2], K = a.dims[nd - 1], N = b.dims[nd - 1];
+	cdims[nd - 2] = M;
+	cdims[nd - 1] = N;
+	if (a.dev != GPU) LTEN_ERR("this build implements matmul for the GPU device type only (l-ten's own CPU path covers lten::CPU)");
+
+	TensorOps ops;
+	ops.device_type = GPU;
+	ops.device_index = a.dev_index;
+	Tensor result = AllocateTensor(cdims, nd, &ops);
+	std::vector<uint64_t> oa, ob;
+	leading_offsets(a, b, cdims, nd, oa, ob);
+	const float* ad = static_cast<const float*>(a.data);
+	const float* bd = static_cast<const float*>(b.data);
+	float* cd = static_cast<float*>(result.impl_->data);
+	// l-ten/md_array_cuda.h:507-515: one NN GEMM per leading index
+	for (size_t i = 0; i < oa.size(); i++)
+		LTEN_HIP_CALL(lten_hip_sgemm(0, 0, M, N, K, 1.0f, ad + oa[i], K, bd + ob[i], N, 0.0f, cd + i * M * N, N));
+
+	auto ai = impl_, bi = other.impl_;
+	result.impl_->children = { ai, bi };
+	result.impl_->autograd = true;
+	result.impl_->grad_fn = [ai, bi, oa, ob, M, N, K](TensorImpl& self, const float* top) {
+		(void)self;
+		// l-ten/backprop.cpp:533-585: per leading index dA += dC B^T (NT), dB += A^T dC (TN), beta = 1 into
+		// zeroed gradients, so a broadcast operand collects the sum over the indices that share it
+		const float* ad = static_cast<const float*>(ai->data);
+		const float* bd = static_cast<const float*>(bi->data);
+		if (wants_gradient(ai)) {
+			Bottom g(ai);
+			for (size_t i = 0; i < oa.size(); i++)
+				LTEN_HIP_CALL(lten_hip_sgemm(0, 1, M, K, N, 1.0f, top + i * M * N, N, bd + ob[i], N, 1.0f, g.ptr + oa[i], K));
+			g.propagate();
+		}
+		if (wants_gradient(bi)) {
+			Bottom g(bi);
+			for (size_t i = 0; i < oa.size(); i++)
+				LTEN_HIP_CALL(lten_hip_sgemm(1, 0, K, N, M, 1.0f, ad + oa[i], K, top + i * M * N, N, 1.0f, g.ptr + ob[i], N));
+			g.propagate();
+		}
+	};
+	return result;
+}
+
+// ------------------------------------------------------------------------------ FullyConnected
+
+static void check_layer_input(const Tensor& input, Tensor& weight, const char* what)
+{
+	// l-ten/fully_connected.cpp:73-78
+	if (input.get_device() != weight.get_device() || input.get_device_index() != weight.get_device_index() ||
+	    input.get_data_type() != weight.get_data_type())
+		LTEN_ERR("Input tensor device type or data type are not the same as this layer's parameters");
+	(void)what;
+}
+
+bool FullyConnected::init()
+{
+	// l-ten/fully_connected.cpp:9-55: weight {1,1,out,in}, bias {out}, U(-sqrt(1/in), sqrt(1/in)) from std::random_device
+	TensorOps options;
+	weight_ = AllocateTensor({ 1, 1, output_features_, input_features_ }, &options);
+	weight_.set_autograd(true);
+	std::random_device generator;
+	std::uniform_real_distribution<float> distribution(-sqrtf(1.0f / input_features_), sqrtf(1.0f / input_features_));
+	float* w = static_cast<float*>(weight_.get_data_ptr());
+	for (uint64_t i = 0; i < weight_.get_numels(); i++) w[i] = distribution(generator);
+	if (use_bias_) {
+		options.alloc_gradient_buffer = true;
+		bias_ = AllocateTensor({ output_features_ }, &options);
+		bias_.set_autograd(true);
+		float* b = static_cast<float*>(bias_.get_data_ptr());
+		for (uint64_t i = 0; i < bias_.get_numels(); i++) b[i] = distribution(generator);
+	}
+	return true;
+}
+
+void FullyConnected::to(device target_device, int target_device_index)
+{
+	// l-ten/fully_connected.cpp:220-289; the bias_multiplier ones vector of l-ten is not needed: the bias is
+	// added in the GEMM epilogue and its gradient is a column sum that needs no operand of ones
+	if (weight_.defined()) weight_ = weight_.to(target_device, target_device_index);
+	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
+}
+
+void FullyConnected::clear_gradients()
+{
+	if (weight_.defined()) weight_.clear_gradients();
+	if (use_bias_ && bias_.defined()) bias_.clear_gradients();
+}
+
+std::vector<Tensor*> FullyConnected::get_all_weights()
+{
+	std::vector<Tensor*> w{ &weight_ };
+	if (use_bias_) w.push_back(&bias_);
+	return w;
+}
+
+Tensor FullyConnected::forward(Tensor& input)
+{
+	const int ndims = input.get_ndims();
+	if (ndims < 3) LTEN_ERR("FullyConnected requires tensors with at least 3 dimensions");  // l-ten/fully_connected.cpp:68-71
+	check_layer_input(input, weight_, "FullyConnected");
+	uint64_t dims[MAX_DIMS];
+	memcpy(dims, input.get_sizes(), sizeof(uint64_t) * ndims);
+	if (dims[ndims - 1] != input_features_) LTEN_ERR("Last dimension must be equal to the number of input features");  // :82-85
+	dims[ndims - 1] = output_features_;
+	if (input.get_device() != GPU)
+		LTEN_ERR("this build implements FullyConnected for the GPU device type only (l-ten's own CPU path covers lten::CPU)");
+
+	TensorOps options;
+	options.data_type = input.get_data_type();
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor(dims, ndims, &options);
+	uint64_t M = 1;  // l-ten/fully_connected.cpp:100-104: all leading dims folded into one GEMM
+	for (int i = 0; i < ndims - 1; i++) M *= dims[i];
+	// l-ten/fully_connected.cpp:150 (NT GEMM) + :165 (bias as a rank-1 GEMM), one launch here
+	LTEN_HIP_CALL(lten_hip_fc_forward_f32(M, input_features_, output_features_, static_cast<const float*>(input.get_data_ptr()),
+	                                      static_cast<const float*>(weight_.get_data_ptr()),
+	                                      use_bias_ ? static_cast<const float*>(bias_.get_data_ptr()) : nullptr,
+	                                      static_cast<float*>(result.get_data_ptr())));
+	if (is_training_) {
+		auto in = input.get_smart_ptr(), wt = weight_.get_smart_ptr();
+		std::shared_ptr<TensorImpl> bs = use_bias_ ? bias_.get_smart_ptr() : nullptr;
+		const uint64_t fin = input_features_, fout = output_features_;
+		result.get_smart_ptr()->children = { in, wt };  // l-ten/fully_connected.cpp:181-184
+		result.get_smart_ptr()->autograd = true;
+		result.get_smart_ptr()->grad_fn = [in, wt, bs, M, fin, fout](TensorImpl&, const float* top) {
+			const float* x = static_cast<const float*>(in->data);
+			const float* w = static_cast<const float*>(wt->data);
+			if (wants_gradient(in)) {  // l-ten/backprop.cpp:2228  dX = dY W (NN)
+				Bottom g(in);
+				LTEN_HIP_CALL(lten_hip_sgemm(0, 0, M, fin, fout, 1.0f, top, fout, w, fin, 1.0f, g.ptr, fin));
+				g.propagate();
+			}
+			if (wants_gradient(wt)) {  // l-ten/backprop.cpp:2252  dW = dY^T X (TN)
+				Bottom g(wt);
+				LTEN_HIP_CALL(lten_hip_sgemm(1, 0, fout, fin, M, 1.0f, top, fout, x, fin, 1.0f, g.ptr, fin));
+			}
+			if (bs) {  // l-ten/backprop.cpp:2267  db += ones dY, straight into the bias gradient buffer
+				bs->ensure_grad();
+				LTEN_HIP_CALL(lten_hip_fc_backward_f32(M, fin, fout, x, w, top, nullptr, nullptr, static_cast<float*>(bs->grad)));
+			}
+		};
+	}
+	return result;
+}
+
+// ------------------------------------------------------------------------------ FullyConnected_q
+
+bool FullyConnected_q::init()
+{
+	// l-ten/fully_connected.cpp:295-320: UINT8 weights {1,1,out,in}, INT32 bias {out}, no initialisation
+	TensorOps options;
+	options.data_type = UINT8;
+	weight_ = AllocateTensor({ 1, 1, output_features_, input_features_ }, &options);
+	weight_.set_autograd(true);
+	if (use_bias_) {
+		options.data_type = INT32;
+		bias_ = AllocateTensor({ output_features_ }, &options);
+		bias_.set_autograd(true);
+	}
+	return true;
+}
+
+void FullyConnected_q::to(device target_device, int target_device_index)
+{
+	// l-ten's FullyConnected_q::to throws "Only CPU device supported" (l-ten/layers.h:86); this is the GPU branch it lacks
+	if (weight_.defined()) weight_ = weight_.to(target_device, target_device_index);
+	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
+	workspace_ = Tensor();
+	max_rows_ = 0;
+}
+
+void FullyConnected_q::clear_gradients()
+{
+	if (weight_.defined()) weight_.clear_gradients();
+	if (use_bias_ && bias_.defined()) bias_.clear_gradients();
+}
+
+std::vector<Tensor*> FullyConnected_q::get_all_weights()
+{
+	std::vector<Tensor*> w{ &weight_ };
+	if (use_bias_) w.push_back(&bias_);
+	return w;
+}
+
+void FullyConnected_q::set_qparams_params(QuantizationParams* qparams, int count)
+{
+	if (qparams && count) qparams_wt_ = qparams[0];  // l-ten/fully_connected.cpp:440-446
+}
+
+Tensor FullyConnected_q::forward(Tensor& input)
+{
+	const int ndims = input.get_ndims();
+	if (ndims < 3) LTEN_ERR("FullyConnected_q requires tensors with at least 3 dimensions");  // l-ten/fully_connected.cpp:331-334
+	check_layer_input(input, weight_, "FullyConnected_q");
+	uint64_t dims[MAX_DIMS];
+	memcpy(dims, input.get_sizes(), sizeof(uint64_t) * ndims);
+	if (dims[ndims - 1] != input_features_) LTEN_ERR("Last dimension must be equal to the number of input features");
+	dims[ndims - 1] = output_features_;
+	if (input.get_device() != GPU)
+		LTEN_ERR("this build implements FullyConnected_q for the GPU device type only (l-ten's own CPU path covers lten::CPU)");
+
+	TensorOps options;
+	options.data_type = UINT8;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor(dims, ndims, &options);
+	// l-ten/fully_connected.cpp:364-396 loops one quantized_matmul over the leading dims with M = dims[ndims-2];
+	// the rows are independent, so the loop is one call with batch * M rows
+	const uint64_t M = dims[ndims - 2];
+	uint64_t batch = 1;
+	for (int i = 0; i < ndims - 2; i++) batch *= dims[i];
+	if (batch * M > max_rows_) {  // :366-371 workspace grown on demand
+		options.data_type = INT32;
+		workspace_ = AllocateTensor({ batch * M + output_features_ }, &options);
+		max_rows_ = batch * M;
+	}
+	lten_hip_qparams qp[3] = { { qparams_in_.scale, qparams_in_.zero_point }, { qparams_wt_.scale, qparams_wt_.zero_point },
+		                   { qparams_out_.scale, qparams_out_.zero_point } };
+	LTEN_HIP_CALL(lten_hip_fcq_forward(batch, M, input_features_, output_features_, static_cast<const uint8_t*>(input.get_data_ptr()),
+	                                   static_cast<const uint8_t*>(weight_.get_data_ptr()),
+	                                   use_bias_ ? static_cast<const int32_t*>(bias_.get_data_ptr()) : nullptr, qp,
+	                                   static_cast<uint8_t*>(result.get_data_ptr()), static_cast<int32_t*>(workspace_.get_data_ptr())));
+	return result;
+}
+
+// ------------------------------------------------------------------------------ Conv2d
+
+bool Conv2d::init()
+{
+	// l-ten/conv2d.cpp:10-53: weight {Cout, Cin, kh*kw}, bias {1,Cout,1,1}, U(+-sqrt(1/(Cin*(kh+kw)))) from a default-seeded engine
+	TensorOps options;
+	weight_ = AllocateTensor({ channels_out_, channels_in_, kernel_h_ * kernel_w_ }, &options);
+	weight_.set_autograd(true);
+	std::default_random_engine generator;
+	const float k = 1.0f / (channels_in_ * (kernel_h_ + kernel_w_));
+	std::uniform_real_distribution<float> distribution(-sqrtf(k), sqrtf(k));
+	float* w = static_cast<float*>(weight_.get_data_ptr());
+	for (uint64_t i = 0; i < weight_.get_numels(); i++) w[i] = distribution(generator);
+	if (use_bias_) {
+		bias_ = AllocateTensor({ 1, channels_out_, 1, 1 }, &options);
+		bias_.set_autograd(true);
+		float* b = static_cast<float*>(bias_.get_data_ptr());
+		for (uint64_t i = 0; i < bias_.get_numels(); i++) b[i] = distribution(generator);
+	}
+	return true;
+}
+
+void Conv2d::to(device target_device, int target_device_index)
+{
+	if (weight_.defined()) weight_ = weight_.to(target_device, target_device_index);
+	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
+	scratch_ = Tensor();
+}
+
+void Conv2d::clear_gradients()
+{
+	if (weight_.defined()) weight_.clear_gradients();
+	if (use_bias_ && bias_.defined()) bias_.clear_gradients();
+}
+
+std::vector<Tensor*> Conv2d::get_all_weights()
+{
+	std::vector<Tensor*> w{ &weight_ };
+	if (use_bias_) w.push_back(&bias_);
+	return w;
+}
+
+// dst += src over n floats, as the K = 1 GEMM dst[1 x n] = one[1 x 1] * src[1 x n] + dst
+static void accumulate(float* dst, const float* src, uint64_t n, const float* device_one)
+{
+	LTEN_HIP_CALL(lten_hip_sgemm(0, 0, 1, n, 1, 1.0f, device_one, 1, src, n, 1.0f, dst, n));
+}
+
+Tensor Conv2d::forward(Tensor& input)
+{
+	if (input.get_data_type() != FLOAT32) LTEN_ERR("Conv2d is only supported for FLOAT32 tensors");  // l-ten/conv2d.cpp:73-76
+	check_layer_input(input, weight_, "Conv2d");
+	if (input.get_ndims() != 4) LTEN_ERR("Conv2d requires tensors with exactly 4 dimensions (NCHW)");  // :86-89
+	const uint64_t* d = input.get_sizes();
+	const uint64_t N = d[0], H = d[2], W = d[3];
+	if (d[1] != channels_in_) LTEN_ERR("Input channel count does not match this layer");
+	const uint64_t Ho = (H + 2 * pad_h_ - kernel_h_) / stride_h_ + 1, Wo = (W + 2 * pad_w_ - kernel_w_) / stride_w_ + 1;  // :102-103
+	if (input.get_device() != GPU)
+		LTEN_ERR("this build implements Conv2d for the GPU device type only (l-ten's own CPU path covers lten::CPU)");
+
+	TensorOps options;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor({ N, channels_out_, Ho, Wo }, &options);
+	const uint64_t Cin = channels_in_, Cout = channels_out_;
+	const int kh = (int)kernel_h_, kw = (int)kernel_w_, ph = (int)pad_h_, pw = (int)pad_w_, sh = (int)stride_h_, sw = (int)stride_w_;
+	// l-ten/conv2d.cpp:164-171 (im2col_gpu + cublasSgemm per image) and :189-192 (bias as a broadcast add): one fused launch
+	LTEN_HIP_CALL(lten_hip_conv2d_forward_f32(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, static_cast<const float*>(input.get_data_ptr()),
+	                                          static_cast<const float*>(weight_.get_data_ptr()),
+	                                          use_bias_ ? static_cast<const float*>(bias_.get_data_ptr()) : nullptr,
+	                                          static_cast<float*>(result.get_data_ptr())));
+
+	// scratch: [one float = 1.0][weight-gradient partials or one column buffer, whichever is larger][temp dW]
+	const uint64_t Kc = Cin * kernel_h_ * kernel_w_, HW = Ho * Wo;
+	const uint64_t ws_bytes = lten_hip_conv2d_wgrad_workspace_bytes(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw);
+	const uint64_t work_floats = std::max<uint64_t>((ws_bytes + 3) / 4, Kc * HW);
+	const uint64_t need = 64 + work_floats + Cout * Kc + Cin * H * W;
+	if (!scratch_.defined() || scratch_.get_numels() < need) {
+		scratch_ = AllocateTensor({ need }, &options);
+		LTEN_HIP_CALL(lten_hip_fill_f32(static_cast<float*>(scratch_.get_data_ptr()), 1, 1.0f));
+	}
+	auto wt = weight_.get_smart_ptr(), in = input.get_smart_ptr(), scratch = scratch_.get_smart_ptr();
+	const bool with_bias = use_bias_;
+	result.get_smart_ptr()->children = { wt, in };  // l-ten/conv2d.cpp:183-187
+	result.get_smart_ptr()->autograd = true;
+	result.get_smart_ptr()->grad_fn = [=](TensorImpl&, const float* top) {
+		if (with_bias) LTEN_ERR("the gradient of the Conv2d bias is not part of the GPU path (l-ten adds the bias as a separate tensor op)");
+		float* one = static_cast<float*>(scratch->data);
+		float* work = one + 64;
+		float* tmp_dw = work + work_floats;
+		float* tmp_dx = tmp_dw + Cout * Kc;
+		const float* x = static_cast<const float*>(in->data);
+		const float* w = static_cast<const float*>(wt->data);
+		if (wants_gradient(wt)) {
+			// l-ten/backprop.cpp:1949-1953 (CPU semantics: the sum over all images), then the leaf accumulate of :246-274
+			Bottom g(wt);
+			LTEN_HIP_CALL(lten_hip_conv2d_wgrad_f32(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, x, top, tmp_dw, work));
+			accumulate(g.ptr, tmp_dw, Cout * Kc, one);
+		}
+		if (wants_gradient(in)) {
+			// l-ten/backprop.cpp:2022-2028: per image col = W^T dY_n (TN GEMM) then col2im
+			Bottom g(in);
+			for (uint64_t n = 0; n < N; n++) {
+				LTEN_HIP_CALL(lten_hip_sgemm(1, 0, Kc, HW, Cout, 1.0f, w, Kc, top + n * Cout * HW, HW, 0.0f, work, HW));
+				LTEN_HIP_CALL(lten_hip_col2im_f32(work, (int)Cin, (int)H, (int)W, kh, kw, ph, pw, sh, sw, 1, 1, tmp_dx));
+				accumulate(g.ptr + n * Cin * H * W, tmp_dx, Cin * H * W, one);
+			}
+			g.propagate();
+		}
+	};
+	return result;
+}
+
+}  // namespace lten

@@ -1,0 +1,191 @@
+// Host-side mirror of l-ten's layer API for the GEMM hot path, over the C ABI of liblten_hip.
+//
+// Same names, argument meaning and error behaviour as l-ten's lten::Tensor / FullyConnected /
+// FullyConnected_q / Conv2d / Tensor::matmul (l-ten/tensor.h, l-ten/layers.h), reduced to what the hot
+// path needs.  It is the shape of the glue a maintainer adds to l-ten's own `#ifdef USE_CUDA` branches:
+// every GPU branch below is one call through include/lten_hip.h.  Tensors on lten::CPU only carry data
+// in and out (TensorFromBuffer, to()); the arithmetic itself exists for lten::GPU tensors only — there
+// is no CPU compute path in this library, l-ten already has one.
+#ifndef LTEN_GPU_H
+#define LTEN_GPU_H
+
+#include <cstdint>
+#include <exception>
+#include <functional>
+#include <initializer_list>
+#include <memory>
+#include <string>
+#include <vector>
+
+// l-ten/md_array.h:37
+#define MAX_DIMS 16
+
+// l-ten/math_fns.h:12-16 (global namespace there too)
+struct QuantizationParams {
+	float scale;
+	uint8_t zero_point;
+};
+
+namespace lten {
+
+// l-ten/tensorimpl.h:46-47
+enum device { CPU, GPU };
+enum dtype { FLOAT32, INT32, UINT8 };
+
+// l-ten/tensorimpl.h:49-63
+struct TensorOps {
+	TensorOps() : data_type(FLOAT32), device_type(CPU), device_index(0), alloc_gradient_buffer(false) {}
+	dtype data_type;
+	device device_type;
+	int device_index;
+	bool alloc_gradient_buffer;
+};
+
+// What LTEN_ERR throws (l-ten/error.h:78-93, l-ten/utils.cpp:303-306).
+class ExceptionInfo : public std::exception {
+public:
+	ExceptionInfo(const char* msg, const char* file, const char* func, int line);
+	const char* what() const noexcept override { return text_.c_str(); }
+
+private:
+	std::string text_;
+};
+[[noreturn]] void ltenFail(const char* msg, const char* file, const char* func, int line);
+#define LTEN_ERR(msg) ::lten::ltenFail(msg, __FILE__, __func__, __LINE__)
+
+struct TensorImpl;
+class Tensor;
+// gradient callback: (node, gradient of the loss with respect to the node's output on the node's device)
+typedef std::function<void(TensorImpl& node, const float* top_gradient)> grad_fn_t;
+
+class Tensor {
+public:
+	Tensor() {}
+	explicit Tensor(std::shared_ptr<TensorImpl> impl) : impl_(impl) {}
+
+	void* get_data_ptr();
+	void* get_grad_ptr();
+	uint64_t get_numels() const;
+	const uint64_t* get_sizes() const;
+	int get_ndims() const;
+	dtype get_data_type() const;
+	device get_device() const;
+	int get_device_index() const;
+	void set_autograd(bool setting);
+	void clear_gradients();
+
+	// l-ten/tensor.h:140-..., l-ten/tensorimpl.cpp:311-412: copy to the other device (synchronous).
+	Tensor to(device target_device, int target_device_index = 0);
+	// l-ten/tensor.h:83-138: batched matrix product over the leading dims, size-1 dims broadcast.
+	Tensor matmul(const Tensor& other);
+	// l-ten/tensor.h:69 backward(MultiDimArray<float>* top_gradient): top_gradient has the tensor's shape and
+	// lives on the tensor's device; null stands for a single 1 and is only valid for one-element tensors.
+	void backward(const Tensor* top_gradient = nullptr);
+
+	std::shared_ptr<TensorImpl> get_smart_ptr() const { return impl_; }
+	bool defined() const { return impl_ != nullptr; }
+
+private:
+	std::shared_ptr<TensorImpl> impl_;
+};
+
+// l-ten/tensor.h:1478-1482
+Tensor TensorFromBuffer(const std::initializer_list<uint64_t>& dims, void* data_ptr, bool own_memory = false, TensorOps* options_ptr = nullptr);
+Tensor TensorFromBuffer(const uint64_t* dims_ptr, int ndims, void* data_ptr, bool own_memory = false, TensorOps* options_ptr = nullptr);
+Tensor AllocateTensor(const std::initializer_list<uint64_t>& dims, TensorOps* options_ptr = nullptr);
+Tensor AllocateTensor(const uint64_t* dims_ptr, int ndims, TensorOps* options_ptr = nullptr);
+
+// l-ten/layers.h:14-31
+class Module {
+public:
+	Module() {}
+	virtual ~Module() {}
+	virtual bool init() = 0;
+	virtual std::vector<Tensor*> get_all_weights() = 0;
+	virtual void clear_gradients() = 0;
+	virtual void to(device target_device, int target_device_index = 0) = 0;
+	void train(bool is_training) { is_training_ = is_training; }
+	virtual void set_qparams_in(QuantizationParams) {}
+	virtual void set_qparams_out(QuantizationParams) {}
+	virtual void set_qparams_params(QuantizationParams*, int) {}
+
+protected:
+	bool is_training_ = true;
+};
+
+// l-ten/layers.h:35-66
+class FullyConnected : public Module {
+public:
+	FullyConnected(int64_t input_features, int64_t output_features, bool use_bias = false, dtype data_type = FLOAT32)
+	    : input_features_(input_features), output_features_(output_features), use_bias_(use_bias) { (void)data_type; }
+	bool init() override;
+	Tensor forward(Tensor& input);
+	Tensor* get_weights() { return &weight_; }
+	Tensor* get_bias() { return use_bias_ ? &bias_ : nullptr; }
+	void clear_gradients() override;
+	std::vector<Tensor*> get_all_weights() override;
+	void to(device target_device, int target_device_index = 0) override;
+	bool is_using_bias() { return use_bias_; }
+
+private:
+	uint64_t input_features_, output_features_;
+	Tensor weight_, bias_;
+	bool use_bias_;
+};
+
+// l-ten/layers.h:69-106; unlike l-ten's, this one runs on the GPU (l-ten: "Only CPU device supported").
+class FullyConnected_q : public Module {
+public:
+	FullyConnected_q(int64_t input_features, int64_t output_features, bool use_bias = false, dtype data_type = FLOAT32)
+	    : input_features_(input_features), output_features_(output_features), use_bias_(use_bias) { (void)data_type; }
+	bool init() override;
+	Tensor forward(Tensor& input);
+	Tensor* get_weights() { return &weight_; }
+	Tensor* get_bias() { return use_bias_ ? &bias_ : nullptr; }
+	void clear_gradients() override;
+	std::vector<Tensor*> get_all_weights() override;
+	void to(device target_device, int target_device_index = 0) override;
+	bool is_using_bias() { return use_bias_; }
+	void set_qparams_in(QuantizationParams qparams_in) override { qparams_in_ = qparams_in; }
+	void set_qparams_out(QuantizationParams qparams_out) override { qparams_out_ = qparams_out; }
+	void set_qparams_params(QuantizationParams* qparams, int count) override;
+
+private:
+	uint64_t input_features_, output_features_;
+	Tensor weight_, bias_, workspace_;
+	bool use_bias_;
+	uint64_t max_rows_ = 0;
+	QuantizationParams qparams_in_{ 1.0f, 0 }, qparams_out_{ 1.0f, 0 }, qparams_wt_{ 1.0f, 0 };
+};
+
+// l-ten/layers.h:392-451
+class Conv2d : public Module {
+public:
+	Conv2d(const int channels_in, const int channels_out, bool use_bias, const int kernel_h, const int kernel_w, const int pad_h = 0,
+	       const int pad_w = 0, const int stride_h = 1, const int stride_w = 1)
+	    : channels_in_(channels_in), channels_out_(channels_out), kernel_h_(kernel_h), kernel_w_(kernel_w), pad_h_(pad_h), pad_w_(pad_w),
+	      stride_h_(stride_h), stride_w_(stride_w), use_bias_(use_bias) {}
+	uint64_t get_channels_out() { return channels_out_; }
+	uint64_t get_channels_in() { return channels_in_; }
+	uint64_t get_kernel_h() { return kernel_h_; }
+	uint64_t get_kernel_w() { return kernel_w_; }
+	uint64_t get_pad_h() { return pad_h_; }
+	uint64_t get_pad_w() { return pad_w_; }
+	uint64_t get_stride_h() { return stride_h_; }
+	uint64_t get_stride_w() { return stride_w_; }
+	bool init() override;
+	Tensor forward(Tensor& input);
+	std::vector<Tensor*> get_all_weights() override;
+	Tensor* get_weights() { return &weight_; }
+	Tensor* get_bias() { return use_bias_ ? &bias_ : nullptr; }
+	void clear_gradients() override;
+	void to(device target_device, int target_device_index = 0) override;
+
+private:
+	uint64_t channels_in_, channels_out_, kernel_h_, kernel_w_, pad_h_, pad_w_, stride_h_, stride_w_;
+	bool use_bias_;
+	Tensor weight_, bias_, scratch_;  // scratch_: weight-gradient partial sums / column buffer of the data gradient
+};
+
+}  // namespace lten
+#endif
