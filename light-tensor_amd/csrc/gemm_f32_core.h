@@ -111,6 +111,22 @@ struct GemmCore {
 		}
 	}
 
+	// Replaces every accumulator of this lane by f(row, col, value).
+	template <typename F>
+	__device__ static __forceinline__ void transform(v16f (&acc)[FM][FN], F f)
+	{
+		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+		const int wm = wave / WN, wn = wave % WN;
+		const int lrow = lane & 31, lk = lane >> 5;
+#pragma unroll
+		for (int j = 0; j < FN; j++)
+#pragma unroll
+			for (int i = 0; i < FM; i++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					acc[i][j][r] = f(wm * TM + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3), wn * TN + j * 32 + lrow, acc[i][j][r]);
+	}
+
 	// Visits every accumulator of this lane with its tile coordinates.
 	template <typename F>
 	__device__ static __forceinline__ void for_each(v16f (&acc)[FM][FN], F f)

@@ -8,6 +8,8 @@
 #include "common.h"
 #include "gemm_f32_core.h"
 
+#include <algorithm>
+
 namespace lten_hip {
 
 struct SProblem {
@@ -58,6 +60,93 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
 		if (p.bias) out += p.bias[n];
 		*c = out;
 	});
+}
+
+// Small outputs with a long K (the FullyConnected GEMMs at batch 128): one workgroup per 32x32 output tile,
+// its WAVES wavefronts each reduce an interleaved share of K with operands loaded straight from global
+// memory in the MFMA lane layout — no LDS staging, no barrier in the loop, loads unrolled ahead of their use —
+// and the WAVES partial tiles meet in LDS, where they are added in wavefront order (deterministic).
+// A k-contiguous operand is fetched 16 bytes per lane: lane (row, g) takes k = base + 4g .. 4g+3 and feeds the
+// t-th of four MFMAs with element t; the other layout is fetched one dword per MFMA (two 128-byte rows per
+// wave-wide load).  The assignment of k to MFMA slots is the same for A and B, which is all a dot product needs.
+template <int WAVES, bool TA, bool TB>
+__global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
+{
+	__shared__ float part[WAVES][32 * 32];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int lrow = lane & 31, g = lane >> 5;
+	const int tiles_n = (p.N + 31) / 32;
+	const int m0 = (blockIdx.x / tiles_n) * 32, n0 = (blockIdx.x % tiles_n) * 32;
+	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
+	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
+	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+	const int m = m0 + lrow, n = n0 + lrow;
+	const bool mok = m < p.M, nok = n < p.N;
+	const bool a_vec = !TA && (p.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
+	const bool b_vec = TB && (p.ldb & 3) == 0 && (reinterpret_cast<uintptr_t>(B) & 15) == 0;
+
+	v16f acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+	// groups of 8 consecutive k, dealt round-robin to the wavefronts
+	const int groups = (p.K + 7) / 8;
+#pragma unroll 4
+	for (int grp = wave; grp < groups; grp += WAVES) {
+		const int k = grp * 8 + g * 4;
+		float a[4] = { 0.f, 0.f, 0.f, 0.f }, b[4] = { 0.f, 0.f, 0.f, 0.f };
+		if (mok) {
+			if (a_vec && k + 4 <= p.K) {
+				const float4 v = *reinterpret_cast<const float4*>(A + (int64_t)m * p.lda + k);
+				a[0] = v.x; a[1] = v.y; a[2] = v.z; a[3] = v.w;
+			} else {
+#pragma unroll
+				for (int t = 0; t < 4; t++)
+					if (k + t < p.K) a[t] = TA ? A[(int64_t)(k + t) * p.lda + m] : A[(int64_t)m * p.lda + k + t];
+			}
+		}
+		if (nok) {
+			if (b_vec && k + 4 <= p.K) {
+				const float4 v = *reinterpret_cast<const float4*>(B + (int64_t)n * p.ldb + k);
+				b[0] = v.x; b[1] = v.y; b[2] = v.z; b[3] = v.w;
+			} else {
+#pragma unroll
+				for (int t = 0; t < 4; t++)
+					if (k + t < p.K) b[t] = TB ? B[(int64_t)n * p.ldb + k + t] : B[(int64_t)(k + t) * p.ldb + n];
+			}
+		}
+#pragma unroll
+		for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
+	}
+
+	// register 4q + e of lane (lrow, g): row 8q + 4g + e, column lrow
+#pragma unroll
+	for (int r = 0; r < 16; r++) part[wave][((r >> 2) * 8 + g * 4 + (r & 3)) * 32 + lrow] = acc[r];
+	__syncthreads();
+	for (int idx = tid; idx < 32 * 32; idx += WAVES * 64) {
+		const int row = idx >> 5, col = idx & 31;
+		if (m0 + row >= p.M || n0 + col >= p.N) continue;
+		float sum = 0.0f;
+#pragma unroll
+		for (int w = 0; w < WAVES; w++) sum += part[w][idx];
+		float* c = C + (int64_t)(m0 + row) * p.ldc + n0 + col;
+		float out = p.alpha * sum;
+		if (p.beta != 0.0f) out += p.beta * *c;
+		if (p.bias) out += p.bias[n0 + col];
+		*c = out;
+	}
+}
+
+static int launch_direct(const SProblem& p, int tA, int tB, uint64_t batch)
+{
+	const dim3 grid((unsigned)(ceil_div(p.M, 32) * ceil_div(p.N, 32)), 1, (unsigned)batch), block(8 * 64);
+	set_kernel_name("sgemm_direct_32x32_w8");
+	if (!tA && !tB) sgemm_direct_kernel<8, false, false><<<grid, block, 0, stream()>>>(p);
+	if (!tA && tB) sgemm_direct_kernel<8, false, true><<<grid, block, 0, stream()>>>(p);
+	if (tA && !tB) sgemm_direct_kernel<8, true, false><<<grid, block, 0, stream()>>>(p);
+	if (tA && tB) sgemm_direct_kernel<8, true, true><<<grid, block, 0, stream()>>>(p);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
 }
 
 // K == 1: the rank-1 update C = alpha * a b^T + beta * C that l-ten uses to add the FC bias
@@ -154,11 +243,18 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	const uint64_t tiles64 = ceil_div(M, 64) * ceil_div(N, 64) * batch;
 	const uint64_t tiles128 = ceil_div(M, 128) * ceil_div(N, 128) * batch;
 	int choice = force;
-	if (choice == 0) choice = tiles128 >= 512 ? 1 : (tiles64 >= 256 ? 2 : 3);
+	if (choice == 0) {
+		// Few output tiles and a long K: the LDS-tiled kernels would leave most CUs idle while a handful of
+		// workgroups walk K in sequence; the direct kernel cuts K across the wavefronts of a workgroup instead.
+		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32) * batch;
+		if (tiles32 <= 1024) choice = 4;
+		else choice = tiles128 >= 128 ? 1 : 2;
+	}
 	switch (choice) {
 	case 1: return launch_sgemm<128, 128, 16, 2, 2>(p, tA, tB, batch, "sgemm_128x128x16");
 	case 2: return launch_sgemm<64, 64, 32, 2, 2>(p, tA, tB, batch, "sgemm_64x64x32");
-	default: return launch_sgemm<32, 32, 32, 1, 1>(p, tA, tB, batch, "sgemm_32x32x32");
+	case 3: return launch_sgemm<32, 32, 32, 1, 1>(p, tA, tB, batch, "sgemm_32x32x32");
+	default: return launch_direct(p, tA, tB, batch);
 	}
 }
 

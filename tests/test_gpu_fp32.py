@@ -33,7 +33,7 @@ def test_sgemm_golden_cases(gpu):
         assert rel_err(got, g[pre + "C"]) < TOL, (i, M, N, K, tA, tB, alpha, beta, gpu.last_kernel())
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])  # 1-3: LDS-tiled kernels, 4: direct (intra-workgroup split-K) kernel
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_integer_valued_exact_with_leading_dims(gpu, tile, tA, tB):
     rng = np.random.default_rng(40 + 2 * tA + tB + 10 * tile)
@@ -77,6 +77,21 @@ def test_cfg2_gemm_shapes_all_layouts(gpu, ob, shape):
         err = rel_err(got, want)
         print(f"  {'TN'[tA]}{'NT'[tB]} {m}x{n}x{k} via {gpu.last_kernel()}: max rel err {err:.2e}")
         assert err < TOL
+
+
+def test_direct_kernel_is_deterministic_and_repeatable(gpu):
+    """The direct kernel adds its wavefronts' partial tiles in wavefront order: bitwise equal results run after run."""
+    rng = np.random.default_rng(3)
+    M, N, K = 128, 1024, 1024
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((N, K)).astype(np.float32)
+    z = np.zeros((M, N), np.float32)
+    first = gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N)
+    assert gpu.last_kernel().startswith("sgemm_direct")
+    for _ in range(5):
+        assert np.array_equal(gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N), first)
+    want = A.astype(np.float64) @ B.astype(np.float64).T
+    assert rel_err(first, want) < TOL
 
 
 def test_rank1_and_rowvec_shapes(gpu, ob):
