@@ -97,24 +97,27 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	}
 	const int m0 = tm * BM, n0 = tn * BN;
 
-	// ---- global -> LDS: what this lane fetches for each of its wavefront's loads
+	// ---- global -> LDS: what this lane fetches for each of its wavefront's loads.  Load q covers rows
+	// q*RPL .. q*RPL+RPL-1 of the stacked [A tile; B tile]; wavefront w issues loads w, w+W, w+2W, ...,
+	// so its first LPW/2 loads are A rows and the rest B rows whatever w is.
+	static_assert((BM / RPL) % W == 0 && LPW % 2 == 0, "A and B loads split evenly over the wavefronts");
 	uint32_t voff[LPW];
-	const uint8_t* gbase[LPW];
 	uint32_t lds_slot[LPW];
 	const uint32_t smem_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
 #pragma unroll
 	for (int i = 0; i < LPW; i++) {
-		const int q = wave + i * W;  // rows q*RPL .. q*RPL+RPL-1 of the stacked [A tile; B tile]
-		const bool is_a = q * RPL < BM;
+		const int q = wave + i * W;
 		const int r = q * RPL + lane / CPR;
 		const int kc = (lane % CPR) ^ swz<CPR>(r);
-		gbase[i] = is_a ? p.A : p.B;
-		voff[i] = (is_a ? (uint32_t)(m0 + r) : (uint32_t)(n0 + r - BM)) * (uint32_t)p.K + kc * 16;
+		voff[i] = (i < LPW / 2 ? (uint32_t)(m0 + r) : (uint32_t)(n0 + r - BM)) * (uint32_t)p.K + kc * 16;
 		lds_slot[i] = smem_addr + q * 1024;
 	}
+	auto load_one = [&](int i, int stage, int kt) {
+		async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? p.A : p.B) + (int64_t)kt * BK, voff[i]);
+	};
 	auto issue = [&](int stage, int kt) {
 #pragma unroll
-		for (int i = 0; i < LPW; i++) async_load16(lds_slot[i] + stage * STAGE, gbase[i] + (int64_t)kt * BK, voff[i]);
+		for (int i = 0; i < LPW; i++) load_one(i, stage, kt);
 	};
 
 	// ---- LDS -> MFMA operands.  Lane (lrow, lgrp) feeds row lrow of a 32-row block with the 16 bytes
@@ -181,8 +184,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 			}
 			if (refill && !(LTEN_HIP_EXP & 1)) {
 #pragma unroll
-				for (int l = m; l < LPW; l += NM)
-					async_load16(lds_slot[l] + refill_stage * STAGE, gbase[l] + (int64_t)refill_kt * BK, voff[l]);
+				for (int l = m; l < LPW; l += NM) load_one(l, refill_stage, refill_kt);
 			}
 			__builtin_amdgcn_sched_barrier(0);
 		}
