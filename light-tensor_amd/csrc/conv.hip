@@ -6,16 +6,12 @@
 // address on the fly (col[k][hw] = x[ci][ho*sh - ph + i][wo*sw - pw + j], zero outside the image), and one
 // launch covers the whole batch.  The standalone im2col / col2im kernels keep the semantics of l-ten's
 // CUDA ones (l-ten/im_col.cu:65-96, 123-162) for callers that still want the buffer.
-#include "common.h"
+#include "conv_common.h"
 #include "gemm_f32_core.h"
 
 #include <algorithm>
 
 namespace lten_hip {
-
-struct ConvGeo {
-	int N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, dh, dw, Ho, Wo;
-};
 
 template <typename T>
 __global__ __launch_bounds__(256) void im2col_kernel(const T* im, ConvGeo g, T* col)
@@ -113,7 +109,7 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, 
 
 // Weight gradient: dw[co][k] = sum_n sum_hw dy[n][co][hw] * col_n[k][hw].  GEMM rows = co, columns = k,
 // reduction over hw.  Workgroup (tile, image, slice) reduces one slice of one image's hw range and writes
-// a partial [Cout x Kc] matrix; conv2d_wgrad_reduce_kernel adds the partials in a fixed order.
+// a partial [Cout x Kc] matrix; conv_reduce_partials adds the partials in a fixed order.
 template <int BM, int BN, int BK, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, const float* x, const float* dy, float* partial, int slices, int slice_len)
 {
@@ -150,15 +146,6 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, co
 		const int co = m0 + row, k = n0 + col;
 		if (co < g.Cout && k < Kc) out[(int64_t)co * Kc + k] = v;
 	});
-}
-
-__global__ __launch_bounds__(256) void conv2d_wgrad_reduce_kernel(const float* partial, int parts, int64_t count, float* dw)
-{
-	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
-	if (idx >= count) return;
-	float s = 0.0f;
-	for (int p = 0; p < parts; p++) s += partial[(int64_t)p * count + idx];
-	dw[idx] = s;
 }
 
 static int make_geo(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
@@ -242,6 +229,8 @@ int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W
 	if (N == 0 || Cout == 0 || g.Ho * g.Wo == 0) return 0;
 	LTEN_HIP_REQUIRE(x && w && y, "conv2d_forward: null pointer");
 	const int HW = g.Ho * g.Wo;
+	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
+	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");
 		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
@@ -262,7 +251,10 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
 	if (make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return 0;
 	int slices, slice_len;
 	wgrad_split(g, slices, slice_len);
-	return (uint64_t)N * slices * Cout * Cin * kh * kw * sizeof(float);
+	// enough for whichever kernel the call picks
+	uint64_t parts = (uint64_t)N * slices;
+	if (conv_patch_wgrad_takes(g)) parts = std::max<uint64_t>(parts, conv_patch_wgrad_parts(g));
+	return parts * Cout * Cin * kh * kw * sizeof(float);
 }
 
 int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
@@ -275,6 +267,11 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	LTEN_HIP_REQUIRE(dw != nullptr, "conv2d_wgrad: dw is null");
 	if (N == 0 || g.Ho * g.Wo == 0) return lten_hip_zero(dw, count * sizeof(float));
 	LTEN_HIP_REQUIRE(x && dy && workspace, "conv2d_wgrad: null pointer");
+	if (get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
+		const int parts = conv_patch_wgrad_parts(g);
+		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
+		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
+	}
 	int slices, slice_len;
 	wgrad_split(g, slices, slice_len);
 	const int parts = (int)N * slices;
@@ -290,9 +287,7 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		conv2d_wgrad_kernel<32, 32, 32, 1, 1><<<grid, dim3(64), 0, stream()>>>(g, x, dy, partial, slices, slice_len);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
-	conv2d_wgrad_reduce_kernel<<<dim3((unsigned)ceil_div(count, 256)), dim3(256), 0, stream()>>>(partial, parts, count, dw);
-	LTEN_HIP_LAUNCH_CHECK();
-	return 0;
+	return conv_reduce_partials(partial, parts, count, dw);
 }
 
 }  // extern "C"

@@ -1,0 +1,387 @@
+// Conv2d forward and weight gradient for stride 1, dilation 1: the input patch of an output tile is staged
+// in LDS once and every kernel tap reads it from there.
+//
+// l-ten writes an im2col buffer per image and multiplies it with the weight matrix (l-ten/conv2d.cpp:164-171
+// forward, l-ten/backprop.cpp:1949-1953 weight gradient); the buffer repeats every input element kh*kw times.
+// Here a workgroup loads the rows of x that its output tile touches (tile + halo) into LDS, and the MFMA
+// operand of tap (i, j) is the same LDS patch read at an offset of i rows and j columns, so x crosses the
+// memory system once per tile instead of kh*kw times and no index arithmetic runs per element.
+//
+// The reduction index of a product is free to be reordered as long as both operands agree.  Both kernels
+// order it so that the two reduction positions one v_mfma_f32_32x32x2f32 consumes (lanes 0-31 and 32-63)
+// differ by a fixed LDS stride: then every operand address is one per-lane base plus an immediate.
+#include "conv_common.h"
+#include "gemm_f32_core.h"
+
+#include <algorithm>
+
+namespace lten_hip {
+
+// Four consecutive floats of a row starting at column gx; columns outside [0, limit) read as 0.  With VEC
+// (limit % 4 == 0, gx % 4 == 0, 16-byte aligned row) the four are inside or outside together.
+template <bool VEC>
+__device__ __forceinline__ float4 load_row4(const float* row, int gx, int limit)
+{
+	float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	if (VEC) {
+		if (gx >= 0 && gx + 3 < limit) v = *reinterpret_cast<const float4*>(row + gx);
+	} else {
+		if (gx >= 0 && gx < limit) v.x = row[gx];
+		if (gx + 1 >= 0 && gx + 1 < limit) v.y = row[gx + 1];
+		if (gx + 2 >= 0 && gx + 2 < limit) v.z = row[gx + 2];
+		if (gx + 3 >= 0 && gx + 3 < limit) v.w = row[gx + 3];
+	}
+	return v;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Forward.  Workgroup tile: 64 output channels x (TH = 4 rows x TW = 128 columns) of one image; wavefront
+// `wave` owns row `wave` (2 x 4 MFMA tiles of 32 x 32).  The input channels are walked in chunks of CB = 8:
+// per chunk the patch [8][TH + KH - 1][PWS] and the weights of those channels are stored to LDS, the next
+// chunk's values are fetched to registers, and (CB / 2) * KH * KW MFMA steps run; step (cp, i, j) multiplies
+// tap (i, j) of channels 2cp (lanes 0-31) and 2cp + 1 (lanes 32-63).
+//
+// LDS patch row: index q holds input column w0 - 4 + q (interior 16-byte aligned, left halo in 4 - pw .. 3).
+// LDS weights: [step][channel parity][WROW = 65] (the odd row length spreads the scattered stores over banks).
+template <int KH, int KW>
+struct PatchFwd {
+	static constexpr int CB = 4, TH = 4, TW = 128, BM = 64, T = 256;
+	static constexpr int PR = TH + KH - 1;
+	static constexpr int PWS = (4 + TW + KW - 1 + 3) / 4 * 4;
+	static constexpr int F4_ROW = PWS / 4;
+	static constexpr int PATCH = CB * PR * PWS;
+	static constexpr int PATCH_F4 = CB * PR * F4_ROW;
+	static constexpr int P_PER_T = (PATCH_F4 + T - 1) / T;
+	static constexpr int TAPS = KH * KW;
+	static constexpr int KSTEPS = (CB / 2) * TAPS;
+	static constexpr int WROW = BM + 1;
+	static constexpr int WTS = KSTEPS * 2 * WROW;
+	static constexpr int WCOUNT = BM * CB * TAPS;
+	static constexpr int W_PER_T = (WCOUNT + T - 1) / T;
+};
+
+template <int KH, int KW, bool VEC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv2d_patch_forward_kernel(
+    ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
+{
+	typedef PatchFwd<KH, KW> P;
+	__shared__ __attribute__((aligned(16))) float s_patch[P::PATCH];
+	__shared__ float s_w[P::WTS];
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
+	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
+	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
+	const int co0 = blockIdx.y * P::BM, n = blockIdx.z;
+	const int Kc = g.Cin * P::TAPS;
+	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+
+	float4 rp[P::P_PER_T];
+	float rw[P::W_PER_T];
+	auto load_chunk = [&](int c0) {
+#pragma unroll
+		for (int q = 0; q < P::P_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
+			const int pr = rowid % P::PR, c = rowid / P::PR;
+			const int gy = h0 + pr - g.ph;
+			float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (idx < P::PATCH_F4 && c0 + c < g.Cin && gy >= 0 && gy < g.H)
+				v = load_row4<VEC>(xn + ((int64_t)(c0 + c) * g.H + gy) * g.W, w0 - 4 + 4 * f, g.W);
+			rp[q] = v;
+		}
+#pragma unroll
+		for (int q = 0; q < P::W_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int co = idx / (P::CB * P::TAPS), kk = idx % (P::CB * P::TAPS);
+			const int k = c0 * P::TAPS + kk;
+			rw[q] = (idx < P::WCOUNT && co0 + co < g.Cout && k < Kc) ? w[(int64_t)(co0 + co) * Kc + k] : 0.0f;
+		}
+	};
+	auto store_chunk = [&]() {
+#pragma unroll
+		for (int q = 0; q < P::P_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			if (idx < P::PATCH_F4) *reinterpret_cast<float4*>(s_patch + idx * 4) = rp[q];
+		}
+#pragma unroll
+		for (int q = 0; q < P::W_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int co = idx / (P::CB * P::TAPS), kk = idx % (P::CB * P::TAPS);
+			const int c = kk / P::TAPS, tap = kk % P::TAPS;
+			if (idx < P::WCOUNT) s_w[(((c >> 1) * P::TAPS + tap) * 2 + (c & 1)) * P::WROW + co] = rw[q];
+		}
+	};
+
+	v16f acc[2][4];
+#pragma unroll
+	for (int m = 0; m < 2; m++)
+#pragma unroll
+		for (int t = 0; t < 4; t++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc[m][t][r] = 0.0f;
+
+	const float* pa = s_w + half * P::WROW + lrow;
+	const float* pb = s_patch + (half * P::PR + wave) * P::PWS + lrow + 4 - g.pw;
+
+	load_chunk(0);
+	for (int c0 = 0; c0 < g.Cin; c0 += P::CB) {
+		store_chunk();
+		__syncthreads();
+		if (c0 + P::CB < g.Cin) load_chunk(c0 + P::CB);
+#pragma unroll
+		for (int s = 0; s < P::KSTEPS; s++) {
+			const int cp = s / P::TAPS, tap = s % P::TAPS, i = tap / KW, j = tap % KW;
+			float fa[2], fb[4];
+#pragma unroll
+			for (int m = 0; m < 2; m++) fa[m] = pa[s * 2 * P::WROW + m * 32];
+#pragma unroll
+			for (int t = 0; t < 4; t++) fb[t] = pb[(2 * cp * P::PR + i) * P::PWS + j + t * 32];
+#pragma unroll
+			for (int m = 0; m < 2; m++)
+#pragma unroll
+				for (int t = 0; t < 4; t++) acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[m], fb[t], acc[m][t], 0, 0, 0);
+		}
+		__syncthreads();
+	}
+
+	const int ho = h0 + wave;
+	if (ho >= g.Ho) return;
+#pragma unroll
+	for (int m = 0; m < 2; m++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int co = co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+			if (co >= g.Cout) continue;
+			const float b = bias ? bias[co] : 0.0f;
+			float* yrow = y + (((int64_t)n * g.Cout + co) * g.Ho + ho) * g.Wo;
+#pragma unroll
+			for (int t = 0; t < 4; t++) {
+				const int wo = w0 + t * 32 + lrow;
+				if (wo < g.Wo) yrow[wo] = acc[m][t][r] + b;
+			}
+		}
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Weight gradient.  dw[co][ci][i][j] = sum over (n, ho, wo) of dy[n][co][ho][wo] * x[n][ci][ho+i-ph][wo+j-pw].
+// As a product: rows = 64 output channels, columns = (tap, 32 input channels), reduction over output pixels.
+// A workgroup owns a co block, a ci block and a contiguous range of chunks (a chunk = TW = 64 pixels of one
+// output row); per chunk it stages dy[64][64] and the patch [32 ci][KH rows][PWS] in LDS.  Wavefront
+// (mt, ph) multiplies MFMA row tile mt against all KH*KW tap tiles over pixel half ph of the chunk; one
+// MFMA step takes pixels 2s (lanes 0-31) and 2s + 1 (lanes 32-63).  At the end the two pixel halves are added
+// through LDS and the workgroup writes one partial [Cout][Cin*KH*KW] block; a second kernel adds the parts.
+template <int KH, int KW>
+struct PatchWgrad {
+	static constexpr int BM = 64, CIB = 32, TW = 64, T = 256, TAPS = KH * KW;
+	static constexpr int PWS = (4 + TW + KW - 1 + 3) / 4 * 4;
+	static constexpr int F4_ROW = PWS / 4;
+	static constexpr int CS = (KH * PWS) | 1;  // odd channel stride: 32 channels hit 32 banks
+	static constexpr int DYS = TW + 1;
+	static constexpr int DY_FLOATS = BM * DYS, PATCH_FLOATS = CIB * CS;
+	static constexpr int LDS_FLOATS = DY_FLOATS + PATCH_FLOATS;
+	static constexpr int DY_F4 = BM * TW / 4, DY_PER_T = DY_F4 / T;
+	static constexpr int PATCH_F4 = CIB * KH * F4_ROW, P_PER_T = (PATCH_F4 + T - 1) / T;
+	static constexpr int TAPS_PER_ROUND = LDS_FLOATS / (2 * 64 * 16);  // taps whose accumulators fit the final exchange
+	static_assert(DY_F4 % T == 0 && TAPS_PER_ROUND >= 1, "tile shape");
+};
+
+template <int KH, int KW, bool VEC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv2d_patch_wgrad_kernel(
+    ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ partial, int chunks_per_part)
+{
+	typedef PatchWgrad<KH, KW> P;
+	__shared__ float lds[P::LDS_FLOATS];
+	float* s_dy = lds;
+	float* s_patch = lds + P::DY_FLOATS;
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
+	const int mt = wave & 1, phalf = wave >> 1;
+	const int co0 = blockIdx.y * P::BM, ci0 = blockIdx.z * P::CIB;
+	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
+	const int total = g.N * g.Ho * tiles_w;
+	const int begin = blockIdx.x * chunks_per_part, end = min(total, begin + chunks_per_part);
+
+	float4 rdy[P::DY_PER_T], rp[P::P_PER_T];
+	auto load_chunk = [&](int chunk) {
+		const int wt = chunk % tiles_w, ho = (chunk / tiles_w) % g.Ho, n = chunk / (tiles_w * g.Ho);
+		const int w0 = wt * P::TW;
+#pragma unroll
+		for (int q = 0; q < P::DY_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int p4 = idx % (P::TW / 4), co = idx / (P::TW / 4);
+			float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (co0 + co < g.Cout) v = load_row4<VEC>(dy + (((int64_t)n * g.Cout + co0 + co) * g.Ho + ho) * g.Wo, w0 + 4 * p4, g.Wo);
+			rdy[q] = v;
+		}
+#pragma unroll
+		for (int q = 0; q < P::P_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
+			const int r = rowid % KH, ci = rowid / KH;
+			const int gy = ho + r - g.ph;
+			float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (idx < P::PATCH_F4 && ci0 + ci < g.Cin && gy >= 0 && gy < g.H)
+				v = load_row4<VEC>(x + (((int64_t)n * g.Cin + ci0 + ci) * g.H + gy) * g.W, w0 - 4 + 4 * f, g.W);
+			rp[q] = v;
+		}
+	};
+	auto store_chunk = [&]() {
+#pragma unroll
+		for (int q = 0; q < P::DY_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			float* d = s_dy + (idx / (P::TW / 4)) * P::DYS + 4 * (idx % (P::TW / 4));
+			d[0] = rdy[q].x; d[1] = rdy[q].y; d[2] = rdy[q].z; d[3] = rdy[q].w;
+		}
+#pragma unroll
+		for (int q = 0; q < P::P_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
+			float* d = s_patch + (rowid / KH) * P::CS + (rowid % KH) * P::PWS + 4 * f;
+			if (idx < P::PATCH_F4) { d[0] = rp[q].x; d[1] = rp[q].y; d[2] = rp[q].z; d[3] = rp[q].w; }
+		}
+	};
+
+	v16f acc[P::TAPS];
+#pragma unroll
+	for (int t = 0; t < P::TAPS; t++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
+
+	const float* pa = s_dy + (mt * 32 + lrow) * P::DYS + phalf * (P::TW / 2) + half;
+	const float* pb = s_patch + lrow * P::CS + phalf * (P::TW / 2) + half + 4 - g.pw;
+
+	if (begin < end) load_chunk(begin);
+	for (int chunk = begin; chunk < end; chunk++) {
+		store_chunk();
+		__syncthreads();
+		if (chunk + 1 < end) load_chunk(chunk + 1);
+#pragma unroll
+		for (int s = 0; s < P::TW / 4; s++) {
+			const float fa = pa[2 * s];
+			float fb[P::TAPS];
+#pragma unroll
+			for (int t = 0; t < P::TAPS; t++) fb[t] = pb[(t / KW) * P::PWS + (t % KW) + 2 * s];
+#pragma unroll
+			for (int t = 0; t < P::TAPS; t++) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb[t], acc[t], 0, 0, 0);
+		}
+		__syncthreads();
+	}
+
+	// pixel half 1 hands its sums to pixel half 0 of the same row tile, TAPS_PER_ROUND taps at a time
+#pragma unroll
+	for (int t0 = 0; t0 < P::TAPS; t0 += P::TAPS_PER_ROUND) {
+		if (phalf == 1) {
+#pragma unroll
+			for (int t = t0; t < t0 + P::TAPS_PER_ROUND && t < P::TAPS; t++)
+#pragma unroll
+				for (int r = 0; r < 16; r++) lds[((mt * P::TAPS_PER_ROUND + (t - t0)) * 16 + r) * 64 + lane] = acc[t][r];
+		}
+		__syncthreads();
+		if (phalf == 0) {
+#pragma unroll
+			for (int t = t0; t < t0 + P::TAPS_PER_ROUND && t < P::TAPS; t++)
+#pragma unroll
+				for (int r = 0; r < 16; r++) acc[t][r] += lds[((mt * P::TAPS_PER_ROUND + (t - t0)) * 16 + r) * 64 + lane];
+		}
+		__syncthreads();
+	}
+	if (phalf != 0) return;
+
+	const int Kc = g.Cin * P::TAPS;
+	float* out = partial + (int64_t)blockIdx.x * g.Cout * Kc;
+	const int ci = ci0 + lrow;
+	if (ci >= g.Cin) return;
+#pragma unroll
+	for (int r = 0; r < 16; r++) {
+		const int co = co0 + mt * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+		if (co >= g.Cout) continue;
+#pragma unroll
+		for (int t = 0; t < P::TAPS; t++) out[(int64_t)co * Kc + ci * P::TAPS + t] = acc[t][r];
+	}
+}
+
+// out[i] = sum over parts of partial[p][i].  A workgroup takes 64 outputs; its 16 groups of 64 lanes each add
+// every 16th part, then the 16 group sums are added in group order.
+__global__ __launch_bounds__(1024) void conv_reduce_partials_kernel(const float* __restrict__ partial, int parts, int64_t count, float* __restrict__ out)
+{
+	__shared__ float s[16][64];
+	const int o = threadIdx.x & 63, grp = threadIdx.x >> 6;
+	const int64_t idx = (int64_t)blockIdx.x * 64 + o;
+	float sum = 0.0f;
+	if (idx < count)
+		for (int p = grp; p < parts; p += 16) sum += partial[(int64_t)p * count + idx];
+	s[grp][o] = sum;
+	__syncthreads();
+	if (grp == 0 && idx < count) {
+		float tot = 0.0f;
+#pragma unroll
+		for (int q = 0; q < 16; q++) tot += s[q][o];
+		out[idx] = tot;
+	}
+}
+
+int conv_reduce_partials(const float* partial, int parts, int64_t count, float* out)
+{
+	conv_reduce_partials_kernel<<<dim3((unsigned)ceil_div(count, 64)), dim3(1024), 0, stream()>>>(partial, parts, count, out);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static bool patch_geometry(const ConvGeo& g)
+{
+	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw <= 4;
+}
+
+bool conv_patch_forward_takes(const ConvGeo& g, const float*, const float*)
+{
+	// below 5 input channels most of an 8-channel chunk would be padding
+	return patch_geometry(g) && g.Cin >= 5 && ceil_div((uint64_t)g.Cout, 64) < 65536;
+}
+
+int conv_patch_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
+{
+	typedef PatchFwd<3, 3> P;
+	const bool vec = g.W % 4 == 0 && aligned16(x);
+	const dim3 grid((unsigned)(ceil_div((uint64_t)g.Wo, P::TW) * ceil_div((uint64_t)g.Ho, P::TH)), (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)g.N);
+	set_kernel_name("conv2d_patch_forward_3x3_64x4x128");
+	if (vec) conv2d_patch_forward_kernel<3, 3, true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	else conv2d_patch_forward_kernel<3, 3, false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+bool conv_patch_wgrad_takes(const ConvGeo& g)
+{
+	return patch_geometry(g) && g.Cin >= 9 && ceil_div((uint64_t)g.Cout, 64) < 65536 && ceil_div((uint64_t)g.Cin, 32) < 65536 &&
+	       (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, 64) < (1ull << 31);
+}
+
+int conv_patch_wgrad_parts(const ConvGeo& g)
+{
+	typedef PatchWgrad<3, 3> P;
+	// two workgroups per CU over all (co block, ci block) pairs, at least four chunks per part
+	const uint64_t blocks = ceil_div((uint64_t)g.Cout, P::BM) * ceil_div((uint64_t)g.Cin, P::CIB);
+	const uint64_t chunks = (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, P::TW);
+	uint64_t parts = std::max<uint64_t>(1, 512 / blocks);
+	parts = std::min<uint64_t>(parts, std::max<uint64_t>(1, chunks / 4));
+	const uint64_t per = ceil_div(chunks, parts);
+	return (int)ceil_div(chunks, per);
+}
+
+int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts)
+{
+	typedef PatchWgrad<3, 3> P;
+	const uint64_t chunks = (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, P::TW);
+	const int per = (int)ceil_div(chunks, (uint64_t)parts);
+	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
+	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)ceil_div((uint64_t)g.Cin, P::CIB));
+	set_kernel_name("conv2d_patch_wgrad_3x3_64x32");
+	if (vec) conv2d_patch_wgrad_kernel<3, 3, true><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	else conv2d_patch_wgrad_kernel<3, 3, false><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+}  // namespace lten_hip

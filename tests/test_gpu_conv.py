@@ -72,8 +72,22 @@ def test_conv_layer_golden(gpu):
 
 @pytest.mark.parametrize("geo", [(2, 3, 9, 8, 4, 3, 3, 1, 1, 1, 1), (1, 2, 10, 7, 3, 3, 2, 0, 1, 2, 1),
                                  (2, 4, 6, 6, 5, 5, 5, 2, 2, 1, 1), (3, 16, 33, 29, 40, 3, 3, 1, 1, 1, 1),
-                                 (2, 8, 40, 40, 70, 3, 3, 1, 1, 2, 2), (2, 1, 64, 64, 32, 3, 3, 1, 1, 1, 1)])
-def test_conv_vs_oracle(gpu, ob, geo):
+                                 (2, 8, 40, 40, 70, 3, 3, 1, 1, 2, 2), (2, 1, 64, 64, 32, 3, 3, 1, 1, 1, 1),
+                                 # 3x3 stride 1 (LDS patch kernels): several column tiles and channel blocks, rows
+                                 # that are / are not a multiple of four floats, pad 0 / 1 / 2, ragged channel counts
+                                 (2, 20, 17, 136, 70, 3, 3, 1, 1, 1, 1), (1, 37, 12, 64, 33, 3, 3, 0, 0, 1, 1),
+                                 (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1)])
+@pytest.mark.parametrize("variant", [0, 1])
+def test_conv_vs_oracle(gpu, ob, geo, variant):
+    """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape."""
+    try:
+        gpu.set_option("conv_variant", variant)
+        _conv_vs_oracle(gpu, ob, geo)
+    finally:
+        gpu.set_option("conv_variant", 0)
+
+
+def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
     x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
@@ -87,8 +101,9 @@ def test_conv_vs_oracle(gpu, ob, geo):
     want_dw = np.empty_like(w)
     ob.oracle().oracle_conv2d_wgrad(*geo, x.reshape(-1), dy.reshape(-1), want_dw.reshape(-1), col)
     y, dw, fk = gpu_conv(gpu, geo, x, w, dy, bias)
+    print(f"  {geo}: forward via {fk}, wgrad via {gpu.last_kernel()}", flush=True)
     assert rel_err(y, want_y + bias[None, :, None, None]) < TOL, fk
-    assert rel_err(dw, want_dw) < TOL
+    assert rel_err(dw, want_dw) < TOL, gpu.last_kernel()
     assert rel_err(y, direct_conv(x, w, ph, pw, sh, sw) + bias[None, :, None, None]) < TOL
 
 
