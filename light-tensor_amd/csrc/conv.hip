@@ -230,6 +230,7 @@ int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W
 	LTEN_HIP_REQUIRE(x && w && y, "conv2d_forward: null pointer");
 	const int HW = g.Ho * g.Wo;
 	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
+	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
 	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");
@@ -253,6 +254,7 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
 	wgrad_split(g, slices, slice_len);
 	// enough for whichever kernel the call picks
 	uint64_t parts = (uint64_t)N * slices;
+	if (conv_smallk_takes(g)) parts = std::max<uint64_t>(parts, conv_smallk_wgrad_parts(g));
 	if (conv_patch_wgrad_takes(g)) parts = std::max<uint64_t>(parts, conv_patch_wgrad_parts(g));
 	return parts * Cout * Cin * kh * kw * sizeof(float);
 }
@@ -267,6 +269,11 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	LTEN_HIP_REQUIRE(dw != nullptr, "conv2d_wgrad: dw is null");
 	if (N == 0 || g.Ho * g.Wo == 0) return lten_hip_zero(dw, count * sizeof(float));
 	LTEN_HIP_REQUIRE(x && dy && workspace, "conv2d_wgrad: null pointer");
+	if (get_option(OPT_CONV_VARIANT) != 1 && conv_smallk_takes(g)) {
+		const int parts = conv_smallk_wgrad_parts(g);
+		if (int rc = conv_smallk_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
+		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
+	}
 	if (get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
 		const int parts = conv_patch_wgrad_parts(g);
 		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;

@@ -17,27 +17,10 @@
 
 namespace lten_hip {
 
-// Four consecutive floats of a row starting at column gx; columns outside [0, limit) read as 0.  With VEC
-// (limit % 4 == 0, gx % 4 == 0, 16-byte aligned row) the four are inside or outside together.
-template <bool VEC>
-__device__ __forceinline__ float4 load_row4(const float* row, int gx, int limit)
-{
-	float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-	if (VEC) {
-		if (gx >= 0 && gx + 3 < limit) v = *reinterpret_cast<const float4*>(row + gx);
-	} else {
-		if (gx >= 0 && gx < limit) v.x = row[gx];
-		if (gx + 1 >= 0 && gx + 1 < limit) v.y = row[gx + 1];
-		if (gx + 2 >= 0 && gx + 2 < limit) v.z = row[gx + 2];
-		if (gx + 3 >= 0 && gx + 3 < limit) v.w = row[gx + 3];
-	}
-	return v;
-}
-
 // ---------------------------------------------------------------------------------------------------------
 // Forward.  Workgroup tile: 64 output channels x (TH = 4 rows x TW = 128 columns) of one image; wavefront
-// `wave` owns row `wave` (2 x 4 MFMA tiles of 32 x 32).  The input channels are walked in chunks of CB = 8:
-// per chunk the patch [8][TH + KH - 1][PWS] and the weights of those channels are stored to LDS, the next
+// `wave` owns row `wave` (2 x 4 MFMA tiles of 32 x 32).  The input channels are walked in chunks of CB = 4:
+// per chunk the patch [4][TH + KH - 1][PWS] and the weights of those channels are stored to LDS, the next
 // chunk's values are fetched to registers, and (CB / 2) * KH * KW MFMA steps run; step (cp, i, j) multiplies
 // tap (i, j) of channels 2cp (lanes 0-31) and 2cp + 1 (lanes 32-63).
 //
@@ -128,18 +111,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		store_chunk();
 		__syncthreads();
 		if (c0 + P::CB < g.Cin) load_chunk(c0 + P::CB);
+		// operands of step s + 1 are read while the MFMAs of step s issue, one LDS read behind each MFMA
+		float fa[2][2], fb[2][4];
+		auto read_operand = [&](int s, int e) {
+			const int cp = s / P::TAPS, tap = s % P::TAPS, i = tap / KW, j = tap % KW;
+			if (e < 2) fa[s & 1][e] = pa[s * 2 * P::WROW + e * 32];
+			else fb[s & 1][e - 2] = pb[(2 * cp * P::PR + i) * P::PWS + j + (e - 2) * 32];
+		};
+#pragma unroll
+		for (int e = 0; e < 6; e++) read_operand(0, e);
 #pragma unroll
 		for (int s = 0; s < P::KSTEPS; s++) {
-			const int cp = s / P::TAPS, tap = s % P::TAPS, i = tap / KW, j = tap % KW;
-			float fa[2], fb[4];
 #pragma unroll
-			for (int m = 0; m < 2; m++) fa[m] = pa[s * 2 * P::WROW + m * 32];
-#pragma unroll
-			for (int t = 0; t < 4; t++) fb[t] = pb[(2 * cp * P::PR + i) * P::PWS + j + t * 32];
-#pragma unroll
-			for (int m = 0; m < 2; m++)
-#pragma unroll
-				for (int t = 0; t < 4; t++) acc[m][t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[m], fb[t], acc[m][t], 0, 0, 0);
+			for (int e = 0; e < 8; e++) {
+				acc[e >> 2][e & 3] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1][e >> 2], fb[s & 1][e & 3], acc[e >> 2][e & 3], 0, 0, 0);
+				if (e < 6 && s + 1 < P::KSTEPS) read_operand(s + 1, e);
+				__builtin_amdgcn_sched_barrier(0);
+			}
 		}
 		__syncthreads();
 	}
@@ -255,14 +243,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		store_chunk();
 		__syncthreads();
 		if (chunk + 1 < end) load_chunk(chunk + 1);
+		// operands of step s + 1 are read while the MFMAs of step s issue
+		float fa[2], fb[2][P::TAPS];
+		auto read_operand = [&](int s, int t) { fb[s & 1][t] = pb[(t / KW) * P::PWS + (t % KW) + 2 * s]; };
+		fa[0] = pa[0];
+#pragma unroll
+		for (int t = 0; t < P::TAPS; t++) read_operand(0, t);
 #pragma unroll
 		for (int s = 0; s < P::TW / 4; s++) {
-			const float fa = pa[2 * s];
-			float fb[P::TAPS];
 #pragma unroll
-			for (int t = 0; t < P::TAPS; t++) fb[t] = pb[(t / KW) * P::PWS + (t % KW) + 2 * s];
-#pragma unroll
-			for (int t = 0; t < P::TAPS; t++) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb[t], acc[t], 0, 0, 0);
+			for (int t = 0; t < P::TAPS; t++) {
+				acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1], fb[s & 1][t], acc[t], 0, 0, 0);
+				if (s + 1 < P::TW / 4) {
+					if (t == 0) fa[(s + 1) & 1] = pa[2 * (s + 1)];
+					read_operand(s + 1, t);
+				}
+				__builtin_amdgcn_sched_barrier(0);
+			}
 		}
 		__syncthreads();
 	}
@@ -326,8 +323,6 @@ int conv_reduce_partials(const float* partial, int parts, int64_t count, float* 
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }
-
-static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 static bool patch_geometry(const ConvGeo& g)
 {

@@ -76,7 +76,12 @@ def test_conv_layer_golden(gpu):
                                  # 3x3 stride 1 (LDS patch kernels): several column tiles and channel blocks, rows
                                  # that are / are not a multiple of four floats, pad 0 / 1 / 2, ragged channel counts
                                  (2, 20, 17, 136, 70, 3, 3, 1, 1, 1, 1), (1, 37, 12, 64, 33, 3, 3, 0, 0, 1, 1),
-                                 (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1)])
+                                 (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1),
+                                 # stride 1 with Cin*kh*kw <= 32 (first-layer kernels): ragged widths, two column
+                                 # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
+                                 (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
+                                 (1, 20, 9, 132, 33, 1, 1, 0, 0, 1, 1), (2, 3, 16, 36, 64, 3, 3, 0, 0, 1, 1),
+                                 (5, 2, 7, 9, 3, 2, 7, 1, 4, 1, 1)])
 @pytest.mark.parametrize("variant", [0, 1])
 def test_conv_vs_oracle(gpu, ob, geo, variant):
     """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape."""
