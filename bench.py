@@ -246,6 +246,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run output check")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config records for configs 1, 2, 4, 5")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="run only the plain copy kernel on buffers of this size (what FETCH_SIZE / WRITE_SIZE "
+                         "counters are scaled against) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (the path has no collective to scale); use --gpus 1")
@@ -253,6 +256,22 @@ def main():
     lt = load_package()
     from light_tensor_amd import workloads as wl
     lt.init(0)
+
+    if args.copy_calibration:
+        nbytes = args.copy_calibration << 20
+        src, dst = lt.DeviceBuffer(nbytes), lt.DeviceBuffer(nbytes)
+        lt.check(lt.lib().lten_hip_zero(src.ptr, nbytes))
+        for _ in range(max(args.warmup, 1)):
+            lt.check(lt.lib().lten_hip_copy_kernel(src.ptr, dst.ptr, nbytes))
+        lt.sync()
+        timer = lt.Timer()
+        timer.start()
+        for _ in range(args.steps):
+            lt.check(lt.lib().lten_hip_copy_kernel(src.ptr, dst.ptr, nbytes))
+        ms = timer.stop_ms() / args.steps
+        print(json.dumps({"copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "us": round(ms * 1e3, 2),
+                          "GB_per_s": round(2 * nbytes / ms / 1e6, 1)}))
+        return
 
     M = N = K = 4096
     X, W, sc, zp = wl.cfg3()

@@ -408,6 +408,11 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
 	}
+	// small outputs: one launch that also takes the zero-point sums (same option switches it off)
+	if (get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+		const int rc = qdirect_dispatch(p, out, bias, zpA, zpB);
+		if (rc >= 0) return rc;
+	}
 
 	const int coef_a = 128 - zpB, coef_b = 128 - zpA;
 	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {

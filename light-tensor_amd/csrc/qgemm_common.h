@@ -68,6 +68,9 @@ __device__ __forceinline__ unsigned requant(int acc, float mult, float zp)
 // Weight-streaming kernel for M <= 16 (qskinny.hip); computes its own zero-point sums.  -1 = does not fit.
 int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b);
 
+// One-launch kernel for small NT products (qdirect.hip); computes its own zero-point sums.  -1 = does not fit.
+int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b);
+
 // Dispatch of the tuned square-ish kernels (qgemm_fast.hip).  Returns -1 when no fast variant fits.
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant);
 

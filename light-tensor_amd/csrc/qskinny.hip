@@ -1,14 +1,14 @@
 // Weight-streaming int8 FC for skinny activations (M <= 16 rows against W[N x K], both contiguous in K).
 //
 // The work is one pass over W (N*K bytes, read once from HBM); everything else is noise, so the kernel is
-// organised around that stream.  A workgroup owns 16 consecutive rows of W; its 8 wavefronts split K among
-// themselves.  Each wavefront pulls its [16 rows x K/8] slab into LDS with direct global->LDS loads — one
+// organised around that stream.  A workgroup takes 16 consecutive rows of W at a time (then the next such
+// group, one workgroup per CU); its 8 wavefronts split K among themselves.  Each wavefront pulls its [16 rows x K/8] slab into LDS with direct global->LDS loads — one
 // wave-wide load covers 1 KB of one row, so every request is a run of whole cache lines — keeps the whole
 // slab in flight at once (128 KB per CU), then walks it with ds_read_b128 in the lane layout of the
 // 16x16x64 int8 MFMA (lane -> row lane%16, 16-byte k-group lane/16).  Rows are padded by 16 bytes in LDS
 // so that the 16 rows a read touches fall in different banks.  The activations (at most 16 x K bytes,
-// L2 resident) are fetched straight into the other MFMA operand; rows beyond M read as the zero of the
-// signed domain.  The 8 partial 16x16 accumulators meet in LDS, and one wavefront applies the zero-point
+// L2 resident) are fetched straight into the other MFMA operand once per workgroup and stay in registers
+// for all its row groups; rows beyond M read as the zero of the signed domain.  The 8 partial 16x16 accumulators meet in LDS, and one wavefront applies the zero-point
 // terms and the requantize of l-ten/math_fns.cpp:1469-1474 and writes the M x 16 outputs.
 //
 // As in the tiled kernels, bytes are XORed with 0x80 on their way into the MFMA (uint8 -> int8) and the
@@ -16,6 +16,8 @@
 // registers with dot4 instructions, only when their coefficient is non-zero.
 #include "common.h"
 #include "qgemm_common.h"
+
+#include <algorithm>
 
 namespace lten_hip {
 
@@ -31,100 +33,120 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 	constexpr int ROW = KW + 16;         // padded LDS row pitch
 	constexpr int SLAB = 16 * ROW;       // one wavefront's slab
 	constexpr int LOADS_PER_ROW = KW / 1024;
-	__shared__ __attribute__((aligned(1024))) uint8_t smem[WAVES * SLAB > WAVES * 1024 ? WAVES * SLAB : WAVES * 1024];
-	__shared__ int sums_a[WAVES][16], sums_b[WAVES][16];
+	__shared__ __attribute__((aligned(1024))) uint8_t smem[WAVES * SLAB];
+	__shared__ __attribute__((aligned(16))) int partial[2][WAVES][64 * 4];  // per row group parity: the k-slices' accumulators
+	__shared__ int sums_a[2][WAVES][16], sums_b[2][WAVES][16];
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int n0 = blockIdx.x * 16;
 	const int kbeg = wave * KW;
 	const uint32_t slab_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + wave * SLAB;
+	const int groups = p.N / 16;
 
-	// the whole slab goes in flight before anything is consumed
+	// the whole slab of a row group goes in flight before anything is consumed
+	auto issue_slab = [&](int group) {
+		const uint8_t* base = p.B + (int64_t)group * 16 * p.K + kbeg;
 #pragma unroll
-	for (int r = 0; r < 16; r++)
+		for (int r = 0; r < 16; r++)
 #pragma unroll
-		for (int c = 0; c < LOADS_PER_ROW; c++)
-			skinny_async_load16(slab_addr + r * ROW + c * 1024, p.B + (int64_t)(n0 + r) * p.K + kbeg + c * 1024, lane * 16);
+			for (int c = 0; c < LOADS_PER_ROW; c++) skinny_async_load16(slab_addr + r * ROW + c * 1024, base + (int64_t)r * p.K + c * 1024, lane * 16);
+	};
+	issue_slab(blockIdx.x);
 
+	// the activations of this wavefront's k-slice stay in registers for every row group the workgroup takes
 	const int lrow = lane & 15, lgrp = lane >> 4;
 	const uint8_t* xrow = p.A + (int64_t)lrow * p.K + kbeg + lgrp * 16;
 	const bool xvalid = lrow < p.M;
 	const uint8_t* wfrag = smem + wave * SLAB + lrow * ROW + lgrp * 16;
-
-	v4i acc = { 0, 0, 0, 0 };
-	int sa = 0, sb = 0;
 	constexpr int STEPS = KW / 64;
 	v4i fx[STEPS];
+	int sa = 0;
 #pragma unroll
 	for (int s = 0; s < STEPS; s++) {
 		fx[s] = v4i{ (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
 		if (xvalid) fx[s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
 	}
-	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab and activations have landed (no other wave reads this slab)
+	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
 	for (int s = 0; s < STEPS; s++) {
-		v4i fw = *reinterpret_cast<const v4i*>(wfrag + s * 64);
-		fw = flip_sign_bits(fw);
-		const v4i fa = flip_sign_bits(fx[s]);
-		if (SUM_B) {
-			sb = __builtin_amdgcn_sdot4(fw.x, 0x01010101, sb, false);
-			sb = __builtin_amdgcn_sdot4(fw.y, 0x01010101, sb, false);
-			sb = __builtin_amdgcn_sdot4(fw.z, 0x01010101, sb, false);
-			sb = __builtin_amdgcn_sdot4(fw.w, 0x01010101, sb, false);
-		}
+		fx[s] = flip_sign_bits(fx[s]);
 		if (SUM_A) {
-			sa = __builtin_amdgcn_sdot4(fa.x, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fa.y, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fa.z, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fa.w, 0x01010101, sa, false);
+			sa = __builtin_amdgcn_sdot4(fx[s].x, 0x01010101, sa, false);
+			sa = __builtin_amdgcn_sdot4(fx[s].y, 0x01010101, sa, false);
+			sa = __builtin_amdgcn_sdot4(fx[s].z, 0x01010101, sa, false);
+			sa = __builtin_amdgcn_sdot4(fx[s].w, 0x01010101, sa, false);
 		}
-		// MFMA A operand = activations (rows m), B operand = weights (columns n):
-		// lane (lrow, lgrp), register e holds out[m = 4*lgrp + e][n = lrow]
-		acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fw, acc, 0, 0, 0);
 	}
-	if (SUM_A || SUM_B) {
-		// a lane holds the sums of its 16-byte k-group only: fold the four k-groups (lanes l, l+16, l+32, l+48)
-		sa += __shfl_xor(sa, 16, 64); sa += __shfl_xor(sa, 32, 64);
-		sb += __shfl_xor(sb, 16, 64); sb += __shfl_xor(sb, 32, 64);
-		if (lane < 16) { sums_a[wave][lane] = sa; sums_b[wave][lane] = sb; }
-	}
+	// a lane holds the sums of its 16-byte k-group only: fold the four k-groups (lanes l, l+16, l+32, l+48)
+	if (SUM_A) { sa += __shfl_xor(sa, 16, 64); sa += __shfl_xor(sa, 32, 64); }
 
-	// partial accumulators of the 8 k-slices meet in LDS (each wave overwrites the head of its own slab)
-	__syncthreads();
-	*reinterpret_cast<v4i*>(smem + wave * 1024 + lane * 16) = acc;
-	__syncthreads();
-	if (wave != 0) return;
-	v4i tot = { 0, 0, 0, 0 };
+	int parity = 0;
+	for (int group = blockIdx.x; group < groups; group += gridDim.x, parity ^= 1) {
+		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab has landed (no other wave reads this slab)
+		v4i acc = { 0, 0, 0, 0 };
+		int sb = 0;
 #pragma unroll
-	for (int w = 0; w < WAVES; w++) tot += *reinterpret_cast<const v4i*>(smem + w * 1024 + lane * 16);
-	int tsa[4] = { 0, 0, 0, 0 }, tsb = 0;
-	if (SUM_A || SUM_B) {
-#pragma unroll
-		for (int w = 0; w < WAVES; w++) {
-			tsb += sums_b[w][lrow];
-#pragma unroll
-			for (int e = 0; e < 4; e++) tsa[e] += sums_a[w][lgrp * 4 + e];
+		for (int s = 0; s < STEPS; s++) {
+			v4i fw = *reinterpret_cast<const v4i*>(wfrag + s * 64);
+			fw = flip_sign_bits(fw);
+			if (SUM_B) {
+				sb = __builtin_amdgcn_sdot4(fw.x, 0x01010101, sb, false);
+				sb = __builtin_amdgcn_sdot4(fw.y, 0x01010101, sb, false);
+				sb = __builtin_amdgcn_sdot4(fw.z, 0x01010101, sb, false);
+				sb = __builtin_amdgcn_sdot4(fw.w, 0x01010101, sb, false);
+			}
+			// MFMA A operand = activations (rows m), B operand = weights (columns n):
+			// lane (lrow, lgrp), register e holds out[m = 4*lgrp + e][n = lrow]
+			acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx[s], fw, acc, 0, 0, 0);
 		}
-	}
-	const int n = n0 + lrow;
-	// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
-	//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-	const int base = coef_b * tsb + p.K * coef_a * coef_b + (bias ? bias[n] : 0);
+		// the slab is consumed (its values sit in registers): the next row group's slab can start to arrive
+		if (group + (int)gridDim.x < groups) {
+			asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+			issue_slab(group + gridDim.x);
+		}
+		if (SUM_A || SUM_B) {
+			sb += __shfl_xor(sb, 16, 64); sb += __shfl_xor(sb, 32, 64);
+			if (lane < 16) { sums_a[parity][wave][lane] = sa; sums_b[parity][wave][lane] = sb; }
+		}
+		// partial accumulators of the k-slices meet in LDS; the two parities keep wave 0's reads of one row
+		// group apart from the other waves' writes of the next
+		*reinterpret_cast<v4i*>(&partial[parity][wave][lane * 4]) = acc;
+		__syncthreads();
+		if (wave != 0) continue;
+		v4i tot = { 0, 0, 0, 0 };
 #pragma unroll
-	for (int e = 0; e < 4; e++) {
-		const int m = lgrp * 4 + e;
-		if (m >= p.M) continue;
-		const int v = tot[e] + base + coef_a * tsa[e];
-		if (OUT == Q_OUT_ACC) static_cast<int*>(p.C)[(int64_t)m * p.N + n] = v;
-		else static_cast<uint8_t*>(p.C)[(int64_t)m * p.N + n] = (uint8_t)requant<OUT>(v, p.mult, p.zp_c);
+		for (int w = 0; w < WAVES; w++) tot += *reinterpret_cast<const v4i*>(&partial[parity][w][lane * 4]);
+		int tsa[4] = { 0, 0, 0, 0 }, tsb = 0;
+		if (SUM_A || SUM_B) {
+#pragma unroll
+			for (int w = 0; w < WAVES; w++) {
+				tsb += sums_b[parity][w][lrow];
+#pragma unroll
+				for (int e = 0; e < 4; e++) tsa[e] += sums_a[parity][w][lgrp * 4 + e];
+			}
+		}
+		const int n = group * 16 + lrow;
+		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
+		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
+		const int base = coef_b * tsb + p.K * coef_a * coef_b + (bias ? bias[n] : 0);
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			const int m = lgrp * 4 + e;
+			if (m >= p.M) continue;
+			const int v = tot[e] + base + coef_a * tsa[e];
+			if (OUT == Q_OUT_ACC) static_cast<int*>(p.C)[(int64_t)m * p.N + n] = v;
+			else static_cast<uint8_t*>(p.C)[(int64_t)m * p.N + n] = (uint8_t)requant<OUT>(v, p.mult, p.zp_c);
+		}
 	}
 }
 
 template <int WAVES, int KW>
 static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, const char* name)
 {
-	const dim3 grid((unsigned)(p.N / 16)), block(WAVES * 64);
+	// as many workgroups as fit the CUs' LDS at once (one per CU at K = 8192); each walks row groups blockIdx.x, blockIdx.x + grid, ...
+	constexpr int LDS_BYTES = WAVES * 16 * (KW + 16) + 2 * WAVES * 1024 + 4 * WAVES * 64;
+	constexpr int PER_CU = (160 * 1024) / LDS_BYTES;
+	const dim3 grid((unsigned)std::min<int64_t>(p.N / 16, 256 * PER_CU)), block(WAVES * 64);
 	set_kernel_name(name);
 	const bool sum_a = coef_a != 0, sum_b = coef_b != 0;
 #define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, KW, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b)

@@ -181,6 +181,40 @@ def test_weight_streaming_kernel(gpu, ob, shape):
         assert np.array_equal(Cg, Ct)
 
 
+@pytest.mark.parametrize("shape", [(64, 512, 784), (1, 10, 16), (17, 33, 48), (100, 70, 1040), (16, 16, 16384), (33, 250, 2064)])
+def test_small_output_kernel(gpu, ob, shape):
+    """At most 512 output tiles of 16x16, K % 16 == 0: the one-launch kernel with in-kernel zero-point sums (ragged
+    M and N, K tails inside a 64-byte step, both wavefront counts), against the oracle and the tiled kernels."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    for zp, scales in (([128, 128, 128], [0.02, 0.013, 0.9]), ([0, 128, 128], [1 / 255, 0.01, 0.05]),
+                       ([128, 200, 0], [0.02, 0.013, 0.9]), ([17, 250, 100], [0.5, 0.5, 0.2])):
+        bias = rng.integers(-9999, 9999, N).astype(np.int32) if zp[0] != 128 else None
+        Cg = run_case(gpu, ob, A, B, scales, np.array(zp, np.uint8), bias=bias)
+        assert gpu.last_kernel().startswith("qdirect_16x16"), gpu.last_kernel()
+        gpu.set_option("qskinny", 2)
+        try:
+            Ct = run_case(gpu, ob, A, B, scales, np.array(zp, np.uint8), bias=bias)
+            assert not gpu.last_kernel().startswith("qdirect")
+        finally:
+            gpu.set_option("qskinny", 0)
+        assert np.array_equal(Cg, Ct)
+
+
+def test_weight_streaming_many_row_groups(gpu, ob):
+    """More groups of 16 weight rows than workgroups (600 against 256): a workgroup walks two or three groups
+    with the activations kept in registers; zero-point sums and bias active."""
+    M, N, K = 5, 9600, 8192
+    rng = np.random.default_rng(11)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    bias = rng.integers(-9999, 9999, N).astype(np.int32)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([17, 250, 100], np.uint8), bias=bias)
+    assert gpu.last_kernel() == "qskinny_mfma_w8_k1024"
+
+
 @pytest.mark.parametrize("M", [1, 4, 16])
 def test_cfg4_skinny(gpu, wl, M):
     X, W, sc, zp = wl.cfg4(M)
