@@ -247,7 +247,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		// Few output tiles and a long K: the LDS-tiled kernels would leave most CUs idle while a handful of
 		// workgroups walk K in sequence; the direct kernel cuts K across the wavefronts of a workgroup instead.
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32) * batch;
-		if (tiles32 <= 1024) choice = 4;
+		// (with a short K and enough 64x64 tiles to occupy half the CUs the tiled kernel is the faster one)
+		if (tiles32 <= 1024 && !(tiles64 >= 128 && K <= 256)) choice = 4;
 		else choice = tiles128 >= 128 ? 1 : 2;
 	}
 	switch (choice) {
