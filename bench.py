@@ -4,10 +4,10 @@
 A step is one lten_hip_quantized_matmul call (the whole FC forward: MFMA GEMM with the
 zero-point correction and the requantize fused in) over one synthetic batch whose operands
 are already resident in HBM.  Prints ONE JSON line.  The headline fields describe config 3;
-"configs" adds one record per other benchmark configuration (1, 2, 4, 5), each with its own
-roofline figure and the CPU path timed beside it.
+"configs" adds one record per other benchmark configuration (1, 2, 4, 5) and one for the Conv2d_q
+forward, each with its own roofline figure and the CPU path timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra] [--copy-calibration MiB]
 """
 import argparse
 import ctypes as C
@@ -29,7 +29,7 @@ FP32_MFMA_PEAK_TFLOPS = 157.3  # MI355X dense fp32 MFMA, published
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published: 8 TB/s
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the
-# same counters on the plain copy kernel (profiles/qgemm_fast_cfg3_4096.md): FETCH_SIZE reads half the bytes
+# same counters on the plain copy kernel (--copy-calibration): FETCH_SIZE reads half the bytes
 # the copy kernel is known to fetch (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
 TRAFFIC_BYTES = {"qgemm_fast_256x256x128_w2x4_s2": 49250 * 1024 * 2.0 + 16384 * 1024 * 1.0}
 
@@ -235,6 +235,26 @@ def extra_configs(lt, wl, with_cpu):
             rec.update(cpu_ms=round(t * 1e3, 1), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)),
                        cpu_sample=f"{sample} of {Nimg} images, scaled", speedup=round(t * 1e3 / (ms_f + ms_w), 1))
         out.append(rec)
+
+    # ---- beyond the five configs: Conv2d_q forward, the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network
+    geo = (64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1)
+    rng = np.random.default_rng(7)
+    xq = rng.integers(0, 256, (64, 1, 28, 28), dtype=np.uint8)
+    wq = rng.integers(0, 256, (10, 1, 5, 5), dtype=np.uint8)
+    sc, zp = [1.0 / 255.0, 0.01, 0.05], [0, 128, 128]
+    dxq, dwq, dyq = D.from_numpy(xq), D.from_numpy(wq), D(64 * 10 * 24 * 24)
+    wsq = D(max(int(l.lten_hip_conv2dq_workspace_bytes(*geo)), 16))
+    qpq = lt.qparams3(sc, zp)
+    ms = timed(lt, lambda: lt.check(l.lten_hip_conv2dq_forward(*geo, dxq.ptr, dwq.ptr, None, qpq, dyq.ptr, wsq.ptr)), 100)
+    nbytes = xq.nbytes + wq.nbytes + 64 * 10 * 24 * 24
+    rec = {"config": "Conv2d_q forward 64x1x28x28 -> 10 ch 5x5 (l-ten's quantized MNIST conv1, batch 64)", "gpu_us": round(ms * 1e3, 2),
+           "kernel": lt.last_kernel(), "bound": "launch latency", "algorithmic_bytes": nbytes}
+    if with_cpu:
+        f = (lambda: ob.ref_conv2dq_forward(geo, xq, wq, sc, zp)) if ob.ref() is not None else (lambda: ob.conv2dq_forward(geo, xq, wq, sc, zp, want_acc=False))
+        t = best_of(f, 3)
+        rec.update(cpu_ms=round(t * 1e3, 3), cpu_cores=1, cpu_kind="reference" if ob.ref() is not None else "port",
+                   speedup=round(t * 1e3 / ms, 1))
+    out.append(rec)
     return out
 
 

@@ -156,6 +156,26 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
                                                int kernel_h, int kernel_w, int pad_h, int pad_w,
                                                int stride_h, int stride_w);
 
+/* Conv2d_q::forward (l-ten/conv2d.cpp:265-387; CPU-only in l-ten, "Conv2d_q only supports the CPU device
+ * type" :376) for the whole batch: x[N][Cin][H][W] u8, w[Cout][Cin*kh*kw] u8, y[N][Cout][Ho][Wo] u8, with
+ * qparams in the order input, weights, output (the layer's qparams_in_, qparams_wt_, qparams_out_; l-ten hands
+ * them to quantized_matmul as [weights, input, output], :347-349).  Positions outside the image count as the
+ * byte 0, as in l-ten's column buffer.  bias, when not null, holds Ho*Wo ints and is added per output position:
+ * that is what l-ten's call computes (quantized_matmul indexes the bias by GEMM column, l-ten/math_fns.cpp:1470-1473,
+ * and the columns of this product are output positions).  workspace: lten_hip_conv2dq_workspace_bytes device
+ * bytes, 16-byte aligned (column buffer and zero-point terms of the fallback for windows above 64 taps). */
+uint64_t lten_hip_conv2dq_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                                          int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w);
+int lten_hip_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kernel_h,
+                             int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w, const uint8_t* x,
+                             const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qparams_in_wt_out,
+                             uint8_t* y, void* workspace);
+/* Same computation, stopping before the requantize (int32 `element` values).  For parity checks. */
+int lten_hip_conv2dq_forward_acc(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kernel_h,
+                                 int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w, const uint8_t* x,
+                                 const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qparams_in_wt_out,
+                                 int32_t* acc, void* workspace);
+
 /* ----------------------------------------------------------------------- measurement */
 
 /* HIP events on the library's stream; no counterpart in l-ten (its benchmarks use

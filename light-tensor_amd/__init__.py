@@ -59,6 +59,9 @@ _SIGNATURES = {
     "lten_hip_conv2d_forward_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),
     "lten_hip_conv2d_wgrad_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),
     "lten_hip_conv2d_wgrad_workspace_bytes": (u64, [u64] * 5 + [C.c_int] * 6),
+    "lten_hip_conv2dq_workspace_bytes": (u64, [u64] * 5 + [C.c_int] * 6),
+    "lten_hip_conv2dq_forward": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, C.POINTER(QParams), vp, vp]),
+    "lten_hip_conv2dq_forward_acc": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, C.POINTER(QParams), vp, vp]),
     "lten_hip_event_create": (C.c_int, [C.POINTER(vp)]),
     "lten_hip_event_record": (C.c_int, [vp]),
     "lten_hip_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
@@ -246,4 +249,26 @@ def qgemm_host(A, B, scales, zps, tA=False, tB=True, bias=None, want_acc=False, 
         dacc = DeviceBuffer(max(4 * M * N, 4))
         quantized_matmul_acc(tA, tB, M, N, K, dA, dB, dacc, qp, dbias, ws)
         acc = dacc.numpy(np.int32, (M, N))
+    return out, acc
+
+
+def conv2dq_host(geo, x, w, scales, zps, bias=None, want_acc=False):
+    """numpy in / numpy out convenience around lten_hip_conv2dq_forward[_acc]; scales / zps ordered (input, weights,
+    output); geo = (N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw).  Copies included."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    Ho, Wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    dx = DeviceBuffer.from_numpy(np.ascontiguousarray(x, dtype=np.uint8))
+    dw = DeviceBuffer.from_numpy(np.ascontiguousarray(w, dtype=np.uint8))
+    db = DeviceBuffer.from_numpy(np.asarray(bias, dtype=np.int32)) if bias is not None else None
+    ws = DeviceBuffer(max(int(lib().lten_hip_conv2dq_workspace_bytes(*geo)), 16))
+    qp = qparams3(scales, zps)
+    count = N * Cout * Ho * Wo
+    dy = DeviceBuffer(max(count, 1))
+    check(lib().lten_hip_conv2dq_forward(*geo, dx.ptr, dw.ptr, _p(db), qp, dy.ptr, ws.ptr))
+    out = dy.numpy(np.uint8, (N, Cout, Ho, Wo))
+    acc = None
+    if want_acc:
+        dacc = DeviceBuffer(max(4 * count, 4))
+        check(lib().lten_hip_conv2dq_forward_acc(*geo, dx.ptr, dw.ptr, _p(db), qp, dacc.ptr, ws.ptr))
+        acc = dacc.numpy(np.int32, (N, Cout, Ho, Wo))
     return out, acc

@@ -1,0 +1,171 @@
+// Conv2d_q forward: uint8 input (NCHW) x uint8 weights -> int32 -> requantized uint8, for the whole batch.
+//
+// l-ten does this per image as a u8 im2col followed by quantized_matmul(false, false, Cout, Ho*Wo, Cin*kh*kw)
+// with the weights as the left operand (l-ten/conv2d.cpp:355-372): element = sum_k w[co][k] * col[k][p]
+//   - zpW * sum_k col[k][p] - zpIn * sum_k w[co][k] + K * zpW * zpIn (+ bias[p]), then the requantize of
+// l-ten/math_fns.cpp:1474.  Positions outside the image hold the byte 0 in the column buffer (not the zero point).
+//
+// Windows of at most 64 taps (the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network has 25) run in one
+// launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
+// and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
+// LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
+// Longer windows follow l-ten's own decomposition per image: im2col_u8 into the caller's workspace, then the
+// int8 GEMM of qgemm.hip.
+#include "conv_common.h"
+#include "qgemm_common.h"
+
+namespace lten_hip {
+
+constexpr int CQ_MAXK = 64, CQ_CO = 64;
+
+template <int OUT>
+__global__ __launch_bounds__(256) void conv2dq_direct_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
+                                                             const int32_t* __restrict__ bias, int zp_in, int zp_w, float mult, float zp_out,
+                                                             void* __restrict__ y)
+{
+	__shared__ __attribute__((aligned(16))) uint32_t s_w[CQ_CO][CQ_MAXK / 4];
+	__shared__ int s_wsum[CQ_CO];
+	const int tid = threadIdx.x;
+	const int K = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	const int co0 = blockIdx.y * CQ_CO, nco = min(CQ_CO, g.Cout - co0);
+
+	// weights of this block's output channels, four taps per dword, taps past K as zero bytes
+	for (int idx = tid; idx < CQ_CO * (CQ_MAXK / 4); idx += 256) {
+		const int co = idx / (CQ_MAXK / 4), d = idx % (CQ_MAXK / 4);
+		uint32_t v = 0;
+		if (co < nco)
+			for (int b = 0; b < 4; b++)
+				if (4 * d + b < K) v |= (uint32_t)w[(int64_t)(co0 + co) * K + 4 * d + b] << (8 * b);
+		s_w[co][d] = v;
+	}
+	__syncthreads();
+	if (tid < CQ_CO) {
+		uint32_t sum = 0;
+		for (int d = 0; d < CQ_MAXK / 4; d++) sum = __builtin_amdgcn_udot4(s_w[tid][d], 0x01010101u, sum, false);
+		s_wsum[tid] = (int)sum;
+	}
+	__syncthreads();
+
+	const int64_t gid = (int64_t)blockIdx.x * 256 + tid;
+	if (gid >= (int64_t)g.N * HW) return;
+	const int n = (int)(gid / HW), pos = (int)(gid % HW);
+	const int ho = pos / g.Wo, wo = pos % g.Wo;
+	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
+	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+
+	// the window, tap k in byte k % 4 of dword k / 4
+	uint32_t xk[CQ_MAXK / 4];
+#pragma unroll
+	for (int d = 0; d < CQ_MAXK / 4; d++) xk[d] = 0;
+#pragma unroll
+	for (int k = 0; k < CQ_MAXK; k++) {
+		if (k >= K) break;
+		const int j = k % g.kw, i = (k / g.kw) % g.kh, ci = k / (g.kw * g.kh);
+		const int yy = y0 + i, xx = x0 + j;
+		if (yy >= 0 && yy < g.H && xx >= 0 && xx < g.W) xk[k / 4] |= (uint32_t)xn[((int64_t)ci * g.H + yy) * g.W + xx] << (8 * (k % 4));
+	}
+	uint32_t xsum = 0;
+#pragma unroll
+	for (int d = 0; d < CQ_MAXK / 4; d++) xsum = __builtin_amdgcn_udot4(xk[d], 0x01010101u, xsum, false);
+	// l-ten/math_fns.cpp:1362-1380,1433: row_vector[p] = -zpA * sum_k B[k][p] with A = weights; broadcast = K zpA zpB
+	const int base = -zp_w * (int)xsum + K * zp_w * zp_in + (bias ? bias[pos] : 0);
+
+	for (int co = 0; co < nco; co++) {
+		uint32_t dot = 0;
+#pragma unroll
+		for (int d = 0; d < CQ_MAXK / 4; d++) dot = __builtin_amdgcn_udot4(s_w[co][d], xk[d], dot, false);
+		const int v = (int)dot + base - zp_in * s_wsum[co];
+		const int64_t o = ((int64_t)n * g.Cout + co0 + co) * HW + pos;
+		if (OUT == Q_OUT_ACC) static_cast<int*>(y)[o] = v;
+		else static_cast<uint8_t*>(y)[o] = (uint8_t)requant<OUT>(v, mult, zp_out);
+	}
+}
+
+static int make_geo_q(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh, int sw)
+{
+	LTEN_HIP_REQUIRE(kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0, "conv2dq: bad kernel geometry");
+	LTEN_HIP_REQUIRE(N < 65536 && Cin < (1u << 20) && Cout < (1u << 20) && H < (1u << 15) && W < (1u << 15), "conv2dq: dimension too large");
+	LTEN_HIP_REQUIRE(Cin * H * W < (1ull << 31) && Cout * H * W < (1ull << 31), "conv2dq: one image must stay below 2^31 elements");
+	const int64_t eh = (int64_t)H + 2 * ph - kh, ew = (int64_t)W + 2 * pw - kw;
+	LTEN_HIP_REQUIRE(eh >= 0 && ew >= 0, "conv2dq: kernel larger than the padded image");
+	LTEN_HIP_REQUIRE(Cin * (uint64_t)kh * kw * 255 * 255 < (1ull << 31), "conv2dq: Cin*kh*kw too large for an int32 accumulator");
+	g.N = (int)N; g.Cin = (int)Cin; g.H = (int)H; g.W = (int)W; g.Cout = (int)Cout;
+	g.kh = kh; g.kw = kw; g.ph = ph; g.pw = pw; g.sh = sh; g.sw = sw; g.dh = 1; g.dw = 1;
+	g.Ho = (int)(eh / sh + 1);  // l-ten/conv2d.cpp:322-323
+	g.Wo = (int)(ew / sw + 1);
+	return 0;
+}
+
+static uint64_t align16(uint64_t v) { return (v + 15) & ~15ull; }
+
+static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh, int sw,
+                       const uint8_t* x, const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qp, void* y, bool out_acc,
+                       void* workspace)
+{
+	ConvGeo g;
+	if (int rc = make_geo_q(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)) return rc;
+	LTEN_HIP_REQUIRE(qp != nullptr, "conv2dq: qparams is null");
+	const int64_t HW = (int64_t)g.Ho * g.Wo, K = (int64_t)Cin * kh * kw;
+	if (N == 0 || Cout == 0 || HW == 0) return 0;
+	LTEN_HIP_REQUIRE(x && w && y, "conv2dq: null pointer");
+	const int zp_in = qp[0].zero_point, zp_w = qp[1].zero_point;
+	// l-ten/math_fns.cpp:1436 with qparams[0] = weights, [1] = input (l-ten/conv2d.cpp:347-349), left to right in fp32
+	volatile float ab = qp[1].scale * qp[0].scale;
+	const float mult = ab / qp[2].scale, zp_out = (float)qp[2].zero_point;
+
+	if (K <= CQ_MAXK && get_option(OPT_CONV_VARIANT) != 1) {
+		const dim3 grid((unsigned)ceil_div((uint64_t)N * HW, 256), (unsigned)ceil_div(Cout, CQ_CO));
+		set_kernel_name("conv2dq_direct");
+		if (out_acc) conv2dq_direct_kernel<Q_OUT_ACC><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+		else if (mult == mult && (mult < 0 ? -mult : mult) <= 0.99f)
+			conv2dq_direct_kernel<Q_OUT_U8_FAST><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+		else conv2dq_direct_kernel<Q_OUT_U8_EXACT><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+
+	// l-ten's own decomposition, image by image: column buffer, then C[Cout x HW] = W[Cout x K] * col[K x HW]
+	LTEN_HIP_REQUIRE(workspace != nullptr, "conv2dq: workspace is null");
+	uint8_t* col = static_cast<uint8_t*>(workspace);
+	int32_t* terms = reinterpret_cast<int32_t*>(col + align16((uint64_t)K * HW));
+	const lten_hip_qparams q3[3] = { qp[1], qp[0], qp[2] };
+	for (uint64_t n = 0; n < N; n++) {
+		if (int rc = lten_hip_im2col_u8(x + n * Cin * H * W, (int)Cin, (int)H, (int)W, kh, kw, ph, pw, sh, sw, 1, 1, col)) return rc;
+		int rc;
+		if (out_acc) rc = lten_hip_quantized_matmul_acc(0, 0, Cout, (uint64_t)HW, (uint64_t)K, w, col, static_cast<int32_t*>(y) + n * Cout * HW, q3, bias, terms);
+		else rc = lten_hip_quantized_matmul(0, 0, Cout, (uint64_t)HW, (uint64_t)K, 1, w, col, 0, static_cast<uint8_t*>(y) + n * Cout * HW, q3, bias, terms);
+		if (rc) return rc;
+	}
+	return 0;
+}
+
+}  // namespace lten_hip
+
+using namespace lten_hip;
+
+extern "C" {
+
+uint64_t lten_hip_conv2dq_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
+                                          int pw, int sh, int sw)
+{
+	ConvGeo g;
+	if (make_geo_q(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)) return 0;
+	const uint64_t HW = (uint64_t)g.Ho * g.Wo, K = Cin * kh * kw;
+	return align16(K * HW) + 4 * (Cout + HW) + 16;
+}
+
+int lten_hip_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh,
+                             int sw, const uint8_t* x, const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qparams_in_wt_out,
+                             uint8_t* y, void* workspace)
+{
+	return conv2dq_run(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, x, w, bias, qparams_in_wt_out, y, false, workspace);
+}
+
+int lten_hip_conv2dq_forward_acc(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw,
+                                 int sh, int sw, const uint8_t* x, const uint8_t* w, const int32_t* bias,
+                                 const lten_hip_qparams* qparams_in_wt_out, int32_t* acc, void* workspace)
+{
+	return conv2dq_run(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, x, w, bias, qparams_in_wt_out, acc, true, workspace);
+}
+
+}  // extern "C"

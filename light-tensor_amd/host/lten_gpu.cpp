@@ -599,4 +599,81 @@ Tensor Conv2d::forward(Tensor& input)
 	return result;
 }
 
+// ------------------------------------------------------------------------------ Conv2d_q
+
+bool Conv2d_q::init()
+{
+	// l-ten/conv2d.cpp:235-263: UINT8 weights {Cout, Cin, kh*kw}, INT32 bias {1,Cout,1,1}, no initialisation
+	TensorOps options;
+	options.data_type = UINT8;
+	weight_ = AllocateTensor({ channels_out_, channels_in_, kernel_h_ * kernel_w_ }, &options);
+	weight_.set_autograd(true);
+	if (use_bias_) {
+		options.data_type = INT32;
+		bias_ = AllocateTensor({ 1, channels_out_, 1, 1 }, &options);
+		bias_.set_autograd(true);
+	}
+	return true;
+}
+
+void Conv2d_q::to(device target_device, int target_device_index)
+{
+	// l-ten's Conv2d_q::to throws "Only CPU device supported" (l-ten/layers.h:498); this is the GPU branch it lacks
+	if (weight_.defined()) weight_ = weight_.to(target_device, target_device_index);
+	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
+	workspace_ = Tensor();
+}
+
+void Conv2d_q::clear_gradients()
+{
+	if (weight_.defined()) weight_.clear_gradients();
+	if (use_bias_ && bias_.defined()) bias_.clear_gradients();
+}
+
+std::vector<Tensor*> Conv2d_q::get_all_weights()
+{
+	std::vector<Tensor*> w{ &weight_ };
+	if (use_bias_) w.push_back(&bias_);
+	return w;
+}
+
+void Conv2d_q::set_qparams_params(QuantizationParams* qparams, int count)
+{
+	if (qparams && count) qparams_wt_ = qparams[0];  // l-ten/conv2d.cpp:415-421
+}
+
+Tensor Conv2d_q::forward(Tensor& input)
+{
+	if (input.get_data_type() != UINT8) LTEN_ERR("Conv2d_q is only supported for UINT8 tensors");  // l-ten/conv2d.cpp:284-288
+	check_layer_input(input, weight_, "Conv2d_q");
+	if (input.get_ndims() != 4) LTEN_ERR("Conv2d_q requires tensors with exactly 4 dimensions (NCHW)");  // :299-302
+	const uint64_t* d = input.get_sizes();
+	const uint64_t N = d[0], H = d[2], W = d[3];
+	if (d[1] != channels_in_) LTEN_ERR("Input channel count does not match this layer");
+	const uint64_t Ho = (H + 2 * pad_h_ - kernel_h_) / stride_h_ + 1, Wo = (W + 2 * pad_w_ - kernel_w_) / stride_w_ + 1;  // :314-315
+	if (input.get_device() != GPU)
+		LTEN_ERR("this build implements Conv2d_q for the GPU device type only (l-ten's own CPU path covers lten::CPU)");
+	// l-ten hands its Cout-element bias to quantized_matmul, which indexes it by output position (l-ten/conv2d.cpp:366,
+	// l-ten/math_fns.cpp:1470-1473): with more output positions than channels that call reads past the buffer.
+	if (use_bias_ && Ho * Wo > channels_out_)
+		LTEN_ERR("Conv2d_q with a bias: l-ten's call indexes the bias by output position and would read past its Cout elements");
+
+	TensorOps options;
+	options.data_type = UINT8;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor({ N, channels_out_, Ho, Wo }, &options);
+	const int kh = (int)kernel_h_, kw = (int)kernel_w_, ph = (int)pad_h_, pw = (int)pad_w_, sh = (int)stride_h_, sw = (int)stride_w_;
+	const uint64_t need = lten_hip_conv2dq_workspace_bytes(N, channels_in_, H, W, channels_out_, kh, kw, ph, pw, sh, sw);
+	if (!workspace_.defined() || workspace_.get_numels() < need) workspace_ = AllocateTensor({ need }, &options);
+	lten_hip_qparams qp[3] = { { qparams_in_.scale, qparams_in_.zero_point }, { qparams_wt_.scale, qparams_wt_.zero_point },
+		                   { qparams_out_.scale, qparams_out_.zero_point } };
+	// l-ten/conv2d.cpp:355-372 (im2col_cpu + quantized_matmul per image): one call for the batch
+	LTEN_HIP_CALL(lten_hip_conv2dq_forward(N, channels_in_, H, W, channels_out_, kh, kw, ph, pw, sh, sw,
+	                                       static_cast<const uint8_t*>(input.get_data_ptr()), static_cast<const uint8_t*>(weight_.get_data_ptr()),
+	                                       use_bias_ ? static_cast<const int32_t*>(bias_.get_data_ptr()) : nullptr, qp,
+	                                       static_cast<uint8_t*>(result.get_data_ptr()), workspace_.get_data_ptr()));
+	return result;
+}
+
 }  // namespace lten

@@ -187,5 +187,39 @@ private:
 	Tensor weight_, bias_, scratch_;  // scratch_: weight-gradient partial sums / column buffer of the data gradient
 };
 
+// l-ten/layers.h:453-524; unlike l-ten's, this one runs on the GPU (l-ten: "Only CPU device supported").  Inference only,
+// as in l-ten (the result carries no usable gradient function for uint8 data).
+class Conv2d_q : public Module {
+public:
+	Conv2d_q(const int channels_in, const int channels_out, bool use_bias, const int kernel_h, const int kernel_w, const int pad_h = 0,
+	         const int pad_w = 0, const int stride_h = 1, const int stride_w = 1)
+	    : channels_in_(channels_in), channels_out_(channels_out), kernel_h_(kernel_h), kernel_w_(kernel_w), pad_h_(pad_h), pad_w_(pad_w),
+	      stride_h_(stride_h), stride_w_(stride_w), use_bias_(use_bias) {}
+	uint64_t get_channels_out() { return channels_out_; }
+	uint64_t get_channels_in() { return channels_in_; }
+	uint64_t get_kernel_h() { return kernel_h_; }
+	uint64_t get_kernel_w() { return kernel_w_; }
+	uint64_t get_pad_h() { return pad_h_; }
+	uint64_t get_pad_w() { return pad_w_; }
+	uint64_t get_stride_h() { return stride_h_; }
+	uint64_t get_stride_w() { return stride_w_; }
+	bool init() override;
+	Tensor forward(Tensor& input);
+	std::vector<Tensor*> get_all_weights() override;
+	Tensor* get_weights() { return &weight_; }
+	Tensor* get_bias() { return use_bias_ ? &bias_ : nullptr; }
+	void clear_gradients() override;
+	void to(device target_device, int target_device_index = 0) override;
+	void set_qparams_in(QuantizationParams qparams_in) override { qparams_in_ = qparams_in; }
+	void set_qparams_out(QuantizationParams qparams_out) override { qparams_out_ = qparams_out; }
+	void set_qparams_params(QuantizationParams* qparams, int count) override;
+
+private:
+	uint64_t channels_in_, channels_out_, kernel_h_, kernel_w_, pad_h_, pad_w_, stride_h_, stride_w_;
+	bool use_bias_;
+	Tensor weight_, bias_, workspace_;
+	QuantizationParams qparams_in_{ 1.0f, 0 }, qparams_out_{ 1.0f, 0 }, qparams_wt_{ 1.0f, 0 };
+};
+
 }  // namespace lten
 #endif

@@ -160,6 +160,53 @@ static int fcq_test()
 	return Compare((uint8_t*)Y.get_data_ptr(), want.data(), want.size());
 }
 
+// Conv2d_q (the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network, plus a padded strided one) against plain loops
+static int convq_test()
+{
+	struct Geo { int N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw; } geos[] = { { 3, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1 }, { 2, 12, 9, 11, 6, 3, 3, 1, 2, 2, 1 } };
+	unsigned s = 1234;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (s >> 16) & 0xFF; };
+	for (const Geo& g : geos) {
+		const int Ho = (g.H + 2 * g.ph - g.kh) / g.sh + 1, Wo = (g.W + 2 * g.pw - g.kw) / g.sw + 1, K = g.Cin * g.kh * g.kw;
+		std::vector<uint8_t> x((size_t)g.N * g.Cin * g.H * g.W), w((size_t)g.Cout * K);
+		for (auto& e : x) e = (uint8_t)rnd();
+		for (auto& e : w) e = (uint8_t)rnd();
+		lten::TensorOps ops;
+		ops.data_type = lten::UINT8;
+		lten::Tensor X = lten::TensorFromBuffer({ (uint64_t)g.N, (uint64_t)g.Cin, (uint64_t)g.H, (uint64_t)g.W }, x.data(), false, &ops).to(lten::GPU);
+		lten::Conv2d_q conv(g.Cin, g.Cout, false, g.kh, g.kw, g.ph, g.pw, g.sh, g.sw);
+		conv.init();
+		conv.train(false);
+		memcpy(conv.get_weights()->get_data_ptr(), w.data(), w.size());
+		QuantizationParams qi{ 0.02f, 9 }, qw{ 0.011f, 120 }, qo{ 0.8f, 90 };
+		conv.set_qparams_in(qi);
+		conv.set_qparams_params(&qw, 1);
+		conv.set_qparams_out(qo);
+		conv.to(lten::GPU);
+		lten::Tensor Y = conv.forward(X).to(lten::CPU);
+		const float mult = qw.scale * qi.scale / qo.scale;  // qparams[0] = weights in l-ten's call
+		std::vector<uint8_t> want((size_t)g.N * g.Cout * Ho * Wo);
+		for (int n = 0; n < g.N; n++)
+			for (int co = 0; co < g.Cout; co++)
+				for (int ho = 0; ho < Ho; ho++)
+					for (int wo = 0; wo < Wo; wo++) {
+						int acc = 0;
+						for (int ci = 0; ci < g.Cin; ci++)
+							for (int i = 0; i < g.kh; i++)
+								for (int j = 0; j < g.kw; j++) {
+									const int yy = ho * g.sh - g.ph + i, xx = wo * g.sw - g.pw + j;
+									const int xv = (yy >= 0 && yy < g.H && xx >= 0 && xx < g.W) ? x[((size_t)(n * g.Cin + ci) * g.H + yy) * g.W + xx] : 0;
+									acc += ((int)w[(size_t)co * K + (ci * g.kh + i) * g.kw + j] - qw.zero_point) * (xv - qi.zero_point);
+								}
+						volatile float p = mult * (float)acc;
+						volatile float sum = p + (float)qo.zero_point;
+						want[((size_t)(n * g.Cout + co) * Ho + ho) * Wo + wo] = (uint8_t)((int)sum & 0xFF);
+					}
+		if (Compare((uint8_t*)Y.get_data_ptr(), want.data(), want.size())) return -1;
+	}
+	return 0;
+}
+
 // Conv2d forward, weight gradient and data gradient against plain loops (stride 2, pad 1, non-square)
 static int conv_test()
 {
@@ -223,7 +270,7 @@ static int error_test()
 int main()
 {
 	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test },
-		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "error_test", error_test } };
+		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;
 	for (auto& t : tests) {
 		printf("running %s\n", t.name);

@@ -91,6 +91,8 @@ def oracle():
     for name in ("oracle_conv2d_forward", "oracle_conv2d_wgrad", "oracle_conv2d_dgrad"):
         getattr(lib, name).restype = None
         getattr(lib, name).argtypes = conv + [f32p, f32p, f32p, f32p]
+    lib.oracle_conv2dq_forward.restype = C.c_int
+    lib.oracle_conv2dq_forward.argtypes = conv + [u8p, u8p, C.POINTER(C.c_int32), C.POINTER(QParams), u8p, C.POINTER(C.c_int32)]
     _oracle = lib
     return lib
 
@@ -123,6 +125,8 @@ def ref():
     lib.ref_fcq_u8.argtypes = [u64, u64, u64, u64, u8p, u8p, C.POINTER(C.c_int32), f32p, u8p, u8p]
     lib.ref_conv2d_f32.restype = C.c_int
     lib.ref_conv2d_f32.argtypes = [u64] * 5 + [C.c_int] * 6 + [f32p, f32p, fp, fp, fp, fp]
+    lib.ref_conv2dq_u8.restype = C.c_int
+    lib.ref_conv2dq_u8.argtypes = [u64] * 5 + [C.c_int] * 6 + [u8p, u8p, f32p, u8p, u8p]
     lib.ref_matmul_f32.restype = C.c_int
     lib.ref_matmul_f32.argtypes = [C.c_int, u64p, u64p, f32p, f32p, fp, fp, fp, fp]
     lib.ref_hardware_threads.restype = C.c_int
@@ -175,3 +179,33 @@ def sgemm(tA, tB, M, N, K, alpha, A, lda, B, ldb, beta, Cm, ldc, f64=False):
 
 def conv_out_hw(H, W, kh, kw, ph, pw, sh, sw):
     return (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+
+
+def conv2dq_forward(geo, x, w, scales, zps, bias=None, want_acc=True):
+    """oracle_conv2dq_forward on numpy arrays; scales / zps ordered (input, weights, output).  Returns (y, acc)."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    Ho, Wo = conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    x = np.ascontiguousarray(x, np.uint8)
+    w = np.ascontiguousarray(w, np.uint8)
+    y = np.empty((N, Cout, Ho, Wo), np.uint8)
+    acc = np.empty((N, Cout, Ho, Wo), np.int32) if want_acc else None
+    b = None
+    if bias is not None:
+        b = np.ascontiguousarray(bias, np.int32)
+        assert b.size >= Ho * Wo
+    rc = oracle().oracle_conv2dq_forward(*geo, x.reshape(-1), w.reshape(-1),
+                                         b.ctypes.data_as(C.POINTER(C.c_int32)) if b is not None else None,
+                                         qparams3(scales, zps), y.reshape(-1),
+                                         acc.ctypes.data_as(C.POINTER(C.c_int32)) if acc is not None else None)
+    assert rc == 0
+    return y, acc
+
+
+def ref_conv2dq_forward(geo, x, w, scales, zps):
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    Ho, Wo = conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    y = np.empty((N, Cout, Ho, Wo), np.uint8)
+    rc = ref().ref_conv2dq_u8(*geo, np.ascontiguousarray(x, np.uint8).reshape(-1), np.ascontiguousarray(w, np.uint8).reshape(-1),
+                              np.asarray(scales, np.float32), np.asarray(zps, np.uint8), y.reshape(-1))
+    assert rc == 0
+    return y

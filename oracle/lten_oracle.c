@@ -422,6 +422,34 @@ void oracle_conv2d_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uin
 	}
 }
 
+int oracle_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                           uint64_t kh, uint64_t kw, uint64_t ph, uint64_t pw, uint64_t sh, uint64_t sw,
+                           const uint8_t* x, const uint8_t* w, const int32_t* bias,
+                           const oracle_qparams* qp_in_wt_out, uint8_t* y, int32_t* acc_out)
+{
+	/* l-ten/conv2d.cpp:318-372: per image, u8 im2col (zero bytes outside the image) then
+	 * quantized_matmul(false, false, Cout, Ho*Wo, Cin*kh*kw) with qparams[0] = weights,
+	 * qparams[1] = input (:347-349).  The bias, when given, is indexed by the GEMM column, i.e. by
+	 * output position (l-ten/math_fns.cpp:1470-1473): it must hold Ho*Wo ints. */
+	uint64_t Ho = (H + 2 * ph - kh) / sh + 1, Wo = (W + 2 * pw - kw) / sw + 1;
+	uint64_t Kc = Cin * kh * kw, HW = Ho * Wo, n;
+	oracle_qparams qp[3];
+	uint8_t* col = (uint8_t*)malloc(Kc * HW + 1);
+	int32_t* ws = (int32_t*)malloc(sizeof(int32_t) * (Cout + HW + 1));
+	int rc = 0;
+	qp[0] = qp_in_wt_out[1];
+	qp[1] = qp_in_wt_out[0];
+	qp[2] = qp_in_wt_out[2];
+	for (n = 0; n < N && rc == 0; n++) {
+		oracle_im2col_u8(x + n * Cin * H * W, Cin, H, W, kh, kw, ph, pw, sh, sw, col);
+		rc = oracle_quantized_matmul(0, 0, Cout, HW, Kc, 1, w, col, 0, y + n * Cout * HW, qp, bias, ws,
+		                             acc_out ? acc_out + n * Cout * HW : NULL);
+	}
+	free(col);
+	free(ws);
+	return rc;
+}
+
 void oracle_conv2d_wgrad(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                          uint64_t kh, uint64_t kw, uint64_t ph, uint64_t pw, uint64_t sh, uint64_t sw,
                          const float* x, const float* dy, float* dw, float* col)

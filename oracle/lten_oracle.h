@@ -15,6 +15,8 @@
  *       (bit-exact), a direct 7-loop convolution, adjointness <im2col x, c> = <x, col2im c>.
  *   oracle_fc_* / oracle_matmul_* / oracle_conv2d_*  pinned: compiled l-ten layers,
  *       reference-held vectors (fc_test, matmul_test), finite differences.
+ *   oracle_conv2dq_forward                     pinned: the compiled l-ten Conv2d_q layer
+ *       (golden cases), the int64 closed form with zero bytes as padding, invariants.
  */
 #ifndef LTEN_ORACLE_H
 #define LTEN_ORACLE_H
@@ -99,6 +101,15 @@ int oracle_matmul_backward(int ndims, const uint64_t* adims, const uint64_t* bdi
                            const float* B, const float* dC, float* dA, float* dB);
 
 /* l-ten/conv2d.cpp:55-197 (CPU branch :134-144): per image im2col + NN GEMM. */
+/* l-ten/conv2d.cpp:265-387 Conv2d_q::forward: per image u8 im2col + quantized_matmul(false, false)
+ * with the weights as the left operand.  bias (or NULL) holds Ho*Wo ints and is added per output
+ * position, as the reference's call does.  acc_out (or NULL) receives the int32 values before the
+ * requantize.  Pinned: the compiled Conv2d_q layer (golden cases), composition of pinned parts. */
+int oracle_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                           uint64_t kh, uint64_t kw, uint64_t ph, uint64_t pw, uint64_t sh, uint64_t sw,
+                           const uint8_t* x, const uint8_t* w, const int32_t* bias,
+                           const oracle_qparams* qp_in_wt_out, uint8_t* y, int32_t* acc_out);
+
 void oracle_conv2d_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                            uint64_t kh, uint64_t kw, uint64_t ph, uint64_t pw, uint64_t sh, uint64_t sw,
                            const float* x, const float* w, float* y, float* col_scratch);

@@ -122,6 +122,34 @@ int ref_fcq_u8(uint64_t batch, uint64_t M, uint64_t in, uint64_t out, const uint
 	return 0;
 }
 
+// lten::Conv2d_q forward (no bias: l-ten's own call indexes the bias by output position), l-ten/conv2d.cpp:265.
+int ref_conv2dq_u8(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw,
+                   int sh, int sw, const uint8_t* x, const uint8_t* w, const float* scales, const uint8_t* zero_points,
+                   uint8_t* y)
+{
+	try {
+		lten::TensorOps ops;
+		ops.data_type = lten::UINT8;
+		lten::Tensor X = lten::TensorFromBuffer({ N, Cin, H, W }, const_cast<uint8_t*>(x), false, &ops);
+		lten::Conv2d_q conv((int)Cin, (int)Cout, false, kh, kw, ph, pw, sh, sw);
+		conv.init();
+		conv.train(false);
+		memcpy(conv.get_weights()->get_data_ptr(), w, Cout * Cin * kh * kw);
+		QuantizationParams qi, qw, qo;
+		qi.scale = scales[0]; qi.zero_point = zero_points[0];
+		qw.scale = scales[1]; qw.zero_point = zero_points[1];
+		qo.scale = scales[2]; qo.zero_point = zero_points[2];
+		conv.set_qparams_in(qi);
+		conv.set_qparams_params(&qw, 1);
+		conv.set_qparams_out(qo);
+		lten::Tensor Y = conv.forward(X);
+		uint64_t Ho = (H + 2 * ph - kh) / sh + 1;
+		uint64_t Wo = (W + 2 * pw - kw) / sw + 1;
+		memcpy(y, Y.get_data_ptr(), N * Cout * Ho * Wo);
+	} catch (...) { return -1; }
+	return 0;
+}
+
 // lten::Conv2d forward + weight/data gradient, l-ten/conv2d.cpp:55, l-ten/backprop.cpp:1841.
 int ref_conv2d_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw,
                    int sh, int sw, const float* x, const float* w, const float* dy, float* y, float* dw, float* dx)

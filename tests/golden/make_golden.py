@@ -206,9 +206,35 @@ def layer_cases():
     print("layer_cases ok")
 
 
+def conv2dq_cases():
+    """The compiled lten::Conv2d_q forward (no bias), including the 1 -> 10 channel 5x5 layer of l-ten's quantized
+    MNIST network (tests/nn_tests.cpp:625), padded / strided / multi-channel windows and zero points that make
+    every correction term non-zero."""
+    rng = np.random.default_rng(77)
+    geos = [(2, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1), (3, 3, 9, 11, 4, 3, 3, 1, 1, 1, 1), (1, 2, 10, 7, 5, 3, 2, 0, 1, 2, 1),
+            (2, 4, 6, 6, 3, 1, 1, 0, 0, 1, 1), (1, 8, 12, 12, 6, 3, 3, 2, 2, 1, 1), (2, 1, 9, 140, 33, 3, 3, 1, 1, 1, 1)]
+    qps = [([1 / 255, 0.01, 0.05], [0, 128, 128]), ([0.02, 0.013, 0.9], [17, 250, 100]), ([0.5, 0.5, 0.1], [128, 128, 0])]
+    out, idx = {}, 0
+    for geo in geos:
+        N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+        x = rng.integers(0, 256, (N, Cin, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (Cout, Cin, kh, kw), dtype=np.uint8)
+        for sc, zp in qps:
+            pre = f"q{idx}_"
+            out[pre + "geo"] = np.array(geo, np.int64)
+            out[pre + "x"], out[pre + "w"] = x, w
+            out[pre + "scales"], out[pre + "zps"] = np.array(sc, np.float32), np.array(zp, np.uint8)
+            out[pre + "y"] = ob.ref_conv2dq_forward(geo, x, w, sc, zp)
+            idx += 1
+    out["count"] = np.array(idx)
+    np.savez_compressed(os.path.join(HERE, "conv2dq_cases.npz"), **out)
+    print("conv2dq_cases", idx)
+
+
 if __name__ == "__main__":
     requant_sweep()
     qmm_cases()
     cfg1_expected()
     sgemm_cases()
     layer_cases()
+    conv2dq_cases()

@@ -1,0 +1,48 @@
+"""GPU parity tests of the Conv2d_q forward (C ABI): int32 accumulators and requantized uint8 outputs bit-exact against
+the oracle, the golden outputs of l-ten's compiled Conv2d_q layer, and the int64 closed form."""
+import numpy as np
+import pytest
+
+from conftest import golden_path
+from test_oracle_conv import conv2dq_closed_form
+
+pytestmark = pytest.mark.gpu
+
+
+def test_conv2dq_golden_from_compiled_layer(gpu):
+    g = np.load(golden_path("conv2dq_cases.npz"))
+    for variant in (0, 1):   # 0: the library's choice (one launch up to 64 taps); 1: im2col + GEMM per image
+        gpu.set_option("conv_variant", variant)
+        try:
+            for i in range(int(g["count"])):
+                pre = f"q{i}_"
+                geo = tuple(int(v) for v in g[pre + "geo"])
+                y, acc = gpu.conv2dq_host(geo, g[pre + "x"], g[pre + "w"], g[pre + "scales"], g[pre + "zps"], want_acc=True)
+                assert np.array_equal(y, g[pre + "y"]), (variant, i, gpu.last_kernel())
+                want = conv2dq_closed_form(geo, g[pre + "x"], g[pre + "w"], int(g[pre + "zps"][0]), int(g[pre + "zps"][1]))
+                assert np.array_equal(acc, want), (variant, i)
+        finally:
+            gpu.set_option("conv_variant", 0)
+
+
+@pytest.mark.parametrize("geo", [(64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1),      # l-ten's quantized MNIST conv1 at batch 64
+                                 (3, 7, 13, 17, 70, 3, 3, 1, 1, 1, 1),       # 63 taps, two channel blocks
+                                 (2, 16, 20, 22, 24, 3, 3, 1, 1, 2, 1),      # 144 taps: column buffer + GEMM
+                                 (1, 3, 33, 300, 5, 7, 3, 3, 0, 2, 3),       # 63 taps, strides, ragged
+                                 (2, 32, 9, 9, 40, 1, 1, 0, 0, 1, 1)])       # 1x1
+def test_conv2dq_vs_oracle(gpu, ob, geo):
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.integers(0, 256, (N, Cin, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (Cout, Cin, kh, kw), dtype=np.uint8)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    K = Cin * kh * kw
+    for sc, zp, with_bias in (([1 / 255, 0.01, 0.05], [0, 128, 128], False), ([0.02, 0.013, 0.9], [17, 250, 100], True),
+                              ([0.5, 0.5, 0.2], [128, 128, 0], False)):
+        bias = rng.integers(-9999, 9999, Ho * Wo).astype(np.int32) if with_bias else None
+        want_y, want_acc = ob.conv2dq_forward(geo, x, w, sc, zp, bias=bias)
+        y, acc = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
+        kern = gpu.last_kernel()
+        assert (kern == "conv2dq_direct") == (K <= 64), kern
+        assert np.array_equal(acc, want_acc), kern
+        assert np.array_equal(y, want_y), kern

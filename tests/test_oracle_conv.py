@@ -125,3 +125,46 @@ def test_conv_forward_and_wgrad_vs_direct(ob, geo):
         e[idx] = 1.0
         want_g = float((dy.astype(np.float64) * direct_conv(e, w, ph, pw, sh, sw)).sum())
         assert abs(dx[idx] - want_g) < 1e-3 * max(1.0, abs(want_g))
+
+
+# ----------------------------------------------------------------------------------------- Conv2d_q
+
+def conv2dq_closed_form(geo, x, w, zp_in, zp_w):
+    """sum over the window of (w - zpW) * (x_or_0 - zpIn) in int64: positions outside the image hold the byte 0
+    (l-ten/im_col.h:24-27 pads the column buffer with T(0), not with the zero point)."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    Ho, Wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+    xp = np.pad(x.astype(np.int64), ((0, 0), (0, 0), (ph, ph), (pw, pw))) - zp_in
+    wz = w.astype(np.int64) - zp_w
+    acc = np.zeros((N, Cout, Ho, Wo), np.int64)
+    for i in range(kh):
+        for j in range(kw):
+            win = xp[:, :, i:i + (Ho - 1) * sh + 1:sh, j:j + (Wo - 1) * sw + 1:sw]
+            acc += np.einsum("nchw,oc->nohw", win, wz[:, :, i, j])
+    return acc
+
+
+def test_conv2dq_golden_from_compiled_layer(ob):
+    g = np.load(golden_path("conv2dq_cases.npz"))
+    for i in range(int(g["count"])):
+        pre = f"q{i}_"
+        geo = tuple(int(v) for v in g[pre + "geo"])
+        y, acc = ob.conv2dq_forward(geo, g[pre + "x"], g[pre + "w"], g[pre + "scales"], g[pre + "zps"])
+        assert np.array_equal(y, g[pre + "y"]), i
+        want = conv2dq_closed_form(geo, g[pre + "x"], g[pre + "w"], int(g[pre + "zps"][0]), int(g[pre + "zps"][1]))
+        assert np.array_equal(acc, want), i
+
+
+def test_conv2dq_bias_is_per_output_position_and_invariants(ob):
+    geo = (2, 2, 7, 6, 3, 3, 3, 1, 1, 1, 1)
+    rng = np.random.default_rng(5)
+    x = rng.integers(0, 256, (2, 2, 7, 6), dtype=np.uint8)
+    w = rng.integers(0, 256, (3, 2, 3, 3), dtype=np.uint8)
+    bias = rng.integers(-5000, 5000, 42).astype(np.int32)
+    _, acc0 = ob.conv2dq_forward(geo, x, w, [0.02, 0.02, 1.0], [9, 200, 3])
+    _, acc1 = ob.conv2dq_forward(geo, x, w, [0.02, 0.02, 1.0], [9, 200, 3], bias=bias)
+    assert np.array_equal(acc1 - acc0, np.broadcast_to(bias.reshape(1, 1, 7, 6), acc0.shape))
+    # weights equal to their zero point: every accumulator is 0, the output is the output zero point
+    wz = np.full_like(w, 200)
+    y, acc = ob.conv2dq_forward(geo, x, wz, [0.02, 0.02, 1.0], [9, 200, 3])
+    assert not acc.any() and (y == 3).all()
