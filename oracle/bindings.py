@@ -35,6 +35,11 @@ def qparams3(scales, zps):
     return arr
 
 
+_FPP = C.POINTER(C.POINTER(C.c_float))
+_MLP_ARGS = [C.c_uint64, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_float), _FPP, _FPP, C.POINTER(C.c_float),
+             C.POINTER(C.c_float), C.POINTER(C.c_float), _FPP, _FPP, C.POINTER(C.c_float)]
+
+
 def _opt(a, ctype):
     return None if a is None else a.ctypes.data_as(C.POINTER(ctype))
 
@@ -91,6 +96,20 @@ def oracle():
     for name in ("oracle_conv2d_forward", "oracle_conv2d_wgrad", "oracle_conv2d_dgrad"):
         getattr(lib, name).restype = None
         getattr(lib, name).argtypes = conv + [f32p, f32p, f32p, f32p]
+    lib.oracle_relu.restype = None
+    lib.oracle_relu.argtypes = [f32p, f32p, u64]
+    lib.oracle_relu_backward.restype = None
+    lib.oracle_relu_backward.argtypes = [f32p, f32p, f32p, u64]
+    lib.oracle_log_softmax.restype = None
+    lib.oracle_log_softmax.argtypes = [u64, u64, f32p, f32p]
+    lib.oracle_log_softmax_backward.restype = None
+    lib.oracle_log_softmax_backward.argtypes = [u64, u64, f32p, f32p, f32p]
+    lib.oracle_nll_loss.restype = C.c_float
+    lib.oracle_nll_loss.argtypes = [f32p, f32p, u64, u64]
+    lib.oracle_nll_backward.restype = None
+    lib.oracle_nll_backward.argtypes = [f32p, u64, u64, C.c_float, f32p]
+    lib.oracle_mlp_step.restype = C.c_int
+    lib.oracle_mlp_step.argtypes = _MLP_ARGS
     lib.oracle_conv2dq_forward.restype = C.c_int
     lib.oracle_conv2dq_forward.argtypes = conv + [u8p, u8p, C.POINTER(C.c_int32), C.POINTER(QParams), u8p, C.POINTER(C.c_int32)]
     _oracle = lib
@@ -125,6 +144,8 @@ def ref():
     lib.ref_fcq_u8.argtypes = [u64, u64, u64, u64, u8p, u8p, C.POINTER(C.c_int32), f32p, u8p, u8p]
     lib.ref_conv2d_f32.restype = C.c_int
     lib.ref_conv2d_f32.argtypes = [u64] * 5 + [C.c_int] * 6 + [f32p, f32p, fp, fp, fp, fp]
+    lib.ref_mlp_step.restype = C.c_int
+    lib.ref_mlp_step.argtypes = _MLP_ARGS
     lib.ref_conv2dq_u8.restype = C.c_int
     lib.ref_conv2dq_u8.argtypes = [u64] * 5 + [C.c_int] * 6 + [u8p, u8p, f32p, u8p, u8p]
     lib.ref_matmul_f32.restype = C.c_int
@@ -209,3 +230,27 @@ def ref_conv2dq_forward(geo, x, w, scales, zps):
                               np.asarray(scales, np.float32), np.asarray(zps, np.uint8), y.reshape(-1))
     assert rc == 0
     return y
+
+
+def mlp_step(X, Ws, bs, target, use_ref=False):
+    """One training step of the FullyConnected/relu/log_softmax/nll network (oracle_mlp_step, or the compiled l-ten
+    network with use_ref).  Returns dict(loss, logp, dW[], db[], dX)."""
+    fpc = C.POINTER(C.c_float)
+    X = np.ascontiguousarray(X, np.float32)
+    Ws = [np.ascontiguousarray(w, np.float32) for w in Ws]
+    bs = [np.ascontiguousarray(b, np.float32) for b in bs] if bs is not None else None
+    target = np.ascontiguousarray(target, np.float32)
+    layers, batch = len(Ws), X.shape[0]
+    sizes = (C.c_uint64 * (layers + 1))(*([X.shape[1]] + [w.shape[0] for w in Ws]))
+    dW = [np.zeros_like(w) for w in Ws]
+    db = [np.zeros_like(b) for b in bs] if bs is not None else None
+    dX, logp, loss = np.zeros_like(X), np.zeros_like(target), C.c_float()
+
+    def arr(lst):
+        return (fpc * layers)(*[a.ctypes.data_as(fpc) for a in lst])
+    fn = ref().ref_mlp_step if use_ref else oracle().oracle_mlp_step
+    rc = fn(batch, layers, sizes, X.ctypes.data_as(fpc), arr(Ws), arr(bs) if bs is not None else None,
+            target.ctypes.data_as(fpc), C.byref(loss), logp.ctypes.data_as(fpc), arr(dW),
+            arr(db) if db is not None else None, dX.ctypes.data_as(fpc))
+    assert rc == 0
+    return dict(loss=float(loss.value), logp=logp, dW=dW, db=db, dX=dX)

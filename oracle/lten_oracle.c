@@ -6,6 +6,7 @@
 #include <limits.h>
 #include <pthread.h>
 #include <stdlib.h>
+#include <math.h>
 #include <string.h>
 
 #define ORACLE_MAX_DIMS 16 /* l-ten/md_array.h:37 */
@@ -474,4 +475,101 @@ void oracle_conv2d_dgrad(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint6
 		oracle_sgemm(1, 0, Kc, HW, Cout, 1.0f, w, Kc, dy + n * Cout * HW, HW, 0.0f, col, HW);
 		oracle_col2im_f32(col, Cin, H, W, kh, kw, ph, pw, sh, sw, dx + n * Cin * H * W);
 	}
+}
+
+/* --------------------------------------------------------------------- element-wise pieces of the MLP step */
+
+void oracle_relu(const float* src, float* dst, uint64_t n)
+{
+	uint64_t i; /* l-ten/layers.cpp:32-43 */
+	for (i = 0; i < n; i++) dst[i] = src[i] > 0 ? src[i] : 0;
+}
+
+void oracle_relu_backward(const float* top, const float* input, float* bottom, uint64_t n)
+{
+	uint64_t i; /* l-ten/backprop.cpp:2300-2311 */
+	for (i = 0; i < n; i++) bottom[i] = input[i] > 0 ? top[i] : 0;
+}
+
+void oracle_log_softmax(uint64_t rows, uint64_t cols, const float* x, float* y)
+{
+	/* l-ten/layers.cpp:93-114 along the last dimension: max, x - max, exp, sum (in index order), exps / sum, log */
+	uint64_t r, c;
+	for (r = 0; r < rows; r++) {
+		const float* xr = x + r * cols;
+		float m = xr[0], sum = 0.0f;
+		for (c = 1; c < cols; c++) if (xr[c] > m) m = xr[c];
+		for (c = 0; c < cols; c++) sum += expf(xr[c] - m);
+		for (c = 0; c < cols; c++) y[r * cols + c] = logf(expf(xr[c] - m) / sum);
+	}
+}
+
+void oracle_log_softmax_backward(uint64_t rows, uint64_t cols, const float* y, const float* dy, float* dx)
+{
+	/* The chain of l-ten's backward functions for log, div, sum, exp, sub and max collapses to
+	 * dx = dy - exp(y) * sum_j dy_j (the two paths through max cancel). */
+	uint64_t r, c;
+	for (r = 0; r < rows; r++) {
+		float s = 0.0f;
+		for (c = 0; c < cols; c++) s += dy[r * cols + c];
+		for (c = 0; c < cols; c++) dx[r * cols + c] = dy[r * cols + c] - expf(y[r * cols + c]) * s;
+	}
+}
+
+float oracle_nll_loss(const float* input, const float* target, uint64_t len, uint64_t batch)
+{
+	uint64_t i; /* l-ten/layers.cpp:243-249 */
+	float val = 0;
+	for (i = 0; i < len; i++) val += input[i] * target[i];
+	return val * (-1.0f / batch);
+}
+
+void oracle_nll_backward(const float* target, uint64_t len, uint64_t batch, float top, float* bottom)
+{
+	uint64_t i; /* l-ten/backprop.cpp:3986-4005: bottom = (-1 / batch * top) * target */
+	float scale = -1.0f / (float)batch;
+	scale *= top;
+	for (i = 0; i < len; i++) bottom[i] = scale * target[i];
+}
+
+int oracle_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const float* X, const float* const* W,
+                    const float* const* b, const float* target, float* loss, float* logp, float** dW, float** db,
+                    float* dX)
+{
+	/* FullyConnected (+ bias) with relu between the layers, log_softmax, nll_loss, then backward() from the loss:
+	 * the network of l-ten's MNIST tests (tests/nn_tests.cpp) with the sizes of the caller's choice. */
+	float* act[17];
+	float* pre[17];
+	float *g, *g2;
+	uint64_t maxw = 0;
+	int l, rc = 0;
+	if (layers < 1 || layers > 16) return -1;
+	for (l = 0; l <= layers; l++) if (sizes[l] > maxw) maxw = sizes[l];
+	act[0] = (float*)X;
+	for (l = 0; l < layers; l++) {
+		pre[l + 1] = (float*)malloc(sizeof(float) * batch * sizes[l + 1]);
+		act[l + 1] = (l + 1 < layers) ? (float*)malloc(sizeof(float) * batch * sizes[l + 1]) : pre[l + 1];
+		oracle_fc_forward(batch, sizes[l], sizes[l + 1], act[l], W[l], b ? b[l] : NULL, pre[l + 1]);
+		if (l + 1 < layers) oracle_relu(pre[l + 1], act[l + 1], batch * sizes[l + 1]);
+	}
+	oracle_log_softmax(batch, sizes[layers], pre[layers], logp);
+	*loss = oracle_nll_loss(logp, target, batch * sizes[layers], batch);
+
+	g = (float*)malloc(sizeof(float) * batch * maxw);
+	g2 = (float*)malloc(sizeof(float) * batch * maxw);
+	oracle_nll_backward(target, batch * sizes[layers], batch, 1.0f, g2);
+	oracle_log_softmax_backward(batch, sizes[layers], logp, g2, g);
+	for (l = layers - 1; l >= 0; l--) {
+		if (db && db[l]) memset(db[l], 0, sizeof(float) * sizes[l + 1]);
+		oracle_fc_backward(batch, sizes[l], sizes[l + 1], act[l], W[l], g, (l > 0 || dX) ? g2 : NULL, dW[l], (b && db) ? db[l] : NULL);
+		if (l > 0) oracle_relu_backward(g2, pre[l], g, batch * sizes[l]);
+		else if (dX) memcpy(dX, g2, sizeof(float) * batch * sizes[0]);
+	}
+	for (l = 0; l < layers; l++) {
+		if (l + 1 < layers) free(act[l + 1]);
+		free(pre[l + 1]);
+	}
+	free(g);
+	free(g2);
+	return rc;
 }

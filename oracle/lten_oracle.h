@@ -122,6 +122,24 @@ void oracle_conv2d_dgrad(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint6
                          uint64_t kh, uint64_t kw, uint64_t ph, uint64_t pw, uint64_t sh, uint64_t sw,
                          const float* w, const float* dy, float* dx, float* col_scratch);
 
+/* Element-wise pieces that sit between the GEMMs of an MLP training step: relu (l-ten/layers.cpp:9-67),
+ * relu_backward (l-ten/backprop.cpp:2282-2327), log_softmax along the last dimension (l-ten/layers.cpp:93-114, a
+ * composition of max, sub, exp, sum, div, log) and the collapsed form of its backward chain, nll_loss
+ * (l-ten/layers.cpp:212-273) and nll_backward (l-ten/backprop.cpp:3975-4040).  Pinned: a whole training step of the
+ * compiled l-ten network (golden case) at 1e-5, finite differences of the loss, closed forms. */
+void oracle_relu(const float* src, float* dst, uint64_t n);
+void oracle_relu_backward(const float* top, const float* input, float* bottom, uint64_t n);
+void oracle_log_softmax(uint64_t rows, uint64_t cols, const float* x, float* y);
+void oracle_log_softmax_backward(uint64_t rows, uint64_t cols, const float* y, const float* dy, float* dx);
+float oracle_nll_loss(const float* input, const float* target, uint64_t len, uint64_t batch);
+void oracle_nll_backward(const float* target, uint64_t len, uint64_t batch, float top, float* bottom);
+/* One training step of FullyConnected(+bias) -> relu -> ... -> FullyConnected -> log_softmax -> nll_loss and
+ * backward(): sizes[0..layers], W[l] is [sizes[l+1] x sizes[l]], target is one-hot [batch x sizes[layers]].
+ * Outputs: loss, logp [batch x sizes[layers]], dW[l], db[l] (may be NULL with b), dX (may be NULL). */
+int oracle_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const float* X, const float* const* W,
+                    const float* const* b, const float* target, float* loss, float* logp, float** dW, float** db,
+                    float* dX);
+
 #ifdef __cplusplus
 }
 #endif

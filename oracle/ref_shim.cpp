@@ -96,6 +96,43 @@ int ref_fc_f32(uint64_t M, uint64_t in, uint64_t out, const float* x, const floa
 	return 0;
 }
 
+// One training step of l-ten's MLP (tests/nn_tests.cpp): FullyConnected(+bias) -> relu -> ... -> FullyConnected ->
+// log_softmax(dim 3) -> nll_loss -> backward().  x: {batch,1,1,sizes[0]}, target one-hot {batch,1,1,sizes[layers]}.
+int ref_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const float* x, const float* const* w,
+                 const float* const* b, const float* target, float* loss, float* logp, float** dw, float** db, float* dx)
+{
+	try {
+		lten::Tensor X = lten::TensorFromBuffer({ batch, 1, 1, sizes[0] }, const_cast<float*>(x), false);
+		X.set_autograd(true);
+		lten::Tensor T = lten::TensorFromBuffer({ batch, 1, 1, sizes[layers] }, const_cast<float*>(target), false);
+		std::vector<lten::FullyConnected*> fcs;
+		for (int l = 0; l < layers; l++) {
+			lten::FullyConnected* fc = new lten::FullyConnected(sizes[l], sizes[l + 1], b != nullptr);
+			fc->init();
+			memcpy(fc->get_weights()->get_data_ptr(), w[l], sizes[l + 1] * sizes[l] * 4);
+			if (b) memcpy(fc->get_bias()->get_data_ptr(), b[l], sizes[l + 1] * 4);
+			fcs.push_back(fc);
+		}
+		lten::Tensor h = X;
+		for (int l = 0; l < layers; l++) {
+			h = fcs[l]->forward(h);
+			if (l + 1 < layers) h = lten::relu(h);
+		}
+		lten::Tensor lp = lten::log_softmax(h, 3);
+		lten::Tensor L = lten::nll_loss(lp, T);
+		*loss = *static_cast<float*>(L.get_data_ptr());
+		memcpy(logp, lp.get_data_ptr(), batch * sizes[layers] * 4);
+		L.backward();
+		for (int l = 0; l < layers; l++) {
+			memcpy(dw[l], fcs[l]->get_weights()->get_grad_ptr(), sizes[l + 1] * sizes[l] * 4);
+			if (b && db) memcpy(db[l], fcs[l]->get_bias()->get_grad_ptr(), sizes[l + 1] * 4);
+		}
+		if (dx) memcpy(dx, X.get_grad_ptr(), batch * sizes[0] * 4);
+		for (auto fc : fcs) delete fc;
+	} catch (...) { return -1; }
+	return 0;
+}
+
 // lten::FullyConnected_q forward, l-ten/fully_connected.cpp:322.  x: {batch,M,in} u8.
 int ref_fcq_u8(uint64_t batch, uint64_t M, uint64_t in, uint64_t out, const uint8_t* x, const uint8_t* w,
                const int* bias, const float* scales, const uint8_t* zero_points, uint8_t* y)

@@ -231,6 +231,31 @@ def conv2dq_cases():
     print("conv2dq_cases", idx)
 
 
+def mlp_step_case():
+    """One training step of the compiled l-ten network FullyConnected(+bias) -> relu -> FullyConnected -> relu ->
+    FullyConnected -> log_softmax -> nll_loss.  Every GEMM dimension stays below 16 (the compiled cpu_gemm's AVX
+    block needs 32-byte aligned outputs from 16 columns on)."""
+    rng = np.random.default_rng(31)
+    sizes, B = [13, 12, 9, 10], 6
+    X = rng.random((B, sizes[0])).astype(np.float32)
+    Ws = [(rng.standard_normal((sizes[i + 1], sizes[i])) * 0.3).astype(np.float32) for i in range(3)]
+    bs = [(rng.standard_normal(sizes[i + 1]) * 0.3).astype(np.float32) for i in range(3)]
+    T = np.eye(10, dtype=np.float32)[rng.integers(0, 10, B)]
+    # l-ten's threaded cpu_gemm multiplies a fresh output buffer by beta = 0 (l-ten/math_fns.cpp:1168-1171), so a NaN
+    # that happens to sit in that uninitialised memory survives: repeat until the run is clean
+    for attempt in range(50):
+        r = ob.mlp_step(X, Ws, bs, T, use_ref=True)
+        if all(np.isfinite(a).all() for a in [r["logp"], r["dX"]] + r["dW"] + r["db"]):
+            break
+    else:
+        raise RuntimeError("no NaN-free run of the compiled network")
+    out = {"X": X, "T": T, "loss": np.float32(r["loss"]), "logp": r["logp"], "dX": r["dX"]}
+    for l in range(3):
+        out[f"W{l}"], out[f"b{l}"], out[f"dW{l}"], out[f"db{l}"] = Ws[l], bs[l], r["dW"][l], r["db"][l]
+    np.savez_compressed(os.path.join(HERE, "mlp_step_case.npz"), **out)
+    print("mlp_step_case loss", r["loss"])
+
+
 if __name__ == "__main__":
     requant_sweep()
     qmm_cases()
@@ -238,3 +263,4 @@ if __name__ == "__main__":
     sgemm_cases()
     layer_cases()
     conv2dq_cases()
+    mlp_step_case()
