@@ -176,6 +176,24 @@ int lten_hip_conv2dq_forward_acc(uint64_t N, uint64_t Cin, uint64_t H, uint64_t 
                                  const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qparams_in_wt_out,
                                  int32_t* acc, void* workspace);
 
+/* ------------------------------------------------- element-wise pieces of a training step */
+
+/* gpu_relu / gpu_relu_backward (l-ten/math_fns.h:231-234; l-ten/layers.cpp:9-67, l-ten/backprop.cpp:2282-2327):
+ * dst = src > 0 ? src : 0;  bottom = input > 0 ? top : 0 (input = the relu's input). */
+int lten_hip_relu_f32(float* dst, const float* src, uint64_t len);
+int lten_hip_relu_backward_f32(float* bottom, const float* top, const float* input, uint64_t len);
+/* gpu_mul(N, alpha, A, B) (l-ten/math_fns.h:137): y = alpha * x; what nll_backward is made of
+ * (l-ten/backprop.cpp:3975-4040: bottom = (-1 / batch * top) * target). */
+int lten_hip_scale_f32(uint64_t n, float alpha, const float* x, float* y);
+/* cublasSaxpy as l-ten uses it to accumulate a leaf's gradient (l-ten/backprop.cpp:246-274): y += alpha * x. */
+int lten_hip_axpy_f32(uint64_t n, float alpha, const float* x, float* y);
+/* lten::log_softmax along the last dimension (l-ten/layers.cpp:93-114: max, sub, exp, sum, div, log as one kernel)
+ * for x[rows][cols], and the sum of l-ten's backward functions of that chain: dx = dy - exp(y) * sum_j dy_j. */
+int lten_hip_log_softmax_f32(uint64_t rows, uint64_t cols, const float* x, float* y);
+int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float* y, const float* dy, float* dx);
+/* gpu_nll (l-ten/math_fns.h:170; l-ten/layers.cpp:212-273): *loss = (sum_i input[i] * target[i]) * (-1 / batches). */
+int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, uint64_t len, uint64_t batches);
+
 /* ----------------------------------------------------------------------- measurement */
 
 /* HIP events on the library's stream; no counterpart in l-ten (its benchmarks use

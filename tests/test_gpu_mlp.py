@@ -1,0 +1,104 @@
+"""GPU parity tests of the element-wise / loss kernels and of a whole MLP training step on the device (C ABI):
+FullyConnected(+bias) -> relu -> FullyConnected -> relu -> FullyConnected -> log_softmax -> nll_loss, then backward.
+fp32: max relative error 1e-4 (conftest.rel_err); relu and its backward are selections and must match exactly."""
+import numpy as np
+import pytest
+
+from conftest import golden_path, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def gpu_mlp_step(gpu, X, Ws, bs, T):
+    """The step through the C ABI, every intermediate resident on the device.  Returns what ob.mlp_step returns."""
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    B, layers = X.shape[0], len(Ws)
+    sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
+    dW_, db_ = [D.from_numpy(w) for w in Ws], [D.from_numpy(b) for b in bs]
+    pre = [None] + [D(4 * B * n) for n in sizes[1:]]
+    act = [D.from_numpy(X)] + [D(4 * B * n) for n in sizes[1:-1]] + [None]
+    act[layers] = pre[layers]
+    for i in range(layers):
+        gpu.check(l.lten_hip_fc_forward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr))
+        if i + 1 < layers:
+            gpu.check(l.lten_hip_relu_f32(act[i + 1].ptr, pre[i + 1].ptr, B * sizes[i + 1]))
+    dT, logp, loss = D.from_numpy(T), D(4 * B * sizes[-1]), D(4)
+    gpu.check(l.lten_hip_log_softmax_f32(B, sizes[-1], pre[layers].ptr, logp.ptr))
+    gpu.check(l.lten_hip_nll_loss_f32(logp.ptr, dT.ptr, loss.ptr, B * sizes[-1], B))
+    # backward from the loss: nll_backward (top = 1), log_softmax backward, then the layers
+    g = [D(4 * B * n) for n in sizes]
+    gl = D(4 * B * sizes[-1])
+    gpu.check(l.lten_hip_scale_f32(B * sizes[-1], -1.0 / B, dT.ptr, gl.ptr))
+    gpu.check(l.lten_hip_log_softmax_backward_f32(B, sizes[-1], logp.ptr, gl.ptr, g[layers].ptr))
+    gW, gb = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
+    tmp = [D(4 * B * n) for n in sizes]
+    for i in range(layers - 1, -1, -1):
+        gpu.check(l.lten_hip_fc_backward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, g[i + 1].ptr, tmp[i].ptr, gW[i].ptr, gb[i].ptr))
+        if i > 0:
+            gpu.check(l.lten_hip_relu_backward_f32(g[i].ptr, tmp[i].ptr, pre[i].ptr, B * sizes[i]))
+    return dict(loss=float(loss.numpy(np.float32, (1,))[0]), logp=logp.numpy(np.float32, T.shape),
+                dW=[gW[i].numpy(np.float32, Ws[i].shape) for i in range(layers)],
+                db=[gb[i].numpy(np.float32, bs[i].shape) for i in range(layers)], dX=tmp[0].numpy(np.float32, X.shape))
+
+
+def check_step(got, want, tag):
+    assert abs(got["loss"] - want["loss"]) < 1e-5 * max(1.0, abs(want["loss"])), tag
+    assert rel_err(got["logp"], want["logp"]) < TOL, tag
+    assert rel_err(got["dX"], want["dX"]) < TOL, tag
+    for i in range(len(want["dW"])):
+        assert rel_err(got["dW"][i], want["dW"][i]) < TOL, (tag, i)
+        assert rel_err(got["db"][i], want["db"][i]) < TOL, (tag, i)
+
+
+def test_mlp_step_golden_from_compiled_network(gpu):
+    g = np.load(golden_path("mlp_step_case.npz"))
+    Ws, bs = [g[f"W{i}"] for i in range(3)], [g[f"b{i}"] for i in range(3)]
+    got = gpu_mlp_step(gpu, g["X"], Ws, bs, g["T"])
+    want = dict(loss=float(g["loss"]), logp=g["logp"], dX=g["dX"], dW=[g[f"dW{i}"] for i in range(3)], db=[g[f"db{i}"] for i in range(3)])
+    check_step(got, want, "golden")
+
+
+def test_cfg2_training_step_full_size(gpu, ob, wl):
+    """784 -> 1024 -> 1024 -> 10 with bias and relu at batch 128, loss = nll(log_softmax), against the oracle's step."""
+    X, Ws, bs, labels = wl.cfg2()
+    T = np.eye(10, dtype=np.float32)[labels]
+    want = ob.mlp_step(X, Ws, bs, T)
+    got = gpu_mlp_step(gpu, X, Ws, bs, T)
+    check_step(got, want, "cfg2")
+    errs = [rel_err(got["dW"][i], want["dW"][i]) for i in range(3)]
+    print(f"  loss {got['loss']:.6f} (oracle {want['loss']:.6f}); dW max rel err {max(errs):.2e}")
+
+
+def test_elementwise_kernels(gpu, ob):
+    rng = np.random.default_rng(9)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    for n in (1, 63, 1000, 1 << 20):
+        x = rng.standard_normal(n).astype(np.float32)
+        x[::5] = 0.0
+        top = rng.standard_normal(n).astype(np.float32)
+        dx, dt, dy, db = D.from_numpy(x), D.from_numpy(top), D(4 * n), D(4 * n)
+        gpu.check(l.lten_hip_relu_f32(dy.ptr, dx.ptr, n))
+        gpu.check(l.lten_hip_relu_backward_f32(db.ptr, dt.ptr, dx.ptr, n))
+        assert np.array_equal(dy.numpy(np.float32, (n,)), np.where(x > 0, x, np.float32(0)))
+        assert np.array_equal(db.numpy(np.float32, (n,)), np.where(x > 0, top, np.float32(0)))
+        gpu.check(l.lten_hip_scale_f32(n, -0.37, dx.ptr, dy.ptr))
+        assert np.array_equal(dy.numpy(np.float32, (n,)), np.float32(-0.37) * x)
+        gpu.check(l.lten_hip_axpy_f32(n, 1.0, dt.ptr, dy.ptr))
+        assert np.array_equal(dy.numpy(np.float32, (n,)), np.float32(-0.37) * x + top)
+    for rows, cols in ((1, 1), (128, 10), (37, 1000), (5, 4097)):
+        z = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+        dyv = rng.standard_normal((rows, cols)).astype(np.float32)
+        T = np.zeros((rows, cols), np.float32)
+        T[np.arange(rows), rng.integers(0, cols, rows)] = 1
+        want_lp, want_dx = np.empty_like(z), np.empty_like(z)
+        ob.oracle().oracle_log_softmax(rows, cols, z.reshape(-1), want_lp.reshape(-1))
+        ob.oracle().oracle_log_softmax_backward(rows, cols, want_lp.reshape(-1), dyv.reshape(-1), want_dx.reshape(-1))
+        dz, dlp, ddy, ddx, dT, dl = D.from_numpy(z), D(z.nbytes), D.from_numpy(dyv), D(z.nbytes), D.from_numpy(T), D(4)
+        gpu.check(l.lten_hip_log_softmax_f32(rows, cols, dz.ptr, dlp.ptr))
+        gpu.check(l.lten_hip_log_softmax_backward_f32(rows, cols, dlp.ptr, ddy.ptr, ddx.ptr))
+        gpu.check(l.lten_hip_nll_loss_f32(dlp.ptr, dT.ptr, dl.ptr, rows * cols, rows))
+        assert rel_err(dlp.numpy(np.float32, z.shape), want_lp) < 1e-5
+        assert rel_err(ddx.numpy(np.float32, z.shape), want_dx) < TOL
+        want_loss = ob.oracle().oracle_nll_loss(want_lp.reshape(-1), T.reshape(-1), rows * cols, rows)
+        assert abs(dl.numpy(np.float32, (1,))[0] - want_loss) < 1e-5 * max(1.0, abs(want_loss))
