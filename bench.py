@@ -136,32 +136,44 @@ def extra_configs(lt, wl, with_cpu):
         out.append(rec)
         del dA, dB, dC, ws
 
-    # ---- config 2: fp32 MLP 784-1024-1024-10, batch 128: 3 forward GEMMs with bias, 3 data-gradient GEMMs,
-    # 3 weight-gradient GEMMs, 3 bias-gradient column sums.  The element-wise pieces between them (ReLU, loss) are
-    # outside this path, so the timed chain feeds each GEMM from resident buffers of the right shape.
+    # ---- config 2: fp32 MLP 784-1024-1024-10, batch 128, one training step resident on the device: 3 forward GEMMs with
+    # bias, relu after the first two, log_softmax + nll_loss, their backward, then per layer the data-gradient GEMM,
+    # the weight-gradient GEMM, the bias-gradient column sum and relu_backward.
     X, Ws, bs, labels = wl.cfg2()
     B_ = X.shape[0]
     sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
-    acts = [D.from_numpy(X)] + [D(4 * B_ * n) for n in sizes[1:]]
+    pre = [None] + [D(4 * B_ * n) for n in sizes[1:]]
+    acts = [D.from_numpy(X)] + [D(4 * B_ * n) for n in sizes[1:-1]] + [pre[-1]]
     grads = [D(4 * B_ * n, zero=True) for n in sizes]
+    tmpg = [D(4 * B_ * n, zero=True) for n in sizes]
     dWs, dbs = [D.from_numpy(w) for w in Ws], [D.from_numpy(b) for b in bs]
     gWs, gbs_ = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
-    lt.check(l.lten_hip_fill_f32(grads[-1].ptr, B_ * sizes[-1], 0.01))
+    dT = D.from_numpy(np.eye(sizes[-1], dtype=np.float32)[labels])
+    logp, gl, loss = D(4 * B_ * sizes[-1]), D(4 * B_ * sizes[-1]), D(4)
 
     def mlp_step():
         for i in range(3):
-            lt.check(l.lten_hip_fc_forward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, dbs[i].ptr, acts[i + 1].ptr))
+            lt.check(l.lten_hip_fc_forward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, dbs[i].ptr, pre[i + 1].ptr))
+            if i < 2:
+                lt.check(l.lten_hip_relu_f32(acts[i + 1].ptr, pre[i + 1].ptr, B_ * sizes[i + 1]))
+        lt.check(l.lten_hip_log_softmax_f32(B_, sizes[-1], pre[3].ptr, logp.ptr))
+        lt.check(l.lten_hip_nll_loss_f32(logp.ptr, dT.ptr, loss.ptr, B_ * sizes[-1], B_))
+        lt.check(l.lten_hip_scale_f32(B_ * sizes[-1], -1.0 / B_, dT.ptr, gl.ptr))
+        lt.check(l.lten_hip_log_softmax_backward_f32(B_, sizes[-1], logp.ptr, gl.ptr, grads[3].ptr))
         for i in (2, 1, 0):
             lt.check(l.lten_hip_fc_backward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, grads[i + 1].ptr,
-                                                grads[i].ptr, gWs[i].ptr, gbs_[i].ptr))
+                                                tmpg[i].ptr, gWs[i].ptr, gbs_[i].ptr))
+            if i > 0:
+                lt.check(l.lten_hip_relu_backward_f32(grads[i].ptr, tmpg[i].ptr, pre[i].ptr, B_ * sizes[i]))
     ms = timed(lt, mlp_step, 100)
     flops = sum(3 * 2.0 * B_ * sizes[i] * sizes[i + 1] for i in range(3))
     tf = flops / ms / 1e9
-    rec = {"config": "cfg2 fp32 MLP 784-1024-1024-10 batch 128, forward + backward GEMMs (9 GEMMs, 3 bias adds fused, 3 column sums)",
+    rec = {"config": "cfg2 fp32 MLP 784-1024-1024-10 batch 128, one training step on the device (9 GEMMs with the bias adds fused, "
+                     "3 column sums, relu x2, log_softmax, nll_loss and their backward: 20 launches)",
            "gpu_us": round(ms * 1e3, 2), "gflop_per_step": round(flops / 1e9, 3),
            "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)},
-           "note": "twelve small launches; launch latency, not the MFMA rate, sets this time"}
+           "note": "twenty small launches; launch and memory latency, not the MFMA rate, set this time (GEMM flops only in the rate)"}
     if with_cpu:
         hA = [np.random.default_rng(i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
         hG = [np.random.default_rng(9 + i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
@@ -177,9 +189,9 @@ def extra_configs(lt, wl, with_cpu):
         cpu_step()
         t = best_of(cpu_step, 5)
         rec.update(cpu_ms=round(t * 1e3, 2), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)), speedup=round(t * 1e3 / ms, 1),
-                   cpu_note="l-ten's own threadpool + AVX cpu_gemm (its non-OpenBLAS build); bias rank-1 and column-sum GEMMs left out of the CPU leg")
+                   cpu_note="l-ten's own threadpool + AVX cpu_gemm (its non-OpenBLAS build); bias, column-sum, relu and loss pieces left out of the CPU leg")
     out.append(rec)
-    del acts, grads, dWs, dbs, gWs, gbs_
+    del acts, pre, grads, tmpg, dWs, dbs, gWs, gbs_
 
     # ---- config 5: Conv2d 3x3 s1 p1, 32x1x128x128 -> 32 ch -> 64 ch: forward + weight gradient of both layers
     x, cws, dyshapes = wl.cfg5()

@@ -406,6 +406,111 @@ Tensor FullyConnected::forward(Tensor& input)
 	return result;
 }
 
+// ------------------------------------------------------------------------------ relu, log_softmax, nll_loss
+
+static void require_gpu_f32(const Tensor& t, const char* what)
+{
+	if (t.get_data_type() != FLOAT32) LTEN_ERR("Not yet implemented");
+	if (t.get_device() != GPU) {
+		static std::string msg;
+		msg = std::string("this build implements ") + what + " for the GPU device type only (l-ten's own CPU path covers lten::CPU)";
+		LTEN_ERR(msg.c_str());
+	}
+}
+
+Tensor relu(Tensor& input)
+{
+	require_gpu_f32(input, "relu");
+	TensorOps options;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor(input.get_sizes(), input.get_ndims(), &options);
+	const uint64_t n = input.get_numels();
+	LTEN_HIP_CALL(lten_hip_relu_f32(static_cast<float*>(result.get_data_ptr()), static_cast<const float*>(input.get_data_ptr()), n));  // gpu_relu
+	auto in = input.get_smart_ptr();
+	result.get_smart_ptr()->children = { in };  // l-ten/layers.cpp:61-63
+	result.get_smart_ptr()->autograd = true;
+	result.get_smart_ptr()->grad_fn = [in, n](TensorImpl&, const float* top) {
+		if (!wants_gradient(in)) return;
+		Bottom g(in);
+		if (g.temporary) {  // l-ten/backprop.cpp:2282-2327: bottom = input > 0 ? top : 0
+			LTEN_HIP_CALL(lten_hip_relu_backward_f32(g.ptr, top, static_cast<const float*>(in->data), n));
+		} else {  // a leaf accumulates (l-ten/backprop.cpp:246-274)
+			float* tmp = static_cast<float*>(TensorImpl::alloc(GPU, n * sizeof(float), false));
+			LTEN_HIP_CALL(lten_hip_relu_backward_f32(tmp, top, static_cast<const float*>(in->data), n));
+			LTEN_HIP_CALL(lten_hip_axpy_f32(n, 1.0f, tmp, g.ptr));
+			LTEN_HIP_CALL(lten_hip_sync());
+			TensorImpl::release(GPU, tmp);
+		}
+		g.propagate();
+	};
+	return result;
+}
+
+Tensor log_softmax(Tensor& input, int dim)
+{
+	require_gpu_f32(input, "log_softmax");
+	const int ndims = input.get_ndims();
+	if (dim != ndims - 1) LTEN_ERR("this build implements log_softmax along the last dimension only");
+	const uint64_t cols = input.get_sizes()[ndims - 1], rows = cols ? input.get_numels() / cols : 0;
+	TensorOps options;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor(input.get_sizes(), ndims, &options);
+	LTEN_HIP_CALL(lten_hip_log_softmax_f32(rows, cols, static_cast<const float*>(input.get_data_ptr()), static_cast<float*>(result.get_data_ptr())));
+	auto in = input.get_smart_ptr(), out = result.get_smart_ptr();
+	TensorImpl* out_raw = out.get();  // the node owns the closure: no shared_ptr cycle
+	result.get_smart_ptr()->children = { in };
+	result.get_smart_ptr()->autograd = true;
+	result.get_smart_ptr()->grad_fn = [in, out_raw, rows, cols](TensorImpl&, const float* top) {
+		if (!wants_gradient(in)) return;
+		Bottom g(in);
+		const uint64_t n = rows * cols;
+		float* tmp = g.temporary ? g.ptr : static_cast<float*>(TensorImpl::alloc(GPU, n * sizeof(float), false));
+		// l-ten's backward functions of log, div, sum, exp, sub and max add up to dy - exp(y) * sum_j dy_j
+		LTEN_HIP_CALL(lten_hip_log_softmax_backward_f32(rows, cols, static_cast<const float*>(out_raw->data), top, tmp));
+		if (!g.temporary) {
+			LTEN_HIP_CALL(lten_hip_axpy_f32(n, 1.0f, tmp, g.ptr));
+			LTEN_HIP_CALL(lten_hip_sync());
+			TensorImpl::release(GPU, tmp);
+		}
+		g.propagate();
+	};
+	return result;
+}
+
+Tensor nll_loss(Tensor& input, Tensor& target)
+{
+	require_gpu_f32(input, "nll_loss");
+	require_gpu_f32(target, "nll_loss");
+	if (input.get_numels() != target.get_numels()) LTEN_ERR("nll_loss: input and target must have the same number of elements");
+	TensorOps options;
+	options.device_index = input.get_device_index();
+	options.device_type = GPU;
+	Tensor result = AllocateTensor({ 1 }, &options);  // l-ten/layers.cpp:231-232
+	const uint64_t len = input.get_numels(), batch = input.get_sizes()[0];
+	LTEN_HIP_CALL(lten_hip_nll_loss_f32(static_cast<const float*>(input.get_data_ptr()), static_cast<const float*>(target.get_data_ptr()),
+	                                    static_cast<float*>(result.get_data_ptr()), len, batch));  // gpu_nll, :254
+	auto in = input.get_smart_ptr(), tg = target.get_smart_ptr();
+	result.get_smart_ptr()->children = { in, tg };  // :266-269
+	result.get_smart_ptr()->autograd = true;
+	result.get_smart_ptr()->grad_fn = [in, tg, len, batch](TensorImpl&, const float* top) {
+		// l-ten/backprop.cpp:3975-4040: scale = -1 / batch * top[0]; bottom = scale * (the other operand)
+		float top_value = 1.0f;
+		LTEN_HIP_CALL(lten_hip_copy_from_gpu(&top_value, top, sizeof(float)));
+		const float scale = (-1.0f / (float)batch) * top_value;
+		const std::shared_ptr<TensorImpl> pair[2][2] = { { in, tg }, { tg, in } };
+		for (auto& p : pair) {
+			if (!wants_gradient(p[0])) continue;
+			Bottom g(p[0]);
+			if (g.temporary) LTEN_HIP_CALL(lten_hip_scale_f32(len, scale, static_cast<const float*>(p[1]->data), g.ptr));
+			else LTEN_HIP_CALL(lten_hip_axpy_f32(len, scale, static_cast<const float*>(p[1]->data), g.ptr));
+			g.propagate();
+		}
+	};
+	return result;
+}
+
 // ------------------------------------------------------------------------------ FullyConnected_q
 
 bool FullyConnected_q::init()

@@ -95,6 +95,11 @@ Tensor TensorFromBuffer(const uint64_t* dims_ptr, int ndims, void* data_ptr, boo
 Tensor AllocateTensor(const std::initializer_list<uint64_t>& dims, TensorOps* options_ptr = nullptr);
 Tensor AllocateTensor(const uint64_t* dims_ptr, int ndims, TensorOps* options_ptr = nullptr);
 
+// l-ten/layers.h (free functions): the element-wise and loss pieces of a training step, GPU tensors only.
+Tensor relu(Tensor& input);                        // l-ten/layers.cpp:9-67
+Tensor log_softmax(Tensor& input, int dim);        // l-ten/layers.cpp:93-114; dim must be the last dimension here
+Tensor nll_loss(Tensor& input, Tensor& target);    // l-ten/layers.cpp:212-273
+
 // l-ten/layers.h:14-31
 class Module {
 public:

@@ -122,6 +122,63 @@ static int fc_chain_test()
 	return 0;
 }
 
+// A whole training step through the layer API, as l-ten's MNIST tests write it: FullyConnected -> relu -> FullyConnected ->
+// log_softmax -> nll_loss, then loss.backward(); against plain loops in double precision.
+static int mlp_step_test()
+{
+	const uint64_t B = 5, F0 = 7, F1 = 6, F2 = 4;
+	std::vector<float> x(B * F0), w1(F1 * F0), b1(F1), w2(F2 * F1), b2(F2), t(B * F2, 0.0f);
+	unsigned s = 777;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (float)((s >> 16) & 0xFF) / 128.0f - 1.0f; };
+	for (auto* v : { &x, &w1, &b1, &w2, &b2 }) for (auto& e : *v) e = rnd();
+	for (uint64_t m = 0; m < B; m++) t[m * F2 + (m * 3) % F2] = 1.0f;
+	lten::Tensor X = lten::TensorFromBuffer({ B, 1, 1, F0 }, x.data());
+	X.set_autograd(true);
+	X = X.to(lten::GPU);
+	lten::Tensor T = lten::TensorFromBuffer({ B, 1, 1, F2 }, t.data()).to(lten::GPU);
+	lten::FullyConnected fc1(F0, F1, true), fc2(F1, F2, true);
+	fc1.init();
+	fc2.init();
+	memcpy(fc1.get_weights()->get_data_ptr(), w1.data(), w1.size() * 4);
+	memcpy(fc1.get_bias()->get_data_ptr(), b1.data(), b1.size() * 4);
+	memcpy(fc2.get_weights()->get_data_ptr(), w2.data(), w2.size() * 4);
+	memcpy(fc2.get_bias()->get_data_ptr(), b2.data(), b2.size() * 4);
+	fc1.to(lten::GPU);
+	fc2.to(lten::GPU);
+	lten::Tensor h = fc1.forward(X);
+	lten::Tensor a = lten::relu(h);
+	lten::Tensor y = fc2.forward(a);
+	lten::Tensor lp = lten::log_softmax(y, 3);
+	lten::Tensor loss = lten::nll_loss(lp, T);
+	loss.backward();
+	// plain loops
+	std::vector<double> H(B * F1), A(B * F1), Y(B * F2), LP(B * F2), dY(B * F2), dA(B * F1, 0), dH(B * F1), dX(B * F0, 0), dW1(F1 * F0, 0), dW2(F2 * F1, 0), dB1(F1, 0), dB2(F2, 0);
+	double L = 0;
+	for (uint64_t m = 0; m < B; m++) {
+		for (uint64_t j = 0; j < F1; j++) { double v = b1[j]; for (uint64_t k = 0; k < F0; k++) v += (double)x[m * F0 + k] * w1[j * F0 + k]; H[m * F1 + j] = v; A[m * F1 + j] = v > 0 ? v : 0; }
+		double mx = -1e300, se = 0;
+		for (uint64_t j = 0; j < F2; j++) { double v = b2[j]; for (uint64_t k = 0; k < F1; k++) v += A[m * F1 + k] * w2[j * F1 + k]; Y[m * F2 + j] = v; if (v > mx) mx = v; }
+		for (uint64_t j = 0; j < F2; j++) se += exp(Y[m * F2 + j] - mx);
+		for (uint64_t j = 0; j < F2; j++) { LP[m * F2 + j] = Y[m * F2 + j] - mx - log(se); L -= LP[m * F2 + j] * t[m * F2 + j] / B; }
+		for (uint64_t j = 0; j < F2; j++) dY[m * F2 + j] = (exp(LP[m * F2 + j]) - t[m * F2 + j]) / B;  // softmax - onehot, over the batch
+		for (uint64_t j = 0; j < F2; j++) { dB2[j] += dY[m * F2 + j]; for (uint64_t k = 0; k < F1; k++) { dA[m * F1 + k] += dY[m * F2 + j] * w2[j * F1 + k]; dW2[j * F1 + k] += dY[m * F2 + j] * A[m * F1 + k]; } }
+		for (uint64_t j = 0; j < F1; j++) { dH[m * F1 + j] = H[m * F1 + j] > 0 ? dA[m * F1 + j] : 0; dB1[j] += dH[m * F1 + j]; for (uint64_t k = 0; k < F0; k++) { dX[m * F0 + k] += dH[m * F1 + j] * w1[j * F0 + k]; dW1[j * F0 + k] += dH[m * F1 + j] * x[m * F0 + k]; } }
+	}
+	auto f32 = [](const std::vector<double>& v) { return std::vector<float>(v.begin(), v.end()); };
+	const double tol = 1e-4;
+	lten::Tensor lc = loss.to(lten::CPU);
+	float Lf = (float)L;
+	if (Compare((float*)lc.get_data_ptr(), &Lf, 1, tol)) return -1;
+	lten::Tensor lpc = lp.to(lten::CPU);
+	if (Compare((float*)lpc.get_data_ptr(), f32(LP).data(), LP.size(), tol)) return -2;
+	if (Compare(grad_to_host(X).data(), f32(dX).data(), dX.size(), tol)) return -3;
+	if (Compare(grad_to_host(*fc1.get_weights()).data(), f32(dW1).data(), dW1.size(), tol)) return -4;
+	if (Compare(grad_to_host(*fc2.get_weights()).data(), f32(dW2).data(), dW2.size(), tol)) return -5;
+	if (Compare(grad_to_host(*fc1.get_bias()).data(), f32(dB1).data(), dB1.size(), tol)) return -6;
+	if (Compare(grad_to_host(*fc2.get_bias()).data(), f32(dB2).data(), dB2.size(), tol)) return -7;
+	return 0;
+}
+
 // FullyConnected_q on {2, 3, 37} with bias: every leading index is its own quantized_matmul in l-ten
 static int fcq_test()
 {
@@ -269,7 +326,7 @@ static int error_test()
 
 int main()
 {
-	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test },
+	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test },
 		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;
 	for (auto& t : tests) {
