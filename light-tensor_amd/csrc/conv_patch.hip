@@ -28,7 +28,7 @@ namespace lten_hip {
 // LDS weights: [step][channel parity][WROW = 65] (the odd row length spreads the scattered stores over banks).
 template <int KH, int KW>
 struct PatchFwd {
-	static constexpr int CB = 4, TH = 4, TW = 128, BM = 64, T = 256;
+	static constexpr int CB = 4, TH = 4, TW = 128, NT = TW / 32, BM = 64, T = 256;
 	static constexpr int PR = TH + KH - 1;
 	static constexpr int PWS = (4 + TW + KW - 1 + 3) / 4 * 4;
 	static constexpr int F4_ROW = PWS / 4;
@@ -95,11 +95,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		}
 	};
 
-	v16f acc[2][4];
+	v16f acc[2][P::NT];
 #pragma unroll
 	for (int m = 0; m < 2; m++)
 #pragma unroll
-		for (int t = 0; t < 4; t++)
+		for (int t = 0; t < P::NT; t++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) acc[m][t][r] = 0.0f;
 
@@ -112,20 +112,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		__syncthreads();
 		if (c0 + P::CB < g.Cin) load_chunk(c0 + P::CB);
 		// operands of step s + 1 are read while the MFMAs of step s issue, one LDS read behind each MFMA
-		float fa[2][2], fb[2][4];
+		constexpr int NR = 2 + P::NT, NM = 2 * P::NT;  // LDS reads and MFMAs per step
+		float fa[2][2], fb[2][P::NT];
 		auto read_operand = [&](int s, int e) {
 			const int cp = s / P::TAPS, tap = s % P::TAPS, i = tap / KW, j = tap % KW;
 			if (e < 2) fa[s & 1][e] = pa[s * 2 * P::WROW + e * 32];
 			else fb[s & 1][e - 2] = pb[(2 * cp * P::PR + i) * P::PWS + j + (e - 2) * 32];
 		};
 #pragma unroll
-		for (int e = 0; e < 6; e++) read_operand(0, e);
+		for (int e = 0; e < NR; e++) read_operand(0, e);
 #pragma unroll
 		for (int s = 0; s < P::KSTEPS; s++) {
 #pragma unroll
-			for (int e = 0; e < 8; e++) {
-				acc[e >> 2][e & 3] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1][e >> 2], fb[s & 1][e & 3], acc[e >> 2][e & 3], 0, 0, 0);
-				if (e < 6 && s + 1 < P::KSTEPS) read_operand(s + 1, e);
+			for (int e = 0; e < NM; e++) {
+				acc[e / P::NT][e % P::NT] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1][e / P::NT], fb[s & 1][e % P::NT], acc[e / P::NT][e % P::NT], 0, 0, 0);
+				if (s + 1 < P::KSTEPS) {
+					if (e < NR) read_operand(s + 1, e);
+					if (e == NM - 1 && NR > NM) read_operand(s + 1, NR - 1);
+				}
 				__builtin_amdgcn_sched_barrier(0);
 			}
 		}
@@ -143,7 +147,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 			const float b = bias ? bias[co] : 0.0f;
 			float* yrow = y + (((int64_t)n * g.Cout + co) * g.Ho + ho) * g.Wo;
 #pragma unroll
-			for (int t = 0; t < 4; t++) {
+			for (int t = 0; t < P::NT; t++) {
 				const int wo = w0 + t * 32 + lrow;
 				if (wo < g.Wo) yrow[wo] = acc[m][t][r] + b;
 			}

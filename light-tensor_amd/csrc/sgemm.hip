@@ -137,9 +137,135 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 	}
 }
 
+// The same decomposition with whole cache lines per load: the direct kernel above asks the texture addresser for 32
+// different lines per wave-wide load (32 rows x 32 bytes), which is what bounds it at these sizes.  Here a wave-wide
+// 16-byte load covers 8 rows x 128 bytes along the operand's contiguous dimension (8 lines), the values pass through
+// a wavefront-private LDS slab (no barrier: LDS operations of one wavefront complete in order) and come back in
+// the MFMA lane layout.  A batch is 32 k-values; wavefront w takes batches w, w + WAVES, ...; the loads of up to
+// UB batches are in flight at once.  Operand rows of 36 floats keep both the 16-byte stores and the reads free of
+// bank conflicts.  Used when the operands allow 16-byte loads (leading dimensions and bases multiples of 4 floats).
+template <int WAVES, bool TA, bool TB>
+__global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
+{
+	constexpr int UB = 4, LD = 36, SLAB = 32 * LD;
+	__shared__ __attribute__((aligned(16))) float lds[WAVES * 2 * SLAB > WAVES * 1024 ? WAVES * 2 * SLAB : WAVES * 1024];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int lrow = lane & 31, g = lane >> 5;
+	const int tiles_n = (p.N + 31) / 32;
+	const int m0 = (blockIdx.x / tiles_n) * 32, n0 = (blockIdx.x % tiles_n) * 32;
+	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
+	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
+	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+	float* sA = lds + wave * 2 * SLAB;
+	float* sB = sA + SLAB;
+	const int r8 = lane >> 3, c4 = (lane & 7) * 4;  // this lane's row within a group of 8 and its 4-float column
+
+	v16f acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+	// one operand, one batch: four 16-byte loads per lane
+	auto fetch = [&](const float* base, int64_t ld, bool k_contig, int rows_limit, int row0, int k0, float4 (&v)[4]) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int q = 8 * i + r8;  // k_contig: tile row, else: k offset inside the batch
+			v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (k_contig) {
+				const int row = row0 + q, k = k0 + c4;
+				if (row < rows_limit && k < p.K) {
+					const float* src = base + (int64_t)row * ld + k;
+					if (k + 3 < p.K) v[i] = *reinterpret_cast<const float4*>(src);
+					else { v[i].x = src[0]; if (k + 1 < p.K) v[i].y = src[1]; if (k + 2 < p.K) v[i].z = src[2]; }
+				}
+			} else {
+				const int k = k0 + q, col = row0 + c4;
+				if (k < p.K && col < rows_limit) {
+					const float* src = base + (int64_t)k * ld + col;
+					if (col + 3 < rows_limit) v[i] = *reinterpret_cast<const float4*>(src);
+					else { v[i].x = src[0]; if (col + 1 < rows_limit) v[i].y = src[1]; if (col + 2 < rows_limit) v[i].z = src[2]; }
+				}
+			}
+		}
+	};
+	// slab layouts: k-contiguous operand [tile row][k], the other [k][tile row]; both rows of LD floats
+	auto stage = [&](float* slab, const float4 (&v)[4]) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) *reinterpret_cast<float4*>(slab + (8 * i + r8) * LD + c4) = v[i];
+	};
+
+	const int batches = (p.K + 31) / 32;
+	for (int b0 = wave; b0 < batches; b0 += WAVES * UB) {
+		float4 va[UB][4], vb[UB][4];
+#pragma unroll
+		for (int u = 0; u < UB; u++) {
+			const int b = b0 + u * WAVES;
+			if (b < batches) {
+				fetch(A, p.lda, !TA, p.M, m0, b * 32, va[u]);
+				fetch(B, p.ldb, TB, p.N, n0, b * 32, vb[u]);
+			}
+		}
+#pragma unroll
+		for (int u = 0; u < UB; u++) {
+			if (b0 + u * WAVES >= batches) break;
+			stage(sA, va[u]);
+			stage(sB, vb[u]);
+#pragma unroll
+			for (int q = 0; q < 4; q++) {
+				// MFMA step (q, t) multiplies k = 8q + 4g + t of the batch
+				float a[4], bb[4];
+				if (!TA) {
+					const float4 t4 = *reinterpret_cast<const float4*>(sA + lrow * LD + 8 * q + 4 * g);
+					a[0] = t4.x; a[1] = t4.y; a[2] = t4.z; a[3] = t4.w;
+				} else {
+#pragma unroll
+					for (int t = 0; t < 4; t++) a[t] = sA[(8 * q + 4 * g + t) * LD + lrow];
+				}
+				if (TB) {
+					const float4 t4 = *reinterpret_cast<const float4*>(sB + lrow * LD + 8 * q + 4 * g);
+					bb[0] = t4.x; bb[1] = t4.y; bb[2] = t4.z; bb[3] = t4.w;
+				} else {
+#pragma unroll
+					for (int t = 0; t < 4; t++) bb[t] = sB[(8 * q + 4 * g + t) * LD + lrow];
+				}
+#pragma unroll
+				for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], bb[t], acc, 0, 0, 0);
+			}
+		}
+	}
+
+	// the wavefronts' partial tiles meet in LDS (the slabs are no longer needed) and are added in wavefront order
+	__syncthreads();
+#pragma unroll
+	for (int r = 0; r < 16; r++) lds[wave * 1024 + ((r >> 2) * 8 + g * 4 + (r & 3)) * 32 + lrow] = acc[r];
+	__syncthreads();
+	for (int idx = tid; idx < 32 * 32; idx += WAVES * 64) {
+		const int row = idx >> 5, col = idx & 31;
+		if (m0 + row >= p.M || n0 + col >= p.N) continue;
+		float sum = 0.0f;
+#pragma unroll
+		for (int w = 0; w < WAVES; w++) sum += lds[w * 1024 + idx];
+		float* c = C + (int64_t)(m0 + row) * p.ldc + n0 + col;
+		float out = p.alpha * sum;
+		if (p.beta != 0.0f) out += p.beta * *c;
+		if (p.bias) out += p.bias[n0 + col];
+		*c = out;
+	}
+}
+
 static int launch_direct(const SProblem& p, int tA, int tB, uint64_t batch)
 {
 	const dim3 grid((unsigned)(ceil_div(p.M, 32) * ceil_div(p.N, 32)), 1, (unsigned)batch), block(8 * 64);
+	const bool vec = (p.lda & 3) == 0 && (p.ldb & 3) == 0 && (p.stride_a & 3) == 0 && (p.stride_b & 3) == 0 &&
+	                 ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
+	if (vec && p.K >= 512 && get_option(OPT_SGEMM_TILE) != 5) {  // at least two batches per wavefront
+		set_kernel_name("sgemm_staged_32x32_w8");
+		if (!tA && !tB) sgemm_staged_kernel<8, false, false><<<grid, block, 0, stream()>>>(p);
+		if (!tA && tB) sgemm_staged_kernel<8, false, true><<<grid, block, 0, stream()>>>(p);
+		if (tA && !tB) sgemm_staged_kernel<8, true, false><<<grid, block, 0, stream()>>>(p);
+		if (tA && tB) sgemm_staged_kernel<8, true, true><<<grid, block, 0, stream()>>>(p);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	set_kernel_name("sgemm_direct_32x32_w8");
 	if (!tA && !tB) sgemm_direct_kernel<8, false, false><<<grid, block, 0, stream()>>>(p);
 	if (!tA && tB) sgemm_direct_kernel<8, false, true><<<grid, block, 0, stream()>>>(p);
@@ -247,8 +373,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		// Few output tiles and a long K: the LDS-tiled kernels would leave most CUs idle while a handful of
 		// workgroups walk K in sequence; the direct kernel cuts K across the wavefronts of a workgroup instead.
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32) * batch;
-		// (with a short K and enough 64x64 tiles to occupy half the CUs the tiled kernel is the faster one)
-		if (tiles32 <= 1024 && !(tiles64 >= 128 && K <= 256)) choice = 4;
+		if (tiles32 <= 1024) choice = 4;
 		else choice = tiles128 >= 128 ? 1 : 2;
 	}
 	switch (choice) {

@@ -79,19 +79,30 @@ def test_cfg2_gemm_shapes_all_layouts(gpu, ob, shape):
         assert err < TOL
 
 
-def test_direct_kernel_is_deterministic_and_repeatable(gpu):
-    """The direct kernel adds its wavefronts' partial tiles in wavefront order: bitwise equal results run after run."""
+@pytest.mark.parametrize("tile,name", [(0, "sgemm_staged"), (5, "sgemm_direct")])
+def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
+    """The small-output kernels (LDS-staged and direct operand loads) add their wavefronts' partial tiles in wavefront
+    order: bitwise equal results run after run; all layouts, ragged M / N / K, beta, batches."""
     rng = np.random.default_rng(3)
-    M, N, K = 128, 1024, 1024
-    A = rng.standard_normal((M, K)).astype(np.float32)
-    B = rng.standard_normal((N, K)).astype(np.float32)
-    z = np.zeros((M, N), np.float32)
-    first = gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N)
-    assert gpu.last_kernel().startswith("sgemm_direct")
-    for _ in range(5):
-        assert np.array_equal(gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N), first)
-    want = A.astype(np.float64) @ B.astype(np.float64).T
-    assert rel_err(first, want) < TOL
+    if True:
+        M, N, K = 128, 1024, 1024
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        B = rng.standard_normal((N, K)).astype(np.float32)
+        z = np.zeros((M, N), np.float32)
+        first = gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N, tile=tile)
+        assert gpu.last_kernel().startswith(name)
+        for _ in range(5):
+            assert np.array_equal(gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N, tile=tile), first)
+        want = A.astype(np.float64) @ B.astype(np.float64).T
+        assert rel_err(first, want) < TOL
+        for (tA, tB, m, n, k) in [(0, 0, 70, 100, 532), (0, 1, 33, 31, 788), (1, 0, 100, 36, 660), (1, 1, 20, 65, 596)]:
+            a = rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32)
+            b = rng.standard_normal((n, k) if tB else (k, n)).astype(np.float32)
+            c0 = rng.standard_normal((m, n)).astype(np.float32)
+            got = gpu_sgemm(gpu, tA, tB, m, n, k, 0.5, a, a.shape[1], b, b.shape[1], 2.0, c0, n, tile=tile)
+            assert gpu.last_kernel().startswith(name), gpu.last_kernel()
+            opa, opb = (a.T if tA else a).astype(np.float64), (b.T if tB else b).astype(np.float64)
+            assert rel_err(got, 0.5 * opa @ opb + 2.0 * c0) < TOL, (tA, tB, m, n, k)
 
 
 def test_rank1_and_rowvec_shapes(gpu, ob):
