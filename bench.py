@@ -203,6 +203,7 @@ def extra_configs(lt, wl, with_cpu):
     ddw = [D(w.nbytes) for w in cws]
     geos = [(Nimg, chans[i], H, Wd, chans[i + 1], 3, 3, 1, 1, 1, 1) for i in range(2)]
     wss = [D(max(int(l.lten_hip_conv2d_wgrad_workspace_bytes(*g)), 4)) for g in geos]
+    wsx = D(x.nbytes)  # the data gradient of layer 1 (not part of the configuration's timed pair) lands here
     for i, g in enumerate(geos):
         Cin, Cout = g[1], g[4]
         fl = 2.0 * Nimg * Cout * H * Wd * Cin * 9
@@ -210,9 +211,13 @@ def extra_configs(lt, wl, with_cpu):
         kf = lt.last_kernel()
         ms_w = timed(lt, lambda: lt.check(l.lten_hip_conv2d_wgrad_f32(*g, dx[i].ptr, ddy[i].ptr, ddw[i].ptr, wss[i].ptr)), 30)
         kw = lt.last_kernel()
+        wsd = D(max(int(l.lten_hip_conv2d_dgrad_workspace_bytes(*g)), 4))
+        ms_d = timed(lt, lambda: lt.check(l.lten_hip_conv2d_dgrad_f32(*g, dw_[i].ptr, ddy[i].ptr, dx[i].ptr if i else wsx.ptr, wsd.ptr)), 30)
+        kd = lt.last_kernel()
         in_b, out_b = 4 * Nimg * Cin * H * Wd, 4 * Nimg * Cout * H * Wd
         rec = {"config": f"cfg5 Conv2d layer {i + 1}: {Cin}->{Cout} ch 3x3 s1 p1 on 32x{Cin}x128x128, forward + weight gradient",
                "forward_us": round(ms_f * 1e3, 1), "wgrad_us": round(ms_w * 1e3, 1), "kernels": [kf, kw],
+               "dgrad_us": round(ms_d * 1e3, 1), "dgrad_kernel": kd,
                "gflop": round(2 * fl / 1e9, 2)}
         if Cin * 9 >= 64:
             tf = 2 * fl / (ms_f + ms_w) / 1e9

@@ -155,6 +155,16 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                                                int kernel_h, int kernel_w, int pad_h, int pad_w,
                                                int stride_h, int stride_w);
+/* conv2_backward's data branch (l-ten/backprop.cpp:1955-1968 CPU, :2007-2028 CUDA: per image col = W^T dy_n, then
+ * col2im) for the whole batch: dx[N,Cin,H,W] is overwritten.  With stride 1 it runs as a convolution of dy with
+ * the flipped, channel-transposed weights on the forward kernels (no column buffer); other strides follow l-ten's
+ * GEMM + col2im per image.  workspace: lten_hip_conv2d_dgrad_workspace_bytes(...) device bytes. */
+int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                              int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                              const float* w, const float* dy, float* dx, void* workspace);
+uint64_t lten_hip_conv2d_dgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
+                                               int kernel_h, int kernel_w, int pad_h, int pad_w,
+                                               int stride_h, int stride_w);
 
 /* Conv2d_q::forward (l-ten/conv2d.cpp:265-387; CPU-only in l-ten, "Conv2d_q only supports the CPU device
  * type" :376) for the whole batch: x[N][Cin][H][W] u8, w[Cout][Cin*kh*kw] u8, y[N][Cout][Ho][Wo] u8, with

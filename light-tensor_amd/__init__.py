@@ -59,6 +59,8 @@ _SIGNATURES = {
     "lten_hip_conv2d_forward_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),
     "lten_hip_conv2d_wgrad_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),
     "lten_hip_conv2d_wgrad_workspace_bytes": (u64, [u64] * 5 + [C.c_int] * 6),
+    "lten_hip_conv2d_dgrad_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),
+    "lten_hip_conv2d_dgrad_workspace_bytes": (u64, [u64] * 5 + [C.c_int] * 6),
     "lten_hip_conv2dq_workspace_bytes": (u64, [u64] * 5 + [C.c_int] * 6),
     "lten_hip_conv2dq_forward": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, C.POINTER(QParams), vp, vp]),
     "lten_hip_conv2dq_forward_acc": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, C.POINTER(QParams), vp, vp]),

@@ -176,6 +176,41 @@ static void wgrad_split(const ConvGeo& g, int& slices, int& slice_len)
 	slices = (int)ceil_div((uint64_t)HW, (uint64_t)slice_len);
 }
 
+// Picks the forward kernel for a geometry (x, w, y non-null, non-empty problem).
+static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
+{
+	const uint64_t Cout = g.Cout, N = g.N;
+	const int HW = g.Ho * g.Wo;
+	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
+	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
+	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
+	if (Cout > 32) {
+		set_kernel_name("conv2d_forward_64x64x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
+		conv2d_forward_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	} else {
+		set_kernel_name("conv2d_forward_32x128x32");
+		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(HW, 128)), 1, (unsigned)N);
+		conv2d_forward_kernel<32, 128, 32, 1, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+// dw2[ci][co][i][j] = w[co][ci][kh-1-i][kw-1-j]: the weights of the stride-1 convolution that maps dy to dx.
+__global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restrict__ w, float* __restrict__ w2, int Cout, int Cin, int kh, int kw)
+{
+	const int total = Cout * Cin * kh * kw;
+	for (int idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+		const int j = idx % kw, i = (idx / kw) % kh, co = (idx / (kw * kh)) % Cout, ci = idx / (kw * kh * Cout);
+		w2[idx] = w[((co * Cin + ci) * kh + (kh - 1 - i)) * kw + (kw - 1 - j)];
+	}
+}
+
+// The data gradient of a stride-1 convolution is a stride-1 convolution of dy with the flipped, channel-transposed
+// weights and pads k - 1 - p; it then runs on the forward kernels.
+static bool dgrad_as_forward(const ConvGeo& g) { return g.sh == 1 && g.sw == 1 && g.ph <= g.kh - 1 && g.pw <= g.kw - 1; }
+
 }  // namespace lten_hip
 
 using namespace lten_hip;
@@ -228,20 +263,43 @@ int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W
 	if (int rc = make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return rc;
 	if (N == 0 || Cout == 0 || g.Ho * g.Wo == 0) return 0;
 	LTEN_HIP_REQUIRE(x && w && y, "conv2d_forward: null pointer");
-	const int HW = g.Ho * g.Wo;
-	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
-	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
-	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
-	if (Cout > 32) {
-		set_kernel_name("conv2d_forward_64x64x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
-		conv2d_forward_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
-	} else {
-		set_kernel_name("conv2d_forward_32x128x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(HW, 128)), 1, (unsigned)N);
-		conv2d_forward_kernel<32, 128, 32, 1, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	return conv_forward_dispatch(g, x, w, bias, y);
+}
+
+uint64_t lten_hip_conv2d_dgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh,
+                                               int kw, int ph, int pw, int sh, int sw)
+{
+	ConvGeo g;
+	if (make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return 0;
+	const uint64_t Kc = Cin * kh * kw;
+	return sizeof(float) * std::max<uint64_t>(Cout * Kc, Kc * (uint64_t)g.Ho * g.Wo) + 16;
+}
+
+int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
+                              int pw, int sh, int sw, const float* w, const float* dy, float* dx, void* workspace)
+{
+	ConvGeo g;
+	if (int rc = make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return rc;
+	const uint64_t HW = (uint64_t)g.Ho * g.Wo, Kc = Cin * kh * kw;
+	if (N == 0 || Cin * H * W == 0) return 0;
+	LTEN_HIP_REQUIRE(dx != nullptr, "conv2d_dgrad: dx is null");
+	if (Cout == 0 || HW == 0) return lten_hip_zero(dx, N * Cin * H * W * sizeof(float));
+	LTEN_HIP_REQUIRE(w && dy && workspace, "conv2d_dgrad: null pointer");
+	float* work = static_cast<float*>(workspace);
+	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1) {
+		flip_weights_kernel<<<dim3((unsigned)std::min<uint64_t>(ceil_div(Cout * Kc, 256), 1024)), dim3(256), 0, stream()>>>(w, work, (int)Cout, (int)Cin, kh, kw);
+		LTEN_HIP_LAUNCH_CHECK();
+		ConvGeo g2;
+		if (int rc = make_geo(g2, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
+		LTEN_HIP_REQUIRE(g2.Ho == (int)H && g2.Wo == (int)W, "conv2d_dgrad: internal geometry mismatch");
+		return conv_forward_dispatch(g2, dy, work, nullptr, dx);
 	}
-	LTEN_HIP_LAUNCH_CHECK();
+	// l-ten/backprop.cpp:2022-2028 per image: col = W^T dy_n (TN GEMM), then col2im
+	for (uint64_t n = 0; n < N; n++) {
+		if (int rc = lten_hip_sgemm(1, 0, Kc, HW, Cout, 1.0f, w, Kc, dy + n * Cout * HW, HW, 0.0f, work, HW)) return rc;
+		if (int rc = lten_hip_col2im_f32(work, (int)Cin, (int)H, (int)W, kh, kw, ph, pw, sh, sw, 1, 1, dx + n * Cin * H * W)) return rc;
+	}
+	set_kernel_name("conv2d_dgrad_sgemm_col2im");
 	return 0;
 }
 

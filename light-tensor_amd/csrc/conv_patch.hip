@@ -18,17 +18,17 @@
 namespace lten_hip {
 
 // ---------------------------------------------------------------------------------------------------------
-// Forward.  Workgroup tile: 64 output channels x (TH = 4 rows x TW = 128 columns) of one image; wavefront
-// `wave` owns row `wave` (2 x 4 MFMA tiles of 32 x 32).  The input channels are walked in chunks of CB = 4:
+// Forward.  Workgroup tile: BM = 64 (or 32) output channels x (TH = 4 rows x TW = 128 columns) of one image;
+// wavefront `wave` owns row `wave` (BM / 32 x 4 MFMA tiles of 32 x 32).  The input channels are walked in chunks of CB = 4:
 // per chunk the patch [4][TH + KH - 1][PWS] and the weights of those channels are stored to LDS, the next
 // chunk's values are fetched to registers, and (CB / 2) * KH * KW MFMA steps run; step (cp, i, j) multiplies
 // tap (i, j) of channels 2cp (lanes 0-31) and 2cp + 1 (lanes 32-63).
 //
 // LDS patch row: index q holds input column w0 - 4 + q (interior 16-byte aligned, left halo in 4 - pw .. 3).
-// LDS weights: [step][channel parity][WROW = 65] (the odd row length spreads the scattered stores over banks).
-template <int KH, int KW>
+// LDS weights: [step][channel parity][WROW = BM + 1] (the odd row length spreads the scattered stores over banks).
+template <int KH, int KW, int BM_>
 struct PatchFwd {
-	static constexpr int CB = 4, TH = 4, TW = 128, NT = TW / 32, BM = 64, T = 256;
+	static constexpr int CB = 4, TH = 4, TW = 128, NT = TW / 32, BM = BM_, MT = BM / 32, T = 256;
 	static constexpr int PR = TH + KH - 1;
 	static constexpr int PWS = (4 + TW + KW - 1 + 3) / 4 * 4;
 	static constexpr int F4_ROW = PWS / 4;
@@ -43,11 +43,11 @@ struct PatchFwd {
 	static constexpr int W_PER_T = (WCOUNT + T - 1) / T;
 };
 
-template <int KH, int KW, bool VEC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv2d_patch_forward_kernel(
+template <int KH, int KW, int BM, bool VEC>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 2 : 3, BM == 64 ? 2 : 3))) void conv2d_patch_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
 {
-	typedef PatchFwd<KH, KW> P;
+	typedef PatchFwd<KH, KW, BM> P;
 	__shared__ __attribute__((aligned(16))) float s_patch[P::PATCH];
 	__shared__ float s_w[P::WTS];
 
@@ -95,9 +95,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		}
 	};
 
-	v16f acc[2][P::NT];
+	v16f acc[P::MT][P::NT];
 #pragma unroll
-	for (int m = 0; m < 2; m++)
+	for (int m = 0; m < P::MT; m++)
 #pragma unroll
 		for (int t = 0; t < P::NT; t++)
 #pragma unroll
@@ -112,12 +112,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		__syncthreads();
 		if (c0 + P::CB < g.Cin) load_chunk(c0 + P::CB);
 		// operands of step s + 1 are read while the MFMAs of step s issue, one LDS read behind each MFMA
-		constexpr int NR = 2 + P::NT, NM = 2 * P::NT;  // LDS reads and MFMAs per step
-		float fa[2][2], fb[2][P::NT];
+		constexpr int NR = P::MT + P::NT, NM = P::MT * P::NT;  // LDS reads and MFMAs per step
+		float fa[2][P::MT], fb[2][P::NT];
 		auto read_operand = [&](int s, int e) {
 			const int cp = s / P::TAPS, tap = s % P::TAPS, i = tap / KW, j = tap % KW;
-			if (e < 2) fa[s & 1][e] = pa[s * 2 * P::WROW + e * 32];
-			else fb[s & 1][e - 2] = pb[(2 * cp * P::PR + i) * P::PWS + j + (e - 2) * 32];
+			if (e < P::MT) fa[s & 1][e] = pa[s * 2 * P::WROW + e * 32];
+			else fb[s & 1][e - P::MT] = pb[(2 * cp * P::PR + i) * P::PWS + j + (e - P::MT) * 32];
 		};
 #pragma unroll
 		for (int e = 0; e < NR; e++) read_operand(0, e);
@@ -128,7 +128,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 				acc[e / P::NT][e % P::NT] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1][e / P::NT], fb[s & 1][e % P::NT], acc[e / P::NT][e % P::NT], 0, 0, 0);
 				if (s + 1 < P::KSTEPS) {
 					if (e < NR) read_operand(s + 1, e);
-					if (e == NM - 1 && NR > NM) read_operand(s + 1, NR - 1);
+					if (e == NM - 1)
+						for (int x = NM; x < NR; x++) read_operand(s + 1, x);
 				}
 				__builtin_amdgcn_sched_barrier(0);
 			}
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	const int ho = h0 + wave;
 	if (ho >= g.Ho) return;
 #pragma unroll
-	for (int m = 0; m < 2; m++)
+	for (int m = 0; m < P::MT; m++)
 #pragma unroll
 		for (int r = 0; r < 16; r++) {
 			const int co = co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
@@ -339,14 +340,26 @@ bool conv_patch_forward_takes(const ConvGeo& g, const float*, const float*)
 	return patch_geometry(g) && g.Cin >= 5 && ceil_div((uint64_t)g.Cout, 64) < 65536;
 }
 
+template <int BM>
+static void launch_patch_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y, bool vec)
+{
+	typedef PatchFwd<3, 3, BM> P;
+	const dim3 grid((unsigned)(ceil_div((uint64_t)g.Wo, P::TW) * ceil_div((uint64_t)g.Ho, P::TH)), (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)g.N);
+	if (vec) conv2d_patch_forward_kernel<3, 3, BM, true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	else conv2d_patch_forward_kernel<3, 3, BM, false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+}
+
 int conv_patch_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
-	typedef PatchFwd<3, 3> P;
 	const bool vec = g.W % 4 == 0 && aligned16(x);
-	const dim3 grid((unsigned)(ceil_div((uint64_t)g.Wo, P::TW) * ceil_div((uint64_t)g.Ho, P::TH)), (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)g.N);
-	set_kernel_name("conv2d_patch_forward_3x3_64x4x128");
-	if (vec) conv2d_patch_forward_kernel<3, 3, true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
-	else conv2d_patch_forward_kernel<3, 3, false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	// 64 output channels per workgroup, or 32 when that leaves fewer padded rows
+	if (ceil_div((uint64_t)g.Cout, 32) % 2 == 1) {
+		set_kernel_name("conv2d_patch_forward_3x3_32x4x128");
+		launch_patch_forward<32>(g, x, w, bias, y, vec);
+	} else {
+		set_kernel_name("conv2d_patch_forward_3x3_64x4x128");
+		launch_patch_forward<64>(g, x, w, bias, y, vec);
+	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

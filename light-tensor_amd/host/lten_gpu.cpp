@@ -633,11 +633,6 @@ std::vector<Tensor*> Conv2d::get_all_weights()
 	return w;
 }
 
-// dst += src over n floats, as the K = 1 GEMM dst[1 x n] = one[1 x 1] * src[1 x n] + dst
-static void accumulate(float* dst, const float* src, uint64_t n, const float* device_one)
-{
-	LTEN_HIP_CALL(lten_hip_sgemm(0, 0, 1, n, 1, 1.0f, device_one, 1, src, n, 1.0f, dst, n));
-}
 
 Tensor Conv2d::forward(Tensor& input)
 {
@@ -663,23 +658,20 @@ Tensor Conv2d::forward(Tensor& input)
 	                                          use_bias_ ? static_cast<const float*>(bias_.get_data_ptr()) : nullptr,
 	                                          static_cast<float*>(result.get_data_ptr())));
 
-	// scratch: [one float = 1.0][weight-gradient partials or one column buffer, whichever is larger][temp dW]
-	const uint64_t Kc = Cin * kernel_h_ * kernel_w_, HW = Ho * Wo;
-	const uint64_t ws_bytes = lten_hip_conv2d_wgrad_workspace_bytes(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw);
-	const uint64_t work_floats = std::max<uint64_t>((ws_bytes + 3) / 4, Kc * HW);
-	const uint64_t need = 64 + work_floats + Cout * Kc + Cin * H * W;
-	if (!scratch_.defined() || scratch_.get_numels() < need) {
-		scratch_ = AllocateTensor({ need }, &options);
-		LTEN_HIP_CALL(lten_hip_fill_f32(static_cast<float*>(scratch_.get_data_ptr()), 1, 1.0f));
-	}
+	// scratch: [workspace of the weight / data gradient calls, whichever is larger][temp dW][temp dX for a whole batch]
+	const uint64_t Kc = Cin * kernel_h_ * kernel_w_;
+	const uint64_t ws_bytes = std::max(lten_hip_conv2d_wgrad_workspace_bytes(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw),
+	                                   lten_hip_conv2d_dgrad_workspace_bytes(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw));
+	const uint64_t work_floats = (ws_bytes + 3) / 4 + 64;
+	const uint64_t need = work_floats + Cout * Kc + N * Cin * H * W;
+	if (!scratch_.defined() || scratch_.get_numels() < need) scratch_ = AllocateTensor({ need }, &options);
 	auto wt = weight_.get_smart_ptr(), in = input.get_smart_ptr(), scratch = scratch_.get_smart_ptr();
 	const bool with_bias = use_bias_;
 	result.get_smart_ptr()->children = { wt, in };  // l-ten/conv2d.cpp:183-187
 	result.get_smart_ptr()->autograd = true;
 	result.get_smart_ptr()->grad_fn = [=](TensorImpl&, const float* top) {
 		if (with_bias) LTEN_ERR("the gradient of the Conv2d bias is not part of the GPU path (l-ten adds the bias as a separate tensor op)");
-		float* one = static_cast<float*>(scratch->data);
-		float* work = one + 64;
+		float* work = static_cast<float*>(scratch->data);
 		float* tmp_dw = work + work_floats;
 		float* tmp_dx = tmp_dw + Cout * Kc;
 		const float* x = static_cast<const float*>(in->data);
@@ -688,16 +680,13 @@ Tensor Conv2d::forward(Tensor& input)
 			// l-ten/backprop.cpp:1949-1953 (CPU semantics: the sum over all images), then the leaf accumulate of :246-274
 			Bottom g(wt);
 			LTEN_HIP_CALL(lten_hip_conv2d_wgrad_f32(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, x, top, tmp_dw, work));
-			accumulate(g.ptr, tmp_dw, Cout * Kc, one);
+			LTEN_HIP_CALL(lten_hip_axpy_f32(Cout * Kc, 1.0f, tmp_dw, g.ptr));
 		}
 		if (wants_gradient(in)) {
-			// l-ten/backprop.cpp:2022-2028: per image col = W^T dY_n (TN GEMM) then col2im
+			// l-ten/backprop.cpp:2022-2028 (per image col = W^T dY_n, then col2im) for the whole batch, then the accumulate
 			Bottom g(in);
-			for (uint64_t n = 0; n < N; n++) {
-				LTEN_HIP_CALL(lten_hip_sgemm(1, 0, Kc, HW, Cout, 1.0f, w, Kc, top + n * Cout * HW, HW, 0.0f, work, HW));
-				LTEN_HIP_CALL(lten_hip_col2im_f32(work, (int)Cin, (int)H, (int)W, kh, kw, ph, pw, sh, sw, 1, 1, tmp_dx));
-				accumulate(g.ptr + n * Cin * H * W, tmp_dx, Cin * H * W, one);
-			}
+			LTEN_HIP_CALL(lten_hip_conv2d_dgrad_f32(N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, w, top, tmp_dx, work));
+			LTEN_HIP_CALL(lten_hip_axpy_f32(N * Cin * H * W, 1.0f, tmp_dx, g.ptr));
 			g.propagate();
 		}
 	};

@@ -60,6 +60,15 @@ def gpu_conv(gpu, geo, x, w, dy=None, bias=None):
     return y, dw, fk
 
 
+def gpu_dgrad(gpu, geo, w, dy):
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    dW, dDY, dDX = D.from_numpy(w), D.from_numpy(dy), D(4 * N * Cin * H * W)
+    ws = D(max(int(l.lten_hip_conv2d_dgrad_workspace_bytes(*geo)), 4))
+    gpu.check(l.lten_hip_conv2d_dgrad_f32(*geo, dW.ptr, dDY.ptr, dDX.ptr, ws.ptr))
+    return dDX.numpy(np.float32, (N, Cin, H, W))
+
+
 def test_conv_layer_golden(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     for i in range(int(g["conv_count"])):
@@ -68,6 +77,7 @@ def test_conv_layer_golden(gpu):
         y, dw, _ = gpu_conv(gpu, geo, g[pre + "x"], g[pre + "w"], g[pre + "dy"])
         assert rel_err(y.reshape(-1), g[pre + "y"]) < TOL, i
         assert rel_err(dw.reshape(-1), g[pre + "dw"]) < TOL, i
+        assert rel_err(gpu_dgrad(gpu, geo, g[pre + "w"], g[pre + "dy"]).reshape(-1), g[pre + "dx"]) < TOL, i
 
 
 @pytest.mark.parametrize("geo", [(2, 3, 9, 8, 4, 3, 3, 1, 1, 1, 1), (1, 2, 10, 7, 3, 3, 2, 0, 1, 2, 1),
@@ -76,7 +86,7 @@ def test_conv_layer_golden(gpu):
                                  # 3x3 stride 1 (LDS patch kernels): several column tiles and channel blocks, rows
                                  # that are / are not a multiple of four floats, pad 0 / 1 / 2, ragged channel counts
                                  (2, 20, 17, 136, 70, 3, 3, 1, 1, 1, 1), (1, 37, 12, 64, 33, 3, 3, 0, 0, 1, 1),
-                                 (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1),
+                                 (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1), (2, 12, 10, 36, 96, 3, 3, 1, 1, 1, 1),
                                  # stride 1 with Cin*kh*kw <= 32 (first-layer kernels): ragged widths, two column
                                  # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
@@ -109,6 +119,11 @@ def _conv_vs_oracle(gpu, ob, geo):
     print(f"  {geo}: forward via {fk}, wgrad via {gpu.last_kernel()}", flush=True)
     assert rel_err(y, want_y + bias[None, :, None, None]) < TOL, fk
     assert rel_err(dw, want_dw) < TOL, gpu.last_kernel()
+    want_dx = np.empty_like(x)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    print(f"  {geo}: dgrad via {gpu.last_kernel()}", flush=True)
+    assert rel_err(dx, want_dx) < TOL, gpu.last_kernel()
     assert rel_err(y, direct_conv(x, w, ph, pw, sh, sw) + bias[None, :, None, None]) < TOL
 
 
@@ -141,4 +156,14 @@ def test_cfg5_full_size(gpu, wl):
         assert rel_err(dw, want_dw) < TOL
         print(f"  layer {layer + 1}: forward via {fk}, wgrad via {gpu.last_kernel()}, "
               f"dw max rel err {rel_err(dw, want_dw):.2e}")
+        # data gradient on sampled input positions: dx[n,ci,y,x] = sum_{c,i,j} dy[n,c,y+1-i,x+1-j] * w[c,ci,i,j]
+        dx = gpu_dgrad(gpu, geo, w, dy)
+        dyp = np.pad(dy64, ((0, 0), (0, 0), (1, 1), (1, 1)))
+        wf = w.astype(np.float64)[:, :, ::-1, ::-1]
+        pts = [(int(rng.integers(0, N)), int(rng.integers(0, Cin)), int(rng.integers(0, H)), int(rng.integers(0, W)))
+               for _ in range(200)] + [(0, 0, 0, 0), (N - 1, Cin - 1, H - 1, W - 1)]
+        want_dx = np.array([(dyp[n, :, yy:yy + 3, xx:xx + 3] * wf[:, ci]).sum() for (n, ci, yy, xx) in pts])
+        got_dx = np.array([dx[p] for p in pts])
+        sc = float(np.sqrt((dx.astype(np.float64) ** 2).mean()))
+        assert (np.abs(got_dx - want_dx) / np.maximum(np.abs(want_dx), sc)).max() < TOL, gpu.last_kernel()
         inp = y
