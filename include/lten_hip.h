@@ -204,6 +204,16 @@ int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float*
 /* gpu_nll (l-ten/math_fns.h:170; l-ten/layers.cpp:212-273): *loss = (sum_i input[i] * target[i]) * (-1 / batches). */
 int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, uint64_t len, uint64_t batches);
 
+/* ------------------------------------------------------------------ quantization helpers */
+
+/* Quantize / Dequantize / GetMinMax of l-ten/utils.h:23-26 (l-ten/utils.cpp:198-262) with the data on the device;
+ * bit-exact with the CPU functions.  qparams is a host pointer.  lten_hip_get_min_max returns its two results to
+ * host memory and synchronises; ComputeQuantizationParams (two floats in, one QuantizationParams out) stays host code. */
+int lten_hip_quantize_u8(const float* data, uint8_t* q_data, uint64_t len, const lten_hip_qparams* qparams);
+int lten_hip_quantize_i32(const float* data, int32_t* q_data, uint64_t len, const lten_hip_qparams* qparams);
+int lten_hip_dequantize_u8(float* data, const uint8_t* q_data, uint64_t len, const lten_hip_qparams* qparams);
+int lten_hip_get_min_max(const float* data, uint64_t len, float* min_val, float* max_val);
+
 /* ----------------------------------------------------------------------- measurement */
 
 /* HIP events on the library's stream; no counterpart in l-ten (its benchmarks use

@@ -71,6 +71,10 @@ _SIGNATURES = {
     "lten_hip_log_softmax_f32": (C.c_int, [u64, u64, vp, vp]),
     "lten_hip_log_softmax_backward_f32": (C.c_int, [u64, u64, vp, vp, vp]),
     "lten_hip_nll_loss_f32": (C.c_int, [vp, vp, vp, u64, u64]),
+    "lten_hip_quantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
+    "lten_hip_quantize_i32": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
+    "lten_hip_dequantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
+    "lten_hip_get_min_max": (C.c_int, [vp, u64, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "lten_hip_event_create": (C.c_int, [C.POINTER(vp)]),
     "lten_hip_event_record": (C.c_int, [vp]),
     "lten_hip_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),

@@ -209,7 +209,10 @@ __global__ __launch_bounds__(256) void flip_weights_kernel(const float* __restri
 
 // The data gradient of a stride-1 convolution is a stride-1 convolution of dy with the flipped, channel-transposed
 // weights and pads k - 1 - p; it then runs on the forward kernels.
-static bool dgrad_as_forward(const ConvGeo& g) { return g.sh == 1 && g.sw == 1 && g.ph <= g.kh - 1 && g.pw <= g.kw - 1; }
+static bool dgrad_as_forward(const ConvGeo& g)
+{
+	return g.sh == 1 && g.sw == 1 && g.ph <= g.kh - 1 && g.pw <= g.kw - 1 && (uint64_t)g.Cout * g.Cin * g.kh * g.kw < (1ull << 31);
+}
 
 }  // namespace lten_hip
 

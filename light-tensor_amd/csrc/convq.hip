@@ -113,7 +113,7 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 	volatile float ab = qp[1].scale * qp[0].scale;
 	const float mult = ab / qp[2].scale, zp_out = (float)qp[2].zero_point;
 
-	if (K <= CQ_MAXK && get_option(OPT_CONV_VARIANT) != 1) {
+	if (K <= CQ_MAXK && ceil_div((uint64_t)N * HW, 256) < (1ull << 31) && get_option(OPT_CONV_VARIANT) != 1) {
 		const dim3 grid((unsigned)ceil_div((uint64_t)N * HW, 256), (unsigned)ceil_div(Cout, CQ_CO));
 		set_kernel_name("conv2dq_direct");
 		if (out_acc) conv2dq_direct_kernel<Q_OUT_ACC><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);

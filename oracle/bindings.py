@@ -110,6 +110,16 @@ def oracle():
     lib.oracle_nll_backward.argtypes = [f32p, u64, u64, C.c_float, f32p]
     lib.oracle_mlp_step.restype = C.c_int
     lib.oracle_mlp_step.argtypes = _MLP_ARGS
+    lib.oracle_min_max.restype = None
+    lib.oracle_min_max.argtypes = [f32p, u64, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    lib.oracle_compute_qparams.restype = None
+    lib.oracle_compute_qparams.argtypes = [C.c_float, C.c_float, C.POINTER(QParams)]
+    lib.oracle_quantize_u8.restype = None
+    lib.oracle_quantize_u8.argtypes = [f32p, u8p, u64, C.POINTER(QParams)]
+    lib.oracle_quantize_i32.restype = None
+    lib.oracle_quantize_i32.argtypes = [f32p, i32p, u64, C.POINTER(QParams)]
+    lib.oracle_dequantize_u8.restype = None
+    lib.oracle_dequantize_u8.argtypes = [f32p, u8p, u64, C.POINTER(QParams)]
     lib.oracle_conv2dq_forward.restype = C.c_int
     lib.oracle_conv2dq_forward.argtypes = conv + [u8p, u8p, C.POINTER(C.c_int32), C.POINTER(QParams), u8p, C.POINTER(C.c_int32)]
     _oracle = lib
@@ -144,6 +154,16 @@ def ref():
     lib.ref_fcq_u8.argtypes = [u64, u64, u64, u64, u8p, u8p, C.POINTER(C.c_int32), f32p, u8p, u8p]
     lib.ref_conv2d_f32.restype = C.c_int
     lib.ref_conv2d_f32.argtypes = [u64] * 5 + [C.c_int] * 6 + [f32p, f32p, fp, fp, fp, fp]
+    lib.ref_min_max.restype = None
+    lib.ref_min_max.argtypes = [f32p, u64, C.POINTER(C.c_float), C.POINTER(C.c_float)]
+    lib.ref_compute_qparams.restype = None
+    lib.ref_compute_qparams.argtypes = [C.c_float, C.c_float, C.POINTER(C.c_float), C.POINTER(C.c_uint8)]
+    lib.ref_quantize_u8.restype = None
+    lib.ref_quantize_u8.argtypes = [f32p, u8p, u64, C.c_float, C.c_uint8]
+    lib.ref_quantize_i32.restype = None
+    lib.ref_quantize_i32.argtypes = [f32p, i32p, u64, C.c_float, C.c_uint8]
+    lib.ref_dequantize_u8.restype = None
+    lib.ref_dequantize_u8.argtypes = [f32p, u8p, u64, C.c_float, C.c_uint8]
     lib.ref_mlp_step.restype = C.c_int
     lib.ref_mlp_step.argtypes = _MLP_ARGS
     lib.ref_conv2dq_u8.restype = C.c_int

@@ -573,3 +573,60 @@ int oracle_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const flo
 	free(g2);
 	return rc;
 }
+
+/* --------------------------------------------------------------------- quantization helpers */
+
+void oracle_min_max(const float* data, uint64_t len, float* min_val, float* max_val)
+{
+	uint64_t i; /* l-ten/utils.cpp:198-225 */
+	float lo = data[0], hi = data[0];
+	for (i = 0; i < len; i++) {
+		if (data[i] > hi) hi = data[i];
+		if (data[i] < lo) lo = data[i];
+	}
+	*min_val = lo;
+	*max_val = hi;
+}
+
+void oracle_compute_qparams(float min_val, float max_val, oracle_qparams* qp)
+{
+	/* l-ten/utils.cpp:265-286 */
+	float zero_point;
+	min_val = (0.f < min_val) ? 0.f : min_val; /* std::min(min_val, 0.f) */
+	max_val = (max_val < 0.f) ? 0.f : max_val; /* std::max(max_val, 0.f) */
+	qp->scale = (max_val - min_val) / (255.f - 0.f);
+	zero_point = 0.f - min_val / qp->scale;
+	qp->zero_point = (uint8_t)roundf(zero_point);
+}
+
+void oracle_quantize_u8(const float* data, uint8_t* q, uint64_t len, const oracle_qparams* qp)
+{
+	uint64_t i; /* l-ten/utils.cpp:241-252 */
+	for (i = 0; i < len; i++) {
+		float val = (float)qp->zero_point + data[i] / qp->scale;
+		val = (val < 255.f) ? val : 255.f; /* std::min(255.f, val) */
+		val = (0.f < val) ? val : 0.f;     /* std::max(0.f, val)   */
+		q[i] = (uint8_t)roundf(val);
+	}
+}
+
+void oracle_quantize_i32(const float* data, int32_t* q, uint64_t len, const oracle_qparams* qp)
+{
+	/* l-ten/utils.cpp:227-239: clamp to [(float)INT_MIN, (float)INT_MAX] (the upper bound rounds up to 2^31), round
+	 * half away from zero, convert: what does not fit an int comes out of x86's conversion as 0x80000000 */
+	uint64_t i;
+	const float lowest = -2147483648.0f, highest = 2147483648.0f;
+	for (i = 0; i < len; i++) {
+		float val = (float)qp->zero_point + data[i] / qp->scale, r;
+		val = (val < highest) ? val : highest;
+		val = (lowest < val) ? val : lowest;
+		r = roundf(val);
+		q[i] = (r >= -2147483648.0f && r < 2147483648.0f) ? (int32_t)r : (int32_t)0x80000000u;
+	}
+}
+
+void oracle_dequantize_u8(float* data, const uint8_t* q, uint64_t len, const oracle_qparams* qp)
+{
+	uint64_t i; /* l-ten/utils.cpp:254-262 */
+	for (i = 0; i < len; i++) data[i] = qp->scale * (float)((int)q[i] - (int)qp->zero_point);
+}

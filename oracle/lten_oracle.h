@@ -140,6 +140,15 @@ int oracle_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const flo
                     const float* const* b, const float* target, float* loss, float* logp, float** dW, float** db,
                     float* dX);
 
+/* l-ten/utils.cpp:198-286: GetMinMax, ComputeQuantizationParams, Quantize (uint8 and int), Dequantize.
+ * Pinned: the compiled l-ten functions on inputs with ties, out-of-range values, infinities and NaN (golden
+ * cases, bit-exact), closed forms (round half away from zero, clamp to [0, 255]). */
+void oracle_min_max(const float* data, uint64_t len, float* min_val, float* max_val);
+void oracle_compute_qparams(float min_val, float max_val, oracle_qparams* qp);
+void oracle_quantize_u8(const float* data, uint8_t* q, uint64_t len, const oracle_qparams* qp);
+void oracle_quantize_i32(const float* data, int32_t* q, uint64_t len, const oracle_qparams* qp);
+void oracle_dequantize_u8(float* data, const uint8_t* q, uint64_t len, const oracle_qparams* qp);
+
 #ifdef __cplusplus
 }
 #endif

@@ -96,6 +96,34 @@ int ref_fc_f32(uint64_t M, uint64_t in, uint64_t out, const float* x, const floa
 	return 0;
 }
 
+// l-ten/utils.cpp:198-286 quantization helpers, as compiled.
+void ref_min_max(const float* data, uint64_t len, float* lo, float* hi) { GetMinMax(const_cast<float*>(data), len, lo, hi); }
+void ref_compute_qparams(float lo, float hi, float* scale, uint8_t* zero_point)
+{
+	QuantizationParams qp;
+	ComputeQuantizationParams(lo, hi, &qp);
+	*scale = qp.scale;
+	*zero_point = qp.zero_point;
+}
+void ref_quantize_u8(const float* data, uint8_t* q, uint64_t len, float scale, uint8_t zero_point)
+{
+	QuantizationParams qp;
+	qp.scale = scale; qp.zero_point = zero_point;
+	Quantize(const_cast<float*>(data), q, len, &qp);
+}
+void ref_quantize_i32(const float* data, int* q, uint64_t len, float scale, uint8_t zero_point)
+{
+	QuantizationParams qp;
+	qp.scale = scale; qp.zero_point = zero_point;
+	Quantize(const_cast<float*>(data), q, len, &qp);
+}
+void ref_dequantize_u8(float* data, const uint8_t* q, uint64_t len, float scale, uint8_t zero_point)
+{
+	QuantizationParams qp;
+	qp.scale = scale; qp.zero_point = zero_point;
+	Dequantize(data, const_cast<uint8_t*>(q), len, &qp);
+}
+
 // One training step of l-ten's MLP (tests/nn_tests.cpp): FullyConnected(+bias) -> relu -> ... -> FullyConnected ->
 // log_softmax(dim 3) -> nll_loss -> backward().  x: {batch,1,1,sizes[0]}, target one-hot {batch,1,1,sizes[layers]}.
 int ref_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const float* x, const float* const* w,

@@ -256,6 +256,47 @@ def mlp_step_case():
     print("mlp_step_case loss", r["loss"])
 
 
+def quant_inputs():
+    """Values that exercise the helpers' corners: ties at .5 after the scale, both clamps, zeros of both signs,
+    infinities, NaN, magnitudes beyond int range."""
+    rng = np.random.default_rng(55)
+    special = np.array([0.0, -0.0, 0.5, -0.5, 1.5, 2.5, -1.5, 127.5, 128.5, 254.5, 255.5, 1e-30, -1e-30, 1e9, -1e9, 3e9, -3e9,
+                        2147483520.0, 2147483648.0, -2147483648.0, np.inf, -np.inf, np.nan, 1e38, -1e38], np.float32)
+    return np.concatenate([special, (rng.standard_normal(3000) * 3).astype(np.float32),
+                           (rng.integers(-600, 600, 500) * 0.25).astype(np.float32),
+                           (rng.standard_normal(200) * 1e10).astype(np.float32)])
+
+
+def quant_cases():
+    """Quantize (uint8 and int), Dequantize, GetMinMax and ComputeQuantizationParams of the compiled l-ten."""
+    data = quant_inputs()
+    out = {"data": data}
+    qps = [(0.5, 0), (0.25, 128), (1.0, 255), (0.0123, 17), (3.7, 200), (1e-3, 1)]
+    out["qps"] = np.array(qps, np.float64)
+    r = ob.ref()
+    for i, (sc, zp) in enumerate(qps):
+        q8, q32 = np.empty(data.size, np.uint8), np.empty(data.size, np.int32)
+        r.ref_quantize_u8(data, q8, data.size, sc, zp)
+        r.ref_quantize_i32(data, q32, data.size, sc, zp)
+        codes = np.arange(256, dtype=np.uint8)
+        dq = np.empty(256, np.float32)
+        r.ref_dequantize_u8(dq, codes, 256, sc, zp)
+        out[f"q8_{i}"], out[f"q32_{i}"], out[f"dq_{i}"] = q8, q32, dq
+    ranges = [(-1.0, 1.0), (0.0, 6.0), (-3.5, 0.0), (0.2, 0.9), (-7.25, 12.5), (-1e-3, 2e-3)]
+    res = []
+    for lo, hi in ranges:
+        sc, zp = C.c_float(), C.c_uint8()
+        r.ref_compute_qparams(lo, hi, C.byref(sc), C.byref(zp))
+        res.append((lo, hi, sc.value, zp.value))
+    out["qparam_cases"] = np.array(res, np.float64)
+    finite = data[np.isfinite(data)]
+    lo, hi = C.c_float(), C.c_float()
+    r.ref_min_max(finite, finite.size, C.byref(lo), C.byref(hi))
+    out["minmax"] = np.array([lo.value, hi.value], np.float32)
+    np.savez_compressed(os.path.join(HERE, "quant_cases.npz"), **out)
+    print("quant_cases", data.size)
+
+
 if __name__ == "__main__":
     requant_sweep()
     qmm_cases()
@@ -264,3 +305,4 @@ if __name__ == "__main__":
     layer_cases()
     conv2dq_cases()
     mlp_step_case()
+    quant_cases()
