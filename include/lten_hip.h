@@ -204,6 +204,15 @@ int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float*
 /* gpu_nll (l-ten/math_fns.h:170; l-ten/layers.cpp:212-273): *loss = (sum_i input[i] * target[i]) * (-1 / batches). */
 int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, uint64_t len, uint64_t batches);
 
+/* gpu_sgd_step (l-ten/math_fns.h:186; SGDOptimizer::step, l-ten/optimizer.cpp:26-84) for one parameter tensor:
+ * grad = wd * w + grad (stored, as in l-ten), velocity = velocity * mo + (1 - mo) * grad, w = w - velocity * lr. */
+int lten_hip_sgd_step_f32(float* weight, float* weight_grad, float* velocity, uint64_t numels, float mo, float wd, float lr);
+/* AdamOptimizer::step (l-ten/optimizer.cpp:107-186) for one parameter tensor: l-ten's eight element-wise launches
+ * (gpu_axpby, gpu_mul, gpu_axpby, gpu_mul, gpu_powx, gpu_add, gpu_div, gpu_axpy) as one pass.  v_dw and s_dw are the
+ * first two thirds of l-ten's history tensor; its last third (scratch) is not needed.  iteration counts from 1. */
+int lten_hip_adam_step_f32(float* weight, const float* weight_grad, float* v_dw, float* s_dw, uint64_t numels, float lr,
+                           float beta1, float beta2, uint64_t iteration);
+
 /* ------------------------------------------------------------------ quantization helpers */
 
 /* Quantize / Dequantize / GetMinMax of l-ten/utils.h:23-26 (l-ten/utils.cpp:198-262) with the data on the device;

@@ -71,6 +71,8 @@ _SIGNATURES = {
     "lten_hip_log_softmax_f32": (C.c_int, [u64, u64, vp, vp]),
     "lten_hip_log_softmax_backward_f32": (C.c_int, [u64, u64, vp, vp, vp]),
     "lten_hip_nll_loss_f32": (C.c_int, [vp, vp, vp, u64, u64]),
+    "lten_hip_sgd_step_f32": (C.c_int, [vp, vp, vp, u64, C.c_float, C.c_float, C.c_float]),
+    "lten_hip_adam_step_f32": (C.c_int, [vp, vp, vp, vp, u64, C.c_float, C.c_float, C.c_float, u64]),
     "lten_hip_quantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_quantize_i32": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_dequantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),

@@ -8,6 +8,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cmath>
 
 namespace lten_hip {
 
@@ -97,6 +98,42 @@ __global__ __launch_bounds__(1024) void nll_loss_kernel(const float* __restrict_
 	}
 }
 
+// SGDOptimizer::step for one tensor (l-ten/optimizer.cpp:52-57; gpu_sgd_step, l-ten/math_fns.h:186): the gradient
+// buffer receives the decayed gradient, as in l-ten.  Every product and sum rounded on its own, in l-ten's order.
+__global__ __launch_bounds__(256) void sgd_step_kernel(float* __restrict__ w, float* __restrict__ g, float* __restrict__ v, uint64_t n, float mo,
+                                                       float wd, float lr)
+{
+#pragma clang fp contract(off)
+	const float one_minus_mo = 1.0f - mo;
+	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+		const float gd = wd * w[i] + g[i];
+		const float vel = v[i] * mo + one_minus_mo * gd;
+		g[i] = gd;
+		v[i] = vel;
+		w[i] = w[i] - (vel * lr);
+	}
+}
+
+// AdamOptimizer::step for one tensor (l-ten/optimizer.cpp:139-155): l-ten's eight element-wise launches (axpby, mul,
+// axpby, mul, powx, add, div, axpy) as one pass, same operations in the same order per element.
+__global__ __launch_bounds__(256) void adam_step_kernel(float* __restrict__ w, const float* __restrict__ g, float* __restrict__ v, float* __restrict__ s,
+                                                        uint64_t n, float a1, float beta1, float a2, float beta2, float inv_bc2, float step)
+{
+#pragma clang fp contract(off)
+	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256) {
+		const float gi = g[i];
+		const float vi = a1 * gi + beta1 * v[i];
+		const float si = a2 * (gi * gi) + beta2 * s[i];
+		float t = inv_bc2 * si;
+		t = powf(t, 0.5f);
+		t = 1.0e-8f + t;
+		t = vi / t;
+		v[i] = vi;
+		s[i] = si;
+		w[i] = (step == 1.0f) ? w[i] + t : w[i] + step * t;
+	}
+}
+
 static unsigned grid_for(uint64_t n) { return (unsigned)std::min<uint64_t>(ceil_div(n, 256), 256 * 16); }
 
 }  // namespace lten_hip
@@ -157,6 +194,29 @@ int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float*
 	LTEN_HIP_REQUIRE(y && dy && dx, "log_softmax_backward: null pointer");
 	LTEN_HIP_REQUIRE(ceil_div(rows, 4) < (1ull << 31), "log_softmax_backward: too many rows");
 	log_softmax_backward_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, y, dy, dx);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_sgd_step_f32(float* weight, float* weight_grad, float* velocity, uint64_t numels, float mo, float wd, float lr)
+{
+	if (numels == 0) return 0;
+	LTEN_HIP_REQUIRE(weight && weight_grad && velocity, "sgd_step: null pointer");
+	sgd_step_kernel<<<dim3(grid_for(numels)), dim3(256), 0, stream()>>>(weight, weight_grad, velocity, numels, mo, wd, lr);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_adam_step_f32(float* weight, const float* weight_grad, float* v_dw, float* s_dw, uint64_t numels, float lr,
+                           float beta1, float beta2, uint64_t iteration)
+{
+	if (numels == 0) return 0;
+	LTEN_HIP_REQUIRE(weight && weight_grad && v_dw && s_dw && iteration > 0, "adam_step: null pointer or iteration 0");
+	// l-ten/optimizer.cpp:136-137, :139-155: host scalars exactly as l-ten forms them
+	const float bc1 = 1.0f - powf(beta1, static_cast<float>(iteration));
+	const float bc2 = 1.0f - powf(beta2, static_cast<float>(iteration));
+	adam_step_kernel<<<dim3(grid_for(numels)), dim3(256), 0, stream()>>>(weight, weight_grad, v_dw, s_dw, numels, 1.0f - beta1, beta1, 1.0f - beta2,
+	                                                                     beta2, 1.0f / bc2, -(1.0f / bc1) * lr);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

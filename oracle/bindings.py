@@ -120,6 +120,10 @@ def oracle():
     lib.oracle_quantize_i32.argtypes = [f32p, i32p, u64, C.POINTER(QParams)]
     lib.oracle_dequantize_u8.restype = None
     lib.oracle_dequantize_u8.argtypes = [f32p, u8p, u64, C.POINTER(QParams)]
+    lib.oracle_sgd_step.restype = None
+    lib.oracle_sgd_step.argtypes = [f32p, f32p, f32p, u64, C.c_float, C.c_float, C.c_float]
+    lib.oracle_adam_step.restype = None
+    lib.oracle_adam_step.argtypes = [f32p, f32p, f32p, f32p, u64, C.c_float, C.c_float, C.c_float, u64]
     lib.oracle_conv2dq_forward.restype = C.c_int
     lib.oracle_conv2dq_forward.argtypes = conv + [u8p, u8p, C.POINTER(C.c_int32), C.POINTER(QParams), u8p, C.POINTER(C.c_int32)]
     _oracle = lib
@@ -164,6 +168,8 @@ def ref():
     lib.ref_quantize_i32.argtypes = [f32p, i32p, u64, C.c_float, C.c_uint8]
     lib.ref_dequantize_u8.restype = None
     lib.ref_dequantize_u8.argtypes = [f32p, u8p, u64, C.c_float, C.c_uint8]
+    lib.ref_optimizer_steps.restype = C.c_int
+    lib.ref_optimizer_steps.argtypes = [C.c_int, u64, C.c_int, f32p, f32p, f32p]
     lib.ref_mlp_step.restype = C.c_int
     lib.ref_mlp_step.argtypes = _MLP_ARGS
     lib.ref_conv2dq_u8.restype = C.c_int

@@ -630,3 +630,36 @@ void oracle_dequantize_u8(float* data, const uint8_t* q, uint64_t len, const ora
 	uint64_t i; /* l-ten/utils.cpp:254-262 */
 	for (i = 0; i < len; i++) data[i] = qp->scale * (float)((int)q[i] - (int)qp->zero_point);
 }
+
+/* --------------------------------------------------------------------- optimizer steps */
+
+void oracle_sgd_step(float* w, float* g, float* v, uint64_t n, float mo, float wd, float lr)
+{
+	uint64_t j; /* l-ten/optimizer.cpp:52-57; the gradient buffer is overwritten with the decayed gradient */
+	for (j = 0; j < n; j++) {
+		g[j] = wd * w[j] + g[j];
+		v[j] = v[j] * mo + (1.0f - mo) * g[j];
+		w[j] = w[j] - (v[j] * lr);
+	}
+}
+
+void oracle_adam_step(float* w, const float* g, float* v, float* s, uint64_t n, float lr, float beta1, float beta2,
+                      uint64_t iteration)
+{
+	/* l-ten/optimizer.cpp:139-155, the eight element-wise passes applied per element in the same order */
+	uint64_t j;
+	const float epsilon = 1.0e-8f;
+	const float bc1 = 1.0f - powf(beta1, (float)iteration), bc2 = 1.0f - powf(beta2, (float)iteration);
+	const float a1 = 1.0f - beta1, a2 = 1.0f - beta2, inv2 = 1.0f / bc2, step = -(1.0f / bc1) * lr;
+	for (j = 0; j < n; j++) {
+		float scratch;
+		v[j] = a1 * g[j] + beta1 * v[j];          /* cpu_axpby */
+		scratch = g[j] * g[j];                     /* cpu_mul   */
+		s[j] = a2 * scratch + beta2 * s[j];        /* cpu_axpby */
+		scratch = inv2 * s[j];                     /* cpu_mul   */
+		scratch = powf(scratch, 0.5f);             /* cpu_powx  */
+		scratch = epsilon + scratch;               /* cpu_add   */
+		scratch = v[j] / scratch;                  /* cpu_div   */
+		w[j] = (step == 1.0f) ? w[j] + scratch : w[j] + step * scratch; /* cpu_axpy */
+	}
+}

@@ -149,6 +149,14 @@ void oracle_quantize_u8(const float* data, uint8_t* q, uint64_t len, const oracl
 void oracle_quantize_i32(const float* data, int32_t* q, uint64_t len, const oracle_qparams* qp);
 void oracle_dequantize_u8(float* data, const uint8_t* q, uint64_t len, const oracle_qparams* qp);
 
+/* SGDOptimizer::step and AdamOptimizer::step for one parameter tensor (l-ten/optimizer.cpp:26-84, 107-186).
+ * sgd: g = wd*w + g (stored), v = v*mo + (1-mo)*g, w = w - v*lr.  adam: v, s are the two history buffers,
+ * iteration counts from 1.  Pinned: the compiled optimizers over several steps (golden case; sgd bit-exact,
+ * adam within 1e-6 because of powf), closed forms. */
+void oracle_sgd_step(float* w, float* g, float* v, uint64_t n, float mo, float wd, float lr);
+void oracle_adam_step(float* w, const float* g, float* v, float* s, uint64_t n, float lr, float beta1, float beta2,
+                      uint64_t iteration);
+
 #ifdef __cplusplus
 }
 #endif

@@ -124,6 +124,40 @@ void ref_dequantize_u8(float* data, const uint8_t* q, uint64_t len, float scale,
 	Dequantize(data, const_cast<uint8_t*>(q), len, &qp);
 }
 
+// SGDOptimizer / AdamOptimizer (l-ten/optimizer.cpp) on a one-layer network whose weight tensor holds `n` values:
+// `steps` calls of step(), gradient `g` restored before each (SGD overwrites it).  kind 0 = SGD (p = mo, wd, lr),
+// kind 1 = Adam (p = lr, beta1, beta2).
+namespace {
+struct OneLayerNet : public lten::NeuralNetwork {
+	explicit OneLayerNet(uint64_t n) { fc = register_module("fc", lten::FullyConnected(n, 1, false)); }
+	lten::FullyConnected* fc;
+};
+}
+int ref_optimizer_steps(int kind, uint64_t n, int steps, const float* p, float* w, const float* g)
+{
+	try {
+		OneLayerNet net(n);
+		lten::Tensor* wt = net.fc->get_weights();
+		memcpy(wt->get_data_ptr(), w, n * 4);
+		lten::Tensor X = lten::AllocateTensor({ 1, 1, 1, n }, nullptr);
+		memset(X.get_data_ptr(), 0, n * 4);
+		lten::Tensor Y = net.fc->forward(X);
+		Y.backward();  // allocates the weight's gradient buffer
+		lten::SGDOptimizer sgd;
+		lten::AdamOptimizer adam;
+		lten::Optimizer* opt;
+		if (kind == 0) { sgd.set_momentum(p[0]); sgd.set_weight_decay(p[1]); sgd.set_learning_rate(p[2]); opt = &sgd; }
+		else { adam.set_learning_rate(p[0]); adam.set_beta1(p[1]); adam.set_beta2(p[2]); opt = &adam; }
+		opt->attach_network(net);
+		for (int s = 0; s < steps; s++) {
+			memcpy(wt->get_grad_ptr(), g, n * 4);
+			opt->step();
+		}
+		memcpy(w, wt->get_data_ptr(), n * 4);
+	} catch (...) { return -1; }
+	return 0;
+}
+
 // One training step of l-ten's MLP (tests/nn_tests.cpp): FullyConnected(+bias) -> relu -> ... -> FullyConnected ->
 // log_softmax(dim 3) -> nll_loss -> backward().  x: {batch,1,1,sizes[0]}, target one-hot {batch,1,1,sizes[layers]}.
 int ref_mlp_step(uint64_t batch, int layers, const uint64_t* sizes, const float* x, const float* const* w,

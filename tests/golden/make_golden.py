@@ -297,6 +297,23 @@ def quant_cases():
     print("quant_cases", data.size)
 
 
+def optimizer_cases():
+    """Five steps of the compiled SGDOptimizer and AdamOptimizer on one parameter tensor with a fixed gradient."""
+    rng = np.random.default_rng(66)
+    n = 1000
+    w0 = rng.standard_normal(n).astype(np.float32)
+    g = rng.standard_normal(n).astype(np.float32)
+    g[:10] = 0.0
+    out = {"w0": w0, "g": g}
+    for name, kind, p in (("sgd", 0, [0.9, 0.0005, 0.01]), ("sgd_plain", 0, [0.0, 0.0, 0.1]), ("adam", 1, [0.01, 0.9, 0.999]),
+                          ("adam_fast", 1, [0.1, 0.5, 0.9])):
+        w = w0.copy()
+        assert ob.ref().ref_optimizer_steps(kind, n, 5, np.array(p, np.float32), w, g) == 0
+        out[name + "_p"], out[name + "_w"] = np.array(p, np.float32), w
+    np.savez_compressed(os.path.join(HERE, "optimizer_cases.npz"), **out)
+    print("optimizer_cases ok")
+
+
 if __name__ == "__main__":
     requant_sweep()
     qmm_cases()
@@ -306,3 +323,4 @@ if __name__ == "__main__":
     conv2dq_cases()
     mlp_step_case()
     quant_cases()
+    optimizer_cases()

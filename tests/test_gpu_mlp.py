@@ -144,3 +144,25 @@ def test_elementwise_kernels(gpu, ob):
         assert rel_err(ddx.numpy(np.float32, z.shape), want_dx) < TOL
         want_loss = ob.oracle().oracle_nll_loss(want_lp.reshape(-1), T.reshape(-1), rows * cols, rows)
         assert abs(dl.numpy(np.float32, (1,))[0] - want_loss) < 1e-5 * max(1.0, abs(want_loss))
+
+
+def test_optimizer_steps(gpu, ob):
+    """Five SGD / Adam steps on the device against the golden weights of the compiled l-ten optimizers: SGD bit-exact
+    (every operation rounded on its own, as on the CPU), Adam within 1e-6 (its powf comes from a different libm)."""
+    g = np.load(golden_path("optimizer_cases.npz"))
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    n = g["w0"].size
+    for name in ("sgd", "sgd_plain", "adam", "adam_fast"):
+        p = [float(v) for v in g[name + "_p"]]
+        dw, dv, ds = D.from_numpy(g["w0"]), D(4 * n, zero=True), D(4 * n, zero=True)
+        for it in range(1, 6):
+            dg = D.from_numpy(g["g"])
+            if name.startswith("sgd"):
+                gpu.check(l.lten_hip_sgd_step_f32(dw.ptr, dg.ptr, dv.ptr, n, p[0], p[1], p[2]))
+            else:
+                gpu.check(l.lten_hip_adam_step_f32(dw.ptr, dg.ptr, dv.ptr, ds.ptr, n, p[0], p[1], p[2], it))
+        got = dw.numpy(np.float32, (n,))
+        if name.startswith("sgd"):
+            assert np.array_equal(got, g[name + "_w"]), name
+        else:
+            assert np.abs(got - g[name + "_w"]).max() < 1e-6 * max(1.0, np.abs(g[name + "_w"]).max()), name

@@ -90,3 +90,34 @@ def test_elementwise_closed_forms(ob):
     g = np.empty_like(T)
     ob.oracle().oracle_nll_backward(T.reshape(-1), 370, 37, 2.0, g.reshape(-1))
     assert np.array_equal(g, np.float32(np.float32(-1.0 / 37) * np.float32(2.0)) * T)
+
+
+# ----------------------------------------------------------------------------------------- optimizer steps
+
+def run_oracle_optimizer(ob, kind, p, w0, g, steps=5):
+    w, v, s = w0.copy(), np.zeros_like(w0), np.zeros_like(w0)
+    for it in range(1, steps + 1):
+        if kind == "sgd":
+            gg = g.copy()    # the step overwrites the gradient with the decayed one
+            ob.oracle().oracle_sgd_step(w, gg, v, w.size, float(p[0]), float(p[1]), float(p[2]))
+        else:
+            ob.oracle().oracle_adam_step(w, g, v, s, w.size, float(p[0]), float(p[1]), float(p[2]), it)
+    return w
+
+
+def test_optimizer_steps_golden_from_compiled_optimizers(ob):
+    g = np.load(golden_path("optimizer_cases.npz"))
+    for name in ("sgd", "sgd_plain", "adam", "adam_fast"):
+        w = run_oracle_optimizer(ob, "sgd" if name.startswith("sgd") else "adam", g[name + "_p"], g["w0"], g["g"])
+        assert np.array_equal(w, g[name + "_w"]), name   # same libm on both sides: bit-exact
+
+
+def test_optimizer_closed_forms(ob):
+    w0 = np.array([1.0, -2.0, 0.5], np.float32)
+    g = np.array([0.5, 0.25, -1.0], np.float32)
+    # no momentum, no decay: plain gradient descent
+    w = run_oracle_optimizer(ob, "sgd", [0.0, 0.0, 0.1], w0, g, steps=1)
+    assert np.allclose(w, w0 - 0.1 * g, rtol=1e-6)
+    # Adam's first step moves every weight by lr * sign(g) (bias corrections cancel the history factors)
+    w = run_oracle_optimizer(ob, "adam", [0.01, 0.9, 0.999], w0, g, steps=1)
+    assert np.allclose(w, w0 - 0.01 * np.sign(g), rtol=0, atol=1e-6)
