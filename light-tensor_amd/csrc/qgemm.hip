@@ -404,7 +404,7 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	// skinny activations: one streaming pass over the weights (option "qskinny": 0 = auto, 2 = off)
 	p.cterm = nullptr;
 	p.rterm = nullptr;
-	if (M <= 16 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+	if (M <= 32 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
 	}

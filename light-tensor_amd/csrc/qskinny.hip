@@ -1,4 +1,4 @@
-// Weight-streaming int8 FC for skinny activations (M <= 16 rows against W[N x K], both contiguous in K).
+// Weight-streaming int8 FC for skinny activations (M <= 32 rows against W[N x K], both contiguous in K).
 //
 // The work is one pass over W (N*K bytes, read once from HBM); everything else is noise, so the kernel is
 // organised around that stream.  A workgroup takes 16 consecutive rows of W at a time (then the next such
@@ -26,7 +26,7 @@ __device__ __forceinline__ void skinny_async_load16(uint32_t lds_addr, const uin
 	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
-template <int WAVES, int KW, int OUT, bool SUM_A, bool SUM_B>
+template <int WAVES, int KW, int MB, int OUT, bool SUM_A, bool SUM_B>
 __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const int32_t* bias, int coef_a, int coef_b)
 {
 	// KW = bytes of K per wavefront (multiple of 1024): K == WAVES * KW
@@ -34,8 +34,11 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 	constexpr int SLAB = 16 * ROW;       // one wavefront's slab
 	constexpr int LOADS_PER_ROW = KW / 1024;
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[WAVES * SLAB];
-	__shared__ __attribute__((aligned(16))) int partial[2][WAVES][64 * 4];  // per row group parity: the k-slices' accumulators
-	__shared__ int sums_a[2][WAVES][16], sums_b[2][WAVES][16];
+	// PAR = 2: wave 0 reads one row group's partial tiles while the others already write the next group's (no second
+	// barrier); with two row blocks only one copy fits beside the slabs, and a barrier ends every row group instead
+	constexpr int PAR = MB == 1 ? 2 : 1;
+	__shared__ __attribute__((aligned(16))) int partial[PAR][WAVES][MB][64 * 4];
+	__shared__ int sums_a[WAVES][MB][16], sums_b[PAR][WAVES][16];
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -55,35 +58,48 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 
 	// the activations of this wavefront's k-slice stay in registers for every row group the workgroup takes
 	const int lrow = lane & 15, lgrp = lane >> 4;
-	const uint8_t* xrow = p.A + (int64_t)lrow * p.K + kbeg + lgrp * 16;
-	const bool xvalid = lrow < p.M;
 	const uint8_t* wfrag = smem + wave * SLAB + lrow * ROW + lgrp * 16;
 	constexpr int STEPS = KW / 64;
-	v4i fx[STEPS];
-	int sa = 0;
+	v4i fx[MB][STEPS];  // activation rows mb * 16 + lrow
+	int sa[MB];
 #pragma unroll
-	for (int s = 0; s < STEPS; s++) {
-		fx[s] = v4i{ (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
-		if (xvalid) fx[s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
+	for (int mb = 0; mb < MB; mb++) {
+		const uint8_t* xrow = p.A + (int64_t)(mb * 16 + lrow) * p.K + kbeg + lgrp * 16;
+		const bool xvalid = mb * 16 + lrow < p.M;
+		sa[mb] = 0;
+#pragma unroll
+		for (int s = 0; s < STEPS; s++) {
+			fx[mb][s] = v4i{ (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+			if (xvalid) fx[mb][s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
+		}
 	}
 	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-	for (int s = 0; s < STEPS; s++) {
-		fx[s] = flip_sign_bits(fx[s]);
+	for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+		for (int s = 0; s < STEPS; s++) {
+			fx[mb][s] = flip_sign_bits(fx[mb][s]);
+			if (SUM_A) {
+				sa[mb] = __builtin_amdgcn_sdot4(fx[mb][s].x, 0x01010101, sa[mb], false);
+				sa[mb] = __builtin_amdgcn_sdot4(fx[mb][s].y, 0x01010101, sa[mb], false);
+				sa[mb] = __builtin_amdgcn_sdot4(fx[mb][s].z, 0x01010101, sa[mb], false);
+				sa[mb] = __builtin_amdgcn_sdot4(fx[mb][s].w, 0x01010101, sa[mb], false);
+			}
+		}
+		// a lane holds the sums of its 16-byte k-group only: fold the four k-groups (lanes l, l+16, l+32, l+48)
 		if (SUM_A) {
-			sa = __builtin_amdgcn_sdot4(fx[s].x, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fx[s].y, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fx[s].z, 0x01010101, sa, false);
-			sa = __builtin_amdgcn_sdot4(fx[s].w, 0x01010101, sa, false);
+			sa[mb] += __shfl_xor(sa[mb], 16, 64);
+			sa[mb] += __shfl_xor(sa[mb], 32, 64);
+			if (lane < 16) sums_a[wave][mb][lane] = sa[mb];  // the same for every row group: written once
 		}
 	}
-	// a lane holds the sums of its 16-byte k-group only: fold the four k-groups (lanes l, l+16, l+32, l+48)
-	if (SUM_A) { sa += __shfl_xor(sa, 16, 64); sa += __shfl_xor(sa, 32, 64); }
 
 	int parity = 0;
-	for (int group = blockIdx.x; group < groups; group += gridDim.x, parity ^= 1) {
+	for (int group = blockIdx.x; group < groups; group += gridDim.x, parity = (parity + 1) & (PAR - 1)) {
 		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab has landed (no other wave reads this slab)
-		v4i acc = { 0, 0, 0, 0 };
+		v4i acc[MB];
+#pragma unroll
+		for (int mb = 0; mb < MB; mb++) acc[mb] = v4i{ 0, 0, 0, 0 };
 		int sb = 0;
 #pragma unroll
 		for (int s = 0; s < STEPS; s++) {
@@ -96,60 +112,74 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 				sb = __builtin_amdgcn_sdot4(fw.w, 0x01010101, sb, false);
 			}
 			// MFMA A operand = activations (rows m), B operand = weights (columns n):
-			// lane (lrow, lgrp), register e holds out[m = 4*lgrp + e][n = lrow]
-			acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx[s], fw, acc, 0, 0, 0);
+			// lane (lrow, lgrp), register e holds out[m = mb*16 + 4*lgrp + e][n = lrow]
+#pragma unroll
+			for (int mb = 0; mb < MB; mb++) acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx[mb][s], fw, acc[mb], 0, 0, 0);
 		}
 		// the slab is consumed (its values sit in registers): the next row group's slab can start to arrive
 		if (group + (int)gridDim.x < groups) {
 			asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 			issue_slab(group + gridDim.x);
 		}
-		if (SUM_A || SUM_B) {
+		if (SUM_B) {
 			sb += __shfl_xor(sb, 16, 64); sb += __shfl_xor(sb, 32, 64);
-			if (lane < 16) { sums_a[parity][wave][lane] = sa; sums_b[parity][wave][lane] = sb; }
+			if (lane < 16) sums_b[parity][wave][lane] = sb;
 		}
 		// partial accumulators of the k-slices meet in LDS; the two parities keep wave 0's reads of one row
 		// group apart from the other waves' writes of the next
-		*reinterpret_cast<v4i*>(&partial[parity][wave][lane * 4]) = acc;
+#pragma unroll
+		for (int mb = 0; mb < MB; mb++) *reinterpret_cast<v4i*>(&partial[parity][wave][mb][lane * 4]) = acc[mb];
 		__syncthreads();
-		if (wave != 0) continue;
-		v4i tot = { 0, 0, 0, 0 };
+		if (wave != 0) {
+			if (PAR == 1) __syncthreads();
+			continue;
+		}
+		int tsb = 0;
+		if (SUM_B) {
 #pragma unroll
-		for (int w = 0; w < WAVES; w++) tot += *reinterpret_cast<const v4i*>(&partial[parity][w][lane * 4]);
-		int tsa[4] = { 0, 0, 0, 0 }, tsb = 0;
-		if (SUM_A || SUM_B) {
-#pragma unroll
-			for (int w = 0; w < WAVES; w++) {
-				tsb += sums_b[parity][w][lrow];
-#pragma unroll
-				for (int e = 0; e < 4; e++) tsa[e] += sums_a[parity][w][lgrp * 4 + e];
-			}
+			for (int w = 0; w < WAVES; w++) tsb += sums_b[parity][w][lrow];
 		}
 		const int n = group * 16 + lrow;
 		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
 		const int base = coef_b * tsb + p.K * coef_a * coef_b + (bias ? bias[n] : 0);
 #pragma unroll
-		for (int e = 0; e < 4; e++) {
-			const int m = lgrp * 4 + e;
-			if (m >= p.M) continue;
-			const int v = tot[e] + base + coef_a * tsa[e];
-			if (OUT == Q_OUT_ACC) static_cast<int*>(p.C)[(int64_t)m * p.N + n] = v;
-			else static_cast<uint8_t*>(p.C)[(int64_t)m * p.N + n] = (uint8_t)requant<OUT>(v, p.mult, p.zp_c);
+		for (int mb = 0; mb < MB; mb++) {
+			v4i tot = { 0, 0, 0, 0 };
+			int tsa[4] = { 0, 0, 0, 0 };
+#pragma unroll
+			for (int w = 0; w < WAVES; w++) {
+				tot += *reinterpret_cast<const v4i*>(&partial[parity][w][mb][lane * 4]);
+				if (SUM_A) {
+#pragma unroll
+					for (int e = 0; e < 4; e++) tsa[e] += sums_a[w][mb][lgrp * 4 + e];
+				}
+			}
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				const int m = mb * 16 + lgrp * 4 + e;
+				if (m >= p.M) continue;
+				const int v = tot[e] + base + coef_a * tsa[e];
+				if (OUT == Q_OUT_ACC) static_cast<int*>(p.C)[(int64_t)m * p.N + n] = v;
+				else static_cast<uint8_t*>(p.C)[(int64_t)m * p.N + n] = (uint8_t)requant<OUT>(v, p.mult, p.zp_c);
+			}
 		}
+		if (PAR == 1) __syncthreads();
 	}
 }
 
-template <int WAVES, int KW>
+template <int WAVES, int KW, int MB>
 static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, const char* name)
 {
 	// as many workgroups as fit the CUs' LDS at once (one per CU at K = 8192); each walks row groups blockIdx.x, blockIdx.x + grid, ...
-	constexpr int LDS_BYTES = WAVES * 16 * (KW + 16) + 2 * WAVES * 1024 + 4 * WAVES * 64;
+	constexpr int PAR = MB == 1 ? 2 : 1;
+	constexpr int LDS_BYTES = WAVES * 16 * (KW + 16) + PAR * WAVES * MB * 1024 + (PAR + MB) * WAVES * 64;
+	static_assert(LDS_BYTES <= 160 * 1024, "slabs and partial tiles must fit the CU's LDS");
 	constexpr int PER_CU = (160 * 1024) / LDS_BYTES;
 	const dim3 grid((unsigned)std::min<int64_t>(p.N / 16, 256 * PER_CU)), block(WAVES * 64);
 	set_kernel_name(name);
 	const bool sum_a = coef_a != 0, sum_b = coef_b != 0;
-#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, KW, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b)
+#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, KW, MB, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b)
 #define LTEN_SK_OUT(OUTV)                                     \
 	if (sum_a && sum_b) LTEN_SK(OUTV, true, true);        \
 	else if (sum_a) LTEN_SK(OUTV, true, false);           \
@@ -167,11 +197,18 @@ static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int co
 // Returns -1 when the problem does not fit the streaming kernel (the caller then uses the tiled kernels).
 int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b)
 {
-	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 16 && p.N % 16 == 0)) return -1;
+	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N % 16 == 0)) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
-	if (p.K == 8 * 1024) return launch_skinny<8, 1024>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w8_k1024");
-	if (p.K == 4 * 1024) return launch_skinny<4, 1024>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w4_k1024");
-	if (p.K == 2 * 1024) return launch_skinny<2, 1024>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w2_k1024");
+	if (p.M <= 16) {
+		if (p.K == 8 * 1024) return launch_skinny<8, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w8_k1024");
+		if (p.K == 4 * 1024) return launch_skinny<4, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w4_k1024");
+		if (p.K == 2 * 1024) return launch_skinny<2, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w2_k1024");
+	} else {
+		// two blocks of 16 activation rows against every weight fragment
+		if (p.K == 8 * 1024) return launch_skinny<8, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w8_k1024_m32");
+		if (p.K == 4 * 1024) return launch_skinny<4, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w4_k1024_m32");
+		if (p.K == 2 * 1024) return launch_skinny<2, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w2_k1024_m32");
+	}
 	return -1;
 }
 
