@@ -315,9 +315,13 @@ static int qgemm_dispatch(const QProblem& p, int out)
 	const uint64_t out_elems = (uint64_t)p.M * p.N;
 	int choice = get_option(OPT_QGEMM_TILE);  // 0 = heuristic
 	if (choice == 0) {
-		// Large problems that tile exactly go to the direct-to-LDS 256x256x128 kernel; it wants enough tiles
-		// to occupy most CUs and a K long enough to amortise its prologue and epilogue.
-		if (out_elems >= 256ull * 256 * 128 && p.K >= 512 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+		// Problems that tile exactly go to the direct-to-LDS kernels when K is long enough to amortise their prologue
+		// and epilogue: 256x256 tiles once those occupy most of the 256 CUs, 128x128 tiles (up to four times as many
+		// workgroups, two per CU) below that.
+		if (p.K >= 512) {
+			if (out_elems > 256ull * 256 * 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
+		}
 		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
 			choice = 1;
 		else if (fits(128, 128, 64) && out_elems >= 128ull * 128 * 128)

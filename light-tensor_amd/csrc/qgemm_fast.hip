@@ -53,10 +53,10 @@ __device__ __forceinline__ void wait_vmcnt()
 #define LTEN_HIP_EXP 0
 #endif
 
-template <int BK, int WM, int WN, int S, int OUT, bool TERMS>
+template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS>
 __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 {
-	constexpr int BM = 256, BN = 256;
+	constexpr int BM = T, BN = T;  // square output tile, 256 or 128
 	constexpr int W = WM * WN;
 	constexpr int CPR = BK / 16;           // 16-byte chunks per tile row
 	constexpr int RPL = 64 / CPR;          // tile rows covered by one wave-wide load
@@ -288,7 +288,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		uint8_t* cout = static_cast<uint8_t*>(p.C) + (int64_t)m0 * p.N + n0;
 #pragma unroll
 		for (int c = tid; c < BM * BN / 16; c += W * 64) {
-			const int row = c >> 4, ch = c & 15;
+			const int row = c / (BN / 16), ch = c % (BN / 16);
 			*reinterpret_cast<v4i*>(cout + (int64_t)row * p.N + ch * 16) = *reinterpret_cast<const v4i*>(smem + row * OLD + ch * 16);
 		}
 	}
@@ -298,17 +298,18 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #endif
 }
 
-template <int BK, int WM, int WN, int S>
+template <int T, int BK, int WM, int WN, int S>
 static int launch_fast(const QProblem& p, int out, const char* name)
 {
-	const dim3 grid((unsigned)((p.M / 256) * (p.N / 256))), block(WM * WN * 64);
+	if (p.M % T != 0 || p.N % T != 0) return -1;
+	const dim3 grid((unsigned)((p.M / T) * (p.N / T))), block(WM * WN * 64);
 	const bool terms = p.rterm != nullptr;
 	set_kernel_name(name);
 #define LTEN_LAUNCH(OUTV)                                                                        \
 	if (terms)                                                                               \
-		qgemm_fast_kernel<BK, WM, WN, S, OUTV, true><<<grid, block, 0, stream()>>>(p);     \
+		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, true><<<grid, block, 0, stream()>>>(p);     \
 	else                                                                                     \
-		qgemm_fast_kernel<BK, WM, WN, S, OUTV, false><<<grid, block, 0, stream()>>>(p);
+		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, false><<<grid, block, 0, stream()>>>(p);
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
@@ -320,20 +321,25 @@ static int launch_fast(const QProblem& p, int out, const char* name)
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M % 256 == 0 && p.N % 256 == 0 && p.K % 128 == 0 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0);
 	if (!fits) return -1;
 	switch (variant) {
-	case 21: return launch_fast<64, 2, 2, 3>(p, out, "qgemm_fast_256x256x64_w2x2_s3");
-	case 23: return launch_fast<64, 2, 4, 3>(p, out, "qgemm_fast_256x256x64_w2x4_s3");
-	case 24: return launch_fast<64, 4, 2, 3>(p, out, "qgemm_fast_256x256x64_w4x2_s3");
-	case 26: return launch_fast<64, 4, 2, 4>(p, out, "qgemm_fast_256x256x64_w4x2_s4");
-	case 28: return launch_fast<64, 4, 2, 2>(p, out, "qgemm_fast_256x256x64_w4x2_s2");
-	case 31: return launch_fast<128, 2, 2, 2>(p, out, "qgemm_fast_256x256x128_w2x2_s2");
-	case 33: return launch_fast<128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
-	case 34: return launch_fast<128, 4, 2, 2>(p, out, "qgemm_fast_256x256x128_w4x2_s2");
+	case 21: return launch_fast<256, 64, 2, 2, 3>(p, out, "qgemm_fast_256x256x64_w2x2_s3");
+	case 23: return launch_fast<256, 64, 2, 4, 3>(p, out, "qgemm_fast_256x256x64_w2x4_s3");
+	case 24: return launch_fast<256, 64, 4, 2, 3>(p, out, "qgemm_fast_256x256x64_w4x2_s3");
+	case 26: return launch_fast<256, 64, 4, 2, 4>(p, out, "qgemm_fast_256x256x64_w4x2_s4");
+	case 28: return launch_fast<256, 64, 4, 2, 2>(p, out, "qgemm_fast_256x256x64_w4x2_s2");
+	case 31: return launch_fast<256, 128, 2, 2, 2>(p, out, "qgemm_fast_256x256x128_w2x2_s2");
+	case 33: return launch_fast<256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
+	case 34: return launch_fast<256, 128, 4, 2, 2>(p, out, "qgemm_fast_256x256x128_w4x2_s2");
+	// 128 x 128 tiles for outputs too small to give every CU a 256 x 256 tile
+	case 41: return launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
+	case 42: return launch_fast<128, 128, 2, 2, 3>(p, out, "qgemm_fast_128x128x128_w2x2_s3");
+	case 43: return launch_fast<128, 64, 2, 2, 3>(p, out, "qgemm_fast_128x128x64_w2x2_s3");
+	case 44: return launch_fast<128, 64, 2, 2, 4>(p, out, "qgemm_fast_128x128x64_w2x2_s4");
 	default: return -1;
 	}
 }

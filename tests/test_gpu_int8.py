@@ -138,6 +138,31 @@ def test_fcq_forward_leading_dims(gpu, ob, wl):
     assert np.array_equal(dY.numpy(np.uint8, (64, 512)), np.load(golden_path("cfg1_expected.npz"))["C"])
 
 
+@pytest.mark.parametrize("variant", [41, 42, 43, 44])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (384, 640, 640), (128, 1152, 2048)])
+def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
+    """The 128x128 form of the direct-to-LDS tiles (what the library picks when 256x256 tiles would leave CUs idle):
+    both k-step sizes, 2 to 4 stages, with and without zero-point terms and bias, short and long K; int32 and u8."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + variant)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=variant)
+    assert gpu.last_kernel().startswith("qgemm_fast_128x128")
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8),
+             bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
+    run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)   # multiplier > 0.99: exact-convert epilogue
+
+
+def test_medium_batch_picks_128_tiles(gpu, ob):
+    """512 x 1024 x 1024: 8 tiles of 256x256 would occupy 8 CUs; the library takes 32 tiles of 128x128."""
+    rng = np.random.default_rng(77)
+    A = rng.integers(0, 256, (512, 1024), dtype=np.uint8)
+    B = rng.integers(0, 256, (1024, 1024), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([9, 131, 100], np.uint8), bias=rng.integers(-5000, 5000, 1024).astype(np.int32))
+    assert gpu.last_kernel().startswith("qgemm_fast_128x128x128")
+
+
 def test_cfg3_full_size_properties(gpu, wl):
     """4096^3: exact closed form of every accumulator (fp64 BLAS holds these integers exactly),
     then the requantize rule on top; plus linearity in the bias."""
