@@ -302,29 +302,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	}
 }
 
-// out[i] = sum over parts of partial[p][i].  A workgroup takes 64 outputs; its 16 groups of 64 lanes each add
-// every 16th part, then the 16 group sums are added in group order.
+// out[i] = sum over parts of partial[p][i].  A workgroup takes OUTS outputs; its 1024 / OUTS groups of lanes each
+// add every GROUPS-th part (eight loads in flight, added in part order), then the group sums are added in
+// group order.  Few outputs (a first layer's weights) get the narrow shape, so that more than a handful of
+// workgroups share the reading.
+template <int OUTS>
 __global__ __launch_bounds__(1024) void conv_reduce_partials_kernel(const float* __restrict__ partial, int parts, int64_t count, float* __restrict__ out)
 {
-	__shared__ float s[16][64];
-	const int o = threadIdx.x & 63, grp = threadIdx.x >> 6;
-	const int64_t idx = (int64_t)blockIdx.x * 64 + o;
+	constexpr int GROUPS = 1024 / OUTS;
+	__shared__ float s[GROUPS][OUTS];
+	const int o = threadIdx.x % OUTS, grp = threadIdx.x / OUTS;
+	const int64_t idx = (int64_t)blockIdx.x * OUTS + o;
 	float sum = 0.0f;
-	if (idx < count)
-		for (int p = grp; p < parts; p += 16) sum += partial[(int64_t)p * count + idx];
+	if (idx < count) {
+		const float* src = partial + idx;
+		int p = grp;
+		for (; p + 7 * GROUPS < parts; p += 8 * GROUPS) {
+			float v[8];
+#pragma unroll
+			for (int q = 0; q < 8; q++) v[q] = src[(int64_t)(p + q * GROUPS) * count];
+#pragma unroll
+			for (int q = 0; q < 8; q++) sum += v[q];
+		}
+		for (; p < parts; p += GROUPS) sum += src[(int64_t)p * count];
+	}
 	s[grp][o] = sum;
 	__syncthreads();
 	if (grp == 0 && idx < count) {
 		float tot = 0.0f;
 #pragma unroll
-		for (int q = 0; q < 16; q++) tot += s[q][o];
+		for (int q = 0; q < GROUPS; q++) tot += s[q][o];
 		out[idx] = tot;
 	}
 }
 
 int conv_reduce_partials(const float* partial, int parts, int64_t count, float* out)
 {
-	conv_reduce_partials_kernel<<<dim3((unsigned)ceil_div(count, 64)), dim3(1024), 0, stream()>>>(partial, parts, count, out);
+	if (count <= 4096) conv_reduce_partials_kernel<16><<<dim3((unsigned)ceil_div(count, 16)), dim3(1024), 0, stream()>>>(partial, parts, count, out);
+	else conv_reduce_partials_kernel<64><<<dim3((unsigned)ceil_div(count, 64)), dim3(1024), 0, stream()>>>(partial, parts, count, out);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

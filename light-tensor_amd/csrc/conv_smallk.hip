@@ -6,10 +6,11 @@
 // 32x32x2 fp32 MFMA tile whose reduction (forward) or column (weight gradient) dimension holds all taps.
 //
 // Work unit: a chunk = TW = 128 consecutive pixels of one output row of one image; the four wavefronts of a
-// workgroup take 32 pixels each.  A workgroup walks a contiguous range of chunks with two LDS patch buffers:
-// the rows of chunk c + 1 are fetched while chunk c is computed and stored to the other buffer after it, one barrier
-// per chunk.  LDS patch row r = ci*kh + i holds input row ho + i - ph of channel ci, index q = input column
-// w0 - 4 + q.
+// workgroup take 32 pixels each and never wait for one another: every wavefront keeps its own two LDS patch
+// buffers (its 32 pixels plus the halo), fetches the rows of chunk c + 1 into registers while chunk c is
+// computed, and stores them to the other buffer afterwards.  LDS operations of one wavefront complete in
+// order, so no barrier separates a wavefront's patch stores from its own later reads.  LDS patch row
+// r = ci*kh + i holds input row ho + i - ph of channel ci, index q = input column w0 + 32*wave - 4 + q.
 #include "conv_common.h"
 #include "gemm_f32_core.h"
 
@@ -22,12 +23,23 @@ namespace {
 constexpr int SK_TW = 128;       // pixels per chunk
 constexpr int SK_MAXK = 32;      // taps: one MFMA tile dimension
 constexpr int SK_MAXKW = 9;      // widest kernel row the patch row has room for
-constexpr int SK_PWS = 4 + SK_TW + SK_MAXKW - 1;  // 140 floats = 35 float4; 140 % 32 = 12 keeps 3x3 taps on 9 banks
+constexpr int SK_PWS = 4 + 32 + SK_MAXKW - 1;     // 44 floats = 11 float4 per wavefront; 44 % 32 = 12 keeps 3x3 taps on 9 banks
 constexpr int SK_F4_ROW = SK_PWS / 4;
-constexpr int SK_PATCH = SK_MAXK * SK_PWS + 4;    // + a slot that stays zero (what padded taps read)
-constexpr int SK_P_PER_T = (SK_MAXK * SK_F4_ROW + 255) / 256;
 static_assert(SK_PWS % 4 == 0, "patch rows are whole float4s");
 
+// Two sizes of each kernel: RC = patch rows (Cin*kh) an LDS buffer has room for.  The small one (up to 8 rows
+// and 16 taps, e.g. one input channel with a kernel of up to 4x4) keeps 9 KB of LDS and half the
+// weight registers, so that more wavefronts share a CU and hide each other's load waits.
+template <int RC>
+struct SkShape {
+	static constexpr int ROWS = RC;
+	static constexpr int STEPS = RC <= 8 ? 8 : SK_MAXK / 2;  // MFMA steps (two taps each) held in registers
+	static constexpr int ZERO = RC * SK_PWS;                  // a slot that stays zero (what padded taps read)
+	static constexpr int PATCH = RC * SK_PWS + 4;
+	static constexpr int P_PER_T = (RC * SK_F4_ROW + 63) / 64;  // float4 per lane
+};
+
+// Coordinates of a chunk.  A workgroup computes them once with divisions and then steps from chunk to chunk.
 struct Chunk {
 	int n, ho, w0;
 };
@@ -41,34 +53,66 @@ __device__ __forceinline__ Chunk chunk_at(const ConvGeo& g, int chunk, int tiles
 	return c;
 }
 
-// This thread's share of the patch rows of a chunk: fetched to registers, stored to an LDS buffer later.
-struct PatchRegs {
-	float4 v[SK_P_PER_T];
+__device__ __forceinline__ Chunk next_chunk(const ConvGeo& g, Chunk c)
+{
+	c.w0 += SK_TW;
+	if (c.w0 >= g.Wo) {
+		c.w0 = 0;
+		if (++c.ho == g.Ho) { c.ho = 0; c.n++; }
+	}
+	return c;
+}
+
+// This lane's share of its wavefront's patch rows: float4 number idx = lane + 64*q of the patch is column
+// group f = idx % 11 of patch row r = idx / 11.  What does not change from chunk to chunk is worked out once:
+// the offset of the row inside its image, and the row / column shifts that decide whether the piece lies
+// inside the image.  The values are fetched to registers and stored to LDS later.
+template <int P_PER_T>
+struct PatchLane {
+	int rel[P_PER_T];  // (ci*H + i - ph)*W + gx: element offset from x[n][0][ho][w0]
+	int gy[P_PER_T];   // i - ph; far below -H for rows the geometry does not have
+	int gx[P_PER_T];   // 32*wave - 4 + 4*f
+	float4 v[P_PER_T];
 };
 
-template <bool VEC>
-__device__ __forceinline__ void fetch_patch(const ConvGeo& g, const float* __restrict__ x, const Chunk& c, int tid, PatchRegs& p)
+template <int P_PER_T>
+__device__ __forceinline__ void init_patch_lane(const ConvGeo& g, int wave, int lane, PatchLane<P_PER_T>& p)
 {
 	const int rows = g.Cin * g.kh;
 #pragma unroll
-	for (int q = 0; q < SK_P_PER_T; q++) {
-		const int idx = tid + q * 256;
+	for (int q = 0; q < P_PER_T; q++) {
+		const int idx = lane + q * 64;
 		const int f = idx % SK_F4_ROW, r = idx / SK_F4_ROW;
-		const int ci = r / g.kh, gy = c.ho + (r - ci * g.kh) - g.ph;
-		p.v[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-		if (r < rows && gy >= 0 && gy < g.H)
-			p.v[q] = load_row4<VEC>(x + (((int64_t)c.n * g.Cin + ci) * g.H + gy) * g.W, c.w0 - 4 + 4 * f, g.W);
+		const int ci = r / g.kh, i = r - ci * g.kh;
+		p.gx[q] = wave * 32 - 4 + 4 * f;
+		p.gy[q] = r < rows ? i - g.ph : -(1 << 30);
+		p.rel[q] = r < rows ? (ci * g.H + i - g.ph) * g.W + p.gx[q] : 0;
 	}
 }
 
-__device__ __forceinline__ void store_patch(const ConvGeo& g, float* buf, int tid, const PatchRegs& p)
+template <bool VEC, int P_PER_T>
+__device__ __forceinline__ void fetch_patch(const ConvGeo& g, const float* __restrict__ x, const Chunk& c, PatchLane<P_PER_T>& p)
 {
-	const int rows = g.Cin * g.kh;
+	const float* origin = x + ((int64_t)c.n * g.Cin * g.H + c.ho) * g.W + c.w0;  // same for the whole workgroup
 #pragma unroll
-	for (int q = 0; q < SK_P_PER_T; q++) {
-		const int idx = tid + q * 256;
-		if (idx / SK_F4_ROW < rows) *reinterpret_cast<float4*>(buf + idx * 4) = p.v[q];
+	for (int q = 0; q < P_PER_T; q++) {
+		p.v[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+		if ((unsigned)(c.ho + p.gy[q]) < (unsigned)g.H) {
+			if (VEC) {  // W % 4 == 0 and gx % 4 == 0: the four columns are inside or outside together
+				if ((unsigned)(c.w0 + p.gx[q]) < (unsigned)g.W) p.v[q] = *reinterpret_cast<const float4*>(origin + p.rel[q]);
+			} else {
+				p.v[q] = load_row4<false>(origin + (p.rel[q] - p.gx[q]) - c.w0, c.w0 + p.gx[q], g.W);
+			}
+		}
 	}
+}
+
+template <int P_PER_T>
+__device__ __forceinline__ void store_patch(float* buf, int lane, const PatchLane<P_PER_T>& p)
+{
+#pragma unroll
+	for (int q = 0; q < P_PER_T; q++)
+		if (p.gy[q] > -(1 << 29)) *reinterpret_cast<float4*>(buf + (lane + q * 64) * 4) = p.v[q];
 }
 
 // LDS offset of tap k = (ci, i, j) relative to the pixel's own position in patch row 0.
@@ -83,11 +127,12 @@ __device__ __forceinline__ int tap_offset(const ConvGeo& g, int k)
 // Forward: y[n][co][ho][wo] = bias[co] + sum_k w[co][k] * patch_k[wo].  MFMA rows = 32 output channels
 // (blockIdx.y picks the block), columns = the wavefront's 32 pixels, reduction = taps, two per step: lanes 0-31
 // take tap 2s, lanes 32-63 tap 2s + 1.  The weights stay in registers for the whole kernel.
-template <bool VEC>
+template <bool VEC, int RC>
 __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ w,
                                                                     const float* __restrict__ bias, float* __restrict__ y, int chunks_per_group)
 {
-	__shared__ __attribute__((aligned(16))) float s_patch[2][SK_PATCH];
+	using S = SkShape<RC>;
+	__shared__ __attribute__((aligned(16))) float s_mem[4 * 2 * S::PATCH];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
 	const int K = g.Cin * g.kh * g.kw, steps = (K + 1) / 2;
 	const int co0 = blockIdx.y * 32;
@@ -95,18 +140,19 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 	const int begin = blockIdx.x * chunks_per_group, end = min(total, begin + chunks_per_group);
 	if (begin >= end) return;
 
-	if (tid < 4) { s_patch[0][SK_MAXK * SK_PWS + tid] = 0.0f; s_patch[1][SK_MAXK * SK_PWS + tid] = 0.0f; }
+	float* const mine = s_mem + wave * 2 * S::PATCH;  // this wavefront's two buffers
+	if (lane < 4) { mine[S::ZERO + lane] = 0.0f; mine[S::PATCH + S::ZERO + lane] = 0.0f; }
 
 	// operand A: w[co0 + lrow][2s + half]; operand B address: this lane's pixel plus the tap offset
-	const int pix = wave * 32 + lrow + 4 - g.pw;
-	float wa[SK_MAXK / 2];
-	int off[SK_MAXK / 2];
+	const int pix = lrow + 4 - g.pw;
+	float wa[S::STEPS];
+	int off[S::STEPS];
 #pragma unroll
-	for (int s = 0; s < SK_MAXK / 2; s++) {
+	for (int s = 0; s < S::STEPS; s++) {
 		const int k = 2 * s + half;
 		const bool valid = k < K;
 		wa[s] = (valid && co0 + lrow < g.Cout) ? w[(int64_t)(co0 + lrow) * K + k] : 0.0f;
-		off[s] = valid ? pix + tap_offset(g, k) : SK_MAXK * SK_PWS;
+		off[s] = valid ? pix + tap_offset(g, k) : S::ZERO;
 	}
 	float bv[16];
 #pragma unroll
@@ -115,35 +161,44 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 		bv[r] = (bias && co < g.Cout) ? bias[co] : 0.0f;
 	}
 
-	PatchRegs pr;
-	fetch_patch<VEC>(g, x, chunk_at(g, begin, tiles_w), tid, pr);
-	store_patch(g, s_patch[0], tid, pr);
-	__syncthreads();
+	// stores: a row of y per register; the address is a part all lanes share plus this lane's offset
+	const int64_t plane = (int64_t)g.Ho * g.Wo;
+	const unsigned y_lane = (unsigned)(half * 4 * plane) + wave * 32 + lrow;
+	const bool all_channels = co0 + 32 <= g.Cout;
+
+	PatchLane<S::P_PER_T> pr;
+	init_patch_lane(g, wave, lane, pr);
+	Chunk c = chunk_at(g, begin, tiles_w);
+	fetch_patch<VEC>(g, x, c, pr);
+	store_patch(mine, lane, pr);
 	for (int chunk = begin; chunk < end; chunk++) {
 		const int cur = (chunk - begin) & 1;
-		const Chunk c = chunk_at(g, chunk, tiles_w);
-		if (chunk + 1 < end) fetch_patch<VEC>(g, x, chunk_at(g, chunk + 1, tiles_w), tid, pr);
+		const Chunk nc = next_chunk(g, c);
+		if (chunk + 1 < end) fetch_patch<VEC>(g, x, nc, pr);
 
 		v16f acc;
 #pragma unroll
 		for (int r = 0; r < 16; r++) acc[r] = bv[r];
-		const float* pb = s_patch[cur];
+		const float* pb = mine + cur * S::PATCH;
 #pragma unroll
-		for (int s = 0; s < SK_MAXK / 2; s++) {
+		for (int s = 0; s < S::STEPS; s++) {
 			if (s >= steps) break;
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wa[s], pb[off[s]], acc, 0, 0, 0);
 		}
 
-		const int wo = c.w0 + wave * 32 + lrow;
-		if (wo < g.Wo) {
+		float* yc = y + (((int64_t)c.n * g.Cout + co0) * g.Ho + c.ho) * g.Wo + c.w0;  // same for the whole workgroup
+		if (c.w0 + wave * 32 + lrow < g.Wo) {
+			if (all_channels) {
 #pragma unroll
-			for (int r = 0; r < 16; r++) {
-				const int co = co0 + (r >> 2) * 8 + half * 4 + (r & 3);
-				if (co < g.Cout) y[(((int64_t)c.n * g.Cout + co) * g.Ho + c.ho) * g.Wo + wo] = acc[r];
+				for (int r = 0; r < 16; r++) (yc + ((r >> 2) * 8 + (r & 3)) * plane)[y_lane] = acc[r];
+			} else {
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					if (co0 + (r >> 2) * 8 + half * 4 + (r & 3) < g.Cout) (yc + ((r >> 2) * 8 + (r & 3)) * plane)[y_lane] = acc[r];
 			}
 		}
-		if (chunk + 1 < end) store_patch(g, s_patch[cur ^ 1], tid, pr);
-		__syncthreads();
+		if (chunk + 1 < end) store_patch(mine + (cur ^ 1) * S::PATCH, lane, pr);
+		c = nc;
 	}
 }
 
@@ -152,26 +207,40 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 // wavefront's 32 pixels of every chunk.  dy goes from global memory straight into the A operand: lane
 // (co, half) loads four consecutive pixels at 8u + 4*half, so the 32-byte pieces a wavefront touches add up
 // to whole rows over four loads.  Step (u, e) multiplies pixels 8u + e (lanes 0-31) and 8u + 4 + e (lanes 32-63).
-template <bool VEC>
+template <bool VEC, int RC>
 __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy,
                                                                   float* __restrict__ partial, int chunks_per_part)
 {
-	__shared__ __attribute__((aligned(16))) float s_patch[2][SK_PATCH];
+	using S = SkShape<RC>;
+	constexpr int RED = 3 * 16 * 64;  // three wavefronts' accumulator tiles for the final sum
+	__shared__ __attribute__((aligned(16))) float s_mem[8 * S::PATCH > RED ? 8 * S::PATCH : RED];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
 	const int K = g.Cin * g.kh * g.kw;
 	const int co0 = blockIdx.y * 32, co = co0 + lrow;
 	const int tiles_w = (g.Wo + SK_TW - 1) / SK_TW, total = g.N * g.Ho * tiles_w;
 	const int begin = blockIdx.x * chunks_per_part, end = min(total, begin + chunks_per_part);
 
-	if (tid < 4) { s_patch[0][SK_MAXK * SK_PWS + tid] = 0.0f; s_patch[1][SK_MAXK * SK_PWS + tid] = 0.0f; }
+	float* const mine = s_mem + wave * 2 * S::PATCH;  // this wavefront's two buffers
 
-	const int boff = (lrow < K ? tap_offset(g, lrow) : 0) + wave * 32 + 4 * half + 4 - g.pw;
+	const int boff = (lrow < K ? tap_offset(g, lrow) : 0) + 4 * half + 4 - g.pw;
+	// dy: the address is a part all lanes share plus this lane's offset; with VEC (Wo % 4 == 0) the four
+	// pixels of a load are inside or outside the row together
+	const int64_t plane = (int64_t)g.Ho * g.Wo;
+	const unsigned dy_lane = (unsigned)(lrow * plane) + wave * 32 + 4 * half;
+	const bool co_ok = co < g.Cout;
 	auto load_dy = [&](const Chunk& c, float4 (&a)[4]) {
+		const float* dc = dy + (((int64_t)c.n * g.Cout + co0) * g.Ho + c.ho) * g.Wo + c.w0;  // same for the whole workgroup
+		const int col = c.w0 + wave * 32 + 4 * half;
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
 			a[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (co < g.Cout)
-				a[u] = load_row4<VEC>(dy + (((int64_t)c.n * g.Cout + co) * g.Ho + c.ho) * g.Wo, c.w0 + wave * 32 + 8 * u + 4 * half, g.Wo);
+			if (co_ok) {
+				if (VEC) {
+					if (col + 8 * u < g.Wo) a[u] = *reinterpret_cast<const float4*>(dc + 8 * u + dy_lane);
+				} else {
+					a[u] = load_row4<false>(dc + dy_lane - (wave * 32 + 4 * half) - c.w0, col + 8 * u, g.Wo);
+				}
+			}
 		}
 	};
 
@@ -180,22 +249,22 @@ __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, con
 	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
 
 	float4 a_cur[4], a_next[4];
-	PatchRegs pr;
+	PatchLane<S::P_PER_T> pr;
+	init_patch_lane(g, wave, lane, pr);
+	Chunk c = chunk_at(g, begin, tiles_w);
 	if (begin < end) {
-		const Chunk c = chunk_at(g, begin, tiles_w);
-		fetch_patch<VEC>(g, x, c, tid, pr);
+		fetch_patch<VEC>(g, x, c, pr);
 		load_dy(c, a_cur);
-		store_patch(g, s_patch[0], tid, pr);
+		store_patch(mine, lane, pr);
 	}
-	__syncthreads();
 	for (int chunk = begin; chunk < end; chunk++) {
 		const int cur = (chunk - begin) & 1;
+		c = next_chunk(g, c);
 		if (chunk + 1 < end) {
-			const Chunk c = chunk_at(g, chunk + 1, tiles_w);
-			fetch_patch<VEC>(g, x, c, tid, pr);
+			fetch_patch<VEC>(g, x, c, pr);
 			load_dy(c, a_next);
 		}
-		const float* pb = s_patch[cur] + boff;
+		const float* pb = mine + cur * S::PATCH + boff;
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[u].x, pb[8 * u + 0], acc, 0, 0, 0);
@@ -204,15 +273,15 @@ __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, con
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[u].w, pb[8 * u + 3], acc, 0, 0, 0);
 		}
 		if (chunk + 1 < end) {
-			store_patch(g, s_patch[cur ^ 1], tid, pr);
+			store_patch(mine + (cur ^ 1) * S::PATCH, lane, pr);
 #pragma unroll
 			for (int u = 0; u < 4; u++) a_cur[u] = a_next[u];
 		}
-		__syncthreads();
 	}
 
 	// add the four wavefronts' tiles in wavefront order, then lanes whose column is a tap store
-	float* red = &s_patch[0][0];
+	float* red = s_mem;
+	__syncthreads();  // every wavefront is done with its patch buffers
 	if (wave != 0) {
 #pragma unroll
 		for (int r = 0; r < 16; r++) red[((wave - 1) * 16 + r) * 64 + lane] = acc[r];
@@ -233,16 +302,20 @@ __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, con
 bool conv_smallk_takes(const ConvGeo& g)
 {
 	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.Cin * g.kh * g.kw <= SK_MAXK && g.kw <= SK_MAXKW && g.pw <= 4 &&
+	       (uint64_t)g.Ho * g.Wo <= (1u << 24) && (uint64_t)g.Cin * g.H * g.W < (1u << 29) &&  // 32-bit lane offsets
 	       ceil_div((uint64_t)g.Cout, 32) < 65536 && (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, SK_TW) < (1ull << 31);
 }
 
+// The small kernel size: patch rows fit 8 and the taps fit 8 MFMA steps.
+static bool smallk_small(const ConvGeo& g) { return g.Cin * g.kh <= 8 && g.Cin * g.kh * g.kw <= 16; }
+
 static uint64_t smallk_chunks(const ConvGeo& g) { return (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, SK_TW); }
 
-// Workgroups along x: about four per CU over all channel blocks, at least two chunks each (none empty).
-static int smallk_groups(const ConvGeo& g)
+// Workgroups along x: about `target` over all channel blocks, at least two chunks each (none empty).
+static int smallk_groups(const ConvGeo& g, int target)
 {
 	const uint64_t chunks = smallk_chunks(g), blocks = ceil_div((uint64_t)g.Cout, 32);
-	uint64_t groups = std::max<uint64_t>(1, 1024 / blocks);
+	uint64_t groups = std::max<uint64_t>(1, (uint64_t)target / blocks);
 	groups = std::min<uint64_t>(groups, std::max<uint64_t>(1, chunks / 2));
 	const uint64_t per = ceil_div(chunks, groups);
 	return (int)ceil_div(chunks, per);
@@ -250,27 +323,40 @@ static int smallk_groups(const ConvGeo& g)
 
 int conv_smallk_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
-	const int groups = smallk_groups(g);
+	const int groups = smallk_groups(g, 1024);  // four workgroups per CU
 	const int per = (int)ceil_div(smallk_chunks(g), (uint64_t)groups);
 	const dim3 grid((unsigned)groups, (unsigned)ceil_div((uint64_t)g.Cout, 32));
-	set_kernel_name("conv2d_smallk_forward_32x128");
-	if (g.W % 4 == 0 && aligned16(x)) conv2d_smallk_forward_kernel<true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
-	else conv2d_smallk_forward_kernel<false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+	const bool vec = g.W % 4 == 0 && aligned16(x);
+	if (smallk_small(g)) {
+		set_kernel_name("conv2d_smallk_forward_32x128_r8");
+		if (vec) conv2d_smallk_forward_kernel<true, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+		else conv2d_smallk_forward_kernel<false, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+	} else {
+		set_kernel_name("conv2d_smallk_forward_32x128");
+		if (vec) conv2d_smallk_forward_kernel<true, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+		else conv2d_smallk_forward_kernel<false, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }
 
-int conv_smallk_wgrad_parts(const ConvGeo& g) { return smallk_groups(g); }
+// Two workgroups per CU: every workgroup leaves a partial sum that has to be written and read again.
+int conv_smallk_wgrad_parts(const ConvGeo& g) { return smallk_groups(g, 512); }
 
 int conv_smallk_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts)
 {
 	const int per = (int)ceil_div(smallk_chunks(g), (uint64_t)parts);
 	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, 32));
-	set_kernel_name("conv2d_smallk_wgrad_32x128");
-	if (g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy))
-		conv2d_smallk_wgrad_kernel<true><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
-	else
-		conv2d_smallk_wgrad_kernel<false><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
+	if (smallk_small(g)) {
+		set_kernel_name("conv2d_smallk_wgrad_32x128_r8");
+		if (vec) conv2d_smallk_wgrad_kernel<true, 8><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		else conv2d_smallk_wgrad_kernel<false, 8><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	} else {
+		set_kernel_name("conv2d_smallk_wgrad_32x128");
+		if (vec) conv2d_smallk_wgrad_kernel<true, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		else conv2d_smallk_wgrad_kernel<false, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }
