@@ -137,21 +137,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 		__syncthreads();
 	}
 
-	const int ho = h0 + wave;
+	// Epilogue.  All bias values are loaded before the first store, so that no store waits behind a load; an
+	// address is a part the wavefront shares (row ho of channel co0 + 32m + 8(r/4) + r%4) plus a lane offset.
+	const int ho = h0 + __builtin_amdgcn_readfirstlane(wave);
 	if (ho >= g.Ho) return;
+	float bv[P::MT][16];
 #pragma unroll
 	for (int m = 0; m < P::MT; m++)
 #pragma unroll
 		for (int r = 0; r < 16; r++) {
 			const int co = co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-			if (co >= g.Cout) continue;
-			const float b = bias ? bias[co] : 0.0f;
-			float* yrow = y + (((int64_t)n * g.Cout + co) * g.Ho + ho) * g.Wo;
+			bv[m][r] = (bias && co < g.Cout) ? bias[co] : 0.0f;
+		}
+	const int64_t plane = (int64_t)g.Ho * g.Wo;
+	float* yw = y + (((int64_t)n * g.Cout + co0) * g.Ho + ho) * g.Wo + w0;
+	const unsigned y_lane = (unsigned)(half * 4 * plane) + lrow;
+	if (co0 + P::BM <= g.Cout && w0 + P::TW <= g.Wo) {
 #pragma unroll
-			for (int t = 0; t < P::NT; t++) {
-				const int wo = w0 + t * 32 + lrow;
-				if (wo < g.Wo) yrow[wo] = acc[m][t][r] + b;
+		for (int m = 0; m < P::MT; m++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+#pragma unroll
+				for (int t = 0; t < P::NT; t++) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
 			}
+		return;
+	}
+#pragma unroll
+	for (int m = 0; m < P::MT; m++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			if (co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3) >= g.Cout) continue;
+			float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+#pragma unroll
+			for (int t = 0; t < P::NT; t++)
+				if (w0 + t * 32 + lrow < g.Wo) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
 		}
 }
 
@@ -346,7 +366,8 @@ int conv_reduce_partials(const float* partial, int parts, int64_t count, float* 
 
 static bool patch_geometry(const ConvGeo& g)
 {
-	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw <= 4;
+	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw <= 4 &&
+	       (uint64_t)g.Ho * g.Wo <= (1u << 26);  // 32-bit lane offsets in the forward epilogue
 }
 
 bool conv_patch_forward_takes(const ConvGeo& g, const float*, const float*)
