@@ -223,6 +223,23 @@ int lten_hip_quantize_i32(const float* data, int32_t* q_data, uint64_t len, cons
 int lten_hip_dequantize_u8(float* data, const uint8_t* q_data, uint64_t len, const lten_hip_qparams* qparams);
 int lten_hip_get_min_max(const float* data, uint64_t len, float* min_val, float* max_val);
 
+/* ----------------------------------------------------------------------- launch graphs */
+
+/* A training or inference step is a fixed sequence of short launches (twenty for a three-layer MLP step), and
+ * the host's launch cost then exceeds the kernels' run time.  lten_hip_graph_begin starts recording the
+ * compute entry points called on this thread instead of running them; lten_hip_graph_end returns the
+ * recording as a handle, and every lten_hip_graph_launch replays it on the library's stream with one submit.
+ * Pointers and sizes are recorded by value: the buffers must stay where they are (new contents are fine).
+ * Between begin and end only compute entry points may be called: no lten_hip_alloc / free / copy_* / sync /
+ * get_min_max (they allocate, copy or wait, which a recording cannot hold), and lten_hip_last_kernel names
+ * what was recorded, not what ran.  When the library is on the null stream the recording uses a stream of
+ * the library's own; replays still go to the library's stream.  One capture at a time per process.
+ * No counterpart in l-ten, whose GPU branches launch eagerly on the default stream. */
+int lten_hip_graph_begin(void);
+int lten_hip_graph_end(void** graph);
+int lten_hip_graph_launch(void* graph);
+int lten_hip_graph_destroy(void* graph);
+
 /* ----------------------------------------------------------------------- measurement */
 
 /* HIP events on the library's stream; no counterpart in l-ten (its benchmarks use

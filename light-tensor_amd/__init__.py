@@ -77,6 +77,10 @@ _SIGNATURES = {
     "lten_hip_quantize_i32": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_dequantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_get_min_max": (C.c_int, [vp, u64, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "lten_hip_graph_begin": (C.c_int, []),
+    "lten_hip_graph_end": (C.c_int, [C.POINTER(vp)]),
+    "lten_hip_graph_launch": (C.c_int, [vp]),
+    "lten_hip_graph_destroy": (C.c_int, [vp]),
     "lten_hip_event_create": (C.c_int, [C.POINTER(vp)]),
     "lten_hip_event_record": (C.c_int, [vp]),
     "lten_hip_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
@@ -219,6 +223,34 @@ class Timer:
         try:
             lib().lten_hip_event_destroy(self.e0)
             lib().lten_hip_event_destroy(self.e1)
+        except Exception:
+            pass
+
+
+class Graph:
+    """A recorded sequence of compute calls: `with Graph() as g: <calls>` records, g.launch() replays.
+    The buffers the calls named must stay allocated at the same addresses."""
+
+    def __init__(self):
+        self.handle = vp()
+
+    def __enter__(self):
+        check(lib().lten_hip_graph_begin())
+        return self
+
+    def __exit__(self, exc_type, exc, tb):
+        rc = lib().lten_hip_graph_end(C.byref(self.handle))
+        if exc_type is None:
+            check(rc)
+        return False
+
+    def launch(self):
+        check(lib().lten_hip_graph_launch(self.handle))
+
+    def __del__(self):
+        try:
+            if self.handle:
+                lib().lten_hip_graph_destroy(self.handle)
         except Exception:
             pass
 

@@ -11,6 +11,12 @@ static thread_local char g_kernel[96] = "";
 static hipStream_t g_stream = nullptr;
 static int g_device = -1;
 
+// Graph capture: the stream the capture runs on (the caller's, or one made here when the library is on the
+// null stream, which cannot be captured) and the stream to go back to afterwards.
+static hipStream_t g_capture_stream = nullptr;
+static hipStream_t g_stream_before_capture = nullptr;
+static bool g_capturing = false;
+
 void set_error(const char* fmt, ...)
 {
 	va_list ap;
@@ -156,6 +162,65 @@ int lten_hip_set_option(const char* name, int value)
 		}
 	set_error("lten_hip_set_option: unknown option '%s'", name);
 	return 2;
+}
+
+int lten_hip_graph_begin(void)
+{
+	LTEN_HIP_REQUIRE(!g_capturing, "lten_hip_graph_begin: a capture is already open");
+	g_stream_before_capture = g_stream;
+	if (g_stream == nullptr) {
+		if (g_capture_stream == nullptr) LTEN_HIP_CHECK(hipStreamCreate(&g_capture_stream));
+		LTEN_HIP_CHECK(hipStreamSynchronize(nullptr));  // earlier work on the null stream comes first
+		g_stream = g_capture_stream;
+	}
+	hipError_t e = hipStreamBeginCapture(g_stream, hipStreamCaptureModeThreadLocal);
+	if (e != hipSuccess) {
+		g_stream = g_stream_before_capture;
+		set_error("lten_hip_graph_begin: %s", hipGetErrorString(e));
+		return 1;
+	}
+	g_capturing = true;
+	return 0;
+}
+
+int lten_hip_graph_end(void** graph)
+{
+	LTEN_HIP_REQUIRE(graph != nullptr, "lten_hip_graph_end: null pointer");
+	LTEN_HIP_REQUIRE(g_capturing, "lten_hip_graph_end: no capture is open");
+	*graph = nullptr;
+	hipGraph_t captured = nullptr;
+	const hipError_t e = hipStreamEndCapture(g_stream, &captured);
+	g_stream = g_stream_before_capture;
+	g_capturing = false;
+	if (e != hipSuccess || captured == nullptr) {
+		(void)hipGetLastError();
+		set_error("lten_hip_graph_end: the capture failed (%s); only compute entry points may run between begin and end",
+		          hipGetErrorString(e));
+		return 1;
+	}
+	hipGraphExec_t exec = nullptr;
+	const hipError_t ei = hipGraphInstantiate(&exec, captured, nullptr, nullptr, 0);
+	(void)hipGraphDestroy(captured);
+	if (ei != hipSuccess) {
+		set_error("lten_hip_graph_end: hipGraphInstantiate: %s", hipGetErrorString(ei));
+		return 1;
+	}
+	*graph = exec;
+	return 0;
+}
+
+int lten_hip_graph_launch(void* graph)
+{
+	LTEN_HIP_REQUIRE(graph != nullptr, "lten_hip_graph_launch: null graph");
+	LTEN_HIP_REQUIRE(!g_capturing, "lten_hip_graph_launch: a capture is open");
+	LTEN_HIP_CHECK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), stream()));
+	return 0;
+}
+
+int lten_hip_graph_destroy(void* graph)
+{
+	if (graph) LTEN_HIP_CHECK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+	return 0;
 }
 
 int lten_hip_event_create(void** event)

@@ -17,6 +17,8 @@ struct SProblem {
 	const float* B;
 	float* C;
 	const float* bias;  // optional, added per output column n (FullyConnected bias), or null
+	float* rowsum;      // optional: rowsum[m] += sum_k op(A)[m][k] (the FullyConnected bias gradient inside the
+	                    // weight-gradient product); only the 32x32 kernels do it, for a single problem
 	int64_t lda, ldb, ldc;
 	int64_t stride_a, stride_b, stride_c;  // per blockIdx.z
 	int M, N, K;
@@ -62,6 +64,24 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
 	});
 }
 
+// Row sums of op(A) from the 32x32 kernels: every lane (row lrow, k-half g) of every wavefront has added the
+// values it fed to the MFMAs; the 2 * WAVES shares of a row meet in LDS (scratch, at least 2 * WAVES * 32 floats
+// that nothing else uses any more) and are added in a fixed order into rowsum[m0 + row].
+template <int WAVES>
+__device__ __forceinline__ void add_row_sums(float* scratch, float asum, float* rowsum, int m0, int M)
+{
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	__syncthreads();
+	scratch[(wave * 2 + (lane >> 5)) * 32 + (lane & 31)] = asum;
+	__syncthreads();
+	if (tid < 32 && m0 + tid < M) {
+		float s = 0.0f;
+#pragma unroll
+		for (int i = 0; i < 2 * WAVES; i++) s += scratch[i * 32 + tid];
+		rowsum[m0 + tid] += s;
+	}
+}
+
 // Small outputs with a long K (the FullyConnected GEMMs at batch 128): one workgroup per 32x32 output tile,
 // its WAVES wavefronts each reduce an interleaved share of K with operands loaded straight from global
 // memory in the MFMA lane layout — no LDS staging, no barrier in the loop, loads unrolled ahead of their use —
@@ -88,6 +108,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 	v16f acc;
 #pragma unroll
 	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	float asum = 0.0f;  // this lane's share of row m of op(A)
 
 	// groups of 8 consecutive k, dealt round-robin to the wavefronts
 	const int groups = (p.K + 7) / 8;
@@ -115,6 +136,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 					if (k + t < p.K) b[t] = TB ? B[(int64_t)n * p.ldb + k + t] : B[(int64_t)(k + t) * p.ldb + n];
 			}
 		}
+		asum += (a[0] + a[1]) + (a[2] + a[3]);
 #pragma unroll
 		for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], b[t], acc, 0, 0, 0);
 	}
@@ -135,6 +157,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 		if (p.bias) out += p.bias[n0 + col];
 		*c = out;
 	}
+	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(&part[0][0], asum, p.rowsum, m0, p.M);
 }
 
 // The same decomposition with whole cache lines per load: the direct kernel above asks the texture addresser for 32
@@ -163,6 +186,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 	v16f acc;
 #pragma unroll
 	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	float asum = 0.0f;  // this lane's share of row m0 + lrow of op(A)
 
 	// one operand, one batch: four 16-byte loads per lane
 	auto fetch = [&](const float* base, int64_t ld, bool k_contig, int rows_limit, int row0, int k0, float4 (&v)[4]) {
@@ -227,6 +251,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 #pragma unroll
 					for (int t = 0; t < 4; t++) bb[t] = sB[(8 * q + 4 * g + t) * LD + lrow];
 				}
+				asum += (a[0] + a[1]) + (a[2] + a[3]);
 #pragma unroll
 				for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[t], bb[t], acc, 0, 0, 0);
 			}
@@ -250,6 +275,7 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 		if (p.bias) out += p.bias[n0 + col];
 		*c = out;
 	}
+	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(lds, asum, p.rowsum, m0, p.M);
 }
 
 static int launch_direct(const SProblem& p, int tA, int tB, uint64_t batch)
@@ -330,8 +356,9 @@ static int launch_sgemm(const SProblem& p, int tA, int tB, uint64_t batch, const
 
 int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
               int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
-              int64_t stride_c, uint64_t batch, const float* bias)
+              int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done)
 {
+	if (rowsum_done) *rowsum_done = false;
 	if (M == 0 || N == 0 || batch == 0) return 0;
 	LTEN_HIP_REQUIRE(C != nullptr, "sgemm: C is null");
 	LTEN_HIP_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "sgemm: null operand");
@@ -341,13 +368,13 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		// every problem writes the same C: run them one after another so the sum has one fixed order
 		for (uint64_t b = 0; b < batch; b++) {
 			int rc = sgemm_run(tA, tB, M, N, K, alpha, A + b * stride_a, lda, 0, B + b * stride_b, ldb, 0,
-			                   (b == 0) ? beta : 1.0f, C, ldc, 0, 1, bias && b == 0 ? bias : nullptr);
+			                   (b == 0) ? beta : 1.0f, C, ldc, 0, 1, bias && b == 0 ? bias : nullptr, nullptr, nullptr);
 			if (rc) return rc;
 		}
 		return 0;
 	}
 	SProblem p;
-	p.A = A; p.B = B; p.C = C; p.bias = bias;
+	p.A = A; p.B = B; p.C = C; p.bias = bias; p.rowsum = nullptr;
 	p.lda = (int64_t)lda; p.ldb = (int64_t)ldb; p.ldc = (int64_t)ldc;
 	p.stride_a = stride_a; p.stride_b = stride_b; p.stride_c = stride_c;
 	p.M = (int)M; p.N = (int)N; p.K = (int)K;
@@ -380,7 +407,12 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	case 1: return launch_sgemm<128, 128, 16, 2, 2>(p, tA, tB, batch, "sgemm_128x128x16");
 	case 2: return launch_sgemm<64, 64, 32, 2, 2>(p, tA, tB, batch, "sgemm_64x64x32");
 	case 3: return launch_sgemm<32, 32, 32, 1, 1>(p, tA, tB, batch, "sgemm_32x32x32");
-	default: return launch_direct(p, tA, tB, batch);
+	default:
+		if (rowsum != nullptr && rowsum_done != nullptr && batch == 1 && K != 0) {
+			p.rowsum = rowsum;
+			*rowsum_done = true;
+		}
+		return launch_direct(p, tA, tB, batch);
 	}
 }
 
@@ -393,21 +425,21 @@ extern "C" {
 int lten_hip_sgemm(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
                    const float* B, uint64_t ldb, float beta, float* C, uint64_t ldc)
 {
-	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, nullptr);
+	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, nullptr, nullptr, nullptr);
 }
 
 int lten_hip_sgemm_strided_batched(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A,
                                    uint64_t lda, int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b,
                                    float beta, float* C, uint64_t ldc, int64_t stride_c, uint64_t batch)
 {
-	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, batch, nullptr);
+	return sgemm_run(tA, tB, M, N, K, alpha, A, lda, stride_a, B, ldb, stride_b, beta, C, ldc, stride_c, batch, nullptr, nullptr, nullptr);
 }
 
 int lten_hip_fc_forward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* bias,
                             float* Y)
 {
 	// l-ten/fully_connected.cpp:150 (NT GEMM) and :165 (ones x bias, beta = 1) in one launch
-	return sgemm_run(0, 1, M, out, in, 1.0f, X, in, 0, W, in, 0, 0.0f, Y, out, 0, 1, bias);
+	return sgemm_run(0, 1, M, out, in, 1.0f, X, in, 0, W, in, 0, 0.0f, Y, out, 0, 1, bias, nullptr, nullptr);
 }
 
 int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
@@ -415,11 +447,13 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
 {
 	int rc = 0;
 	// l-ten/backprop.cpp:2228  dX[M x in] = dY[M x out] W[out x in]
-	if (dX) rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr);
-	// :2252  dW[out x in] = dY[M x out]^T X[M x in]
-	if (!rc && dW) rc = sgemm_run(1, 0, out, in, M, 1.0f, dY, out, 0, X, in, 0, 0.0f, dW, in, 0, 1, nullptr);
+	if (dX) rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr, nullptr, nullptr);
+	// :2252  dW[out x in] = dY[M x out]^T X[M x in].  The rows of dY^T summed over the batch are the bias gradient
+	// of :2267, so a kernel that can do it adds them into db on the way.
+	bool db_done = false;
+	if (!rc && dW) rc = sgemm_run(1, 0, out, in, M, 1.0f, dY, out, 0, X, in, 0, 0.0f, dW, in, 0, 1, nullptr, db, &db_done);
 	// :2267  db[1 x out] += ones[1 x M] dY[M x out]; the ones vector is never materialised: a = 1 for every k
-	if (!rc && db && M != 0 && out != 0) {
+	if (!rc && db && !db_done && M != 0 && out != 0) {
 		SProblem p = {};
 		p.A = nullptr;  // a[k] = 1
 		p.B = dY; p.C = db;

@@ -169,6 +169,34 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
                 assert np.abs(got - want).max() <= tol   # l-ten's own abs tolerance for fc_test
 
 
+@pytest.mark.parametrize("M,fin,fout,kernels", [
+    (128, 200, 75, ("sgemm_direct_32x32_w8",)),                      # bias gradient inside the direct kernel
+    (37, 33, 10, ("sgemm_direct_32x32_w8",)),                        # ragged in every dimension
+    (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: the staged kernel, ragged K
+    (1024, 1100, 1000, ("sgemm_rowvec",)),                           # many tiles: tiled GEMM, then the column-sum kernel
+])
+def test_fc_backward_bias_gradient_accumulates_on_every_route(gpu, M, fin, fout, kernels):
+    """db += column sums of dY (l-ten/backprop.cpp:2267, beta = 1) whichever kernel computes dW: integer-valued
+    inputs make the sums exact in any order, so db must equal its start value plus the sum, bit for bit."""
+    rng = np.random.default_rng(M + fin)
+    x = rng.integers(-3, 4, (M, fin)).astype(np.float32)
+    w = rng.integers(-3, 4, (fout, fin)).astype(np.float32)
+    dy = rng.integers(-4, 5, (M, fout)).astype(np.float32)
+    db0 = rng.integers(-50, 50, fout).astype(np.float32)
+    D = gpu.DeviceBuffer
+    dX, dW, dDY, dDB = D.from_numpy(x), D.from_numpy(w), D.from_numpy(dy), D.from_numpy(db0)
+    dDX, dDW = D(x.nbytes), D(w.nbytes)
+    gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, dDX.ptr, dDW.ptr, dDB.ptr))
+    assert gpu.last_kernel() in kernels
+    assert np.array_equal(dDB.numpy(np.float32, (fout,)), db0 + dy.sum(axis=0))
+    assert np.array_equal(dDW.numpy(np.float32, w.shape), dy.T @ x)
+    assert np.array_equal(dDX.numpy(np.float32, x.shape), dy @ w)
+    # without dW the column-sum kernel still serves db
+    dDB2 = D.from_numpy(db0)
+    gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, None, None, dDB2.ptr))
+    assert np.array_equal(dDB2.numpy(np.float32, (fout,)), db0 + dy.sum(axis=0))
+
+
 def test_lten_matmul_test_vectors(gpu):
     """tests/unit_tests.cpp matmul_test through the strided-batched entry point: exact values."""
     v = json.load(open(golden_path("lten_unit_test_vectors.json")))["matmul_test"]

@@ -166,3 +166,58 @@ def test_optimizer_steps(gpu, ob):
             assert np.array_equal(got, g[name + "_w"]), name
         else:
             assert np.abs(got - g[name + "_w"]).max() < 1e-6 * max(1.0, np.abs(g[name + "_w"]).max()), name
+
+
+def test_recorded_step_replays_like_the_eager_step(gpu):
+    """Two FullyConnected layers with relu, forward and backward, recorded once and replayed four times with new
+    inputs, eager work and synchronisation between the replays: every replay must equal the eager calls bit for bit
+    (same kernels, same order)."""
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    rng = np.random.default_rng(77)
+    B, n0, n1, n2 = 64, 200, 320, 48
+    W1, b1 = rng.standard_normal((n1, n0)).astype(np.float32) * 0.1, rng.standard_normal(n1).astype(np.float32)
+    W2, b2 = rng.standard_normal((n2, n1)).astype(np.float32) * 0.1, rng.standard_normal(n2).astype(np.float32)
+    dW1, db1, dW2, db2 = D.from_numpy(W1), D.from_numpy(b1), D.from_numpy(W2), D.from_numpy(b2)
+    x, h, a, y = D(4 * B * n0), D(4 * B * n1), D(4 * B * n1), D(4 * B * n2)
+    gy, ga, gh, gx = D(4 * B * n2), D(4 * B * n1), D(4 * B * n1), D(4 * B * n0)
+    gW1, gb1, gW2, gb2 = D(W1.nbytes), D(b1.nbytes), D(W2.nbytes), D(b2.nbytes)
+    outs = [(y, (B, n2)), (gx, (B, n0)), (gW1, W1.shape), (gb1, b1.shape), (gW2, W2.shape), (gb2, b2.shape)]
+
+    def step():
+        gpu.check(l.lten_hip_fill_f32(gb1.ptr, n1, 0.0))
+        gpu.check(l.lten_hip_fill_f32(gb2.ptr, n2, 0.0))
+        gpu.check(l.lten_hip_fc_forward_f32(B, n0, n1, x.ptr, dW1.ptr, db1.ptr, h.ptr))
+        gpu.check(l.lten_hip_relu_f32(a.ptr, h.ptr, B * n1))
+        gpu.check(l.lten_hip_fc_forward_f32(B, n1, n2, a.ptr, dW2.ptr, db2.ptr, y.ptr))
+        gpu.check(l.lten_hip_fc_backward_f32(B, n1, n2, a.ptr, dW2.ptr, gy.ptr, ga.ptr, gW2.ptr, gb2.ptr))
+        gpu.check(l.lten_hip_relu_backward_f32(gh.ptr, ga.ptr, h.ptr, B * n1))
+        gpu.check(l.lten_hip_fc_backward_f32(B, n0, n1, x.ptr, dW1.ptr, gh.ptr, gx.ptr, gW1.ptr, gb1.ptr))
+
+    def load_inputs(seed):
+        r = np.random.default_rng(seed)
+        x.upload(r.standard_normal((B, n0)).astype(np.float32))
+        gy.upload(r.standard_normal((B, n2)).astype(np.float32))
+
+    def read():
+        return [buf.numpy(np.float32, shape).copy() for buf, shape in outs]
+
+    load_inputs(0)
+    step()
+    with gpu.Graph() as graph:
+        step()
+    for replay in range(4):
+        load_inputs(100 + replay)
+        step()
+        want = read()
+        for buf, shape in outs:  # eager work between the replays: wipe what the replay has to rewrite
+            gpu.check(l.lten_hip_fill_f32(buf.ptr, int(np.prod(shape)), -7.0))
+        gpu.sync()
+        graph.launch()
+        got = read()
+        for w, g_ in zip(want, got):
+            assert np.array_equal(w, g_), replay
+    # misuse is reported, not recorded
+    assert l.lten_hip_graph_launch(None) != 0
+    import ctypes
+    p = ctypes.c_void_p()
+    assert l.lten_hip_graph_end(ctypes.byref(p)) != 0 and b"no capture" in l.lten_hip_last_error()
