@@ -19,23 +19,9 @@
 // written in whole 256-byte rows.
 #include "common.h"
 #include "qgemm_common.h"
+#include "lds_async.h"
 
 namespace lten_hip {
-
-// One wave-wide 16-byte-per-lane load straight into LDS: lane L's bytes go to lds_addr + 16*L.
-// lds_addr and base are wave-uniform; voff is the lane's byte offset from base.
-__device__ __forceinline__ void async_load16(uint32_t lds_addr, const uint8_t* base, uint32_t voff)
-{
-	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
-}
-
-// s_waitcnt vmcnt(n) only (expcnt and lgkmcnt fields left at "no wait"); n < 64.
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-	static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
-	__builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
 
 // Phase timestamps for tuning builds (-DLTEN_HIP_STAMPS): slots 0..3 = start, main loop start, main loop
 // end, end in the 100 MHz wall clock; slots 4..5 = start / main loop end in shader clocks.

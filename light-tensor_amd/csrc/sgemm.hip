@@ -7,23 +7,12 @@
 // rank-1 bias update, M == 1 column sum) and the dispatch.
 #include "common.h"
 #include "gemm_f32_core.h"
+#include "sgemm_common.h"
 
 #include <algorithm>
 
 namespace lten_hip {
 
-struct SProblem {
-	const float* A;
-	const float* B;
-	float* C;
-	const float* bias;  // optional, added per output column n (FullyConnected bias), or null
-	float* rowsum;      // optional: rowsum[m] += sum_k op(A)[m][k] (the FullyConnected bias gradient inside the
-	                    // weight-gradient product); only the 32x32 kernels do it, for a single problem
-	int64_t lda, ldb, ldc;
-	int64_t stride_a, stride_b, stride_c;  // per blockIdx.z
-	int M, N, K;
-	float alpha, beta;
-};
 
 template <int BM, int BN, int BK, int WM, int WN, bool TA, bool TB>
 __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
@@ -278,11 +267,17 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(lds, asum, p.rowsum, m0, p.M);
 }
 
+// Both operands allow 16-byte loads along their contiguous dimension.
+static bool operands_vec(const SProblem& p)
+{
+	return (p.lda & 3) == 0 && (p.ldb & 3) == 0 && (p.stride_a & 3) == 0 && (p.stride_b & 3) == 0 &&
+	       ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
+}
+
 static int launch_direct(const SProblem& p, int tA, int tB, uint64_t batch)
 {
 	const dim3 grid((unsigned)(ceil_div(p.M, 32) * ceil_div(p.N, 32)), 1, (unsigned)batch), block(8 * 64);
-	const bool vec = (p.lda & 3) == 0 && (p.ldb & 3) == 0 && (p.stride_a & 3) == 0 && (p.stride_b & 3) == 0 &&
-	                 ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0;
+	const bool vec = operands_vec(p);
 	if (vec && p.K >= 512 && get_option(OPT_SGEMM_TILE) != 5) {  // at least two batches per wavefront
 		set_kernel_name("sgemm_staged_32x32_w8");
 		if (!tA && !tB) sgemm_staged_kernel<8, false, false><<<grid, block, 0, stream()>>>(p);
@@ -396,11 +391,31 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	const uint64_t tiles64 = ceil_div(M, 64) * ceil_div(N, 64) * batch;
 	const uint64_t tiles128 = ceil_div(M, 128) * ceil_div(N, 128) * batch;
 	int choice = force;
+	if (choice >= 10) {  // a direct-to-LDS tile by number; falls through to the heuristic when the problem does not fit
+		if (sgemm_fast_dispatch(p, tA, tB, batch, choice) == 0) return 0;
+		choice = 0;
+	}
+	if (choice == 0 && tiles128 >= 128 && K >= 256) {
+		// large problems: 256 x 256 tiles when they fill the chip, else 128 x 128.  The tiles walk K in steps of 32:
+		// what is left over is added by a second, general launch (beta = 1, no bias).
+		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192;
+		const uint64_t k_main = K & ~31ull;
+		p.K = (int)k_main;
+		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : 21) == 0) {
+			if (k_main == K) return 0;
+			return sgemm_run(tA, tB, M, N, K - k_main, alpha, A + (tA ? k_main * lda : k_main), lda, stride_a,
+			                 B + (tB ? k_main : k_main * ldb), ldb, stride_b, 1.0f, C, ldc, stride_c, batch, nullptr, nullptr, nullptr);
+		}
+		p.K = (int)K;
+	}
 	if (choice == 0) {
 		// Few output tiles and a long K: the LDS-tiled kernels would leave most CUs idle while a handful of
 		// workgroups walk K in sequence; the direct kernel cuts K across the wavefronts of a workgroup instead.
+		// With 16-byte loads the 32x32 kernels stay ahead of the LDS-tiled ones at every size measured (1280^3: 58 vs
+		// 40 TFLOP/s, 4000^3 with K a multiple of 4: 74 vs 63, 3000 x 3000 x 300: 65 vs 44); without them only while
+		// the tiles are few (4095^3: 25 vs 66).
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32) * batch;
-		if (tiles32 <= 1024) choice = 4;
+		if (tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20))) choice = 4;
 		else choice = tiles128 >= 128 ? 1 : 2;
 	}
 	switch (choice) {

@@ -173,7 +173,8 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     (128, 200, 75, ("sgemm_direct_32x32_w8",)),                      # bias gradient inside the direct kernel
     (37, 33, 10, ("sgemm_direct_32x32_w8",)),                        # ragged in every dimension
     (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: the staged kernel, ragged K
-    (1024, 1100, 1000, ("sgemm_rowvec",)),                           # many tiles: tiled GEMM, then the column-sum kernel
+    (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
+    (640, 1101, 999, ("sgemm_rowvec",)),                             # unaligned rows, many tiles: LDS-tiled GEMM, then the column sum
 ])
 def test_fc_backward_bias_gradient_accumulates_on_every_route(gpu, M, fin, fout, kernels):
     """db += column sums of dY (l-ten/backprop.cpp:2267, beta = 1) whichever kernel computes dW: integer-valued
@@ -235,3 +236,98 @@ def test_large_gemm_linearity_property(gpu):
     rows = rng.integers(0, n, 64)
     want = R[rows].astype(np.float64) @ S.astype(np.float64).T
     assert rel_err(got[rows], want) < TOL
+
+
+FAST_TILES = {11: "sgemm_fast_256x256x32_w2x4_s2", 12: "sgemm_fast_256x256x32_w4x2_s2", 21: "sgemm_fast_128x128x32_w2x2_s2",
+              22: "sgemm_fast_128x128x32_w2x2_s3", 23: "sgemm_fast_128x128x32_w2x2_s4"}
+
+
+@pytest.mark.parametrize("tile", sorted(FAST_TILES))
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_direct_to_lds_tiles_exact_all_layouts(gpu, tile, tA, tB):
+    """The direct-to-LDS tiles by number: integer-valued operands make every summation order exact, so the result
+    must equal the int64 product bit for bit, with padded leading dimensions, alpha / beta and an untouched pad."""
+    rng = np.random.default_rng(500 + 10 * tile + 2 * tA + tB)
+    M, N, K = (512, 256, 160) if tile < 20 else (256, 384, 96)   # K / 32 = 5 or 3 k-steps: prologue, steady state, drain
+    A = rng.integers(-8, 9, (M, K)).astype(np.float32)
+    B = rng.integers(-8, 9, (K, N)).astype(np.float32)
+    want = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    lda, ldb, ldc = (M if tA else K) + 4, (K if tB else N) + 8, N + 3
+    As = np.zeros(((K if tA else M), lda), np.float32)
+    As[:, :(M if tA else K)] = A.T if tA else A
+    Bs = np.zeros(((N if tB else K), ldb), np.float32)
+    Bs[:, :(K if tB else N)] = B.T if tB else B
+    C0 = np.full((M, ldc), 7.0, np.float32)
+    got = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, C0, ldc, tile)
+    assert gpu.last_kernel() == FAST_TILES[tile]
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, tA, tB, M, N, K, 2.0, As, lda, Bs, ldb, -1.0, got, ldc, tile)
+    assert np.array_equal(got2[:, :N], want)
+
+
+def test_direct_to_lds_tiles_are_the_default_for_large_aligned_problems(gpu):
+    """Heuristic, long K (many trips round the stage ring), FullyConnected bias, and a strided batch; an unaligned
+    operand must fall back to the general kernels and still be right."""
+    rng = np.random.default_rng(9)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    M, fin, fout = 4096, 1024, 4096
+    x = rng.integers(-4, 5, (M, fin)).astype(np.float32)
+    w = rng.integers(-4, 5, (fout, fin)).astype(np.float32)
+    b = rng.integers(-9, 10, fout).astype(np.float32)
+    dX, dW, dB, dY = D.from_numpy(x), D.from_numpy(w), D.from_numpy(b), D(4 * M * fout)
+    gpu.check(l.lten_hip_fc_forward_f32(M, fin, fout, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel() == FAST_TILES[12]
+    assert np.array_equal(dY.numpy(np.float32, (M, fout)), x @ w.T + b)
+    # 2048 x 1024 output: too few 256-tiles, so 128-tiles
+    gpu.check(l.lten_hip_fc_forward_f32(2048, fin, 1024, dX.ptr, dW.ptr, None, dY.ptr))
+    assert gpu.last_kernel() == FAST_TILES[21]
+    assert np.array_equal(dY.numpy(np.float32, (2048, 1024)), x[:2048] @ w[:1024].T)
+    # strided batch of 4 (Tensor::matmul over a leading dimension), NN
+    a4 = rng.integers(-4, 5, (4, 512, 256)).astype(np.float32)   # 4 x (4 x 8) tiles of 128
+    b4 = rng.integers(-4, 5, (4, 256, 1024)).astype(np.float32)
+    dA4, dB4, dC4 = D.from_numpy(a4), D.from_numpy(b4), D(4 * 4 * 512 * 1024)
+    gpu.check(l.lten_hip_sgemm_strided_batched(0, 0, 512, 1024, 256, 1.0, dA4.ptr, 256, 512 * 256, dB4.ptr, 1024, 256 * 1024, 0.0,
+                                               dC4.ptr, 1024, 512 * 1024, 4))
+    assert gpu.last_kernel() == FAST_TILES[21]
+    assert np.array_equal(dC4.numpy(np.float32, (4, 512, 1024)), a4 @ b4)
+    # an operand base that is not 16-byte aligned: general kernel
+    dXo = D(x.nbytes + 16)
+    dXo.upload(x, offset=4)
+    gpu.check(l.lten_hip_fc_forward_f32(M, fin, fout, dXo.ptr + 4, dW.ptr, dB.ptr, dY.ptr))
+    assert not gpu.last_kernel().startswith("sgemm_fast")
+    assert np.array_equal(dY.numpy(np.float32, (M, fout)), x @ w.T + b)
+    # ragged M: still the tiles (edge rows are fetched twice and not stored)
+    gpu.check(l.lten_hip_fc_forward_f32(M - 1, fin, fout, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel() == FAST_TILES[12]
+    assert np.array_equal(dY.numpy(np.float32, (M - 1, fout)), x[:-1] @ w.T + b)
+
+
+@pytest.mark.parametrize("tA,tB,M,N,K", [(0, 1, 1999, 2001, 1000), (0, 0, 1501, 2004, 488), (1, 0, 2000, 1532, 520),
+                                         (1, 1, 1796, 1801, 1032), (0, 1, 129, 16385, 256)])
+def test_direct_to_lds_tiles_ragged_sizes(gpu, tA, tB, M, N, K):
+    """Sizes that are no multiple of the tile or of the k-step: edge tiles fetch an existing row twice and store only
+    what exists; the k remainder is added by a second launch.  Exact on integer-valued data, pad columns untouched."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    want = A @ B   # exact: |sum| < 2^24
+    lda, ldb, ldc = (M if tA else K), (K if tB else N), N + 1
+    As = np.ascontiguousarray(A.T if tA else A)
+    Bs = np.ascontiguousarray(B.T if tB else B)
+    C0 = np.full((M, ldc), 3.0, np.float32)
+    D = gpu.DeviceBuffer
+    dA, dB, dC = D.from_numpy(As), D.from_numpy(Bs), D.from_numpy(C0)
+    gpu.sgemm(tA, tB, M, N, K, 1.0, dA, lda, dB, ldb, 0.0, dC, ldc)
+    first = gpu.last_kernel()
+    got = dC.numpy(np.float32, C0.shape)
+    assert np.array_equal(got[:, :N], want), first
+    assert (got[:, N:] == 3.0).all()
+    gpu.set_option("sgemm_tile", 21)
+    try:
+        gpu.sgemm(tA, tB, M, N, K & ~31, 0.5, dA, lda, dB, ldb, 2.0, dC, ldc)
+        assert gpu.last_kernel() == FAST_TILES[21]
+    finally:
+        gpu.set_option("sgemm_tile", 0)
+    Am, Bm = A[:, :K & ~31], B[:K & ~31]
+    assert np.array_equal(dC.numpy(np.float32, C0.shape)[:, :N], 0.5 * (Am @ Bm) + 2.0 * want)
