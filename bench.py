@@ -276,6 +276,37 @@ def extra_configs(lt, wl, with_cpu):
         rec.update(cpu_ms=round(t * 1e3, 3), cpu_cores=1, cpu_kind="reference" if ob.ref() is not None else "port",
                    speedup=round(t * 1e3 / ms, 1))
     out.append(rec)
+
+    # ---- beyond the five configs: a large fp32 product in the three layouts l-ten's layers use (FullyConnected forward
+    # NT, data gradient NN, weight gradient TN), synthetic N(0,1) operands
+    n = 4096
+    ga = D.from_numpy(np.random.default_rng(11).standard_normal((n, n)).astype(np.float32))
+    gb = D.from_numpy(np.random.default_rng(12).standard_normal((n, n)).astype(np.float32))
+    gc = D(4 * n * n)
+    per_layout = {}
+    for name, (ta, tb) in (("NT", (0, 1)), ("NN", (0, 0)), ("TN", (1, 0))):
+        ms = timed(lt, lambda: lt.sgemm(ta, tb, n, n, n, 1.0, ga, n, gb, n, 0.0, gc, n), 10)
+        per_layout[name] = round(ms * 1e3, 1)
+    kname = lt.last_kernel()
+    ms = sum(per_layout.values()) / 3e3
+    tf = 2.0 * n ** 3 / ms / 1e9
+    out.append({"config": "fp32 sgemm 4096^3 (Tensor::matmul / FullyConnected at scale), mean of NT, NN, TN", "gpu_us": round(ms * 1e3, 1),
+                "per_layout_us": per_layout, "kernel": kname,
+                "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                             "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)}})
+    del ga, gb, gc
+
+    # ---- beyond the five configs: one GRU time step's two M = 1 products (l-ten/gru.cpp:267-268), input = hidden = 1024
+    hid = 1024
+    gx = D.from_numpy(np.random.default_rng(13).standard_normal(hid).astype(np.float32))
+    gu = D.from_numpy(np.random.default_rng(14).standard_normal((hid, 3 * hid)).astype(np.float32))
+    gy = D(4 * 3 * hid)
+    ms = timed(lt, lambda: lt.sgemm(0, 0, 1, 3 * hid, hid, 1.0, gx, hid, gu, 3 * hid, 0.0, gy, 3 * hid), 100)
+    nbytes = 4 * (hid + hid * 3 * hid + 3 * hid)
+    out.append({"config": "GRU step product 1 x 1024 times 1024 x 3072 (fp32, M = 1)", "gpu_us": round(ms * 1e3, 2), "kernel": lt.last_kernel(),
+                "algorithmic_bytes": nbytes,
+                "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}})
     return out
 
 

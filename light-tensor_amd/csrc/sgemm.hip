@@ -312,27 +312,52 @@ __global__ __launch_bounds__(256) void sgemm_rank1_kernel(SProblem p, int tA, in
 }
 
 // M == 1 with B not transposed: c[n] = alpha * sum_k a[k] B[k][n] + beta * c[n] — the column sum that
-// l-ten uses for the bias gradient with a = ones (l-ten/backprop.cpp:2267).  256 threads = 64 columns x
-// 4 k-slices; the slices are combined in a fixed order.  A null A stands for a vector of ones, so the
-// bias_multiplier tensor of l-ten's FullyConnected is never needed on the device.
-__global__ __launch_bounds__(256) void sgemm_rowvec_kernel(SProblem p, int tA)
+// l-ten uses for the bias gradient with a = ones (l-ten/backprop.cpp:2267) and the two products of a GRU time
+// step (l-ten/gru.cpp:267-268).  A workgroup takes COLS columns and cuts K into SLICES slices, one thread per
+// (column, slice) with eight loads in flight; the slices are combined in slice order.  A null A stands for a
+// vector of ones, so the bias_multiplier tensor of l-ten's FullyConnected is never needed on the device.
+// Two shapes: 64 columns x 4 slices when the columns alone give every CU a workgroup, else 16 x 64 (rows
+// are then read in 64-byte pieces, but four times as many workgroups share a long K).
+template <int COLS, int SLICES>
+__global__ __launch_bounds__(COLS* SLICES) void sgemm_rowvec_kernel(SProblem p, int tA)
 {
-	__shared__ float part[4][64];
-	const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-	const int n = blockIdx.x * 64 + tx;
+	__shared__ float part[SLICES][COLS];
+	const int tx = threadIdx.x % COLS, ty = threadIdx.x / COLS;
+	const int n = blockIdx.x * COLS + tx;
 	float s = 0.0f;
-	if (n < p.N)
-		for (int k = ty; k < p.K; k += 4) {
-			const float a = p.A == nullptr ? 1.0f : (tA ? p.A[(int64_t)k * p.lda] : p.A[k]);
-			s = fmaf(a, p.B[(int64_t)k * p.ldb + n], s);
+	if (n < p.N) {
+		auto a_at = [&](int k) { return p.A == nullptr ? 1.0f : (tA ? p.A[(int64_t)k * p.lda] : p.A[k]); };
+		const float* bcol = p.B + n;
+		int k = ty;
+		for (; k + 7 * SLICES < p.K; k += 8 * SLICES) {
+			float bv[8], av[8];
+#pragma unroll
+			for (int u = 0; u < 8; u++) {
+				bv[u] = bcol[(int64_t)(k + u * SLICES) * p.ldb];
+				av[u] = a_at(k + u * SLICES);
+			}
+#pragma unroll
+			for (int u = 0; u < 8; u++) s = fmaf(av[u], bv[u], s);
 		}
+		for (; k < p.K; k += SLICES) s = fmaf(a_at(k), bcol[(int64_t)k * p.ldb], s);
+	}
 	part[ty][tx] = s;
 	__syncthreads();
 	if (ty == 0 && n < p.N) {
-		float v = p.alpha * (((part[0][tx] + part[1][tx]) + part[2][tx]) + part[3][tx]);
+		float v = part[0][tx];
+#pragma unroll
+		for (int q = 1; q < SLICES; q++) v += part[q][tx];
+		v *= p.alpha;
 		if (p.beta != 0.0f) v += p.beta * p.C[n];
 		p.C[n] = v;
 	}
+}
+
+static void launch_rowvec(const SProblem& p, int tA)
+{
+	set_kernel_name("sgemm_rowvec");
+	if (ceil_div(p.N, 64) >= 256 || p.K < 128) sgemm_rowvec_kernel<64, 4><<<dim3((unsigned)ceil_div(p.N, 64)), dim3(256), 0, stream()>>>(p, tA);
+	else sgemm_rowvec_kernel<16, 64><<<dim3((unsigned)ceil_div(p.N, 16)), dim3(1024), 0, stream()>>>(p, tA);
 }
 
 template <int BM, int BN, int BK, int WM, int WN>
@@ -383,8 +408,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		return 0;
 	}
 	if (force == 0 && batch == 1 && bias == nullptr && M == 1 && !tB) {
-		set_kernel_name("sgemm_rowvec");
-		sgemm_rowvec_kernel<<<dim3((unsigned)ceil_div(N, 64)), dim3(256), 0, stream()>>>(p, tA);
+		launch_rowvec(p, tA);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}
@@ -475,8 +499,7 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
 		p.ldb = (int64_t)out; p.ldc = (int64_t)out;
 		p.M = 1; p.N = (int)out; p.K = (int)M;
 		p.alpha = 1.0f; p.beta = 1.0f;
-		set_kernel_name("sgemm_rowvec");
-		sgemm_rowvec_kernel<<<dim3((unsigned)ceil_div(out, 64)), dim3(256), 0, stream()>>>(p, 0);
+		launch_rowvec(p, 0);
 		LTEN_HIP_LAUNCH_CHECK();
 	}
 	return rc;
