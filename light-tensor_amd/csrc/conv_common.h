@@ -15,6 +15,9 @@ struct ConvGeo {
 // *_takes: whether the kernel family covers this geometry and these pointers.
 bool conv_patch_forward_takes(const ConvGeo& g, const float* x, const float* y);
 int conv_patch_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y);
+// the same tile with the LDS patch filled by direct global->LDS loads (conv_patch_fast.hip)
+bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float* w);
+int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y);
 bool conv_patch_wgrad_takes(const ConvGeo& g);
 int conv_patch_wgrad_parts(const ConvGeo& g);  // partial [Cout x Cin*kh*kw] matrices the kernel writes
 int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts);

@@ -215,9 +215,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	const int begin = blockIdx.x * chunks_per_part, end = min(total, begin + chunks_per_part);
 
 	float4 rdy[P::DY_PER_T], rp[P::P_PER_T];
-	auto load_chunk = [&](int chunk) {
-		const int wt = chunk % tiles_w, ho = (chunk / tiles_w) % g.Ho, n = chunk / (tiles_w * g.Ho);
-		const int w0 = wt * P::TW;
+	// What does not change from chunk to chunk is worked out once per lane: the offset of each of its float4s from
+	// the chunk's origin, and the row / column shifts that decide whether the float4 lies inside the image (with
+	// VEC, rows are whole float4s: inside or outside together).  Chunk coordinates advance without divisions.
+	int n_c = begin / (tiles_w * g.Ho), ho_c = (begin / tiles_w) % g.Ho, w0_c = (begin % tiles_w) * P::TW;
+	const int64_t plane_o = (int64_t)g.Ho * g.Wo;
+	const int dy_rel = (int)((tid / (P::TW / 4)) * plane_o) + 4 * (tid % (P::TW / 4));  // + q * 16 rows of dy
+	int x_rel[P::P_PER_T], x_gy[P::P_PER_T], x_gx[P::P_PER_T];
+#pragma unroll
+	for (int q = 0; q < P::P_PER_T; q++) {
+		const int idx = tid + q * P::T;
+		const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
+		const int r = rowid % KH, ci = rowid / KH;
+		const bool exists = idx < P::PATCH_F4 && ci0 + ci < g.Cin;
+		x_gx[q] = 4 * f - 4;
+		x_gy[q] = exists ? r - g.ph : -(1 << 30);
+		x_rel[q] = exists ? (ci * g.H + r - g.ph) * g.W + x_gx[q] : 0;
+	}
+	auto load_chunk = [&]() {  // the chunk at (n_c, ho_c, w0_c)
+		if (VEC) {
+			const float* dyc = dy + (((int64_t)n_c * g.Cout + co0) * g.Ho + ho_c) * g.Wo + w0_c;
+			const float* xc = x + (((int64_t)n_c * g.Cin + ci0) * g.H + ho_c) * g.W + w0_c;
+			const bool dy_col = w0_c + 4 * (tid % (P::TW / 4)) < g.Wo;
+#pragma unroll
+			for (int q = 0; q < P::DY_PER_T; q++) {
+				rdy[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+				if (dy_col && co0 + tid / (P::TW / 4) + q * (P::T / (P::TW / 4)) < g.Cout)
+					rdy[q] = *reinterpret_cast<const float4*>(dyc + dy_rel + q * (P::T / (P::TW / 4)) * plane_o);
+			}
+#pragma unroll
+			for (int q = 0; q < P::P_PER_T; q++) {
+				rp[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+				if ((unsigned)(ho_c + x_gy[q]) < (unsigned)g.H && (unsigned)(w0_c + x_gx[q]) < (unsigned)g.W)
+					rp[q] = *reinterpret_cast<const float4*>(xc + x_rel[q]);
+			}
+			return;
+		}
+		const int ho = ho_c, n = n_c, w0 = w0_c;
 #pragma unroll
 		for (int q = 0; q < P::DY_PER_T; q++) {
 			const int idx = tid + q * P::T;
@@ -236,6 +270,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 			if (idx < P::PATCH_F4 && ci0 + ci < g.Cin && gy >= 0 && gy < g.H)
 				v = load_row4<VEC>(x + (((int64_t)n * g.Cin + ci0 + ci) * g.H + gy) * g.W, w0 - 4 + 4 * f, g.W);
 			rp[q] = v;
+		}
+	};
+	auto next_chunk = [&]() {
+		w0_c += P::TW;
+		if (w0_c >= g.Wo) {
+			w0_c = 0;
+			if (++ho_c == g.Ho) { ho_c = 0; n_c++; }
 		}
 	};
 	auto store_chunk = [&]() {
@@ -263,11 +304,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	const float* pa = s_dy + (mt * 32 + lrow) * P::DYS + phalf * (P::TW / 2) + half;
 	const float* pb = s_patch + lrow * P::CS + phalf * (P::TW / 2) + half + 4 - g.pw;
 
-	if (begin < end) load_chunk(begin);
+	if (begin < end) load_chunk();
 	for (int chunk = begin; chunk < end; chunk++) {
 		store_chunk();
 		__syncthreads();
-		if (chunk + 1 < end) load_chunk(chunk + 1);
+		next_chunk();
+		if (chunk + 1 < end) load_chunk();
 		// operands of step s + 1 are read while the MFMAs of step s issue
 		float fa[2], fb[2][P::TAPS];
 		auto read_operand = [&](int s, int t) { fb[s & 1][t] = pb[(t / KW) * P::PWS + (t % KW) + 2 * s]; };
@@ -403,7 +445,8 @@ int conv_patch_forward(const ConvGeo& g, const float* x, const float* w, const f
 bool conv_patch_wgrad_takes(const ConvGeo& g)
 {
 	return patch_geometry(g) && g.Cin >= 9 && ceil_div((uint64_t)g.Cout, 64) < 65536 && ceil_div((uint64_t)g.Cin, 32) < 65536 &&
-	       (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, 64) < (1ull << 31);
+	       (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, 64) < (1ull << 31) &&
+	       (uint64_t)g.H * g.W < (1u << 25) && (uint64_t)g.Ho * g.Wo < (1u << 25);  // 32-bit lane offsets over 32 channels
 }
 
 int conv_patch_wgrad_parts(const ConvGeo& g)

@@ -1,0 +1,240 @@
+// Conv2d forward, 3x3, stride 1, with the LDS patch filled by direct global->LDS loads.
+//
+// The same tile and the same MFMA schedule as conv2d_patch_forward_kernel (a workgroup = BM output channels x
+// 4 rows x 128 columns of one image, wavefront `wave` owns row `wave`, input channels in chunks of four, step
+// (cp, i, j) multiplies tap (i, j) of channels 2cp (lanes 0-31) and 2cp + 1 (lanes 32-63)), but a chunk reaches
+// LDS without passing through registers: two LDS stages, chunk c + 1 lands in one while chunk c is multiplied
+// from the other, one barrier per chunk.
+//
+// A stage holds the patch [4 channels][6 rows][136 columns] (column q = input column w0 - 4 + q) and the weights
+// [BM channels][36] exactly as they lie in memory, so both are filled by wave-wide loads whose lane L writes 16
+// bytes at 16 L: patch float4 number idx is (channel idx / 204, row (idx / 34) % 6, columns 4 (idx % 34) ..);
+// weight float4 number idx is (channel idx / 9, floats 4 (idx % 9) ..).  Whether a float4 lies inside the image
+// (or names an existing output channel) does not depend on the chunk: lanes whose float4 does not exist never
+// load, and their LDS slots keep the zeros written once before the first chunk.  That is the zero padding.
+//
+// Needs Cin % 4 == 0 (whole chunks, 16-byte aligned weight rows), W % 4 == 0 and 16-byte aligned x and w.
+#include "conv_common.h"
+#include "gemm_f32_core.h"
+#include "lds_async.h"
+
+namespace lten_hip {
+
+namespace {
+
+template <int BM_>
+struct FastFwd {
+	static constexpr int BM = BM_, MT = BM / 32, NT = 4, CB = 4, TH = 4, TW = 128, PR = TH + 2, PWS = 136, F4R = 34;
+	static constexpr int PATCH_F4 = CB * PR * F4R;                 // 816
+	static constexpr int PATCH_LOADS = (PATCH_F4 + 63) / 64;       // 13
+	static constexpr int PATCH_BYTES = PATCH_LOADS * 1024;
+	static constexpr int W_F4 = BM * 9;                            // 36 floats per channel
+	static constexpr int W_LOADS = (W_F4 + 63) / 64;
+	static constexpr int W_BYTES = W_LOADS * 1024;
+	static constexpr int STAGE = PATCH_BYTES + W_BYTES;
+	static constexpr int LOADS = PATCH_LOADS + W_LOADS;
+	static constexpr int LPW = (LOADS + 3) / 4;                    // per wavefront, the last ones may not exist
+	static constexpr int STEPS = (CB / 2) * 9;                     // 18 MFMA steps per chunk
+	static constexpr int NR = MT + NT, NM = MT * NT;
+};
+
+}  // namespace
+
+template <int BM>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 2 : 4, BM == 64 ? 2 : 4))) void conv2d_patch_fast_forward_kernel(
+    ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
+{
+	typedef FastFwd<BM> P;
+	__shared__ __attribute__((aligned(1024))) uint8_t smem[2 * P::STAGE];
+
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int lrow = lane & 31, half = lane >> 5;
+	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
+	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
+	const int co0 = blockIdx.y * BM, n = blockIdx.z;
+	const int Kc = g.Cin * 9;
+	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+	const float* wb = w + (int64_t)co0 * Kc;
+
+	// ---- what this lane fetches for each of its wavefront's loads (load q = wave + 4 i)
+	uint32_t voff[P::LPW], slot[P::LPW];
+	bool valid[P::LPW];
+	const uint32_t smem_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+#pragma unroll
+	for (int i = 0; i < P::LPW; i++) {
+		const int q = wave + 4 * i;
+		valid[i] = false;
+		voff[i] = 0;
+		slot[i] = smem_addr + q * 1024;
+		if (q < P::PATCH_LOADS) {
+			const int idx = q * 64 + lane;
+			const int f = idx % P::F4R, r = (idx / P::F4R) % P::PR, c = idx / (P::F4R * P::PR);
+			const int gy = h0 - g.ph + r, gx = w0 - 4 + 4 * f;
+			if (idx < P::PATCH_F4 && gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
+				valid[i] = true;
+				voff[i] = (uint32_t)(((c * g.H + gy) * g.W + gx) * 4);
+			}
+		} else if (q < P::LOADS) {
+			const int idx = (q - P::PATCH_LOADS) * 64 + lane;
+			const int f = idx % 9, co = idx / 9;
+			if (idx < P::W_F4 && co0 + co < g.Cout) {
+				valid[i] = true;
+				voff[i] = (uint32_t)((co * Kc + 4 * f) * 4);
+			}
+		}
+	}
+	const int64_t x_step = (int64_t)P::CB * g.H * g.W;
+	auto load_one = [&](int i, int stage, int kt) {
+		if (wave + 4 * i >= P::LOADS) return;  // the same for the whole wavefront
+		const float* base = wave + 4 * i < P::PATCH_LOADS ? xn + kt * x_step : wb + kt * (P::CB * 9);
+		if (valid[i]) async_load16(slot[i] + stage * P::STAGE, base, voff[i]);
+	};
+
+	// ---- zeros everywhere once: what no load ever writes is the padding
+	for (int i = tid; i < 2 * P::STAGE / 16; i += 256) reinterpret_cast<float4*>(smem)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	__syncthreads();
+
+#if defined(LTEN_CONV_EXP) && LTEN_CONV_EXP == 2
+	const int KT = g.Cin / P::CB / 2;
+#else
+	const int KT = g.Cin / P::CB;
+#endif
+#pragma unroll
+	for (int i = 0; i < P::LPW; i++) load_one(i, 0, 0);
+	if (KT > 1) {
+#pragma unroll
+		for (int i = 0; i < P::LPW; i++) load_one(i, 1, 1);
+	}
+
+	// ---- operand addresses: a per-lane base plus immediates
+	const int off_a = P::PATCH_BYTES + (lrow * 36 + half * 9) * 4;
+	const int off_b = ((half * P::PR + wave) * P::PWS + lrow + 4 - g.pw) * 4;
+	auto read_one = [&](float (&fa)[P::MT], float (&fb)[P::NT], const uint8_t* sbase, int s, int e) {
+		const int cp = s / 9, tap = s % 9, ti = tap / 3, tj = tap % 3;
+		if (e < P::MT) fa[e] = *reinterpret_cast<const float*>(sbase + off_a + (e * 32 * 36 + 2 * cp * 9 + tap) * 4);
+		else fb[e - P::MT] = *reinterpret_cast<const float*>(sbase + off_b + ((2 * cp * P::PR + ti) * P::PWS + tj + (e - P::MT) * 32) * 4);
+	};
+
+	v16f acc[P::MT][P::NT];
+#pragma unroll
+	for (int m = 0; m < P::MT; m++)
+#pragma unroll
+		for (int t = 0; t < P::NT; t++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) acc[m][t][r] = 0.0f;
+
+	// One step in the exact instruction order wanted: its MFMAs and, behind them, the LDS reads of the next step's
+	// operands and (in the step after the barrier) this wavefront's loads of the chunk after next.
+	auto beat = [&](const float (&ca)[P::MT], const float (&cb)[P::NT], float (&na)[P::MT], float (&nb)[P::NT], int stg, int s, bool read_next,
+	                bool refill, int refill_stage, int refill_kt) {
+		const uint8_t* sbase = smem + stg * P::STAGE;
+#pragma unroll
+		for (int m = 0; m < P::NM; m++) {
+			acc[m / P::NT][m % P::NT] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[m / P::NT], cb[m % P::NT], acc[m / P::NT][m % P::NT], 0, 0, 0);
+			if (read_next) {
+#pragma unroll
+				for (int e = m; e < P::NR; e += P::NM) read_one(na, nb, sbase, s, e);
+			}
+			if (refill) {
+#pragma unroll
+				for (int l = m; l < P::LPW; l += P::NM) load_one(l, refill_stage, refill_kt);
+			}
+			__builtin_amdgcn_sched_barrier(0);
+		}
+	};
+
+	float fa0[P::MT], fb0[P::NT], fa1[P::MT], fb1[P::NT];
+	wait_vmcnt_lgkm0<0>();
+	__syncthreads();
+#pragma unroll
+	for (int e = 0; e < P::NR; e++) read_one(fa0, fb0, smem, 0, e);
+
+	auto inner_beats = [&](int stg) {
+#pragma unroll
+		for (int s = 0; s + 1 < P::STEPS; s++) {
+			if (s & 1) beat(fa1, fb1, fa0, fb0, stg, s + 1, true, false, 0, 0);
+			else beat(fa0, fb0, fa1, fb1, stg, s + 1, true, false, 0, 0);
+		}
+	};
+	int stage = 0, kt = 0;
+	for (; kt + 2 < KT; kt++) {
+		inner_beats(stage);
+		wait_vmcnt_lgkm0<0>();  // own loads of chunk kt + 1 have landed, own reads of chunk kt are done
+		__syncthreads();
+		// STEPS is even: the last step's operands sit in set 1; the stage just read is refilled with chunk kt + 2
+		beat(fa1, fb1, fa0, fb0, stage ^ 1, 0, true, true, stage, kt + 2);
+		stage ^= 1;
+	}
+	if (kt + 1 < KT) {  // the last but one chunk: nothing left to load
+		inner_beats(stage);
+		wait_vmcnt_lgkm0<0>();
+		__syncthreads();
+		beat(fa1, fb1, fa0, fb0, stage ^ 1, 0, true, false, 0, 0);
+		stage ^= 1;
+	}
+	inner_beats(stage);
+	beat(fa1, fb1, fa0, fb0, stage, 0, false, false, 0, 0);
+
+#ifdef LTEN_CONV_EXP  // tuning builds only (results are wrong): 1 = no stores, 2 = half the chunks
+	if (LTEN_CONV_EXP == 1 && acc[0][0][0] != 12345.678f) return;
+#endif
+	// Epilogue: all bias values first, then stores whose address is a shared part plus a lane offset.
+	const int ho = h0 + wave;
+	if (ho >= g.Ho) return;
+	float bv[P::MT][16];
+#pragma unroll
+	for (int m = 0; m < P::MT; m++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int co = co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+			bv[m][r] = (bias && co < g.Cout) ? bias[co] : 0.0f;
+		}
+	const int64_t plane = (int64_t)g.Ho * g.Wo;
+	float* yw = y + (((int64_t)n * g.Cout + co0) * g.Ho + ho) * g.Wo + w0;
+	const unsigned y_lane = (unsigned)(half * 4 * plane) + lrow;
+	if (co0 + BM <= g.Cout && w0 + P::TW <= g.Wo) {
+#pragma unroll
+		for (int m = 0; m < P::MT; m++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+#pragma unroll
+				for (int t = 0; t < P::NT; t++) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
+			}
+		return;
+	}
+#pragma unroll
+	for (int m = 0; m < P::MT; m++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			if (co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3) >= g.Cout) continue;
+			float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
+#pragma unroll
+			for (int t = 0; t < P::NT; t++)
+				if (w0 + t * 32 + lrow < g.Wo) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
+		}
+}
+
+bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float* w)
+{
+	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw <= 4 && g.Cin % 4 == 0 && g.Cin >= 8 &&
+	       g.W % 4 == 0 && aligned16(x) && aligned16(w) && (uint64_t)g.H * g.W < (1u << 26) && (uint64_t)g.Ho * g.Wo <= (1u << 26) &&
+	       (uint64_t)64 * g.Cin * 9 * 4 < (1ull << 31) && ceil_div((uint64_t)g.Cout, 32) < 65536 && g.N < 65536;
+}
+
+int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
+{
+	const unsigned tiles = (unsigned)(ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 4));
+	if (ceil_div((uint64_t)g.Cout, 32) % 2 == 1) {
+		set_kernel_name("conv2d_patch_fast_forward_3x3_32x4x128");
+		conv2d_patch_fast_forward_kernel<32><<<dim3(tiles, (unsigned)ceil_div((uint64_t)g.Cout, 32), (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	} else {
+		set_kernel_name("conv2d_patch_fast_forward_3x3_64x4x128");
+		conv2d_patch_fast_forward_kernel<64><<<dim3(tiles, (unsigned)ceil_div((uint64_t)g.Cout, 64), (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+}  // namespace lten_hip

@@ -87,14 +87,18 @@ def test_conv_layer_golden(gpu):
                                  # that are / are not a multiple of four floats, pad 0 / 1 / 2, ragged channel counts
                                  (2, 20, 17, 136, 70, 3, 3, 1, 1, 1, 1), (1, 37, 12, 64, 33, 3, 3, 0, 0, 1, 1),
                                  (2, 9, 8, 20, 8, 3, 3, 2, 2, 1, 1), (1, 64, 5, 260, 130, 3, 3, 1, 0, 1, 1), (2, 12, 10, 36, 96, 3, 3, 1, 1, 1, 1),
+                                 # input channels a multiple of four (patch filled by direct-to-LDS loads): 64-channel
+                                 # workgroups with a ragged second column tile, ragged channel count with pad 2, one chunk pair
+                                 (2, 8, 9, 132, 64, 3, 3, 1, 1, 1, 1), (1, 16, 6, 128, 100, 3, 3, 2, 2, 1, 1), (1, 32, 7, 12, 128, 3, 3, 0, 1, 1, 1),
                                  # stride 1 with Cin*kh*kw <= 32 (first-layer kernels): ragged widths, two column
                                  # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
                                  (1, 20, 9, 132, 33, 1, 1, 0, 0, 1, 1), (2, 3, 16, 36, 64, 3, 3, 0, 0, 1, 1),
                                  (5, 2, 7, 9, 3, 2, 7, 1, 4, 1, 1)])
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 2])
 def test_conv_vs_oracle(gpu, ob, geo, variant):
-    """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape."""
+    """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape; 2: the register-staged
+    patch kernel also where the direct-to-LDS one would run."""
     try:
         gpu.set_option("conv_variant", variant)
         _conv_vs_oracle(gpu, ob, geo)
