@@ -770,4 +770,131 @@ Tensor Conv2d_q::forward(Tensor& input)
 	return result;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// NeuralNetwork and the optimizers (l-ten/net.h, l-ten/optimizer.{h,cpp})
+
+NeuralNetwork::~NeuralNetwork()
+{
+	for (auto& p : params_) delete p.param_data_;
+	for (Module* m : modules_) delete m;
+}
+
+NetworkParms* NeuralNetwork::get_parameters(int* num_params_ptr)
+{
+	if (!num_params_ptr) return nullptr;
+	*num_params_ptr = (int)params_.size();
+	return params_.data();
+}
+
+void NeuralNetwork::to(device target_device, int target_device_index)
+{
+	for (Module* m : modules_) m->to(target_device, target_device_index);
+	for (auto& p : params_)
+		if (p.param_data_) *p.param_data_ = p.param_data_->to(target_device, target_device_index);
+}
+
+void NeuralNetwork::train(bool is_training)
+{
+	for (Module* m : modules_) m->train(is_training);
+}
+
+Module* NeuralNetwork::get_module(int index)
+{
+	return index >= 0 && index < (int)modules_.size() ? modules_[index] : nullptr;
+}
+
+void Optimizer::attach_network(NeuralNetwork& net)
+{
+	network_params_ptr_ = net.get_parameters(&num_params_);
+	setup_optimizer();
+}
+
+void Optimizer::zero_grad()
+{
+	for (int i = 0; i < num_params_; i++) network_params_ptr_[i].param_->clear_gradients();
+}
+
+Tensor* Optimizer::make_state(int param_index, uint64_t copies)
+{
+	Tensor* param = network_params_ptr_[param_index].param_;
+	uint64_t dims[MAX_DIMS];
+	memcpy(dims, param->get_sizes(), sizeof(uint64_t) * param->get_ndims());
+	dims[0] *= copies;
+	Tensor* state = new Tensor;
+	*state = AllocateTensor(dims, param->get_ndims(), nullptr);
+	memset(state->get_data_ptr(), 0, sizeof(float) * state->get_numels());
+	if (param->get_device() == GPU) *state = state->to(GPU, param->get_device_index());
+	return state;
+}
+
+void SGDOptimizer::setup_optimizer()
+{
+	for (int i = 0; i < num_params_; i++) {
+		delete network_params_ptr_[i].param_data_;
+		network_params_ptr_[i].param_data_ = make_state(i, 1);  // velocity
+	}
+}
+
+void SGDOptimizer::step()
+{
+	if (!num_params_) LTEN_ERR("No parameters have been added to the optimizer");
+	for (int i = 0; i < num_params_; i++) {
+		Tensor* param = network_params_ptr_[i].param_;
+		float* w = (float*)param->get_data_ptr();
+		float* g = (float*)param->get_grad_ptr();
+		float* v = (float*)network_params_ptr_[i].param_data_->get_data_ptr();
+		const uint64_t numels = param->get_numels();
+		if (!g) continue;  // a parameter that took no part in the last backward pass
+		if (param->get_device() != network_params_ptr_[i].param_data_->get_device()) LTEN_ERR("Optimizer state and parameter are on different devices");
+		if (param->get_device() == GPU) {
+			LTEN_HIP_CALL(lten_hip_sgd_step_f32(w, g, v, numels, mo_, wd_, lr_));  // l-ten/optimizer.cpp:66
+		} else {
+			for (uint64_t j = 0; j < numels; j++) {  // l-ten/optimizer.cpp:49-54
+				g[j] = wd_ * w[j] + g[j];
+				v[j] = v[j] * mo_ + (1.0f - mo_) * g[j];
+				w[j] = w[j] - (v[j] * lr_);
+			}
+		}
+	}
+}
+
+void AdamOptimizer::setup_optimizer()
+{
+	for (int i = 0; i < num_params_; i++) {
+		delete network_params_ptr_[i].param_data_;
+		network_params_ptr_[i].param_data_ = make_state(i, 3);  // first moments, second moments, l-ten's scratch third
+	}
+}
+
+void AdamOptimizer::step()
+{
+	if (!num_params_) LTEN_ERR("No parameters have been added to the optimizer");
+	iteration_++;
+	for (int i = 0; i < num_params_; i++) {
+		Tensor* param = network_params_ptr_[i].param_;
+		float* w = (float*)param->get_data_ptr();
+		const float* g = (const float*)param->get_grad_ptr();
+		const uint64_t numels = param->get_numels();
+		float* v_dw = (float*)network_params_ptr_[i].param_data_->get_data_ptr();
+		float* s_dw = v_dw + numels;
+		if (!g) continue;
+		if (param->get_device() != network_params_ptr_[i].param_data_->get_device()) LTEN_ERR("Optimizer state and parameter are on different devices");
+		if (param->get_device() == GPU) {
+			LTEN_HIP_CALL(lten_hip_adam_step_f32(w, g, v_dw, s_dw, numels, lr_, beta1_, beta2_, iteration_));  // l-ten/optimizer.cpp:165-172
+		} else {
+			// l-ten/optimizer.cpp:146-158, the eight element-wise passes in their order
+			const float epsilon = 1.0e-8f;
+			const float bc1 = 1.0f - powf(beta1_, (float)iteration_), bc2 = 1.0f - powf(beta2_, (float)iteration_);
+			for (uint64_t j = 0; j < numels; j++) {
+				v_dw[j] = (1.0f - beta1_) * g[j] + beta1_ * v_dw[j];
+				s_dw[j] = (1.0f - beta2_) * (g[j] * g[j]) + beta2_ * s_dw[j];
+				float t = (1.0f / bc2) * s_dw[j];
+				t = powf(t, 0.5f) + epsilon;
+				t = v_dw[j] / t;
+				w[j] = -(1.0f / bc1) * lr_ * t + w[j];
+			}
+		}
+	}
+}
+
 }  // namespace lten

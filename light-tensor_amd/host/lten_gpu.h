@@ -226,5 +226,90 @@ private:
 	QuantizationParams qparams_in_{ 1.0f, 0 }, qparams_out_{ 1.0f, 0 }, qparams_wt_{ 1.0f, 0 };
 };
 
+// l-ten/net.h:8-19
+struct NetworkParms {
+	std::string name;
+	Tensor* param_;       // trainable parameter
+	Tensor* param_data_;  // what an optimizer keeps for it (velocity, moment histories), or null
+};
+
+// l-ten/net.h:21-117: owns the modules registered with it and lists their trainable parameters for an optimizer.
+// A network class derives from it and registers its layers in its constructor, as in l-ten.
+class NeuralNetwork {
+public:
+	NeuralNetwork() {}
+	NeuralNetwork(const NeuralNetwork&) = delete;
+	NeuralNetwork& operator=(const NeuralNetwork&) = delete;
+	~NeuralNetwork();
+
+	template <typename T>
+	T* register_module(const char* module_name, T&& temp)
+	{
+		T* network_module = new T(temp);
+		network_module->init();
+		for (Tensor* param : network_module->get_all_weights()) params_.push_back(NetworkParms{ module_name ? module_name : "", param, nullptr });
+		modules_.push_back(network_module);
+		return network_module;
+	}
+	NetworkParms* get_parameters(int* num_params_ptr);
+	void to(device target_device, int target_device_index = 0);
+	void train(bool is_training);
+	Module* get_module(int index);
+
+private:
+	std::vector<NetworkParms> params_;
+	std::vector<Module*> modules_;
+};
+
+// l-ten/optimizer.h:6-33.  The state tensors live where the parameters live when the network is attached and
+// move with NeuralNetwork::to afterwards; l-ten allocates them on the CPU and relies on a later to().
+class Optimizer {
+public:
+	Optimizer() {}
+	virtual ~Optimizer() {}
+	void attach_network(NeuralNetwork& net);
+	virtual void setup_optimizer() = 0;
+	virtual void step() = 0;
+	void zero_grad();
+
+protected:
+	Tensor* make_state(int param_index, uint64_t copies);  // zero-filled, copies x the parameter's first dimension
+	int num_params_ = 0;
+	NetworkParms* network_params_ptr_ = nullptr;
+};
+
+// l-ten/optimizer.h:35-58, l-ten/optimizer.cpp:10-84
+class SGDOptimizer : public Optimizer {
+public:
+	void setup_optimizer() override;
+	void step() override;
+	void set_learning_rate(float lr) { lr_ = lr; }
+	float get_learning_rate() { return lr_; }
+	void set_momentum(float mo) { mo_ = mo; }
+	float get_momentum() { return mo_; }
+	void set_weight_decay(float wd) { wd_ = wd; }
+	float get_weight_decay() { return wd_; }
+
+private:
+	float lr_ = 0.01f, wd_ = 0.0005f, mo_ = 0.9f;
+};
+
+// l-ten/optimizer.h:60-84, l-ten/optimizer.cpp:88-186
+class AdamOptimizer : public Optimizer {
+public:
+	void setup_optimizer() override;
+	void step() override;
+	void set_learning_rate(float lr) { lr_ = lr; }
+	float get_learning_rate() { return lr_; }
+	void set_beta1(float beta1) { beta1_ = beta1; }
+	float get_beta1() { return beta1_; }
+	void set_beta2(float beta2) { beta2_ = beta2; }
+	float get_beta2() { return beta2_; }
+
+private:
+	uint64_t iteration_ = 0;
+	float lr_ = 0.01f, beta1_ = 0.9f, beta2_ = 0.999f;
+};
+
 }  // namespace lten
 #endif

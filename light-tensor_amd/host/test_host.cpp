@@ -179,6 +179,74 @@ static int mlp_step_test()
 	return 0;
 }
 
+// A network class in l-ten's style (modules registered in the constructor, l-ten tests/nn_tests.cpp:17-42) trained on the
+// device with each optimizer: a 4-class problem whose label is the largest of four fixed projections of the input.
+// The loss must fall well below its start value; attach-then-move and move-then-attach must both work.
+static int training_test()
+{
+	class Net : public lten::NeuralNetwork {
+	public:
+		Net()
+		{
+			fc1 = register_module("fc1", lten::FullyConnected(8, 32, true));
+			fc2 = register_module("fc2", lten::FullyConnected(32, 4, true));
+		}
+		lten::Tensor forward(lten::Tensor input)
+		{
+			lten::Tensor h = fc1->forward(input);
+			lten::Tensor a = lten::relu(h);
+			return fc2->forward(a);
+		}
+		lten::FullyConnected *fc1, *fc2;
+	};
+	const uint64_t B = 64, F = 8, C = 4;
+	unsigned s = 4242;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (float)((s >> 8) & 0xFFFF) / 32768.0f - 1.0f; };
+	std::vector<float> proj(C * F);
+	for (auto& e : proj) e = rnd();
+	for (int which = 0; which < 2; which++) {
+		Net net;
+		lten::SGDOptimizer sgd;
+		lten::AdamOptimizer adam;
+		lten::Optimizer* opt = which == 0 ? (lten::Optimizer*)&sgd : (lten::Optimizer*)&adam;
+		sgd.set_learning_rate(0.2f);
+		sgd.set_weight_decay(0.0f);
+		adam.set_learning_rate(0.01f);
+		if (which == 0) { opt->attach_network(net); net.to(lten::GPU); }  // state allocated on the host, moved with the network
+		else { net.to(lten::GPU); opt->attach_network(net); }             // state allocated on the device
+		float first = 0.0f, last = 0.0f;
+		for (int it = 0; it < 300; it++) {
+			std::vector<float> x(B * F), t(B * C, 0.0f);
+			for (uint64_t m = 0; m < B; m++) {
+				for (uint64_t k = 0; k < F; k++) x[m * F + k] = rnd();
+				uint64_t best = 0;
+				float bv = -1e30f;
+				for (uint64_t c = 0; c < C; c++) {
+					float v = 0.0f;
+					for (uint64_t k = 0; k < F; k++) v += proj[c * F + k] * x[m * F + k];
+					if (v > bv) { bv = v; best = c; }
+				}
+				t[m * C + best] = 1.0f;
+			}
+			lten::Tensor X = lten::TensorFromBuffer({ B, 1, 1, F }, x.data()).to(lten::GPU);
+			lten::Tensor T = lten::TensorFromBuffer({ B, 1, 1, C }, t.data()).to(lten::GPU);
+			lten::Tensor y = net.forward(X);
+			lten::Tensor lp = lten::log_softmax(y, 3);
+			lten::Tensor loss = lten::nll_loss(lp, T);
+			loss.backward();
+			opt->step();
+			opt->zero_grad();
+			if (it == 0 || it == 299) {
+				lten::Tensor lc = loss.to(lten::CPU);
+				(it == 0 ? first : last) = *(float*)lc.get_data_ptr();
+			}
+		}
+		printf("  %s: loss %.4f -> %.4f\n", which == 0 ? "SGD" : "Adam", first, last);
+		if (!(last < 0.5f * first) || !(last < 0.7f)) return -1 - which;
+	}
+	return 0;
+}
+
 // FullyConnected_q on {2, 3, 37} with bias: every leading index is its own quantized_matmul in l-ten
 static int fcq_test()
 {
@@ -326,7 +394,7 @@ static int error_test()
 
 int main()
 {
-	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test },
+	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test }, { "training_test", training_test },
 		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;
 	for (auto& t : tests) {
