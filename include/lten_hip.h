@@ -257,7 +257,7 @@ int lten_hip_measure_last_clocks(double* cycles_per_mfma, double* shader_mhz);
 int lten_hip_copy_kernel(const void* device_src, void* device_dst, uint64_t bytes);
 
 /* Kernel-selection override for tests and tuning sweeps; 0 restores the built-in heuristic.
- * Options: "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant".  No counterpart in l-ten. */
+ * Options: "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant", "qgemm_split".  No counterpart in l-ten. */
 int lten_hip_set_option(const char* name, int value);
 
 /* Name of the kernel variant the last GEMM-type call on this thread dispatched to

@@ -16,9 +16,10 @@ namespace lten_hip {
 void set_error(const char* fmt, ...);
 void set_kernel_name(const char* name);
 hipStream_t stream();
+bool capturing();  // a launch graph is being recorded: no allocation, no synchronisation
 
 // Tuning / test switches behind lten_hip_set_option.
-enum Option { OPT_QGEMM_TILE = 0, OPT_SGEMM_TILE, OPT_QSKINNY, OPT_CONV_VARIANT, OPT_COUNT };
+enum Option { OPT_QGEMM_TILE = 0, OPT_SGEMM_TILE, OPT_QSKINNY, OPT_CONV_VARIANT, OPT_QGEMM_SPLIT, OPT_COUNT };
 int get_option(Option o);
 
 inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }

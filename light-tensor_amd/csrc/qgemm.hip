@@ -320,6 +320,16 @@ static int qgemm_dispatch(const QProblem& p, int out)
 		// workgroups, two per CU) below that.
 		if (p.K >= 512) {
 			if (out_elems > 256ull * 256 * 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+			// Outputs that give 128 x 128 tiles to at most a quarter of the CUs, with a long K: several workgroups share a
+			// tile, each with a slice of K (option "qgemm_split": 0 automatic, 1 off, 2 / 4 / 8 forced).  The exchange of
+			// partial sums between workgroups is dear on this part, so the split pays only there: 1024 x 4096 weights
+			// at M = 256 27 -> 19 us, 2048 x 8192 at M = 128 51 -> 27 us, but 4096 x 4096 at M = 512 30 -> 35 us.
+			const int want = get_option(OPT_QGEMM_SPLIT);
+			const uint64_t tiles = out_elems / (128 * 128);
+			int splits = 1;
+			if (want >= 2) splits = want;
+			else if (want == 0 && tiles <= 64 && p.K >= 4096) splits = tiles <= 32 ? 4 : 2;
+			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits) == 0) return 0;
 			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
 		}
 		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
@@ -391,6 +401,9 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	p.mult = ab / qp[2].scale;
 	p.zp_c = (float)qp[2].zero_point;
 	p.stamps = nullptr;
+	p.split_partial = nullptr;
+	p.split_counters = nullptr;
+	p.splits = 1;
 #ifdef LTEN_HIP_STAMPS
 	if (workspace) p.stamps = reinterpret_cast<long long*>(workspace + ((M + N + 3) & ~3ull));
 #endif

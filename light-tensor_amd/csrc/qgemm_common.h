@@ -25,6 +25,10 @@ struct QProblem {
 	float zp_c;            // (float) output zero point
 	int vec_ok;            // operand bases and row strides are multiples of 16 bytes
 	long long* stamps;     // tuning builds only: per-workgroup phase timestamps, else null
+	// split-K launches of the direct-to-LDS tiles: `splits` workgroups share an output tile, each takes K / splits
+	int32_t* split_partial;     // [tile][split][T*T] partial sums in register order
+	unsigned* split_counters;   // [tile] arrivals; zero between launches
+	int splits;
 };
 
 // 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).
@@ -73,5 +77,6 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 
 // Dispatch of the tuned square-ish kernels (qgemm_fast.hip).  Returns -1 when no fast variant fits.
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant);
+int qgemm_fast_split_dispatch(const QProblem& p, int out, int splits);
 
 }  // namespace lten_hip

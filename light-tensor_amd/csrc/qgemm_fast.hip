@@ -39,7 +39,7 @@ namespace lten_hip {
 #define LTEN_HIP_EXP 0
 #endif
 
-template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS>
+template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false>
 __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 {
 	constexpr int BM = T, BN = T;  // square output tile, 256 or 128
@@ -98,8 +98,12 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		voff[i] = (i < LPW / 2 ? (uint32_t)(m0 + r) : (uint32_t)(n0 + r - BM)) * (uint32_t)p.K + kc * 16;
 		lds_slot[i] = smem_addr + q * 1024;
 	}
+	// with SPLIT, blockIdx.y picks this workgroup's share of K
+	const int KT = SPLIT ? p.K / BK / p.splits : p.K / BK;
+	const uint8_t* const a_base = p.A + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
+	const uint8_t* const b_base = p.B + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
 	auto load_one = [&](int i, int stage, int kt) {
-		async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? p.A : p.B) + (int64_t)kt * BK, voff[i]);
+		async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
 	};
 	auto issue = [&](int stage, int kt) {
 #pragma unroll
@@ -120,8 +124,6 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		for (int j = 0; j < FM; j++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
-
-	const int KT = p.K / BK;
 
 	auto read_frags = [&](v4i(&fw)[FN], v4i(&fx)[FM], int stg, int s) {
 		const uint8_t* sbase = smem + stg * STAGE;
@@ -225,6 +227,45 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	LTEN_STAMP(2);
 	LTEN_STAMP(5);
 
+	// Split K: every workgroup of a tile publishes its partial sums (in register order, so a wavefront of any of them
+	// reads back exactly what the same wavefront of another wrote), then counts itself in; the one that arrives last
+	// adds the others' sums to its own and carries on to the epilogue.  int32 sums do not depend on the order.  The
+	// partial sums travel as device-scope atomic stores and loads (they pass the per-XCD L2s; plain stores behind a
+	// release fence measured slower, because the fence writes back the whole L2), with a release fence before the count
+	// and an acquire fence after it; nobody waits for anybody.  The last workgroup resets the counter for the next
+	// launch on the stream.
+	if (SPLIT) {
+		constexpr int NACC = FN * FM * 16;
+		int32_t* const tile_slabs = p.split_partial + (int64_t)blockIdx.x * p.splits * (NACC * W * 64);
+		int32_t* const mine = tile_slabs + (int64_t)blockIdx.y * (NACC * W * 64);
+#pragma unroll
+		for (int i = 0; i < FN; i++)
+#pragma unroll
+			for (int j = 0; j < FM; j++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					__hip_atomic_store(mine + ((i * FM + j) * 16 + r) * (W * 64) + tid, acc[i][j][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+		__syncthreads();
+		unsigned* const arrived = reinterpret_cast<unsigned*>(smem);  // the operand stages are no longer read
+		if (tid == 0) *arrived = __hip_atomic_fetch_add(p.split_counters + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__syncthreads();
+		if (*arrived != (unsigned)p.splits - 1) return;
+		__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+		for (int s2 = 0; s2 < p.splits; s2++) {
+			if (s2 == (int)blockIdx.y) continue;
+			const int32_t* other = tile_slabs + (int64_t)s2 * (NACC * W * 64);
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int j = 0; j < FM; j++)
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						acc[i][j][r] += __hip_atomic_load(other + ((i * FM + j) * 16 + r) * (W * 64) + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		}
+		if (tid == 0) __hip_atomic_store(p.split_counters + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+
 	// Epilogue: lane (lrow, lgrp), register 4q + e of block (i, j) is the output at
 	//   m = m0 + wm*TM + j*32 + lrow,  n = n0 + wn*TN + i*32 + 8q + 4*lgrp + e.
 	if (OUT == Q_OUT_ACC) {
@@ -296,6 +337,57 @@ static int launch_fast(const QProblem& p, int out, const char* name)
 		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, true><<<grid, block, 0, stream()>>>(p);     \
 	else                                                                                     \
 		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, false><<<grid, block, 0, stream()>>>(p);
+	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
+	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
+	else { LTEN_LAUNCH(Q_OUT_ACC) }
+#undef LTEN_LAUNCH
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+// Scratch of the split-K launches: owned by the library, allocated on first use (never while a launch graph is
+// being recorded), kept until the process ends.  One stream uses it at a time, as everything else in this library.
+static int32_t* g_split_partial = nullptr;
+static unsigned* g_split_counters = nullptr;
+constexpr size_t SPLIT_PARTIAL_BYTES = 32u << 20;
+constexpr int SPLIT_MAX_TILES = 4096;
+
+static bool split_scratch_ready()
+{
+	if (g_split_partial != nullptr) return true;
+	if (capturing()) return false;
+	void* partial = nullptr;
+	void* counters = nullptr;
+	if (hipMalloc(&partial, SPLIT_PARTIAL_BYTES) != hipSuccess) { (void)hipGetLastError(); return false; }
+	if (hipMalloc(&counters, SPLIT_MAX_TILES * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(partial); return false; }
+	if (hipMemset(counters, 0, SPLIT_MAX_TILES * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(partial); (void)hipFree(counters); return false; }
+	g_split_partial = static_cast<int32_t*>(partial);
+	g_split_counters = static_cast<unsigned*>(counters);
+	return true;
+}
+
+// 128 x 128 tiles with K cut into `splits` shares; -1 when the problem or the scratch does not allow it.
+int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits)
+{
+	constexpr int T = 128, BK = 128;
+	QProblem p = q;
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M % T == 0 && p.N % T == 0 && p.K % (BK * splits) == 0 &&
+	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
+	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
+	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
+	                  (uint64_t)p.M * p.N * 4 * splits <= SPLIT_PARTIAL_BYTES && (uint64_t)(p.M / T) * (p.N / T) <= SPLIT_MAX_TILES;
+	if (!fits || !split_scratch_ready()) return -1;
+	p.split_partial = g_split_partial;
+	p.split_counters = g_split_counters;
+	p.splits = splits;
+	const dim3 grid((unsigned)((p.M / T) * (p.N / T)), (unsigned)splits), block(256);
+	const bool terms = p.rterm != nullptr;
+	set_kernel_name("qgemm_fast_128x128x128_w2x2_s2_splitk");
+#define LTEN_LAUNCH(OUTV)                                                                              \
+	if (terms)                                                                                     \
+		qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, true, true><<<grid, block, 0, stream()>>>(p);       \
+	else                                                                                           \
+		qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, false, true><<<grid, block, 0, stream()>>>(p);
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }

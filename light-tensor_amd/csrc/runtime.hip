@@ -32,9 +32,10 @@ void set_kernel_name(const char* name)
 }
 
 hipStream_t stream() { return g_stream; }
+bool capturing() { return g_capturing; }
 
 static int g_options[OPT_COUNT] = { 0 };
-static const char* const g_option_names[OPT_COUNT] = { "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant" };
+static const char* const g_option_names[OPT_COUNT] = { "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant", "qgemm_split" };
 int get_option(Option o) { return g_options[o]; }
 
 template <typename T>

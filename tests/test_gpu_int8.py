@@ -163,6 +163,64 @@ def test_medium_batch_picks_128_tiles(gpu, ob):
     assert gpu.last_kernel().startswith("qgemm_fast_128x128x128")
 
 
+@pytest.mark.parametrize("splits", [2, 4, 8])
+def test_split_k_tiles_forced(gpu, ob, splits):
+    """Several workgroups per 128 x 128 tile, each with a share of K, the last to arrive adds the shares: forced by
+    option on a shape the oracle still finishes (10 tiles, K = 2048), with zero-point terms, bias, the exact-convert
+    epilogue, int32 and u8 outputs; repeated launches check that the arrival counters return to zero."""
+    rng = np.random.default_rng(splits)
+    M, N, K = 256, 640, 2048
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    gpu.set_option("qgemm_split", splits)
+    try:
+        for rep in range(3):
+            run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8))
+            assert gpu.last_kernel().endswith("splitk")
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8), bias=rng.integers(-5000, 5000, N).astype(np.int32))
+        assert gpu.last_kernel().endswith("splitk")
+        run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8))
+    finally:
+        gpu.set_option("qgemm_split", 0)
+
+
+def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
+    """256 x 1024 x 4096 (16 tiles): the library splits K in four; the closed form in int64 is the check.  With the
+    option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
+    rng = np.random.default_rng(5)
+    M, N, K = 256, 1024, 4096
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    zp = [7, 200, 128]
+    sc = [0.02, 0.02, 2.5]
+    dA, dB = gpu.DeviceBuffer.from_numpy(A), gpu.DeviceBuffer.from_numpy(B)
+    dC, dacc, ws = gpu.DeviceBuffer(M * N), gpu.DeviceBuffer(4 * M * N), gpu.DeviceBuffer(4 * (M + N))
+    qp = gpu.qparams3(sc, zp)
+    gpu.quantized_matmul_acc(False, True, M, N, K, dA, dB, dacc, qp, None, ws)
+    assert gpu.last_kernel().endswith("splitk")
+    want = exact_acc(A, B, zp[0], zp[1])
+    assert np.array_equal(dacc.numpy(np.int32, (M, N)), want)
+    gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
+    assert gpu.last_kernel().endswith("splitk")
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    split_out = dC.numpy(np.uint8, (M, N)).copy()
+    assert np.array_equal(split_out, requant_numpy(want, mult, zp[2]))
+    gpu.set_option("qgemm_split", 1)
+    try:
+        gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
+        assert not gpu.last_kernel().endswith("splitk")
+        assert np.array_equal(dC.numpy(np.uint8, (M, N)), split_out)
+    finally:
+        gpu.set_option("qgemm_split", 0)
+    gpu.check(gpu.lib().lten_hip_fill_u8(dC.ptr, M * N, 0))
+    with gpu.Graph() as graph:
+        gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
+    for _ in range(3):
+        gpu.check(gpu.lib().lten_hip_fill_u8(dC.ptr, M * N, 0))
+        graph.launch()
+        assert np.array_equal(dC.numpy(np.uint8, (M, N)), split_out)
+
+
 def test_cfg3_full_size_properties(gpu, wl):
     """4096^3: exact closed form of every accumulator (fp64 BLAS holds these integers exactly),
     then the requantize rule on top; plus linearity in the bias."""
