@@ -319,13 +319,13 @@ static int qgemm_dispatch(const QProblem& p, int out)
 		// and epilogue: 256x256 tiles once those occupy most of the 256 CUs, 128x128 tiles (up to four times as many
 		// workgroups, two per CU) below that.
 		if (p.K >= 512) {
-			if (out_elems > 256ull * 256 * 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+			if (ceil_div(p.M, 256) * ceil_div(p.N, 256) > 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
 			// Outputs that give 128 x 128 tiles to at most a quarter of the CUs, with a long K: several workgroups share a
 			// tile, each with a slice of K (option "qgemm_split": 0 automatic, 1 off, 2 / 4 / 8 forced).  The exchange of
 			// partial sums between workgroups is dear on this part, so the split pays only there: 1024 x 4096 weights
 			// at M = 256 27 -> 19 us, 2048 x 8192 at M = 128 51 -> 27 us, but 4096 x 4096 at M = 512 30 -> 35 us.
 			const int want = get_option(OPT_QGEMM_SPLIT);
-			const uint64_t tiles = out_elems / (128 * 128);
+			const uint64_t tiles = ceil_div(p.M, 128) * ceil_div(p.N, 128);
 			int splits = 1;
 			if (want >= 2) splits = want;
 			else if (want == 0 && tiles <= 64 && p.K >= 4096) splits = tiles <= 32 ? 4 : 2;
@@ -424,6 +424,19 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	if (M <= 32 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
+	}
+	// 33 to 64 rows: two streaming passes (32 rows, then the rest) still beat one pass of 128-row tiles, three would not
+	if (M > 32 && M <= 64 && N >= 2048 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+		QProblem top = p, rest = p;
+		top.M = 32;
+		rest.M = (int)M - 32;
+		rest.A = p.A + 32 * p.a_rs;
+		rest.C = static_cast<uint8_t*>(p.C) + (uint64_t)32 * N * (out == Q_OUT_ACC ? 4 : 1);
+		if (qskinny_dispatch(top, out, bias, zpA, zpB) == 0) {
+			const int rc = qskinny_dispatch(rest, out, bias, zpA, zpB);
+			LTEN_HIP_REQUIRE(rc == 0, "quantized_matmul: the second streaming pass did not launch");
+			return 0;
+		}
 	}
 	// small outputs: one launch that also takes the zero-point sums (same option switches it off)
 	if (get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {

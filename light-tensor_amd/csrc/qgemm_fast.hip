@@ -1,5 +1,7 @@
-// Tuned int8 GEMM tiles for large NT problems (both operands contiguous in K, every dimension a
-// multiple of the tile): 256 x 256 output tile, k-steps of BK bytes, a ring of S LDS stages filled by
+// Tuned int8 GEMM tiles for large NT problems (both operands contiguous in K, K a multiple of the
+// k-step, N a multiple of 16; M and N need not be multiples of the tile: a load that would start past the
+// last row of an operand fetches the last row instead, and what is computed from it is not stored):
+// 256 x 256 output tile, k-steps of BK bytes, a ring of S LDS stages filled by
 // direct global->LDS loads (no register staging), MFMA 32x32x32 int8.
 //
 // Data path per k-step: every wavefront issues its share of the stage's wave-wide 16-byte-per-lane
@@ -65,7 +67,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 
 	// Workgroup -> tile.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2;
 	// every XCD gets one compact 4 x 8 block of tiles so that its CUs stream the same A and B rows.
-	const int tiles_m = p.M / BM, tiles_n = p.N / BN;
+	const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
 	int tm, tn;
 	{
 		const int nb = tiles_m * tiles_n, bid = blockIdx.x;
@@ -95,7 +97,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		const int q = wave + i * W;
 		const int r = q * RPL + lane / CPR;
 		const int kc = (lane % CPR) ^ swz<CPR>(r);
-		voff[i] = (i < LPW / 2 ? (uint32_t)(m0 + r) : (uint32_t)(n0 + r - BM)) * (uint32_t)p.K + kc * 16;
+		voff[i] = (i < LPW / 2 ? (uint32_t)min(m0 + r, p.M - 1) : (uint32_t)min(n0 + r - BM, p.N - 1)) * (uint32_t)p.K + kc * 16;
 		lds_slot[i] = smem_addr + q * 1024;
 	}
 	// with SPLIT, blockIdx.y picks this workgroup's share of K
@@ -272,12 +274,14 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
 			const int m = m0 + wm * TM + j * 32 + lrow;
+			if (m >= p.M) continue;
 			const int rt = TERMS ? p.rterm[m] + p.konst : p.konst;
 #pragma unroll
 			for (int i = 0; i < FN; i++)
 #pragma unroll
 				for (int q = 0; q < 4; q++) {
 					const int n = n0 + wn * TN + i * 32 + q * 8 + lgrp * 4;
+					if (n >= p.N) continue;  // N is a multiple of 4: the four columns exist together
 					v4i v = { acc[i][j][q * 4] + rt, acc[i][j][q * 4 + 1] + rt, acc[i][j][q * 4 + 2] + rt, acc[i][j][q * 4 + 3] + rt };
 					if (TERMS) v += *reinterpret_cast<const v4i*>(p.cterm + n);
 					*reinterpret_cast<v4i*>(static_cast<int*>(p.C) + (int64_t)m * p.N + n) = v;
@@ -293,7 +297,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
 			const int row = wm * TM + j * 32 + lrow;
-			const int rt = TERMS ? p.rterm[m0 + row] + p.konst : p.konst;
+			const int rt = TERMS ? p.rterm[min(m0 + row, p.M - 1)] + p.konst : p.konst;
 #pragma unroll
 			for (int i = 0; i < FN; i++)
 #pragma unroll
@@ -302,7 +306,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 					int v[4];
 #pragma unroll
 					for (int e = 0; e < 4; e++) v[e] = acc[i][j][q * 4 + e] + rt;
-					if (TERMS) {
+					if (TERMS && n0 + col < p.N) {
 						const v4i ct = *reinterpret_cast<const v4i*>(p.cterm + n0 + col);
 						v[0] += ct.x; v[1] += ct.y; v[2] += ct.z; v[3] += ct.w;
 					}
@@ -316,7 +320,8 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #pragma unroll
 		for (int c = tid; c < BM * BN / 16; c += W * 64) {
 			const int row = c / (BN / 16), ch = c % (BN / 16);
-			*reinterpret_cast<v4i*>(cout + (int64_t)row * p.N + ch * 16) = *reinterpret_cast<const v4i*>(smem + row * OLD + ch * 16);
+			if (m0 + row < p.M && n0 + ch * 16 < p.N)  // N is a multiple of 16: whole 16-byte pieces
+				*reinterpret_cast<v4i*>(cout + (int64_t)row * p.N + ch * 16) = *reinterpret_cast<const v4i*>(smem + row * OLD + ch * 16);
 		}
 	}
 #ifdef LTEN_HIP_STAMPS
@@ -328,8 +333,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 template <int T, int BK, int WM, int WN, int S>
 static int launch_fast(const QProblem& p, int out, const char* name)
 {
-	if (p.M % T != 0 || p.N % T != 0) return -1;
-	const dim3 grid((unsigned)((p.M / T) * (p.N / T))), block(WM * WN * 64);
+	const dim3 grid((unsigned)(ceil_div(p.M, T) * ceil_div(p.N, T))), block(WM * WN * 64);
 	const bool terms = p.rterm != nullptr;
 	set_kernel_name(name);
 #define LTEN_LAUNCH(OUTV)                                                                        \
@@ -371,16 +375,16 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits)
 {
 	constexpr int T = 128, BK = 128;
 	QProblem p = q;
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M % T == 0 && p.N % T == 0 && p.K % (BK * splits) == 0 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 16 == 0 && p.K % (BK * splits) == 0 &&
 	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
-	                  (uint64_t)p.M * p.N * 4 * splits <= SPLIT_PARTIAL_BYTES && (uint64_t)(p.M / T) * (p.N / T) <= SPLIT_MAX_TILES;
+	                  ceil_div(p.M, T) * ceil_div(p.N, T) * T * T * 4 * splits <= SPLIT_PARTIAL_BYTES && ceil_div(p.M, T) * ceil_div(p.N, T) <= SPLIT_MAX_TILES;
 	if (!fits || !split_scratch_ready()) return -1;
 	p.split_partial = g_split_partial;
 	p.split_counters = g_split_counters;
 	p.splits = splits;
-	const dim3 grid((unsigned)((p.M / T) * (p.N / T)), (unsigned)splits), block(256);
+	const dim3 grid((unsigned)(ceil_div(p.M, T) * ceil_div(p.N, T)), (unsigned)splits), block(256);
 	const bool terms = p.rterm != nullptr;
 	set_kernel_name("qgemm_fast_128x128x128_w2x2_s2_splitk");
 #define LTEN_LAUNCH(OUTV)                                                                              \
@@ -399,7 +403,7 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits)
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M % 128 == 0 && p.N % 128 == 0 && p.K % 128 == 0 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 16 == 0 && p.K % 128 == 0 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0);

@@ -139,7 +139,9 @@ def test_fcq_forward_leading_dims(gpu, ob, wl):
 
 
 @pytest.mark.parametrize("variant", [41, 42, 43, 44])
-@pytest.mark.parametrize("shape", [(128, 128, 128), (384, 640, 640), (128, 1152, 2048)])
+@pytest.mark.parametrize("shape", [(128, 128, 128), (384, 640, 640), (128, 1152, 2048),
+                                   # ragged M and N (N a multiple of 16): edge tiles fetch the last row again and store what exists
+                                   (33, 144, 512), (200, 656, 1152), (1, 16, 128)])
 def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
     """The 128x128 form of the direct-to-LDS tiles (what the library picks when 256x256 tiles would leave CUs idle):
     both k-step sizes, 2 to 4 stages, with and without zero-point terms and bias, short and long K; int32 and u8."""
@@ -152,6 +154,38 @@ def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
     run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8),
              bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
     run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)   # multiplier > 0.99: exact-convert epilogue
+
+
+@pytest.mark.parametrize("variant", [31, 33, 34])
+def test_direct_to_lds_256_tiles_ragged(gpu, ob, variant):
+    """300 x 272 x 640 on 256 x 256 tiles: two row tiles and two column tiles, all of them edge tiles."""
+    rng = np.random.default_rng(variant)
+    A = rng.integers(0, 256, (300, 640), dtype=np.uint8)
+    B = rng.integers(0, 256, (272, 640), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8), bias=rng.integers(-5000, 5000, 272).astype(np.int32), tile=variant)
+    assert gpu.last_kernel().startswith("qgemm_fast_256x256")
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=variant)
+
+
+def test_batch_sizes_between_the_tile_sizes(gpu):
+    """M = 65, 100, 200 against 4096 x 4096 or 2048 x 4096 weights (more rows than the streaming kernel takes, no multiple of 128): the
+    tiles with K split, checked against the closed form; M = 200 against 4096 x 1024 (no split)."""
+    rng = np.random.default_rng(3)
+    for (M, N, K, split) in ((65, 4096, 4096, True), (100, 2048, 4096, True), (200, 2048, 4096, True), (200, 4096, 1024, False)):
+        A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+        B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+        zp, sc = [11, 140, 120], [0.02, 0.02, 3.0]
+        bias = rng.integers(-9000, 9000, N).astype(np.int32)
+        dA, dB, dBias = gpu.DeviceBuffer.from_numpy(A), gpu.DeviceBuffer.from_numpy(B), gpu.DeviceBuffer.from_numpy(bias)
+        dC, dacc, ws = gpu.DeviceBuffer(M * N), gpu.DeviceBuffer(4 * M * N), gpu.DeviceBuffer(4 * (M + N))
+        qp = gpu.qparams3(sc, zp)
+        gpu.quantized_matmul_acc(False, True, M, N, K, dA, dB, dacc, qp, dBias, ws)
+        assert gpu.last_kernel().startswith("qgemm_fast_128x128") and gpu.last_kernel().endswith("splitk") == split, gpu.last_kernel()
+        want = exact_acc(A, B, zp[0], zp[1]) + bias[None, :]
+        assert np.array_equal(dacc.numpy(np.int32, (M, N)), want)
+        gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, dBias, ws)
+        mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+        assert np.array_equal(dC.numpy(np.uint8, (M, N)), requant_numpy(want, mult, zp[2]))
 
 
 def test_medium_batch_picks_128_tiles(gpu, ob):
@@ -263,6 +297,19 @@ def test_weight_streaming_kernel(gpu, ob, shape):
         finally:
             gpu.set_option("qskinny", 0)
         assert np.array_equal(Cg, Ct)
+
+
+@pytest.mark.parametrize("M", [33, 47, 64])
+def test_weight_streaming_in_two_passes(gpu, ob, M):
+    """33 to 64 activation rows against 2048 x 2048 weights: the streaming kernel runs on the first 32 rows and then on
+    the rest; with zero-point terms and bias, u8 and int32 outputs, against the oracle."""
+    rng = np.random.default_rng(M)
+    A = rng.integers(0, 256, (M, 2048), dtype=np.uint8)
+    B = rng.integers(0, 256, (2048, 2048), dtype=np.uint8)
+    for zp in ([128, 128, 128], [17, 250, 100]):
+        bias = rng.integers(-9999, 9999, 2048).astype(np.int32) if zp[0] != 128 else None
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array(zp, np.uint8), bias=bias)
+        assert gpu.last_kernel().startswith("qskinny_mfma_w2_k1024"), gpu.last_kernel()
 
 
 @pytest.mark.parametrize("shape", [(64, 512, 784), (1, 10, 16), (17, 33, 48), (100, 70, 1040), (16, 16, 16384), (33, 250, 2064)])
