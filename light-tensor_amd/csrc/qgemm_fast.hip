@@ -1,5 +1,5 @@
 // Tuned int8 GEMM tiles for large NT problems (both operands contiguous in K, K a multiple of the
-// k-step, N a multiple of 16; M and N need not be multiples of the tile: a load that would start past the
+// k-step or, for two of the tiles, of 16; N a multiple of 4; M and N need not be multiples of the tile: a load that would start past the
 // last row of an operand fetches the last row instead, and what is computed from it is not stored):
 // 256 x 256 output tile, k-steps of BK bytes, a ring of S LDS stages filled by
 // direct global->LDS loads (no register staging), MFMA 32x32x32 int8.
@@ -41,7 +41,7 @@ namespace lten_hip {
 #define LTEN_HIP_EXP 0
 #endif
 
-template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false>
+template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false, bool TAIL = false>
 __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 {
 	constexpr int BM = T, BN = T;  // square output tile, 256 or 128
@@ -91,6 +91,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	static_assert((BM / RPL) % W == 0 && LPW % 2 == 0, "A and B loads split evenly over the wavefronts");
 	uint32_t voff[LPW];
 	uint32_t lds_slot[LPW];
+	bool in_tail[LPW];  // TAIL: this lane's chunk lies inside the last, partial k-step
 	const uint32_t smem_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
 #pragma unroll
 	for (int i = 0; i < LPW; i++) {
@@ -99,12 +100,24 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		const int kc = (lane % CPR) ^ swz<CPR>(r);
 		voff[i] = (i < LPW / 2 ? (uint32_t)min(m0 + r, p.M - 1) : (uint32_t)min(n0 + r - BM, p.N - 1)) * (uint32_t)p.K + kc * 16;
 		lds_slot[i] = smem_addr + q * 1024;
+		in_tail[i] = kc * 16 < p.K % BK;
 	}
-	// with SPLIT, blockIdx.y picks this workgroup's share of K
-	const int KT = SPLIT ? p.K / BK / p.splits : p.K / BK;
+	// with SPLIT, blockIdx.y picks this workgroup's share of K; with TAIL the last k-step is partial (K % 16 == 0)
+	const int KT = SPLIT ? p.K / BK / p.splits : (TAIL ? (p.K + BK - 1) / BK : p.K / BK);
 	const uint8_t* const a_base = p.A + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
 	const uint8_t* const b_base = p.B + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
+	// In the partial k-step a lane whose chunk lies past K loads nothing.  For the A tile it stores bytes of 0x80
+	// instead, which the sign flip turns into zeros, so whatever the B tile still holds there is multiplied by 0.
 	auto load_one = [&](int i, int stage, int kt) {
+		if (TAIL && kt == KT - 1 && p.K % BK != 0) {
+			if (in_tail[i]) {
+				async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
+			} else if (i < LPW / 2) {
+				const v4i pad = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+				*reinterpret_cast<v4i*>(smem + (lds_slot[i] - smem_addr) + stage * STAGE + lane * 16) = pad;
+			}
+			return;
+		}
 		async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
 	};
 	auto issue = [&](int stage, int kt) {
@@ -317,11 +330,19 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		}
 		__syncthreads();
 		uint8_t* cout = static_cast<uint8_t*>(p.C) + (int64_t)m0 * p.N + n0;
+		if ((p.N & 15) == 0) {  // rows of C start on 16-byte boundaries: whole 16-byte pieces
 #pragma unroll
-		for (int c = tid; c < BM * BN / 16; c += W * 64) {
-			const int row = c / (BN / 16), ch = c % (BN / 16);
-			if (m0 + row < p.M && n0 + ch * 16 < p.N)  // N is a multiple of 16: whole 16-byte pieces
-				*reinterpret_cast<v4i*>(cout + (int64_t)row * p.N + ch * 16) = *reinterpret_cast<const v4i*>(smem + row * OLD + ch * 16);
+			for (int c = tid; c < BM * BN / 16; c += W * 64) {
+				const int row = c / (BN / 16), ch = c % (BN / 16);
+				if (m0 + row < p.M && n0 + ch * 16 < p.N)
+					*reinterpret_cast<v4i*>(cout + (int64_t)row * p.N + ch * 16) = *reinterpret_cast<const v4i*>(smem + row * OLD + ch * 16);
+			}
+		} else {  // N is a multiple of 4: four bytes at a time
+			for (int c = tid; c < BM * BN / 4; c += W * 64) {
+				const int row = c / (BN / 4), dw = c % (BN / 4);
+				if (m0 + row < p.M && n0 + dw * 4 < p.N)
+					*reinterpret_cast<int*>(cout + (int64_t)row * p.N + dw * 4) = *reinterpret_cast<const int*>(smem + row * OLD + dw * 4);
+			}
 		}
 	}
 #ifdef LTEN_HIP_STAMPS
@@ -330,17 +351,18 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #endif
 }
 
-template <int T, int BK, int WM, int WN, int S>
+template <int T, int BK, int WM, int WN, int S, bool TAIL = false>
 static int launch_fast(const QProblem& p, int out, const char* name)
 {
+	if (!TAIL && p.K % BK != 0) return -1;
 	const dim3 grid((unsigned)(ceil_div(p.M, T) * ceil_div(p.N, T))), block(WM * WN * 64);
 	const bool terms = p.rterm != nullptr;
 	set_kernel_name(name);
-#define LTEN_LAUNCH(OUTV)                                                                        \
-	if (terms)                                                                               \
-		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, true><<<grid, block, 0, stream()>>>(p);     \
-	else                                                                                     \
-		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, false><<<grid, block, 0, stream()>>>(p);
+#define LTEN_LAUNCH(OUTV)                                                                                      \
+	if (terms)                                                                                             \
+		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, true, false, TAIL><<<grid, block, 0, stream()>>>(p);      \
+	else                                                                                                   \
+		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, false, false, TAIL><<<grid, block, 0, stream()>>>(p);
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
@@ -375,7 +397,7 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits)
 {
 	constexpr int T = 128, BK = 128;
 	QProblem p = q;
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 16 == 0 && p.K % (BK * splits) == 0 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % (BK * splits) == 0 &&
 	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
@@ -403,7 +425,8 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits)
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 16 == 0 && p.K % 128 == 0 &&
+	// K: a multiple of the k-step, or (variants 33 and 41) any multiple of 16 at least one k-step long
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % 16 == 0 && p.K >= 128 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0);
@@ -415,10 +438,14 @@ int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 	case 26: return launch_fast<256, 64, 4, 2, 4>(p, out, "qgemm_fast_256x256x64_w4x2_s4");
 	case 28: return launch_fast<256, 64, 4, 2, 2>(p, out, "qgemm_fast_256x256x64_w4x2_s2");
 	case 31: return launch_fast<256, 128, 2, 2, 2>(p, out, "qgemm_fast_256x256x128_w2x2_s2");
-	case 33: return launch_fast<256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
+	case 33:
+		if (p.K % 128 != 0) return launch_fast<256, 128, 2, 4, 2, true>(p, out, "qgemm_fast_256x256x128_w2x4_s2_ktail");
+		return launch_fast<256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
 	case 34: return launch_fast<256, 128, 4, 2, 2>(p, out, "qgemm_fast_256x256x128_w4x2_s2");
 	// 128 x 128 tiles for outputs too small to give every CU a 256 x 256 tile
-	case 41: return launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
+	case 41:
+		if (p.K % 128 != 0) return launch_fast<128, 128, 2, 2, 2, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail");
+		return launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
 	case 42: return launch_fast<128, 128, 2, 2, 3>(p, out, "qgemm_fast_128x128x128_w2x2_s3");
 	case 43: return launch_fast<128, 64, 2, 2, 3>(p, out, "qgemm_fast_128x128x64_w2x2_s3");
 	case 44: return launch_fast<128, 64, 2, 2, 4>(p, out, "qgemm_fast_128x128x64_w2x2_s4");

@@ -141,7 +141,9 @@ def test_fcq_forward_leading_dims(gpu, ob, wl):
 @pytest.mark.parametrize("variant", [41, 42, 43, 44])
 @pytest.mark.parametrize("shape", [(128, 128, 128), (384, 640, 640), (128, 1152, 2048),
                                    # ragged M and N (N a multiple of 16): edge tiles fetch the last row again and store what exists
-                                   (33, 144, 512), (200, 656, 1152), (1, 16, 128)])
+                                   (33, 144, 512), (200, 656, 1152), (1, 16, 128),
+                                   # N a multiple of 4 only: output rows are stored four bytes at a time
+                                   (130, 1000, 256), (64, 12, 640)])
 def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
     """The 128x128 form of the direct-to-LDS tiles (what the library picks when 256x256 tiles would leave CUs idle):
     both k-step sizes, 2 to 4 stages, with and without zero-point terms and bias, short and long K; int32 and u8."""
@@ -154,6 +156,21 @@ def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
     run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8),
              bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
     run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)   # multiplier > 0.99: exact-convert epilogue
+
+
+@pytest.mark.parametrize("variant,shape", [(41, (128, 128, 144)), (41, (200, 272, 784)), (41, (64, 160, 2064)), (33, (300, 272, 400)),
+                                           (33, (256, 512, 912)), (33, (256, 256, 128 + 16))])
+def test_direct_to_lds_tiles_partial_last_k_step(gpu, ob, variant, shape):
+    """K a multiple of 16 but not of the 128-byte k-step: the last step loads only what exists and pads the A tile
+    with bytes that the sign flip turns into zeros; with and without zero-point terms, exact-convert epilogue."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=variant)
+    assert gpu.last_kernel().endswith("ktail"), gpu.last_kernel()
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8), bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
+    run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)
 
 
 @pytest.mark.parametrize("variant", [31, 33, 34])
