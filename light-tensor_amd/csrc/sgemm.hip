@@ -267,6 +267,111 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(lds, asum, p.rowsum, m0, p.M);
 }
 
+// FullyConnected forward at small batch sizes: C[M x N] = A[M x K] B[N x K]^T with M <= 32, a stream over the
+// weights B.  The 32x32 kernels above give such a product N / 32 workgroups; here a workgroup takes 16 columns
+// (N / 16 workgroups: 256 for a 4096-wide layer) on 16x16x4 MFMA tiles, MB = 1 or 2 blocks of 16 activation rows.
+// K is cut into batches of 32, dealt round-robin to the 8 wavefronts; a wave-wide 16-byte load covers 8 rows x 128
+// bytes (whole cache lines), the values pass through a wavefront-private LDS slab (no barrier: LDS operations of one
+// wavefront complete in order) and come back in the MFMA lane layout: lane (r = lane % 16, q = lane / 16) feeds row
+// (or column) r with k = 16h + 4q + t for the MFMA number (h, t) of the batch, the same for both operands.  The loads
+// of the next UB batches are in flight while the current UB are multiplied.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int MB>
+__global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
+{
+	constexpr int WAVES = 8, UB = 2, LD = 36;
+	constexpr int A_SLAB = MB * 16 * LD, B_SLAB = 16 * LD;
+	__shared__ __attribute__((aligned(16))) float lds[WAVES * (A_SLAB + B_SLAB) > WAVES * MB * 256 ? WAVES * (A_SLAB + B_SLAB) : WAVES * MB * 256];
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int r16 = lane & 15, q4 = lane >> 4;
+	const int r8 = lane >> 3, c4 = (lane & 7) * 4;
+	const int n0 = blockIdx.x * 16;
+	float* sA = lds + wave * (A_SLAB + B_SLAB);
+	float* sB = sA + A_SLAB;
+
+	v4f acc[MB];
+#pragma unroll
+	for (int b = 0; b < MB; b++) acc[b] = v4f{ 0.0f, 0.0f, 0.0f, 0.0f };
+
+	struct Batch {
+		float4 a[2 * MB], b[2];
+	};
+	// K % 4 == 0: a float4 lies inside K or outside as a whole
+	auto fetch = [&](int batch, Batch& v) {
+		const int k = batch * 32 + c4;
+#pragma unroll
+		for (int i = 0; i < 2 * MB; i++) {
+			const int m = 8 * i + r8;
+			v.a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (m < p.M && k < p.K) v.a[i] = *reinterpret_cast<const float4*>(p.A + (int64_t)m * p.lda + k);
+		}
+#pragma unroll
+		for (int i = 0; i < 2; i++) {
+			const int n = n0 + 8 * i + r8;
+			v.b[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (n < p.N && k < p.K) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)n * p.ldb + k);
+		}
+	};
+	auto multiply = [&](const Batch& v) {
+#pragma unroll
+		for (int i = 0; i < 2 * MB; i++) *reinterpret_cast<float4*>(sA + (8 * i + r8) * LD + c4) = v.a[i];
+#pragma unroll
+		for (int i = 0; i < 2; i++) *reinterpret_cast<float4*>(sB + (8 * i + r8) * LD + c4) = v.b[i];
+#pragma unroll
+		for (int h = 0; h < 2; h++) {
+			const float4 fb = *reinterpret_cast<const float4*>(sB + r16 * LD + 16 * h + 4 * q4);
+#pragma unroll
+			for (int b = 0; b < MB; b++) {
+				const float4 fa = *reinterpret_cast<const float4*>(sA + (16 * b + r16) * LD + 16 * h + 4 * q4);
+				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.x, fb.x, acc[b], 0, 0, 0);
+				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.y, fb.y, acc[b], 0, 0, 0);
+				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.z, fb.z, acc[b], 0, 0, 0);
+				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.w, fb.w, acc[b], 0, 0, 0);
+			}
+		}
+	};
+
+	const int batches = (p.K + 31) / 32;
+	Batch cur[UB], nxt[UB];
+	int b0 = wave;
+#pragma unroll
+	for (int u = 0; u < UB; u++)
+		if (b0 + u * WAVES < batches) fetch(b0 + u * WAVES, cur[u]);
+	for (; b0 < batches; b0 += WAVES * UB) {
+		const int n0b = b0 + WAVES * UB;
+#pragma unroll
+		for (int u = 0; u < UB; u++)
+			if (n0b + u * WAVES < batches) fetch(n0b + u * WAVES, nxt[u]);
+#pragma unroll
+		for (int u = 0; u < UB; u++)
+			if (b0 + u * WAVES < batches) multiply(cur[u]);
+#pragma unroll
+		for (int u = 0; u < UB; u++) cur[u] = nxt[u];
+	}
+
+	// accumulator register e of lane (r16, q4) of block b: row 16b + 4 q4 + e, column r16.  The wavefronts' partial
+	// tiles meet in LDS (the slabs are no longer needed) and are added in wavefront order.
+	__syncthreads();
+#pragma unroll
+	for (int b = 0; b < MB; b++)
+#pragma unroll
+		for (int e = 0; e < 4; e++) lds[wave * (MB * 256) + (16 * b + 4 * q4 + e) * 16 + r16] = acc[b][e];
+	__syncthreads();
+	for (int idx = tid; idx < MB * 256; idx += WAVES * 64) {
+		const int row = idx >> 4, col = idx & 15;
+		if (row >= p.M || n0 + col >= p.N) continue;
+		float sum = 0.0f;
+#pragma unroll
+		for (int w = 0; w < WAVES; w++) sum += lds[w * (MB * 256) + idx];
+		float* c = p.C + (int64_t)row * p.ldc + n0 + col;
+		float out = p.alpha * sum;
+		if (p.beta != 0.0f) out += p.beta * *c;
+		if (p.bias) out += p.bias[n0 + col];
+		*c = out;
+	}
+}
+
 // Both operands allow 16-byte loads along their contiguous dimension.
 static bool operands_vec(const SProblem& p)
 {
@@ -409,6 +514,15 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	}
 	if (force == 0 && batch == 1 && bias == nullptr && M == 1 && !tB) {
 		launch_rowvec(p, tA);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+	if (force == 0 && !tA && tB && M <= 32 && N >= 512 && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p)) {
+		// a weight stream: 16 columns per workgroup
+		set_kernel_name(M <= 16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
+		const dim3 grid((unsigned)ceil_div(N, 16));
+		if (M <= 16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
+		else sgemm_skinny_nt_kernel<2><<<grid, dim3(512), 0, stream()>>>(p);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}

@@ -331,3 +331,24 @@ def test_direct_to_lds_tiles_ragged_sizes(gpu, tA, tB, M, N, K):
         gpu.set_option("sgemm_tile", 0)
     Am, Bm = A[:, :K & ~31], B[:K & ~31]
     assert np.array_equal(dC.numpy(np.float32, C0.shape)[:, :N], 0.5 * (Am @ Bm) + 2.0 * want)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 512, 256), (5, 1000, 1024), (16, 4096, 512), (17, 520, 4100), (32, 2048, 2048), (29, 1001, 300)])
+def test_small_batch_weight_stream(gpu, M, N, K):
+    """FullyConnected forward with at most 32 rows: the streaming kernel (16 columns per workgroup, 16x16x4 tiles).
+    Integer-valued data make the sums exact in any order; bias, alpha / beta and a padded C are covered."""
+    rng = np.random.default_rng(M * 3 + N + K)
+    x = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    w = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    b = rng.integers(-9, 10, N).astype(np.float32)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    dX, dW, dB, dY = D.from_numpy(x), D.from_numpy(w), D.from_numpy(b), D(4 * M * N)
+    gpu.check(l.lten_hip_fc_forward_f32(M, K, N, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel().startswith("sgemm_skinny_nt"), gpu.last_kernel()
+    assert np.array_equal(dY.numpy(np.float32, (M, N)), x @ w.T + b)
+    ldc = N + 3
+    C0 = np.full((M, ldc), 2.0, np.float32)
+    got = gpu_sgemm(gpu, 0, 1, M, N, K, 0.5, x, K, w, K, 3.0, C0, ldc)
+    assert gpu.last_kernel().startswith("sgemm_skinny_nt")
+    assert np.array_equal(got[:, :N], 0.5 * (x @ w.T) + 6.0)
+    assert (got[:, N:] == 2.0).all()
