@@ -352,3 +352,42 @@ def test_small_batch_weight_stream(gpu, M, N, K):
     assert gpu.last_kernel().startswith("sgemm_skinny_nt")
     assert np.array_equal(got[:, :N], 0.5 * (x @ w.T) + 6.0)
     assert (got[:, N:] == 2.0).all()
+
+
+def test_seeded_sweep_over_dispatch_boundaries(gpu):
+    """Fifty seeded products in all four layouts around the limits at which the library changes kernels (1 / 32 rows,
+    few and many 32x32 tiles, 128-tile counts, leading dimensions that do and do not allow 16-byte loads, K = 1, K a
+    multiple of 32 or not), random alpha / beta, against an fp64 product within 1e-4."""
+    rng = np.random.default_rng(777)
+    seen = set()
+    Ms = [1, 3, 16, 32, 33, 100, 128, 256, 500, 1024, 1536]
+    Ns = [1, 10, 31, 64, 130, 512, 1000, 1024, 2048]
+    Ks = [1, 2, 33, 64, 100, 256, 300, 512, 1000, 1024, 2080]
+    larger = [(2048, 1024, 256), (1030, 2052, 288), (2048, 1024, 300)]   # enough 128 x 128 tiles for the direct-to-LDS kernels
+    for case in range(50 + 4 * len(larger)):
+        if case < 50:
+            M, N, K = int(rng.choice(Ms)), int(rng.choice(Ns)), int(rng.choice(Ks))
+            while M * N * K > 3e8:
+                M = max(1, M // 2)
+            tA, tB = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+            pad_a, pad_b = int(rng.choice([0, 0, 1, 4])), int(rng.choice([0, 0, 3, 4]))
+        else:
+            M, N, K = larger[(case - 50) // 4]
+            tA, tB = (case - 50) % 4 // 2, (case - 50) % 2
+            pad_a, pad_b = 4, 0
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        B = rng.standard_normal((K, N)).astype(np.float32)
+        lda, ldb, ldc = (M if tA else K) + pad_a, (K if tB else N) + pad_b, N + int(rng.choice([0, 5]))
+        As = np.zeros(((K if tA else M), lda), np.float32)
+        As[:, :(M if tA else K)] = A.T if tA else A
+        Bs = np.zeros(((N if tB else K), ldb), np.float32)
+        Bs[:, :(K if tB else N)] = B.T if tB else B
+        alpha, beta = float(rng.choice([1.0, 0.5, -2.0])), float(rng.choice([0.0, 0.0, 1.0, 0.25]))
+        C0 = rng.standard_normal((M, ldc)).astype(np.float32)
+        got = gpu_sgemm(gpu, tA, tB, M, N, K, alpha, As, lda, Bs, ldb, beta, C0, ldc)
+        name = gpu.last_kernel()
+        seen.add(name.split("_")[1])
+        want = alpha * (A.astype(np.float64) @ B.astype(np.float64)) + beta * C0[:, :N].astype(np.float64)
+        assert rel_err(got[:, :N], want) < TOL, (case, tA, tB, M, N, K, lda, ldb, alpha, beta, name)
+        assert np.array_equal(got[:, N:], C0[:, N:]), (case, name)
+    assert {"fast", "staged", "direct", "rowvec", "rank1"} <= seen, seen

@@ -374,3 +374,30 @@ def test_cfg4_skinny(gpu, wl, M):
     assert np.array_equal(accg, want)
     mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
     assert np.array_equal(Cg, requant_numpy(want, mult, int(zp[2])))
+
+
+def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
+    """Sixty seeded shapes around the limits at which the library changes kernels (32 / 64 rows, 128-tile edges, N a
+    multiple of 4 or not, K a multiple of 16 / 128 or not, short and long K), each with random zero points, with and
+    without bias, u8 and int32 outputs against the oracle; the kernel names show that every family took part."""
+    rng = np.random.default_rng(20240607)
+    seen = set()
+    Ms = [1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 100, 127, 128, 129, 200, 255, 257, 300]
+    Ns = [1, 10, 16, 36, 100, 128, 130, 132, 256, 500, 512, 1000, 1024, 2048, 2052]
+    Ks = [1, 7, 16, 48, 100, 128, 144, 512, 528, 784, 1000, 1024, 2048, 2064, 4096]
+    larger = [(300, 1000, 1024), (129, 2052, 784), (257, 516, 2064), (200, 1024, 144)]   # past the one-launch kernel's 512 tiles
+    for case in range(60 + len(larger)):
+        if case < 60:
+            M, N, K = int(rng.choice(Ms)), int(rng.choice(Ns)), int(rng.choice(Ks))
+            while M * N * K > 6e7:
+                M = max(1, M // 2)
+        else:
+            M, N, K = larger[case - 60]
+        A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+        B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+        zp = np.array([rng.choice([0, 128, int(rng.integers(0, 256))]) for _ in range(3)], np.uint8)
+        sc = [0.02, 0.013, float(rng.choice([0.9, 0.05, 7.0]))]
+        bias = rng.integers(-20000, 20000, N).astype(np.int32) if rng.integers(0, 2) else None
+        run_case(gpu, ob, A, B, sc, zp, bias=bias)
+        seen.add(gpu.last_kernel().split("_")[0] + "_" + gpu.last_kernel().split("_")[1])
+    assert {"qskinny_mfma", "qdirect_16x16", "qgemm_fast", "qgemm_guard"} <= seen, seen
