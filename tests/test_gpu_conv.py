@@ -171,3 +171,23 @@ def test_cfg5_full_size(gpu, wl):
         sc = float(np.sqrt((dx.astype(np.float64) ** 2).mean()))
         assert (np.abs(got_dx - want_dx) / np.maximum(np.abs(want_dx), sc)).max() < TOL, gpu.last_kernel()
         inp = y
+
+
+def test_seeded_sweep_over_geometries(gpu, ob):
+    """Forty seeded geometries (channel counts on both sides of the kernels' limits, 1x1 / 3x3 / 5x5 / oblong windows,
+    stride 1 and 2, pad 0..2, widths that are and are not multiples of four): forward, weight gradient and data gradient
+    against the oracle, with whatever kernel the library picks."""
+    rng = np.random.default_rng(31415)
+    seen = set()
+    for case in range(40):
+        Cin = int(rng.choice([1, 2, 3, 4, 8, 12, 16, 20, 33]))
+        Cout = int(rng.choice([1, 7, 16, 32, 40, 64, 70]))
+        kh, kw = [(1, 1), (3, 3), (3, 3), (3, 3), (5, 5), (2, 3), (3, 1)][int(rng.integers(0, 7))]
+        sh = sw = int(rng.choice([1, 1, 1, 2]))
+        ph, pw = int(rng.integers(0, min(kh, 3))), int(rng.integers(0, min(kw, 3)))
+        H, W = int(rng.integers(kh + 1, 24)), int(rng.choice([8, 12, 17, 20, 36, 132, 140]))
+        N = int(rng.integers(1, 4))
+        geo = (N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)
+        _conv_vs_oracle(gpu, ob, geo)
+        seen.add(gpu.last_kernel())
+    print(sorted(seen))
