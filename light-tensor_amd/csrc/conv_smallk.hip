@@ -204,44 +204,67 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 
 // Weight gradient: dw[co][k] = sum over pixels of dy[co][pixel] * patch_k[pixel].  MFMA rows = 32 output
 // channels, columns = taps (lanes whose column is >= K compute values nobody stores), reduction = the
-// wavefront's 32 pixels of every chunk.  dy goes from global memory straight into the A operand: lane
-// (co, half) loads four consecutive pixels at 8u + 4*half, so the 32-byte pieces a wavefront touches add up
-// to whole rows over four loads.  Step (u, e) multiplies pixels 8u + e (lanes 0-31) and 8u + 4 + e (lanes 32-63).
-template <bool VEC, int RC>
-__global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy,
+// wavefront's 32 pixels of every chunk.  Step (u, e) multiplies pixels 8u + e (lanes 0-31) and 8u + 4 + e
+// (lanes 32-63), so lane (co, half) needs the four consecutive pixels at 8u + 4*half of row co.  With VEC the
+// wavefront's 32 x 32 piece of dy is fetched as four loads of 8 rows x 128 bytes (whole cache lines: a load in the
+// operand's own layout would touch 32 lines for 32 bytes each, and the line lookups, not the bytes, then set the
+// pace) and turned into that layout through a wavefront-private LDS slab.
+// WPG = 4 or 8 wavefronts per workgroup: with 8, wavefronts 4-7 take every other chunk of the workgroup's range, so
+// that twice as many loads are in flight per CU for the same number of partial sums.
+template <bool VEC, int RC, int WPG>
+__global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy,
                                                                   float* __restrict__ partial, int chunks_per_part)
 {
 	using S = SkShape<RC>;
-	constexpr int RED = 3 * 16 * 64;  // three wavefronts' accumulator tiles for the final sum
-	__shared__ __attribute__((aligned(16))) float s_mem[8 * S::PATCH > RED ? 8 * S::PATCH : RED];
-	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
+	constexpr int RED = (WPG - 1) * 16 * 64;  // the other wavefronts' accumulator tiles for the final sum
+	constexpr int DLD = 36, DSLAB = 32 * DLD;  // dy slab of a wavefront: [32 channels][32 pixels], rows of 36 floats
+	constexpr int USED = WPG * 2 * S::PATCH + WPG * DSLAB;
+	constexpr int STRIDE = WPG / 4;            // chunks between two of a wavefront's
+	__shared__ __attribute__((aligned(16))) float s_mem[USED > RED ? USED : RED];
+	const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, lrow = lane & 31, half = lane >> 5;
+	const int wave = wid & 3;  // which 32 pixels of a chunk
 	const int K = g.Cin * g.kh * g.kw;
 	const int co0 = blockIdx.y * 32, co = co0 + lrow;
 	const int tiles_w = (g.Wo + SK_TW - 1) / SK_TW, total = g.N * g.Ho * tiles_w;
-	const int begin = blockIdx.x * chunks_per_part, end = min(total, begin + chunks_per_part);
+	const int begin = blockIdx.x * chunks_per_part + (wid >> 2), end = min(total, (int)blockIdx.x * chunks_per_part + chunks_per_part);
 
-	float* const mine = s_mem + wave * 2 * S::PATCH;  // this wavefront's two buffers
+	float* const mine = s_mem + wid * 2 * S::PATCH;  // this wavefront's two buffers
+	float* const dslab = s_mem + WPG * 2 * S::PATCH + wid * DSLAB;
+	const int r8 = lane >> 3, c4 = (lane & 7) * 4;     // whole-line loads: lane -> (row within a group of 8, 4 pixels)
 
 	const int boff = (lrow < K ? tap_offset(g, lrow) : 0) + 4 * half + 4 - g.pw;
 	// dy: the address is a part all lanes share plus this lane's offset; with VEC (Wo % 4 == 0) the four
 	// pixels of a load are inside or outside the row together
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
-	const unsigned dy_lane = (unsigned)(lrow * plane) + wave * 32 + 4 * half;
+	const unsigned dy_lane = VEC ? (unsigned)(r8 * plane) + wave * 32 + c4 : (unsigned)(lrow * plane) + wave * 32 + 4 * half;
 	const bool co_ok = co < g.Cout;
+	// VEC: a[i] = rows 8i + r8, pixels c4 .. c4+3 (to be staged); else a[u] = the operand itself
 	auto load_dy = [&](const Chunk& c, float4 (&a)[4]) {
 		const float* dc = dy + (((int64_t)c.n * g.Cout + co0) * g.Ho + c.ho) * g.Wo + c.w0;  // same for the whole workgroup
+		if (VEC) {
+			const bool col_ok = c.w0 + wave * 32 + c4 < g.Wo;
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+				if (col_ok && co0 + 8 * i + r8 < g.Cout) a[i] = *reinterpret_cast<const float4*>(dc + 8 * i * plane + dy_lane);
+			}
+			return;
+		}
 		const int col = c.w0 + wave * 32 + 4 * half;
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
 			a[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (co_ok) {
-				if (VEC) {
-					if (col + 8 * u < g.Wo) a[u] = *reinterpret_cast<const float4*>(dc + 8 * u + dy_lane);
-				} else {
-					a[u] = load_row4<false>(dc + dy_lane - (wave * 32 + 4 * half) - c.w0, col + 8 * u, g.Wo);
-				}
-			}
+			if (co_ok) a[u] = load_row4<false>(dc + dy_lane - (wave * 32 + 4 * half) - c.w0, col + 8 * u, g.Wo);
 		}
+	};
+	// VEC: through the slab into the operand layout
+	auto stage_dy = [&](const float4 (&v)[4]) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) *reinterpret_cast<float4*>(dslab + (8 * i + r8) * DLD + c4) = v[i];
+	};
+	auto operand_dy = [&](float4 (&a)[4]) {
+#pragma unroll
+		for (int u = 0; u < 4; u++) a[u] = *reinterpret_cast<const float4*>(dslab + lrow * DLD + 8 * u + 4 * half);
 	};
 
 	v16f acc;
@@ -256,14 +279,17 @@ __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, con
 		fetch_patch<VEC>(g, x, c, pr);
 		load_dy(c, a_cur);
 		store_patch(mine, lane, pr);
+		if (VEC) stage_dy(a_cur);
 	}
-	for (int chunk = begin; chunk < end; chunk++) {
-		const int cur = (chunk - begin) & 1;
-		c = next_chunk(g, c);
-		if (chunk + 1 < end) {
+	for (int chunk = begin; chunk < end; chunk += STRIDE) {
+		const int cur = ((chunk - begin) / STRIDE) & 1;
+#pragma unroll
+		for (int q = 0; q < STRIDE; q++) c = next_chunk(g, c);
+		if (chunk + STRIDE < end) {
 			fetch_patch<VEC>(g, x, c, pr);
 			load_dy(c, a_next);
 		}
+		if (VEC) operand_dy(a_cur);  // the slab is free again once these reads are issued (one wavefront, in order)
 		const float* pb = mine + cur * S::PATCH + boff;
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
@@ -272,28 +298,31 @@ __global__ __launch_bounds__(256) void conv2d_smallk_wgrad_kernel(ConvGeo g, con
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[u].z, pb[8 * u + 2], acc, 0, 0, 0);
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[u].w, pb[8 * u + 3], acc, 0, 0, 0);
 		}
-		if (chunk + 1 < end) {
+		if (chunk + STRIDE < end) {
 			store_patch(mine + (cur ^ 1) * S::PATCH, lane, pr);
+			if (VEC) stage_dy(a_next);
+			else {
 #pragma unroll
-			for (int u = 0; u < 4; u++) a_cur[u] = a_next[u];
+				for (int u = 0; u < 4; u++) a_cur[u] = a_next[u];
+			}
 		}
 	}
 
 	// add the four wavefronts' tiles in wavefront order, then lanes whose column is a tap store
 	float* red = s_mem;
 	__syncthreads();  // every wavefront is done with its patch buffers
-	if (wave != 0) {
+	if (wid != 0) {
 #pragma unroll
-		for (int r = 0; r < 16; r++) red[((wave - 1) * 16 + r) * 64 + lane] = acc[r];
+		for (int r = 0; r < 16; r++) red[((wid - 1) * 16 + r) * 64 + lane] = acc[r];
 	}
 	__syncthreads();
-	if (wave != 0 || lrow >= K) return;
+	if (wid != 0 || lrow >= K) return;
 	float* out = partial + (int64_t)blockIdx.x * g.Cout * K;
 #pragma unroll
 	for (int r = 0; r < 16; r++) {
 		float v = acc[r];
 #pragma unroll
-		for (int q = 0; q < 3; q++) v += red[(q * 16 + r) * 64 + lane];
+		for (int q = 0; q < WPG - 1; q++) v += red[(q * 16 + r) * 64 + lane];
 		const int row = co0 + (r >> 2) * 8 + half * 4 + (r & 3);
 		if (row < g.Cout) out[(int64_t)row * K + lrow] = v;
 	}
@@ -350,12 +379,12 @@ int conv_smallk_wgrad(const ConvGeo& g, const float* x, const float* dy, float* 
 	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
 	if (smallk_small(g)) {
 		set_kernel_name("conv2d_smallk_wgrad_32x128_r8");
-		if (vec) conv2d_smallk_wgrad_kernel<true, 8><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
-		else conv2d_smallk_wgrad_kernel<false, 8><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		if (vec) conv2d_smallk_wgrad_kernel<true, 8, 8><<<grid, dim3(512), 0, stream()>>>(g, x, dy, partial, per);
+		else conv2d_smallk_wgrad_kernel<false, 8, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
 	} else {
 		set_kernel_name("conv2d_smallk_wgrad_32x128");
-		if (vec) conv2d_smallk_wgrad_kernel<true, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
-		else conv2d_smallk_wgrad_kernel<false, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		if (vec) conv2d_smallk_wgrad_kernel<true, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		else conv2d_smallk_wgrad_kernel<false, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
