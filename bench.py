@@ -285,7 +285,7 @@ def extra_configs(lt, wl, with_cpu):
     gc = D(4 * n * n)
     per_layout = {}
     for name, (ta, tb) in (("NT", (0, 1)), ("NN", (0, 0)), ("TN", (1, 0))):
-        ms = timed(lt, lambda: lt.sgemm(ta, tb, n, n, n, 1.0, ga, n, gb, n, 0.0, gc, n), 10)
+        ms = timed(lt, lambda: lt.sgemm(ta, tb, n, n, n, 1.0, ga, n, gb, n, 0.0, gc, n), 10, warmup=10)
         per_layout[name] = round(ms * 1e3, 1)
     kname = lt.last_kernel()
     ms = sum(per_layout.values()) / 3e3
