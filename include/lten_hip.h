@@ -213,6 +213,12 @@ int lten_hip_sgd_step_f32(float* weight, float* weight_grad, float* velocity, ui
 int lten_hip_adam_step_f32(float* weight, const float* weight_grad, float* v_dw, float* s_dw, uint64_t numels, float lr,
                            float beta1, float beta2, uint64_t iteration);
 
+/* The gradient of a Conv2d bias: db[c] = (accumulate ? db[c] : 0) + sum over n, h, w of dy[n][c][h*w].  l-ten adds the
+ * bias {1, C, 1, 1} to the convolution's result as a tensor op (l-ten/conv2d.cpp:189-192), so this is the backward
+ * pass of that broadcast add (l-ten/backprop.cpp:605-690: the top gradient summed over the broadcast dimensions).
+ * Up to 4096 channels; two launches, partial sums in a device array of the library. */
+int lten_hip_conv2d_bias_grad_f32(uint64_t N, uint64_t C, uint64_t HW, const float* dy, float* db, int accumulate);
+
 /* ------------------------------------------------------------------ quantization helpers */
 
 /* Quantize / Dequantize / GetMinMax of l-ten/utils.h:23-26 (l-ten/utils.cpp:198-262) with the data on the device;

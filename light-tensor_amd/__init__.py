@@ -77,6 +77,7 @@ _SIGNATURES = {
     "lten_hip_quantize_i32": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_dequantize_u8": (C.c_int, [vp, vp, u64, C.POINTER(QParams)]),
     "lten_hip_get_min_max": (C.c_int, [vp, u64, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "lten_hip_conv2d_bias_grad_f32": (C.c_int, [u64, u64, u64, vp, vp, C.c_int]),
     "lten_hip_graph_begin": (C.c_int, []),
     "lten_hip_graph_end": (C.c_int, [C.POINTER(vp)]),
     "lten_hip_graph_launch": (C.c_int, [vp]),

@@ -136,6 +136,45 @@ __global__ __launch_bounds__(256) void adam_step_kernel(float* __restrict__ w, c
 
 static unsigned grid_for(uint64_t n) { return (unsigned)std::min<uint64_t>(ceil_div(n, 256), 256 * 16); }
 
+// Channel sums of an NCHW gradient: db[c] (+)= sum over n, h, w of dy[n][c][h][w] — what the backward pass of the
+// broadcast add leaves in the bias of a convolution (l-ten/conv2d.cpp:189-192 adds the bias {1, C, 1, 1} as a
+// tensor op; l-ten/backprop.cpp:605-690 sums the top gradient over the broadcast dimensions).  Workgroup (c, s) adds
+// slice s of the images of channel c; a second launch adds the slices in slice order.  The partial sums live in a
+// small device array of the library.
+constexpr int CHANNEL_SUM_SLOTS = 4096;
+static __device__ float g_channel_partial[CHANNEL_SUM_SLOTS];
+
+__global__ __launch_bounds__(256) void channel_sum_partial_kernel(const float* __restrict__ dy, int N, int C, int64_t HW, int slices, float* __restrict__ partial)
+{
+	__shared__ float part[4];
+	const int c = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+	// the slice's share of the N * HW values of channel c, taken in runs of 256 consecutive values; (n, hw) advance
+	// by a fixed step without a division per element
+	const int64_t step = (int64_t)slices * 256, step_n = step / HW, step_hw = step % HW;
+	int64_t n = ((int64_t)s * 256 + tid) / HW, hw = ((int64_t)s * 256 + tid) % HW;
+	float sum = 0.0f;
+	while (n < N) {
+		sum += dy[(n * C + c) * HW + hw];
+		n += step_n;
+		hw += step_hw;
+		if (hw >= HW) { hw -= HW; n++; }
+	}
+#pragma unroll
+	for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off);
+	if ((tid & 63) == 0) part[tid >> 6] = sum;
+	__syncthreads();
+	if (tid == 0) partial[c * slices + s] = ((part[0] + part[1]) + part[2]) + part[3];
+}
+
+__global__ __launch_bounds__(256) void channel_sum_final_kernel(const float* __restrict__ partial, int C, int slices, float* __restrict__ db, int accumulate)
+{
+	const int c = blockIdx.x * 256 + threadIdx.x;
+	if (c >= C) return;
+	float sum = 0.0f;
+	for (int s = 0; s < slices; s++) sum += partial[c * slices + s];
+	db[c] = accumulate ? db[c] + sum : sum;
+}
+
 }  // namespace lten_hip
 
 using namespace lten_hip;
@@ -226,6 +265,24 @@ int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, 
 	LTEN_HIP_REQUIRE(loss != nullptr && batches > 0, "nll_loss: null loss pointer or zero batch");
 	LTEN_HIP_REQUIRE(len == 0 || (input && target), "nll_loss: null pointer");
 	nll_loss_kernel<<<dim3(1), dim3(1024), 0, stream()>>>(input, target, loss, len, -1.0f / (float)batches);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_conv2d_bias_grad_f32(uint64_t N, uint64_t C, uint64_t HW, const float* dy, float* db, int accumulate)
+{
+	if (C == 0) return 0;
+	LTEN_HIP_REQUIRE(db != nullptr, "conv2d_bias_grad: db is null");
+	LTEN_HIP_REQUIRE(N * HW == 0 || dy != nullptr, "conv2d_bias_grad: dy is null");
+	LTEN_HIP_REQUIRE(C <= CHANNEL_SUM_SLOTS && N < (1ull << 31) && HW < (1ull << 40), "conv2d_bias_grad: more than %d channels", CHANNEL_SUM_SLOTS);
+	const uint64_t runs = ceil_div(N * HW, 256);
+	const int slices = (int)std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(CHANNEL_SUM_SLOTS / C, 64), runs));
+	float* partial = nullptr;
+	LTEN_HIP_CHECK(hipGetSymbolAddress(reinterpret_cast<void**>(&partial), HIP_SYMBOL(g_channel_partial)));
+	set_kernel_name("channel_sum");
+	channel_sum_partial_kernel<<<dim3((unsigned)C, (unsigned)slices), dim3(256), 0, stream()>>>(dy, (int)N, (int)C, (int64_t)HW, slices, partial);
+	LTEN_HIP_LAUNCH_CHECK();
+	channel_sum_final_kernel<<<dim3((unsigned)ceil_div(C, 256)), dim3(256), 0, stream()>>>(partial, (int)C, slices, db, accumulate);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

@@ -667,10 +667,16 @@ Tensor Conv2d::forward(Tensor& input)
 	if (!scratch_.defined() || scratch_.get_numels() < need) scratch_ = AllocateTensor({ need }, &options);
 	auto wt = weight_.get_smart_ptr(), in = input.get_smart_ptr(), scratch = scratch_.get_smart_ptr();
 	const bool with_bias = use_bias_;
+	auto bs = use_bias_ ? bias_.get_smart_ptr() : std::shared_ptr<TensorImpl>();
 	result.get_smart_ptr()->children = { wt, in };  // l-ten/conv2d.cpp:183-187
 	result.get_smart_ptr()->autograd = true;
 	result.get_smart_ptr()->grad_fn = [=](TensorImpl&, const float* top) {
-		if (with_bias) LTEN_ERR("the gradient of the Conv2d bias is not part of the GPU path (l-ten adds the bias as a separate tensor op)");
+		if (with_bias && wants_gradient(bs)) {
+			// l-ten/conv2d.cpp:189-192 adds the bias as a broadcast tensor op; its backward pass (l-ten/backprop.cpp:605-690)
+			// sums the top gradient over N, H, W into the bias gradient
+			bs->ensure_grad();
+			LTEN_HIP_CALL(lten_hip_conv2d_bias_grad_f32(N, Cout, (uint64_t)Ho * Wo, top, static_cast<float*>(bs->grad), 1));
+		}
 		float* work = static_cast<float*>(scratch->data);
 		float* tmp_dw = work + work_floats;
 		float* tmp_dx = tmp_dw + Cout * Kc;

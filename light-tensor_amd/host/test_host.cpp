@@ -344,14 +344,21 @@ static int conv_test()
 	lten::Tensor X = lten::TensorFromBuffer({ (uint64_t)N, (uint64_t)Cin, (uint64_t)H, (uint64_t)W }, x.data());
 	X.set_autograd(true);
 	X = X.to(lten::GPU);
-	lten::Conv2d conv(Cin, Cout, false, kh, kw, ph, pw, sh, sw);
+	lten::Conv2d conv(Cin, Cout, true, kh, kw, ph, pw, sh, sw);  // with bias: its gradient is the channel sum of dy
 	conv.init();
 	memcpy(conv.get_weights()->get_data_ptr(), w.data(), w.size() * 4);
+	std::vector<float> bias(Cout);
+	for (auto& e : bias) e = rnd();
+	memcpy(conv.get_bias()->get_data_ptr(), bias.data(), bias.size() * 4);
 	conv.to(lten::GPU);
 	lten::Tensor Y = conv.forward(X);
 	lten::Tensor T = lten::TensorFromBuffer({ (uint64_t)N, (uint64_t)Cout, (uint64_t)Ho, (uint64_t)Wo }, dy.data()).to(lten::GPU);
 	Y.backward(&T);
-	std::vector<float> y(N * Cout * Ho * Wo, 0), dw(w.size(), 0), dx(x.size(), 0);
+	std::vector<float> y(N * Cout * Ho * Wo, 0), dw(w.size(), 0), dx(x.size(), 0), db(Cout, 0);
+	for (int n = 0; n < N; n++) for (int co = 0; co < Cout; co++) for (int p = 0; p < Ho * Wo; p++) {
+		y[(n * Cout + co) * Ho * Wo + p] = bias[co];
+		db[co] += dy[(n * Cout + co) * Ho * Wo + p];
+	}
 	for (int n = 0; n < N; n++) for (int co = 0; co < Cout; co++) for (int ho = 0; ho < Ho; ho++) for (int wo = 0; wo < Wo; wo++)
 		for (int ci = 0; ci < Cin; ci++) for (int i = 0; i < kh; i++) for (int j = 0; j < kw; j++) {
 			const int yy = ho * sh - ph + i, xx = wo * sw - pw + j;
@@ -366,6 +373,7 @@ static int conv_test()
 	if (Compare((float*)Yc.get_data_ptr(), y.data(), y.size(), tol)) return -1;
 	if (Compare(grad_to_host(*conv.get_weights()).data(), dw.data(), dw.size(), tol)) return -2;
 	if (Compare(grad_to_host(X).data(), dx.data(), dx.size(), tol)) return -3;
+	if (Compare(grad_to_host(*conv.get_bias()).data(), db.data(), db.size(), tol)) return -4;
 	return 0;
 }
 

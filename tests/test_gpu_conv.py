@@ -191,3 +191,24 @@ def test_seeded_sweep_over_geometries(gpu, ob):
         _conv_vs_oracle(gpu, ob, geo)
         seen.add(gpu.last_kernel())
     print(sorted(seen))
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (2, 5, 7), (3, 70, 33 * 29), (32, 64, 128 * 128), (4, 4096, 6), (5, 3, 1000)])
+def test_conv_bias_gradient(gpu, shape):
+    """db[c] = sum over n, h, w of dy: integer-valued data make the sum exact in any order; then random data against
+    an fp64 sum, overwrite and accumulate."""
+    N, C, HW = shape
+    rng = np.random.default_rng(N + C + HW)
+    dy = rng.integers(-3, 4, (N, C, HW)).astype(np.float32)
+    db0 = rng.integers(-20, 20, C).astype(np.float32)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    dDY, dDB = D.from_numpy(dy), D.from_numpy(db0)
+    gpu.check(l.lten_hip_conv2d_bias_grad_f32(N, C, HW, dDY.ptr, dDB.ptr, 1))
+    assert np.array_equal(dDB.numpy(np.float32, (C,)), db0 + dy.sum(axis=(0, 2)))
+    gpu.check(l.lten_hip_conv2d_bias_grad_f32(N, C, HW, dDY.ptr, dDB.ptr, 0))
+    assert np.array_equal(dDB.numpy(np.float32, (C,)), dy.sum(axis=(0, 2)))
+    r = rng.standard_normal((N, C, HW)).astype(np.float32)
+    dR = D.from_numpy(r)
+    gpu.check(l.lten_hip_conv2d_bias_grad_f32(N, C, HW, dR.ptr, dDB.ptr, 0))
+    assert rel_err(dDB.numpy(np.float32, (C,)), r.astype(np.float64).sum(axis=(0, 2))) < TOL
+    assert l.lten_hip_conv2d_bias_grad_f32(1, 5000, 4, dR.ptr, dDB.ptr, 0) != 0   # more channels than the library's partial array
