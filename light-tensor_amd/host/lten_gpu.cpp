@@ -418,6 +418,35 @@ static void require_gpu_f32(const Tensor& t, const char* what)
 	}
 }
 
+Tensor Tensor::reshape(const std::initializer_list<uint64_t>& dims)
+{
+	uint64_t count = 1;
+	for (uint64_t d : dims) count *= d;
+	if (count != impl_->numels) LTEN_ERR("reshape: the number of elements must stay the same");
+	TensorOps options;
+	options.data_type = impl_->data_type;
+	options.device_type = impl_->dev;
+	options.device_index = impl_->dev_index;
+	Tensor result = TensorFromBuffer(dims, impl_->data, false, &options);
+	auto in = impl_;
+	result.get_smart_ptr()->children = { in };  // keeps the shared buffer alive (l-ten/tensorimpl.cpp:2044)
+	if (wants_gradient(in)) {
+		if (impl_->data_type != FLOAT32) LTEN_ERR("reshape: gradients are implemented for FLOAT32 tensors only");
+		const uint64_t n = impl_->numels;
+		result.get_smart_ptr()->autograd = true;
+		result.get_smart_ptr()->grad_fn = [in, n](TensorImpl&, const float* top) {  // l-ten/backprop.cpp:2475-2505: a copy of the top gradient
+			if (in->grad_fn) {
+				in->grad_fn(*in, top);  // same values, same order: handed on as it is
+			} else {
+				in->ensure_grad();
+				if (in->dev == GPU) LTEN_HIP_CALL(lten_hip_axpy_f32(n, 1.0f, top, static_cast<float*>(in->grad)));
+				else for (uint64_t i = 0; i < n; i++) static_cast<float*>(in->grad)[i] += top[i];
+			}
+		};
+	}
+	return result;
+}
+
 Tensor relu(Tensor& input)
 {
 	require_gpu_f32(input, "relu");

@@ -78,6 +78,9 @@ public:
 	Tensor to(device target_device, int target_device_index = 0);
 	// l-ten/tensor.h:83-138: batched matrix product over the leading dims, size-1 dims broadcast.
 	Tensor matmul(const Tensor& other);
+	// l-ten/tensor.h:1152-1200, l-ten/tensorimpl.cpp:2033-2052: the same buffer under other dimensions (same element
+	// count); the source stays alive as the result's child and receives the result's gradient unchanged.
+	Tensor reshape(const std::initializer_list<uint64_t>& dims);
 	// l-ten/tensor.h:69 backward(MultiDimArray<float>* top_gradient): top_gradient has the tensor's shape and
 	// lives on the tensor's device; null stands for a single 1 and is only valid for one-element tensors.
 	void backward(const Tensor* top_gradient = nullptr);

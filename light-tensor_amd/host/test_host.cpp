@@ -247,6 +247,61 @@ static int training_test()
 	return 0;
 }
 
+// Conv2d (with bias) -> relu -> reshape -> FullyConnected trained on the device in l-ten's style: 12 x 12 images with
+// a bright 4 x 4 blob in one of four quadrants, the label is the quadrant.
+static int conv_training_test()
+{
+	class Net : public lten::NeuralNetwork {
+	public:
+		Net()
+		{
+			conv1 = register_module("conv1", lten::Conv2d(1, 8, true, 3, 3, 1, 1));
+			fc1 = register_module("fc1", lten::FullyConnected(8 * 12 * 12, 4, true));
+		}
+		lten::Tensor forward(lten::Tensor input)
+		{
+			lten::Tensor c = conv1->forward(input);
+			lten::Tensor a = lten::relu(c);
+			lten::Tensor flat = a.reshape({ input.get_sizes()[0], 1, 1, 8 * 12 * 12 });
+			return fc1->forward(flat);
+		}
+		lten::Conv2d* conv1;
+		lten::FullyConnected* fc1;
+	};
+	const uint64_t B = 32, S = 12, C = 4;
+	unsigned s = 99;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (float)((s >> 8) & 0xFFFF) / 65536.0f; };
+	Net net;
+	lten::AdamOptimizer adam;
+	adam.set_learning_rate(0.003f);
+	net.to(lten::GPU);
+	adam.attach_network(net);
+	float first = 0.0f, last = 0.0f;
+	for (int it = 0; it < 150; it++) {
+		std::vector<float> x(B * S * S), t(B * C, 0.0f);
+		for (uint64_t m = 0; m < B; m++) {
+			const int quadrant = (int)(rnd() * 4) & 3, oy = (quadrant / 2) * 6 + 1, ox = (quadrant % 2) * 6 + 1;
+			for (uint64_t p = 0; p < S * S; p++) x[m * S * S + p] = 0.2f * rnd();
+			for (int dy = 0; dy < 4; dy++) for (int dx = 0; dx < 4; dx++) x[m * S * S + (oy + dy) * S + ox + dx] += 1.0f;
+			t[m * C + quadrant] = 1.0f;
+		}
+		lten::Tensor X = lten::TensorFromBuffer({ B, 1, S, S }, x.data()).to(lten::GPU);
+		lten::Tensor T = lten::TensorFromBuffer({ B, 1, 1, C }, t.data()).to(lten::GPU);
+		lten::Tensor y = net.forward(X);
+		lten::Tensor lp = lten::log_softmax(y, 3);
+		lten::Tensor loss = lten::nll_loss(lp, T);
+		loss.backward();
+		adam.step();
+		adam.zero_grad();
+		if (it == 0 || it == 149) {
+			lten::Tensor lc = loss.to(lten::CPU);
+			(it == 0 ? first : last) = *(float*)lc.get_data_ptr();
+		}
+	}
+	printf("  conv net: loss %.4f -> %.4f\n", first, last);
+	return (last < 0.2f * first && last < 0.3f) ? 0 : -1;
+}
+
 // FullyConnected_q on {2, 3, 37} with bias: every leading index is its own quantized_matmul in l-ten
 static int fcq_test()
 {
@@ -402,7 +457,7 @@ static int error_test()
 
 int main()
 {
-	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test }, { "training_test", training_test },
+	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test }, { "training_test", training_test }, { "conv_training_test", conv_training_test },
 		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;
 	for (auto& t : tests) {
