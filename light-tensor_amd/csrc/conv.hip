@@ -318,7 +318,7 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
 	// enough for whichever kernel the call picks
 	uint64_t parts = (uint64_t)N * slices;
 	if (conv_smallk_takes(g)) parts = std::max<uint64_t>(parts, conv_smallk_wgrad_parts(g));
-	if (conv_patch_wgrad_takes(g)) parts = std::max<uint64_t>(parts, conv_patch_wgrad_parts(g));
+	if (conv_patch_wgrad_takes(g)) parts = std::max<uint64_t>(parts, conv_patch_wgrad_parts(g, true));
 	return parts * Cout * Cin * kh * kw * sizeof(float);
 }
 

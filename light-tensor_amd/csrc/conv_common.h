@@ -19,7 +19,7 @@ int conv_patch_forward(const ConvGeo& g, const float* x, const float* w, const f
 bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float* w);
 int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y);
 bool conv_patch_wgrad_takes(const ConvGeo& g);
-int conv_patch_wgrad_parts(const ConvGeo& g);  // partial [Cout x Cin*kh*kw] matrices the kernel writes
+int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound = false);  // partial [Cout x Cin*kh*kw] matrices the kernel writes
 int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts);
 
 // Kernels for stride 1, dilation 1 and Cin*kh*kw <= 32 (first layers): the whole reduction fits one MFMA tile

@@ -14,6 +14,7 @@
 #include "gemm_f32_core.h"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace lten_hip {
 
@@ -198,12 +199,17 @@ struct PatchWgrad {
 	static_assert(DY_F4 % T == 0 && TAPS_PER_ROUND >= 1, "tile shape");
 };
 
-template <int KH, int KW, bool VEC>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv2d_patch_wgrad_kernel(
+// PIPE: one workgroup per CU with two LDS buffers.  The tiles of chunk c + 1 are stored to the other buffer during
+// the last third of chunk c's MFMAs, one 4-byte store behind each MFMA, so that the matrix pipe does not wait while
+// a workgroup refills its tiles, and a chunk costs one barrier.  Without PIPE: two workgroups per CU, one buffer,
+// store - barrier - multiply - barrier (each workgroup's refill is meant to hide behind the other's MFMAs, which
+// works only when the two are out of step).
+template <int KH, int KW, bool VEC, bool PIPE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 2, PIPE ? 1 : 2))) void conv2d_patch_wgrad_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ partial, int chunks_per_part)
 {
 	typedef PatchWgrad<KH, KW> P;
-	__shared__ float lds[P::LDS_FLOATS];
+	__shared__ float lds[(PIPE ? 2 : 1) * P::LDS_FLOATS];
 	float* s_dy = lds;
 	float* s_patch = lds + P::DY_FLOATS;
 
@@ -304,6 +310,74 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	const float* pa = s_dy + (mt * 32 + lrow) * P::DYS + phalf * (P::TW / 2) + half;
 	const float* pb = s_patch + lrow * P::CS + phalf * (P::TW / 2) + half + 4 - g.pw;
 
+	if (PIPE) {
+		// piece k of the 16 + 4 * P_PER_T four-byte stores that put this thread's share of a chunk into a buffer
+		constexpr int PIECES = 4 * (P::DY_PER_T + P::P_PER_T), STEPS = P::TW / 4, SLOTS = STEPS * P::TAPS;
+		static_assert(PIECES <= SLOTS, "one store behind each MFMA at most");
+		int off_d[P::DY_PER_T], off_p[P::P_PER_T];
+#pragma unroll
+		for (int q = 0; q < P::DY_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			off_d[q] = (idx / (P::TW / 4)) * P::DYS + 4 * (idx % (P::TW / 4));
+		}
+#pragma unroll
+		for (int q = 0; q < P::P_PER_T; q++) {
+			const int idx = tid + q * P::T;
+			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
+			off_p[q] = idx < P::PATCH_F4 ? P::DY_FLOATS + (rowid / KH) * P::CS + (rowid % KH) * P::PWS + 4 * f : -1;
+		}
+		auto store_piece = [&](float* buf, int k) {
+			if (k < 4 * P::DY_PER_T) {
+				const float4 v = rdy[k / 4];
+				buf[off_d[k / 4] + (k % 4)] = (k % 4) == 0 ? v.x : (k % 4) == 1 ? v.y : (k % 4) == 2 ? v.z : v.w;
+			} else {
+				const int kk = k - 4 * P::DY_PER_T;
+				const float4 v = rp[kk / 4];
+				if (off_p[kk / 4] >= 0) buf[off_p[kk / 4] + (kk % 4)] = (kk % 4) == 0 ? v.x : (kk % 4) == 1 ? v.y : (kk % 4) == 2 ? v.z : v.w;
+			}
+		};
+		if (begin < end) {
+			load_chunk();
+#pragma unroll
+			for (int k = 0; k < PIECES; k++) store_piece(lds, k);
+			__syncthreads();
+			next_chunk();
+			if (begin + 1 < end) load_chunk();
+		}
+		// MORE: a chunk follows, whose tiles are stored to the other buffer on the way
+		auto run_chunk = [&](int chunk, auto more_tag) {
+			constexpr bool MORE = decltype(more_tag)::value;
+			const int cur = (chunk - begin) & 1;
+			const float* pac = pa + cur * P::LDS_FLOATS;
+			const float* pbc = pb + cur * P::LDS_FLOATS;
+			float* other = lds + (cur ^ 1) * P::LDS_FLOATS;
+			float fa[2], fb[2][P::TAPS];
+			auto read_operand = [&](int s, int t) { fb[s & 1][t] = pbc[(t / KW) * P::PWS + (t % KW) + 2 * s]; };
+			fa[0] = pac[0];
+#pragma unroll
+			for (int t = 0; t < P::TAPS; t++) read_operand(0, t);
+#pragma unroll
+			for (int s = 0; s < STEPS; s++) {
+#pragma unroll
+				for (int t = 0; t < P::TAPS; t++) {
+					acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[s & 1], fb[s & 1][t], acc[t], 0, 0, 0);
+					if (s + 1 < STEPS) {
+						if (t == 0) fa[(s + 1) & 1] = pac[2 * (s + 1)];
+						read_operand(s + 1, t);
+					}
+					const int k = s * P::TAPS + t - (SLOTS - PIECES);
+					if (MORE && k >= 0) store_piece(other, k);
+					__builtin_amdgcn_sched_barrier(0);
+				}
+			}
+			// the registers are free again: fetch the chunk after next, then let everybody finish with both buffers
+			next_chunk();
+			if (chunk + 2 < end) load_chunk();
+			__syncthreads();
+		};
+		for (int chunk = begin; chunk + 1 < end; chunk++) run_chunk(chunk, std::true_type{});
+		if (begin < end) run_chunk(end - 1, std::false_type{});
+	} else {
 	if (begin < end) load_chunk();
 	for (int chunk = begin; chunk < end; chunk++) {
 		store_chunk();
@@ -329,6 +403,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 			}
 		}
 		__syncthreads();
+	}
 	}
 
 	// pixel half 1 hands its sums to pixel half 0 of the same row tile, TAPS_PER_ROUND taps at a time
@@ -449,13 +524,17 @@ bool conv_patch_wgrad_takes(const ConvGeo& g)
 	       (uint64_t)g.H * g.W < (1u << 25) && (uint64_t)g.Ho * g.Wo < (1u << 25);  // 32-bit lane offsets over 32 channels
 }
 
-int conv_patch_wgrad_parts(const ConvGeo& g)
+// upper_bound: the largest count any kernel choice can give (for sizing the workspace, so that a change of the
+// tuning option between the size query and the call can never make the kernel write past it)
+int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound)
 {
 	typedef PatchWgrad<3, 3> P;
 	// two workgroups per CU over all (co block, ci block) pairs, at least four chunks per part
 	const uint64_t blocks = ceil_div((uint64_t)g.Cout, P::BM) * ceil_div((uint64_t)g.Cin, P::CIB);
 	const uint64_t chunks = (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, P::TW);
-	uint64_t parts = std::max<uint64_t>(1, 512 / blocks);
+	// one workgroup per CU; two with the unpipelined kernel (rows that do not allow 16-byte loads, or conv_variant 3)
+	const bool vec = g.W % 4 == 0 && g.Wo % 4 == 0;
+	uint64_t parts = std::max<uint64_t>(1, (upper_bound || get_option(OPT_CONV_VARIANT) == 3 || !vec ? 512 : 256) / blocks);
 	parts = std::min<uint64_t>(parts, std::max<uint64_t>(1, chunks / 4));
 	const uint64_t per = ceil_div(chunks, parts);
 	return (int)ceil_div(chunks, per);
@@ -469,8 +548,13 @@ int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* p
 	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
 	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)ceil_div((uint64_t)g.Cin, P::CIB));
 	set_kernel_name("conv2d_patch_wgrad_3x3_64x32");
-	if (vec) conv2d_patch_wgrad_kernel<3, 3, true><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
-	else conv2d_patch_wgrad_kernel<3, 3, false><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	if (get_option(OPT_CONV_VARIANT) == 3 || !vec) {
+		set_kernel_name("conv2d_patch_wgrad_3x3_64x32_unpipelined");
+		if (vec) conv2d_patch_wgrad_kernel<3, 3, true, false><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		else conv2d_patch_wgrad_kernel<3, 3, false, false><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	} else {
+		conv2d_patch_wgrad_kernel<3, 3, true, true><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }
