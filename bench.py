@@ -172,11 +172,12 @@ def extra_configs(lt, wl, with_cpu):
     flops = sum(3 * 2.0 * B_ * sizes[i] * sizes[i + 1] for i in range(3))
     tf = flops / ms / 1e9
     rec = {"config": "cfg2 fp32 MLP 784-1024-1024-10 batch 128, one training step on the device (9 GEMMs with the bias adds and the bias "
-                     "gradients fused in, relu x2, log_softmax, nll_loss and their backward: 17 launches)",
+                     "gradients fused in and the two backward products of a layer sharing a launch, relu x2, log_softmax, nll_loss "
+                     "and their backward: 14 launches)",
            "gpu_us": round(ms * 1e3, 2), "graph_replay_us": round(graph_ms * 1e3, 2), "gflop_per_step": round(flops / 1e9, 3),
            "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)},
-           "note": "seventeen dependent launches of about 5 us each; the launch-to-launch latency, not the MFMA rate, sets this time "
+           "note": "fourteen dependent launches of about 5 us each; the launch-to-launch latency, not the MFMA rate, sets this time "
                    "(GEMM flops only in the rate); replaying the step as one recorded graph does not shorten it"}
     if with_cpu:
         hA = [np.random.default_rng(i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]

@@ -21,6 +21,9 @@ int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, co
 bool conv_patch_wgrad_takes(const ConvGeo& g);
 int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound = false);  // partial [Cout x Cin*kh*kw] matrices the kernel writes
 int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts);
+// the same product with both LDS tiles filled by direct global->LDS loads (padding 1, W % 64 == 0, 16-byte aligned x and dy)
+bool conv_patch_fast_wgrad_takes(const ConvGeo& g, const float* x, const float* dy);
+int conv_patch_fast_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts);
 
 // Kernels for stride 1, dilation 1 and Cin*kh*kw <= 32 (first layers): the whole reduction fits one MFMA tile
 // dimension, the work is bound by the HBM traffic of y / dy (conv_smallk.hip).

@@ -547,6 +547,7 @@ int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* p
 	const int per = (int)ceil_div(chunks, (uint64_t)parts);
 	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
 	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)ceil_div((uint64_t)g.Cin, P::CIB));
+	if (get_option(OPT_CONV_VARIANT) == 0 && conv_patch_fast_wgrad_takes(g, x, dy)) return conv_patch_fast_wgrad(g, x, dy, partial, parts);
 	set_kernel_name("conv2d_patch_wgrad_3x3_64x32");
 	if (get_option(OPT_CONV_VARIANT) == 3 || !vec) {
 		set_kernel_name("conv2d_patch_wgrad_3x3_64x32_unpipelined");

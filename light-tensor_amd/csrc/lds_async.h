@@ -13,6 +13,23 @@ __device__ __forceinline__ void async_load16(uint32_t lds_addr, const void* base
 	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// The same for the lanes of `mask` only, without a branch: a taken branch costs a wavefront that is alone on its
+// SIMD far more than the load (its MFMA stream stops while instructions are fetched again).  To be called where
+// all 64 lanes are active; the execution mask is all ones again afterwards.
+__device__ __forceinline__ void async_load16_masked(uint64_t mask, uint32_t lds_addr, const void* base, uint32_t voff)
+{
+	asm volatile("s_mov_b64 exec, %0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, -1"
+	             : : "s"(mask), "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+// 16 bytes of zeros to LDS byte address lds_lane_addr (per lane) for the lanes of `mask`, without a branch; same
+// conditions as above.  `zero` is a register quadruple holding zeros.
+typedef float lds_v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void lds_zero16_masked(uint64_t mask, uint32_t lds_lane_addr, lds_v4f zero)
+{
+	asm volatile("s_mov_b64 exec, %0\n\tds_write_b128 %1, %2\n\ts_mov_b64 exec, -1" : : "s"(mask), "v"(lds_lane_addr), "v"(zero) : "memory");
+}
+
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt fields left at "no wait"); n < 64.
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()

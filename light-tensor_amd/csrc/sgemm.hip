@@ -78,17 +78,17 @@ __device__ __forceinline__ void add_row_sums(float* scratch, float asum, float* 
 // A k-contiguous operand is fetched 16 bytes per lane: lane (row, g) takes k = base + 4g .. 4g+3 and feeds the
 // t-th of four MFMAs with element t; the other layout is fetched one dword per MFMA (two 128-byte rows per
 // wave-wide load).  The assignment of k to MFMA slots is the same for A and B, which is all a dot product needs.
+// `block`: index of the 32x32 output tile, `z`: batch index, `part`: WAVES * 1024 floats of LDS.
 template <int WAVES, bool TA, bool TB>
-__global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
+__device__ __forceinline__ void sgemm_direct_body(const SProblem& p, int block, int z, float (*part)[32 * 32])
 {
-	__shared__ float part[WAVES][32 * 32];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int lrow = lane & 31, g = lane >> 5;
 	const int tiles_n = (p.N + 31) / 32;
-	const int m0 = (blockIdx.x / tiles_n) * 32, n0 = (blockIdx.x % tiles_n) * 32;
-	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
-	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
-	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+	const int m0 = (block / tiles_n) * 32, n0 = (block % tiles_n) * 32;
+	const float* A = p.A + (int64_t)z * p.stride_a;
+	const float* B = p.B + (int64_t)z * p.stride_b;
+	float* C = p.C + (int64_t)z * p.stride_c;
 	const int m = m0 + lrow, n = n0 + lrow;
 	const bool mok = m < p.M, nok = n < p.N;
 	const bool a_vec = !TA && (p.lda & 3) == 0 && (reinterpret_cast<uintptr_t>(A) & 15) == 0;
@@ -149,6 +149,13 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(&part[0][0], asum, p.rowsum, m0, p.M);
 }
 
+template <int WAVES, bool TA, bool TB>
+__global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
+{
+	__shared__ float part[WAVES][32 * 32];
+	sgemm_direct_body<WAVES, TA, TB>(p, blockIdx.x, blockIdx.z, part);
+}
+
 // The same decomposition with whole cache lines per load: the direct kernel above asks the texture addresser for 32
 // different lines per wave-wide load (32 rows x 32 bytes), which is what bounds it at these sizes.  Here a wave-wide
 // 16-byte load covers 8 rows x 128 bytes along the operand's contiguous dimension (8 lines), the values pass through
@@ -156,18 +163,24 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_direct_kernel(SProblem p)
 // the MFMA lane layout.  A batch is 32 k-values; wavefront w takes batches w, w + WAVES, ...; the loads of up to
 // UB batches are in flight at once.  Operand rows of 36 floats keep both the 16-byte stores and the reads free of
 // bank conflicts.  Used when the operands allow 16-byte loads (leading dimensions and bases multiples of 4 floats).
+template <int WAVES>
+struct StagedLds {
+	static constexpr int LD = 36, SLAB = 32 * LD;
+	static constexpr int FLOATS = WAVES * 2 * SLAB > WAVES * 1024 ? WAVES * 2 * SLAB : WAVES * 1024;
+};
+
+// `block`: index of the 32x32 output tile, `z`: batch index, `lds`: StagedLds<WAVES>::FLOATS floats, 16-byte aligned.
 template <int WAVES, bool TA, bool TB>
-__global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
+__device__ __forceinline__ void sgemm_staged_body(const SProblem& p, int block, int z, float* lds)
 {
-	constexpr int UB = 4, LD = 36, SLAB = 32 * LD;
-	__shared__ __attribute__((aligned(16))) float lds[WAVES * 2 * SLAB > WAVES * 1024 ? WAVES * 2 * SLAB : WAVES * 1024];
+	constexpr int UB = 4, LD = StagedLds<WAVES>::LD, SLAB = StagedLds<WAVES>::SLAB;
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int lrow = lane & 31, g = lane >> 5;
 	const int tiles_n = (p.N + 31) / 32;
-	const int m0 = (blockIdx.x / tiles_n) * 32, n0 = (blockIdx.x % tiles_n) * 32;
-	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
-	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
-	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+	const int m0 = (block / tiles_n) * 32, n0 = (block % tiles_n) * 32;
+	const float* A = p.A + (int64_t)z * p.stride_a;
+	const float* B = p.B + (int64_t)z * p.stride_b;
+	float* C = p.C + (int64_t)z * p.stride_c;
 	float* sA = lds + wave * 2 * SLAB;
 	float* sB = sA + SLAB;
 	const int r8 = lane >> 3, c4 = (lane & 7) * 4;  // this lane's row within a group of 8 and its 4-float column
@@ -265,6 +278,30 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 		*c = out;
 	}
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(lds, asum, p.rowsum, m0, p.M);
+}
+
+template <int WAVES, bool TA, bool TB>
+__global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
+{
+	__shared__ __attribute__((aligned(16))) float lds[StagedLds<WAVES>::FLOATS];
+	sgemm_staged_body<WAVES, TA, TB>(p, blockIdx.x, blockIdx.z, lds);
+}
+
+// Both products of FullyConnected backward in one launch: the first `blocks_x` workgroups compute tiles of
+// dX = dY W (NN), the others tiles of dW = dY^T X (TN, with the bias gradient as its row sums).  The two are
+// independent and each fills the chip for a few microseconds only, so a launch of their own for each costs about
+// as much again as the work.  STAGED_*: whether that product has K >= 512 and takes the whole-line loads.
+template <bool STAGED_X, bool STAGED_W>
+__global__ __launch_bounds__(512) void sgemm_fc_backward_pair_kernel(SProblem px, SProblem pw, int blocks_x)
+{
+	__shared__ __attribute__((aligned(16))) float lds[(STAGED_X || STAGED_W) ? StagedLds<8>::FLOATS : 8 * 1024];
+	if ((int)blockIdx.x < blocks_x) {
+		if (STAGED_X) sgemm_staged_body<8, false, false>(px, blockIdx.x, 0, lds);
+		else sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, reinterpret_cast<float (*)[32 * 32]>(lds));
+	} else {
+		if (STAGED_W) sgemm_staged_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, lds);
+		else sgemm_direct_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, reinterpret_cast<float (*)[32 * 32]>(lds));
+	}
 }
 
 // FullyConnected forward at small batch sizes: C[M x N] = A[M x K] B[N x K]^T with M <= 32, a stream over the
@@ -569,6 +606,16 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	}
 }
 
+// Whether sgemm_run sends a product without bias and batch (M x N x K, neither M, N nor K equal to 1) to the 32x32
+// kernels: not large enough for the direct-to-LDS tiles, and few tiles or operands that allow 16-byte loads.
+static bool takes_32x32(const SProblem& p, uint64_t M, uint64_t N, uint64_t K)
+{
+	if (K <= 1 || M <= 1) return false;
+	if (ceil_div(M, 128) * ceil_div(N, 128) >= 128 && K >= 256) return false;
+	const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);
+	return tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20));
+}
+
 }  // namespace lten_hip
 
 using namespace lten_hip;
@@ -599,6 +646,29 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
                              float* dX, float* dW, float* db)
 {
 	int rc = 0;
+	// Both products wanted and both of the kind the 32x32 kernels take (few tiles, or 16-byte loads possible; not
+	// one of the degenerate shapes with a kernel of their own, not large enough for the direct-to-LDS tiles):
+	// one launch computes the two.
+	if (dX && dW && get_option(OPT_SGEMM_TILE) == 0 && M > 1 && out > 1 && in > 0) {
+		SProblem px = {}, pw = {};
+		px.A = dY; px.B = W; px.C = dX; px.lda = (int64_t)out; px.ldb = (int64_t)in; px.ldc = (int64_t)in;
+		px.M = (int)M; px.N = (int)in; px.K = (int)out; px.alpha = 1.0f; px.beta = 0.0f;
+		pw.A = dY; pw.B = X; pw.C = dW; pw.lda = (int64_t)out; pw.ldb = (int64_t)in; pw.ldc = (int64_t)in;
+		pw.M = (int)out; pw.N = (int)in; pw.K = (int)M; pw.alpha = 1.0f; pw.beta = 0.0f;
+		pw.rowsum = db;
+		const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
+		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
+			const bool sx = operands_vec(px) && px.K >= 512, sw = operands_vec(pw) && pw.K >= 512;
+			const dim3 grid((unsigned)(blocks_x + blocks_w)), block(512);
+			set_kernel_name("sgemm_fc_backward_pair_32x32_w8");
+			if (sx && sw) sgemm_fc_backward_pair_kernel<true, true><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
+			else if (sx) sgemm_fc_backward_pair_kernel<true, false><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
+			else if (sw) sgemm_fc_backward_pair_kernel<false, true><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
+			else sgemm_fc_backward_pair_kernel<false, false><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
+			LTEN_HIP_LAUNCH_CHECK();
+			return 0;
+		}
+	}
 	// l-ten/backprop.cpp:2228  dX[M x in] = dY[M x out] W[out x in]
 	if (dX) rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr, nullptr, nullptr);
 	// :2252  dW[out x in] = dY[M x out]^T X[M x in].  The rows of dY^T summed over the batch are the bias gradient

@@ -90,6 +90,12 @@ def test_conv_layer_golden(gpu):
                                  # input channels a multiple of four (patch filled by direct-to-LDS loads): 64-channel
                                  # workgroups with a ragged second column tile, ragged channel count with pad 2, one chunk pair
                                  (2, 8, 9, 132, 64, 3, 3, 1, 1, 1, 1), (1, 16, 6, 128, 100, 3, 3, 2, 2, 1, 1), (1, 32, 7, 12, 128, 3, 3, 0, 1, 1, 1),
+                                 # pad 1 and rows of whole 64-pixel chunks (weight gradient with both tiles filled by
+                                 # direct-to-LDS loads): ragged channel blocks on both sides with one column tile, a
+                                 # single image row (halo above and below at once), three column tiles (the middle
+                                 # one has no halo outside the image), two full blocks each way
+                                 (2, 40, 5, 64, 70, 3, 3, 1, 1, 1, 1), (1, 32, 1, 64, 64, 3, 3, 1, 1, 1, 1),
+                                 (3, 12, 3, 192, 33, 3, 3, 1, 1, 1, 1), (2, 64, 6, 128, 128, 3, 3, 1, 1, 1, 1),
                                  # stride 1 with Cin*kh*kw <= 32 (first-layer kernels): ragged widths, two column
                                  # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
@@ -189,6 +195,21 @@ def test_seeded_sweep_over_geometries(gpu, ob):
         N = int(rng.integers(1, 4))
         geo = (N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)
         _conv_vs_oracle(gpu, ob, geo)
+        seen.add(gpu.last_kernel())
+    print(sorted(seen))
+
+
+def test_seeded_sweep_over_chunked_rows(gpu, ob):
+    """Twelve seeded 3x3, stride 1, pad 1 geometries whose rows are whole 64-pixel chunks (the shapes the
+    direct-to-LDS weight-gradient kernel takes), channel counts on both sides of its 64 x 32 blocks."""
+    rng = np.random.default_rng(2718)
+    seen = set()
+    for case in range(12):
+        Cin = int(rng.choice([9, 16, 31, 32, 33, 48, 64, 70]))
+        Cout = int(rng.choice([1, 16, 63, 64, 65, 100, 128]))
+        H, W = int(rng.integers(1, 9)), int(rng.choice([64, 64, 128, 192]))
+        N = int(rng.integers(1, 4))
+        _conv_vs_oracle(gpu, ob, (N, Cin, H, W, Cout, 3, 3, 1, 1, 1, 1))
         seen.add(gpu.last_kernel())
     print(sorted(seen))
 

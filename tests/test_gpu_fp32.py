@@ -170,9 +170,12 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
 
 
 @pytest.mark.parametrize("M,fin,fout,kernels", [
-    (128, 200, 75, ("sgemm_direct_32x32_w8",)),                      # bias gradient inside the direct kernel
-    (37, 33, 10, ("sgemm_direct_32x32_w8",)),                        # ragged in every dimension
-    (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: the staged kernel, ragged K
+    (128, 200, 75, ("sgemm_fc_backward_pair_32x32_w8",)),            # both products in one launch, bias gradient inside it
+    (37, 33, 10, ("sgemm_fc_backward_pair_32x32_w8",)),              # ragged in every dimension
+    (777, 96, 132, ("sgemm_fc_backward_pair_32x32_w8",)),            # batch >= 512: whole-line loads for dW only, ragged K
+    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_w8",)),          # out >= 512: whole-line loads for dX only (config 2, layer 1)
+    (640, 64, 512, ("sgemm_fc_backward_pair_32x32_w8",)),            # whole-line loads for both
+    (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
     (640, 1101, 999, ("sgemm_rowvec",)),                             # unaligned rows, many tiles: LDS-tiled GEMM, then the column sum
 ])
@@ -192,6 +195,14 @@ def test_fc_backward_bias_gradient_accumulates_on_every_route(gpu, M, fin, fout,
     assert np.array_equal(dDB.numpy(np.float32, (fout,)), db0 + dy.sum(axis=0))
     assert np.array_equal(dDW.numpy(np.float32, w.shape), dy.T @ x)
     assert np.array_equal(dDX.numpy(np.float32, x.shape), dy @ w)
+    # one product at a time goes through the GEMM entry's own choice of kernel
+    dDX2, dDW2, dDB3 = D(x.nbytes), D(w.nbytes), D.from_numpy(db0)
+    gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, dDX2.ptr, None, None))
+    assert not gpu.last_kernel().startswith("sgemm_fc_backward_pair")
+    gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, None, dDW2.ptr, dDB3.ptr))
+    assert np.array_equal(dDX2.numpy(np.float32, x.shape), dy @ w)
+    assert np.array_equal(dDW2.numpy(np.float32, w.shape), dy.T @ x)
+    assert np.array_equal(dDB3.numpy(np.float32, (fout,)), db0 + dy.sum(axis=0))
     # without dW the column-sum kernel still serves db
     dDB2 = D.from_numpy(db0)
     gpu.check(gpu.lib().lten_hip_fc_backward_f32(M, fin, fout, dX.ptr, dW.ptr, dDY.ptr, None, None, dDB2.ptr))
