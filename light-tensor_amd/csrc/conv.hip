@@ -183,8 +183,9 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	const int HW = g.Ho * g.Wo;
 	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
 	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
-	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run
-	if (variant == 0 && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
+	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
+	// one with its four-row tile also where the two-row tile would be picked
+	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
 	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");

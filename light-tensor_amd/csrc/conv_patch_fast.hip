@@ -1,14 +1,15 @@
 // Conv2d forward, 3x3, stride 1, with the LDS patch filled by direct global->LDS loads.
 //
 // The same tile and the same MFMA schedule as conv2d_patch_forward_kernel (a workgroup = BM output channels x
-// 4 rows x 128 columns of one image, wavefront `wave` owns row `wave`, input channels in chunks of four, step
+// TH rows x 128 columns of one image; TH = 4: wavefront `wave` owns row `wave`, TH = 2: row wave % 2, columns
+// 64 (wave / 2) .. + 63; input channels in chunks of four, step
 // (cp, i, j) multiplies tap (i, j) of channels 2cp (lanes 0-31) and 2cp + 1 (lanes 32-63)), but a chunk reaches
 // LDS without passing through registers: two LDS stages, chunk c + 1 lands in one while chunk c is multiplied
 // from the other, one barrier per chunk.
 //
-// A stage holds the patch [4 channels][6 rows][136 columns] (column q = input column w0 - 4 + q) and the weights
+// A stage holds the patch [4 channels][TH + 2 rows][136 columns] (column q = input column w0 - 4 + q) and the weights
 // [BM channels][36] exactly as they lie in memory, so both are filled by wave-wide loads whose lane L writes 16
-// bytes at 16 L: patch float4 number idx is (channel idx / 204, row (idx / 34) % 6, columns 4 (idx % 34) ..);
+// bytes at 16 L: patch float4 number idx is (channel idx / (34 (TH + 2)), row (idx / 34) % (TH + 2), columns 4 (idx % 34) ..);
 // weight float4 number idx is (channel idx / 9, floats 4 (idx % 9) ..).  Whether a float4 lies inside the image
 // (or names an existing output channel) does not depend on the chunk: lanes whose float4 does not exist never
 // load, and their LDS slots keep the zeros written once before the first chunk.  That is the zero padding.
@@ -22,9 +23,10 @@ namespace lten_hip {
 
 namespace {
 
-template <int BM_>
+template <int BM_, int TH_>
 struct FastFwd {
-	static constexpr int BM = BM_, MT = BM / 32, NT = 4, CB = 4, TH = 4, TW = 128, PR = TH + 2, PWS = 136, F4R = 34;
+	static_assert(TH_ == 4 || TH_ == 2, "a wavefront owns a whole row of the tile (TH = 4) or half a row (TH = 2)");
+	static constexpr int BM = BM_, MT = BM / 32, TH = TH_, NT = TH, CB = 4, TW = 128, PR = TH + 2, PWS = 136, F4R = 34;
 	static constexpr int PATCH_F4 = CB * PR * F4R;                 // 816
 	static constexpr int PATCH_LOADS = (PATCH_F4 + 63) / 64;       // 13
 	static constexpr int PATCH_BYTES = PATCH_LOADS * 1024;
@@ -40,16 +42,17 @@ struct FastFwd {
 
 }  // namespace
 
-template <int BM>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 2 : 4, BM == 64 ? 2 : 4))) void conv2d_patch_fast_forward_kernel(
+template <int BM, int TH>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 256 ? 2 : 4, BM * TH == 256 ? 2 : 4))) void conv2d_patch_fast_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
 {
-	typedef FastFwd<BM> P;
+	typedef FastFwd<BM, TH> P;
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[2 * P::STAGE];
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int lrow = lane & 31, half = lane >> 5;
+	const int wrow = TH == 4 ? wave : (wave & 1), wcol = TH == 4 ? 0 : (wave >> 1) * 64;  // this wavefront's row and first column in the tile
 	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
 	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
 	const int co0 = blockIdx.y * BM, n = blockIdx.z;
@@ -109,7 +112,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 
 	// ---- operand addresses: a per-lane base plus immediates
 	const int off_a = P::PATCH_BYTES + (lrow * 36 + half * 9) * 4;
-	const int off_b = ((half * P::PR + wave) * P::PWS + lrow + 4 - g.pw) * 4;
+	const int off_b = ((half * P::PR + wrow) * P::PWS + wcol + lrow + 4 - g.pw) * 4;
 	auto read_one = [&](float (&fa)[P::MT], float (&fb)[P::NT], const uint8_t* sbase, int s, int e) {
 		const int cp = s / 9, tap = s % 9, ti = tap / 3, tj = tap % 3;
 		if (e < P::MT) fa[e] = *reinterpret_cast<const float*>(sbase + off_a + (e * 32 * 36 + 2 * cp * 9 + tap) * 4);
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 	if (LTEN_CONV_EXP == 1 && acc[0][0][0] != 12345.678f) return;
 #endif
 	// Epilogue: all bias values first, then stores whose address is a shared part plus a lane offset.
-	const int ho = h0 + wave;
+	const int ho = h0 + wrow;
 	if (ho >= g.Ho) return;
 	float bv[P::MT][16];
 #pragma unroll
@@ -191,7 +194,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 			bv[m][r] = (bias && co < g.Cout) ? bias[co] : 0.0f;
 		}
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
-	float* yw = y + (((int64_t)n * g.Cout + co0) * g.Ho + ho) * g.Wo + w0;
+	float* yw = y + (((int64_t)n * g.Cout + co0) * g.Ho + ho) * g.Wo + w0 + wcol;
 	const unsigned y_lane = (unsigned)(half * 4 * plane) + lrow;
 	if (co0 + BM <= g.Cout && w0 + P::TW <= g.Wo) {
 #pragma unroll
@@ -212,7 +215,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 			float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
 #pragma unroll
 			for (int t = 0; t < P::NT; t++)
-				if (w0 + t * 32 + lrow < g.Wo) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
+				if (w0 + wcol + t * 32 + lrow < g.Wo) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
 		}
 }
 
@@ -225,13 +228,23 @@ bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float
 
 int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
-	const unsigned tiles = (unsigned)(ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 4));
-	if (ceil_div((uint64_t)g.Cout, 32) % 2 == 1) {
+	const unsigned tiles_w = (unsigned)ceil_div((uint64_t)g.Wo, 128);
+	const unsigned blocks64 = (unsigned)ceil_div((uint64_t)g.Cout, 64), blocks32 = (unsigned)ceil_div((uint64_t)g.Cout, 32);
+	const unsigned tiles = tiles_w * (unsigned)ceil_div((uint64_t)g.Ho, 4);
+	if (blocks32 % 2 == 1) {
 		set_kernel_name("conv2d_patch_fast_forward_3x3_32x4x128");
-		conv2d_patch_fast_forward_kernel<32><<<dim3(tiles, (unsigned)ceil_div((uint64_t)g.Cout, 32), (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		conv2d_patch_fast_forward_kernel<32, 4><<<dim3(tiles, blocks32, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+	} else if ((uint64_t)tiles * blocks64 * g.N < 2048 && get_option(OPT_CONV_VARIANT) != 5) {
+		// Few workgroups per CU slot (two at a time fit): all of them reach their store epilogue together and the
+		// matrix pipe waits while y is written.  Tiles of two rows double the workgroups and fit four to a CU, so
+		// one workgroup's stores overlap another's MFMAs (config 5 layer 2: 192 -> 178 us on the same box); with
+		// many rounds of workgroups the taller tile's smaller halo wins.  conv_variant 5 keeps the taller tile.
+		set_kernel_name("conv2d_patch_fast_forward_3x3_64x2x128");
+		const unsigned tiles2 = tiles_w * (unsigned)ceil_div((uint64_t)g.Ho, 2);
+		conv2d_patch_fast_forward_kernel<64, 2><<<dim3(tiles2, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	} else {
 		set_kernel_name("conv2d_patch_fast_forward_3x3_64x4x128");
-		conv2d_patch_fast_forward_kernel<64><<<dim3(tiles, (unsigned)ceil_div((uint64_t)g.Cout, 64), (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		conv2d_patch_fast_forward_kernel<64, 4><<<dim3(tiles, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;

@@ -101,10 +101,11 @@ def test_conv_layer_golden(gpu):
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
                                  (1, 20, 9, 132, 33, 1, 1, 0, 0, 1, 1), (2, 3, 16, 36, 64, 3, 3, 0, 0, 1, 1),
                                  (5, 2, 7, 9, 3, 2, 7, 1, 4, 1, 1)])
-@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 5])
 def test_conv_vs_oracle(gpu, ob, geo, variant):
     """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape; 2: the register-staged
-    patch kernel also where the direct-to-LDS one would run; 3: also the unpipelined weight-gradient kernel."""
+    patch kernel also where the direct-to-LDS one would run; 3: also the unpipelined weight-gradient kernel; 5: the
+    direct-to-LDS forward kernel with four-row tiles also where it would pick two-row tiles."""
     try:
         gpu.set_option("conv_variant", variant)
         _conv_vs_oracle(gpu, ob, geo)
