@@ -200,6 +200,38 @@ def test_seeded_sweep_over_geometries(gpu, ob):
     print(sorted(seen))
 
 
+@pytest.mark.parametrize("geo", [(2, 16, 6, 128, 64, 3, 3, 1, 1, 1, 1), (1, 12, 5, 64, 40, 3, 3, 1, 1, 1, 1)])
+def test_conv_operands_aligned_to_four_bytes_only(gpu, ob, geo):
+    """x, w, dy and y that start 4 bytes into their allocations (views into larger tensors, as l-ten's per-image
+    offsets produce): the kernels that need 16-byte aligned operands must step aside, the results stay the same."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo) + 1)
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * H * W, np.float32)
+    want_y, want_dw, want_dx = np.empty_like(dy), np.empty_like(w), np.empty_like(x)
+    ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
+    ob.oracle().oracle_conv2d_wgrad(*geo, x.reshape(-1), dy.reshape(-1), want_dw.reshape(-1), col)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    dX, dW, dDY = D(x.nbytes + 16), D(w.nbytes + 16), D(dy.nbytes + 16)
+    dX.upload(x, offset=4); dW.upload(w, offset=4); dDY.upload(dy, offset=4)
+    dY, dDW, dDX = D(dy.nbytes + 16), D(w.nbytes + 16), D(x.nbytes + 16)
+    gpu.check(l.lten_hip_conv2d_forward_f32(*geo, dX.ptr + 4, dW.ptr + 4, None, dY.ptr + 4))
+    fk = gpu.last_kernel()
+    ws = D(max(int(l.lten_hip_conv2d_wgrad_workspace_bytes(*geo)), int(l.lten_hip_conv2d_dgrad_workspace_bytes(*geo)), 4))
+    gpu.check(l.lten_hip_conv2d_wgrad_f32(*geo, dX.ptr + 4, dDY.ptr + 4, dDW.ptr + 4, ws.ptr))
+    wk = gpu.last_kernel()
+    gpu.check(l.lten_hip_conv2d_dgrad_f32(*geo, dW.ptr + 4, dDY.ptr + 4, dDX.ptr + 4, ws.ptr))
+    print(f"  {geo}: forward via {fk}, wgrad via {wk}, dgrad via {gpu.last_kernel()}", flush=True)
+    assert "fast" not in fk and "fast" not in wk
+    got = lambda buf, shape: buf.numpy(np.uint8, (buf.nbytes,))[4:4 + 4 * int(np.prod(shape))].view(np.float32).reshape(shape)
+    assert rel_err(got(dY, dy.shape), want_y) < TOL, fk
+    assert rel_err(got(dDW, w.shape), want_dw) < TOL, wk
+    assert rel_err(got(dDX, x.shape), want_dx) < TOL, gpu.last_kernel()
+
+
 def test_seeded_sweep_over_chunked_rows(gpu, ob):
     """Twelve seeded 3x3, stride 1, pad 1 geometries whose rows are whole 64-pixel chunks (the shapes the
     direct-to-LDS weight-gradient kernel takes), channel counts on both sides of its 64 x 32 blocks."""
