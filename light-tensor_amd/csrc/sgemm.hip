@@ -288,20 +288,16 @@ __global__ __launch_bounds__(WAVES * 64) void sgemm_staged_kernel(SProblem p)
 }
 
 // Both products of FullyConnected backward in one launch: the first `blocks_x` workgroups compute tiles of
-// dX = dY W (NN), the others tiles of dW = dY^T X (TN, with the bias gradient as its row sums).  The two are
-// independent and each fills the chip for a few microseconds only, so a launch of their own for each costs about
-// as much again as the work.  STAGED_*: whether that product has K >= 512 and takes the whole-line loads.
-template <bool STAGED_X, bool STAGED_W>
+// dX = dY W (NN), the others tiles of dW = dY^T X (TN, with the bias gradient as its row sums), both with the
+// direct body (32 KB of LDS, four workgroups per CU).  The two are independent and each fills the chip for a few
+// microseconds only, so a launch of their own for each costs about as much again as the work.  The whole-line
+// body is not used here: its 74 KB of LDS would halve the number of resident workgroups for both products
+// (measured at batch 128, 1024 -> 1024: 18.6 us with it, 14.8 without, 17.9 as two launches).
 __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_kernel(SProblem px, SProblem pw, int blocks_x)
 {
-	__shared__ __attribute__((aligned(16))) float lds[(STAGED_X || STAGED_W) ? StagedLds<8>::FLOATS : 8 * 1024];
-	if ((int)blockIdx.x < blocks_x) {
-		if (STAGED_X) sgemm_staged_body<8, false, false>(px, blockIdx.x, 0, lds);
-		else sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, reinterpret_cast<float (*)[32 * 32]>(lds));
-	} else {
-		if (STAGED_W) sgemm_staged_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, lds);
-		else sgemm_direct_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, reinterpret_cast<float (*)[32 * 32]>(lds));
-	}
+	__shared__ float part[8][32 * 32];
+	if ((int)blockIdx.x < blocks_x) sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, part);
+	else sgemm_direct_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, part);
 }
 
 // FullyConnected forward at small batch sizes: C[M x N] = A[M x K] B[N x K]^T with M <= 32, a stream over the
@@ -646,10 +642,10 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
                              float* dX, float* dW, float* db)
 {
 	int rc = 0;
-	// Both products wanted and both of the kind the 32x32 kernels take (few tiles, or 16-byte loads possible; not
-	// one of the degenerate shapes with a kernel of their own, not large enough for the direct-to-LDS tiles):
-	// one launch computes the two.
-	if (dX && dW && get_option(OPT_SGEMM_TILE) == 0 && M > 1 && out > 1 && in > 0) {
+	// Both products wanted, both of the kind the 32x32 kernels take (few tiles, or 16-byte loads possible; not one of
+	// the degenerate shapes with a kernel of their own, not large enough for the direct-to-LDS tiles) and the batch
+	// small enough that the weight-gradient product would not take the whole-line loads: one launch computes the two.
+	if (dX && dW && get_option(OPT_SGEMM_TILE) == 0 && M > 1 && M < 512 && out > 1 && out <= 2048 && in > 0) {
 		SProblem px = {}, pw = {};
 		px.A = dY; px.B = W; px.C = dX; px.lda = (int64_t)out; px.ldb = (int64_t)in; px.ldc = (int64_t)in;
 		px.M = (int)M; px.N = (int)in; px.K = (int)out; px.alpha = 1.0f; px.beta = 0.0f;
@@ -658,13 +654,8 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
 		pw.rowsum = db;
 		const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
 		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
-			const bool sx = operands_vec(px) && px.K >= 512, sw = operands_vec(pw) && pw.K >= 512;
-			const dim3 grid((unsigned)(blocks_x + blocks_w)), block(512);
 			set_kernel_name("sgemm_fc_backward_pair_32x32_w8");
-			if (sx && sw) sgemm_fc_backward_pair_kernel<true, true><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
-			else if (sx) sgemm_fc_backward_pair_kernel<true, false><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
-			else if (sw) sgemm_fc_backward_pair_kernel<false, true><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
-			else sgemm_fc_backward_pair_kernel<false, false><<<grid, block, 0, stream()>>>(px, pw, (int)blocks_x);
+			sgemm_fc_backward_pair_kernel<<<dim3((unsigned)(blocks_x + blocks_w)), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
 			LTEN_HIP_LAUNCH_CHECK();
 			return 0;
 		}

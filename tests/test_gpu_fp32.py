@@ -172,9 +172,9 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
 @pytest.mark.parametrize("M,fin,fout,kernels", [
     (128, 200, 75, ("sgemm_fc_backward_pair_32x32_w8",)),            # both products in one launch, bias gradient inside it
     (37, 33, 10, ("sgemm_fc_backward_pair_32x32_w8",)),              # ragged in every dimension
-    (777, 96, 132, ("sgemm_fc_backward_pair_32x32_w8",)),            # batch >= 512: whole-line loads for dW only, ragged K
-    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_w8",)),          # out >= 512: whole-line loads for dX only (config 2, layer 1)
-    (640, 64, 512, ("sgemm_fc_backward_pair_32x32_w8",)),            # whole-line loads for both
+    (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: two launches, dW with whole-line loads, ragged K
+    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_w8",)),          # config 2, layer 1
+    (511, 64, 2048, ("sgemm_fc_backward_pair_32x32_w8",)),           # the largest batch and width the paired launch takes
     (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
     (640, 1101, 999, ("sgemm_rowvec",)),                             # unaligned rows, many tiles: LDS-tiled GEMM, then the column sum
