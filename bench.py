@@ -384,6 +384,8 @@ def main():
 
     measured_peak = lt.measure_mfma_peak(0, 1)
     _, shader_mhz = lt.measure_last_clocks()
+    measured_peak_data = lt.measure_mfma_peak(2, 1)  # the same loop on operands that change like a GEMM's
+    _, shader_mhz_data = lt.measure_last_clocks()
 
     out = {
         "metric": "int8_fc_forward_tops_4096",
@@ -406,8 +408,13 @@ def main():
                      "kernel": kernel, "kernel_us": round(kernel_ms * 1e3, 2), "algorithmic_bytes": 3 * M * N,
                      "measured_mfma_only_tops": round(measured_peak, 1), "measured_mfma_only_shader_mhz": round(shader_mhz),
                      "frac_of_measured_mfma_only": round(achieved / measured_peak, 4),
+                     "measured_mfma_only_data_operands_tops": round(measured_peak_data, 1),
+                     "measured_mfma_only_data_operands_shader_mhz": round(shader_mhz_data),
+                     "frac_of_measured_mfma_only_data_operands": round(achieved / measured_peak_data, 4),
                      "note": "int8 multiply-add counted as 2 ops; achieved/peak in tera-ops per second; "
-                             "measured_mfma_only = a kernel that issues nothing but 32x32x32 int8 MFMAs"},
+                             "measured_mfma_only = a kernel that issues nothing but 32x32x32 int8 MFMAs on constant operands; "
+                             "_data_operands = the same with pseudo-random operands that change with every MFMA (the part "
+                             "lowers its clock under that load although nothing but the matrix pipes is busy)"},
         "verified_bit_exact": verified,
     }
     if not args.no_cpu:

@@ -47,6 +47,68 @@ __global__ __launch_bounds__(256) void mfma_f32_peak_kernel(int iters, float* si
 	if (s == 12345.678f) *sink = s;
 }
 
+// The same loops on operands that look like data: every lane holds eight pseudo-random register sets per operand and
+// every MFMA takes another pair, so the multiplier inputs toggle as they do in a GEMM (with the constant operands
+// above they do not, and the part draws much less power).
+__device__ __forceinline__ unsigned mix32(unsigned x)
+{
+	x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+	return x;
+}
+
+__global__ __launch_bounds__(256) void mfma_i8_peak_random_kernel(int iters, int* sink, long long* clocks)
+{
+	v16i acc0 = {}, acc1 = {}, acc2 = {}, acc3 = {};
+	v4i a[8], b[8];
+	unsigned seed = (blockIdx.x * 256 + threadIdx.x) * 97u + 12345u;
+#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		a[i] = v4i{ (int)mix32(seed + 8 * i), (int)mix32(seed + 8 * i + 1), (int)mix32(seed + 8 * i + 2), (int)mix32(seed + 8 * i + 3) };
+		b[i] = v4i{ (int)mix32(seed + 8 * i + 4), (int)mix32(seed + 8 * i + 5), (int)mix32(seed + 8 * i + 6), (int)mix32(seed + 8 * i + 7) };
+	}
+	const long long c0 = clock64(), w0 = wall_clock64();
+	for (int i = 0; i < iters; i += 2) {
+#pragma unroll
+		for (int u = 0; u < 2; u++) {
+			acc0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[4 * u + 0], b[4 * u + 0], acc0, 0, 0, 0);
+			acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[4 * u + 1], b[4 * u + 1], acc1, 0, 0, 0);
+			acc2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[4 * u + 2], b[4 * u + 2], acc2, 0, 0, 0);
+			acc3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[4 * u + 3], b[4 * u + 3], acc3, 0, 0, 0);
+		}
+	}
+	int s = 0;
+	for (int r = 0; r < 16; r++) s += acc0[r] + acc1[r] + acc2[r] + acc3[r];
+	if (clocks && blockIdx.x == 0 && threadIdx.x == 0) {
+		clocks[0] = clock64() - c0;
+		clocks[1] = wall_clock64() - w0;
+	}
+	if (s == 0x7fffffff) *sink = s;
+}
+
+__global__ __launch_bounds__(256) void mfma_f32_peak_random_kernel(int iters, float* sink)
+{
+	v16f acc0 = {}, acc1 = {}, acc2 = {}, acc3 = {};
+	float a[8], b[8];
+	unsigned seed = (blockIdx.x * 256 + threadIdx.x) * 97u + 12345u;
+#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		a[i] = (float)(int)(mix32(seed + 2 * i) >> 8) * (1.0f / 8388608.0f) - 1.0f;      // uniform in [-1, 1)
+		b[i] = (float)(int)(mix32(seed + 2 * i + 1) >> 8) * (1.0f / 8388608.0f) - 1.0f;
+	}
+	for (int i = 0; i < iters; i += 2) {
+#pragma unroll
+		for (int u = 0; u < 2; u++) {
+			acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * u + 0], b[4 * u + 0], acc0, 0, 0, 0);
+			acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * u + 1], b[4 * u + 1], acc1, 0, 0, 0);
+			acc2 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * u + 2], b[4 * u + 2], acc2, 0, 0, 0);
+			acc3 = __builtin_amdgcn_mfma_f32_32x32x2f32(a[4 * u + 3], b[4 * u + 3], acc3, 0, 0, 0);
+		}
+	}
+	float s = 0;
+	for (int r = 0; r < 16; r++) s += acc0[r] + acc1[r] + acc2[r] + acc3[r];
+	if (s == 12345.678f) *sink = s;
+}
+
 __global__ __launch_bounds__(256) void copy_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, uint64_t n16)
 {
 	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256) dst[i] = src[i];
@@ -60,16 +122,18 @@ using namespace lten_hip;
 
 extern "C" {
 
-// kind 0: int8 32x32x32 MFMA, result in tera-ops/s.  kind 1: fp32 32x32x2 MFMA, result in TFLOP/s.
+// kind 0: int8 32x32x32 MFMA, result in tera-ops/s.  kind 1: fp32 32x32x2 MFMA, result in TFLOP/s.  kinds 2 and 3:
+// the same two with pseudo-random operands that change from one MFMA to the next.
 int lten_hip_measure_mfma_peak(int kind, int waves_per_simd, float* tera_per_s)
 {
-	LTEN_HIP_REQUIRE(tera_per_s != nullptr && (kind == 0 || kind == 1) && waves_per_simd >= 1 && waves_per_simd <= 8, "measure_mfma_peak: bad argument");
+	LTEN_HIP_REQUIRE(tera_per_s != nullptr && kind >= 0 && kind <= 3 && waves_per_simd >= 1 && waves_per_simd <= 8, "measure_mfma_peak: bad argument");
 	hipDeviceProp_t prop;
 	int dev = 0;
 	LTEN_HIP_CHECK(hipGetDevice(&dev));
 	LTEN_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
 	const int blocks = prop.multiProcessorCount * waves_per_simd;  // 4 waves per block = 1 per SIMD
-	const int iters = kind == 0 ? 4096 : 2048;
+	const bool int8 = kind == 0 || kind == 2;
+	const int iters = int8 ? 4096 : 2048;
 	void* sink = nullptr;
 	LTEN_HIP_CHECK(hipMalloc(&sink, 64));
 	hipEvent_t e0, e1;
@@ -80,17 +144,21 @@ int lten_hip_measure_mfma_peak(int kind, int waves_per_simd, float* tera_per_s)
 		LTEN_HIP_CHECK(hipEventRecord(e0, stream()));
 		if (kind == 0)
 			mfma_i8_peak_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<int*>(sink), static_cast<long long*>(sink) + 1);
-		else
+		else if (kind == 2)
+			mfma_i8_peak_random_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<int*>(sink), static_cast<long long*>(sink) + 1);
+		else if (kind == 1)
 			mfma_f32_peak_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<float*>(sink));
+		else
+			mfma_f32_peak_random_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(iters, static_cast<float*>(sink));
 		LTEN_HIP_CHECK(hipEventRecord(e1, stream()));
 		LTEN_HIP_CHECK(hipEventSynchronize(e1));
 		float ms = 0;
 		LTEN_HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
 		if (rep > 0 && ms < best) best = ms;
 	}
-	const double ops_per_mfma = kind == 0 ? 2.0 * 32 * 32 * 32 : 2.0 * 32 * 32 * 2;
+	const double ops_per_mfma = int8 ? 2.0 * 32 * 32 * 32 : 2.0 * 32 * 32 * 2;
 	*tera_per_s = (float)(ops_per_mfma * 4.0 * iters * 4.0 * blocks / (best * 1e-3) / 1e12);
-	if (kind == 0) {
+	if (int8) {
 		long long clk[2] = { 0, 0 };
 		LTEN_HIP_CHECK(hipMemcpy(clk, static_cast<long long*>(sink) + 1, sizeof(clk), hipMemcpyDeviceToHost));
 		g_last_cycles_per_mfma = (double)clk[0] / (4.0 * iters);
