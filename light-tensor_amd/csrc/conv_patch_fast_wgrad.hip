@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 		const bool never = rem == P::PITCH_F4 - 1 || ci >= P::CIB || ci0 + ci >= g.Cin;
 		p_flags[i] = never ? 0 : (r == 0 ? P::TOP : 0) | (r == 2 ? P::BOTTOM : 0) | (f == 0 ? P::LEFT : 0) | (f == P::F4_ROW - 1 ? P::RIGHT : 0);
 		p_exists[i] = __ballot(!never);
-		p_voff[i] = never ? 0 : (uint32_t)(((ci * g.H + r) * g.W + 4 * f) * 4);  // from (row ho - 1, column w0 - 4) of channel ci0
+		p_voff[i] = never ? 0 : (uint32_t)((((int64_t)ci * g.H + r) * g.W + 4 * f) * 4);  // from (row ho - 1, column w0 - 4) of channel ci0
 	}
 	// The chunk's position is kept as two byte addresses that advance with it: dyb = (image, channel co0, row ho,
 	// column w0) of dy, xb = (image, channel ci0, row ho - 1, column w0 - 4) of x (which may lie before the array;
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 bool conv_patch_fast_wgrad_takes(const ConvGeo& g, const float* x, const float* dy)
 {
 	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.ph == 1 && g.pw == 1 && g.W % 64 == 0 &&
-	       aligned16(x) && aligned16(dy) && (uint64_t)g.H * g.W < (1u << 24);
+	       aligned16(x) && aligned16(dy) && (uint64_t)(g.H + 2) * g.W < (1u << 24);  // lane offsets of up to 32 channel planes fit 32 bits
 }
 
 int conv_patch_fast_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts)
