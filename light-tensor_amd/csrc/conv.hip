@@ -183,6 +183,7 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	const int HW = g.Ho * g.Wo;
 	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
 	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
+	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
 	// one with its four-row tile also where the two-row tile would be picked
 	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
@@ -293,6 +294,10 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	LTEN_HIP_REQUIRE(w && dy && workspace, "conv2d_dgrad: null pointer");
 	float* work = static_cast<float*>(workspace);
 	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1) {
+		ConvGeo gt;  // the transposed problem: dy is the input, dx the output
+		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
+		if (get_option(OPT_CONV_VARIANT) == 0 && gt.Ho == (int)H && gt.Wo == (int)W && !conv_smallk_takes(gt) && conv_fewout_takes(gt, dy, dx))
+			return conv_fewout_forward(gt, dy, w, nullptr, dx, true);  // reads w transposed and flipped in place
 		flip_weights_kernel<<<dim3((unsigned)std::min<uint64_t>(ceil_div(Cout * Kc, 256), 1024)), dim3(256), 0, stream()>>>(w, work, (int)Cout, (int)Cin, kh, kw);
 		LTEN_HIP_LAUNCH_CHECK();
 		ConvGeo g2;

@@ -25,6 +25,11 @@ int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* p
 bool conv_patch_fast_wgrad_takes(const ConvGeo& g, const float* x, const float* dy);
 int conv_patch_fast_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts);
 
+// 3x3, stride 1, at most four output channels: a stream over x on the vector ALUs (conv_fewout.hip).  dgrad: w is the
+// weight array of the convolution whose data gradient is computed, read transposed and flipped in place.
+bool conv_fewout_takes(const ConvGeo& g, const float* x, const float* y);
+int conv_fewout_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y, bool dgrad);
+
 // Kernels for stride 1, dilation 1 and Cin*kh*kw <= 32 (first layers): the whole reduction fits one MFMA tile
 // dimension, the work is bound by the HBM traffic of y / dy (conv_smallk.hip).
 bool conv_smallk_takes(const ConvGeo& g);

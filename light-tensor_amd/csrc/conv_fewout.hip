@@ -1,0 +1,181 @@
+// Conv2d forward, 3x3, stride 1, column padding 1, with at most four output channels — and through it the data
+// gradient of a first layer (few input channels), which is such a convolution of dy with the flipped,
+// channel-transposed weights.
+//
+// With so few output channels an MFMA tile would be almost empty (the 32-channel tile of the patch kernels spends
+// 31/32 of its work on channels that do not exist when there is one); the work is a stream over x instead: every
+// input value is read once from HBM and used for 9 * Cout multiply-adds.  A workgroup computes 8 rows x 128 columns
+// of one image; a thread owns four consecutive pixels of one row and all output channels.  Input channels come in
+// chunks of four: the patch [4 channels][10 rows][136 columns] (column q = input column w0 - 4 + q) is filled by
+// direct global->LDS loads exactly as it lies in memory, two stages (a third did not help: 26.0 against 24.5 us on a
+// 32-channel 128 x 128 data gradient at batch 32).  Whether a float4 of the patch lies inside the
+// image does not depend on the chunk: lanes whose float4 does not exist never load, and their slots keep the zeros
+// written once.  Per channel and patch row a thread needs six columns (4 t + 3 .. 4 t + 8): its own four in one 16-byte
+// read, the two neighbours from the lanes beside it, and multiplies them with the 3 * Cout weights of that row, which are wave-uniform and come
+// through scalar loads.  DGRAD reads the weights of the transposed problem in place (w[ci][co][2 - i][2 - j]), so
+// no flipped copy is made.
+//
+// Needs Cin % 4 == 0, W % 4 == 0 and 16-byte aligned x and y.
+#include "conv_common.h"
+#include "lds_async.h"
+
+namespace lten_hip {
+
+namespace {
+
+struct FewOut {
+	static constexpr int CB = 4, TH = 8, TW = 128, PR = TH + 2, PWS = 136, F4R = 34;
+	static constexpr int PATCH_F4 = CB * PR * F4R;              // 1360
+	static constexpr int LPW = (PATCH_F4 + 255) / 256;          // loads per wavefront and chunk: 6
+	static constexpr int STAGE = LPW * 4 * 1024;                // bytes
+	static constexpr int S = 2;                                 // stages: one chunk in flight while one is used
+};
+
+}  // namespace
+
+template <int COUT, bool DGRAD>
+__global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ w,
+                                                                    const float* __restrict__ bias, float* __restrict__ y)
+{
+	typedef FewOut P;
+	__shared__ __attribute__((aligned(1024))) uint8_t smem[P::S * P::STAGE];
+
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int trow = tid >> 5, tq = tid & 31;  // this thread's row of the tile and its group of four pixels
+	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
+	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
+	const int n = blockIdx.y;
+	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+
+	// ---- what this lane fetches for each of its wavefront's loads (load q = wave + 4 i); always the same lanes
+	uint32_t voff[P::LPW];
+	uint64_t mask[P::LPW];
+	const uint32_t smem_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem;
+#pragma unroll
+	for (int i = 0; i < P::LPW; i++) {
+		const int idx = (wave + 4 * i) * 64 + lane;
+		const int f = idx % P::F4R, r = (idx / P::F4R) % P::PR, c = idx / (P::F4R * P::PR);
+		const int gy = h0 - g.ph + r, gx = w0 - 4 + 4 * f;
+		const bool valid = idx < P::PATCH_F4 && gy >= 0 && gy < g.H && gx >= 0 && gx < g.W;
+		voff[i] = valid ? (uint32_t)((((int64_t)c * g.H + gy) * g.W + gx) * 4) : 0;
+		mask[i] = __ballot(valid);
+	}
+	// loads of this wavefront that fetch anything at all (a load whose lanes are all switched off may or may not
+	// count as in flight; waiting for this many per chunk is right either way)
+	int nload = 0;
+#pragma unroll
+	for (int i = 0; i < P::LPW; i++) nload += mask[i] != 0 ? 1 : 0;
+	// waits until at most the loads of `chunks` chunks are in flight (loads return in order)
+	auto wait_all_but = [&](int chunks) {
+		switch (chunks * nload) {
+		case 0: wait_vmcnt<0>(); break;
+		case 1: wait_vmcnt<1>(); break;
+		case 2: wait_vmcnt<2>(); break;
+		case 3: wait_vmcnt<3>(); break;
+		case 4: wait_vmcnt<4>(); break;
+		case 5: wait_vmcnt<5>(); break;
+		case 6: wait_vmcnt<6>(); break;
+		case 8: wait_vmcnt<8>(); break;
+		case 10: wait_vmcnt<10>(); break;
+		default: wait_vmcnt<12>(); break;
+		}
+	};
+	static_assert(P::LPW == 6 && P::S <= 3, "the switch above lists the products of 0..2 chunks and 0..6 loads");
+	const int64_t x_step = (int64_t)P::CB * g.H * g.W;
+	auto issue = [&](int stage, int kt) {
+#pragma unroll
+		for (int i = 0; i < P::LPW; i++) async_load16_masked(mask[i], smem_addr + stage * P::STAGE + (wave + 4 * i) * 1024, xn + kt * x_step, voff[i]);
+	};
+
+	// ---- zeros everywhere once: what no load ever writes is the padding
+	for (int i = tid; i < P::S * P::STAGE / 16; i += 256) reinterpret_cast<float4*>(smem)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	__syncthreads();
+	const int KT = g.Cin / P::CB;
+#pragma unroll
+	for (int st = 0; st < P::S; st++)
+		if (st < KT) issue(st, st);
+
+	float acc[COUT][4];
+#pragma unroll
+	for (int co = 0; co < COUT; co++)
+#pragma unroll
+		for (int j = 0; j < 4; j++) acc[co][j] = 0.0f;
+
+	// columns 4 tq + 3 .. 4 tq + 8 of patch row trow + i hold input columns (w0 + 4 tq - 1) .. + 5
+	const int off = (trow * P::PWS + 4 * tq + 3) * 4;
+	int stage = 0;
+	for (int kt = 0; kt < KT; kt++) {
+		wait_all_but(min(P::S - 1, KT - 1 - kt));  // chunk kt has landed; the chunks after it may still be on their way
+		__syncthreads();
+		const uint8_t* sbase = smem + stage * P::STAGE + off;
+#pragma unroll
+		for (int c = 0; c < P::CB; c++) {
+			const int ci = kt * P::CB + c;
+#pragma unroll
+			for (int i = 0; i < 3; i++) {
+				const float* sp = reinterpret_cast<const float*>(sbase + ((c * P::PR + i) * P::PWS) * 4);
+				// the four own columns in one read; the neighbours' from the lanes beside this one (their own reads), except
+				// at the ends of the tile row: a 4-byte read per lane would put eight lanes on every bank it touches
+				const float4 mid = *reinterpret_cast<const float4*>(sp + 1);
+				float left = __shfl_up(mid.w, 1, 64), right = __shfl_down(mid.x, 1, 64);
+				if (tq == 0) left = sp[0];
+				if (tq == 31) right = sp[5];
+				const float v[6] = { left, mid.x, mid.y, mid.z, mid.w, right };
+#pragma unroll
+				for (int co = 0; co < COUT; co++) {
+					// weight (co, ci, i, j) of the convolution computed here
+					const float* wr = DGRAD ? w + (((int64_t)ci * g.Cout + co) * 3 + (2 - i)) * 3 : w + (((int64_t)co * g.Cin + ci) * 3 + i) * 3;
+#pragma unroll
+					for (int j = 0; j < 3; j++) {
+						const float wv = DGRAD ? wr[2 - j] : wr[j];
+#pragma unroll
+						for (int p = 0; p < 4; p++) acc[co][p] = fmaf(v[p + j], wv, acc[co][p]);
+					}
+				}
+			}
+		}
+		__syncthreads();  // everybody is done with this stage
+		if (kt + P::S < KT) issue(stage, kt + P::S);
+		stage = stage + 1 == P::S ? 0 : stage + 1;
+	}
+
+	const int ho = h0 + trow, wo = w0 + 4 * tq;
+	if (ho >= g.Ho || wo >= g.Wo) return;
+	const int64_t plane = (int64_t)g.Ho * g.Wo;
+	float* yp = y + ((int64_t)n * g.Cout * g.Ho + ho) * g.Wo + wo;
+#pragma unroll
+	for (int co = 0; co < COUT; co++) {
+		const float b = bias ? bias[co] : 0.0f;
+		*reinterpret_cast<float4*>(yp + co * plane) = make_float4(acc[co][0] + b, acc[co][1] + b, acc[co][2] + b, acc[co][3] + b);
+	}
+}
+
+bool conv_fewout_takes(const ConvGeo& g, const float* x, const float* y)
+{
+	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw == 1 && g.ph <= 2 && g.Cout >= 1 && g.Cout <= 4 &&
+	       g.Cin % 4 == 0 && g.Cin >= 4 && g.W % 4 == 0 && aligned16(x) && aligned16(y) && (uint64_t)g.H * g.W < (1u << 26) && g.N < 65536;
+}
+
+// dgrad: w is the weight array of the convolution whose data gradient this is ([g.Cin][g.Cout][3][3] in terms of g)
+template <bool DGRAD>
+static int launch_fewout(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
+{
+	const dim3 grid((unsigned)(ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 8)), (unsigned)g.N), block(256);
+	switch (g.Cout) {
+	case 1: conv2d_fewout_forward_kernel<1, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
+	case 2: conv2d_fewout_forward_kernel<2, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
+	case 3: conv2d_fewout_forward_kernel<3, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
+	default: conv2d_fewout_forward_kernel<4, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
+	}
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int conv_fewout_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y, bool dgrad)
+{
+	set_kernel_name(dgrad ? "conv2d_fewout_dgrad_3x3_8x128" : "conv2d_fewout_forward_3x3_8x128");
+	return dgrad ? launch_fewout<true>(g, x, w, bias, y) : launch_fewout<false>(g, x, w, bias, y);
+}
+
+}  // namespace lten_hip
