@@ -106,12 +106,22 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 	const int off = (trow * P::PWS + 4 * tq + 3) * 4;
 	int stage = 0;
 	for (int kt = 0; kt < KT; kt++) {
+		// this chunk's weights first (wave-uniform, scalar loads), so that they arrive while the patch is awaited
+		float wt[P::CB][COUT][9];
+#pragma unroll
+		for (int c = 0; c < P::CB; c++)
+#pragma unroll
+			for (int co = 0; co < COUT; co++) {
+				const int ci = kt * P::CB + c;
+				const float* wr = DGRAD ? w + ((int64_t)ci * g.Cout + co) * 9 : w + ((int64_t)co * g.Cin + ci) * 9;
+#pragma unroll
+				for (int t = 0; t < 9; t++) wt[c][co][t] = DGRAD ? wr[8 - t] : wr[t];  // tap t = 3 i + j of the convolution computed here
+			}
 		wait_all_but(min(P::S - 1, KT - 1 - kt));  // chunk kt has landed; the chunks after it may still be on their way
 		__syncthreads();
 		const uint8_t* sbase = smem + stage * P::STAGE + off;
 #pragma unroll
 		for (int c = 0; c < P::CB; c++) {
-			const int ci = kt * P::CB + c;
 #pragma unroll
 			for (int i = 0; i < 3; i++) {
 				const float* sp = reinterpret_cast<const float*>(sbase + ((c * P::PR + i) * P::PWS) * 4);
@@ -124,11 +134,9 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 				const float v[6] = { left, mid.x, mid.y, mid.z, mid.w, right };
 #pragma unroll
 				for (int co = 0; co < COUT; co++) {
-					// weight (co, ci, i, j) of the convolution computed here
-					const float* wr = DGRAD ? w + (((int64_t)ci * g.Cout + co) * 3 + (2 - i)) * 3 : w + (((int64_t)co * g.Cin + ci) * 3 + i) * 3;
 #pragma unroll
 					for (int j = 0; j < 3; j++) {
-						const float wv = DGRAD ? wr[2 - j] : wr[j];
+						const float wv = wt[c][co][3 * i + j];
 #pragma unroll
 						for (int p = 0; p < 4; p++) acc[co][p] = fmaf(v[p + j], wv, acc[co][p]);
 					}
