@@ -182,6 +182,7 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	const uint64_t Cout = g.Cout, N = g.N;
 	const int HW = g.Ho * g.Wo;
 	const int variant = get_option(OPT_CONV_VARIANT);  // 0 automatic, 1 implicit GEMM for every shape
+	if (variant == 0 && conv_fewin_takes(g, x, y)) return conv_fewin_forward(g, x, w, bias, y);
 	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
 	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS

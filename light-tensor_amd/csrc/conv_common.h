@@ -30,6 +30,10 @@ int conv_patch_fast_wgrad(const ConvGeo& g, const float* x, const float* dy, flo
 bool conv_fewout_takes(const ConvGeo& g, const float* x, const float* y);
 int conv_fewout_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y, bool dgrad);
 
+// 3x3, stride 1, one or two input channels: a stream of y from registers, no LDS (conv_fewin.hip).
+bool conv_fewin_takes(const ConvGeo& g, const float* x, const float* y);
+int conv_fewin_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y);
+
 // Kernels for stride 1, dilation 1 and Cin*kh*kw <= 32 (first layers): the whole reduction fits one MFMA tile
 // dimension, the work is bound by the HBM traffic of y / dy (conv_smallk.hip).
 bool conv_smallk_takes(const ConvGeo& g);
