@@ -15,21 +15,12 @@
 
 namespace lten_hip {
 
+// v[ci][i][0..5] = input columns wo - 1 .. wo + 4 of input row ho - ph + i of image n (zero outside the image, all
+// zero for a thread that is not `inside` the output).  To be called by all 64 lanes of a wavefront: the columns
+// beside a thread's own four come from the adjacent lanes.
 template <int CIN>
-__global__ __launch_bounds__(256) void conv2d_fewin_forward_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ w,
-                                                                   const float* __restrict__ bias, float* __restrict__ y)
+__device__ __forceinline__ void load_window(const ConvGeo& g, const float* __restrict__ x, int n, int ho, int wo, int tq, bool inside, float (&v)[CIN][3][6])
 {
-	constexpr int TH = 8, TW = 128, CG = 8;
-	const int tid = threadIdx.x;
-	const int trow = tid >> 5, tq = tid & 31;
-	const int tiles_w = (g.Wo + TW - 1) / TW;
-	const int w0 = (int)(blockIdx.x % tiles_w) * TW, h0 = (int)(blockIdx.x / tiles_w) * TH;
-	const int n = blockIdx.y;
-	const int ho = h0 + trow, wo = w0 + 4 * tq;  // Wo == W: the pixel columns are the input columns
-	const bool inside = ho < g.Ho && wo < g.W;
-
-	// v[ci][i][0..5]: input columns wo - 1 .. wo + 4 of input row ho - ph + i
-	float v[CIN][3][6];
 #pragma unroll
 	for (int ci = 0; ci < CIN; ci++) {
 		const float* xc = x + ((int64_t)n * g.Cin + ci) * g.H * g.W;
@@ -46,6 +37,23 @@ __global__ __launch_bounds__(256) void conv2d_fewin_forward_kernel(ConvGeo g, co
 			v[ci][i][0] = left; v[ci][i][1] = mid.x; v[ci][i][2] = mid.y; v[ci][i][3] = mid.z; v[ci][i][4] = mid.w; v[ci][i][5] = right;
 		}
 	}
+}
+
+template <int CIN>
+__global__ __launch_bounds__(256) void conv2d_fewin_forward_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ w,
+                                                                   const float* __restrict__ bias, float* __restrict__ y)
+{
+	constexpr int TH = 8, TW = 128, CG = 8;
+	const int tid = threadIdx.x;
+	const int trow = tid >> 5, tq = tid & 31;
+	const int tiles_w = (g.Wo + TW - 1) / TW;
+	const int w0 = (int)(blockIdx.x % tiles_w) * TW, h0 = (int)(blockIdx.x / tiles_w) * TH;
+	const int n = blockIdx.y;
+	const int ho = h0 + trow, wo = w0 + 4 * tq;  // Wo == W: the pixel columns are the input columns
+	const bool inside = ho < g.Ho && wo < g.W;
+
+	float v[CIN][3][6];
+	load_window<CIN>(g, x, n, ho, wo, tq, inside, v);
 	if (!inside) return;
 
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
