@@ -7,8 +7,8 @@
 // input value is read once from HBM and used for 9 * Cout multiply-adds.  A workgroup computes 8 rows x 128 columns
 // of one image; a thread owns four consecutive pixels of one row and all output channels.  Input channels come in
 // chunks of four: the patch [4 channels][10 rows][136 columns] (column q = input column w0 - 4 + q) is filled by
-// direct global->LDS loads exactly as it lies in memory, two stages (a third did not help: 26.0 against 24.5 us on a
-// 32-channel 128 x 128 data gradient at batch 32).  Whether a float4 of the patch lies inside the
+// direct global->LDS loads exactly as it lies in memory, two stages (on a 32-channel 128 x 128 data gradient at batch
+// 32 a third stage did not help, 26.0 against 24.5 us, nor did tiles of four rows with twice the workgroups).  Whether a float4 of the patch lies inside the
 // image does not depend on the chunk: lanes whose float4 does not exist never load, and their slots keep the zeros
 // written once.  Per channel and patch row a thread needs six columns (4 t + 3 .. 4 t + 8): its own four in one 16-byte
 // read, the two neighbours from the lanes beside it, and multiplies them with the 3 * Cout weights of that row, which are wave-uniform and come
