@@ -100,6 +100,9 @@ def test_conv_layer_golden(gpu):
                                  # pad 1: the streaming kernel on the vector ALUs; ragged tiles both ways, row pad 0 / 1 / 2
                                  (2, 8, 9, 132, 3, 3, 3, 1, 1, 1, 1), (1, 4, 5, 8, 1, 3, 3, 0, 1, 1, 1), (2, 12, 17, 260, 4, 3, 3, 2, 1, 1, 1),
                                  (2, 2, 10, 64, 16, 3, 3, 1, 1, 1, 1), (1, 4, 7, 36, 8, 3, 3, 0, 1, 1, 1), (3, 1, 20, 128, 32, 3, 3, 1, 1, 1, 1),
+                                 # one or two input channels at the smallest sizes: a single quad of pixels, one row, row pad 2,
+                                 # a channel count that is no multiple of the groups of eight
+                                 (1, 1, 1, 4, 1, 3, 3, 1, 1, 1, 1), (2, 2, 3, 4, 5, 3, 3, 2, 1, 1, 1), (1, 1, 9, 260, 19, 3, 3, 0, 1, 1, 1),
                                  # stride 1 with Cin*kh*kw <= 32 (first-layer kernels): ragged widths, two column
                                  # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
