@@ -1,13 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the int8 FullyConnected_q forward at M=N=K=4096 on one MI355X.
 
-A step is one lten_hip_quantized_matmul call (the whole FC forward: MFMA GEMM with the
+A step is one FullyConnected_q forward (lten_hip_fcq_forward_prepared: MFMA GEMM with the
 zero-point correction and the requantize fused in) over one synthetic batch whose operands
-are already resident in HBM.  Prints ONE JSON line.  The headline fields describe config 3;
+are already resident in HBM; the layer's weights were converted to int8 once, when the layer
+was set up, as the host-side FullyConnected_q does in to(GPU).  The same step on l-ten's raw
+uint8 weight bytes (lten_hip_quantized_matmul) is timed beside it.  Prints ONE JSON line.  The headline fields describe config 3;
 "configs" adds one record per other benchmark configuration (1, 2, 4, 5) and one for the Conv2d_q
 forward, each with its own roofline figure and the CPU path timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra] [--copy-calibration MiB]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra] [--no-vendor] [--copy-calibration MiB]
 """
 import argparse
 import ctypes as C
@@ -31,7 +33,46 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published: 8 TB/s
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the
 # same counters on the plain copy kernel (--copy-calibration): FETCH_SIZE reads half the bytes
 # the copy kernel is known to fetch (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
-TRAFFIC_BYTES = {"qgemm_fast_256x256x128_w2x4_s2": 49250 * 1024 * 2.0 + 16384 * 1024 * 1.0}
+# Source of the figures: profiles/qgemm_fast_256x256x128_cfg3_4096.md (KiB per dispatch as rocprofv3 printed them).
+TRAFFIC_KIB = {"qgemm_fast_256x256x128_w4x2_s2_wpre": {"FETCH_SIZE": None, "WRITE_SIZE": None},
+               "qgemm_fast_256x256x128_w4x2_s2": {"FETCH_SIZE": None, "WRITE_SIZE": None}}
+
+
+def traffic_bytes(kernel):
+    t = TRAFFIC_KIB.get(kernel)
+    if not t or t["FETCH_SIZE"] is None or t["WRITE_SIZE"] is None:
+        return None
+    return t["FETCH_SIZE"] * 1024 * 2.0 + t["WRITE_SIZE"] * 1024 * 1.0
+
+
+VENDOR_SCRIPT = r"""
+import json, sys, torch
+n = 4096
+a = torch.randint(0, 256, (n, n), device="cuda").sub(128).to(torch.int8)
+w = (torch.randn(n, n, device="cuda") * 40).round().clamp(-127, 127).to(torch.int8)
+b = w.t()   # the FullyConnected layout: weights [N, K], K contiguous
+for _ in range(300): torch._int_mm(a, b)
+torch.cuda.synchronize()
+e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+e0.record()
+for _ in range(300): torch._int_mm(a, b)
+e1.record(); torch.cuda.synchronize()
+us = e0.elapsed_time(e1) / 300 * 1e3
+print(json.dumps({"us": round(us, 2), "tops": round(2 * n ** 3 / us / 1e6, 1), "torch": torch.__version__}))
+"""
+
+
+def vendor_int8(timeout_s=240):
+    """The vendor's int8 GEMM (torch._int_mm, i.e. hipBLASLt) on the same shape and value distributions, in a
+    process of its own: a calibration of what the part sustains, not part of the product.  None when torch
+    cannot run here."""
+    import subprocess
+    try:
+        r = subprocess.run([sys.executable, "-c", VENDOR_SCRIPT], capture_output=True, text=True, timeout=timeout_s)
+        line = [l for l in r.stdout.splitlines() if l.startswith("{")]
+        return json.loads(line[-1]) if r.returncode == 0 and line else {"error": (r.stderr or r.stdout)[-300:]}
+    except Exception as e:  # noqa: BLE001
+        return {"error": repr(e)[:300]}
 
 
 def timed(lt, fn, iters, warmup=3):
@@ -180,21 +221,64 @@ def extra_configs(lt, wl, with_cpu):
            "note": "fourteen dependent launches of about 5 us each; the launch-to-launch latency, not the MFMA rate, sets this time "
                    "(GEMM flops only in the rate); replaying the step as one recorded graph does not shorten it"}
     if with_cpu:
-        hA = [np.random.default_rng(i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
-        hG = [np.random.default_rng(9 + i).standard_normal((B_, n)).astype(np.float32) for i, n in enumerate(sizes)]
+        # The CPU step on the configuration's own data: activations and gradients of the real network.  Two columns:
+        # l-ten's default build multiplies with OpenBLAS (makefile USE_OPENBLAS=1; numpy's matmul is its bundled
+        # OpenBLAS sgemm), its other build with its own threadpool + AVX cpu_gemm (compiled from l-ten's sources where
+        # present).  Bias add, relu, log_softmax, the loss and their backward run in numpy in both.
+        onehot = np.eye(sizes[-1], dtype=np.float32)[labels]
+
+        def cpu_step(gemm):
+            acts_h, pre_h = [X], [None]
+            for i in range(3):
+                y = gemm(acts_h[i], Ws[i], "nt") + bs[i]
+                pre_h.append(y)
+                acts_h.append(np.maximum(y, 0) if i < 2 else y)
+            z = pre_h[3] - pre_h[3].max(axis=1, keepdims=True)
+            logp_h = z - np.log(np.exp(z).sum(axis=1, keepdims=True))
+            loss_h = -(logp_h * onehot).sum() / B_
+            g = (np.exp(logp_h) - onehot) / np.float32(B_)
+            for i in (2, 1, 0):
+                dw_h = gemm(g, acts_h[i], "tn")
+                db_h = g.sum(axis=0)
+                if i > 0:
+                    g = gemm(g, Ws[i], "nn") * (pre_h[i] > 0)
+            return loss_h, dw_h, db_h
+
+        def gemm_openblas(a, b, mode):
+            return a @ b.T if mode == "nt" else (a.T @ b if mode == "tn" else a @ b)
+
         kinds = set()
 
-        def cpu_step():
-            for i in range(3):
-                kinds.add(cpu_sgemm(ob, 0, 1, B_, sizes[i + 1], sizes[i], hA[i], Ws[i], hA[i + 1], 0.0, threads))
-            for i in (2, 1, 0):
-                kinds.add(cpu_sgemm(ob, 0, 0, B_, sizes[i], sizes[i + 1], hG[i + 1], Ws[i], hG[i], 0.0, threads))
-                dw = np.empty_like(Ws[i])
-                kinds.add(cpu_sgemm(ob, 1, 0, sizes[i + 1], sizes[i], B_, hG[i + 1], hA[i], dw, 0.0, threads))
-        cpu_step()
-        t = best_of(cpu_step, 5)
-        rec.update(cpu_ms=round(t * 1e3, 2), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)), speedup=round(t * 1e3 / ms, 1),
-                   cpu_note="l-ten's own threadpool + AVX cpu_gemm (its non-OpenBLAS build); bias, column-sum, relu and loss pieces left out of the CPU leg")
+        def gemm_lten(a, b, mode):
+            a, b = np.ascontiguousarray(a, np.float32), np.ascontiguousarray(b, np.float32)
+            if mode == "nt":
+                Mg, Kg, Ng = a.shape[0], a.shape[1], b.shape[0]
+                tA, tB = 0, 1
+            elif mode == "tn":
+                Kg, Mg, Ng = a.shape[0], a.shape[1], b.shape[1]
+                tA, tB = 1, 0
+            else:
+                Mg, Kg, Ng = a.shape[0], a.shape[1], b.shape[1]
+                tA, tB = 0, 0
+            c = np.empty((Mg, Ng), np.float32)
+            kinds.add(cpu_sgemm(ob, tA, tB, Mg, Ng, Kg, a, b, c, 0.0, threads))
+            return c
+
+        cpu_step(gemm_openblas)
+        t_blas = best_of(lambda: cpu_step(gemm_openblas), 7)
+        cpu_step(gemm_lten)
+        t_lten = best_of(lambda: cpu_step(gemm_lten), 5)
+        try:
+            from threadpoolctl import threadpool_info
+            blas = [f"{i.get('internal_api')} {i.get('version')} x{i.get('num_threads')}" for i in threadpool_info() if i.get("user_api") == "blas"]
+        except Exception:  # noqa: BLE001
+            blas = []
+        t = min(t_blas, t_lten)
+        rec.update(cpu_ms=round(t * 1e3, 2), cpu_cores=threads, speedup=round(t * 1e3 / ms, 1),
+                   cpu_openblas_ms=round(t_blas * 1e3, 2), cpu_openblas=blas or "numpy matmul",
+                   cpu_lten_threadpool_avx_ms=round(t_lten * 1e3, 2), cpu_kind="+".join(sorted(kinds)),
+                   cpu_note="one training step on the configuration's own activations, GEMMs through numpy's OpenBLAS sgemm (l-ten's "
+                            "default backend) and through l-ten's threadpool + AVX cpu_gemm; speedup is quoted against the faster of the two")
     out.append(rec)
     del acts, pre, grads, tmpg, dWs, dbs, gWs, gbs_
 
@@ -253,9 +337,23 @@ def extra_configs(lt, wl, with_cpu):
                     im2col(xin[n].reshape(-1), Cin, H, Wd, 3, 3, 1, 1, 1, 1, col.reshape(-1))
                     kinds.add(cpu_sgemm(ob, 0, 1, Cout, Kc, HW, np.ascontiguousarray(dyh[n].reshape(Cout, HW)), col, dwh, 1.0, threads))
             cpu_pass()
-            t = best_of(cpu_pass, 2) * (Nimg / sample)
+            t_lten = best_of(cpu_pass, 2) * (Nimg / sample)
+
+            def cpu_pass_openblas():  # the same loop with the products through numpy's OpenBLAS sgemm (l-ten's default backend)
+                col2 = col.reshape(Kc, HW)
+                for n in range(sample):
+                    im2col(xin[n].reshape(-1), Cin, H, Wd, 3, 3, 1, 1, 1, 1, col.reshape(-1))
+                    np.matmul(wmat, col2, out=yimg)
+                for n in range(sample):
+                    im2col(xin[n].reshape(-1), Cin, H, Wd, 3, 3, 1, 1, 1, 1, col.reshape(-1))
+                    dwh[...] += dyh[n].reshape(Cout, HW) @ col2.T
+            cpu_pass_openblas()
+            t_blas = best_of(cpu_pass_openblas, 2) * (Nimg / sample)
+            t = min(t_lten, t_blas)
             rec.update(cpu_ms=round(t * 1e3, 1), cpu_cores=threads, cpu_kind="+".join(sorted(kinds)),
-                       cpu_sample=f"{sample} of {Nimg} images, scaled", speedup=round(t * 1e3 / (ms_f + ms_w), 1))
+                       cpu_openblas_ms=round(t_blas * 1e3, 1), cpu_lten_threadpool_avx_ms=round(t_lten * 1e3, 1),
+                       cpu_sample=f"{sample} of {Nimg} images, scaled; speedup against the faster of the two CPU columns",
+                       speedup=round(t * 1e3 / (ms_f + ms_w), 1))
         out.append(rec)
 
     # ---- beyond the five configs: Conv2d_q forward, the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network
@@ -319,6 +417,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run output check")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config records for configs 1, 2, 4, 5")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the torch._int_mm (hipBLASLt) calibration leg")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="run only the plain copy kernel on buffers of this size (what FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -348,13 +447,43 @@ def main():
 
     M = N = K = 4096
     X, W, sc, zp = wl.cfg3()
+    l = lt.lib()
     dA, dB = lt.DeviceBuffer.from_numpy(X), lt.DeviceBuffer.from_numpy(W)
+    dBp = lt.DeviceBuffer(N * K)
+    lt.check(l.lten_hip_fcq_prepare_weights(dB.ptr, dBp.ptr, N * K))   # once per layer, as FullyConnected_q::to(GPU) does
     dC = lt.DeviceBuffer(M * N)
     ws = lt.DeviceBuffer(4 * (M + N))
     qp = lt.qparams3(sc, zp)
 
     def step():
+        lt.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dA.ptr, dBp.ptr, None, qp, dC.ptr, ws.ptr))
+
+    def step_raw():
         lt.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
+
+    # The sustained figure: clocks settle only after tens of milliseconds of load, so the roofline fraction is taken
+    # from 300 back-to-back launches that follow at least 60 ms of the same launches.  It runs before the timed region,
+    # which therefore starts on a part that is already in its steady state.
+    def sustained(fn):
+        t_end = time.perf_counter() + 0.06
+        n = 0
+        while time.perf_counter() < t_end or n < 600:
+            fn()
+            n += 1
+            if n % 100 == 0:
+                lt.sync()
+        lt.sync()
+        t = lt.Timer()
+        t.start()
+        for _ in range(300):
+            fn()
+        return t.stop_ms() / 300
+
+    ops = 2.0 * M * N * K
+    raw_ms = sustained(step_raw)
+    raw_kernel = lt.last_kernel()
+    sustained_ms = sustained(step)
+    achieved = ops / (sustained_ms * 1e-3) / 1e12
 
     for _ in range(args.warmup):
         step()
@@ -369,10 +498,8 @@ def main():
     wall = time.perf_counter() - t0
     kernel = lt.last_kernel()
 
-    ops = 2.0 * M * N * K
     ms_per_step = wall / args.steps * 1e3
     value = ops / (ms_per_step * 1e-3) / 1e12
-    achieved = ops / (kernel_ms * 1e-3) / 1e12
 
     # The same call as an l-ten caller without device-resident tensors sees it: synchronous upload of both operands,
     # the product, synchronous download of the output (never the reported value).
@@ -381,7 +508,7 @@ def main():
     def with_copies():
         dA.upload(X)
         dB.upload(W)
-        step()
+        step_raw()
         lt.check(lt.lib().lten_hip_copy_from_gpu(host_out.ctypes.data, dC.ptr, host_out.nbytes))
     with_copies()
     copies_ms = best_of(with_copies, 3) * 1e3
@@ -390,14 +517,24 @@ def main():
     if not args.no_verify:
         acc = ((X.astype(np.float64) - float(zp[0])) @ (W.astype(np.float64) - float(zp[1])).T)
         mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
-        s = (acc.astype(np.float32) * mult).astype(np.float32) + np.float32(zp[2])
-        want = (np.trunc(s).astype(np.int64) & 0xFF).astype(np.uint8)
-        verified = bool(np.array_equal(dC.numpy(np.uint8, (M, N)), want))
+        sfl = (acc.astype(np.float32) * mult).astype(np.float32) + np.float32(zp[2])
+        want = (np.trunc(sfl).astype(np.int64) & 0xFF).astype(np.uint8)
+        step()
+        ok_prepared = bool(np.array_equal(dC.numpy(np.uint8, (M, N)), want))
+        lt.check(l.lten_hip_zero(dC.ptr, M * N))
+        step_raw()
+        verified = ok_prepared and bool(np.array_equal(dC.numpy(np.uint8, (M, N)), want))
 
+    # MFMA-only ceilings of this part: constant operands, and operands that change like a GEMM's, at 1, 2 and 4
+    # wavefronts per SIMD
     measured_peak = lt.measure_mfma_peak(0, 1)
     _, shader_mhz = lt.measure_last_clocks()
-    measured_peak_data = lt.measure_mfma_peak(2, 1)  # the same loop on operands that change like a GEMM's
-    _, shader_mhz_data = lt.measure_last_clocks()
+    data_peaks, data_mhz = {}, {}
+    for wps in (1, 2, 4):
+        data_peaks[wps] = lt.measure_mfma_peak(2, wps)
+        data_mhz[wps] = lt.measure_last_clocks()[1]
+    measured_peak_data = max(data_peaks.values())
+    vendor = None if args.no_vendor else vendor_int8()
 
     out = {
         "metric": "int8_fc_forward_tops_4096",
@@ -415,18 +552,24 @@ def main():
         "config": {"workload": "cfg3 int8 FullyConnected_q forward M=N=K=4096: uint8 activations (zero point 128) x "
                                "8-bit weights (N(0,40) clipped, zero point 128) -> int32 -> fused requantize to uint8",
                    "M": M, "N": N, "K": K, "input_digest": wl.digest(X, W)},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": TRAFFIC_BYTES.get(kernel),
-                     "kernel": kernel, "kernel_us": round(kernel_ms * 1e3, 2), "algorithmic_bytes": 3 * M * N,
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
+                     "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic_bytes(kernel),
+                     "kernel": kernel, "sustained_kernel_us": round(sustained_ms * 1e3, 2),
+                     "timed_region_kernel_us": round(kernel_ms * 1e3, 2), "algorithmic_bytes": 3 * M * N,
+                     "raw_uint8_weights": {"kernel": raw_kernel, "sustained_kernel_us": round(raw_ms * 1e3, 2),
+                                           "tops": round(ops / (raw_ms * 1e-3) / 1e12, 1)},
                      "measured_mfma_only_tops": round(measured_peak, 1), "measured_mfma_only_shader_mhz": round(shader_mhz),
-                     "frac_of_measured_mfma_only": round(achieved / measured_peak, 4),
-                     "measured_mfma_only_data_operands_tops": round(measured_peak_data, 1),
-                     "measured_mfma_only_data_operands_shader_mhz": round(shader_mhz_data),
+                     "measured_mfma_only_data_operands_tops": {str(k): round(v, 1) for k, v in data_peaks.items()},
+                     "measured_mfma_only_data_operands_shader_mhz": {str(k): round(v) for k, v in data_mhz.items()},
                      "frac_of_measured_mfma_only_data_operands": round(achieved / measured_peak_data, 4),
-                     "note": "int8 multiply-add counted as 2 ops; achieved/peak in tera-ops per second; "
-                             "measured_mfma_only = a kernel that issues nothing but 32x32x32 int8 MFMAs on constant operands; "
-                             "_data_operands = the same with pseudo-random operands that change with every MFMA (the part "
-                             "lowers its clock under that load although nothing but the matrix pipes is busy)"},
+                     "vendor_int8_gemm_same_shape": vendor,
+                     "note": "int8 multiply-add counted as 2 ops; achieved = 2*4096^3 / sustained_kernel_us (300 back-to-back "
+                             "launches after at least 60 ms of the same load, HIP events on the library's stream); "
+                             "timed_region_kernel_us = the same over the --steps launches; measured_mfma_only = a kernel that "
+                             "issues nothing but 32x32x32 int8 MFMAs on constant operands; _data_operands = the same with "
+                             "pseudo-random operands that change with every MFMA, per wavefronts per SIMD (the part lowers its "
+                             "clock under that load although nothing but the matrix pipes is busy); vendor_int8_gemm_same_shape = "
+                             "torch._int_mm (hipBLASLt) at 4096^3 in a process of its own, a calibration only"},
         "verified_bit_exact": verified,
         "with_pcie_copies": {"ms_per_step": round(copies_ms, 3), "tops": round(ops / (copies_ms * 1e-3) / 1e12, 2),
                              "note": "operands uploaded and the output downloaded with the library's synchronous copies around "
@@ -434,7 +577,7 @@ def main():
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, W, sc, zp)
-    del dA, dB, dC, ws
+    del dA, dB, dBp, dC, ws
     if not args.no_extra:
         out["configs"] = extra_configs(lt, wl, not args.no_cpu)
     print(json.dumps(out), flush=True)

@@ -123,6 +123,19 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
                          const uint8_t* X, const uint8_t* W, const int32_t* bias,
                          const lten_hip_qparams* qparams_in_wt_out, uint8_t* Y, int32_t* workspace);
 
+/* Weights of a FullyConnected_q layer never change between forward calls (l-ten keeps them in the layer,
+ * l-ten/fully_connected.cpp:301-303, and fills them once from a checkpoint).  lten_hip_fcq_prepare_weights turns
+ * the layer's uint8 weight bytes into the int8 values w - 128 the matrix cores multiply (one pass, `count` bytes,
+ * both buffers 16-byte aligned; in place when W_prepared == W), to be done once when the layer moves to the GPU;
+ * lten_hip_fcq_forward_prepared is lten_hip_fcq_forward on such weights and returns bit-identical outputs.  What
+ * it saves is the per-use conversion of the weight operand inside the GEMM's main loop.  qparams are the layer's
+ * unchanged (the weight zero point still refers to the uint8 representation).  No counterpart in l-ten, whose
+ * quantized layers are CPU-only. */
+int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t count);
+int lten_hip_fcq_forward_prepared(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features,
+                                  const uint8_t* X, const uint8_t* W_prepared, const int32_t* bias,
+                                  const lten_hip_qparams* qparams_in_wt_out, uint8_t* Y, int32_t* workspace);
+
 /* ------------------------------------------------------------------ im2col / conv */
 
 /* Replace im2col_gpu / col2im_gpu (l-ten/im_col.h:60-73, l-ten/im_col.cu:98-118,164-184).
@@ -236,8 +249,9 @@ int lten_hip_get_min_max(const float* data, uint64_t len, float* min_val, float*
  * compute entry points called on this thread instead of running them; lten_hip_graph_end returns the
  * recording as a handle, and every lten_hip_graph_launch replays it on the library's stream with one submit.
  * Pointers and sizes are recorded by value: the buffers must stay where they are (new contents are fine).
- * Between begin and end only compute entry points may be called: no lten_hip_alloc / free / copy_* / sync /
- * get_min_max (they allocate, copy or wait, which a recording cannot hold), and lten_hip_last_kernel names
+ * Between begin and end only compute entry points may be called: lten_hip_alloc / free / copy_* / sync /
+ * set_stream / get_min_max / event_elapsed_ms fail with a message (they allocate, copy or wait, which a recording
+ * cannot hold), and lten_hip_last_kernel names
  * what was recorded, not what ran.  When the library is on the null stream the recording uses a stream of
  * the library's own; replays still go to the library's stream.  One capture at a time per process.
  * No counterpart in l-ten, whose GPU branches launch eagerly on the default stream. */

@@ -275,6 +275,7 @@ int lten_hip_conv2d_bias_grad_f32(uint64_t N, uint64_t C, uint64_t HW, const flo
 	LTEN_HIP_REQUIRE(db != nullptr, "conv2d_bias_grad: db is null");
 	LTEN_HIP_REQUIRE(N * HW == 0 || dy != nullptr, "conv2d_bias_grad: dy is null");
 	LTEN_HIP_REQUIRE(C <= CHANNEL_SUM_SLOTS && N < (1ull << 31) && HW < (1ull << 40), "conv2d_bias_grad: more than %d channels", CHANNEL_SUM_SLOTS);
+	if (N * HW == 0) return accumulate ? 0 : lten_hip_zero(db, C * sizeof(float));  // nothing to sum
 	const uint64_t runs = ceil_div(N * HW, 256);
 	const int slices = (int)std::max<uint64_t>(1, std::min<uint64_t>(std::min<uint64_t>(CHANNEL_SUM_SLOTS / C, 64), runs));
 	float* partial = nullptr;

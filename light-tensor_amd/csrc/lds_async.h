@@ -8,26 +8,33 @@ namespace lten_hip {
 
 // One wave-wide 16-byte-per-lane load straight into LDS: lane L's bytes go to lds_addr + 16*L.
 // lds_addr and base are wave-uniform; voff is the lane's byte offset from base.
+// m0 is not named as a clobber: the backend treats it as a reserved register (naming it draws the warning that
+// reserved registers on a clobber list are not preserved anyway), never keeps a value in it across statements and
+// writes it itself immediately before each instruction of its own that reads it.
 __device__ __forceinline__ void async_load16(uint32_t lds_addr, const void* base, uint32_t voff)
 {
 	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
 // The same for the lanes of `mask` only, without a branch: a taken branch costs a wavefront that is alone on its
-// SIMD far more than the load (its MFMA stream stops while instructions are fetched again).  To be called where
-// all 64 lanes are active; the execution mask is all ones again afterwards.
+// SIMD far more than the load (its MFMA stream stops while instructions are fetched again).  The execution mask is
+// saved and put back inside the statement, so the compiler never sees it change; lanes that are inactive on entry
+// stay out whatever `mask` says.
 __device__ __forceinline__ void async_load16_masked(uint64_t mask, uint32_t lds_addr, const void* base, uint32_t voff)
 {
-	asm volatile("s_mov_b64 exec, %0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b64 exec, -1"
-	             : : "s"(mask), "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+	uint64_t saved;
+	asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, %0, %1\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %4\n\ts_mov_b64 exec, %0"
+	             : "=&s"(saved) : "s"(mask), "s"(lds_addr), "v"(voff), "s"(base) : "memory", "scc");
 }
 
 // 16 bytes of zeros to LDS byte address lds_lane_addr (per lane) for the lanes of `mask`, without a branch; same
-// conditions as above.  `zero` is a register quadruple holding zeros.
+// handling of the execution mask.  `zero` is a register quadruple holding zeros.
 typedef float lds_v4f __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void lds_zero16_masked(uint64_t mask, uint32_t lds_lane_addr, lds_v4f zero)
 {
-	asm volatile("s_mov_b64 exec, %0\n\tds_write_b128 %1, %2\n\ts_mov_b64 exec, -1" : : "s"(mask), "v"(lds_lane_addr), "v"(zero) : "memory");
+	uint64_t saved;
+	asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, %0, %1\n\tds_write_b128 %2, %3\n\ts_mov_b64 exec, %0"
+	             : "=&s"(saved) : "s"(mask), "v"(lds_lane_addr), "v"(zero) : "memory", "scc");
 }
 
 // s_waitcnt vmcnt(n) only (expcnt and lgkmcnt fields left at "no wait"); n < 64.

@@ -30,6 +30,7 @@ __global__ __launch_bounds__(WAVES * 64) void qdirect_kernel(QProblem p, const i
 	const uint8_t* brow = p.B + (int64_t)(n0 + lrow) * p.b_rs + lgrp * 16;
 	const int steps = (p.K + 63) / 64;
 	const v4i zero = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+	const v4i zero_b = { (int)p.b_flip, (int)p.b_flip, (int)p.b_flip, (int)p.b_flip };  // prepared weights: int8 zeros
 
 	v4i acc = { 0, 0, 0, 0 };
 	int sa = 0, sb = 0;
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(WAVES * 64) void qdirect_kernel(QProblem p, const i
 		for (int u = 0; u < U; u++) {
 			const int k = (s0 + u * WAVES) * 64 + lgrp * 16;
 			fa[u] = zero;
-			fb[u] = zero;
+			fb[u] = zero_b;
 			if (k < p.K) {
 				if (a_ok) fa[u] = *reinterpret_cast<const v4i*>(arow + (int64_t)(s0 + u * WAVES) * 64);
 				if (b_ok) fb[u] = *reinterpret_cast<const v4i*>(brow + (int64_t)(s0 + u * WAVES) * 64);
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(WAVES * 64) void qdirect_kernel(QProblem p, const i
 		}
 #pragma unroll
 		for (int u = 0; u < U; u++) {
-			const v4i a = flip_sign_bits(fa[u]), b = flip_sign_bits(fb[u]);
+			const v4i a = flip_sign_bits(fa[u]), b = flip_bits(fb[u], p.b_flip);
 			sa = __builtin_amdgcn_sdot4(a.x, 0x01010101, sa, false);
 			sa = __builtin_amdgcn_sdot4(a.y, 0x01010101, sa, false);
 			sa = __builtin_amdgcn_sdot4(a.z, 0x01010101, sa, false);

@@ -24,12 +24,14 @@
 #include "common.h"
 #include "qgemm_common.h"
 
+#include <algorithm>
+
 namespace lten_hip {
 
 // One 16-byte chunk of an operand tile, raw bytes (before the XOR), as four dwords.
-// Out-of-range bytes read as 0x80, which becomes 0 after the XOR.
+// Out-of-range bytes read as `pad` (0x80 for uint8 data), which becomes 0 after the XOR.
 template <bool GUARD>
-__device__ __forceinline__ v4i load_chunk(const uint8_t* base, int64_t rs, int64_t ks, int row, int rows, int k, int K, int vec_ok)
+__device__ __forceinline__ v4i load_chunk(const uint8_t* base, int64_t rs, int64_t ks, int row, int rows, int k, int K, int vec_ok, unsigned pad)
 {
 	if (!GUARD) {
 		return *reinterpret_cast<const v4i*>(base + (int64_t)row * rs + k);
@@ -44,7 +46,7 @@ __device__ __forceinline__ v4i load_chunk(const uint8_t* base, int64_t rs, int64
 #pragma unroll
 			for (int b = 0; b < 4; b++) {
 				int kk = k + d * 4 + b;
-				unsigned byte = 0x80u;
+				unsigned byte = pad;
 				if (row < rows && kk < K) byte = base[(int64_t)row * rs + (int64_t)kk * ks];
 				w |= byte << (8 * b);
 			}
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_kernel(QProblem p)
 			// K-strided operands: neighbouring threads take neighbouring rows.
 			int row = (!GUARD || a_kmajor) ? c / CPR : c % BM;
 			int kc = (!GUARD || a_kmajor) ? c % CPR : c / BM;
-			stage_a[i] = load_chunk<GUARD>(p.A, p.a_rs, p.a_ks, m0 + row, p.M, k0 + kc * 16, p.K, p.vec_ok);
+			stage_a[i] = load_chunk<GUARD>(p.A, p.a_rs, p.a_ks, m0 + row, p.M, k0 + kc * 16, p.K, p.vec_ok, 0x80u);
 		}
 #pragma unroll
 		for (int i = 0; i < B_PER_T; i++) {
@@ -118,7 +120,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_kernel(QProblem p)
 			if (B_CHUNKS % T != 0 && c >= B_CHUNKS) break;
 			int row = (!GUARD || b_kmajor) ? c / CPR : c % BN;
 			int kc = (!GUARD || b_kmajor) ? c % CPR : c / BN;
-			stage_b[i] = load_chunk<GUARD>(p.B, p.b_rs, p.b_ks, n0 + row, p.N, k0 + kc * 16, p.K, p.vec_ok);
+			stage_b[i] = load_chunk<GUARD>(p.B, p.b_rs, p.b_ks, n0 + row, p.N, k0 + kc * 16, p.K, p.vec_ok, p.b_flip & 0xffu);
 		}
 	};
 
@@ -139,7 +141,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_kernel(QProblem p)
 			if (B_CHUNKS % T != 0 && c >= B_CHUNKS) break;
 			int row = (!GUARD || b_kmajor) ? c / CPR : c % BN;
 			int kc = (!GUARD || b_kmajor) ? c % CPR : c / BN;
-			*reinterpret_cast<v4i*>(sb + row * BK + ((kc ^ swz<CPR>(row)) << 4)) = flip_sign_bits(stage_b[i]);
+			*reinterpret_cast<v4i*>(sb + row * BK + ((kc ^ swz<CPR>(row)) << 4)) = flip_bits(stage_b[i], p.b_flip);
 		}
 	};
 
@@ -252,6 +254,7 @@ __global__ __launch_bounds__(256) void qgemm_terms_kernel(QProblem p, int coef_a
 	const uint8_t* base = is_a ? p.A : p.B;
 	const int64_t rs = is_a ? p.a_rs : p.b_rs, ks = is_a ? p.a_ks : p.b_ks;
 	const int coef = is_a ? coef_a : coef_b;
+	const unsigned unflip = is_a ? 0u : (0x80808080u ^ p.b_flip);  // prepared weights hold b ^ 0x80
 	unsigned sum = 0;
 	if (coef != 0) {
 		const uint8_t* r = base + row * rs;
@@ -260,16 +263,16 @@ __global__ __launch_bounds__(256) void qgemm_terms_kernel(QProblem p, int coef_a
 			for (; k + 16 <= p.K; k += 64 * 16) {
 				v4i v = *reinterpret_cast<const v4i*>(r + k);
 				const unsigned one = 0x01010101u;
-				sum = __builtin_amdgcn_udot4((unsigned)v.x, one, sum, false);
-				sum = __builtin_amdgcn_udot4((unsigned)v.y, one, sum, false);
-				sum = __builtin_amdgcn_udot4((unsigned)v.z, one, sum, false);
-				sum = __builtin_amdgcn_udot4((unsigned)v.w, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.x ^ unflip, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.y ^ unflip, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.z ^ unflip, one, sum, false);
+				sum = __builtin_amdgcn_udot4((unsigned)v.w ^ unflip, one, sum, false);
 			}
 			// tail shorter than 16 bytes: the lane whose chunk straddles K finishes it
 			if (k < p.K)
-				for (int kk = k; kk < p.K && kk < k + 16; kk++) sum += r[kk];
+				for (int kk = k; kk < p.K && kk < k + 16; kk++) sum += r[kk] ^ (unflip & 0xffu);
 		} else {
-			for (int k = lane; k < p.K; k += 64) sum += r[(int64_t)k * ks];
+			for (int k = lane; k < p.K; k += 64) sum += r[(int64_t)k * ks] ^ (unflip & 0xffu);
 		}
 #pragma unroll
 		for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
@@ -305,7 +308,7 @@ static int launch_tile(const QProblem& p, int out, const char* name)
 	return 0;
 }
 
-static int qgemm_dispatch(const QProblem& p, int out)
+static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratch)
 {
 	const bool kmajor = p.a_ks == 1 && p.b_ks == 1;
 	const bool c_ok = (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
@@ -329,7 +332,7 @@ static int qgemm_dispatch(const QProblem& p, int out)
 			int splits = 1;
 			if (want >= 2) splits = want;
 			else if (want == 0 && tiles <= 64 && p.K >= 4096) splits = tiles <= 32 ? 4 : 2;
-			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits) == 0) return 0;
+			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits, scratch) == 0) return 0;
 			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
 		}
 		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
@@ -355,23 +358,22 @@ static int qgemm_dispatch(const QProblem& p, int out)
 		return launch_tile<128, 128, 64, 2, 2, false>(p, out, "qgemm_nt_128x128x64");
 	case 3:
 		return launch_tile<64, 64, 64, 2, 2, true>(p, out, "qgemm_guard_64x64x64");
-#ifdef LTEN_HIP_TUNING_VARIANTS
-	case 11: return launch_tile<256, 256, 64, 2, 4, false>(p, out, "x_256x256x64_w2x4");
-	case 12: return launch_tile<256, 256, 64, 4, 2, false>(p, out, "x_256x256x64_w4x2");
-	case 13: return launch_tile<256, 256, 128, 2, 2, false>(p, out, "x_256x256x128_w2x2");
-	case 14: return launch_tile<256, 256, 128, 2, 4, false>(p, out, "x_256x256x128_w2x4");
-	case 15: return launch_tile<256, 128, 64, 2, 2, false>(p, out, "x_256x128x64_w2x2");
-	case 16: return launch_tile<128, 256, 64, 2, 2, false>(p, out, "x_128x256x64_w2x2");
-	case 17: return launch_tile<256, 128, 128, 2, 2, false>(p, out, "x_256x128x128_w2x2");
-	case 18: return launch_tile<256, 256, 32, 2, 2, false>(p, out, "x_256x256x32_w2x2");
-#endif
 	default:
 		return launch_tile<32, 32, 64, 1, 1, true>(p, out, "qgemm_guard_32x32x64");
 	}
 }
 
+// Scratch for an entry point that must not allocate: the zero-point terms (instead of the caller's workspace) and the
+// split-K buffers (instead of the library's own, which are allocated on first use).
+struct RunScratch {
+	int32_t* terms;      // terms_ints ints
+	uint64_t terms_ints;
+	SplitScratch split;
+};
+
 static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A, const uint8_t* B, void* C,
-                     int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace)
+                     int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace,
+                     bool weights_prepared = false, const RunScratch* scratch = nullptr)
 {
 	LTEN_HIP_REQUIRE(qp != nullptr, "quantized_matmul: qparams is null");
 	if (M == 0 || N == 0) return 0;
@@ -400,13 +402,10 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	volatile float ab = qp[0].scale * qp[1].scale;
 	p.mult = ab / qp[2].scale;
 	p.zp_c = (float)qp[2].zero_point;
-	p.stamps = nullptr;
+	p.b_flip = weights_prepared ? 0u : 0x80808080u;
 	p.split_partial = nullptr;
 	p.split_counters = nullptr;
 	p.splits = 1;
-#ifdef LTEN_HIP_STAMPS
-	if (workspace) p.stamps = reinterpret_cast<long long*>(workspace + ((M + N + 3) & ~3ull));
-#endif
 	p.vec_ok = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (K & 15) == 0 &&
 	           p.a_ks == 1 && p.b_ks == 1;
 
@@ -446,6 +445,11 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 
 	const int coef_a = 128 - zpB, coef_b = 128 - zpA;
 	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {
+		if (scratch != nullptr) {
+			LTEN_HIP_REQUIRE(M + N <= scratch->terms_ints, "quantized_matmul: M + N = %llu exceeds the %llu rows and columns the static scratch holds",
+			                 (unsigned long long)(M + N), (unsigned long long)scratch->terms_ints);
+			workspace = scratch->terms;
+		}
 		LTEN_HIP_REQUIRE(workspace != nullptr, "quantized_matmul: workspace is null");
 		p.cterm = workspace;      // N ints, where l-ten keeps row_vector (:1325)
 		p.rterm = workspace + N;  // M ints, where l-ten keeps col_vector (:1326)
@@ -453,7 +457,14 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		qgemm_terms_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(p, coef_a, coef_b, bias, workspace + N, workspace);
 		LTEN_HIP_LAUNCH_CHECK();
 	}
-	return qgemm_dispatch(p, out);
+	return qgemm_dispatch(p, out, scratch ? &scratch->split : nullptr);
+}
+
+__global__ __launch_bounds__(256) void fcq_prepare_weights_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, uint64_t n16,
+                                                                  const uint8_t* __restrict__ src_tail, uint8_t* __restrict__ dst_tail, int tail)
+{
+	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256) dst[i] = flip_sign_bits(src[i]);
+	if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x] ^ 0x80;
 }
 
 }  // namespace lten_hip
@@ -486,6 +497,28 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
 	// index against the same weights.  Rows of the output are independent of each other, so the loop is
 	// one GEMM with batch * M rows.
 	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, workspace);
+}
+
+int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t count)
+{
+	if (count == 0) return 0;
+	LTEN_HIP_REQUIRE(W && W_prepared, "lten_hip_fcq_prepare_weights: null pointer");
+	LTEN_HIP_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(W_prepared)) & 15) == 0,
+	                 "lten_hip_fcq_prepare_weights: both buffers must be 16-byte aligned");
+	const uint64_t n16 = count / 16;
+	const int tail = (int)(count % 16);
+	const unsigned blocks = (unsigned)std::min<uint64_t>(std::max<uint64_t>(ceil_div(n16, 256), 1), 4096);
+	fcq_prepare_weights_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(reinterpret_cast<const v4i*>(W), reinterpret_cast<v4i*>(W_prepared), n16,
+	                                                                      W + n16 * 16, W_prepared + n16 * 16, tail);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_fcq_forward_prepared(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features, const uint8_t* X,
+                                  const uint8_t* W_prepared, const int32_t* bias, const lten_hip_qparams* qparams, uint8_t* Y,
+                                  int32_t* workspace)
+{
+	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W_prepared, Y, 0, qparams, bias, workspace, true);
 }
 
 }  // extern "C"

@@ -24,7 +24,9 @@ struct QProblem {
 	float mult;            // real_multiplier
 	float zp_c;            // (float) output zero point
 	int vec_ok;            // operand bases and row strides are multiples of 16 bytes
-	long long* stamps;     // tuning builds only: per-workgroup phase timestamps, else null
+	// 0x80808080 when B holds l-ten's uint8 bytes (XORed into int8 on the way into the MFMA), 0 when B was prepared
+	// by lten_hip_fcq_prepare_weights and already holds the int8 values b - 128
+	uint32_t b_flip;
 	// split-K launches of the direct-to-LDS tiles: `splits` workgroups share an output tile, each takes K / splits
 	int32_t* split_partial;     // [tile][split][T*T] partial sums in register order
 	unsigned* split_counters;   // [tile] arrivals; zero between launches
@@ -52,6 +54,30 @@ __device__ __forceinline__ v4i flip_sign_bits(v4i v)
 	return v;
 }
 
+// The same with a wave-uniform pattern: QProblem::b_flip for the weight operand.
+__device__ __forceinline__ v4i flip_bits(v4i v, uint32_t pattern)
+{
+	v.x ^= (int)pattern;
+	v.y ^= (int)pattern;
+	v.z ^= (int)pattern;
+	v.w ^= (int)pattern;
+	return v;
+}
+
+// requant<Q_OUT_U8_FAST> whose result byte lands in byte BYTE of `word`, the other bytes untouched: the
+// convert instruction writes its low byte there itself, so packing four outputs costs no further instruction.
+template <int BYTE>
+__device__ __forceinline__ void requant_into(unsigned& word, int acc, float mult, float zp)
+{
+#pragma clang fp contract(off)
+	float prod = (float)acc * mult;
+	float s = prod + zp;
+	if (BYTE == 0) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(word) : "v"(s));
+	if (BYTE == 1) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(word) : "v"(s));
+	if (BYTE == 2) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(word) : "v"(s));
+	if (BYTE == 3) asm("v_cvt_i32_f32_sdwa %0, %1 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD" : "+v"(word) : "v"(s));
+}
+
 // Exact image of l-ten/math_fns.cpp:1474 for one accumulator.
 template <int OUT>
 __device__ __forceinline__ unsigned requant(int acc, float mult, float zp)
@@ -77,6 +103,14 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 
 // Dispatch of the tuned square-ish kernels (qgemm_fast.hip).  Returns -1 when no fast variant fits.
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant);
-int qgemm_fast_split_dispatch(const QProblem& p, int out, int splits);
+// Split-K launch; scratch == nullptr takes the library's own buffers (allocated on first use), otherwise the
+// caller's SplitScratch (the entry point that allocates nothing hands in its static device array).
+struct SplitScratch {
+	int32_t* partial;
+	size_t partial_bytes;
+	unsigned* counters;  // zero between launches
+	int max_tiles;
+};
+int qgemm_fast_split_dispatch(const QProblem& p, int out, int splits, const SplitScratch* scratch);
 
 }  // namespace lten_hip

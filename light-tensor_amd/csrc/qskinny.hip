@@ -104,7 +104,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 #pragma unroll
 		for (int s = 0; s < STEPS; s++) {
 			v4i fw = *reinterpret_cast<const v4i*>(wfrag + s * 64);
-			fw = flip_sign_bits(fw);
+			fw = flip_bits(fw, p.b_flip);
 			if (SUM_B) {
 				sb = __builtin_amdgcn_sdot4(fw.x, 0x01010101, sb, false);
 				sb = __builtin_amdgcn_sdot4(fw.y, 0x01010101, sb, false);

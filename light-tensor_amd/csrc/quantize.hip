@@ -134,6 +134,7 @@ int lten_hip_get_min_max(const float* data, uint64_t len, float* min_val, float*
 {
 	// l-ten/utils.cpp:203-206
 	LTEN_HIP_REQUIRE(data && min_val && max_val && len > 0, "Invalid argument");
+	LTEN_HIP_REQUIRE(!capturing(), "lten_hip_get_min_max: not allowed between lten_hip_graph_begin and lten_hip_graph_end");
 	const int blocks = (int)std::min<uint64_t>(ceil_div(len, 256), MINMAX_BLOCKS);
 	minmax_partial_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(data, len);
 	LTEN_HIP_LAUNCH_CHECK();

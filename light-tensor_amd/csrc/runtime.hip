@@ -88,14 +88,21 @@ int lten_hip_get_device(int* device)
 	return 0;
 }
 
+// What a recording cannot hold: allocation, freeing, host copies and waits.  They fail with a message of their own
+// while a launch graph is being recorded (the runtime would otherwise invalidate the capture with a generic one).
+#define LTEN_HIP_NOT_WHILE_RECORDING(name) \
+	LTEN_HIP_REQUIRE(!capturing(), name ": not allowed between lten_hip_graph_begin and lten_hip_graph_end")
+
 int lten_hip_set_stream(void* hip_stream)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_set_stream");
 	g_stream = static_cast<hipStream_t>(hip_stream);
 	return 0;
 }
 
 int lten_hip_sync(void)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_sync");
 	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
 	return 0;
 }
@@ -103,14 +110,16 @@ int lten_hip_sync(void)
 int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
 {
 	LTEN_HIP_REQUIRE(device_ptr != nullptr, "lten_hip_alloc: null pointer");
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_alloc");
 	*device_ptr = nullptr;
 	LTEN_HIP_CHECK(hipMalloc(device_ptr, size ? size : 1));
-	if (zero_memory && size) LTEN_HIP_CHECK(hipMemsetAsync(*device_ptr, 0, size, stream()));
+	if (zero_memory && size) return lten_hip_zero(*device_ptr, size);  // a fill kernel, stream ordered
 	return 0;
 }
 
 int lten_hip_free(void* device_ptr)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_free");
 	if (device_ptr) LTEN_HIP_CHECK(hipFree(device_ptr));
 	return 0;
 }
@@ -128,6 +137,7 @@ int lten_hip_zero(void* device_ptr, size_t size)
 
 int lten_hip_copy_to_gpu(void* device_dst, const void* host_src, size_t size)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_copy_to_gpu");
 	if (size == 0) return 0;
 	LTEN_HIP_CHECK(hipMemcpyAsync(device_dst, host_src, size, hipMemcpyHostToDevice, stream()));
 	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
@@ -136,6 +146,7 @@ int lten_hip_copy_to_gpu(void* device_dst, const void* host_src, size_t size)
 
 int lten_hip_copy_from_gpu(void* host_dst, const void* device_src, size_t size)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_copy_from_gpu");
 	if (size == 0) return 0;
 	LTEN_HIP_CHECK(hipMemcpyAsync(host_dst, device_src, size, hipMemcpyDeviceToHost, stream()));
 	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
@@ -144,6 +155,7 @@ int lten_hip_copy_from_gpu(void* host_dst, const void* device_src, size_t size)
 
 int lten_hip_copy_gpu_to_gpu(void* device_dst, const void* device_src, size_t size)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_copy_gpu_to_gpu");
 	if (size == 0) return 0;
 	LTEN_HIP_CHECK(hipMemcpyAsync(device_dst, device_src, size, hipMemcpyDeviceToDevice, stream()));
 	return 0;
@@ -241,6 +253,7 @@ int lten_hip_event_record(void* event)
 
 int lten_hip_event_elapsed_ms(void* start, void* stop, float* ms)
 {
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_event_elapsed_ms");
 	LTEN_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
 	LTEN_HIP_CHECK(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
 	return 0;

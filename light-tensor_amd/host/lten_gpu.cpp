@@ -214,12 +214,6 @@ void Tensor::backward(const Tensor* top_gradient)
 
 // ------------------------------------------------------------------------------ matmul
 
-struct BatchPlan {
-	uint64_t count = 1;
-	int64_t stride_a = 0, stride_b = 0, stride_c = 0;
-	bool uniform = true;  // one strided call covers it
-};
-
 static void leading_offsets(const TensorImpl& a, const TensorImpl& b, const uint64_t* cdims, int ndims, std::vector<uint64_t>& oa,
                             std::vector<uint64_t>& ob)
 {
@@ -242,6 +236,17 @@ static void leading_offsets(const TensorImpl& a, const TensorImpl& b, const uint
 		oa[idx] = offa * ma;
 		ob[idx] = offb * mb;
 	}
+}
+
+// True when the operand offsets of consecutive leading indices advance by constant strides (stride 0 = one operand
+// broadcast over every leading dim), so that one strided-batched launch covers the loop.
+static bool uniform_strides(const std::vector<uint64_t>& oa, const std::vector<uint64_t>& ob, int64_t& sa, int64_t& sb)
+{
+	sa = oa.size() > 1 ? (int64_t)oa[1] : 0;
+	sb = ob.size() > 1 ? (int64_t)ob[1] : 0;
+	for (size_t i = 0; i < oa.size(); i++)
+		if (oa[i] != (uint64_t)sa * i || ob[i] != (uint64_t)sb * i) return false;
+	return true;
 }
 
 Tensor Tensor::matmul(const Tensor& other)
@@ -274,14 +279,20 @@ Tensor Tensor::matmul(const Tensor& other)
 	const float* ad = static_cast<const float*>(a.data);
 	const float* bd = static_cast<const float*>(b.data);
 	float* cd = static_cast<float*>(result.impl_->data);
-	// l-ten/md_array_cuda.h:507-515: one NN GEMM per leading index
-	for (size_t i = 0; i < oa.size(); i++)
-		LTEN_HIP_CALL(lten_hip_sgemm(0, 0, M, N, K, 1.0f, ad + oa[i], K, bd + ob[i], N, 0.0f, cd + i * M * N, N));
+	// l-ten/md_array_cuda.h:507-515 runs one NN GEMM per leading index.  When the operand offsets advance by a constant
+	// stride (no broadcast, or one operand broadcast over all leading dims: stride 0) the whole loop is one launch.
+	int64_t sa = 0, sb = 0;
+	const bool uniform = uniform_strides(oa, ob, sa, sb);
+	if (uniform)
+		LTEN_HIP_CALL(lten_hip_sgemm_strided_batched(0, 0, M, N, K, 1.0f, ad, K, sa, bd, N, sb, 0.0f, cd, N, (int64_t)(M * N), oa.size()));
+	else
+		for (size_t i = 0; i < oa.size(); i++)
+			LTEN_HIP_CALL(lten_hip_sgemm(0, 0, M, N, K, 1.0f, ad + oa[i], K, bd + ob[i], N, 0.0f, cd + i * M * N, N));
 
 	auto ai = impl_, bi = other.impl_;
 	result.impl_->children = { ai, bi };
 	result.impl_->autograd = true;
-	result.impl_->grad_fn = [ai, bi, oa, ob, M, N, K](TensorImpl& self, const float* top) {
+	result.impl_->grad_fn = [ai, bi, oa, ob, M, N, K, uniform, sa, sb](TensorImpl& self, const float* top) {
 		(void)self;
 		// l-ten/backprop.cpp:533-585: per leading index dA += dC B^T (NT), dB += A^T dC (TN), beta = 1 into
 		// zeroed gradients, so a broadcast operand collects the sum over the indices that share it
@@ -289,14 +300,20 @@ Tensor Tensor::matmul(const Tensor& other)
 		const float* bd = static_cast<const float*>(bi->data);
 		if (wants_gradient(ai)) {
 			Bottom g(ai);
-			for (size_t i = 0; i < oa.size(); i++)
-				LTEN_HIP_CALL(lten_hip_sgemm(0, 1, M, K, N, 1.0f, top + i * M * N, N, bd + ob[i], N, 1.0f, g.ptr + oa[i], K));
+			if (uniform)
+				LTEN_HIP_CALL(lten_hip_sgemm_strided_batched(0, 1, M, K, N, 1.0f, top, N, (int64_t)(M * N), bd, N, sb, 1.0f, g.ptr, K, sa, oa.size()));
+			else
+				for (size_t i = 0; i < oa.size(); i++)
+					LTEN_HIP_CALL(lten_hip_sgemm(0, 1, M, K, N, 1.0f, top + i * M * N, N, bd + ob[i], N, 1.0f, g.ptr + oa[i], K));
 			g.propagate();
 		}
 		if (wants_gradient(bi)) {
 			Bottom g(bi);
-			for (size_t i = 0; i < oa.size(); i++)
-				LTEN_HIP_CALL(lten_hip_sgemm(1, 0, K, N, M, 1.0f, ad + oa[i], K, top + i * M * N, N, 1.0f, g.ptr + ob[i], N));
+			if (uniform)
+				LTEN_HIP_CALL(lten_hip_sgemm_strided_batched(1, 0, K, N, M, 1.0f, ad, K, sa, top, N, (int64_t)(M * N), 1.0f, g.ptr, N, sb, oa.size()));
+			else
+				for (size_t i = 0; i < oa.size(); i++)
+					LTEN_HIP_CALL(lten_hip_sgemm(1, 0, K, N, M, 1.0f, ad + oa[i], K, top + i * M * N, N, 1.0f, g.ptr + ob[i], N));
 			g.propagate();
 		}
 	};
@@ -564,6 +581,8 @@ void FullyConnected_q::to(device target_device, int target_device_index)
 	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
 	workspace_ = Tensor();
 	max_rows_ = 0;
+	prepared_ = Tensor();  // the int8 copy of the weights is made again by the next forward
+	prepared_valid_ = false;
 }
 
 void FullyConnected_q::clear_gradients()
@@ -613,10 +632,19 @@ Tensor FullyConnected_q::forward(Tensor& input)
 	}
 	lten_hip_qparams qp[3] = { { qparams_in_.scale, qparams_in_.zero_point }, { qparams_wt_.scale, qparams_wt_.zero_point },
 		                   { qparams_out_.scale, qparams_out_.zero_point } };
-	LTEN_HIP_CALL(lten_hip_fcq_forward(batch, M, input_features_, output_features_, static_cast<const uint8_t*>(input.get_data_ptr()),
-	                                   static_cast<const uint8_t*>(weight_.get_data_ptr()),
-	                                   use_bias_ ? static_cast<const int32_t*>(bias_.get_data_ptr()) : nullptr, qp,
-	                                   static_cast<uint8_t*>(result.get_data_ptr()), static_cast<int32_t*>(workspace_.get_data_ptr())));
+	// The weights are constant between forward calls: their int8 form (w - 128, what the matrix cores multiply) is
+	// made once per to() / weights_changed() and every forward runs on it.
+	if (!prepared_valid_) {
+		options.data_type = UINT8;
+		if (!prepared_.defined()) prepared_ = AllocateTensor({ 1, 1, output_features_, input_features_ }, &options);
+		LTEN_HIP_CALL(lten_hip_fcq_prepare_weights(static_cast<const uint8_t*>(weight_.get_data_ptr()), static_cast<uint8_t*>(prepared_.get_data_ptr()),
+		                                           output_features_ * input_features_));
+		prepared_valid_ = true;
+	}
+	LTEN_HIP_CALL(lten_hip_fcq_forward_prepared(batch, M, input_features_, output_features_, static_cast<const uint8_t*>(input.get_data_ptr()),
+	                                            static_cast<const uint8_t*>(prepared_.get_data_ptr()),
+	                                            use_bias_ ? static_cast<const int32_t*>(bias_.get_data_ptr()) : nullptr, qp,
+	                                            static_cast<uint8_t*>(result.get_data_ptr()), static_cast<int32_t*>(workspace_.get_data_ptr())));
 	return result;
 }
 

@@ -157,10 +157,14 @@ public:
 	void set_qparams_in(QuantizationParams qparams_in) override { qparams_in_ = qparams_in; }
 	void set_qparams_out(QuantizationParams qparams_out) override { qparams_out_ = qparams_out; }
 	void set_qparams_params(QuantizationParams* qparams, int count) override;
+	// to be called after writing new weight bytes into get_weights() while the layer is on the GPU (to() does it itself)
+	void weights_changed() { prepared_valid_ = false; }
 
 private:
 	uint64_t input_features_, output_features_;
 	Tensor weight_, bias_, workspace_;
+	Tensor prepared_;  // int8 form of weight_ for the GEMM (lten_hip_fcq_prepare_weights)
+	bool prepared_valid_ = false;
 	bool use_bias_;
 	uint64_t max_rows_ = 0;
 	QuantizationParams qparams_in_{ 1.0f, 0 }, qparams_out_{ 1.0f, 0 }, qparams_wt_{ 1.0f, 0 };

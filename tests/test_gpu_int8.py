@@ -67,15 +67,18 @@ def test_fast_tiles(gpu, ob, tile, shape):
                  bias=rng.integers(-5000, 5000, N).astype(np.int32) if zp[0] else None, tile=tile)
 
 
-@pytest.mark.parametrize("variant", [21, 23, 24, 26, 28, 31, 33, 34])
-@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 640), (256, 1024, 2048)])
+@pytest.mark.parametrize("variant", [33, 34, 41])
+@pytest.mark.parametrize("shape", [(256, 256, 128), (512, 768, 640), (256, 1024, 2048), (256, 512, 256), (200, 260, 384), (256, 256, 400)])
 def test_direct_to_lds_tiles(gpu, ob, variant, shape):
-    """The tuned 256x256 tiles (LDS stage ring filled by direct global->LDS loads): every wave layout, both
-    k-step sizes, with and without zero-point terms and bias, short and long K (prologue/drain paths)."""
+    """The direct-to-LDS tiles (256 x 256 in both wavefront layouts, 128 x 128): with and without zero-point terms
+    and bias, one to sixteen k-steps (prologue, the half-open refill at the end of the steady loop, drain), ragged
+    M and N, a K that is no multiple of the k-step."""
     M, N, K = shape
     rng = np.random.default_rng(M + N + K + variant)
     A = rng.integers(0, 256, (M, K), dtype=np.uint8)
     B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    if K % 128 != 0 and variant == 34:
+        pytest.skip("this layout takes whole k-steps only")
     run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=variant)
     run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8),
              bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
@@ -87,7 +90,7 @@ def test_requantize_exact_epilogue_in_tiled_kernels(gpu, ob):
     A = rng.integers(0, 256, (256, 256), dtype=np.uint8)
     B = rng.integers(0, 256, (256, 256), dtype=np.uint8)
     for scales in ([300.0, 500.0, 1.0], [1.0, 1.0, 1e-6]):
-        for tile in (0, 1, 3, 31):
+        for tile in (0, 1, 3, 33, 41):
             run_case(gpu, ob, A, B, scales, np.array([128, 128, 9], np.uint8), tile=tile)
 
 
@@ -138,7 +141,7 @@ def test_fcq_forward_leading_dims(gpu, ob, wl):
     assert np.array_equal(dY.numpy(np.uint8, (64, 512)), np.load(golden_path("cfg1_expected.npz"))["C"])
 
 
-@pytest.mark.parametrize("variant", [41, 42, 43, 44])
+@pytest.mark.parametrize("variant", [41])
 @pytest.mark.parametrize("shape", [(128, 128, 128), (384, 640, 640), (128, 1152, 2048),
                                    # ragged M and N (N a multiple of 16): edge tiles fetch the last row again and store what exists
                                    (33, 144, 512), (200, 656, 1152), (1, 16, 128),
@@ -146,7 +149,7 @@ def test_fcq_forward_leading_dims(gpu, ob, wl):
                                    (130, 1000, 256), (64, 12, 640)])
 def test_direct_to_lds_128_tiles(gpu, ob, variant, shape):
     """The 128x128 form of the direct-to-LDS tiles (what the library picks when 256x256 tiles would leave CUs idle):
-    both k-step sizes, 2 to 4 stages, with and without zero-point terms and bias, short and long K; int32 and u8."""
+    with and without zero-point terms and bias, short and long K; int32 and u8."""
     M, N, K = shape
     rng = np.random.default_rng(M + N + K + variant)
     A = rng.integers(0, 256, (M, K), dtype=np.uint8)
@@ -173,7 +176,7 @@ def test_direct_to_lds_tiles_partial_last_k_step(gpu, ob, variant, shape):
     run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)
 
 
-@pytest.mark.parametrize("variant", [31, 33, 34])
+@pytest.mark.parametrize("variant", [33, 34])
 def test_direct_to_lds_256_tiles_ragged(gpu, ob, variant):
     """300 x 272 x 640 on 256 x 256 tiles: two row tiles and two column tiles, all of them edge tiles."""
     rng = np.random.default_rng(variant)
@@ -401,3 +404,60 @@ def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
         run_case(gpu, ob, A, B, sc, zp, bias=bias)
         seen.add(gpu.last_kernel().split("_")[0] + "_" + gpu.last_kernel().split("_")[1])
     assert {"qskinny_mfma", "qdirect_16x16", "qgemm_fast", "qgemm_guard"} <= seen, seen
+
+
+def fcq(gpu, entry, X, W, sc, zp, bias=None, prepared=False):
+    """One FullyConnected_q forward through `entry` (lten_hip_fcq_forward or _prepared); numpy in, numpy out."""
+    D = gpu.DeviceBuffer
+    M, K = X.shape
+    N = W.shape[0]
+    dX, dW, dY, ws = D.from_numpy(X), D.from_numpy(W), D(M * N), D(4 * (M + N))
+    db = D.from_numpy(np.asarray(bias, np.int32)) if bias is not None else None
+    if prepared:
+        dWp = D(W.size + 16)
+        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, W.size))
+        assert np.array_equal(dWp.numpy(np.uint8, W.shape), W ^ 0x80)
+        dW = dWp
+    gpu.check(entry(1, M, K, N, dX.ptr, dW.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
+    return dY.numpy(np.uint8, (M, N)), gpu.last_kernel()
+
+
+@pytest.mark.parametrize("shape", [(64, 512, 784), (16, 2048, 2048), (40, 4096, 2048), (256, 512, 640), (128, 1024, 4096),
+                                   (512, 8192, 512), (300, 260, 400), (70, 50, 5760), (33, 65, 100)])
+def test_prepared_weights_match_unprepared(gpu, ob, shape):
+    """lten_hip_fcq_forward_prepared on int8 weights (w - 128) returns what lten_hip_fcq_forward returns on l-ten's
+    uint8 weights, on every kernel family the shapes select (one-launch, streaming, split-K, 128 and 256 tiles with and
+    without a partial k-step, the guarded general kernel), with all three zero-point patterns and a bias; the
+    unprepared result is checked against the oracle."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    l = gpu.lib()
+    for zp, with_bias in (([128, 128, 128], False), ([0, 128, 3], True), ([200, 17, 99], True)):
+        bias = rng.integers(-5000, 5000, N).astype(np.int32) if with_bias else None
+        sc = [0.02, 0.013, 0.9 * K / 512]
+        want, k0 = fcq(gpu, l.lten_hip_fcq_forward, X, W, sc, zp, bias)
+        got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, X, W, sc, zp, bias, prepared=True)
+        assert np.array_equal(got, want), (shape, zp, k0, k1)
+        Co, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias)
+        assert np.array_equal(want, Co), (shape, zp, k0)
+
+
+def test_prepare_weights_in_place_and_odd_count(gpu):
+    rng = np.random.default_rng(5)
+    for n in (1, 15, 16, 17, 4099, 1 << 20):
+        w = rng.integers(0, 256, n, dtype=np.uint8)
+        d = gpu.DeviceBuffer.from_numpy(w)
+        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, n))
+        assert np.array_equal(d.numpy(np.uint8, (n,)), w ^ 0x80)
+
+
+def test_cfg3_prepared_weights_full_size(gpu, wl):
+    """Config 3 at full size through the prepared-weights entry point: bit-identical to the plain entry point."""
+    X, W, sc, zp = wl.cfg3()
+    l = gpu.lib()
+    want, k0 = fcq(gpu, l.lten_hip_fcq_forward, X, W, sc, zp)
+    got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, X, W, sc, zp, prepared=True)
+    assert k1.endswith("_wpre") and not k0.endswith("_wpre"), (k0, k1)
+    assert np.array_equal(got, want)
