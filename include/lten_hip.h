@@ -136,6 +136,17 @@ int lten_hip_fcq_forward_prepared(uint64_t batch, uint64_t M, uint64_t in_featur
                                   const uint8_t* X, const uint8_t* W_prepared, const int32_t* bias,
                                   const lten_hip_qparams* qparams_in_wt_out, uint8_t* Y, int32_t* workspace);
 
+/* lten_hip_fcq_forward for callers that cannot allocate device memory or hand over a workspace (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in l-ten.  It calls no
+ * hipMalloc / hipFree: the zero-point terms and, for small outputs with a long reduction, the split-K partial sums
+ * and arrival counters live in one static device array of the library (8.3 MB per GPU, held until the process ends).
+ * Limit: batch * M + out_features <= 65536; beyond it the call fails with a message.  Products whose partial sums
+ * would not fit the array's 8 MB run unsplit.  Same outputs as lten_hip_fcq_forward, bit for bit.  Every call on a GPU
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features,
+                                const uint8_t* X, const uint8_t* W, const int32_t* bias,
+                                const lten_hip_qparams* qparams_in_wt_out, uint8_t* Y);
+
 /* ------------------------------------------------------------------ im2col / conv */
 
 /* Replace im2col_gpu / col2im_gpu (l-ten/im_col.h:60-73, l-ten/im_col.cu:98-118,164-184).

@@ -467,6 +467,39 @@ __global__ __launch_bounds__(256) void fcq_prepare_weights_kernel(const v4i* __r
 	if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x] ^ 0x80;
 }
 
+// Scratch of lten_hip_fcq_forward_static: device memory that exists from the moment the library is loaded, so the
+// entry point never allocates.  One copy per GPU (every device the code object is loaded on holds its own); the
+// array's name is only a host-side handle, its device address comes from hipGetSymbolAddress.
+constexpr uint64_t STATIC_TERMS_INTS = 64 * 1024;             // M + N of one call
+constexpr uint64_t STATIC_SPLIT_BYTES = 8u << 20;             // partial sums of a split-K launch
+constexpr int STATIC_SPLIT_TILES = 1024;
+constexpr uint64_t STATIC_SCRATCH_BYTES = STATIC_SPLIT_BYTES + STATIC_TERMS_INTS * 4 + STATIC_SPLIT_TILES * 4;
+static __device__ __align__(256) unsigned char fcq_static_scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 8;  // l-ten/globals.h:15
+static unsigned char* g_static_scratch[MAX_DEVICES] = { nullptr };
+
+// Device address of the current device's copy of the array, looked up once per device.
+static int static_scratch(RunScratch* rs)
+{
+	int dev = -1;
+	LTEN_HIP_CHECK(hipGetDevice(&dev));
+	LTEN_HIP_REQUIRE(dev >= 0 && dev < MAX_DEVICES, "lten_hip_fcq_forward_static: device %d out of range", dev);
+	if (g_static_scratch[dev] == nullptr) {
+		void* ptr = nullptr;
+		LTEN_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(fcq_static_scratch)));
+		LTEN_HIP_REQUIRE(ptr != nullptr, "lten_hip_fcq_forward_static: no device address for the static scratch");
+		g_static_scratch[dev] = static_cast<unsigned char*>(ptr);  // zero-filled when the code object was loaded
+	}
+	unsigned char* base = g_static_scratch[dev];
+	rs->split.partial = reinterpret_cast<int32_t*>(base);
+	rs->split.partial_bytes = STATIC_SPLIT_BYTES;
+	rs->terms = reinterpret_cast<int32_t*>(base + STATIC_SPLIT_BYTES);
+	rs->terms_ints = STATIC_TERMS_INTS;
+	rs->split.counters = reinterpret_cast<unsigned*>(base + STATIC_SPLIT_BYTES + STATIC_TERMS_INTS * 4);
+	rs->split.max_tiles = STATIC_SPLIT_TILES;
+	return 0;
+}
+
 }  // namespace lten_hip
 
 using namespace lten_hip;
@@ -519,6 +552,19 @@ int lten_hip_fcq_forward_prepared(uint64_t batch, uint64_t M, uint64_t in_featur
                                   int32_t* workspace)
 {
 	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W_prepared, Y, 0, qparams, bias, workspace, true);
+}
+
+int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features, const uint8_t* X,
+                                const uint8_t* W, const int32_t* bias, const lten_hip_qparams* qparams, uint8_t* Y)
+{
+	LTEN_HIP_REQUIRE(batch * M + out_features <= STATIC_TERMS_INTS,
+	                 "lten_hip_fcq_forward_static: batch * M + out_features = %llu exceeds the limit of %llu",
+	                 (unsigned long long)(batch * M + out_features), (unsigned long long)STATIC_TERMS_INTS);
+	RunScratch rs;
+	if (int rc = static_scratch(&rs)) return rc;
+	// the array keeps whatever the last call left: the arrival counters of a split-K launch must start at zero
+	if (int rc = lten_hip_zero(rs.split.counters, (size_t)rs.split.max_tiles * sizeof(unsigned))) return rc;
+	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, nullptr, false, &rs);
 }
 
 }  // extern "C"
