@@ -33,9 +33,9 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published: 8 TB/s
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled by the
 # same counters on the plain copy kernel (--copy-calibration): FETCH_SIZE reads half the bytes
 # the copy kernel is known to fetch (factor 2.0), WRITE_SIZE reads them exactly (factor 1.0).
-# Source of the figures: profiles/qgemm_fast_256x256x128_cfg3_4096.md (KiB per dispatch as rocprofv3 printed them).
-TRAFFIC_KIB = {"qgemm_fast_256x256x128_w4x2_s2_wpre": {"FETCH_SIZE": None, "WRITE_SIZE": None},
-               "qgemm_fast_256x256x128_w4x2_s2": {"FETCH_SIZE": None, "WRITE_SIZE": None}}
+# Source of the figures: profiles/qgemm_fast_256x256x128_w4x2_cfg3_4096.md (KiB per dispatch as rocprofv3 printed them).
+TRAFFIC_KIB = {"qgemm_fast_256x256x128_w4x2_s2_wpre": {"FETCH_SIZE": 49240, "WRITE_SIZE": 16384},
+               "qgemm_fast_256x256x128_w4x2_s2": {"FETCH_SIZE": 49240, "WRITE_SIZE": 16384}}
 
 
 def traffic_bytes(kernel):
