@@ -99,6 +99,18 @@ int lten_hip_fc_forward_f32(uint64_t M, uint64_t in_features, uint64_t out_featu
 int lten_hip_fc_backward_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X,
                              const float* W, const float* dY, float* dX, float* dW, float* db);
 
+/* The same two calls with the relu that l-ten places around a hidden layer folded into the GEMM's store, so that a
+ * training step needs fewer dependent launches (each costs about 5 us on this part whatever it computes):
+ * lten_hip_fc_forward_relu_f32 writes the layer's output Y and Y_relu = relu(Y) (lten::relu of the result,
+ * l-ten/layers.cpp:9-67; gpu_relu); lten_hip_fc_backward_relu_f32 applies relu_backward to the data gradient on the
+ * way out, dX = relu_input > 0 ? (dY W) : 0 with relu_input[M x in] the input of the relu that produced X
+ * (l-ten/backprop.cpp:2282-2327; gpu_relu_backward).  Same values as the unfused sequences, bit for bit. */
+int lten_hip_fc_forward_relu_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X,
+                                 const float* W, const float* bias, float* Y, float* Y_relu);
+int lten_hip_fc_backward_relu_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X,
+                                  const float* W, const float* dY, const float* relu_input, float* dX, float* dW,
+                                  float* db);
+
 /* ------------------------------------------------------------------ quantized GEMM */
 
 /* GPU counterpart of quantized_matmul (l-ten/math_fns.h:104, l-ten/math_fns.cpp:1311-1478),
@@ -227,6 +239,13 @@ int lten_hip_log_softmax_f32(uint64_t rows, uint64_t cols, const float* x, float
 int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float* y, const float* dy, float* dx);
 /* gpu_nll (l-ten/math_fns.h:170; l-ten/layers.cpp:212-273): *loss = (sum_i input[i] * target[i]) * (-1 / batches). */
 int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, uint64_t len, uint64_t batches);
+
+/* lten_hip_log_softmax_f32 followed by lten_hip_nll_loss_f32 (batches = rows) as one launch (calls that overlap on
+ * one GPU would share its arrival counter: one stream at a time), and lten_hip_scale_f32(alpha, target) followed by lten_hip_log_softmax_backward_f32 as one:
+ * dx = alpha * target - exp(y) * sum_j alpha * target_j, alpha = -top / rows for l-ten's nll_backward
+ * (l-ten/backprop.cpp:3975-4040).  Same values as the separate calls, bit for bit. */
+int lten_hip_log_softmax_nll_loss_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float* y, float* loss);
+int lten_hip_nll_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float* y, const float* target, float alpha, float* dx);
 
 /* gpu_sgd_step (l-ten/math_fns.h:186; SGDOptimizer::step, l-ten/optimizer.cpp:26-84) for one parameter tensor:
  * grad = wd * w + grad (stored, as in l-ten), velocity = velocity * mo + (1 - mo) * grad, w = w - velocity * lr. */

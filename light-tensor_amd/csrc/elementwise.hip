@@ -98,6 +98,74 @@ __global__ __launch_bounds__(1024) void nll_loss_kernel(const float* __restrict_
 	}
 }
 
+// log_softmax and nll_loss in one launch: the rows are spread over workgroups as in log_softmax_kernel (a wavefront per
+// row), every workgroup counts itself in when its rows are written, and the one that arrives last sums the loss over the
+// whole array in exactly the order nll_loss_kernel uses (reading the log-probabilities past the per-CU cache, since
+// other CUs wrote them) — both results are bit-identical to the two separate launches.  The counter lives in a static
+// device word and is zero again when the kernel ends.
+static __device__ unsigned g_loss_arrivals;
+
+__global__ __launch_bounds__(256) void log_softmax_nll_kernel(uint64_t rows, uint64_t cols, const float* __restrict__ x, const float* __restrict__ target,
+                                                              float* y, float* __restrict__ loss, float scale)
+{
+	__shared__ float part[4];
+	__shared__ unsigned arrived;
+	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+	const uint64_t row = (uint64_t)blockIdx.x * 4 + wave;
+	if (row < rows) {
+		const float* xr = x + row * cols;
+		float m = -INFINITY;
+		for (uint64_t c = lane; c < cols; c += 64) m = fmaxf(m, xr[c]);
+		m = wave_max(m);
+		float s = 0.0f;
+		for (uint64_t c = lane; c < cols; c += 64) s += expf(xr[c] - m);
+		s = wave_sum(s);
+		for (uint64_t c = lane; c < cols; c += 64) y[row * cols + c] = logf(expf(xr[c] - m) / s);
+	}
+	__threadfence();
+	__syncthreads();
+	if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&g_loss_arrivals, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+	__syncthreads();
+	if (arrived != gridDim.x - 1) return;
+	// the last workgroup: every row is in memory
+	const uint64_t len = rows * cols;
+	float s = 0.0f;
+	// nll_loss_kernel's order: 1024 strided partial sums, folded per wavefront, sixteen wavefront sums added in order.
+	// This workgroup has 256 threads: thread t plays the threads t, t + 256, t + 512, t + 768 of that kernel in turn.
+	float tot = 0.0f;
+	for (int quarter = 0; quarter < 4; quarter++) {
+		s = 0.0f;
+		for (uint64_t i = (uint64_t)quarter * 256 + threadIdx.x; i < len; i += 1024)
+			s += __hip_atomic_load(y + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * target[i];
+		s = wave_sum(s);
+		__syncthreads();
+		if (lane == 0) part[wave] = s;
+		__syncthreads();
+		if (threadIdx.x == 0) {
+#pragma unroll
+			for (int w = 0; w < 4; w++) tot += part[w];
+		}
+	}
+	if (threadIdx.x == 0) {
+		*loss = tot * scale;
+		__hip_atomic_store(&g_loss_arrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+}
+
+// nll_backward (dy = alpha * target, gpu_mul) and the backward of log_softmax in one pass; the same operations per
+// element as scale_kernel followed by log_softmax_backward_kernel.
+__global__ __launch_bounds__(256) void nll_log_softmax_backward_kernel(uint64_t rows, uint64_t cols, const float* __restrict__ y,
+                                                                       const float* __restrict__ target, float alpha, float* __restrict__ dx)
+{
+	const int lane = threadIdx.x & 63;
+	const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= rows) return;
+	float s = 0.0f;
+	for (uint64_t c = lane; c < cols; c += 64) s += alpha * target[row * cols + c];
+	s = wave_sum(s);
+	for (uint64_t c = lane; c < cols; c += 64) dx[row * cols + c] = alpha * target[row * cols + c] - expf(y[row * cols + c]) * s;
+}
+
 // SGDOptimizer::step for one tensor (l-ten/optimizer.cpp:52-57; gpu_sgd_step, l-ten/math_fns.h:186): the gradient
 // buffer receives the decayed gradient, as in l-ten.  Every product and sum rounded on its own, in l-ten's order.
 __global__ __launch_bounds__(256) void sgd_step_kernel(float* __restrict__ w, float* __restrict__ g, float* __restrict__ v, uint64_t n, float mo,
@@ -265,6 +333,26 @@ int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, 
 	LTEN_HIP_REQUIRE(loss != nullptr && batches > 0, "nll_loss: null loss pointer or zero batch");
 	LTEN_HIP_REQUIRE(len == 0 || (input && target), "nll_loss: null pointer");
 	nll_loss_kernel<<<dim3(1), dim3(1024), 0, stream()>>>(input, target, loss, len, -1.0f / (float)batches);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_log_softmax_nll_loss_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float* y, float* loss)
+{
+	LTEN_HIP_REQUIRE(loss != nullptr && rows > 0, "log_softmax_nll_loss: null loss pointer or zero batch");
+	LTEN_HIP_REQUIRE(cols == 0 || (x && target && y), "log_softmax_nll_loss: null pointer");
+	if (cols == 0) return lten_hip_nll_loss_f32(y, target, loss, 0, rows);
+	set_kernel_name("log_softmax_nll");
+	log_softmax_nll_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, x, target, y, loss, -1.0f / (float)rows);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_nll_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float* y, const float* target, float alpha, float* dx)
+{
+	if (rows == 0 || cols == 0) return 0;
+	LTEN_HIP_REQUIRE(y && target && dx, "nll_log_softmax_backward: null pointer");
+	nll_log_softmax_backward_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, y, target, alpha, dx);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
 		float out = p.alpha * v;
 		if (p.beta != 0.0f) out += p.beta * *c;  // beta == 0 overwrites: NaN/Inf in C must not survive
 		if (p.bias) out += p.bias[n];
-		*c = out;
+		sgemm_store(p, c, out);
 	});
 }
 
@@ -144,7 +144,7 @@ __device__ __forceinline__ void sgemm_direct_body(const SProblem& p, int block, 
 		float out = p.alpha * sum;
 		if (p.beta != 0.0f) out += p.beta * *c;
 		if (p.bias) out += p.bias[n0 + col];
-		*c = out;
+		sgemm_store(p, c, out);
 	}
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(&part[0][0], asum, p.rowsum, m0, p.M);
 }
@@ -275,7 +275,7 @@ __device__ __forceinline__ void sgemm_staged_body(const SProblem& p, int block, 
 		float out = p.alpha * sum;
 		if (p.beta != 0.0f) out += p.beta * *c;
 		if (p.bias) out += p.bias[n0 + col];
-		*c = out;
+		sgemm_store(p, c, out);
 	}
 	if (p.rowsum != nullptr && n0 == 0) add_row_sums<WAVES>(lds, asum, p.rowsum, m0, p.M);
 }
@@ -300,6 +300,76 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_kernel(SProblem px
 	else sgemm_direct_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, part);
 }
 
+// C = A^T B (TN) with a short K (the weight gradient dW = dY^T X at a small batch): a 32x32 output tile per wavefront
+// over the whole K, operands straight from global memory in the MFMA lane layout (both are read along their contiguous
+// dimension: two 128-byte rows per wave-wide load), the loads of eight groups of 8 k in flight together, no LDS, no
+// barrier — cutting a K of 128 over eight wavefronts leaves each with two groups and a workgroup with more exchange than
+// arithmetic.  `tile` counts 32x32 tiles row-major.  The wavefronts of the first column tile add the row sums of op(A)
+// into p.rowsum.
+__device__ __forceinline__ void sgemm_tn_wave_tile(const SProblem& p, int tile)
+{
+	const int lane = threadIdx.x & 63, lrow = lane & 31, g = lane >> 5;
+	const int tiles_n = (p.N + 31) / 32;
+	const int m0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+	if (m0 >= p.M) return;
+	const int m = m0 + lrow, n = n0 + lrow;
+	const bool mok = m < p.M, nok = n < p.N;
+	const float* a_col = p.A + (mok ? m : 0);
+	const float* b_col = p.B + (nok ? n : 0);
+	v16f acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	float asum = 0.0f;
+	const int groups = (p.K + 7) / 8;
+	constexpr int U = 8;
+	for (int g0 = 0; g0 < groups; g0 += U) {
+		float a[U][4], b[U][4];
+#pragma unroll
+		for (int u = 0; u < U; u++) {
+			const int k = (g0 + u) * 8 + g * 4;
+#pragma unroll
+			for (int t = 0; t < 4; t++) {
+				// rows past K are not read; columns past M or N read column 0 and are never stored
+				const int kk = k + t < p.K ? k + t : 0;
+				const float av = a_col[(int64_t)kk * p.lda], bv = b_col[(int64_t)kk * p.ldb];
+				a[u][t] = (k + t < p.K && mok) ? av : 0.0f;
+				b[u][t] = (k + t < p.K && nok) ? bv : 0.0f;
+			}
+		}
+#pragma unroll
+		for (int u = 0; u < U; u++) {
+			if (g0 + u >= groups) break;
+			asum += (a[u][0] + a[u][1]) + (a[u][2] + a[u][3]);
+#pragma unroll
+			for (int t = 0; t < 4; t++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t], b[u][t], acc, 0, 0, 0);
+		}
+	}
+	// register 4q + e of lane (lrow, g): row 8q + 4g + e, column lrow
+	if (nok) {
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int row = m0 + (r >> 2) * 8 + g * 4 + (r & 3);
+			if (row >= p.M) continue;
+			float* c = p.C + (int64_t)row * p.ldc + n;
+			float out = p.alpha * acc[r];
+			if (p.beta != 0.0f) out += p.beta * *c;
+			sgemm_store(p, c, out);
+		}
+	}
+	if (p.rowsum != nullptr && n0 == 0) {
+		const float s = asum + __shfl_xor(asum, 32, 64);
+		if (g == 0 && mok) p.rowsum[m] += s;
+	}
+}
+
+// The same pair with the weight gradient on sgemm_tn_wave_tile: eight of its tiles per workgroup.
+__global__ __launch_bounds__(512) void sgemm_fc_backward_pair_shortk_kernel(SProblem px, SProblem pw, int blocks_x)
+{
+	__shared__ float part[8][32 * 32];
+	if ((int)blockIdx.x < blocks_x) sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, part);
+	else sgemm_tn_wave_tile(pw, ((int)blockIdx.x - blocks_x) * 8 + (int)(threadIdx.x >> 6));
+}
+
 // FullyConnected forward at small batch sizes: C[M x N] = A[M x K] B[N x K]^T with M <= 32, a stream over the
 // weights B.  The 32x32 kernels above give such a product N / 32 workgroups; here a workgroup takes 16 columns
 // (N / 16 workgroups: 256 for a 4096-wide layer) on 16x16x4 MFMA tiles, MB = 1 or 2 blocks of 16 activation rows.
@@ -320,6 +390,7 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 	const int r16 = lane & 15, q4 = lane >> 4;
 	const int r8 = lane >> 3, c4 = (lane & 7) * 4;
 	const int n0 = blockIdx.x * 16;
+	const int mrow0 = blockIdx.y * (MB * 16);  // blockIdx.y: which block of MB * 16 activation rows
 	float* sA = lds + wave * (A_SLAB + B_SLAB);
 	float* sB = sA + A_SLAB;
 
@@ -335,7 +406,7 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 		const int k = batch * 32 + c4;
 #pragma unroll
 		for (int i = 0; i < 2 * MB; i++) {
-			const int m = 8 * i + r8;
+			const int m = mrow0 + 8 * i + r8;
 			v.a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 			if (m < p.M && k < p.K) v.a[i] = *reinterpret_cast<const float4*>(p.A + (int64_t)m * p.lda + k);
 		}
@@ -392,7 +463,7 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 		for (int e = 0; e < 4; e++) lds[wave * (MB * 256) + (16 * b + 4 * q4 + e) * 16 + r16] = acc[b][e];
 	__syncthreads();
 	for (int idx = tid; idx < MB * 256; idx += WAVES * 64) {
-		const int row = idx >> 4, col = idx & 15;
+		const int row = mrow0 + (idx >> 4), col = idx & 15;
 		if (row >= p.M || n0 + col >= p.N) continue;
 		float sum = 0.0f;
 #pragma unroll
@@ -401,7 +472,7 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 		float out = p.alpha * sum;
 		if (p.beta != 0.0f) out += p.beta * *c;
 		if (p.bias) out += p.bias[n0 + col];
-		*c = out;
+		sgemm_store(p, c, out);
 	}
 }
 
@@ -514,9 +585,11 @@ static int launch_sgemm(const SProblem& p, int tA, int tB, uint64_t batch, const
 
 int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
               int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
-              int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done)
+              int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done, float* relu_out = nullptr,
+              const float* relu_in = nullptr, bool* relu_done = nullptr)
 {
 	if (rowsum_done) *rowsum_done = false;
+	if (relu_done) *relu_done = false;
 	if (M == 0 || N == 0 || batch == 0) return 0;
 	LTEN_HIP_REQUIRE(C != nullptr, "sgemm: C is null");
 	LTEN_HIP_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "sgemm: null operand");
@@ -532,7 +605,9 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		return 0;
 	}
 	SProblem p;
-	p.A = A; p.B = B; p.C = C; p.bias = bias; p.rowsum = nullptr;
+	p.A = A; p.B = B; p.C = C; p.bias = bias; p.rowsum = nullptr; p.relu_out = nullptr; p.relu_in = nullptr;
+	// the relu pieces ride on the kernels whose epilogue goes through sgemm_store; elsewhere the caller launches them
+	const bool want_relu = relu_done != nullptr && batch == 1 && (relu_out != nullptr || relu_in != nullptr);
 	p.lda = (int64_t)lda; p.ldb = (int64_t)ldb; p.ldc = (int64_t)ldc;
 	p.stride_a = stride_a; p.stride_b = stride_b; p.stride_c = stride_c;
 	p.M = (int)M; p.N = (int)N; p.K = (int)K;
@@ -550,10 +625,15 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}
-	if (force == 0 && !tA && tB && M <= 32 && N >= 512 && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p)) {
-		// a weight stream: 16 columns per workgroup
+	// FullyConnected forward with few activation rows: 16 columns of the weights per workgroup, and for more than 32
+	// rows one workgroup per block of 32 rows as well (the weights then come from the L2 for all but the first), while
+	// that gives at most a few workgroups per CU: 128 rows against a 1024-wide layer are 256 tiles of 32 x 16 where the
+	// 32 x 32 tiles of the general small-GEMM kernels would occupy half of the CUs.
+	if (force == 0 && !tA && tB && N >= 512 && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
+	    (M <= 32 || ceil_div(M, 32) * ceil_div(N, 16) <= 1024)) {
 		set_kernel_name(M <= 16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
-		const dim3 grid((unsigned)ceil_div(N, 16));
+		if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
+		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(M <= 16 ? 1 : ceil_div(M, 32)));
 		if (M <= 16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
 		else sgemm_skinny_nt_kernel<2><<<grid, dim3(512), 0, stream()>>>(p);
 		LTEN_HIP_LAUNCH_CHECK();
@@ -589,6 +669,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		if (tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20))) choice = 4;
 		else choice = tiles128 >= 128 ? 1 : 2;
 	}
+	if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
 	switch (choice) {
 	case 1: return launch_sgemm<128, 128, 16, 2, 2>(p, tA, tB, batch, "sgemm_128x128x16");
 	case 2: return launch_sgemm<64, 64, 32, 2, 2>(p, tA, tB, batch, "sgemm_64x64x32");
@@ -638,30 +719,56 @@ int lten_hip_fc_forward_f32(uint64_t M, uint64_t in, uint64_t out, const float* 
 	return sgemm_run(0, 1, M, out, in, 1.0f, X, in, 0, W, in, 0, 0.0f, Y, out, 0, 1, bias, nullptr, nullptr);
 }
 
-int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
-                             float* dX, float* dW, float* db)
+int lten_hip_fc_forward_relu_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* bias,
+                                 float* Y, float* Y_relu)
+{
+	LTEN_HIP_REQUIRE(Y_relu != nullptr || M * out == 0, "fc_forward_relu: Y_relu is null");
+	bool relu_done = false;
+	int rc = sgemm_run(0, 1, M, out, in, 1.0f, X, in, 0, W, in, 0, 0.0f, Y, out, 0, 1, bias, nullptr, nullptr, Y_relu, nullptr, &relu_done);
+	// kernels without the fused store (the large direct-to-LDS tiles, the degenerate shapes): relu as a launch of its own
+	if (!rc && !relu_done) rc = lten_hip_relu_f32(Y_relu, Y, M * out);
+	return rc;
+}
+
+}  // extern "C"
+
+static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
+                       const float* relu_input, float* dX, float* dW, float* db)
 {
 	int rc = 0;
 	// Both products wanted, both of the kind the 32x32 kernels take (few tiles, or 16-byte loads possible; not one of
 	// the degenerate shapes with a kernel of their own, not large enough for the direct-to-LDS tiles) and the batch
 	// small enough that the weight-gradient product would not take the whole-line loads: one launch computes the two.
-	if (dX && dW && get_option(OPT_SGEMM_TILE) == 0 && M > 1 && M < 512 && out > 1 && out <= 2048 && in > 0) {
+	// option "sgemm_tile" 7: the paired launch with the weight gradient's K cut over the wavefronts whatever the batch
+	const int pair_opt = get_option(OPT_SGEMM_TILE);
+	if (dX && dW && (pair_opt == 0 || pair_opt == 7) && M > 1 && M < 512 && out > 1 && out <= 2048 && in > 0) {
 		SProblem px = {}, pw = {};
 		px.A = dY; px.B = W; px.C = dX; px.lda = (int64_t)out; px.ldb = (int64_t)in; px.ldc = (int64_t)in;
 		px.M = (int)M; px.N = (int)in; px.K = (int)out; px.alpha = 1.0f; px.beta = 0.0f;
+		px.relu_in = relu_input;
 		pw.A = dY; pw.B = X; pw.C = dW; pw.lda = (int64_t)out; pw.ldb = (int64_t)in; pw.ldc = (int64_t)in;
 		pw.M = (int)out; pw.N = (int)in; pw.K = (int)M; pw.alpha = 1.0f; pw.beta = 0.0f;
 		pw.rowsum = db;
 		const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
 		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
-			set_kernel_name("sgemm_fc_backward_pair_32x32_w8");
-			sgemm_fc_backward_pair_kernel<<<dim3((unsigned)(blocks_x + blocks_w)), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
+			if (M <= 256 && blocks_w >= 256 && pair_opt == 0) {  // a short reduction and many tiles for dW: whole-K tiles per wavefront
+				set_kernel_name("sgemm_fc_backward_pair_32x32_shortk");
+				sgemm_fc_backward_pair_shortk_kernel<<<dim3((unsigned)(blocks_x + ceil_div(blocks_w, 8))), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
+			} else {
+				set_kernel_name("sgemm_fc_backward_pair_32x32_w8");
+				sgemm_fc_backward_pair_kernel<<<dim3((unsigned)(blocks_x + blocks_w)), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
+			}
 			LTEN_HIP_LAUNCH_CHECK();
 			return 0;
 		}
 	}
 	// l-ten/backprop.cpp:2228  dX[M x in] = dY[M x out] W[out x in]
-	if (dX) rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr, nullptr, nullptr);
+	if (dX) {
+		bool relu_done = false;
+		rc = sgemm_run(0, 0, M, in, out, 1.0f, dY, out, 0, W, in, 0, 0.0f, dX, in, 0, 1, nullptr, nullptr, nullptr, nullptr, relu_input,
+		               relu_input ? &relu_done : nullptr);
+		if (!rc && relu_input && !relu_done) rc = lten_hip_relu_backward_f32(dX, dX, relu_input, M * in);
+	}
 	// :2252  dW[out x in] = dY[M x out]^T X[M x in].  The rows of dY^T summed over the batch are the bias gradient
 	// of :2267, so a kernel that can do it adds them into db on the way.
 	bool db_done = false;
@@ -678,6 +785,21 @@ int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float*
 		LTEN_HIP_LAUNCH_CHECK();
 	}
 	return rc;
+}
+
+extern "C" {
+
+int lten_hip_fc_backward_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
+                             float* dX, float* dW, float* db)
+{
+	return fc_backward(M, in, out, X, W, dY, nullptr, dX, dW, db);
+}
+
+int lten_hip_fc_backward_relu_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* dY,
+                                  const float* relu_input, float* dX, float* dW, float* db)
+{
+	LTEN_HIP_REQUIRE(relu_input != nullptr || dX == nullptr || M * in == 0, "fc_backward_relu: relu_input is null");
+	return fc_backward(M, in, out, X, W, dY, relu_input, dX, dW, db);
 }
 
 }  // extern "C"

@@ -15,11 +15,22 @@ struct SProblem {
 	const float* bias;  // optional, added per output column n (FullyConnected bias), or null
 	float* rowsum;      // optional: rowsum[m] += sum_k op(A)[m][k] (the FullyConnected bias gradient inside the
 	                    // weight-gradient product); only the 32x32 kernels do it, for a single problem
+	// Optional relu pieces of a training step folded into the store (single problems only; same indexing as C):
+	float* relu_out;       // also receives max(C, 0): the activation next to the pre-activation (l-ten/layers.cpp:9-67)
+	const float* relu_in;  // C = relu_in > 0 ? C : 0: relu_backward on the data gradient (l-ten/backprop.cpp:2282-2327)
 	int64_t lda, ldb, ldc;
 	int64_t stride_a, stride_b, stride_c;  // per blockIdx.z
 	int M, N, K;
 	float alpha, beta;
 };
+
+// The last step of every epilogue that supports the relu pieces: c points into p.C (batch index 0).
+__device__ __forceinline__ void sgemm_store(const SProblem& p, float* c, float out)
+{
+	if (p.relu_in != nullptr && !(p.relu_in[c - p.C] > 0)) out = 0.0f;
+	*c = out;
+	if (p.relu_out != nullptr) p.relu_out[c - p.C] = out > 0 ? out : 0.0f;
+}
 
 // Direct-to-LDS tiles for large aligned problems; returns -1 when the problem does not fit them.
 int sgemm_fast_dispatch(const SProblem& p, int tA, int tB, uint64_t batch, int variant);

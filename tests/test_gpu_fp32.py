@@ -85,15 +85,15 @@ def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
     order: bitwise equal results run after run; all layouts, ragged M / N / K, beta, batches."""
     rng = np.random.default_rng(3)
     if True:
-        M, N, K = 128, 1024, 1024
+        M, N, K = 128, 1024, 1024   # the data-gradient product of a 1024-wide layer at batch 128 (NN)
         A = rng.standard_normal((M, K)).astype(np.float32)
-        B = rng.standard_normal((N, K)).astype(np.float32)
+        B = rng.standard_normal((K, N)).astype(np.float32)
         z = np.zeros((M, N), np.float32)
-        first = gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N, tile=tile)
+        first = gpu_sgemm(gpu, 0, 0, M, N, K, 1.0, A, K, B, N, 0.0, z, N, tile=tile)
         assert gpu.last_kernel().startswith(name)
         for _ in range(5):
-            assert np.array_equal(gpu_sgemm(gpu, 0, 1, M, N, K, 1.0, A, K, B, K, 0.0, z, N, tile=tile), first)
-        want = A.astype(np.float64) @ B.astype(np.float64).T
+            assert np.array_equal(gpu_sgemm(gpu, 0, 0, M, N, K, 1.0, A, K, B, N, 0.0, z, N, tile=tile), first)
+        want = A.astype(np.float64) @ B.astype(np.float64)
         assert rel_err(first, want) < TOL
         for (tA, tB, m, n, k) in [(0, 0, 70, 100, 532), (0, 1, 33, 31, 788), (1, 0, 100, 36, 660), (1, 1, 20, 65, 596)]:
             a = rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32)
@@ -172,8 +172,10 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
 @pytest.mark.parametrize("M,fin,fout,kernels", [
     (128, 200, 75, ("sgemm_fc_backward_pair_32x32_w8",)),            # both products in one launch, bias gradient inside it
     (37, 33, 10, ("sgemm_fc_backward_pair_32x32_w8",)),              # ragged in every dimension
+    (100, 530, 490, ("sgemm_fc_backward_pair_32x32_shortk",)),       # many weight-gradient tiles, short K: a whole-K tile per wavefront, ragged
+    (300, 600, 500, ("sgemm_fc_backward_pair_32x32_w8",)),           # batch above 256: the weight gradient cuts K over the wavefronts
     (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: two launches, dW with whole-line loads, ragged K
-    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_w8",)),          # config 2, layer 1
+    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_shortk",)),      # config 2, layer 1
     (511, 64, 2048, ("sgemm_fc_backward_pair_32x32_w8",)),           # the largest batch and width the paired launch takes
     (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel

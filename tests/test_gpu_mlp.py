@@ -10,8 +10,11 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-4
 
 
-def gpu_mlp_step(gpu, X, Ws, bs, T):
-    """The step through the C ABI, every intermediate resident on the device.  Returns what ob.mlp_step returns."""
+def gpu_mlp_step(gpu, X, Ws, bs, T, fused=False):
+    """The step through the C ABI, every intermediate resident on the device.  Returns what ob.mlp_step returns.
+    fused: the entry points that fold relu, relu_backward, the loss and nll_backward into their neighbours."""
+    if fused:
+        return gpu_mlp_step_fused(gpu, X, Ws, bs, T)
     D, l = gpu.DeviceBuffer, gpu.lib()
     B, layers = X.shape[0], len(Ws)
     sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
@@ -41,6 +44,35 @@ def gpu_mlp_step(gpu, X, Ws, bs, T):
                 pre=[pre[i + 1].numpy(np.float32, (B, sizes[i + 1])) for i in range(layers)],
                 dW=[gW[i].numpy(np.float32, Ws[i].shape) for i in range(layers)],
                 db=[gb[i].numpy(np.float32, bs[i].shape) for i in range(layers)], dX=tmp[0].numpy(np.float32, X.shape))
+
+
+def gpu_mlp_step_fused(gpu, X, Ws, bs, T):
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    B, layers = X.shape[0], len(Ws)
+    sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
+    dW_, db_ = [D.from_numpy(w) for w in Ws], [D.from_numpy(b) for b in bs]
+    pre = [None] + [D(4 * B * n) for n in sizes[1:]]
+    act = [D.from_numpy(X)] + [D(4 * B * n) for n in sizes[1:-1]] + [None]
+    for i in range(layers):
+        if i + 1 < layers:
+            gpu.check(l.lten_hip_fc_forward_relu_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr, act[i + 1].ptr))
+        else:
+            gpu.check(l.lten_hip_fc_forward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr))
+    dT, logp, loss = D.from_numpy(T), D(4 * B * sizes[-1]), D(4)
+    gpu.check(l.lten_hip_log_softmax_nll_loss_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, logp.ptr, loss.ptr))
+    g = [D(4 * B * n) for n in sizes]
+    gpu.check(l.lten_hip_nll_log_softmax_backward_f32(B, sizes[-1], logp.ptr, dT.ptr, -1.0 / B, g[layers].ptr))
+    gW, gb = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
+    for i in range(layers - 1, -1, -1):
+        if i > 0:
+            gpu.check(l.lten_hip_fc_backward_relu_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, g[i + 1].ptr, pre[i].ptr,
+                                                      g[i].ptr, gW[i].ptr, gb[i].ptr))
+        else:
+            gpu.check(l.lten_hip_fc_backward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, g[i + 1].ptr, g[i].ptr, gW[i].ptr, gb[i].ptr))
+    return dict(loss=float(loss.numpy(np.float32, (1,))[0]), logp=logp.numpy(np.float32, T.shape),
+                pre=[pre[i + 1].numpy(np.float32, (B, sizes[i + 1])) for i in range(layers)],
+                dW=[gW[i].numpy(np.float32, Ws[i].shape) for i in range(layers)],
+                db=[gb[i].numpy(np.float32, bs[i].shape) for i in range(layers)], dX=g[0].numpy(np.float32, X.shape))
 
 
 def check_step(got, want, tag):
@@ -110,6 +142,67 @@ def test_cfg2_training_step_full_size(gpu, ob, wl):
     errs = [rel_err(got["dW"][i], ref["dW"][i]) for i in range(3)]
     print(f"  loss {got['loss']:.6f} (oracle {want['loss']:.6f}); relu decisions that differ from fp64: {flips}; "
           f"dW max rel err {max(errs):.2e}")
+    # the route with the fused entry points (8 launches instead of 14) computes the same values bit for bit
+    fused = gpu_mlp_step(gpu, X, Ws, bs, T, fused=True)
+    assert fused["loss"] == got["loss"]
+    for key in ("logp", "dX"):
+        assert np.array_equal(fused[key], got[key]), key
+    for key in ("pre", "dW", "db"):
+        for a, b in zip(fused[key], got[key]):
+            assert np.array_equal(a, b), key
+
+
+@pytest.mark.parametrize("shape", [(128, 784, 1024), (7, 33, 50), (20, 2048, 640), (600, 96, 200), (300, 2048, 4096), (1, 64, 32)])
+def test_fused_fc_relu_entry_points_match_the_unfused_calls(gpu, shape):
+    """lten_hip_fc_forward_relu_f32 / lten_hip_fc_backward_relu_f32 against fc_forward + relu / fc_backward + relu_backward
+    on shapes that reach every GEMM family (32x32 tiles, weight stream, LDS tiles, the large direct-to-LDS tiles, M = 1):
+    bit-identical, whether the relu rides on the store or runs as a launch of its own."""
+    M, fin, fout = shape
+    rng = np.random.default_rng(M + fin + fout)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    X = rng.standard_normal((M, fin)).astype(np.float32)
+    W = (rng.standard_normal((fout, fin)) * 0.05).astype(np.float32)
+    b = rng.standard_normal(fout).astype(np.float32)
+    dY = rng.standard_normal((M, fout)).astype(np.float32)
+    Rin = rng.standard_normal((M, fin)).astype(np.float32)
+    Rin[::3] = 0.0
+    dX_, dW_, db_, ddY, dR = D.from_numpy(X), D.from_numpy(W), D.from_numpy(b), D.from_numpy(dY), D.from_numpy(Rin)
+    y0, a0, y1, a1 = (D(4 * M * fout) for _ in range(4))
+    gpu.check(l.lten_hip_fc_forward_f32(M, fin, fout, dX_.ptr, dW_.ptr, db_.ptr, y0.ptr))
+    gpu.check(l.lten_hip_relu_f32(a0.ptr, y0.ptr, M * fout))
+    gpu.check(l.lten_hip_fc_forward_relu_f32(M, fin, fout, dX_.ptr, dW_.ptr, db_.ptr, y1.ptr, a1.ptr))
+    k_fwd = gpu.last_kernel()
+    assert np.array_equal(y0.numpy(np.float32, (M, fout)), y1.numpy(np.float32, (M, fout)))
+    assert np.array_equal(a0.numpy(np.float32, (M, fout)), a1.numpy(np.float32, (M, fout)))
+    t0, g0, g1 = (D(4 * M * fin) for _ in range(3))
+    w0, w1 = D(W.nbytes), D(W.nbytes)
+    b0, b1 = D(b.nbytes, zero=True), D(b.nbytes, zero=True)
+    gpu.check(l.lten_hip_fc_backward_f32(M, fin, fout, dX_.ptr, dW_.ptr, ddY.ptr, t0.ptr, w0.ptr, b0.ptr))
+    gpu.check(l.lten_hip_relu_backward_f32(g0.ptr, t0.ptr, dR.ptr, M * fin))
+    gpu.check(l.lten_hip_fc_backward_relu_f32(M, fin, fout, dX_.ptr, dW_.ptr, ddY.ptr, dR.ptr, g1.ptr, w1.ptr, b1.ptr))
+    print(f"  {shape}: forward via {k_fwd}, backward via {gpu.last_kernel()}", flush=True)
+    assert np.array_equal(g0.numpy(np.float32, (M, fin)), g1.numpy(np.float32, (M, fin)))
+    assert np.array_equal(w0.numpy(np.float32, W.shape), w1.numpy(np.float32, W.shape))
+    assert np.array_equal(b0.numpy(np.float32, b.shape), b1.numpy(np.float32, b.shape))
+
+
+def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
+    rng = np.random.default_rng(11)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    for rows, cols in ((1, 1), (128, 10), (37, 400), (16, 1024), (5, 4097)):
+        x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+        t = np.eye(cols, dtype=np.float32)[rng.integers(0, cols, rows)]
+        dx, dt = D.from_numpy(x), D.from_numpy(t)
+        y0, y1, l0, l1, s0, g0, g1 = D(x.nbytes), D(x.nbytes), D(4), D(4), D(x.nbytes), D(x.nbytes), D(x.nbytes)
+        gpu.check(l.lten_hip_log_softmax_f32(rows, cols, dx.ptr, y0.ptr))
+        gpu.check(l.lten_hip_nll_loss_f32(y0.ptr, dt.ptr, l0.ptr, rows * cols, rows))
+        gpu.check(l.lten_hip_log_softmax_nll_loss_f32(rows, cols, dx.ptr, dt.ptr, y1.ptr, l1.ptr))
+        assert np.array_equal(y0.numpy(np.float32, x.shape), y1.numpy(np.float32, x.shape)), (rows, cols)
+        assert l0.numpy(np.float32, (1,))[0] == l1.numpy(np.float32, (1,))[0], (rows, cols)
+        gpu.check(l.lten_hip_scale_f32(rows * cols, -1.0 / rows, dt.ptr, s0.ptr))
+        gpu.check(l.lten_hip_log_softmax_backward_f32(rows, cols, y0.ptr, s0.ptr, g0.ptr))
+        gpu.check(l.lten_hip_nll_log_softmax_backward_f32(rows, cols, y0.ptr, dt.ptr, -1.0 / rows, g1.ptr))
+        assert np.array_equal(g0.numpy(np.float32, x.shape), g1.numpy(np.float32, x.shape)), (rows, cols)
 
 
 def test_elementwise_kernels(gpu, ob):
