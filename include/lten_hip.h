@@ -240,12 +240,16 @@ int lten_hip_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float*
 /* gpu_nll (l-ten/math_fns.h:170; l-ten/layers.cpp:212-273): *loss = (sum_i input[i] * target[i]) * (-1 / batches). */
 int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, uint64_t len, uint64_t batches);
 
-/* lten_hip_log_softmax_f32 followed by lten_hip_nll_loss_f32 (batches = rows) as one launch (calls that overlap on
- * one GPU would share its arrival counter: one stream at a time), and lten_hip_scale_f32(alpha, target) followed by lten_hip_log_softmax_backward_f32 as one:
- * dx = alpha * target - exp(y) * sum_j alpha * target_j, alpha = -top / rows for l-ten's nll_backward
- * (l-ten/backprop.cpp:3975-4040).  Same values as the separate calls, bit for bit. */
+/* Fewer launches around the loss, same values bit for bit: lten_hip_log_softmax_nll_loss_f32 = lten_hip_log_softmax_f32
+ * followed by lten_hip_nll_loss_f32 (batches = rows); lten_hip_nll_log_softmax_backward_f32 = lten_hip_scale_f32(alpha,
+ * target) followed by lten_hip_log_softmax_backward_f32, i.e. dx = alpha * target - exp(y) * sum_j alpha * target_j with
+ * alpha = -top / rows for l-ten's nll_backward (l-ten/backprop.cpp:3975-4040); lten_hip_log_softmax_nll_loss_grad_f32 =
+ * both of them.  The first and the third are one launch for up to 1024 rows of up to 16 columns (a classifier's
+ * logits) and the separate launches otherwise. */
 int lten_hip_log_softmax_nll_loss_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float* y, float* loss);
 int lten_hip_nll_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const float* y, const float* target, float alpha, float* dx);
+int lten_hip_log_softmax_nll_loss_grad_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float alpha, float* y,
+                                           float* loss, float* dx);
 
 /* gpu_sgd_step (l-ten/math_fns.h:186; SGDOptimizer::step, l-ten/optimizer.cpp:26-84) for one parameter tensor:
  * grad = wd * w + grad (stored, as in l-ten), velocity = velocity * mo + (1 - mo) * grad, w = w - velocity * lr. */

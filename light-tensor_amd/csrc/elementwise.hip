@@ -98,57 +98,77 @@ __global__ __launch_bounds__(1024) void nll_loss_kernel(const float* __restrict_
 	}
 }
 
-// log_softmax and nll_loss in one launch: the rows are spread over workgroups as in log_softmax_kernel (a wavefront per
-// row), every workgroup counts itself in when its rows are written, and the one that arrives last sums the loss over the
-// whole array in exactly the order nll_loss_kernel uses (reading the log-probabilities past the per-CU cache, since
-// other CUs wrote them) — both results are bit-identical to the two separate launches.  The counter lives in a static
-// device word and is zero again when the kernel ends.
-static __device__ unsigned g_loss_arrivals;
-
-__global__ __launch_bounds__(256) void log_softmax_nll_kernel(uint64_t rows, uint64_t cols, const float* __restrict__ x, const float* __restrict__ target,
-                                                              float* y, float* __restrict__ loss, float scale)
+// log_softmax, nll_loss and (GRAD) the gradient of the loss with respect to the logits for a small batch of narrow
+// rows (rows <= 1024, cols <= 16) in one launch of one workgroup: a thread per row, the row in registers.  The separate
+// kernels fold a row across a wavefront by lane exchanges; with the row in one thread the same sums are taken in the
+// same order (pairs 8 apart, then 4, 2, 1: what the exchange tree leaves in lane 0 when all lanes past the row hold
+// zeros), so the log-probabilities and the gradient are bit-identical to theirs, and the loss is summed from an LDS copy
+// of the log-probabilities exactly as nll_loss_kernel sums it from memory.  One workgroup because a hand-over between
+// workgroups (release fence, arrival counter) costs more on this part than the whole computation.
+__device__ __forceinline__ float tree_sum16(float (&v)[16])
 {
-	__shared__ float part[4];
-	__shared__ unsigned arrived;
-	const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-	const uint64_t row = (uint64_t)blockIdx.x * 4 + wave;
-	if (row < rows) {
-		const float* xr = x + row * cols;
-		float m = -INFINITY;
-		for (uint64_t c = lane; c < cols; c += 64) m = fmaxf(m, xr[c]);
-		m = wave_max(m);
-		float s = 0.0f;
-		for (uint64_t c = lane; c < cols; c += 64) s += expf(xr[c] - m);
-		s = wave_sum(s);
-		for (uint64_t c = lane; c < cols; c += 64) y[row * cols + c] = logf(expf(xr[c] - m) / s);
-	}
-	__threadfence();
-	__syncthreads();
-	if (threadIdx.x == 0) arrived = __hip_atomic_fetch_add(&g_loss_arrivals, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-	__syncthreads();
-	if (arrived != gridDim.x - 1) return;
-	// the last workgroup: every row is in memory
-	const uint64_t len = rows * cols;
-	float s = 0.0f;
-	// nll_loss_kernel's order: 1024 strided partial sums, folded per wavefront, sixteen wavefront sums added in order.
-	// This workgroup has 256 threads: thread t plays the threads t, t + 256, t + 512, t + 768 of that kernel in turn.
-	float tot = 0.0f;
-	for (int quarter = 0; quarter < 4; quarter++) {
-		s = 0.0f;
-		for (uint64_t i = (uint64_t)quarter * 256 + threadIdx.x; i < len; i += 1024)
-			s += __hip_atomic_load(y + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * target[i];
-		s = wave_sum(s);
-		__syncthreads();
-		if (lane == 0) part[wave] = s;
-		__syncthreads();
-		if (threadIdx.x == 0) {
+	float t[16];
 #pragma unroll
-			for (int w = 0; w < 4; w++) tot += part[w];
+	for (int i = 0; i < 16; i++) t[i] = v[i];
+#pragma unroll
+	for (int o = 8; o > 0; o >>= 1)
+#pragma unroll
+		for (int i = 0; i < o; i++) t[i] = t[i] + t[i + o];
+	return t[0];
+}
+
+template <bool GRAD>
+__global__ __launch_bounds__(1024) void loss_rows_kernel(int rows, int cols, const float* __restrict__ x, const float* __restrict__ target, float alpha,
+                                                         float* __restrict__ y, float* __restrict__ loss, float loss_scale, float* __restrict__ dx)
+{
+	__shared__ float logp[16384];
+	__shared__ float part[16];
+	const int r = threadIdx.x;
+	if (r < rows) {
+		float xv[16], tv[16];
+#pragma unroll
+		for (int c = 0; c < 16; c++) {
+			xv[c] = c < cols ? x[r * cols + c] : -INFINITY;
+			tv[c] = (GRAD && c < cols) ? target[r * cols + c] : 0.0f;
+		}
+		float m = -INFINITY;
+#pragma unroll
+		for (int c = 0; c < 16; c++) m = fmaxf(m, xv[c]);
+		float e[16];
+#pragma unroll
+		for (int c = 0; c < 16; c++) e[c] = c < cols ? expf(xv[c] - m) : 0.0f;
+		const float s = tree_sum16(e);
+		float lp[16];
+#pragma unroll
+		for (int c = 0; c < 16; c++) {
+			lp[c] = logf(e[c] / s);
+			if (c < cols) {
+				y[r * cols + c] = lp[c];
+				logp[r * cols + c] = lp[c];
+			}
+		}
+		if (GRAD) {
+			float dy[16];
+#pragma unroll
+			for (int c = 0; c < 16; c++) dy[c] = c < cols ? alpha * tv[c] : 0.0f;
+			const float sdy = tree_sum16(dy);
+#pragma unroll
+			for (int c = 0; c < 16; c++)
+				if (c < cols) dx[r * cols + c] = dy[c] - expf(lp[c]) * sdy;
 		}
 	}
+	__syncthreads();
+	const int len = rows * cols;
+	float acc = 0.0f;
+	for (int i = threadIdx.x; i < len; i += 1024) acc += logp[i] * target[i];
+	acc = wave_sum(acc);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = acc;
+	__syncthreads();
 	if (threadIdx.x == 0) {
-		*loss = tot * scale;
-		__hip_atomic_store(&g_loss_arrivals, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		float tot = 0.0f;
+#pragma unroll
+		for (int w = 0; w < 16; w++) tot += part[w];
+		*loss = tot * loss_scale;
 	}
 }
 
@@ -337,13 +357,33 @@ int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, 
 	return 0;
 }
 
+static bool loss_rows_fits(uint64_t rows, uint64_t cols) { return rows >= 1 && rows <= 1024 && cols >= 1 && cols <= 16; }
+
 int lten_hip_log_softmax_nll_loss_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float* y, float* loss)
 {
 	LTEN_HIP_REQUIRE(loss != nullptr && rows > 0, "log_softmax_nll_loss: null loss pointer or zero batch");
 	LTEN_HIP_REQUIRE(cols == 0 || (x && target && y), "log_softmax_nll_loss: null pointer");
-	if (cols == 0) return lten_hip_nll_loss_f32(y, target, loss, 0, rows);
-	set_kernel_name("log_softmax_nll");
-	log_softmax_nll_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, x, target, y, loss, -1.0f / (float)rows);
+	if (!loss_rows_fits(rows, cols)) {  // the two launches it stands for
+		if (int rc = lten_hip_log_softmax_f32(rows, cols, x, y)) return rc;
+		return lten_hip_nll_loss_f32(y, target, loss, rows * cols, rows);
+	}
+	set_kernel_name("loss_rows");
+	loss_rows_kernel<false><<<dim3(1), dim3(1024), 0, stream()>>>((int)rows, (int)cols, x, target, 0.0f, y, loss, -1.0f / (float)rows, nullptr);
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
+int lten_hip_log_softmax_nll_loss_grad_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float alpha, float* y,
+                                           float* loss, float* dx)
+{
+	LTEN_HIP_REQUIRE(loss != nullptr && rows > 0, "log_softmax_nll_loss_grad: null loss pointer or zero batch");
+	LTEN_HIP_REQUIRE(cols == 0 || (x && target && y && dx), "log_softmax_nll_loss_grad: null pointer");
+	if (!loss_rows_fits(rows, cols)) {  // the launches it stands for
+		if (int rc = lten_hip_log_softmax_nll_loss_f32(rows, cols, x, target, y, loss)) return rc;
+		return lten_hip_nll_log_softmax_backward_f32(rows, cols, y, target, alpha, dx);
+	}
+	set_kernel_name("loss_rows_grad");
+	loss_rows_kernel<true><<<dim3(1), dim3(1024), 0, stream()>>>((int)rows, (int)cols, x, target, alpha, y, loss, -1.0f / (float)rows, dx);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

@@ -12,9 +12,10 @@ TOL = 1e-4
 
 def gpu_mlp_step(gpu, X, Ws, bs, T, fused=False):
     """The step through the C ABI, every intermediate resident on the device.  Returns what ob.mlp_step returns.
-    fused: the entry points that fold relu, relu_backward, the loss and nll_backward into their neighbours."""
+    fused: the entry points that fold relu, relu_backward, the loss and nll_backward into their neighbours; "head": the
+    loss and its gradient as one call."""
     if fused:
-        return gpu_mlp_step_fused(gpu, X, Ws, bs, T)
+        return gpu_mlp_step_fused(gpu, X, Ws, bs, T, head=fused == "head")
     D, l = gpu.DeviceBuffer, gpu.lib()
     B, layers = X.shape[0], len(Ws)
     sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
@@ -46,22 +47,25 @@ def gpu_mlp_step(gpu, X, Ws, bs, T, fused=False):
                 db=[gb[i].numpy(np.float32, bs[i].shape) for i in range(layers)], dX=tmp[0].numpy(np.float32, X.shape))
 
 
-def gpu_mlp_step_fused(gpu, X, Ws, bs, T):
+def gpu_mlp_step_fused(gpu, X, Ws, bs, T, head=False):
     D, l = gpu.DeviceBuffer, gpu.lib()
     B, layers = X.shape[0], len(Ws)
     sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
     dW_, db_ = [D.from_numpy(w) for w in Ws], [D.from_numpy(b) for b in bs]
     pre = [None] + [D(4 * B * n) for n in sizes[1:]]
     act = [D.from_numpy(X)] + [D(4 * B * n) for n in sizes[1:-1]] + [None]
+    dT, logp, loss = D.from_numpy(T), D(4 * B * sizes[-1]), D(4)
+    g = [D(4 * B * n) for n in sizes]
     for i in range(layers):
         if i + 1 < layers:
             gpu.check(l.lten_hip_fc_forward_relu_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr, act[i + 1].ptr))
         else:
             gpu.check(l.lten_hip_fc_forward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr))
-    dT, logp, loss = D.from_numpy(T), D(4 * B * sizes[-1]), D(4)
-    gpu.check(l.lten_hip_log_softmax_nll_loss_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, logp.ptr, loss.ptr))
-    g = [D(4 * B * n) for n in sizes]
-    gpu.check(l.lten_hip_nll_log_softmax_backward_f32(B, sizes[-1], logp.ptr, dT.ptr, -1.0 / B, g[layers].ptr))
+    if head:
+        gpu.check(l.lten_hip_log_softmax_nll_loss_grad_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, -1.0 / B, logp.ptr, loss.ptr, g[layers].ptr))
+    else:
+        gpu.check(l.lten_hip_log_softmax_nll_loss_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, logp.ptr, loss.ptr))
+        gpu.check(l.lten_hip_nll_log_softmax_backward_f32(B, sizes[-1], logp.ptr, dT.ptr, -1.0 / B, g[layers].ptr))
     gW, gb = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
     for i in range(layers - 1, -1, -1):
         if i > 0:
@@ -150,6 +154,14 @@ def test_cfg2_training_step_full_size(gpu, ob, wl):
     for key in ("pre", "dW", "db"):
         for a, b in zip(fused[key], got[key]):
             assert np.array_equal(a, b), key
+    # and with the loss and its gradient as one call (7 launches)
+    headed = gpu_mlp_step(gpu, X, Ws, bs, T, fused="head")
+    assert headed["loss"] == got["loss"]
+    for key in ("logp", "dX"):
+        assert np.array_equal(headed[key], got[key]), key
+    for key in ("pre", "dW", "db"):
+        for a, b in zip(headed[key], got[key]):
+            assert np.array_equal(a, b), key
 
 
 @pytest.mark.parametrize("shape", [(128, 784, 1024), (7, 33, 50), (20, 2048, 640), (600, 96, 200), (300, 2048, 4096), (1, 64, 32)])
@@ -189,7 +201,7 @@ def test_fused_fc_relu_entry_points_match_the_unfused_calls(gpu, shape):
 def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
     rng = np.random.default_rng(11)
     D, l = gpu.DeviceBuffer, gpu.lib()
-    for rows, cols in ((1, 1), (128, 10), (37, 400), (16, 1024), (5, 4097)):
+    for rows, cols in ((1, 1), (128, 10), (1024, 16), (1000, 7), (3, 16), (1025, 16), (37, 400), (16, 1024), (5, 4097), (64, 17)):
         x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
         t = np.eye(cols, dtype=np.float32)[rng.integers(0, cols, rows)]
         dx, dt = D.from_numpy(x), D.from_numpy(t)
@@ -203,6 +215,11 @@ def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
         gpu.check(l.lten_hip_log_softmax_backward_f32(rows, cols, y0.ptr, s0.ptr, g0.ptr))
         gpu.check(l.lten_hip_nll_log_softmax_backward_f32(rows, cols, y0.ptr, dt.ptr, -1.0 / rows, g1.ptr))
         assert np.array_equal(g0.numpy(np.float32, x.shape), g1.numpy(np.float32, x.shape)), (rows, cols)
+        y2, l2, g2 = D(x.nbytes), D(4), D(x.nbytes)
+        gpu.check(l.lten_hip_log_softmax_nll_loss_grad_f32(rows, cols, dx.ptr, dt.ptr, -1.0 / rows, y2.ptr, l2.ptr, g2.ptr))
+        assert np.array_equal(y0.numpy(np.float32, x.shape), y2.numpy(np.float32, x.shape)), (rows, cols)
+        assert l0.numpy(np.float32, (1,))[0] == l2.numpy(np.float32, (1,))[0], (rows, cols)
+        assert np.array_equal(g0.numpy(np.float32, x.shape), g2.numpy(np.float32, x.shape)), (rows, cols)
 
 
 def test_elementwise_kernels(gpu, ob):
