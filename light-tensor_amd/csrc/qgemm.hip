@@ -420,12 +420,15 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	// skinny activations: one streaming pass over the weights (option "qskinny": 0 = auto, 2 = off)
 	p.cterm = nullptr;
 	p.rterm = nullptr;
-	if (M <= 32 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+	const bool may_stream = get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0;
+	// below a megabyte of weights the one-launch kernel's many small workgroups win (option "qskinny" 1: stream anyway)
+	const bool large_weights = N * K >= (1ull << 20) || get_option(OPT_QSKINNY) == 1;
+	if (M <= 32 && large_weights && may_stream) {
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
 	}
 	// 33 to 64 rows: two streaming passes (32 rows, then the rest) still beat one pass of 128-row tiles, three would not
-	if (M > 32 && M <= 64 && N >= 2048 && get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
+	if (M > 32 && M <= 64 && N >= 2048 && K <= 8192 && may_stream) {
 		QProblem top = p, rest = p;
 		top.M = 32;
 		rest.M = (int)M - 32;
@@ -438,9 +441,14 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		}
 	}
 	// small outputs: one launch that also takes the zero-point sums (same option switches it off)
-	if (get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0) {
-		const int rc = qdirect_dispatch(p, out, bias, zpA, zpB);
+	if (may_stream) {
+		int rc = qdirect_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
+		// few rows against weights that kernel does not take: still one streaming launch rather than the tiled kernels
+		if (M <= 32) {
+			rc = qskinny_dispatch(p, out, bias, zpA, zpB);
+			if (rc >= 0) return rc;
+		}
 	}
 
 	const int coef_a = 128 - zpB, coef_b = 128 - zpA;

@@ -1,4 +1,5 @@
-// Weight-streaming int8 FC for skinny activations (M <= 32 rows against W[N x K], both contiguous in K).
+// Weight-streaming int8 FC for skinny activations (M <= 32 rows against W[N x K], both contiguous in K, K any multiple
+// of 16 up to 8192 — up to 16384 for M <= 16 — and any N).
 //
 // The work is one pass over W (N*K bytes, read once from HBM); everything else is noise, so the kernel is
 // organised around that stream.  A workgroup takes 16 consecutive rows of W at a time (then the next such
@@ -16,23 +17,20 @@
 // registers with dot4 instructions, only when their coefficient is non-zero.
 #include "common.h"
 #include "qgemm_common.h"
+#include "lds_async.h"
 
 #include <algorithm>
 
 namespace lten_hip {
 
-__device__ __forceinline__ void skinny_async_load16(uint32_t lds_addr, const uint8_t* base, uint32_t voff)
+template <int WAVES, int SMAX, int MB, int OUT, bool SUM_A, bool SUM_B>
+__global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const int32_t* bias, int coef_a, int coef_b, int kw)
 {
-	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
-}
-
-template <int WAVES, int KW, int MB, int OUT, bool SUM_A, bool SUM_B>
-__global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const int32_t* bias, int coef_a, int coef_b)
-{
-	// KW = bytes of K per wavefront (multiple of 1024): K == WAVES * KW
-	constexpr int ROW = KW + 16;         // padded LDS row pitch
+	// kw = bytes of K per wavefront, a multiple of 64, at most SMAX * 64; wavefront w owns k in [w * kw, w * kw + kw) as
+	// far as it lies inside K (any multiple of 16).  A slab holds 1 KB of 16 weight rows: SMAX / 16 passes per row group.
+	constexpr int ROW = 1024 + 16;       // padded LDS row pitch
 	constexpr int SLAB = 16 * ROW;       // one wavefront's slab
-	constexpr int LOADS_PER_ROW = KW / 1024;
+	constexpr int PASSES = SMAX / 16;
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[WAVES * SLAB];
 	// PAR = 2: wave 0 reads one row group's partial tiles while the others already write the next group's (no second
 	// barrier); with two row blocks only one copy fits beside the slabs, and a barrier ends every row group instead
@@ -42,42 +40,49 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int kbeg = wave * KW;
+	const int kbeg = wave * kw;
+	const int klen = max(0, min(kw, p.K - kbeg));   // this wavefront's share of K (0 for wavefronts past a short K)
+	const int steps = (klen + 63) / 64;              // MFMA steps of 64 k; the last may be partial (K % 64 != 0)
 	const uint32_t slab_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + wave * SLAB;
-	const int groups = p.N / 16;
+	const int groups = (p.N + 15) / 16;
 
-	// the whole slab of a row group goes in flight before anything is consumed
-	auto issue_slab = [&](int group) {
-		const uint8_t* base = p.B + (int64_t)group * 16 * p.K + kbeg;
+	// One pass of a row group's slab: 1 KB of each of the 16 rows, one wave-wide load per row (every request a run of whole
+	// cache lines); lanes whose 16 bytes lie past the wavefront's share load nothing.  Rows past N repeat the last row;
+	// their outputs are not stored.
+	auto issue_slab = [&](int group, int pass) {
+		// which lanes take part, as an execution mask: the addresses stay wave-uniform scalars outside any branch
+		const uint64_t live = __ballot(pass * 1024 + lane * 16 < klen);
+		if (live == 0) return;
 #pragma unroll
-		for (int r = 0; r < 16; r++)
-#pragma unroll
-			for (int c = 0; c < LOADS_PER_ROW; c++) skinny_async_load16(slab_addr + r * ROW + c * 1024, base + (int64_t)r * p.K + c * 1024, lane * 16);
+		for (int r = 0; r < 16; r++) {
+			const int row = min(group * 16 + r, p.N - 1);
+			async_load16_masked(live, slab_addr + r * ROW, p.B + (int64_t)row * p.K + kbeg + pass * 1024, lane * 16);
+		}
 	};
-	issue_slab(blockIdx.x);
+	issue_slab(blockIdx.x, 0);
 
 	// the activations of this wavefront's k-slice stay in registers for every row group the workgroup takes
 	const int lrow = lane & 15, lgrp = lane >> 4;
 	const uint8_t* wfrag = smem + wave * SLAB + lrow * ROW + lgrp * 16;
-	constexpr int STEPS = KW / 64;
-	v4i fx[MB][STEPS];  // activation rows mb * 16 + lrow
+	v4i fx[MB][SMAX];  // activation rows mb * 16 + lrow
 	int sa[MB];
+	const v4i zero_u8 = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
 #pragma unroll
 	for (int mb = 0; mb < MB; mb++) {
 		const uint8_t* xrow = p.A + (int64_t)(mb * 16 + lrow) * p.K + kbeg + lgrp * 16;
 		const bool xvalid = mb * 16 + lrow < p.M;
 		sa[mb] = 0;
 #pragma unroll
-		for (int s = 0; s < STEPS; s++) {
-			fx[mb][s] = v4i{ (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
-			if (xvalid) fx[mb][s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
+		for (int s = 0; s < SMAX; s++) {
+			fx[mb][s] = zero_u8;  // what the sign flip turns into zeros: rows past M, k past the share
+			if (xvalid && s * 64 + lgrp * 16 < klen) fx[mb][s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
 		}
 	}
 	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
 	for (int mb = 0; mb < MB; mb++) {
 #pragma unroll
-		for (int s = 0; s < STEPS; s++) {
+		for (int s = 0; s < SMAX; s++) {
 			fx[mb][s] = flip_sign_bits(fx[mb][s]);
 			if (SUM_A) {
 				sa[mb] = __builtin_amdgcn_sdot4(fx[mb][s].x, 0x01010101, sa[mb], false);
@@ -96,30 +101,37 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 
 	int parity = 0;
 	for (int group = blockIdx.x; group < groups; group += gridDim.x, parity = (parity + 1) & (PAR - 1)) {
-		asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab has landed (no other wave reads this slab)
 		v4i acc[MB];
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) acc[mb] = v4i{ 0, 0, 0, 0 };
 		int sb = 0;
 #pragma unroll
-		for (int s = 0; s < STEPS; s++) {
-			v4i fw = *reinterpret_cast<const v4i*>(wfrag + s * 64);
-			fw = flip_bits(fw, p.b_flip);
-			if (SUM_B) {
-				sb = __builtin_amdgcn_sdot4(fw.x, 0x01010101, sb, false);
-				sb = __builtin_amdgcn_sdot4(fw.y, 0x01010101, sb, false);
-				sb = __builtin_amdgcn_sdot4(fw.z, 0x01010101, sb, false);
-				sb = __builtin_amdgcn_sdot4(fw.w, 0x01010101, sb, false);
-			}
-			// MFMA A operand = activations (rows m), B operand = weights (columns n):
-			// lane (lrow, lgrp), register e holds out[m = mb*16 + 4*lgrp + e][n = lrow]
+		for (int pass = 0; pass < PASSES; pass++) {
+			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab has landed (no other wave reads this slab)
 #pragma unroll
-			for (int mb = 0; mb < MB; mb++) acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx[mb][s], fw, acc[mb], 0, 0, 0);
-		}
-		// the slab is consumed (its values sit in registers): the next row group's slab can start to arrive
-		if (group + (int)gridDim.x < groups) {
+			for (int s = 0; s < 16; s++) {
+				const int gs = pass * 16 + s;
+				if (gs < steps) {
+					v4i fw = *reinterpret_cast<const v4i*>(wfrag + s * 64);
+					fw = flip_bits(fw, p.b_flip);
+					// the 16 bytes of a partial last step that lie past K were never loaded
+					if (gs * 64 + lgrp * 16 >= klen) fw = v4i{ 0, 0, 0, 0 };
+					if (SUM_B) {
+						sb = __builtin_amdgcn_sdot4(fw.x, 0x01010101, sb, false);
+						sb = __builtin_amdgcn_sdot4(fw.y, 0x01010101, sb, false);
+						sb = __builtin_amdgcn_sdot4(fw.z, 0x01010101, sb, false);
+						sb = __builtin_amdgcn_sdot4(fw.w, 0x01010101, sb, false);
+					}
+					// MFMA A operand = activations (rows m), B operand = weights (columns n):
+					// lane (lrow, lgrp), register e holds out[m = mb*16 + 4*lgrp + e][n = lrow]
+#pragma unroll
+					for (int mb = 0; mb < MB; mb++) acc[mb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fx[mb][gs], fw, acc[mb], 0, 0, 0);
+				}
+			}
+			// the slab is consumed (its values sit in registers): the next pass or the next row group's slab can start to arrive
 			asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-			issue_slab(group + gridDim.x);
+			if (pass + 1 < PASSES) issue_slab(group, pass + 1);
+			else if (group + (int)gridDim.x < groups) issue_slab(group + gridDim.x, 0);
 		}
 		if (SUM_B) {
 			sb += __shfl_xor(sb, 16, 64); sb += __shfl_xor(sb, 32, 64);
@@ -142,7 +154,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 		const int n = group * 16 + lrow;
 		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-		const int base = coef_b * tsb + p.K * coef_a * coef_b + (bias ? bias[n] : 0);
+		const int base = coef_b * tsb + p.K * coef_a * coef_b + ((bias && n < p.N) ? bias[n] : 0);
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) {
 			v4i tot = { 0, 0, 0, 0 };
@@ -158,7 +170,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
 				const int m = mb * 16 + lgrp * 4 + e;
-				if (m >= p.M) continue;
+				if (m >= p.M || n >= p.N) continue;
 				const int v = tot[e] + base + coef_a * tsa[e];
 				if (OUT == Q_OUT_ACC) static_cast<int*>(p.C)[(int64_t)m * p.N + n] = v;
 				else static_cast<uint8_t*>(p.C)[(int64_t)m * p.N + n] = (uint8_t)requant<OUT>(v, p.mult, p.zp_c);
@@ -168,18 +180,18 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 	}
 }
 
-template <int WAVES, int KW, int MB>
-static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, const char* name)
+template <int WAVES, int SMAX, int MB>
+static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, int kw, const char* name)
 {
-	// as many workgroups as fit the CUs' LDS at once (one per CU at K = 8192); each walks row groups blockIdx.x, blockIdx.x + grid, ...
+	// as many workgroups as fit the CUs' LDS at once (one per CU with eight wavefronts); each walks row groups blockIdx.x, blockIdx.x + grid, ...
 	constexpr int PAR = MB == 1 ? 2 : 1;
-	constexpr int LDS_BYTES = WAVES * 16 * (KW + 16) + PAR * WAVES * MB * 1024 + (PAR + MB) * WAVES * 64;
+	constexpr int LDS_BYTES = WAVES * 16 * (1024 + 16) + PAR * WAVES * MB * 1024 + (PAR + MB) * WAVES * 64;
 	static_assert(LDS_BYTES <= 160 * 1024, "slabs and partial tiles must fit the CU's LDS");
 	constexpr int PER_CU = (160 * 1024) / LDS_BYTES;
-	const dim3 grid((unsigned)std::min<int64_t>(p.N / 16, 256 * PER_CU)), block(WAVES * 64);
+	const dim3 grid((unsigned)std::min<int64_t>((p.N + 15) / 16, 256 * PER_CU)), block(WAVES * 64);
 	set_kernel_name(name);
 	const bool sum_a = coef_a != 0, sum_b = coef_b != 0;
-#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, KW, MB, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b)
+#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, SMAX, MB, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b, kw)
 #define LTEN_SK_OUT(OUTV)                                     \
 	if (sum_a && sum_b) LTEN_SK(OUTV, true, true);        \
 	else if (sum_a) LTEN_SK(OUTV, true, false);           \
@@ -194,22 +206,27 @@ static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int co
 	return 0;
 }
 
-// Returns -1 when the problem does not fit the streaming kernel (the caller then uses the tiled kernels).
+// Returns -1 when the problem does not fit the streaming kernel (the caller then uses the other kernels): up to 32
+// activation rows against weights with 16-byte aligned rows (K a multiple of 16), K up to 8192, or up to 16384 with at
+// most 16 rows (the activations of a wavefront's share of K stay in registers).  N is arbitrary.
 int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b)
 {
-	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N % 16 == 0)) return -1;
+	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N >= 1 && p.K >= 64 && p.K <= 16384)) return -1;
+	if (p.K > 8192 && p.M > 16) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
+	// fewest wavefronts whose share of K fits one slab pass (1 KB): more workgroups per CU for a short K
+	const int waves = p.K <= 2048 ? 2 : (p.K <= 4096 ? 4 : 8);
+	const int kw = (int)ceil_div(ceil_div((uint64_t)p.K, (uint64_t)waves), 64) * 64;
+	if (p.K > 8192) return launch_skinny<8, 32, 1>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w8_2pass");
 	if (p.M <= 16) {
-		if (p.K == 8 * 1024) return launch_skinny<8, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w8_k1024");
-		if (p.K == 4 * 1024) return launch_skinny<4, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w4_k1024");
-		if (p.K == 2 * 1024) return launch_skinny<2, 1024, 1>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w2_k1024");
-	} else {
-		// two blocks of 16 activation rows against every weight fragment
-		if (p.K == 8 * 1024) return launch_skinny<8, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w8_k1024_m32");
-		if (p.K == 4 * 1024) return launch_skinny<4, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w4_k1024_m32");
-		if (p.K == 2 * 1024) return launch_skinny<2, 1024, 2>(p, out, bias, coef_a, coef_b, "qskinny_mfma_w2_k1024_m32");
+		if (waves == 8) return launch_skinny<8, 16, 1>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w8");
+		if (waves == 4) return launch_skinny<4, 16, 1>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w4");
+		return launch_skinny<2, 16, 1>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w2");
 	}
-	return -1;
+	// two blocks of 16 activation rows against every weight fragment
+	if (waves == 8) return launch_skinny<8, 16, 2>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w8_m32");
+	if (waves == 4) return launch_skinny<4, 16, 2>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w4_m32");
+	return launch_skinny<2, 16, 2>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w2_m32");
 }
 
 }  // namespace lten_hip

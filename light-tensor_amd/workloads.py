@@ -95,6 +95,19 @@ def cfg4(M, seed=4, K=8192, N=8192):
     return int8_fc(M, N, K, 128, 0.02, 0.014, 1.0, 128, seed)
 
 
+# (scales, zero points) of the int8 configurations without generating their operands
+def cfg1_params():
+    return np.array([1.0 / 255.0, 0.01, 0.05], np.float32), np.array([0, 128, 128], np.uint8)
+
+
+def cfg3_params():
+    return np.array([0.02, 0.02, 1.0], np.float32), np.array([128, 128, 128], np.uint8)
+
+
+def cfg4_params():
+    return np.array([0.02, 0.014, 1.0], np.float32), np.array([128, 128, 128], np.uint8)
+
+
 def cfg2(seed=2, batch=128, sizes=(784, 1024, 1024, 10)):
     """fp32 MLP: X uniform [0,1), W_l and b_l ~ N(0,0.05), labels uniform 0..9."""
     X = uniform_f64(batch * sizes[0], seed, 1).astype(np.float32).reshape(batch, sizes[0])

@@ -122,6 +122,26 @@ def test_rank1_and_rowvec_shapes(gpu, ob):
     assert rel_err(got, db0 + Y0.astype(np.float64).sum(0, keepdims=True)) < TOL
 
 
+def test_gru_step_products(gpu, ob):
+    """The two M = 1 products of a GRU time step (l-ten/gru.cpp:267-268, 358-361: a 1 x K row times K x 3H, not
+    transposed) at input = hidden = 1024, and at a ragged size, against the oracle's GEMM."""
+    rng = np.random.default_rng(21)
+    for K, N in ((1024, 3072), (1000, 300), (3, 3072)):
+        x = rng.standard_normal((1, K)).astype(np.float32)
+        u = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+        want = np.zeros((1, N), np.float32)
+        ob.sgemm(0, 0, 1, N, K, 1.0, x, K, u, N, 0.0, want, N)
+        got = gpu_sgemm(gpu, 0, 0, 1, N, K, 1.0, x, K, u, N, 0.0, np.zeros((1, N), np.float32), N)
+        assert gpu.last_kernel() == "sgemm_rowvec"
+        assert rel_err(got, want) < TOL, (K, N)
+        assert rel_err(got, x.astype(np.float64) @ u.astype(np.float64)) < TOL, (K, N)
+    # small integers: exact in any order
+    x = rng.integers(-3, 4, (1, 1024)).astype(np.float32)
+    u = rng.integers(-3, 4, (1024, 3072)).astype(np.float32)
+    got = gpu_sgemm(gpu, 0, 0, 1, 3072, 1024, 1.0, x, 1024, u, 3072, 0.0, np.zeros((1, 3072), np.float32), 3072)
+    assert np.array_equal(got, x @ u)
+
+
 def test_strided_batched_and_broadcast(gpu, ob):
     g = np.load(golden_path("layer_cases.npz"))
     # case 0: a{2,1,4,8} x b{1,1,8,15}: b broadcast over the leading index (stride 0)

@@ -106,11 +106,16 @@ def test_alpha_beta_rejected(ob):
     assert ob.oracle().oracle_quantized_matmul(0, 1, 2, 2, 1, 1, A, A, 1, A, qp, None, ws, None) == -1
 
 
-def test_requant_numpy_helper_matches_oracle(ob):
-    # the array helper used for full-size GPU checks is itself checked against the oracle
+def test_requant_numpy_helper_matches_oracle(ob, wl):
+    # the array helper used for full-size GPU checks is itself checked against the oracle, on the multipliers and
+    # zero points of the configurations it is used for (configs 1, 3 and 4) among others
     rng = np.random.default_rng(3)
-    acc = rng.integers(-600000, 600000, 5000).astype(np.int32)
-    for mult, zp in [(4e-4, 128), (7.84e-4, 128), (2.8e-4, 0)]:
+    acc = np.concatenate([rng.integers(-600000, 600000, 5000), rng.integers(-(1 << 24), 1 << 24, 3000),
+                          rng.integers(-300, 300, 500)]).astype(np.int32)
+    cases = [(4e-4, 128), (7.84e-4, 128), (2.8e-4, 0)]
+    for sc, zp in (wl.cfg1_params(), wl.cfg3_params(), wl.cfg4_params()):
+        cases.append((float(np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])), int(zp[2])))
+    for mult, zp in cases:
         got = requant_numpy(acc, np.float32(mult), zp)
         want = np.fromiter((ob.oracle().oracle_requantize(float(np.float32(mult)), int(a), zp) for a in acc), np.uint8)
         assert np.array_equal(got, want)
