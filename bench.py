@@ -529,6 +529,18 @@ def main():
     with_copies()
     copies_ms = best_of(with_copies, 3) * 1e3
 
+    # and through the host-side mirror of l-ten's layer API (lten::Tensor::to, lten::FullyConnected_q::forward, C++)
+    host_api = None
+    host_exe = os.path.join(ROOT, "light-tensor_amd", "host", "test_host")
+    if os.path.exists(host_exe):
+        import subprocess
+        try:
+            r = subprocess.run([host_exe, "bench"], capture_output=True, text=True, timeout=120)
+            lines = [ln for ln in r.stdout.splitlines() if ln.startswith("{")]
+            host_api = json.loads(lines[-1]) if r.returncode == 0 and lines else {"error": (r.stdout + r.stderr)[-300:]}
+        except Exception as e:  # noqa: BLE001
+            host_api = {"error": repr(e)[:300]}
+
     verified = None
     if not args.no_verify:
         acc = ((X.astype(np.float64) - float(zp[0])) @ (W.astype(np.float64) - float(zp[1])).T)
@@ -589,7 +601,8 @@ def main():
         "verified_bit_exact": verified,
         "with_pcie_copies": {"ms_per_step": round(copies_ms, 3), "tops": round(ops / (copies_ms * 1e-3) / 1e12, 2),
                              "note": "operands uploaded and the output downloaded with the library's synchronous copies around "
-                                     "the same call, pageable host memory; for reference only"},
+                                     "the same call, pageable host memory; for reference only",
+                             "through_host_layer_api": host_api},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, W, sc, zp)

@@ -47,9 +47,13 @@ int lten_hip_sync(void);
 
 /* ------------------------------------------------------------------------- memory */
 
-/* Replaces AllocateMemoryOnGPU / gpu_alloc (l-ten/utils.h:29,33; l-ten/utils.cu:8-28,30-58). */
+/* Replaces AllocateMemoryOnGPU / gpu_alloc (l-ten/utils.h:29,33; l-ten/utils.cu:8-28,30-58), memory pool included
+ * (l-ten's default build serves GPU buffers from its power-of-two MemoryPool, l-ten/utils.cu:33-37,
+ * l-ten/memorypool.h:142-173): sizes are rounded up to a power of two (to a multiple of 64 MB above 64 MB), freed
+ * blocks are kept and handed out again without a wait — correct for work issued in order on the library's stream.  Up
+ * to 64 GB stay cached; they go back to the driver when an allocation would otherwise fail. */
 int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory);
-/* Replaces FreeMemoryOnGPU / gpu_free (l-ten/utils.h:30,35; l-ten/utils.cu:60-71). */
+/* Replaces FreeMemoryOnGPU / gpu_free (l-ten/utils.h:30,35; l-ten/utils.cu:60-71).  Freeing a block twice fails. */
 int lten_hip_free(void* device_ptr);
 /* Replaces ZeroMemoryOnGPU (l-ten/utils.h:34; l-ten/utils.cu:49-52). */
 int lten_hip_zero(void* device_ptr, size_t size);
@@ -161,18 +165,28 @@ int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features
 
 /* ------------------------------------------------------------------ im2col / conv */
 
-/* Replace im2col_gpu / col2im_gpu (l-ten/im_col.h:60-73, l-ten/im_col.cu:98-118,164-184).
- * col is [C*kh*kw, Hout*Wout]; col2im overwrites im with the gathered sums, as the
- * CUDA kernel does (l-ten/im_col.cu:123-162). */
+/* Replace im2col_gpu<T> / col2im_gpu<T> (l-ten/im_col.h:60-73, l-ten/im_col.cu:98-118,164-184) in the three
+ * instantiations l-ten compiles, float, int and uint8_t (l-ten/im_col.cu:199-218).  col is [C*kh*kw, Hout*Wout];
+ * col2im overwrites im with the gathered sums, as the CUDA kernel does (l-ten/im_col.cu:123-162); integer sums
+ * wrap as the template's `+=` on T does. */
 int lten_hip_im2col_f32(const float* im, int channels, int height, int width, int kernel_h, int kernel_w,
                         int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                         float* col);
+int lten_hip_im2col_i32(const int32_t* im, int channels, int height, int width, int kernel_h, int kernel_w,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                        int32_t* col);
 int lten_hip_im2col_u8(const uint8_t* im, int channels, int height, int width, int kernel_h, int kernel_w,
                        int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                        uint8_t* col);
 int lten_hip_col2im_f32(const float* col, int channels, int height, int width, int kernel_h, int kernel_w,
                         int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
                         float* im);
+int lten_hip_col2im_i32(const int32_t* col, int channels, int height, int width, int kernel_h, int kernel_w,
+                        int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                        int32_t* im);
+int lten_hip_col2im_u8(const uint8_t* col, int channels, int height, int width, int kernel_h, int kernel_w,
+                       int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                       uint8_t* im);
 
 /* Conv2d::forward's per-image im2col + cublasSgemm loop (l-ten/conv2d.cpp:164-171) as one
  * implicit-GEMM launch over the whole batch; no col buffer is materialised.

@@ -57,6 +57,9 @@ _SIGNATURES = {
     "lten_hip_fcq_prepare_weights": (C.c_int, [vp, vp, u64]),
     "lten_hip_fcq_forward_static": (C.c_int, [u64, u64, u64, u64, vp, vp, vp, C.POINTER(QParams), vp]),
     "lten_hip_im2col_f32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
+    "lten_hip_im2col_i32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
+    "lten_hip_col2im_i32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
+    "lten_hip_col2im_u8": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
     "lten_hip_im2col_u8": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
     "lten_hip_col2im_f32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
     "lten_hip_conv2d_forward_f32": (C.c_int, [u64] * 5 + [C.c_int] * 6 + [vp, vp, vp, vp]),

@@ -28,14 +28,15 @@ __global__ __launch_bounds__(256) void im2col_kernel(const T* im, ConvGeo g, T* 
 	}
 }
 
-__global__ __launch_bounds__(256) void col2im_kernel(const float* col, ConvGeo g, float* im)
+template <typename T>
+__global__ __launch_bounds__(256) void col2im_kernel(const T* col, ConvGeo g, T* im)
 {
 	// one thread per image element gathers every column entry that maps to it, kernel taps in increasing
 	// (i, j) order — the order in which l-ten's CPU scatter-add reaches that element (l-ten/im_col.h:41-55)
 	const int64_t total = (int64_t)g.Cin * g.H * g.W;
 	for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
 		const int x = (int)(idx % g.W), y = (int)((idx / g.W) % g.H), c = (int)(idx / ((int64_t)g.W * g.H));
-		float s = 0.0f;
+		T s = (T)0;  // integer types wrap as l-ten's `+=` on T does
 		for (int i = 0; i < g.kh; i++) {
 			const int yy = y + g.ph - i * g.dh;
 			if (yy < 0 || yy % g.sh != 0 || yy / g.sh >= g.Ho) continue;
@@ -223,45 +224,58 @@ static bool dgrad_as_forward(const ConvGeo& g)
 
 using namespace lten_hip;
 
-extern "C" {
-
-int lten_hip_im2col_f32(const float* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
-                        int dw, float* col)
+template <typename T>
+static int im2col_run(const T* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, T* col)
 {
 	ConvGeo g;
 	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
 	const int64_t total = (int64_t)C * kh * kw * g.Ho * g.Wo;
 	if (total == 0) return 0;
 	LTEN_HIP_REQUIRE(im && col, "im2col: null pointer");
-	im2col_kernel<float><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(im, g, col);
+	im2col_kernel<T><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(im, g, col);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }
 
-int lten_hip_im2col_u8(const uint8_t* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
-                       int dw, uint8_t* col)
-{
-	ConvGeo g;
-	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
-	const int64_t total = (int64_t)C * kh * kw * g.Ho * g.Wo;
-	if (total == 0) return 0;
-	LTEN_HIP_REQUIRE(im && col, "im2col: null pointer");
-	im2col_kernel<uint8_t><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(im, g, col);
-	LTEN_HIP_LAUNCH_CHECK();
-	return 0;
-}
-
-int lten_hip_col2im_f32(const float* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh,
-                        int dw, float* im)
+template <typename T>
+static int col2im_run(const T* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, T* im)
 {
 	ConvGeo g;
 	if (int rc = make_geo(g, 1, C, H, W, 1, kh, kw, ph, pw, sh, sw, dh, dw)) return rc;
 	const int64_t total = (int64_t)C * H * W;
 	if (total == 0) return 0;
 	LTEN_HIP_REQUIRE(im && col, "col2im: null pointer");
-	col2im_kernel<<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(col, g, im);
+	col2im_kernel<T><<<dim3((unsigned)std::min<uint64_t>(ceil_div(total, 256), 65536)), dim3(256), 0, stream()>>>(col, g, im);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
+}
+
+extern "C" {
+
+// the three instantiations of l-ten/im_col.cu:199-218 each
+int lten_hip_im2col_f32(const float* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, float* col)
+{
+	return im2col_run<float>(im, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, col);
+}
+int lten_hip_im2col_i32(const int32_t* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, int32_t* col)
+{
+	return im2col_run<int32_t>(im, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, col);
+}
+int lten_hip_im2col_u8(const uint8_t* im, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, uint8_t* col)
+{
+	return im2col_run<uint8_t>(im, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, col);
+}
+int lten_hip_col2im_f32(const float* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, float* im)
+{
+	return col2im_run<float>(col, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, im);
+}
+int lten_hip_col2im_i32(const int32_t* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, int32_t* im)
+{
+	return col2im_run<int32_t>(col, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, im);
+}
+int lten_hip_col2im_u8(const uint8_t* col, int C, int H, int W, int kh, int kw, int ph, int pw, int sh, int sw, int dh, int dw, uint8_t* im)
+{
+	return col2im_run<uint8_t>(col, C, H, W, kh, kw, ph, pw, sh, sw, dh, dw, im);
 }
 
 int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,

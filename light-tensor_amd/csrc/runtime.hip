@@ -3,6 +3,10 @@
 #include "common.h"
 
 #include <cstring>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
 
 namespace lten_hip {
 
@@ -37,6 +41,27 @@ bool capturing() { return g_capturing; }
 static int g_options[OPT_COUNT] = { 0 };
 static const char* const g_option_names[OPT_COUNT] = { "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant", "qgemm_split" };
 int get_option(Option o) { return g_options[o]; }
+
+// Device memory pool behind lten_hip_alloc / lten_hip_free, the counterpart of l-ten's MemoryPool for GPU buffers
+// (l-ten/utils.cu:30-47 with USE_MEMORYPOOL, l-ten/memorypool.h:142-173): sizes are rounded up to a power of two (to a
+// multiple of 64 MB above that), freed blocks are kept per size and handed out again, so that a layer's forward pass,
+// which allocates its result tensor on every call, does not pay a hipMalloc each time.  Blocks are reused without any
+// wait: safe for work issued in order on the library's stream, which is the only order this library creates.  At most
+// POOL_CACHE_LIMIT bytes stay cached; beyond that a freed block goes back to the driver.
+constexpr uint64_t POOL_CACHE_LIMIT = 64ull << 30;
+static std::mutex g_pool_mutex;
+static std::map<uint64_t, std::vector<void*>> g_pool_free;  // rounded size -> cached blocks
+static std::unordered_map<void*, uint64_t> g_pool_size;     // every block handed out or cached -> its rounded size, bit 0 set while cached
+static uint64_t g_pool_cached = 0;
+
+static uint64_t pool_round(uint64_t size)
+{
+	if (size <= 256) return 256;
+	if (size > (64ull << 20)) return (size + (64ull << 20) - 1) / (64ull << 20) * (64ull << 20);
+	uint64_t r = 256;
+	while (r < size) r <<= 1;
+	return r;
+}
 
 template <typename T>
 __global__ void fill_kernel(T* p, uint64_t n, T v)
@@ -112,7 +137,37 @@ int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
 	LTEN_HIP_REQUIRE(device_ptr != nullptr, "lten_hip_alloc: null pointer");
 	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_alloc");
 	*device_ptr = nullptr;
-	LTEN_HIP_CHECK(hipMalloc(device_ptr, size ? size : 1));
+	const uint64_t rounded = pool_round(size);
+	{
+		std::lock_guard<std::mutex> lock(g_pool_mutex);
+		auto it = g_pool_free.find(rounded);
+		if (it != g_pool_free.end() && !it->second.empty()) {
+			*device_ptr = it->second.back();
+			it->second.pop_back();
+			g_pool_cached -= rounded;
+			g_pool_size[*device_ptr] = rounded;
+		}
+	}
+	if (*device_ptr == nullptr) {
+		hipError_t e = hipMalloc(device_ptr, rounded);
+		if (e != hipSuccess) {
+			// out of memory with blocks cached: give them back and try once more
+			(void)hipGetLastError();
+			std::vector<void*> drop;
+			{
+				std::lock_guard<std::mutex> lock(g_pool_mutex);
+				for (auto& kv : g_pool_free) {
+					for (void* q : kv.second) { drop.push_back(q); g_pool_size.erase(q); }
+					kv.second.clear();
+				}
+				g_pool_cached = 0;
+			}
+			for (void* q : drop) (void)hipFree(q);
+			LTEN_HIP_CHECK(hipMalloc(device_ptr, rounded));
+		}
+		std::lock_guard<std::mutex> lock(g_pool_mutex);
+		g_pool_size[*device_ptr] = rounded;
+	}
 	if (zero_memory && size) return lten_hip_zero(*device_ptr, size);  // a fill kernel, stream ordered
 	return 0;
 }
@@ -120,7 +175,20 @@ int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
 int lten_hip_free(void* device_ptr)
 {
 	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_free");
-	if (device_ptr) LTEN_HIP_CHECK(hipFree(device_ptr));
+	if (device_ptr == nullptr) return 0;
+	{
+		std::lock_guard<std::mutex> lock(g_pool_mutex);
+		auto it = g_pool_size.find(device_ptr);
+		LTEN_HIP_REQUIRE(it == g_pool_size.end() || (it->second & 1) == 0, "lten_hip_free: %p was freed already", device_ptr);
+		if (it != g_pool_size.end() && g_pool_cached + it->second <= POOL_CACHE_LIMIT) {
+			g_pool_free[it->second].push_back(device_ptr);
+			g_pool_cached += it->second;
+			it->second |= 1;
+			return 0;
+		}
+		if (it != g_pool_size.end()) g_pool_size.erase(it);
+	}
+	LTEN_HIP_CHECK(hipFree(device_ptr));  // memory that did not come from lten_hip_alloc, or a full cache
 	return 0;
 }
 

@@ -455,8 +455,63 @@ static int error_test()
 	return caught == 5 ? 0 : -1;
 }
 
-int main()
+// `test_host bench`: the int8 FullyConnected_q forward at 4096^3 as a caller of the layer API sees it, copies included:
+// input tensor on the CPU -> to(GPU), forward, result -> to(CPU); and the forward alone on a resident input.  The layer
+// (weights, their int8 form) is moved to the GPU once beforehand, as a network is.  Prints one JSON line.
+#include <algorithm>
+#include <chrono>
+#include "../../include/lten_hip.h"
+static int api_bench()
 {
+	const uint64_t M = 4096, K = 4096, N = 4096;
+	std::vector<uint8_t> x(M * K), w(N * K);
+	unsigned s = 7;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (s >> 16) & 0xFF; };
+	for (auto& e : x) e = (uint8_t)rnd();
+	for (auto& e : w) e = (uint8_t)(128 + (int)(rnd() % 81) - 40);
+	lten::TensorOps ops;
+	ops.data_type = lten::UINT8;
+	lten::FullyConnected_q fc(K, N, false);
+	fc.init();
+	fc.train(false);
+	memcpy(fc.get_weights()->get_data_ptr(), w.data(), w.size());
+	QuantizationParams qi{ 0.02f, 128 }, qw{ 0.02f, 128 }, qo{ 1.0f, 128 };
+	fc.set_qparams_in(qi);
+	fc.set_qparams_params(&qw, 1);
+	fc.set_qparams_out(qo);
+	fc.to(lten::GPU);
+	lten::Tensor Xc = lten::TensorFromBuffer({ 1, M, K }, x.data(), false, &ops);
+	auto now = [] { return std::chrono::steady_clock::now(); };
+	auto ms = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::milli>(b - a).count(); };
+	double best_api = 1e30, best_resident = 1e30;
+	for (int rep = 0; rep < 5; rep++) {
+		auto t0 = now();
+		lten::Tensor Xg = Xc.to(lten::GPU);
+		lten::Tensor Y = fc.forward(Xg).to(lten::CPU);  // the download waits for the product
+		best_api = std::min(best_api, ms(t0, now()));
+	}
+	lten::Tensor Xg = Xc.to(lten::GPU);
+	for (int rep = 0; rep < 3; rep++) {
+		lten::Tensor warm = fc.forward(Xg);
+		lten_hip_sync();
+		const int iters = 200;
+		auto t0 = now();
+		for (int i = 0; i < iters; i++) lten::Tensor Y = fc.forward(Xg);
+		lten_hip_sync();
+		best_resident = std::min(best_resident, ms(t0, now()) / iters);
+	}
+	const double ops2 = 2.0 * M * N * K;
+	printf("{\"api\": \"lten::Tensor::to + lten::FullyConnected_q::forward\", \"with_copies_ms\": %.3f, \"with_copies_tops\": %.2f, "
+	       "\"resident_ms_per_forward\": %.5f, \"resident_tops\": %.1f}\n",
+	       best_api, ops2 / (best_api * 1e-3) / 1e12, best_resident, ops2 / (best_resident * 1e-3) / 1e12);
+	return 0;
+}
+
+int main(int argc, char** argv)
+{
+	if (argc > 1 && strcmp(argv[1], "bench") == 0) {
+		try { return api_bench(); } catch (std::exception& e) { printf("exception: %s\n", e.what()); return 1; }
+	}
 	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test }, { "training_test", training_test }, { "conv_training_test", conv_training_test },
 		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;

@@ -37,6 +37,26 @@ def test_im2col_col2im_bit_exact(gpu, ob, geo):
     dC, dBack = D.from_numpy(c), D(im.nbytes)
     gpu.check(gpu.lib().lten_hip_col2im_f32(dC.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dBack.ptr))
     assert np.array_equal(dBack.numpy(np.float32, im.shape), back)
+    # the int and uint8 instantiations (l-ten/im_col.cu:199-218): integers small enough to be exact as floats go through
+    # the same oracle functions; uint8 sums wrap modulo 256 as the template's `+=` on uint8_t does
+    imi = rng.integers(-100000, 100000, (C, H, W)).astype(np.int32)
+    coli = np.empty(col.shape, np.float32)
+    ob.oracle().oracle_im2col_f32(imi.astype(np.float32).reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, coli.reshape(-1))
+    dImi, dColi = D.from_numpy(imi), D(4 * col.size)
+    gpu.check(gpu.lib().lten_hip_im2col_i32(dImi.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dColi.ptr))
+    assert np.array_equal(dColi.numpy(np.int32, col.shape), coli.astype(np.int32))
+    ci = rng.integers(-1000, 1000, col.shape).astype(np.int32)
+    backi = np.zeros(im.shape, np.float32)
+    ob.oracle().oracle_col2im_f32(ci.astype(np.float32).reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, backi.reshape(-1))
+    dCi, dBacki = D.from_numpy(ci), D(4 * im.size)
+    gpu.check(gpu.lib().lten_hip_col2im_i32(dCi.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dBacki.ptr))
+    assert np.array_equal(dBacki.numpy(np.int32, im.shape), backi.astype(np.int32))
+    cu = rng.integers(0, 256, col.shape, dtype=np.uint8)
+    backu = np.zeros(im.shape, np.float32)
+    ob.oracle().oracle_col2im_f32(cu.astype(np.float32).reshape(-1), C, H, W, kh, kw, ph, pw, sh, sw, backu.reshape(-1))
+    dCu, dBacku = D.from_numpy(cu), D(im.size)
+    gpu.check(gpu.lib().lten_hip_col2im_u8(dCu.ptr, C, H, W, kh, kw, ph, pw, sh, sw, 1, 1, dBacku.ptr))
+    assert np.array_equal(dBacku.numpy(np.uint8, im.shape), (backu.astype(np.int64) % 256).astype(np.uint8))
 
 
 def gpu_conv(gpu, geo, x, w, dy=None, bias=None):

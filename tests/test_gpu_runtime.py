@@ -35,9 +35,20 @@ def test_fill_zero_copy_and_get_device(gpu):
     src = D.from_numpy(np.arange(n, dtype=np.int32))
     gpu.check(l.lten_hip_copy_gpu_to_gpu(a.ptr, src.ptr, 4 * n))
     assert np.array_equal(a.numpy(np.int32, (n,)), np.arange(n, dtype=np.int32))
-    # alloc with zero_memory hands out zeros
-    z = D(4096 + 3, zero=True)
-    assert not z.numpy(np.uint8, (4099,)).any()
+    # alloc with zero_memory hands out zeros, also when the block comes back from the pool with old contents
+    for _ in range(3):
+        z = D(4096 + 3, zero=True)
+        assert not z.numpy(np.uint8, (4099,)).any()
+        gpu.check(l.lten_hip_fill_u8(z.ptr, 4099, 0x5A))
+        z.free()
+    # the pool hands a freed block of the same rounded size out again; freeing twice is an error
+    p1, p2 = C.c_void_p(), C.c_void_p()
+    gpu.check(l.lten_hip_alloc(C.byref(p1), 3000000, 0))
+    gpu.check(l.lten_hip_free(p1))
+    gpu.check(l.lten_hip_alloc(C.byref(p2), 2500000, 0))   # both round to 4 MiB
+    assert p2.value == p1.value
+    gpu.check(l.lten_hip_free(p2))
+    assert l.lten_hip_free(p2) != 0 and b"freed already" in l.lten_hip_last_error()
 
 
 def test_calls_that_cannot_be_recorded_fail_with_a_message(gpu):
