@@ -59,26 +59,47 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 			async_load16_masked(live, slab_addr + r * ROW, p.B + (int64_t)row * p.K + kbeg + pass * 1024, lane * 16);
 		}
 	};
-	issue_slab(blockIdx.x, 0);
-
 	// the activations of this wavefront's k-slice stay in registers for every row group the workgroup takes
 	const int lrow = lane & 15, lgrp = lane >> 4;
 	const uint8_t* wfrag = smem + wave * SLAB + lrow * ROW + lgrp * 16;
 	v4i fx[MB][SMAX];  // activation rows mb * 16 + lrow
 	int sa[MB];
 	const v4i zero_u8 = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+	// They are fetched with four neighbouring lanes on the 64 bytes a row contributes to a step (lane 4 r + g: row r,
+	// 16-byte group g), which the memory pipeline handles as one access per row, and exchanged into the MFMA layout
+	// (lane r + 16 g) afterwards: fetched in the MFMA layout directly, neighbouring lanes name different rows and every
+	// lane costs a cache look-up of its own (four times as many for 16 rows; 3 us of a 15 us kernel).
+	// With fewer than four rows the exchange costs more than it saves and the lanes fetch in the MFMA layout.
+	const bool exchange = p.M >= 4;
+	const int ld_row = exchange ? lane >> 2 : lrow, ld_grp = exchange ? lane & 3 : lgrp;
 #pragma unroll
 	for (int mb = 0; mb < MB; mb++) {
-		const uint8_t* xrow = p.A + (int64_t)(mb * 16 + lrow) * p.K + kbeg + lgrp * 16;
-		const bool xvalid = mb * 16 + lrow < p.M;
+		const uint8_t* xrow = p.A + (int64_t)(mb * 16 + ld_row) * p.K + kbeg + ld_grp * 16;
+		const bool xvalid = mb * 16 + ld_row < p.M;
 		sa[mb] = 0;
 #pragma unroll
 		for (int s = 0; s < SMAX; s++) {
 			fx[mb][s] = zero_u8;  // what the sign flip turns into zeros: rows past M, k past the share
-			if (xvalid && s * 64 + lgrp * 16 < klen) fx[mb][s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
+			if (xvalid && s * 64 + ld_grp * 16 < klen) fx[mb][s] = *reinterpret_cast<const v4i*>(xrow + s * 64);
 		}
 	}
-	asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	// the first row group's slab goes in flight behind the activations, so that the exchange below can wait for the
+	// activations alone (loads complete in order) while the slab is still arriving
+	issue_slab(blockIdx.x, 0);
+	if (klen > 0) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+	else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+	if (exchange) {
+		const int src = 4 * lrow + lgrp;  // the lane that fetched what this lane feeds to the MFMA
+#pragma unroll
+		for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+			for (int s = 0; s < SMAX; s++) {
+				fx[mb][s].x = __shfl(fx[mb][s].x, src, 64);
+				fx[mb][s].y = __shfl(fx[mb][s].y, src, 64);
+				fx[mb][s].z = __shfl(fx[mb][s].z, src, 64);
+				fx[mb][s].w = __shfl(fx[mb][s].w, src, 64);
+			}
+	}
 #pragma unroll
 	for (int mb = 0; mb < MB; mb++) {
 #pragma unroll
