@@ -75,10 +75,20 @@ def vendor_int8(timeout_s=240):
         return {"error": repr(e)[:300]}
 
 
+SETTLE_S = 0.06
+
+
 def timed(lt, fn, iters, warmup=3):
-    """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on the library's stream)."""
-    for _ in range(warmup):
+    """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on the library's stream), in the
+    steady state: after an idle spell the part needs tens of milliseconds of load before its clocks settle (the first
+    launches of an MFMA-bound kernel run up to 1.5x slower), so the same call is repeated for SETTLE_S seconds first."""
+    t_end = time.perf_counter() + SETTLE_S
+    n = 0
+    while n < warmup or time.perf_counter() < t_end:
         fn()
+        n += 1
+        if n % 100 == 0:
+            lt.sync()
     lt.sync()
     t = lt.Timer()
     t.start()

@@ -140,6 +140,14 @@ def test_conv_vs_oracle(gpu, ob, geo, variant):
         gpu.set_option("conv_variant", 0)
 
 
+@pytest.mark.parametrize("geo", [(41, 8, 37, 132, 64, 3, 3, 1, 1, 1, 1), (40, 8, 37, 132, 128, 3, 3, 1, 1, 1, 1),
+                                 (60, 8, 37, 132, 32, 3, 3, 1, 1, 1, 1)])
+def test_conv_many_tiles(gpu, ob, geo):
+    """Many tiles of the direct-to-LDS forward kernel in one launch (820, 1600 and 1200, more than the chip holds at a
+    time), with a ragged last row tile, a ragged second column tile and several images."""
+    _conv_vs_oracle(gpu, ob, geo)
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
