@@ -1,27 +1,30 @@
-// Conv2d weight gradient, 3x3, stride 1, padding 1, with both LDS tiles filled by direct global->LDS loads.
+// Conv2d weight gradient, 3x3, stride 1, padding 1, with both LDS tiles filled by direct global->LDS loads and every
+// input row fetched once per column strip.
 //
 // The same tile and MFMA schedule as conv2d_patch_wgrad_kernel (rows = 64 output channels, columns = (tap, 32
 // input channels), reduction over pixels in chunks of 64 pixels of one output row; wavefront (row tile mt, pixel
-// half) holds the nine tap tiles), one workgroup per CU, two LDS stages, one barrier per chunk.  What differs is
-// how a chunk reaches LDS: no registers, no LDS stores, no branches and little vector ALU work on the way.
+// half) holds the nine tap tiles), one workgroup per CU, one barrier per chunk.  What differs is how a chunk
+// reaches LDS: no registers, no LDS stores, no branches and little vector ALU work on the way.
 // Measured on this part, for a wavefront that is alone on its SIMD: a vector ALU instruction between two fp32
 // MFMAs delays the second one by about 12 shader clocks (4 for every further one), a taken branch by far more,
-// while LDS reads and scalar instructions (a dozen per MFMA) cost nothing.  The register-staged kernel spends 12 %
-// of its cycles fetching and 4 % on the staging stores; this one keeps the matrix pipe about 90 % busy.
+// while LDS reads and scalar instructions (a dozen per MFMA) cost nothing.
+//
+// Chunks are walked down a strip of 64 columns: (image, strip, row) with the row running fastest.  Output row ho
+// needs input rows ho - 1 .. ho + 1, of which the chunk before it (row ho - 1) already had two, so the input rows
+// live in a ring of eight LDS slots and a chunk fetches one new row (a third of the patch).  Only the first chunk of
+// a workgroup and the first row of a strip fetch all three.  A ring slot holds [32 channels][19 float4]: float4 f
+// of a channel is input columns w0 - 4 + 4 f .. + 3 (f = 0 and f = 17 are the halo, f = 18 is padding that keeps
+// the 32 channels of an operand read on eight banks).
 //
 // A wave-wide direct load writes lane L's 16 bytes at LDS address base + 16 L, so the LDS layout is fixed by
 // which global float4 each lane fetches:
 //   dy tile   load j = 4 fg + cg (fg = group of four pixel quads, cg = group of 16 channels): lane L = 16 fq + cq
 //             fetches pixels 4 (4 fg + fq) .. + 3 of channel 16 cg + cq: 16 rows x 64 contiguous bytes per load
-//   patch     [32 channels][3 rows][18 float4] with a channel pitch of 55 float4; float4 number c = 64 j + L of
-//             load j is (channel c / 55, row (c % 55) / 18, input columns w0 - 4 + 4 ((c % 55) % 18) ..)
-// With 16-byte granules the 32 lanes of an operand read (32 channels, one pixel) cannot all fall on different
-// banks (several lanes per bank with any pitch); the reads are issued nine MFMAs ahead and the loop without its
-// loads still runs at 97 % of the MFMA rate, so that does not matter here.
-// Lanes whose float4 never exists (pad slot, channel beyond Cin or Cout) never load; their slots keep the zeros
-// written once.  Lanes whose float4 lies outside the image in this chunk only (halo row above the first / below
-// the last image row, halo float4 left of the first / right of the last column) store zeros instead of loading.
-// Both are done by setting the execution mask, not by branching.
+//   row       float4 number c = 64 j + L of load j is (channel c / 19, float4 c % 19)
+// Lanes whose float4 never exists (pad slot, channel beyond Cin or Cout) never load.  Lanes whose float4 lies
+// outside the image (a whole row above the first / below the last image row, the halo float4 left of the first /
+// right of the last column) store zeros instead of loading.  Both are done by setting the execution mask, not by
+// branching.
 //
 // Needs W % 64 == 0 (whole chunks; the halo float4s are then inside or outside the image as a whole) and 16-byte
 // aligned x and dy.
@@ -36,18 +39,16 @@ namespace lten_hip {
 namespace {
 
 struct FastWgrad {
-	static constexpr int BM = 64, CIB = 32, TW = 64, TAPS = 9, STEPS = TW / 4, SLOTS = STEPS * TAPS;
-	static constexpr int DY_LOADS = 16, DY_BYTES = DY_LOADS * 1024;
-	static constexpr int F4_ROW = 18, PITCH_F4 = 55, PWS = F4_ROW * 4, CS = PITCH_F4 * 4;
-	static constexpr int PATCH_F4 = CIB * PITCH_F4;             // 1760
-	static constexpr int PATCH_LOADS = (PATCH_F4 + 63) / 64;    // 28
-	static constexpr int PATCH_BYTES = PATCH_LOADS * 1024;
-	static constexpr int STAGE = DY_BYTES + PATCH_BYTES;        // 45056
-	static constexpr int DPW = DY_LOADS / 4, PPW = PATCH_LOADS / 4;  // loads per wavefront
-	static constexpr int TAPS_PER_ROUND = 2 * STAGE / 4 / (2 * 64 * 16);  // taps whose accumulators fit the final exchange
-	static_assert(PATCH_LOADS % 4 == 0 && TAPS_PER_ROUND >= 1, "tile shape");
-	// chunk flags: why a float4 does not exist in this chunk
-	static constexpr unsigned TOP = 1, BOTTOM = 2, LEFT = 4, RIGHT = 8;
+	static constexpr int BM = 64, CIB = 32, TW = 64, TAPS = 9, STEPS = TW / 4;
+	static constexpr int DY_LOADS = 16, DY_BYTES = DY_LOADS * 1024, DPW = DY_LOADS / 4;
+	static constexpr int F4_ROW = 18, PITCH_F4 = 19, CS = PITCH_F4 * 4;
+	static constexpr int ROW_F4 = CIB * PITCH_F4;               // 608
+	static constexpr int ROW_LOADS = (ROW_F4 + 63) / 64;        // 10
+	static constexpr int ROW_BYTES = ROW_LOADS * 1024;
+	static constexpr int RPW = (ROW_LOADS + 3) / 4;             // row loads per wavefront; the last may not exist
+	static constexpr int RING = 8, RING0 = 2 * DY_BYTES;        // two dy stages, then the ring
+	static constexpr int TOTAL = RING0 + RING * ROW_BYTES;      // 114688
+	static_assert(TOTAL / 4 >= 2 * 64 * 16 * TAPS, "the final exchange of the nine tap tiles fits LDS in one round");
 };
 
 }  // namespace
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ partial, int chunks_per_part)
 {
 	typedef FastWgrad P;
-	__shared__ __attribute__((aligned(1024))) uint8_t smem[2 * P::STAGE];
+	__shared__ __attribute__((aligned(1024))) uint8_t smem[P::TOTAL];
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -71,70 +72,63 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 	const uint32_t lane16 = lane * 16;
 	const lds_v4f zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
 
-	// ---- what this lane fetches: dy loads j = 4 wave + i, patch loads j = wave + 4 i
+	// ---- what this lane fetches: dy loads j = 4 wave + i, row loads j = wave + 4 i
 	const int cq = lane & 15, fq = lane >> 4;
 	const uint32_t dy_voff = (uint32_t)((cq * plane + 4 * (4 * wave + fq)) * 4);  // + i * 16 channels, in the base
 	// which lanes take part is kept as execution masks (wave-wide bit sets in scalar registers)
-	uint64_t dy_mask[P::DPW], p_exists[P::PPW];
+	uint64_t dy_mask[P::DPW], r_exists[P::RPW], r_left[P::RPW], r_right[P::RPW];
 #pragma unroll
 	for (int i = 0; i < P::DPW; i++) dy_mask[i] = __ballot(co0 + 16 * i + cq < g.Cout);
-	uint32_t p_voff[P::PPW], p_flags[P::PPW];
+	uint32_t r_voff[P::RPW];
 #pragma unroll
-	for (int i = 0; i < P::PPW; i++) {
-		const int c = (wave + 4 * i) * 64 + lane;
-		const int ci = c / P::PITCH_F4, rem = c % P::PITCH_F4, r = rem / P::F4_ROW, f = rem % P::F4_ROW;
-		const bool never = rem == P::PITCH_F4 - 1 || ci >= P::CIB || ci0 + ci >= g.Cin;
-		p_flags[i] = never ? 0 : (r == 0 ? P::TOP : 0) | (r == 2 ? P::BOTTOM : 0) | (f == 0 ? P::LEFT : 0) | (f == P::F4_ROW - 1 ? P::RIGHT : 0);
-		p_exists[i] = __ballot(!never);
-		p_voff[i] = never ? 0 : (uint32_t)((((int64_t)ci * g.H + r) * g.W + 4 * f) * 4);  // from (row ho - 1, column w0 - 4) of channel ci0
+	for (int i = 0; i < P::RPW; i++) {
+		const int j = wave + 4 * i, c = j * 64 + lane;
+		const int ci = c / P::PITCH_F4, f = c % P::PITCH_F4;
+		const bool exists = j < P::ROW_LOADS && f < P::F4_ROW && ci < P::CIB && ci0 + ci < g.Cin;
+		r_exists[i] = __ballot(exists);
+		r_left[i] = __ballot(exists && f == 0);
+		r_right[i] = __ballot(exists && f == P::F4_ROW - 1);
+		r_voff[i] = exists ? (uint32_t)((ci * plane + 4 * f) * 4) : 0;  // from (row, column w0 - 4) of channel ci0
 	}
-	// The chunk's position is kept as two byte addresses that advance with it: dyb = (image, channel co0, row ho,
-	// column w0) of dy, xb = (image, channel ci0, row ho - 1, column w0 - 4) of x (which may lie before the array;
-	// lanes that would read there are masked).  Rows follow each other in memory, so the next chunk is 256 bytes
-	// on, except after the last row of an image, where the remaining channels of that image are skipped.
-	int ho_c = (begin / tiles_w) % g.H, w0_c = (begin % tiles_w) * P::TW;
-	const int n_first = begin / (tiles_w * g.H);
-	const char* dyb = reinterpret_cast<const char*>(dy + (((int64_t)n_first * g.Cout + co0) * g.H + ho_c) * g.W + w0_c);
-	const char* xb = reinterpret_cast<const char*>(x + (((int64_t)n_first * g.Cin + ci0) * g.H + ho_c - 1) * g.W + w0_c - 4);
-	const int64_t dy_image_skip = (int64_t)(g.Cout - 1) * plane * 4, x_image_skip = (int64_t)(g.Cin - 1) * plane * 4;
-	const int64_t dy_group_step = 16 * plane * 4;  // 16 channels on
-	auto next_chunk = [&]() {
-		w0_c += P::TW;
-		dyb += P::TW * 4;
-		xb += P::TW * 4;
-		if (w0_c >= g.W) {
-			w0_c = 0;
-			if (++ho_c == g.H) {
-				ho_c = 0;
-				dyb += dy_image_skip;
-				xb += x_image_skip;
+
+	// ---- the load cursor: the chunk whose loads go out next, as (image, strip, row)
+	int ld_n = begin / (tiles_w * g.H), ld_strip = (begin / g.H) % tiles_w, ld_ho = begin % g.H;
+	auto advance = [&]() {
+		if (++ld_ho == g.H) {
+			ld_ho = 0;
+			if (++ld_strip == tiles_w) {
+				ld_strip = 0;
+				ld_n++;
 			}
 		}
 	};
-	// one load of the chunk at (dyb, xb, ho_c, w0_c) into `stage`: k < DPW is a dy load, the others are patch loads
-	auto load_piece = [&](int stage, int k) {
-		const uint32_t stage_addr = smem_addr + stage * P::STAGE;
-		if (k < P::DPW) {
-			async_load16_masked(dy_mask[k], stage_addr + (4 * wave + k) * 1024, dyb + k * dy_group_step, dy_voff);
-			return;
-		}
-		const int i = k - P::DPW;
-		const unsigned cf = (ho_c == 0 ? P::TOP : 0) | (ho_c == g.H - 1 ? P::BOTTOM : 0) | (w0_c == 0 ? P::LEFT : 0) |
-		                    (w0_c + P::TW >= g.W ? P::RIGHT : 0);
-		const uint64_t outside = __ballot((p_flags[i] & cf) != 0);
-		const uint32_t slot = stage_addr + P::DY_BYTES + (wave + 4 * i) * 1024;
-		async_load16_masked(p_exists[i] & ~outside, slot, xb, p_voff[i]);
+	// one piece of the dy tile of the chunk under the cursor
+	auto load_dy = [&](int stage, int k) {
+		const float* dyb = dy + (((int64_t)ld_n * g.Cout + co0 + 16 * k) * g.H + ld_ho) * g.W + ld_strip * P::TW;
+		async_load16_masked(dy_mask[k], smem_addr + stage * P::DY_BYTES + (4 * wave + k) * 1024, dyb, dy_voff);
+	};
+	// piece i of input row y (of the cursor's image and strip; -1 and H are the padding rows) into ring slot seq % 8
+	auto load_row = [&](int y, int seq, int i) {
+		const int w0 = ld_strip * P::TW;
+		const float* xrow = x + (((int64_t)ld_n * g.Cin + ci0) * g.H + y) * g.W + w0 - 4;  // may lie before x: such lanes are masked
+		const bool no_row = y < 0 || y >= g.H;
+		const uint64_t outside = no_row ? r_exists[i] : ((w0 == 0 ? r_left[i] : 0) | (w0 + P::TW >= g.W ? r_right[i] : 0));
+		const uint32_t slot = smem_addr + P::RING0 + (seq & (P::RING - 1)) * P::ROW_BYTES + (wave + 4 * i) * 1024;
+		async_load16_masked(r_exists[i] & ~outside, slot, xrow, r_voff[i]);
 		lds_zero16_masked(outside, slot + lane16, zero4);
 	};
-	constexpr int PIECES = P::DPW + P::PPW;
+	constexpr int PIECES = P::DPW + P::RPW;
 
-	// ---- zeros everywhere once, then the first chunk
-	for (int i = tid; i < 2 * P::STAGE / 16; i += 256) reinterpret_cast<float4*>(smem)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-	__syncthreads();
+	// ---- the first chunk: its dy tile and all three rows
+	int top_cur = 0, newest = 2;  // ring sequence numbers: of the current chunk's first row, of the last row fetched
 	if (begin < end) {
 #pragma unroll
-		for (int k = 0; k < PIECES; k++) load_piece(0, k);
-		next_chunk();
+		for (int k = 0; k < P::DPW; k++) load_dy(0, k);
+#pragma unroll
+		for (int r = 0; r < 3; r++)
+#pragma unroll
+			for (int i = 0; i < P::RPW; i++) load_row(ld_ho - 1 + r, r, i);
+		advance();
 	}
 
 	v16f acc[P::TAPS];
@@ -143,21 +137,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
 		for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
 
-	// operand addresses: a per-lane base plus immediates
+	// operand addresses: a per-lane base plus immediates (the patch rows: plus the ring slot of each tap row)
 	const int off_a = ((phalf * 8 + mt * 2 + (lrow >> 4)) * 1024) + (lrow & 15) * 16 + half * 4;
-	const int off_b = P::DY_BYTES + (lrow * P::CS + phalf * (P::TW / 2) + half + 3) * 4;
+	const int off_b = P::RING0 + (lrow * P::CS + phalf * (P::TW / 2) + half + 3) * 4;
 
 	wait_vmcnt_lgkm0<0>();
 	__syncthreads();
 
-	// MORE: a chunk follows (at (n_c, ho_c, w0_c)), whose loads go out behind the first MFMAs into the other stage
+	// MORE: a chunk follows (under the cursor), whose loads go out behind the first MFMAs
 	auto run_chunk = [&](int cur, auto more_tag) {
 		constexpr bool MORE = decltype(more_tag)::value;
-		const uint8_t* sa = smem + cur * P::STAGE + off_a;
-		const uint8_t* sb = smem + cur * P::STAGE + off_b;
+		int top_next = top_cur + 1;
+		if (MORE) {
+			if (ld_ho == 0) {
+				// first row of a strip: nothing of it is in the ring yet.  Two rows now, the third with the others below.
+				top_next = newest + 1;
+#pragma unroll
+				for (int r = 0; r < 2; r++)
+#pragma unroll
+					for (int i = 0; i < P::RPW; i++) load_row(r - 1, top_next + r, i);
+				newest += 2;
+			}
+			newest++;
+		}
+		const uint8_t* sa = smem + cur * P::DY_BYTES + off_a;
+		const uint8_t* sb[3];
+#pragma unroll
+		for (int r = 0; r < 3; r++) sb[r] = smem + off_b + ((top_cur + r) & (P::RING - 1)) * P::ROW_BYTES;
 		float fa[2], fb[2][P::TAPS];
 		auto read_a = [&](int s) { fa[s & 1] = *reinterpret_cast<const float*>(sa + (s / 8) * 4096 + ((s / 2) % 4) * 256 + (s % 2) * 8); };
-		auto read_b = [&](int s, int t) { fb[s & 1][t] = *reinterpret_cast<const float*>(sb + ((t / 3) * P::PWS + (t % 3) + 2 * s) * 4); };
+		auto read_b = [&](int s, int t) { fb[s & 1][t] = *reinterpret_cast<const float*>(sb[t / 3] + ((t % 3) + 2 * s) * 4); };
 		read_a(0);
 #pragma unroll
 		for (int t = 0; t < P::TAPS; t++) read_b(0, t);
@@ -171,11 +180,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 					read_b(s + 1, t);
 				}
 				const int k = s * P::TAPS + t;
-				if (MORE && k < PIECES) load_piece(cur ^ 1, k);
+				if (MORE && k < P::DPW) load_dy(cur ^ 1, k);
+				if (MORE && k >= P::DPW && k < PIECES) load_row(ld_ho + 1, newest, k - P::DPW);
 				__builtin_amdgcn_sched_barrier(0);
 			}
 		}
-		if (MORE) next_chunk();
+		if (MORE) advance();
+		top_cur = top_next;
 		wait_vmcnt_lgkm0<0>();  // own loads of the next chunk have landed, own reads of this one are done
 		__syncthreads();
 	};
@@ -186,26 +197,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 	}
 	if (begin < end) run_chunk(cur, std::false_type{});
 
-	// pixel half 1 hands its sums to pixel half 0 of the same row tile, TAPS_PER_ROUND taps at a time
+	// pixel half 1 hands its sums to pixel half 0 of the same row tile
 	float* lds = reinterpret_cast<float*>(smem);
+	if (phalf == 1) {
 #pragma unroll
-	for (int t0 = 0; t0 < P::TAPS; t0 += P::TAPS_PER_ROUND) {
-		if (phalf == 1) {
+		for (int t = 0; t < P::TAPS; t++)
 #pragma unroll
-			for (int t = t0; t < t0 + P::TAPS_PER_ROUND && t < P::TAPS; t++)
-#pragma unroll
-				for (int r = 0; r < 16; r++) lds[((mt * P::TAPS_PER_ROUND + (t - t0)) * 16 + r) * 64 + lane] = acc[t][r];
-		}
-		__syncthreads();
-		if (phalf == 0) {
-#pragma unroll
-			for (int t = t0; t < t0 + P::TAPS_PER_ROUND && t < P::TAPS; t++)
-#pragma unroll
-				for (int r = 0; r < 16; r++) acc[t][r] += lds[((mt * P::TAPS_PER_ROUND + (t - t0)) * 16 + r) * 64 + lane];
-		}
-		__syncthreads();
+			for (int r = 0; r < 16; r++) lds[((mt * P::TAPS + t) * 16 + r) * 64 + lane] = acc[t][r];
 	}
+	__syncthreads();
 	if (phalf != 0) return;
+#pragma unroll
+	for (int t = 0; t < P::TAPS; t++)
+#pragma unroll
+		for (int r = 0; r < 16; r++) acc[t][r] += lds[((mt * P::TAPS + t) * 16 + r) * 64 + lane];
 
 	const int Kc = g.Cin * P::TAPS;
 	float* out = partial + (int64_t)blockIdx.x * g.Cout * Kc;
