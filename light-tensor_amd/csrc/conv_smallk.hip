@@ -20,6 +20,8 @@ namespace lten_hip {
 
 namespace {
 
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 constexpr int SK_TW = 128;       // pixels per chunk
 constexpr int SK_MAXK = 32;      // taps: one MFMA tile dimension
 constexpr int SK_MAXKW = 9;      // widest kernel row the patch row has room for
@@ -220,8 +222,13 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 	constexpr int DLD = 36, DSLAB = 32 * DLD;  // dy slab of a wavefront: [32 channels][32 pixels], rows of 36 floats
 	constexpr int USED = WPG * 2 * S::PATCH + WPG * DSLAB;
 	constexpr int STRIDE = WPG / 4;            // chunks between two of a wavefront's
+	// At most 16 taps (a first layer with one input channel): 16x16x4 MFMA tiles, columns = taps, two row tiles of 16
+	// channels, four pixels per step (lane l: tap or channel l % 16, pixel l / 16 of the step).  Half the matrix-pipe
+	// time of the 32x32x2 tile, whose columns 16-31 would be padding.
+	constexpr bool M16 = VEC && RC <= 8;
 	__shared__ __attribute__((aligned(16))) float s_mem[USED > RED ? USED : RED];
 	const int tid = threadIdx.x, lane = tid & 63, wid = tid >> 6, lrow = lane & 31, half = lane >> 5;
+	const int l16 = lane & 15, kq = lane >> 4;
 	const int wave = wid & 3;  // which 32 pixels of a chunk
 	const int K = g.Cin * g.kh * g.kw;
 	const int co0 = blockIdx.y * 32, co = co0 + lrow;
@@ -232,7 +239,7 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 	float* const dslab = s_mem + WPG * 2 * S::PATCH + wid * DSLAB;
 	const int r8 = lane >> 3, c4 = (lane & 7) * 4;     // whole-line loads: lane -> (row within a group of 8, 4 pixels)
 
-	const int boff = (lrow < K ? tap_offset(g, lrow) : 0) + 4 * half + 4 - g.pw;
+	const int boff = M16 ? (l16 < K ? tap_offset(g, l16) : 0) + 4 * kq + 4 - g.pw : (lrow < K ? tap_offset(g, lrow) : 0) + 4 * half + 4 - g.pw;
 	// dy: the address is a part all lanes share plus this lane's offset; with VEC (Wo % 4 == 0) the four
 	// pixels of a load are inside or outside the row together
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
@@ -262,14 +269,18 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 #pragma unroll
 		for (int i = 0; i < 4; i++) *reinterpret_cast<float4*>(dslab + (8 * i + r8) * DLD + c4) = v[i];
 	};
+	// M16: a[2 ct + h] = channel 16 ct + l16, pixels 16 h + 4 kq .. + 3
 	auto operand_dy = [&](float4 (&a)[4]) {
 #pragma unroll
-		for (int u = 0; u < 4; u++) a[u] = *reinterpret_cast<const float4*>(dslab + lrow * DLD + 8 * u + 4 * half);
+		for (int u = 0; u < 4; u++)
+			a[u] = M16 ? *reinterpret_cast<const float4*>(dslab + (16 * (u >> 1) + l16) * DLD + 16 * (u & 1) + 4 * kq)
+			           : *reinterpret_cast<const float4*>(dslab + lrow * DLD + 8 * u + 4 * half);
 	};
 
 	v16f acc;
 #pragma unroll
 	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	v4f acc16[2] = { { 0.0f, 0.0f, 0.0f, 0.0f }, { 0.0f, 0.0f, 0.0f, 0.0f } };
 
 	float4 a_cur[4], a_next[4];
 	PatchLane<S::P_PER_T> pr;
@@ -291,6 +302,19 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 		}
 		if (VEC) operand_dy(a_cur);  // the slab is free again once these reads are issued (one wavefront, in order)
 		const float* pb = mine + cur * S::PATCH + boff;
+		if constexpr (M16) {
+#pragma unroll
+			for (int h = 0; h < 2; h++) {
+				const float b0 = pb[16 * h + 0], b1 = pb[16 * h + 1], b2 = pb[16 * h + 2], b3 = pb[16 * h + 3];
+#pragma unroll
+				for (int ct = 0; ct < 2; ct++) {
+					acc16[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[2 * ct + h].x, b0, acc16[ct], 0, 0, 0);
+					acc16[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[2 * ct + h].y, b1, acc16[ct], 0, 0, 0);
+					acc16[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[2 * ct + h].z, b2, acc16[ct], 0, 0, 0);
+					acc16[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_cur[2 * ct + h].w, b3, acc16[ct], 0, 0, 0);
+				}
+			}
+		} else
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
 			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a_cur[u].x, pb[8 * u + 0], acc, 0, 0, 0);
@@ -308,16 +332,34 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 		}
 	}
 
-	// add the four wavefronts' tiles in wavefront order, then lanes whose column is a tap store
+	// add the wavefronts' tiles in wavefront order, then lanes whose column is a tap store
 	float* red = s_mem;
 	__syncthreads();  // every wavefront is done with its patch buffers
+	float* out = partial + (int64_t)blockIdx.x * g.Cout * K;
+	if constexpr (M16) {
+		// register r of tile ct in lane (l16, kq): channel 16 ct + 4 kq + r, tap l16
+		if (wid != 0) {
+#pragma unroll
+			for (int r = 0; r < 8; r++) red[((wid - 1) * 8 + r) * 64 + lane] = acc16[r >> 2][r & 3];
+		}
+		__syncthreads();
+		if (wid != 0 || l16 >= K) return;
+#pragma unroll
+		for (int r = 0; r < 8; r++) {
+			float v = acc16[r >> 2][r & 3];
+#pragma unroll
+			for (int q = 0; q < WPG - 1; q++) v += red[(q * 8 + r) * 64 + lane];
+			const int row = co0 + 16 * (r >> 2) + 4 * kq + (r & 3);
+			if (row < g.Cout) out[(int64_t)row * K + l16] = v;
+		}
+		return;
+	}
 	if (wid != 0) {
 #pragma unroll
 		for (int r = 0; r < 16; r++) red[((wid - 1) * 16 + r) * 64 + lane] = acc[r];
 	}
 	__syncthreads();
 	if (wid != 0 || lrow >= K) return;
-	float* out = partial + (int64_t)blockIdx.x * g.Cout * K;
 #pragma unroll
 	for (int r = 0; r < 16; r++) {
 		float v = acc[r];
