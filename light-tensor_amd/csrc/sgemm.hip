@@ -629,7 +629,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// rows one workgroup per block of 32 rows as well (the weights then come from the L2 for all but the first), while
 	// that gives at most a few workgroups per CU: 128 rows against a 1024-wide layer are 256 tiles of 32 x 16 where the
 	// 32 x 32 tiles of the general small-GEMM kernels would occupy half of the CUs.
-	if (force == 0 && !tA && tB && N >= 512 && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
+	// A classifier head (a few output columns) takes the same kernel: one column block, K cut over eight wavefronts.
+	if (force == 0 && !tA && tB && (N >= 512 || N <= 32) && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
 	    (M <= 32 || ceil_div(M, 32) * ceil_div(N, 16) <= 1024)) {
 		set_kernel_name(M <= 16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
 		if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }

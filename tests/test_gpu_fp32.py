@@ -95,7 +95,7 @@ def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
             assert np.array_equal(gpu_sgemm(gpu, 0, 0, M, N, K, 1.0, A, K, B, N, 0.0, z, N, tile=tile), first)
         want = A.astype(np.float64) @ B.astype(np.float64)
         assert rel_err(first, want) < TOL
-        for (tA, tB, m, n, k) in [(0, 0, 70, 100, 532), (0, 1, 33, 31, 788), (1, 0, 100, 36, 660), (1, 1, 20, 65, 596)]:
+        for (tA, tB, m, n, k) in [(0, 0, 70, 100, 532), (0, 1, 33, 47, 788), (1, 0, 100, 36, 660), (1, 1, 20, 65, 596)]:
             a = rng.standard_normal((k, m) if tA else (m, k)).astype(np.float32)
             b = rng.standard_normal((n, k) if tB else (k, n)).astype(np.float32)
             c0 = rng.standard_normal((m, n)).astype(np.float32)
@@ -103,6 +103,20 @@ def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
             assert gpu.last_kernel().startswith(name), gpu.last_kernel()
             opa, opb = (a.T if tA else a).astype(np.float64), (b.T if tB else b).astype(np.float64)
             assert rel_err(got, 0.5 * opa @ opb + 2.0 * c0) < TOL, (tA, tB, m, n, k)
+
+
+def test_classifier_head_on_the_weight_streaming_kernel(gpu):
+    """NT products with at most 32 output columns (a classifier head: 128 x 10 x 1024) run on the 16-column
+    weight-streaming kernel: ragged column block, ragged rows, alpha and beta, repeatable bit for bit."""
+    rng = np.random.default_rng(21)
+    for (m, n, k) in [(128, 10, 1024), (33, 31, 788), (200, 16, 256), (5, 1, 512)]:
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((n, k)).astype(np.float32)
+        c0 = rng.standard_normal((m, n)).astype(np.float32)
+        got = gpu_sgemm(gpu, 0, 1, m, n, k, 0.5, a, k, b, k, 2.0, c0, n)
+        assert gpu.last_kernel().startswith("sgemm_skinny_nt"), gpu.last_kernel()
+        assert np.array_equal(got, gpu_sgemm(gpu, 0, 1, m, n, k, 0.5, a, k, b, k, 2.0, c0, n))
+        assert rel_err(got, 0.5 * a.astype(np.float64) @ b.astype(np.float64).T + 2.0 * c0) < TOL, (m, n, k)
 
 
 def test_rank1_and_rowvec_shapes(gpu, ob):
