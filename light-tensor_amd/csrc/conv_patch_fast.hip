@@ -98,11 +98,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	for (int i = tid; i < 2 * P::STAGE / 16; i += 256) reinterpret_cast<float4*>(smem)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 	__syncthreads();
 
-#if defined(LTEN_CONV_EXP) && LTEN_CONV_EXP == 2
-	const int KT = g.Cin / P::CB / 2;
-#else
 	const int KT = g.Cin / P::CB;
-#endif
 #pragma unroll
 	for (int i = 0; i < P::LPW; i++) load_one(i, 0, 0);
 	if (KT > 1) {
@@ -179,9 +175,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	inner_beats(stage);
 	beat(fa1, fb1, fa0, fb0, stage, 0, false, false, 0, 0);
 
-#ifdef LTEN_CONV_EXP  // tuning builds only (results are wrong): 1 = no stores, 2 = half the chunks
-	if (LTEN_CONV_EXP == 1 && acc[0][0][0] != 12345.678f) return;
-#endif
 	// Epilogue: all bias values first, then stores whose address is a shared part plus a lane offset.
 	const int ho = h0 + wrow;
 	if (ho >= g.Ho) return;
