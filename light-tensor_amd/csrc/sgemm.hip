@@ -380,17 +380,30 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_shortk_kernel(SPro
 // of the next UB batches are in flight while the current UB are multiplied.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int MB>
-__global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
+// BT: B is [N x K] (the NT product above); otherwise B is [K x N], rows contiguous in n (the NN product, the data
+// gradient dX = dY W of a FullyConnected layer): a wave-wide 16-byte load then covers 16 k-rows x 64 bytes of the
+// column block, the slab holds [32 k][16 n] and the operand is read one float per MFMA (lane (n, q): k = 16h + 4q + t).
+template <int MB, bool BT>
+struct SkinnyShape {
+	static constexpr int WAVES = 8, LD = 36, LDB = 20;
+	static constexpr int A_SLAB = MB * 16 * LD, B_SLAB = BT ? 16 * LD : 32 * LDB;
+	static constexpr int SLABS = WAVES * (A_SLAB + B_SLAB), TILES = WAVES * MB * 256;
+	static constexpr int LDS_FLOATS = SLABS > TILES ? SLABS : TILES;
+};
+
+// col_block: which 16 columns, row_block: which MB * 16 rows; lds: SkinnyShape<MB, BT>::LDS_FLOATS floats
+template <int MB, bool BT>
+__device__ __forceinline__ void sgemm_skinny_body(const SProblem& p, int col_block, int row_block, float* lds)
 {
-	constexpr int WAVES = 8, UB = 2, LD = 36;
-	constexpr int A_SLAB = MB * 16 * LD, B_SLAB = 16 * LD;
-	__shared__ __attribute__((aligned(16))) float lds[WAVES * (A_SLAB + B_SLAB) > WAVES * MB * 256 ? WAVES * (A_SLAB + B_SLAB) : WAVES * MB * 256];
+	typedef SkinnyShape<MB, BT> S;
+	constexpr int WAVES = S::WAVES, UB = 2, LD = S::LD, LDB = S::LDB;
+	constexpr int A_SLAB = S::A_SLAB, B_SLAB = S::B_SLAB;
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int r16 = lane & 15, q4 = lane >> 4;
 	const int r8 = lane >> 3, c4 = (lane & 7) * 4;
-	const int n0 = blockIdx.x * 16;
-	const int mrow0 = blockIdx.y * (MB * 16);  // blockIdx.y: which block of MB * 16 activation rows
+	const int k16 = lane >> 2, n4 = (lane & 3) * 4;  // NN: this lane's k-row within 16 and its four columns
+	const int n0 = col_block * 16;
+	const int mrow0 = row_block * (MB * 16);
 	float* sA = lds + wave * (A_SLAB + B_SLAB);
 	float* sB = sA + A_SLAB;
 
@@ -412,19 +425,32 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 		}
 #pragma unroll
 		for (int i = 0; i < 2; i++) {
-			const int n = n0 + 8 * i + r8;
 			v.b[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (n < p.N && k < p.K) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)n * p.ldb + k);
+			if (BT) {
+				const int n = n0 + 8 * i + r8;
+				if (n < p.N && k < p.K) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)n * p.ldb + k);
+			} else {  // N % 4 == 0: the four columns are inside N or outside together
+				const int kb = batch * 32 + 16 * i + k16;
+				if (kb < p.K && n0 + n4 < p.N) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)kb * p.ldb + n0 + n4);
+			}
 		}
 	};
 	auto multiply = [&](const Batch& v) {
 #pragma unroll
 		for (int i = 0; i < 2 * MB; i++) *reinterpret_cast<float4*>(sA + (8 * i + r8) * LD + c4) = v.a[i];
 #pragma unroll
-		for (int i = 0; i < 2; i++) *reinterpret_cast<float4*>(sB + (8 * i + r8) * LD + c4) = v.b[i];
+		for (int i = 0; i < 2; i++) {
+			if (BT) *reinterpret_cast<float4*>(sB + (8 * i + r8) * LD + c4) = v.b[i];
+			else *reinterpret_cast<float4*>(sB + (16 * i + k16) * LDB + n4) = v.b[i];
+		}
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
-			const float4 fb = *reinterpret_cast<const float4*>(sB + r16 * LD + 16 * h + 4 * q4);
+			float4 fb;
+			if (BT) fb = *reinterpret_cast<const float4*>(sB + r16 * LD + 16 * h + 4 * q4);
+			else {
+				const float* col = sB + (16 * h + 4 * q4) * LDB + r16;
+				fb = make_float4(col[0], col[LDB], col[2 * LDB], col[3 * LDB]);
+			}
 #pragma unroll
 			for (int b = 0; b < MB; b++) {
 				const float4 fa = *reinterpret_cast<const float4*>(sA + (16 * b + r16) * LD + 16 * h + 4 * q4);
@@ -474,6 +500,20 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 		if (p.bias) out += p.bias[n0 + col];
 		sgemm_store(p, c, out);
 	}
+}
+
+template <int MB>
+__global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
+{
+	__shared__ __attribute__((aligned(16))) float lds[SkinnyShape<MB, true>::LDS_FLOATS];
+	sgemm_skinny_body<MB, true>(p, blockIdx.x, blockIdx.y, lds);
+}
+
+template <int MB>
+__global__ __launch_bounds__(512) void sgemm_skinny_nn_kernel(SProblem p)
+{
+	__shared__ __attribute__((aligned(16))) float lds[SkinnyShape<MB, false>::LDS_FLOATS];
+	sgemm_skinny_body<MB, false>(p, blockIdx.x, blockIdx.y, lds);
 }
 
 // Both operands allow 16-byte loads along their contiguous dimension.
@@ -637,6 +677,15 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(M <= 16 ? 1 : ceil_div(M, 32)));
 		if (M <= 16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
 		else sgemm_skinny_nt_kernel<2><<<grid, dim3(512), 0, stream()>>>(p);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+	// The NN product with few rows (the data gradient of such a layer) on the same tiles.
+	if (force == 0 && !tA && !tB && N >= 512 && N % 4 == 0 && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) && M > 16 &&
+	    ceil_div(M, 32) * ceil_div(N, 16) <= 1024) {
+		set_kernel_name("sgemm_skinny_nn_32x16");
+		if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
+		sgemm_skinny_nn_kernel<2><<<dim3((unsigned)ceil_div(N, 16), (unsigned)ceil_div(M, 32)), dim3(512), 0, stream()>>>(p);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}

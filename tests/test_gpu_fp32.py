@@ -79,7 +79,7 @@ def test_cfg2_gemm_shapes_all_layouts(gpu, ob, shape):
         assert err < TOL
 
 
-@pytest.mark.parametrize("tile,name", [(0, "sgemm_staged"), (5, "sgemm_direct")])
+@pytest.mark.parametrize("tile,name", [(4, "sgemm_staged"), (5, "sgemm_direct")])
 def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
     """The small-output kernels (LDS-staged and direct operand loads) add their wavefronts' partial tiles in wavefront
     order: bitwise equal results run after run; all layouts, ragged M / N / K, beta, batches."""
@@ -117,6 +117,21 @@ def test_classifier_head_on_the_weight_streaming_kernel(gpu):
         assert gpu.last_kernel().startswith("sgemm_skinny_nt"), gpu.last_kernel()
         assert np.array_equal(got, gpu_sgemm(gpu, 0, 1, m, n, k, 0.5, a, k, b, k, 2.0, c0, n))
         assert rel_err(got, 0.5 * a.astype(np.float64) @ b.astype(np.float64).T + 2.0 * c0) < TOL, (m, n, k)
+
+
+def test_data_gradient_on_the_weight_streaming_kernel(gpu):
+    """NN products with few rows against a wide weight matrix (dX = dY W of a FullyConnected layer at batch 128) run
+    on the 16-column weight-streaming tiles with the weights read along n: ragged row blocks, a ragged last column
+    block, K that is no multiple of 32, alpha and beta, repeatable bit for bit."""
+    rng = np.random.default_rng(22)
+    for (m, n, k) in [(128, 1024, 1024), (128, 784, 1024), (40, 520, 260), (17, 512, 1000)]:
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        b = rng.standard_normal((k, n)).astype(np.float32)
+        c0 = rng.standard_normal((m, n)).astype(np.float32)
+        got = gpu_sgemm(gpu, 0, 0, m, n, k, 0.5, a, k, b, n, 2.0, c0, n)
+        assert gpu.last_kernel().startswith("sgemm_skinny_nn"), gpu.last_kernel()
+        assert np.array_equal(got, gpu_sgemm(gpu, 0, 0, m, n, k, 0.5, a, k, b, n, 2.0, c0, n))
+        assert rel_err(got, 0.5 * a.astype(np.float64) @ b.astype(np.float64) + 2.0 * c0) < TOL, (m, n, k)
 
 
 def test_rank1_and_rowvec_shapes(gpu, ob):
