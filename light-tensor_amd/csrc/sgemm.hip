@@ -362,12 +362,91 @@ __device__ __forceinline__ void sgemm_tn_wave_tile(const SProblem& p, int tile)
 	}
 }
 
-// The same pair with the weight gradient on sgemm_tn_wave_tile: eight of its tiles per workgroup.
+// The same tile with whole cache lines per load: a wave-wide 16-byte load covers 8 k-rows x 128 bytes of an operand (the
+// loads above fetch 4 bytes per lane, two rows of 128 bytes per instruction: eight times as many instructions for the
+// memory pipeline), the values pass through a wavefront-private LDS slab ([32 k][36] floats per operand; no barrier: LDS
+// operations of one wavefront complete in order) and come back one float per MFMA in its lane layout.  The next batch
+// of 32 k is in flight while the current one is multiplied.  Needs M % 4 == 0, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0
+// and 16-byte aligned operands.  `slab`: 2 * 32 * 36 floats of this wavefront.
+__device__ __forceinline__ void sgemm_tn_wave_tile_lines(const SProblem& p, int tile, float* slab)
+{
+	constexpr int LD = 36;
+	const int lane = threadIdx.x & 63, lrow = lane & 31, g = lane >> 5;
+	const int kr = lane >> 3, c4 = (lane & 7) * 4;
+	const int tiles_n = (p.N + 31) / 32;
+	const int m0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+	if (m0 >= p.M) return;
+	const bool a_ok = m0 + c4 < p.M, b_ok = n0 + c4 < p.N;
+	const float* a_src = p.A + m0 + c4;
+	const float* b_src = p.B + n0 + c4;
+	float* sA = slab;
+	float* sB = slab + 32 * LD;
+	struct Batch {
+		float4 a[4], b[4];
+	};
+	auto fetch = [&](int kb, Batch& v) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int k = kb + 8 * i + kr;
+			v.a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			v.b[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (k < p.K) {
+				if (a_ok) v.a[i] = *reinterpret_cast<const float4*>(a_src + (int64_t)k * p.lda);
+				if (b_ok) v.b[i] = *reinterpret_cast<const float4*>(b_src + (int64_t)k * p.ldb);
+			}
+		}
+	};
+	v16f acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	float asum = 0.0f;
+	Batch cur, nxt;
+	fetch(0, cur);
+	for (int kb = 0; kb < p.K; kb += 32) {
+		if (kb + 32 < p.K) fetch(kb + 32, nxt);
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			*reinterpret_cast<float4*>(sA + (8 * i + kr) * LD + c4) = cur.a[i];
+			*reinterpret_cast<float4*>(sB + (8 * i + kr) * LD + c4) = cur.b[i];
+		}
+#pragma unroll
+		for (int s = 0; s < 16; s++) {
+			const float fa = sA[(2 * s + g) * LD + lrow], fb = sB[(2 * s + g) * LD + lrow];
+			asum += fa;
+			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
+		}
+		cur = nxt;
+	}
+	const int m = m0 + lrow, n = n0 + lrow;
+	// register 4q + e of lane (lrow, g): row 8q + 4g + e, column lrow
+	if (n < p.N) {
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int row = m0 + (r >> 2) * 8 + g * 4 + (r & 3);
+			if (row >= p.M) continue;
+			float* c = p.C + (int64_t)row * p.ldc + n;
+			float out = p.alpha * acc[r];
+			if (p.beta != 0.0f) out += p.beta * *c;
+			sgemm_store(p, c, out);
+		}
+	}
+	if (p.rowsum != nullptr && n0 == 0) {
+		const float sum = asum + __shfl_xor(asum, 32, 64);
+		if (g == 0 && m < p.M) p.rowsum[m] += sum;
+	}
+}
+
+// The same pair with the weight gradient on whole-K tiles per wavefront: eight of its tiles per workgroup.  LINES: the
+// weight gradient's operands allow whole-line loads.
+template <bool LINES>
 __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_shortk_kernel(SProblem px, SProblem pw, int blocks_x)
 {
-	__shared__ float part[8][32 * 32];
-	if ((int)blockIdx.x < blocks_x) sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, part);
-	else sgemm_tn_wave_tile(pw, ((int)blockIdx.x - blocks_x) * 8 + (int)(threadIdx.x >> 6));
+	constexpr int SLAB = 2 * 32 * 36;
+	__shared__ __attribute__((aligned(16))) float lds[LINES ? 8 * SLAB : 8 * 32 * 32];
+	const int wave = (int)(threadIdx.x >> 6);
+	if ((int)blockIdx.x < blocks_x) sgemm_direct_body<8, false, false>(px, blockIdx.x, 0, reinterpret_cast<float (*)[32 * 32]>(lds));
+	else if (LINES) sgemm_tn_wave_tile_lines(pw, ((int)blockIdx.x - blocks_x) * 8 + wave, lds + wave * SLAB);
+	else sgemm_tn_wave_tile(pw, ((int)blockIdx.x - blocks_x) * 8 + wave);
 }
 
 // FullyConnected forward at small batch sizes: C[M x N] = A[M x K] B[N x K]^T with M <= 32, a stream over the
@@ -803,7 +882,9 @@ static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, co
 		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
 			if (M <= 256 && blocks_w >= 256 && pair_opt == 0) {  // a short reduction and many tiles for dW: whole-K tiles per wavefront
 				set_kernel_name("sgemm_fc_backward_pair_32x32_shortk");
-				sgemm_fc_backward_pair_shortk_kernel<<<dim3((unsigned)(blocks_x + ceil_div(blocks_w, 8))), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
+				const dim3 grid((unsigned)(blocks_x + ceil_div(blocks_w, 8)));
+				if (operands_vec(pw) && out % 4 == 0 && in % 4 == 0) sgemm_fc_backward_pair_shortk_kernel<true><<<grid, dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
+				else sgemm_fc_backward_pair_shortk_kernel<false><<<grid, dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
 			} else {
 				set_kernel_name("sgemm_fc_backward_pair_32x32_w8");
 				sgemm_fc_backward_pair_kernel<<<dim3((unsigned)(blocks_x + blocks_w)), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);
