@@ -403,7 +403,7 @@ __device__ __forceinline__ void sgemm_tn_wave_tile_lines(const SProblem& p, int 
 	Batch cur, nxt;
 	fetch(0, cur);
 	for (int kb = 0; kb < p.K; kb += 32) {
-		if (kb + 32 < p.K) fetch(kb + 32, nxt);
+		fetch(kb + 32, nxt);  // rows past K read as zeros without a load
 #pragma unroll
 		for (int i = 0; i < 4; i++) {
 			*reinterpret_cast<float4*>(sA + (8 * i + kr) * LD + c4) = cur.a[i];
