@@ -127,7 +127,11 @@ def test_conv_layer_golden(gpu):
                                  # tiles, more than 32 output channels, 5x5 and 1x1 windows, pad 0 / 1 / 2
                                  (2, 1, 11, 200, 40, 3, 3, 1, 1, 1, 1), (3, 1, 9, 131, 7, 5, 5, 2, 2, 1, 1),
                                  (1, 20, 9, 132, 33, 1, 1, 0, 0, 1, 1), (2, 3, 16, 36, 64, 3, 3, 0, 0, 1, 1),
-                                 (5, 2, 7, 9, 3, 2, 7, 1, 4, 1, 1)])
+                                 (5, 2, 7, 9, 3, 2, 7, 1, 4, 1, 1),
+                                 # at most 16 taps with rows that allow 16-byte loads: the weight gradient on 16x16x4 MFMA
+                                 # tiles (12 taps of a 4x3 window, 15 taps of five channels with a 1x3 window; 33 and 40
+                                 # output channels: a ragged second block of 32)
+                                 (2, 1, 12, 64, 40, 4, 3, 1, 1, 1, 1), (2, 5, 9, 128, 33, 1, 3, 0, 1, 1, 1)])
 @pytest.mark.parametrize("variant", [0, 1, 2, 3, 5])
 def test_conv_vs_oracle(gpu, ob, geo, variant):
     """variant 0: the kernel the library picks; 1: the implicit-GEMM kernels for every shape; 2: the register-staged
