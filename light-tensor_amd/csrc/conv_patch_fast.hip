@@ -144,7 +144,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	};
 
 	float fa0[P::MT], fb0[P::NT], fa1[P::MT], fb1[P::NT];
-	wait_vmcnt_lgkm0<0>();
+	// Only the first chunk has to be there: every workgroup of the chip asks for its first two chunks at the same moment
+	// (38 MB at config 5's second layer), and waiting for both kept the matrix pipe idle twice as long.  Loads complete
+	// in order, so chunk 0 has landed once no more loads are out than were issued for chunk 1 (a load none of whose
+	// lanes takes part is not issued, hence the count).
+	int behind = 0;
+	if (KT > 1) {
+#pragma unroll
+		for (int i = 0; i < P::LPW; i++)
+			if (wave + 4 * i < P::LOADS && __ballot(valid[i]) != 0) behind++;
+	}
+	switch (behind) {
+	case 0: wait_vmcnt_lgkm0<0>(); break;
+	case 1: wait_vmcnt_lgkm0<1>(); break;
+	case 2: wait_vmcnt_lgkm0<2>(); break;
+	case 3: wait_vmcnt_lgkm0<3>(); break;
+	case 4: wait_vmcnt_lgkm0<4>(); break;
+	case 5: wait_vmcnt_lgkm0<5>(); break;
+	case 6: wait_vmcnt_lgkm0<6>(); break;
+	default: wait_vmcnt_lgkm0<0>(); break;
+	}
 	__syncthreads();
 #pragma unroll
 	for (int e = 0; e < P::NR; e++) read_one(fa0, fb0, smem, 0, e);
