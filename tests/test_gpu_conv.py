@@ -272,14 +272,15 @@ def test_conv_operands_aligned_to_four_bytes_only(gpu, ob, geo):
 
 
 def test_seeded_sweep_over_chunked_rows(gpu, ob):
-    """Twelve seeded 3x3, stride 1, pad 1 geometries whose rows are whole 64-pixel chunks (the shapes the
-    direct-to-LDS weight-gradient kernel takes), channel counts on both sides of its 64 x 32 blocks."""
+    """Sixteen seeded 3x3, stride 1, pad 1 geometries whose rows are whole 64-pixel chunks (the shapes the
+    direct-to-LDS weight-gradient kernel takes), channel counts on both sides of its 64 x 32 blocks, images of one row
+    up to 40 (a workgroup's run of chunks then starts anywhere in a 64-column strip and crosses strips and images)."""
     rng = np.random.default_rng(2718)
     seen = set()
-    for case in range(12):
+    for case in range(16):
         Cin = int(rng.choice([9, 16, 31, 32, 33, 48, 64, 70]))
         Cout = int(rng.choice([1, 16, 63, 64, 65, 100, 128]))
-        H, W = int(rng.integers(1, 9)), int(rng.choice([64, 64, 128, 192]))
+        H, W = int(rng.choice([1, 2, 3, 5, 8, 17, 40])), int(rng.choice([64, 64, 128, 192]))
         N = int(rng.integers(1, 4))
         _conv_vs_oracle(gpu, ob, (N, Cin, H, W, Cout, 3, 3, 1, 1, 1, 1))
         seen.add(gpu.last_kernel())
