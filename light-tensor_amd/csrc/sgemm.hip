@@ -595,6 +595,107 @@ __global__ __launch_bounds__(512) void sgemm_skinny_nn_kernel(SProblem p)
 	sgemm_skinny_body<MB, false>(p, blockIdx.x, blockIdx.y, lds);
 }
 
+// sgemm_tn_wave_tile_lines over k in [k_begin, k_end) only, the sums left in `acc` and `asum` (this lane's share of the
+// row sums of op(A)).
+__device__ __forceinline__ void sgemm_tn_tile_lines_partial(const SProblem& p, int tile, int k_begin, int k_end, float* slab, v16f& acc, float& asum)
+{
+	constexpr int LD = 36;
+	const int lane = threadIdx.x & 63, lrow = lane & 31, g = lane >> 5;
+	const int kr = lane >> 3, c4 = (lane & 7) * 4;
+	const int tiles_n = (p.N + 31) / 32;
+	const int m0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+	const bool a_ok = m0 + c4 < p.M, b_ok = n0 + c4 < p.N;
+	const float* a_src = p.A + m0 + c4;
+	const float* b_src = p.B + n0 + c4;
+	float* sA = slab;
+	float* sB = slab + 32 * LD;
+	struct Batch {
+		float4 a[4], b[4];
+	};
+	auto fetch = [&](int kb, Batch& v) {
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			const int k = kb + 8 * i + kr;
+			v.a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			v.b[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+			if (k < k_end) {
+				if (a_ok) v.a[i] = *reinterpret_cast<const float4*>(a_src + (int64_t)k * p.lda);
+				if (b_ok) v.b[i] = *reinterpret_cast<const float4*>(b_src + (int64_t)k * p.ldb);
+			}
+		}
+	};
+	Batch cur, nxt;
+	fetch(k_begin, cur);
+	for (int kb = k_begin; kb < k_end; kb += 32) {
+		fetch(kb + 32, nxt);  // rows past the range read as zeros without a load
+#pragma unroll
+		for (int i = 0; i < 4; i++) {
+			*reinterpret_cast<float4*>(sA + (8 * i + kr) * LD + c4) = cur.a[i];
+			*reinterpret_cast<float4*>(sB + (8 * i + kr) * LD + c4) = cur.b[i];
+		}
+#pragma unroll
+		for (int s = 0; s < 16; s++) {
+			const float fa = sA[(2 * s + g) * LD + lrow], fb = sB[(2 * s + g) * LD + lrow];
+			asum += fa;
+			acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, acc, 0, 0, 0);
+		}
+		cur = nxt;
+	}
+}
+
+// Both products of FullyConnected backward in one launch, each on as many workgroups as the chip has CUs: dW on the
+// whole-line tiles, four per workgroup (wavefront w multiplies tile w % 4 over half w / 4 of the batch; the halves are
+// added through LDS, the lower half first), dX on the weight-streaming tiles.  With 128 workgroups per product (eight
+// whole-K tiles of dW, or one 32 x 32 tile of dX, per workgroup) each product kept half of the CUs busy for 11-13 us.
+__global__ __launch_bounds__(512) void sgemm_fc_backward_pair_wide_kernel(SProblem px, SProblem pw, int blocks_w, int tiles_w, int cols_x)
+{
+	constexpr int SLAB = 2 * 32 * 36;
+	constexpr int FLOATS = SkinnyShape<2, false>::LDS_FLOATS > 8 * SLAB ? SkinnyShape<2, false>::LDS_FLOATS : 8 * SLAB;
+	static_assert(8 * SLAB >= 4 * 16 * 64 + 4 * 32, "the exchange of the halves fits the slabs");
+	__shared__ __attribute__((aligned(16))) float lds[FLOATS];
+	if ((int)blockIdx.x >= blocks_w) {
+		const int b = (int)blockIdx.x - blocks_w;
+		sgemm_skinny_body<2, false>(px, b % cols_x, b / cols_x, lds);
+		return;
+	}
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, g = lane >> 5;
+	const int slot = wave & 3, khalf = wave >> 2;
+	const int tile = (int)blockIdx.x * 4 + slot;
+	const bool active = tile < tiles_w;
+	const int k_mid = min(pw.K, (((pw.K + 1) / 2 + 31) / 32) * 32);  // whole batches of 32 k in the lower half
+	v16f acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+	float asum = 0.0f;
+	if (active) sgemm_tn_tile_lines_partial(pw, tile, khalf ? k_mid : 0, khalf ? pw.K : k_mid, lds + wave * SLAB, acc, asum);
+	asum += __shfl_xor(asum, 32, 64);
+	float* sums = lds + 4 * 16 * 64;
+	__syncthreads();  // the slabs are no longer read
+	if (khalf == 1) {
+#pragma unroll
+		for (int r = 0; r < 16; r++) lds[(slot * 16 + r) * 64 + lane] = acc[r];
+		if (g == 0) sums[slot * 32 + lrow] = asum;
+	}
+	__syncthreads();
+	if (khalf != 0 || !active) return;
+	const int tiles_n = (pw.N + 31) / 32;
+	const int m0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
+	const int n = n0 + lrow;
+	if (n < pw.N) {
+		// register 4q + e of lane (lrow, g): row 8q + 4g + e, column lrow
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int row = m0 + (r >> 2) * 8 + g * 4 + (r & 3);
+			if (row >= pw.M) continue;
+			float* c = pw.C + (int64_t)row * pw.ldc + n;
+			float out = pw.alpha * (acc[r] + lds[(slot * 16 + r) * 64 + lane]);
+			if (pw.beta != 0.0f) out += pw.beta * *c;
+			sgemm_store(pw, c, out);
+		}
+	}
+	if (pw.rowsum != nullptr && n0 == 0 && g == 0 && m0 + lrow < pw.M) pw.rowsum[m0 + lrow] += asum + sums[slot * 32 + lrow];
+}
+
 // Both operands allow 16-byte loads along their contiguous dimension.
 static bool operands_vec(const SProblem& p)
 {
@@ -880,7 +981,12 @@ static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, co
 		pw.rowsum = db;
 		const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
 		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
-			if (M <= 256 && blocks_w >= 256 && pair_opt == 0) {  // a short reduction and many tiles for dW: whole-K tiles per wavefront
+			const uint64_t cols_x = ceil_div(in, 16), skinny_x = cols_x * ceil_div(M, 32), w4 = ceil_div(blocks_w, 4);
+			if (pair_opt == 0 && M > 16 && M <= 256 && blocks_w >= 256 && in >= 512 && in % 4 == 0 && out >= 256 && out % 4 == 0 &&
+			    operands_vec(px) && operands_vec(pw) && skinny_x <= 1024) {
+				set_kernel_name("sgemm_fc_backward_pair_wide");
+				sgemm_fc_backward_pair_wide_kernel<<<dim3((unsigned)(w4 + skinny_x)), dim3(512), 0, stream()>>>(px, pw, (int)w4, (int)blocks_w, (int)cols_x);
+			} else if (M <= 256 && blocks_w >= 256 && pair_opt == 0) {  // a short reduction and many tiles for dW: whole-K tiles per wavefront
 				set_kernel_name("sgemm_fc_backward_pair_32x32_shortk");
 				const dim3 grid((unsigned)(blocks_x + ceil_div(blocks_w, 8)));
 				if (operands_vec(pw) && out % 4 == 0 && in % 4 == 0) sgemm_fc_backward_pair_shortk_kernel<true><<<grid, dim3(512), 0, stream()>>>(px, pw, (int)blocks_x);

@@ -224,7 +224,9 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     (100, 530, 490, ("sgemm_fc_backward_pair_32x32_shortk",)),       # many weight-gradient tiles, short K: a whole-K tile per wavefront, ragged
     (300, 600, 500, ("sgemm_fc_backward_pair_32x32_w8",)),           # batch above 256: the weight gradient cuts K over the wavefronts
     (777, 96, 132, ("sgemm_staged_32x32_w8",)),                      # batch >= 512: two launches, dW with whole-line loads, ragged K
-    (128, 784, 1024, ("sgemm_fc_backward_pair_32x32_shortk",)),      # config 2, layer 1
+    (128, 784, 1024, ("sgemm_fc_backward_pair_wide",)),              # config 2, layer 1: both products on 16-byte loads, each on a workgroup per CU
+    (100, 1024, 516, ("sgemm_fc_backward_pair_wide",)),              # the same with a ragged batch (two halves of 64 and 36 rows) and ragged tiles
+    (128, 786, 1024, ("sgemm_fc_backward_pair_32x32_shortk",)),      # rows of X that allow no 16-byte loads: whole-K tiles from dword loads
     (511, 64, 2048, ("sgemm_fc_backward_pair_32x32_w8",)),           # the largest batch and width the paired launch takes
     (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
