@@ -852,10 +852,12 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// A classifier head (a few output columns) takes the same kernel: one column block, K cut over eight wavefronts.
 	if (force == 0 && !tA && tB && (N >= 512 || N <= 32) && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
 	    (M <= 32 || ceil_div(M, 32) * ceil_div(N, 16) <= 1024)) {
-		set_kernel_name(M <= 16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
+		// few column blocks (a classifier head): blocks of 16 rows, twice the workgroups
+		const bool rows16 = M <= 16 || ceil_div(N, 16) * ceil_div(M, 32) < 64;
+		set_kernel_name(rows16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
 		if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
-		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(M <= 16 ? 1 : ceil_div(M, 32)));
-		if (M <= 16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
+		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(rows16 ? ceil_div(M, 16) : ceil_div(M, 32)));
+		if (rows16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
 		else sgemm_skinny_nt_kernel<2><<<grid, dim3(512), 0, stream()>>>(p);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
