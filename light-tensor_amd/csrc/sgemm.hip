@@ -530,14 +530,18 @@ __device__ __forceinline__ void sgemm_skinny_body(const SProblem& p, int col_blo
 				const float* col = sB + (16 * h + 4 * q4) * LDB + r16;
 				fb = make_float4(col[0], col[LDB], col[2 * LDB], col[3 * LDB]);
 			}
+			// the row blocks take turns, so that consecutive MFMAs do not wait for each other's sums
+			float4 fa[MB];
 #pragma unroll
-			for (int b = 0; b < MB; b++) {
-				const float4 fa = *reinterpret_cast<const float4*>(sA + (16 * b + r16) * LD + 16 * h + 4 * q4);
-				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.x, fb.x, acc[b], 0, 0, 0);
-				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.y, fb.y, acc[b], 0, 0, 0);
-				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.z, fb.z, acc[b], 0, 0, 0);
-				acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa.w, fb.w, acc[b], 0, 0, 0);
-			}
+			for (int b = 0; b < MB; b++) fa[b] = *reinterpret_cast<const float4*>(sA + (16 * b + r16) * LD + 16 * h + 4 * q4);
+#pragma unroll
+			for (int b = 0; b < MB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[b].x, fb.x, acc[b], 0, 0, 0);
+#pragma unroll
+			for (int b = 0; b < MB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[b].y, fb.y, acc[b], 0, 0, 0);
+#pragma unroll
+			for (int b = 0; b < MB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[b].z, fb.z, acc[b], 0, 0, 0);
+#pragma unroll
+			for (int b = 0; b < MB; b++) acc[b] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[b].w, fb.w, acc[b], 0, 0, 0);
 		}
 	};
 
