@@ -56,7 +56,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 #pragma unroll
 		for (int r = 0; r < 16; r++) {
 			const int row = min(group * 16 + r, p.N - 1);
-			async_load16_masked(live, slab_addr + r * ROW, p.B + (int64_t)row * p.K + kbeg + pass * 1024, lane * 16);
+			async_load16_masked_nt(live, slab_addr + r * ROW, p.B + (int64_t)row * p.K + kbeg + pass * 1024, lane * 16);
 		}
 	};
 	// the activations of this wavefront's k-slice stay in registers for every row group the workgroup takes
