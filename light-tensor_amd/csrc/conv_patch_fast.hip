@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 			for (int r = 0; r < 16; r++) {
 				float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
 #pragma unroll
-				for (int t = 0; t < P::NT; t++) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
+				for (int t = 0; t < P::NT; t++) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * 32]);  // y is written once and not read here
 			}
 		return;
 	}
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 			float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
 #pragma unroll
 			for (int t = 0; t < P::NT; t++)
-				if (w0 + wcol + t * 32 + lrow < g.Wo) yr[y_lane + t * 32] = acc[m][t][r] + bv[m][r];
+				if (w0 + wcol + t * 32 + lrow < g.Wo) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * 32]);
 		}
 }
 
