@@ -222,7 +222,7 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 				for (int j = 0; j < FN; j++) {
 					float v = p.alpha * acc[i][j][r];
 					if (p.beta != 0.0f) v += p.beta * cr[c_lane + j * 32];
-					cr[c_lane + j * 32] = v + bv[j];
+					__builtin_nontemporal_store(v + bv[j], &cr[c_lane + j * 32]);  // C is written once and not read again here
 				}
 			}
 		return;
