@@ -27,15 +27,12 @@ __device__ __forceinline__ void async_load16_masked(uint64_t mask, uint32_t lds_
 	             : "=&s"(saved) : "s"(mask), "s"(lds_addr), "v"(voff), "s"(base) : "memory", "scc");
 }
 
-#ifndef LTEN_STREAM_HINT
-#define LTEN_STREAM_HINT "nt"
-#endif
 // The same with the non-temporal hint: for data that is read once (a weight stream) and should not displace what the
 // caches hold.
 __device__ __forceinline__ void async_load16_masked_nt(uint64_t mask, uint32_t lds_addr, const void* base, uint32_t voff)
 {
 	uint64_t saved;
-	asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, %0, %1\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %4 " LTEN_STREAM_HINT "\n\ts_mov_b64 exec, %0"
+	asm volatile("s_mov_b64 %0, exec\n\ts_and_b64 exec, %0, %1\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %3, %4 nt\n\ts_mov_b64 exec, %0"
 	             : "=&s"(saved) : "s"(mask), "s"(lds_addr), "v"(voff), "s"(base) : "memory", "scc");
 }
 
