@@ -265,6 +265,15 @@ int lten_hip_nll_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const fl
 int lten_hip_log_softmax_nll_loss_grad_f32(uint64_t rows, uint64_t cols, const float* x, const float* target, float alpha, float* y,
                                            float* loss, float* dx);
 
+/* The loss and the backward pass of the layer that produced the logits, in one launch: lten_hip_log_softmax_nll_loss_grad_f32
+ * (rows = M, cols = out_features, x = logits; writes log_probs, *loss and dlogits) followed by lten_hip_fc_backward_f32 with
+ * dY = dlogits (l-ten/layers.cpp:93-114,212-273; l-ten/backprop.cpp:3975-4040,2083-2280), or, with relu_input not NULL,
+ * by lten_hip_fc_backward_relu_f32; same values bit for bit.  One launch for a classifier's last layer (out_features <= 16,
+ * M * out_features <= 4096, M < 512, dX and dW both wanted), the separate launches otherwise. */
+int lten_hip_fc_backward_log_softmax_nll_loss_f32(uint64_t M, uint64_t in_features, uint64_t out_features, const float* X, const float* W,
+                                                  const float* logits, const float* target, float alpha, float* log_probs, float* loss,
+                                                  float* dlogits, const float* relu_input, float* dX, float* dW, float* db);
+
 /* gpu_sgd_step (l-ten/math_fns.h:186; SGDOptimizer::step, l-ten/optimizer.cpp:26-84) for one parameter tensor:
  * grad = wd * w + grad (stored, as in l-ten), velocity = velocity * mo + (1 - mo) * grad, w = w - velocity * lr. */
 int lten_hip_sgd_step_f32(float* weight, float* weight_grad, float* velocity, uint64_t numels, float mo, float wd, float lr);

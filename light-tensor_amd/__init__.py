@@ -75,6 +75,7 @@ _SIGNATURES = {
     "lten_hip_log_softmax_nll_loss_f32": (C.c_int, [u64, u64, vp, vp, vp, vp]),
     "lten_hip_nll_log_softmax_backward_f32": (C.c_int, [u64, u64, vp, vp, C.c_float, vp]),
     "lten_hip_log_softmax_nll_loss_grad_f32": (C.c_int, [u64, u64, vp, vp, C.c_float, vp, vp, vp]),
+    "lten_hip_fc_backward_log_softmax_nll_loss_f32": (C.c_int, [u64, u64, u64, vp, vp, vp, vp, C.c_float, vp, vp, vp, vp, vp, vp, vp]),
     "lten_hip_relu_f32": (C.c_int, [vp, vp, u64]),
     "lten_hip_relu_backward_f32": (C.c_int, [vp, vp, vp, u64]),
     "lten_hip_scale_f32": (C.c_int, [u64, C.c_float, vp, vp]),

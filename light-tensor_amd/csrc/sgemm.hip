@@ -300,6 +300,101 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_kernel(SProblem px
 	else sgemm_direct_body<8, true, false>(pw, blockIdx.x - blocks_x, 0, part);
 }
 
+// The pair above for the last layer of a classifier, with the loss in front: every workgroup works out the gradient
+// of the loss with respect to the logits (log_softmax, nll_loss and their backward functions: a few thousand values)
+// into LDS for itself and reads the dY operand of its tile from there, so the loss needs no launch of its own and no
+// hand-over between workgroups; one workgroup also writes the log-probabilities, that gradient and the loss.
+// Sixteen lanes per row, one per column: max and sums by lane exchanges in the order of the separate kernels (pairs 8
+// apart, then 4, 2, 1, lanes past the row holding zeros), the loss summed as nll_loss_kernel sums it (1024 strided
+// shares, here two per thread; wavefront trees; 16 partial sums in order): every value is bit-identical to what
+// lten_hip_log_softmax_nll_loss_grad_f32 followed by lten_hip_fc_backward_f32 gives.
+struct LossRows {
+	int rows, cols;  // rows * cols <= 4096, cols <= 16
+	const float* x;  // logits [rows][cols]
+	const float* target;
+	float alpha, loss_scale;
+	float* y;  // log-probabilities
+	float* loss;
+	float* dx;  // gradient with respect to the logits
+};
+
+__device__ __forceinline__ float row16_sum(float v)
+{
+#pragma unroll
+	for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+	return __shfl(v, 0, 16);  // lane 0 holds the tree the separate kernels build
+}
+
+__global__ __launch_bounds__(512) void sgemm_fc_backward_pair_loss_kernel(SProblem px, SProblem pw, int blocks_x, LossRows L)
+{
+	__shared__ float part[8][32 * 32];
+	__shared__ float sdy[4096];
+	__shared__ float part16[16];
+	const int tid = threadIdx.x, c = tid & 15;
+	// A tile of dX needs the 32 rows of its own row block; a tile of dW needs them all, and the first of those writes
+	// the loss outputs as well.
+	const bool for_x = (int)blockIdx.x < blocks_x;
+	const bool first = (int)blockIdx.x == blocks_x;
+	float* logp = &part[0][0];  // free until the tile's partial sums are exchanged
+	auto rows_from = [&](int r) {
+		const bool ok = r < L.rows && c < L.cols;
+		const float xv = ok ? L.x[r * L.cols + c] : -INFINITY;
+		const float tv = ok ? L.target[r * L.cols + c] : 0.0f;
+		float m = xv;
+#pragma unroll
+		for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 16));
+		const float e = ok ? expf(xv - m) : 0.0f;
+		const float s = row16_sum(e);
+		const float lp = logf(e / s);
+		const float dy = ok ? L.alpha * tv : 0.0f;
+		const float sd = row16_sum(dy);
+		const float g = dy - expf(lp) * sd;
+		if (ok) {
+			sdy[r * L.cols + c] = g;
+			if (first) {
+				L.y[r * L.cols + c] = lp;
+				L.dx[r * L.cols + c] = g;
+				logp[r * L.cols + c] = lp;
+			}
+		}
+	};
+	if (for_x) {
+		const int tiles_n = (px.N + 31) / 32;
+		rows_from(((int)blockIdx.x / tiles_n) * 32 + (tid >> 4));
+	} else {
+		// four rows per thread at a time: independent chains of exchanges and transcendentals that overlap
+		for (int r0 = 0; r0 < L.rows; r0 += 128) {
+#pragma unroll
+			for (int u = 0; u < 4; u++) rows_from(r0 + 32 * u + (tid >> 4));
+		}
+	}
+	__syncthreads();
+	if (first) {
+		const int len = L.rows * L.cols;
+#pragma unroll
+		for (int v = 0; v < 2; v++) {
+			const int vt = tid + 512 * v;
+			float acc = 0.0f;
+			for (int i = vt; i < len; i += 1024) acc += logp[i] * L.target[i];
+#pragma unroll
+			for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+			if ((tid & 63) == 0) part16[vt >> 6] = acc;
+		}
+		__syncthreads();
+		if (tid == 0) {
+			float tot = 0.0f;
+#pragma unroll
+			for (int w = 0; w < 16; w++) tot += part16[w];
+			*L.loss = tot * L.loss_scale;
+		}
+	}
+	SProblem qx = px, qw = pw;
+	qx.A = sdy;
+	qw.A = sdy;
+	if ((int)blockIdx.x < blocks_x) sgemm_direct_body<8, false, false>(qx, blockIdx.x, 0, part);
+	else sgemm_direct_body<8, true, false>(qw, blockIdx.x - blocks_x, 0, part);
+}
+
 // C = A^T B (TN) with a short K (the weight gradient dW = dY^T X at a small batch): a 32x32 output tile per wavefront
 // over the whole K, operands straight from global memory in the MFMA lane layout (both are read along their contiguous
 // dimension: two 128-byte rows per wave-wide load), the loads of eight groups of 8 k in flight together, no LDS, no
@@ -1043,6 +1138,35 @@ int lten_hip_fc_backward_relu_f32(uint64_t M, uint64_t in, uint64_t out, const f
 {
 	LTEN_HIP_REQUIRE(relu_input != nullptr || dX == nullptr || M * in == 0, "fc_backward_relu: relu_input is null");
 	return fc_backward(M, in, out, X, W, dY, relu_input, dX, dW, db);
+}
+
+int lten_hip_fc_backward_log_softmax_nll_loss_f32(uint64_t M, uint64_t in, uint64_t out, const float* X, const float* W, const float* logits,
+                                                  const float* target, float alpha, float* log_probs, float* loss, float* dlogits,
+                                                  const float* relu_input, float* dX, float* dW, float* db)
+{
+	LTEN_HIP_REQUIRE(loss != nullptr && M > 0, "fc_backward_log_softmax_nll_loss: null loss pointer or zero batch");
+	LTEN_HIP_REQUIRE(out == 0 || (logits && target && log_probs && dlogits), "fc_backward_log_softmax_nll_loss: null pointer");
+	const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
+	if (dX && dW && X && W && get_option(OPT_SGEMM_TILE) == 0 && M > 1 && M < 512 && out > 1 && out <= 16 && M * out <= 4096 && in > 0 &&
+	    blocks_w < 256) {
+		SProblem px = {}, pw = {};
+		px.A = dlogits; px.B = W; px.C = dX; px.lda = (int64_t)out; px.ldb = (int64_t)in; px.ldc = (int64_t)in;
+		px.M = (int)M; px.N = (int)in; px.K = (int)out; px.alpha = 1.0f; px.beta = 0.0f;
+		px.relu_in = relu_input;
+		pw.A = dlogits; pw.B = X; pw.C = dW; pw.lda = (int64_t)out; pw.ldb = (int64_t)in; pw.ldc = (int64_t)in;
+		pw.M = (int)out; pw.N = (int)in; pw.K = (int)M; pw.alpha = 1.0f; pw.beta = 0.0f;
+		pw.rowsum = db;
+		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
+			LossRows L = { (int)M, (int)out, logits, target, alpha, -1.0f / (float)M, log_probs, loss, dlogits };
+			set_kernel_name("sgemm_fc_backward_pair_loss");
+			sgemm_fc_backward_pair_loss_kernel<<<dim3((unsigned)(blocks_x + blocks_w)), dim3(512), 0, stream()>>>(px, pw, (int)blocks_x, L);
+			LTEN_HIP_LAUNCH_CHECK();
+			return 0;
+		}
+	}
+	// the launches it stands for
+	if (int rc = lten_hip_log_softmax_nll_loss_grad_f32(M, out, logits, target, alpha, log_probs, loss, dlogits)) return rc;
+	return fc_backward(M, in, out, X, W, dlogits, relu_input, dX, dW, db);
 }
 
 }  // extern "C"

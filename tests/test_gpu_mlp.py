@@ -13,9 +13,9 @@ TOL = 1e-4
 def gpu_mlp_step(gpu, X, Ws, bs, T, fused=False):
     """The step through the C ABI, every intermediate resident on the device.  Returns what ob.mlp_step returns.
     fused: the entry points that fold relu, relu_backward, the loss and nll_backward into their neighbours; "head": the
-    loss and its gradient as one call."""
+    loss and its gradient as one call; "tail": the loss, its gradient and the last layer's backward as one call."""
     if fused:
-        return gpu_mlp_step_fused(gpu, X, Ws, bs, T, head=fused == "head")
+        return gpu_mlp_step_fused(gpu, X, Ws, bs, T, head=fused if fused in ("head", "tail") else False)
     D, l = gpu.DeviceBuffer, gpu.lib()
     B, layers = X.shape[0], len(Ws)
     sizes = [X.shape[1]] + [w.shape[0] for w in Ws]
@@ -61,13 +61,20 @@ def gpu_mlp_step_fused(gpu, X, Ws, bs, T, head=False):
             gpu.check(l.lten_hip_fc_forward_relu_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr, act[i + 1].ptr))
         else:
             gpu.check(l.lten_hip_fc_forward_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, db_[i].ptr, pre[i + 1].ptr))
-    if head:
+    gW, gb = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
+    last = layers - 1
+    if head == "tail":
+        i = last  # a single layer has no relu in front of it
+        gpu.check(l.lten_hip_fc_backward_log_softmax_nll_loss_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, pre[layers].ptr, dT.ptr,
+                                                                  -1.0 / B, logp.ptr, loss.ptr, g[layers].ptr, pre[i].ptr if i > 0 else None,
+                                                                  g[i].ptr, gW[i].ptr, gb[i].ptr))
+        last -= 1
+    elif head:
         gpu.check(l.lten_hip_log_softmax_nll_loss_grad_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, -1.0 / B, logp.ptr, loss.ptr, g[layers].ptr))
     else:
         gpu.check(l.lten_hip_log_softmax_nll_loss_f32(B, sizes[-1], pre[layers].ptr, dT.ptr, logp.ptr, loss.ptr))
         gpu.check(l.lten_hip_nll_log_softmax_backward_f32(B, sizes[-1], logp.ptr, dT.ptr, -1.0 / B, g[layers].ptr))
-    gW, gb = [D(w.nbytes) for w in Ws], [D(b.nbytes, zero=True) for b in bs]
-    for i in range(layers - 1, -1, -1):
+    for i in range(last, -1, -1):
         if i > 0:
             gpu.check(l.lten_hip_fc_backward_relu_f32(B, sizes[i], sizes[i + 1], act[i].ptr, dW_[i].ptr, g[i + 1].ptr, pre[i].ptr,
                                                       g[i].ptr, gW[i].ptr, gb[i].ptr))
@@ -162,6 +169,14 @@ def test_cfg2_training_step_full_size(gpu, ob, wl):
     for key in ("pre", "dW", "db"):
         for a, b in zip(headed[key], got[key]):
             assert np.array_equal(a, b), key
+    # and with the last layer's backward in that call as well (6 launches)
+    tailed = gpu_mlp_step(gpu, X, Ws, bs, T, fused="tail")
+    assert tailed["loss"] == got["loss"]
+    for key in ("logp", "dX"):
+        assert np.array_equal(tailed[key], got[key]), key
+    for key in ("pre", "dW", "db"):
+        for a, b in zip(tailed[key], got[key]):
+            assert np.array_equal(a, b), key
 
 
 @pytest.mark.parametrize("shape", [(128, 784, 1024), (7, 33, 50), (20, 2048, 640), (600, 96, 200), (300, 2048, 4096), (1, 64, 32)])
@@ -220,6 +235,46 @@ def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
         assert np.array_equal(y0.numpy(np.float32, x.shape), y2.numpy(np.float32, x.shape)), (rows, cols)
         assert l0.numpy(np.float32, (1,))[0] == l2.numpy(np.float32, (1,))[0], (rows, cols)
         assert np.array_equal(g0.numpy(np.float32, x.shape), g2.numpy(np.float32, x.shape)), (rows, cols)
+
+
+@pytest.mark.parametrize("shape", [(128, 1024, 10), (2, 40, 2), (100, 516, 16), (255, 33, 16), (409, 64, 10), (300, 128, 16), (64, 9000, 10),
+                                   (511, 20, 8), (128, 1024, 17), (1, 64, 10), (512, 64, 8), (37, 12, 1)])
+def test_loss_with_the_last_layers_backward_matches_the_separate_calls(gpu, shape):
+    """lten_hip_fc_backward_log_softmax_nll_loss_f32 against lten_hip_log_softmax_nll_loss_grad_f32 followed by
+    lten_hip_fc_backward_f32: log-probabilities, loss, gradient of the logits, dX, dW and db bit-identical, on shapes the
+    one-launch kernel takes (ragged tiles, full LDS, a wide input) and on shapes it hands to the separate launches."""
+    M, fin, fout = shape
+    rng = np.random.default_rng(M * 7 + fin + fout)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    X = rng.standard_normal((M, fin)).astype(np.float32)
+    W = (rng.standard_normal((fout, fin)) * 0.05).astype(np.float32)
+    logits = (rng.standard_normal((M, fout)) * 3).astype(np.float32)
+    T = np.eye(fout, dtype=np.float32)[rng.integers(0, fout, M)]
+    b = rng.standard_normal(fout).astype(np.float32)
+    dX_, dW_, dL, dT = D.from_numpy(X), D.from_numpy(W), D.from_numpy(logits), D.from_numpy(T)
+    out = []
+    for fused in (False, True):
+        y, loss, gl, gx, gw, gb = D(logits.nbytes), D(4), D(logits.nbytes), D(X.nbytes), D(W.nbytes), D.from_numpy(b)
+        if fused:
+            gpu.check(l.lten_hip_fc_backward_log_softmax_nll_loss_f32(M, fin, fout, dX_.ptr, dW_.ptr, dL.ptr, dT.ptr, -1.0 / M, y.ptr, loss.ptr,
+                                                                      gl.ptr, None, gx.ptr, gw.ptr, gb.ptr))
+            print(f"  {shape}: {gpu.last_kernel()}", flush=True)
+        else:
+            gpu.check(l.lten_hip_log_softmax_nll_loss_grad_f32(M, fout, dL.ptr, dT.ptr, -1.0 / M, y.ptr, loss.ptr, gl.ptr))
+            gpu.check(l.lten_hip_fc_backward_f32(M, fin, fout, dX_.ptr, dW_.ptr, gl.ptr, gx.ptr, gw.ptr, gb.ptr))
+        out.append([y.numpy(np.float32, logits.shape), loss.numpy(np.float32, (1,)), gl.numpy(np.float32, logits.shape),
+                    gx.numpy(np.float32, X.shape), gw.numpy(np.float32, W.shape), gb.numpy(np.float32, b.shape)])
+    if shape == (128, 1024, 10):
+        assert gpu.last_kernel() == "sgemm_fc_backward_pair_loss"
+    for name, a, c in zip(("log_probs", "loss", "dlogits", "dX", "dW", "db"), out[0], out[1]):
+        assert np.array_equal(a, c), (shape, name)
+    # against numpy in fp64
+    z = logits.astype(np.float64) - logits.max(axis=1, keepdims=True)
+    lp = z - np.log(np.exp(z).sum(axis=1, keepdims=True))
+    g = (np.exp(lp) - T) / M
+    assert rel_err(out[1][0], lp) < TOL and rel_err(out[1][2], g) < TOL
+    assert abs(out[1][1][0] + (lp * T).sum() / M) < 1e-5 * max(1.0, abs((lp * T).sum() / M))
+    assert rel_err(out[1][3], g @ W) < TOL and rel_err(out[1][4], g.T @ X) < TOL and rel_err(out[1][5], b + g.sum(axis=0)) < TOL
 
 
 def test_elementwise_kernels(gpu, ob):
