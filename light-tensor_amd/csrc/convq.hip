@@ -18,67 +18,101 @@ namespace lten_hip {
 
 constexpr int CQ_MAXK = 64, CQ_CO = 64;
 
-template <int OUT>
+// ND = dwords of packed taps a thread holds (4 taps each): 4, 8, 12 or 16, the smallest that covers K.
+template <int OUT, int ND>
 __global__ __launch_bounds__(256) void conv2dq_direct_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
                                                              const int32_t* __restrict__ bias, int zp_in, int zp_w, float mult, float zp_out,
                                                              void* __restrict__ y)
 {
-	__shared__ __attribute__((aligned(16))) uint32_t s_w[CQ_CO][CQ_MAXK / 4];
-	__shared__ int s_wsum[CQ_CO];
+	__shared__ __attribute__((aligned(16))) uint32_t s_w[CQ_CO][ND];
 	const int tid = threadIdx.x;
 	const int K = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
 	const int co0 = blockIdx.y * CQ_CO, nco = min(CQ_CO, g.Cout - co0);
 
-	// weights of this block's output channels, four taps per dword, taps past K as zero bytes
-	for (int idx = tid; idx < CQ_CO * (CQ_MAXK / 4); idx += 256) {
-		const int co = idx / (CQ_MAXK / 4), d = idx % (CQ_MAXK / 4);
+	// N * HW < 2^31 (checked by the host): 32-bit divisions
+	const uint32_t gid = blockIdx.x * 256u + tid;
+	const bool live = gid < (uint32_t)g.N * (uint32_t)HW;
+	const int n = live ? (int)(gid / (uint32_t)HW) : 0, pos = live ? (int)(gid - (uint32_t)n * (uint32_t)HW) : 0;
+	const int ho = (int)((uint32_t)pos / (uint32_t)g.Wo), wo = pos - ho * g.Wo;
+	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
+	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W + (int64_t)y0 * g.W + x0;  // tap (0, 0, 0) of this position's window
+
+	// The window, tap k in byte k % 4 of dword k / 4; (ci, i, j) of tap k is the same for every thread and is stepped,
+	// not divided out.  The loads are issued before the weights are staged, so that the two latencies overlap.
+	uint8_t tap[4 * ND];
+	{
+		int i = 0, j = 0, plane_row = 0;  // plane_row = ci * H + i
+#pragma unroll
+		for (int k = 0; k < 4 * ND; k++) {
+			tap[k] = 0;
+			if (k < K) {
+				const int yy = y0 + i, xx = x0 + j;
+				if (live && yy >= 0 && yy < g.H && xx >= 0 && xx < g.W) tap[k] = xn[(int64_t)plane_row * g.W + j];
+				if (++j == g.kw) {
+					j = 0;
+					plane_row++;
+					if (++i == g.kh) {
+						i = 0;
+						plane_row += g.H - g.kh;
+					}
+				}
+			}
+		}
+	}
+
+	// weights of this block's output channels, four taps per dword, taps past K as zero bytes (every load issued, the
+	// byte of a tap past K discarded)
+	for (int idx = tid; idx < CQ_CO * ND; idx += 256) {
+		const int co = idx / ND, d = idx % ND;
 		uint32_t v = 0;
-		if (co < nco)
-			for (int b = 0; b < 4; b++)
-				if (4 * d + b < K) v |= (uint32_t)w[(int64_t)(co0 + co) * K + 4 * d + b] << (8 * b);
+		if (co < nco && K > 0) {
+			const uint8_t* wr = w + (int64_t)(co0 + co) * K;
+#pragma unroll
+			for (int b = 0; b < 4; b++) {
+				const int k = 4 * d + b;
+				const uint32_t byte = wr[min(k, K - 1)];
+				v |= (k < K ? byte : 0u) << (8 * b);
+			}
+		}
 		s_w[co][d] = v;
 	}
 	__syncthreads();
-	if (tid < CQ_CO) {
-		uint32_t sum = 0;
-		for (int d = 0; d < CQ_MAXK / 4; d++) sum = __builtin_amdgcn_udot4(s_w[tid][d], 0x01010101u, sum, false);
-		s_wsum[tid] = (int)sum;
-	}
-	__syncthreads();
+	if (!live) return;
 
-	const int64_t gid = (int64_t)blockIdx.x * 256 + tid;
-	if (gid >= (int64_t)g.N * HW) return;
-	const int n = (int)(gid / HW), pos = (int)(gid % HW);
-	const int ho = pos / g.Wo, wo = pos % g.Wo;
-	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
-	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
-
-	// the window, tap k in byte k % 4 of dword k / 4
-	uint32_t xk[CQ_MAXK / 4];
+	uint32_t xk[ND];
 #pragma unroll
-	for (int d = 0; d < CQ_MAXK / 4; d++) xk[d] = 0;
-#pragma unroll
-	for (int k = 0; k < CQ_MAXK; k++) {
-		if (k >= K) break;
-		const int j = k % g.kw, i = (k / g.kw) % g.kh, ci = k / (g.kw * g.kh);
-		const int yy = y0 + i, xx = x0 + j;
-		if (yy >= 0 && yy < g.H && xx >= 0 && xx < g.W) xk[k / 4] |= (uint32_t)xn[((int64_t)ci * g.H + yy) * g.W + xx] << (8 * (k % 4));
-	}
+	for (int d = 0; d < ND; d++)
+		xk[d] = (uint32_t)tap[4 * d] | (uint32_t)tap[4 * d + 1] << 8 | (uint32_t)tap[4 * d + 2] << 16 | (uint32_t)tap[4 * d + 3] << 24;
 	uint32_t xsum = 0;
 #pragma unroll
-	for (int d = 0; d < CQ_MAXK / 4; d++) xsum = __builtin_amdgcn_udot4(xk[d], 0x01010101u, xsum, false);
+	for (int d = 0; d < ND; d++) xsum = __builtin_amdgcn_udot4(xk[d], 0x01010101u, xsum, false);
 	// l-ten/math_fns.cpp:1362-1380,1433: row_vector[p] = -zpA * sum_k B[k][p] with A = weights; broadcast = K zpA zpB
 	const int base = -zp_w * (int)xsum + K * zp_w * zp_in + (bias ? bias[pos] : 0);
 
 	for (int co = 0; co < nco; co++) {
-		uint32_t dot = 0;
+		// the byte sum of the channel's weights rides along: the dwords are in registers anyway
+		uint32_t dot = 0, wsum = 0;
 #pragma unroll
-		for (int d = 0; d < CQ_MAXK / 4; d++) dot = __builtin_amdgcn_udot4(s_w[co][d], xk[d], dot, false);
-		const int v = (int)dot + base - zp_in * s_wsum[co];
+		for (int d = 0; d < ND; d++) {
+			const uint32_t wd = s_w[co][d];
+			dot = __builtin_amdgcn_udot4(wd, xk[d], dot, false);
+			wsum = __builtin_amdgcn_udot4(wd, 0x01010101u, wsum, false);
+		}
+		const int v = (int)dot + base - zp_in * (int)wsum;
 		const int64_t o = ((int64_t)n * g.Cout + co0 + co) * HW + pos;
 		if (OUT == Q_OUT_ACC) static_cast<int*>(y)[o] = v;
 		else static_cast<uint8_t*>(y)[o] = (uint8_t)requant<OUT>(v, mult, zp_out);
 	}
+}
+
+template <int OUT>
+static void launch_conv2dq_direct(const dim3& grid, int K, const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in,
+                                  int zp_w, float mult, float zp_out, void* y)
+{
+	if (K <= 16) conv2dq_direct_kernel<OUT, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+	else if (K <= 32) conv2dq_direct_kernel<OUT, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+	else if (K <= 48) conv2dq_direct_kernel<OUT, 12><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+	else conv2dq_direct_kernel<OUT, 16><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
 }
 
 static int make_geo_q(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh, int sw)
@@ -113,13 +147,13 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 	volatile float ab = qp[1].scale * qp[0].scale;
 	const float mult = ab / qp[2].scale, zp_out = (float)qp[2].zero_point;
 
-	if (K <= CQ_MAXK && ceil_div((uint64_t)N * HW, 256) < (1ull << 31) && get_option(OPT_CONV_VARIANT) != 1) {
+	if (K <= CQ_MAXK && (uint64_t)N * HW < (1ull << 31) && get_option(OPT_CONV_VARIANT) != 1) {
 		const dim3 grid((unsigned)ceil_div((uint64_t)N * HW, 256), (unsigned)ceil_div(Cout, CQ_CO));
 		set_kernel_name("conv2dq_direct");
-		if (out_acc) conv2dq_direct_kernel<Q_OUT_ACC><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+		if (out_acc) launch_conv2dq_direct<Q_OUT_ACC>(grid, (int)K, g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
 		else if (mult == mult && (mult < 0 ? -mult : mult) <= 0.99f)
-			conv2dq_direct_kernel<Q_OUT_U8_FAST><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
-		else conv2dq_direct_kernel<Q_OUT_U8_EXACT><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+			launch_conv2dq_direct<Q_OUT_U8_FAST>(grid, (int)K, g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
+		else launch_conv2dq_direct<Q_OUT_U8_EXACT>(grid, (int)K, g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}

@@ -29,7 +29,11 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (3, 7, 13, 17, 70, 3, 3, 1, 1, 1, 1),       # 63 taps, two channel blocks
                                  (2, 16, 20, 22, 24, 3, 3, 1, 1, 2, 1),      # 144 taps: column buffer + GEMM
                                  (1, 3, 33, 300, 5, 7, 3, 3, 0, 2, 3),       # 63 taps, strides, ragged
-                                 (2, 32, 9, 9, 40, 1, 1, 0, 0, 1, 1)])       # 1x1
+                                 (2, 32, 9, 9, 40, 1, 1, 0, 0, 1, 1),        # 1x1
+                                 (2, 5, 11, 13, 9, 3, 3, 1, 0, 1, 2),        # 45 taps: twelve packed dwords
+                                 (1, 4, 8, 8, 3, 2, 2, 1, 1, 1, 1),          # 16 taps: four dwords, all full
+                                 (2, 11, 7, 9, 5, 1, 3, 0, 1, 1, 1),         # 33 taps: one tap in the ninth dword
+                                 (1, 3, 12, 10, 7, 4, 4, 1, 2, 1, 1)])       # 48 taps
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
