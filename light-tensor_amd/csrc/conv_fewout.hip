@@ -8,11 +8,11 @@
 // of one image; a thread owns four consecutive pixels of one row and all output channels.  Input channels come in
 // chunks of four: the patch [4 channels][10 rows][136 columns] (column q = input column w0 - 4 + q) is filled by
 // direct global->LDS loads exactly as it lies in memory, two stages (on a 32-channel 128 x 128 data gradient at batch
-// 32 a third stage did not help, 26.0 against 24.5 us, nor did tiles of four rows with twice the workgroups).  Whether a float4 of the patch lies inside the
-// image does not depend on the chunk: lanes whose float4 does not exist never load, and their slots keep the zeros
-// written once.  Per channel and patch row a thread needs six columns (4 t + 3 .. 4 t + 8): its own four in one 16-byte
-// read, the two neighbours from the lanes beside it, and multiplies them with the 3 * Cout weights of that row, which are wave-uniform and come
-// through scalar loads.  DGRAD reads the weights of the transposed problem in place (w[ci][co][2 - i][2 - j]), so
+// 32 a third stage is slower, 17.1 against 15.9 us).  Whether a float4 of the patch lies inside the image does not
+// depend on the chunk: lanes whose float4 does not exist never load, and their slots keep the zeros written once.
+// Per channel and patch row a thread needs six columns (4 t + 3 .. 4 t + 8): its own four in one 16-byte read, the two
+// neighbours from the lanes beside it (a lane shift in the vector ALU), and multiplies them with the 3 * Cout
+// weights of that row, which are wave-uniform and come through scalar loads.  DGRAD reads the weights of the transposed problem in place (w[ci][co][2 - i][2 - j]), so
 // no flipped copy is made.
 //
 // Needs Cin % 4 == 0, W % 4 == 0 and 16-byte aligned x and y.
@@ -44,8 +44,15 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int trow = tid >> 5, tq = tid & 31;  // this thread's row of the tile and its group of four pixels
 	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
-	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
-	const int n = blockIdx.y;
+	// Consecutive workgroup ids go round the eight XCDs: each XCD gets a contiguous run of (image, tile) items, so that
+	// the tiles above and below a tile (two of its ten patch rows each) run on the same L2, close in time.  The grid is
+	// 8 * per workgroups; the ones past the last item leave.
+	const int tiles = tiles_w * ((g.Ho + P::TH - 1) / P::TH), total = tiles * g.N;
+	const int per = (total + 7) / 8;
+	const int item = ((int)blockIdx.x & 7) * per + ((int)blockIdx.x >> 3);
+	if (item >= total) return;
+	const int bx = item % tiles, n = item / tiles;
+	const int w0 = (bx % tiles_w) * P::TW, h0 = (bx / tiles_w) * P::TH;
 	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
 
 	// ---- what this lane fetches for each of its wavefront's loads (load q = wave + 4 i); always the same lanes
@@ -88,9 +95,16 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 		for (int i = 0; i < P::LPW; i++) async_load16_masked(mask[i], smem_addr + stage * P::STAGE + (wave + 4 * i) * 1024, xn + kt * x_step, voff[i]);
 	};
 
-	// ---- zeros everywhere once: what no load ever writes is the padding
-	for (int i = tid; i < P::S * P::STAGE / 16; i += 256) reinterpret_cast<float4*>(smem)[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-	__syncthreads();
+	// ---- zeros once in the slots no load ever writes (that is the padding): each lane clears its own, in every stage;
+	// the slots that are loaded are never stored to, so the first loads need not wait for this
+#pragma unroll
+	for (int i = 0; i < P::LPW; i++) {
+		const bool mine = !((mask[i] >> lane) & 1);
+		if (mine)
+#pragma unroll
+			for (int st = 0; st < P::S; st++)
+				*reinterpret_cast<float4*>(smem + st * P::STAGE + (wave + 4 * i) * 1024 + lane * 16) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	}
 	const int KT = g.Cin / P::CB;
 #pragma unroll
 	for (int st = 0; st < P::S; st++)
@@ -125,12 +139,17 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 #pragma unroll
 			for (int i = 0; i < 3; i++) {
 				const float* sp = reinterpret_cast<const float*>(sbase + ((c * P::PR + i) * P::PWS) * 4);
-				// the four own columns in one read; the neighbours' from the lanes beside this one (their own reads), except
-				// at the ends of the tile row: a 4-byte read per lane would put eight lanes on every bank it touches
+				// the four own columns in one read
 				const float4 mid = *reinterpret_cast<const float4*>(sp + 1);
-				float left = __shfl_up(mid.w, 1, 64), right = __shfl_down(mid.x, 1, 64);
-				if (tq == 0) left = sp[0];
-				if (tq == 31) right = sp[5];
+				// the neighbours' columns by a lane shift in the vector ALU (DPP wave_shr:1 / wave_shl:1: lane i takes lane
+				// i - 1 / i + 1), and at the ends of the tile row from the patch: every lane reads its row's two edge values
+				// (one address per row: a broadcast, no bank conflict) and keeps them only there — a branch around an LDS
+				// read in the middle of the multiply-adds cost a fifth of the kernel's time
+				float left = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(mid.w), 0x138, 0xf, 0xf, false));
+				float right = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(mid.x), 0x130, 0xf, 0xf, false));
+				const float* rowp = sp - 4 * tq;
+				left = tq == 0 ? rowp[0] : left;
+				right = tq == 31 ? rowp[4 * 31 + 5] : right;
 				const float v[6] = { left, mid.x, mid.y, mid.z, mid.w, right };
 #pragma unroll
 				for (int co = 0; co < COUT; co++) {
@@ -162,14 +181,16 @@ __global__ __launch_bounds__(256) void conv2d_fewout_forward_kernel(ConvGeo g, c
 bool conv_fewout_takes(const ConvGeo& g, const float* x, const float* y)
 {
 	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw == 1 && g.ph <= 2 && g.Cout >= 1 && g.Cout <= 4 &&
-	       g.Cin % 4 == 0 && g.Cin >= 4 && g.W % 4 == 0 && aligned16(x) && aligned16(y) && (uint64_t)g.H * g.W < (1u << 26) && g.N < 65536;
+	       g.Cin % 4 == 0 && g.Cin >= 4 && g.W % 4 == 0 && aligned16(x) && aligned16(y) && (uint64_t)g.H * g.W < (1u << 26) && g.N < 65536 &&
+	       ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 8) * g.N < (1u << 28);
 }
 
 // dgrad: w is the weight array of the convolution whose data gradient this is ([g.Cin][g.Cout][3][3] in terms of g)
 template <bool DGRAD>
 static int launch_fewout(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
-	const dim3 grid((unsigned)(ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 8)), (unsigned)g.N), block(256);
+	const uint64_t total = ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 8) * g.N;
+	const dim3 grid((unsigned)(8 * ceil_div(total, 8))), block(256);
 	switch (g.Cout) {
 	case 1: conv2d_fewout_forward_kernel<1, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
 	case 2: conv2d_fewout_forward_kernel<2, DGRAD><<<grid, block, 0, stream()>>>(g, x, w, bias, y); break;
