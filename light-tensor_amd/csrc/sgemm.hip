@@ -588,34 +588,31 @@ __device__ __forceinline__ void sgemm_skinny_body(const SProblem& p, int col_blo
 	struct Batch {
 		float4 a[2 * MB], b[2];
 	};
-	// K % 4 == 0: a float4 lies inside K or outside as a whole
+	// K % 4 == 0: a float4 lies inside K or outside as a whole.  Every load is issued, from an address clamped into the
+	// operand, and what lies outside is replaced by zeros when the batch is multiplied: with the loads under conditions
+	// the compiler can no longer count how many are in flight and waits for all of them before the first multiply, the
+	// prefetched ones included.
 	auto fetch = [&](int batch, Batch& v) {
-		const int k = batch * 32 + c4;
+		const int kc = min(batch * 32 + c4, p.K - 4);
 #pragma unroll
-		for (int i = 0; i < 2 * MB; i++) {
-			const int m = mrow0 + 8 * i + r8;
-			v.a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (m < p.M && k < p.K) v.a[i] = *reinterpret_cast<const float4*>(p.A + (int64_t)m * p.lda + k);
-		}
+		for (int i = 0; i < 2 * MB; i++)
+			v.a[i] = *reinterpret_cast<const float4*>(p.A + (int64_t)min(mrow0 + 8 * i + r8, p.M - 1) * p.lda + kc);
 #pragma unroll
 		for (int i = 0; i < 2; i++) {
-			v.b[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (BT) {
-				const int n = n0 + 8 * i + r8;
-				if (n < p.N && k < p.K) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)n * p.ldb + k);
-			} else {  // N % 4 == 0: the four columns are inside N or outside together
-				const int kb = batch * 32 + 16 * i + k16;
-				if (kb < p.K && n0 + n4 < p.N) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)kb * p.ldb + n0 + n4);
-			}
+			if (BT) v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)min(n0 + 8 * i + r8, p.N - 1) * p.ldb + kc);
+			else  // N % 4 == 0: the four columns are inside N or outside together
+				v.b[i] = *reinterpret_cast<const float4*>(p.B + (int64_t)min(batch * 32 + 16 * i + k16, p.K - 1) * p.ldb + min(n0 + n4, p.N - 4));
 		}
 	};
-	auto multiply = [&](const Batch& v) {
+	auto keep = [](const float4& t, bool in) { return make_float4(in ? t.x : 0.0f, in ? t.y : 0.0f, in ? t.z : 0.0f, in ? t.w : 0.0f); };
+	auto multiply = [&](int batch, const Batch& v) {
+		const bool k_in = batch * 32 + c4 < p.K;
 #pragma unroll
-		for (int i = 0; i < 2 * MB; i++) *reinterpret_cast<float4*>(sA + (8 * i + r8) * LD + c4) = v.a[i];
+		for (int i = 0; i < 2 * MB; i++) *reinterpret_cast<float4*>(sA + (8 * i + r8) * LD + c4) = keep(v.a[i], mrow0 + 8 * i + r8 < p.M && k_in);
 #pragma unroll
 		for (int i = 0; i < 2; i++) {
-			if (BT) *reinterpret_cast<float4*>(sB + (8 * i + r8) * LD + c4) = v.b[i];
-			else *reinterpret_cast<float4*>(sB + (16 * i + k16) * LDB + n4) = v.b[i];
+			if (BT) *reinterpret_cast<float4*>(sB + (8 * i + r8) * LD + c4) = keep(v.b[i], n0 + 8 * i + r8 < p.N && k_in);
+			else *reinterpret_cast<float4*>(sB + (16 * i + k16) * LDB + n4) = keep(v.b[i], batch * 32 + 16 * i + k16 < p.K && n0 + n4 < p.N);
 		}
 #pragma unroll
 		for (int h = 0; h < 2; h++) {
@@ -640,23 +637,25 @@ __device__ __forceinline__ void sgemm_skinny_body(const SProblem& p, int col_blo
 		}
 	};
 
+	// No load stands under a condition (a load in a conditional block costs a wait for everything in flight at the first
+	// use behind it): while a further round exists its batches are fetched, one past the end as the last one again, and
+	// the round in hand is multiplied whole; the last round is multiplied as far as it exists, with no fetch beside it.
 	const int batches = (p.K + 31) / 32;
 	Batch cur[UB], nxt[UB];
 	int b0 = wave;
 #pragma unroll
-	for (int u = 0; u < UB; u++)
-		if (b0 + u * WAVES < batches) fetch(b0 + u * WAVES, cur[u]);
-	for (; b0 < batches; b0 += WAVES * UB) {
-		const int n0b = b0 + WAVES * UB;
+	for (int u = 0; u < UB; u++) fetch(min(b0 + u * WAVES, batches - 1), cur[u]);
+	for (; b0 + WAVES * UB < batches; b0 += WAVES * UB) {
 #pragma unroll
-		for (int u = 0; u < UB; u++)
-			if (n0b + u * WAVES < batches) fetch(n0b + u * WAVES, nxt[u]);
+		for (int u = 0; u < UB; u++) fetch(min(b0 + (UB + u) * WAVES, batches - 1), nxt[u]);
 #pragma unroll
-		for (int u = 0; u < UB; u++)
-			if (b0 + u * WAVES < batches) multiply(cur[u]);
+		for (int u = 0; u < UB; u++) multiply(b0 + u * WAVES, cur[u]);
 #pragma unroll
 		for (int u = 0; u < UB; u++) cur[u] = nxt[u];
 	}
+#pragma unroll
+	for (int u = 0; u < UB; u++)
+		if (b0 + u * WAVES < batches) multiply(b0 + u * WAVES, cur[u]);
 
 	// accumulator register e of lane (r16, q4) of block b: row 16b + 4 q4 + e, column r16.  The wavefronts' partial
 	// tiles meet in LDS (the slabs are no longer needed) and are added in wavefront order.
