@@ -304,7 +304,7 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_kernel(SProblem px
 // of the loss with respect to the logits (log_softmax, nll_loss and their backward functions: a few thousand values)
 // into LDS for itself and reads the dY operand of its tile from there, so the loss needs no launch of its own and no
 // hand-over between workgroups; one workgroup also writes the log-probabilities, that gradient and the loss.
-// Sixteen lanes per row, one per column: max and sums by lane exchanges in the order of the separate kernels (pairs 8
+// Sixteen lanes per row, one per column: max and sums over the row in the order of the separate kernels (pairs 8
 // apart, then 4, 2, 1, lanes past the row holding zeros), the loss summed as nll_loss_kernel sums it (1024 strided
 // shares, here two per thread; wavefront trees; 16 partial sums in order): every value is bit-identical to what
 // lten_hip_log_softmax_nll_loss_grad_f32 followed by lten_hip_fc_backward_f32 gives.
@@ -318,11 +318,31 @@ struct LossRows {
 	float* dx;  // gradient with respect to the logits
 };
 
+// Sum and maximum over the 16 lanes of a row by rotations within the row in the vector ALU (DPP row_ror:8, 4, 2, 1).
+// Every lane ends with the same value: pairs 8 apart, then pairs of pairs 4 apart, 2, 1 — the tree the separate kernels
+// build with lane exchanges, operands commuted at most.
+template <int CTRL>
+__device__ __forceinline__ float row_rotate(float v)
+{
+	return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
 __device__ __forceinline__ float row16_sum(float v)
 {
-#pragma unroll
-	for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
-	return __shfl(v, 0, 16);  // lane 0 holds the tree the separate kernels build
+	v += row_rotate<0x128>(v);
+	v += row_rotate<0x124>(v);
+	v += row_rotate<0x122>(v);
+	v += row_rotate<0x121>(v);
+	return v;
+}
+
+__device__ __forceinline__ float row16_max(float v)
+{
+	v = fmaxf(v, row_rotate<0x128>(v));
+	v = fmaxf(v, row_rotate<0x124>(v));
+	v = fmaxf(v, row_rotate<0x122>(v));
+	v = fmaxf(v, row_rotate<0x121>(v));
+	return v;
 }
 
 __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_loss_kernel(SProblem px, SProblem pw, int blocks_x, LossRows L)
@@ -340,9 +360,7 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_loss_kernel(SProbl
 		const bool ok = r < L.rows && c < L.cols;
 		const float xv = ok ? L.x[r * L.cols + c] : -INFINITY;
 		const float tv = ok ? L.target[r * L.cols + c] : 0.0f;
-		float m = xv;
-#pragma unroll
-		for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 16));
+		const float m = row16_max(xv);
 		const float e = ok ? expf(xv - m) : 0.0f;
 		const float s = row16_sum(e);
 		const float lp = logf(e / s);
