@@ -126,9 +126,14 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) acc[mb] = v4i{ 0, 0, 0, 0 };
 		int sb = 0;
+		// The bias of this row group is fetched here and taken into a register behind the wait for the slab: the compiler
+		// waits for a load of its own before its first use, and behind the next slab's loads that wait would cover them too.
+		int bias_n = 0;
+		if (wave == 0 && bias && group * 16 + lrow < p.N) bias_n = bias[group * 16 + lrow];
 #pragma unroll
 		for (int pass = 0; pass < PASSES; pass++) {
 			asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // own slab has landed (no other wave reads this slab)
+			if (pass == 0) asm volatile("" : "+v"(bias_n));
 #pragma unroll
 			for (int s = 0; s < 16; s++) {
 				const int gs = pass * 16 + s;
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 		const int n = group * 16 + lrow;
 		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-		const int base = coef_b * tsb + p.K * coef_a * coef_b + ((bias && n < p.N) ? bias[n] : 0);
+		const int base = coef_b * tsb + p.K * coef_a * coef_b + bias_n;
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) {
 			v4i tot = { 0, 0, 0, 0 };
