@@ -98,7 +98,9 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 {
 	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.M >= 1 && p.N >= 1 && p.K >= 1)) return -1;
 	const int64_t tiles = (int64_t)ceil_div((uint64_t)p.M, 16) * ceil_div((uint64_t)p.N, 16);
-	if (tiles > 512 || p.K > 16384) return -1;
+	// up to 512 tiles; with an N the direct-to-LDS tiles do not take (no multiple of 4) up to 8192, where the alternative
+	// is the guarded kernel (4096 x 50 x 5760: 83 us there)
+	if (tiles > (p.N % 4 != 0 ? 8192 : 512) || p.K > 16384) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
 	const dim3 grid((unsigned)tiles);
 	if (p.K <= 1024) {

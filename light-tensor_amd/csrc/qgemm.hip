@@ -427,8 +427,9 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
 	}
-	// 33 to 64 rows: two streaming passes (32 rows, then the rest) still beat one pass of 128-row tiles, three would not
-	if (M > 32 && M <= 64 && N >= 2048 && K <= 8192 && may_stream) {
+	// 33 to 64 rows: two streaming passes (32 rows, then the rest) still beat one pass of 128-row tiles, three would not;
+	// with a short K the tiles win (4096 x 1024 weights: 8.2 us against 9.7-11.3 us)
+	if (M > 32 && M <= 64 && N >= 2048 && K >= 2048 && K <= 8192 && may_stream) {
 		QProblem top = p, rest = p;
 		top.M = 32;
 		rest.M = (int)M - 32;
