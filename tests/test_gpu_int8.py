@@ -353,9 +353,10 @@ def test_weight_streaming_in_two_passes(gpu, ob, M):
         assert gpu.last_kernel().startswith("qskinny_mfma_w2"), gpu.last_kernel()
 
 
-@pytest.mark.parametrize("shape", [(64, 512, 784), (1, 10, 16), (17, 33, 48), (100, 70, 1040), (16, 16, 16384), (33, 250, 2064)])
+@pytest.mark.parametrize("shape", [(64, 512, 784), (1, 10, 16), (17, 33, 48), (100, 70, 1040), (16, 16, 16384), (33, 250, 2064),
+                                   (2100, 50, 784), (600, 210, 1040)])
 def test_small_output_kernel(gpu, ob, shape):
-    """At most 512 output tiles of 16x16, K % 16 == 0: the one-launch kernel with in-kernel zero-point sums (ragged
+    """At most 512 output tiles of 16x16 (8192 when N is no multiple of 4: 528 and 532 tiles in the last two), K % 16 == 0: the one-launch kernel with in-kernel zero-point sums (ragged
     M and N, K tails inside a 64-byte step, both wavefront counts), against the oracle and the tiled kernels."""
     M, N, K = shape
     rng = np.random.default_rng(M * 7 + N * 3 + K)
