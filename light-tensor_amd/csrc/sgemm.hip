@@ -775,6 +775,13 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_wide_kernel(SProbl
 		return;
 	}
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, g = lane >> 5;
+	if (blocks_w * 4 < tiles_w) {
+		// so many tiles of dW that eight per workgroup still give every CU several workgroups: a whole-K tile per wavefront,
+		// no exchange and no barrier (4096 x 4096 weights at batch 32: 58 -> 36 us for the pair)
+		const int tile = (int)blockIdx.x * 8 + wave;
+		if (tile < tiles_w) sgemm_tn_wave_tile_lines(pw, tile, lds + wave * SLAB);
+		return;
+	}
 	const int slot = wave & 3, khalf = wave >> 2;
 	const int tile = (int)blockIdx.x * 4 + slot;
 	const bool active = tile < tiles_w;
@@ -966,7 +973,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// that gives at most a few workgroups per CU: 128 rows against a 1024-wide layer are 256 tiles of 32 x 16 where the
 	// 32 x 32 tiles of the general small-GEMM kernels would occupy half of the CUs.
 	// A classifier head (a few output columns) takes the same kernel: one column block, K cut over eight wavefronts.
-	if (force == 0 && !tA && tB && (N >= 512 || N <= 32) && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
+	if (force == 0 && !tA && tB && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
 	    (M <= 32 || ceil_div(M, 32) * ceil_div(N, 16) <= 1024)) {
 		// few column blocks (a classifier head): blocks of 16 rows, twice the workgroups
 		const bool rows16 = M <= 16 || ceil_div(N, 16) * ceil_div(M, 32) < 64;
@@ -1089,7 +1096,7 @@ static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, co
 	// small enough that the weight-gradient product would not take the whole-line loads: one launch computes the two.
 	// option "sgemm_tile" 7: the paired launch with the weight gradient's K cut over the wavefronts whatever the batch
 	const int pair_opt = get_option(OPT_SGEMM_TILE);
-	if (dX && dW && (pair_opt == 0 || pair_opt == 7) && M > 1 && M < 512 && out > 1 && out <= 2048 && in > 0) {
+	if (dX && dW && (pair_opt == 0 || pair_opt == 7) && M > 1 && M < 512 && out > 1 && out <= 8192 && in > 0) {
 		SProblem px = {}, pw = {};
 		px.A = dY; px.B = W; px.C = dX; px.lda = (int64_t)out; px.ldb = (int64_t)in; px.ldc = (int64_t)in;
 		px.M = (int)M; px.N = (int)in; px.K = (int)out; px.alpha = 1.0f; px.beta = 0.0f;
@@ -1099,8 +1106,9 @@ static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, co
 		pw.rowsum = db;
 		const uint64_t blocks_x = ceil_div(M, 32) * ceil_div(in, 32), blocks_w = ceil_div(out, 32) * ceil_div(in, 32);
 		if (takes_32x32(px, M, in, out) && takes_32x32(pw, out, in, M) && blocks_x + blocks_w < (1u << 20)) {
-			const uint64_t cols_x = ceil_div(in, 16), skinny_x = cols_x * ceil_div(M, 32), w4 = ceil_div(blocks_w, 4);
-			if (pair_opt == 0 && M > 16 && M <= 256 && blocks_w >= 256 && in >= 512 && in % 4 == 0 && out >= 256 && out % 4 == 0 &&
+			// dW: four tiles per workgroup (K cut in two over the wavefronts), eight whole-K tiles when that still leaves 2048 workgroups
+			const uint64_t cols_x = ceil_div(in, 16), skinny_x = cols_x * ceil_div(M, 32), w4 = blocks_w >= 4096 ? ceil_div(blocks_w, 8) : ceil_div(blocks_w, 4);
+			if (pair_opt == 0 && M > 1 && M <= 256 && blocks_w >= 256 && in >= 512 && in % 4 == 0 && out >= 256 && out % 4 == 0 &&
 			    operands_vec(px) && operands_vec(pw) && skinny_x <= 1024) {
 				set_kernel_name("sgemm_fc_backward_pair_wide");
 				sgemm_fc_backward_pair_wide_kernel<<<dim3((unsigned)(w4 + skinny_x)), dim3(512), 0, stream()>>>(px, pw, (int)w4, (int)blocks_w, (int)cols_x);

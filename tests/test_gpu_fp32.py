@@ -106,10 +106,10 @@ def test_small_output_kernels_are_deterministic_and_repeatable(gpu, tile, name):
 
 
 def test_classifier_head_on_the_weight_streaming_kernel(gpu):
-    """NT products with at most 32 output columns (a classifier head: 128 x 10 x 1024) run on the 16-column
-    weight-streaming kernel: ragged column block, ragged rows, alpha and beta, repeatable bit for bit."""
+    """NT products with few output columns (a classifier head: 128 x 10 x 1024; l-ten's 5760 -> 50 layer) run on the
+    16-column weight-streaming kernel: ragged column block, ragged rows, alpha and beta, repeatable bit for bit."""
     rng = np.random.default_rng(21)
-    for (m, n, k) in [(128, 10, 1024), (33, 31, 788), (200, 16, 256), (5, 1, 512)]:
+    for (m, n, k) in [(128, 10, 1024), (33, 31, 788), (200, 16, 256), (5, 1, 512), (64, 50, 5760), (130, 300, 1024), (7, 511, 260)]:
         a = rng.standard_normal((m, k)).astype(np.float32)
         b = rng.standard_normal((n, k)).astype(np.float32)
         c0 = rng.standard_normal((m, n)).astype(np.float32)
@@ -227,7 +227,11 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     (128, 784, 1024, ("sgemm_fc_backward_pair_wide",)),              # config 2, layer 1: both products on 16-byte loads, each on a workgroup per CU
     (100, 1024, 516, ("sgemm_fc_backward_pair_wide",)),              # the same with a ragged batch (two halves of 64 and 36 rows) and ragged tiles
     (128, 786, 1024, ("sgemm_fc_backward_pair_32x32_shortk",)),      # rows of X that allow no 16-byte loads: whole-K tiles from dword loads
-    (511, 64, 2048, ("sgemm_fc_backward_pair_32x32_w8",)),           # the largest batch and width the paired launch takes
+    (511, 64, 2048, ("sgemm_fc_backward_pair_32x32_w8",)),           # the largest batch the paired launch takes
+    (8, 1024, 1024, ("sgemm_fc_backward_pair_wide",)),               # fewer rows than a block of the data-gradient tiles
+    (20, 2048, 2048, ("sgemm_fc_backward_pair_wide",)),              # 4096 tiles of dW: a whole-K tile per wavefront, eight per workgroup
+    (70, 2052, 2060, ("sgemm_fc_backward_pair_wide",)),              # the same with ragged tiles on every side and a ragged batch
+    (3, 512, 4096, ("sgemm_fc_backward_pair_wide",)),                # 4096 outputs wide, 2048 tiles: four per workgroup
     (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
     (640, 1101, 999, ("sgemm_rowvec",)),                             # unaligned rows, many tiles: LDS-tiled GEMM, then the column sum
