@@ -87,8 +87,8 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 			const int c = (lane & 7) ^ swz<8>(r);
 			voff[i] = ((uint32_t)min(row0 + r, rows - 1) * ld + c * 4) * 4;
 		} else {
-			constexpr int KPL = 256 / T;  // k rows per load
-			const int k = q * KPL + (KPL == 2 ? lane >> 5 : 0), r4 = (KPL == 2 ? lane & 31 : lane) * 4;
+			constexpr int KPL = 256 / T, LPR = T / 4;  // k rows per load, lanes per k row
+			const int k = q * KPL + lane / LPR, r4 = (lane % LPR) * 4;
 			voff[i] = (k * ld + (uint32_t)min(row0 + r4, rows - 4)) * 4;  // rows is a multiple of 4 here
 		}
 		lds_slot[i] = smem_addr + (is_a ? 0 : TILE) + q * 1024;
@@ -274,6 +274,15 @@ int sgemm_fast_dispatch(const SProblem& p, int tA, int tB, uint64_t batch, int v
 	case 21: return launch_fast<128, 2, 2, 2>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s2");
 	case 22: return launch_fast<128, 2, 2, 3>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s3");
 	case 23: return launch_fast<128, 2, 2, 4>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s4");
+	case 31: {
+		// 64 x 64 tiles, NT only: with a row-contiguous operand a 32 x 32 wavefront tile has fewer MFMAs per slice than LDS reads
+		if (tA || !tB) return -1;
+		const dim3 grid((unsigned)(ceil_div(p.M, 64) * ceil_div(p.N, 64)), 1, (unsigned)batch), block(256);
+		set_kernel_name("sgemm_fast_64x64x32_w2x2_s2");
+		sgemm_fast_kernel<64, 2, 2, 2, true, true><<<grid, block, 0, stream()>>>(p);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	default: return -1;
 	}
 }

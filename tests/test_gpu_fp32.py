@@ -307,7 +307,7 @@ def test_large_gemm_linearity_property(gpu):
 
 
 FAST_TILES = {11: "sgemm_fast_256x256x32_w2x4_s2", 12: "sgemm_fast_256x256x32_w4x2_s2", 21: "sgemm_fast_128x128x32_w2x2_s2",
-              22: "sgemm_fast_128x128x32_w2x2_s3", 23: "sgemm_fast_128x128x32_w2x2_s4"}
+              22: "sgemm_fast_128x128x32_w2x2_s3", 23: "sgemm_fast_128x128x32_w2x2_s4", 31: "sgemm_fast_64x64x32_w2x2_s2"}
 
 
 @pytest.mark.parametrize("tile", sorted(FAST_TILES))
@@ -315,6 +315,8 @@ FAST_TILES = {11: "sgemm_fast_256x256x32_w2x4_s2", 12: "sgemm_fast_256x256x32_w4
 def test_direct_to_lds_tiles_exact_all_layouts(gpu, tile, tA, tB):
     """The direct-to-LDS tiles by number: integer-valued operands make every summation order exact, so the result
     must equal the int64 product bit for bit, with padded leading dimensions, alpha / beta and an untouched pad."""
+    if tile == 31 and (tA, tB) != (0, 1):
+        pytest.skip("the 64 x 64 tiles exist for NT products only")
     rng = np.random.default_rng(500 + 10 * tile + 2 * tA + tB)
     M, N, K = (512, 256, 160) if tile < 20 else (256, 384, 96)   # K / 32 = 5 or 3 k-steps: prologue, steady state, drain
     A = rng.integers(-8, 9, (M, K)).astype(np.float32)
@@ -347,10 +349,17 @@ def test_direct_to_lds_tiles_are_the_default_for_large_aligned_problems(gpu):
     gpu.check(l.lten_hip_fc_forward_f32(M, fin, fout, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
     assert gpu.last_kernel() == FAST_TILES[12]
     assert np.array_equal(dY.numpy(np.float32, (M, fout)), x @ w.T + b)
-    # 2048 x 1024 output: too few 256-tiles, so 128-tiles
-    gpu.check(l.lten_hip_fc_forward_f32(2048, fin, 1024, dX.ptr, dW.ptr, None, dY.ptr))
+    # 2048 x 2048 output: too few 256-tiles, so 128-tiles
+    gpu.check(l.lten_hip_fc_forward_f32(2048, fin, 2048, dX.ptr, dW.ptr, None, dY.ptr))
     assert gpu.last_kernel() == FAST_TILES[21]
-    assert np.array_equal(dY.numpy(np.float32, (2048, 1024)), x[:2048] @ w[:1024].T)
+    assert np.array_equal(dY.numpy(np.float32, (2048, 2048)), x[:2048] @ w[:2048].T)
+    # 2048 x 1024 and 300 x 3400 outputs (NT): 128-tiles would leave CUs without a workgroup, 64-tiles do not
+    gpu.check(l.lten_hip_fc_forward_f32(2048, fin, 1024, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel() == FAST_TILES[31]
+    assert np.array_equal(dY.numpy(np.float32, (2048, 1024)), x[:2048] @ w[:1024].T + b[:1024])
+    gpu.check(l.lten_hip_fc_forward_f32(300, fin, 3400, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel() == FAST_TILES[31]
+    assert np.array_equal(dY.numpy(np.float32, (300, 3400)), x[:300] @ w[:3400].T + b[:3400])
     # strided batch of 4 (Tensor::matmul over a leading dimension), NN
     a4 = rng.integers(-4, 5, (4, 512, 256)).astype(np.float32)   # 4 x (4 x 8) tiles of 128
     b4 = rng.integers(-4, 5, (4, 256, 1024)).astype(np.float32)
