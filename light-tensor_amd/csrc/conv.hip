@@ -188,8 +188,13 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
 	// one with its four-row tile also where the two-row tile would be picked
-	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
-	if (variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
+	// The patch kernels' tiles are 128 columns wide: on images narrower than 32 columns three quarters of a tile are
+	// padding and the implicit GEMM over the flattened pixels is ahead (64 x 32 x 28 x 28 -> 64 channels: 61 against
+	// 74 us; 8 x 256 x 14 x 14 -> 512: 158 against 325 us, and as many again for the data gradient that runs through here).
+	// (with at most 32 output channels the implicit GEMM's 32 x 128 tile is the slower one: 84 against 73 us)
+	const bool narrow = variant == 0 && g.Wo < 32 && g.Cout > 32;
+	if (!narrow && (variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
+	if (!narrow && variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");
 		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
@@ -308,7 +313,10 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	if (Cout == 0 || HW == 0) return lten_hip_zero(dx, N * Cin * H * W * sizeof(float));
 	LTEN_HIP_REQUIRE(w && dy && workspace, "conv2d_dgrad: null pointer");
 	float* work = static_cast<float*>(workspace);
-	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1) {
+	// Few images of at most 16 columns: l-ten's decomposition (GEMM + col2im per image) is ahead of a convolution on
+	// tiles an eighth full (8 x 256 x 14 x 14 <- 512 channels: 167 against 425 us)
+	const bool few_narrow = get_option(OPT_CONV_VARIANT) == 0 && W <= 16 && N <= 16 && Cin > 32;
+	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1 && !few_narrow) {
 		ConvGeo gt;  // the transposed problem: dy is the input, dx the output
 		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
 		if (get_option(OPT_CONV_VARIANT) == 0 && gt.Ho == (int)H && gt.Wo == (int)W && !conv_smallk_takes(gt) && conv_fewout_takes(gt, dy, dx))
@@ -358,7 +366,9 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		if (int rc = conv_smallk_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
 		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
 	}
-	if (get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
+	// images of at most 16 columns: an eighth of the patch kernel's 128-column tile (8 x 256 x 14 x 14 -> 512: 129 against 199 us)
+	const bool narrow = get_option(OPT_CONV_VARIANT) == 0 && g.Wo <= 16;
+	if (!narrow && get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
 		const int parts = conv_patch_wgrad_parts(g);
 		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
 		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
