@@ -188,12 +188,12 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
 	// one with its four-row tile also where the two-row tile would be picked
-	// The patch kernels' tiles are 128 columns wide: on images narrower than 32 columns three quarters of a tile are
-	// padding and the implicit GEMM over the flattened pixels is ahead (64 x 32 x 28 x 28 -> 64 channels: 61 against
-	// 74 us; 8 x 256 x 14 x 14 -> 512: 158 against 325 us, and as many again for the data gradient that runs through here).
-	// (with at most 32 output channels the implicit GEMM's 32 x 128 tile is the slower one: 84 against 73 us)
+	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
+	// The register-staged patch kernel's tiles are 128 columns wide (the direct-to-LDS one above has 16 x 32 tiles for
+	// narrow images): on images narrower than 32 columns three quarters of a tile are padding and the implicit GEMM over
+	// the flattened pixels is ahead (8 x 256 x 14 x 14 -> 512 channels: 158 against 325 us), unless it has at most 32
+	// output channels to offer its 32 x 128 tile.
 	const bool narrow = variant == 0 && g.Wo < 32 && g.Cout > 32;
-	if (!narrow && (variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
 	if (!narrow && variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");

@@ -23,10 +23,16 @@ namespace lten_hip {
 
 namespace {
 
-template <int BM_, int TH_>
+// VERT: the tile for narrow images, 16 rows x 32 columns: a wavefront owns four rows of 32 pixels (its four MFMA column
+// blocks lie below one another instead of side by side), the patch is [4 channels][18 rows][40 columns].  On a 28 x 28
+// image 77 % of such tiles are pixels that exist, against 22 % of the 128-column tiles.
+template <int BM_, int TH_, bool VERT_ = false>
 struct FastFwd {
 	static_assert(TH_ == 4 || TH_ == 2, "a wavefront owns a whole row of the tile (TH = 4) or half a row (TH = 2)");
-	static constexpr int BM = BM_, MT = BM / 32, TH = TH_, NT = TH, CB = 4, TW = 128, PR = TH + 2, PWS = 136, F4R = 34;
+	static constexpr bool VERT = VERT_;
+	static constexpr int BM = BM_, MT = BM / 32, TH = TH_, NT = VERT ? 4 : TH, CB = 4;
+	static constexpr int TW = VERT ? 32 : 128, TROWS = VERT ? 16 : TH, PR = TROWS + 2, PWS = TW + 8, F4R = PWS / 4;
+	static constexpr int BLOCK_STEP = VERT ? PWS : 32;            // floats between a wavefront's MFMA column blocks in the patch
 	static constexpr int PATCH_F4 = CB * PR * F4R;                 // 816
 	static constexpr int PATCH_LOADS = (PATCH_F4 + 63) / 64;       // 13
 	static constexpr int PATCH_BYTES = PATCH_LOADS * 1024;
@@ -42,19 +48,20 @@ struct FastFwd {
 
 }  // namespace
 
-template <int BM, int TH>
+template <int BM, int TH, bool VERT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 256 ? 2 : 4, BM * TH == 256 ? 2 : 4))) void conv2d_patch_fast_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
 {
-	typedef FastFwd<BM, TH> P;
+	typedef FastFwd<BM, TH, VERT> P;
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[2 * P::STAGE];
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int lrow = lane & 31, half = lane >> 5;
-	const int wrow = TH == 4 ? wave : (wave & 1), wcol = TH == 4 ? 0 : (wave >> 1) * 64;  // this wavefront's row and first column in the tile
+	// this wavefront's (first) row and first column in the tile
+	const int wrow = VERT ? 4 * wave : (TH == 4 ? wave : (wave & 1)), wcol = (VERT || TH == 4) ? 0 : (wave >> 1) * 64;
 	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
-	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TH;
+	const int w0 = (int)(blockIdx.x % tiles_w) * P::TW, h0 = (int)(blockIdx.x / tiles_w) * P::TROWS;
 	const int co0 = blockIdx.y * BM, n = blockIdx.z;
 	const int Kc = g.Cin * 9;
 	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
@@ -112,7 +119,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	auto read_one = [&](float (&fa)[P::MT], float (&fb)[P::NT], const uint8_t* sbase, int s, int e) {
 		const int cp = s / 9, tap = s % 9, ti = tap / 3, tj = tap % 3;
 		if (e < P::MT) fa[e] = *reinterpret_cast<const float*>(sbase + off_a + (e * 32 * 36 + 2 * cp * 9 + tap) * 4);
-		else fb[e - P::MT] = *reinterpret_cast<const float*>(sbase + off_b + ((2 * cp * P::PR + ti) * P::PWS + tj + (e - P::MT) * 32) * 4);
+		else fb[e - P::MT] = *reinterpret_cast<const float*>(sbase + off_b + ((2 * cp * P::PR + ti) * P::PWS + tj + (e - P::MT) * P::BLOCK_STEP) * 4);
 	};
 
 	v16f acc[P::MT][P::NT];
@@ -208,14 +215,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
 	float* yw = y + (((int64_t)n * g.Cout + co0) * g.Ho + ho) * g.Wo + w0 + wcol;
 	const unsigned y_lane = (unsigned)(half * 4 * plane) + lrow;
-	if (co0 + BM <= g.Cout && w0 + P::TW <= g.Wo) {
+	const unsigned y_step = VERT ? (unsigned)g.Wo : 32u;  // from one of the wavefront's column blocks to the next: a row down, or 32 columns on
+	if (co0 + BM <= g.Cout && w0 + P::TW <= g.Wo && (!VERT || h0 + P::TROWS <= g.Ho)) {
 #pragma unroll
 		for (int m = 0; m < P::MT; m++)
 #pragma unroll
 			for (int r = 0; r < 16; r++) {
 				float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
 #pragma unroll
-				for (int t = 0; t < P::NT; t++) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * 32]);  // y is written once and not read here
+				for (int t = 0; t < P::NT; t++) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * y_step]);  // y is written once and not read here
 			}
 		return;
 	}
@@ -226,8 +234,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 			if (co0 + m * 32 + (r >> 2) * 8 + half * 4 + (r & 3) >= g.Cout) continue;
 			float* yr = yw + (m * 32 + (r >> 2) * 8 + (r & 3)) * plane;
 #pragma unroll
-			for (int t = 0; t < P::NT; t++)
-				if (w0 + wcol + t * 32 + lrow < g.Wo) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * 32]);
+			for (int t = 0; t < P::NT; t++) {
+				const bool inside = VERT ? (ho + t < g.Ho && w0 + lrow < g.Wo) : (w0 + wcol + t * 32 + lrow < g.Wo);
+				if (inside) __builtin_nontemporal_store(acc[m][t][r] + bv[m][r], &yr[y_lane + t * y_step]);
+			}
 		}
 }
 
@@ -238,10 +248,27 @@ bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float
 	       (uint64_t)64 * g.Cin * 9 * 4 < (1ull << 31) && ceil_div((uint64_t)g.Cout, 32) < 65536 && g.N < 65536;
 }
 
+// Images of at most 96 output columns take the 16 x 32 tiles (a quarter or more of a 128-column tile would be padding;
+// measured equal at 100 to 112 columns, ahead below: 16 x 64 x 64 x 64 -> 64 channels 77 -> 39 us, 64 x 32 x 28 x 28 -> 64: 61 -> 23 us).
+bool conv_patch_fast_forward_vertical(const ConvGeo& g) { return g.Wo <= 96; }
+
 int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
-	const unsigned tiles_w = (unsigned)ceil_div((uint64_t)g.Wo, 128);
 	const unsigned blocks64 = (unsigned)ceil_div((uint64_t)g.Cout, 64), blocks32 = (unsigned)ceil_div((uint64_t)g.Cout, 32);
+	if (conv_patch_fast_forward_vertical(g) && get_option(OPT_CONV_VARIANT) != 5) {
+		const unsigned vtiles = (unsigned)(ceil_div((uint64_t)g.Wo, 32) * ceil_div((uint64_t)g.Ho, 16));
+		// 64 output channels per workgroup when that still gives every CU two workgroups, else 32
+		if (blocks32 % 2 == 0 && (uint64_t)vtiles * blocks64 * g.N >= 512) {
+			set_kernel_name("conv2d_patch_fast_forward_3x3_64x16x32");
+			conv2d_patch_fast_forward_kernel<64, 4, true><<<dim3(vtiles, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		} else {
+			set_kernel_name("conv2d_patch_fast_forward_3x3_32x16x32");
+			conv2d_patch_fast_forward_kernel<32, 4, true><<<dim3(vtiles, blocks32, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		}
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+	const unsigned tiles_w = (unsigned)ceil_div((uint64_t)g.Wo, 128);
 	const unsigned tiles = tiles_w * (unsigned)ceil_div((uint64_t)g.Ho, 4);
 	if (blocks32 % 2 == 1) {
 		set_kernel_name("conv2d_patch_fast_forward_3x3_32x4x128");

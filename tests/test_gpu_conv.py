@@ -152,6 +152,26 @@ def test_conv_many_tiles(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)
 
 
+@pytest.mark.parametrize("geo", [(3, 8, 28, 28, 64, 3, 3, 1, 1, 1, 1),      # MNIST-sized: one column tile, two row tiles (the second 12 rows of 16)
+                                 (2, 12, 37, 44, 70, 3, 3, 2, 1, 1, 1),     # two column tiles, three row tiles, ragged on every side, row pad 2
+                                 (1, 16, 16, 32, 32, 3, 3, 0, 0, 1, 1),     # no padding: 14 x 30 outputs, 32 channels per workgroup
+                                 (2, 8, 50, 96, 33, 3, 3, 1, 1, 1, 1),      # the widest image that takes these tiles: three column tiles, ragged channels
+                                 (5, 64, 9, 8, 128, 3, 3, 1, 1, 1, 1)])     # a quarter of a tile's columns, two channel blocks of 64
+def test_conv_narrow_images_on_16x32_tiles(gpu, ob, geo):
+    """Images of at most 96 columns: forward (and the stride-1 data gradient through it) on the direct-to-LDS kernel
+    with tiles of 16 rows x 32 columns, against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    y, _, fk = gpu_conv(gpu, geo, x, w, dy, bias)
+    assert fk.startswith("conv2d_patch_fast_forward_3x3_") and fk.endswith("x16x32"), fk
+    _conv_vs_oracle(gpu, ob, geo)
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
