@@ -184,17 +184,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM == 64 ? 
 // (mt, ph) multiplies MFMA row tile mt against all KH*KW tap tiles over pixel half ph of the chunk; one
 // MFMA step takes pixels 2s (lanes 0-31) and 2s + 1 (lanes 32-63).  At the end the two pixel halves are added
 // through LDS and the workgroup writes one partial [Cout][Cin*KH*KW] block; a second kernel adds the parts.
-template <int KH, int KW>
+// V2: the chunk for narrow images, two rows of 32 pixels (pixel p of the chunk: row p / 32, column p % 32): the patch has
+// one row more and 32 columns less.  A 28 x 28 image fills 7/8 of such chunks, against 7/16 of the 64-pixel row segments.
+template <int KH, int KW, bool V2 = false>
 struct PatchWgrad {
 	static constexpr int BM = 64, CIB = 32, TW = 64, T = 256, TAPS = KH * KW;
-	static constexpr int PWS = (4 + TW + KW - 1 + 3) / 4 * 4;
+	static constexpr int CW = V2 ? 32 : 64, CR = V2 ? 2 : 1;  // columns and rows of a chunk
+	static constexpr int PROWS = KH + CR - 1;                // patch rows
+	static constexpr int PWS = (4 + CW + KW - 1 + 3) / 4 * 4;
 	static constexpr int F4_ROW = PWS / 4;
-	static constexpr int CS = (KH * PWS) | 1;  // odd channel stride: 32 channels hit 32 banks
+	static constexpr int CS = (PROWS * PWS) | 1;  // odd channel stride: 32 channels hit 32 banks
 	static constexpr int DYS = TW + 1;
 	static constexpr int DY_FLOATS = BM * DYS, PATCH_FLOATS = CIB * CS;
 	static constexpr int LDS_FLOATS = DY_FLOATS + PATCH_FLOATS;
 	static constexpr int DY_F4 = BM * TW / 4, DY_PER_T = DY_F4 / T;
-	static constexpr int PATCH_F4 = CIB * KH * F4_ROW, P_PER_T = (PATCH_F4 + T - 1) / T;
+	static constexpr int PATCH_F4 = CIB * PROWS * F4_ROW, P_PER_T = (PATCH_F4 + T - 1) / T;
 	static constexpr int TAPS_PER_ROUND = LDS_FLOATS / (2 * 64 * 16);  // taps whose accumulators fit the final exchange
 	static_assert(DY_F4 % T == 0 && TAPS_PER_ROUND >= 1, "tile shape");
 };
@@ -204,11 +208,12 @@ struct PatchWgrad {
 // a workgroup refills its tiles, and a chunk costs one barrier.  Without PIPE: two workgroups per CU, one buffer,
 // store - barrier - multiply - barrier (each workgroup's refill is meant to hide behind the other's MFMAs, which
 // works only when the two are out of step).
-template <int KH, int KW, bool VEC, bool PIPE>
+template <int KH, int KW, bool VEC, bool PIPE, bool V2 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 2, PIPE ? 1 : 2))) void conv2d_patch_wgrad_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy, float* __restrict__ partial, int chunks_per_part)
 {
-	typedef PatchWgrad<KH, KW> P;
+	typedef PatchWgrad<KH, KW, V2> P;
+	static_assert(!V2 || VEC, "the two-row chunk is loaded 16 bytes at a time");
 	__shared__ float lds[(PIPE ? 2 : 1) * P::LDS_FLOATS];
 	float* s_dy = lds;
 	float* s_patch = lds + P::DY_FLOATS;
@@ -216,23 +221,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
 	const int mt = wave & 1, phalf = wave >> 1;
 	const int co0 = blockIdx.y * P::BM, ci0 = blockIdx.z * P::CIB;
-	const int tiles_w = (g.Wo + P::TW - 1) / P::TW;
-	const int total = g.N * g.Ho * tiles_w;
+	const int tiles_w = (g.Wo + P::CW - 1) / P::CW, rows_c = (g.Ho + P::CR - 1) / P::CR;
+	const int total = g.N * rows_c * tiles_w;
 	const int begin = blockIdx.x * chunks_per_part, end = min(total, begin + chunks_per_part);
 
 	float4 rdy[P::DY_PER_T], rp[P::P_PER_T];
 	// What does not change from chunk to chunk is worked out once per lane: the offset of each of its float4s from
 	// the chunk's origin, and the row / column shifts that decide whether the float4 lies inside the image (with
 	// VEC, rows are whole float4s: inside or outside together).  Chunk coordinates advance without divisions.
-	int n_c = begin / (tiles_w * g.Ho), ho_c = (begin / tiles_w) % g.Ho, w0_c = (begin % tiles_w) * P::TW;
+	int n_c = begin / (tiles_w * rows_c), ho_c = ((begin / tiles_w) % rows_c) * P::CR, w0_c = (begin % tiles_w) * P::CW;
 	const int64_t plane_o = (int64_t)g.Ho * g.Wo;
-	const int dy_rel = (int)((tid / (P::TW / 4)) * plane_o) + 4 * (tid % (P::TW / 4));  // + q * 16 rows of dy
+	// this thread's float4 of a dy row of the chunk: pixels 4 (tid % 16) ..: row dy_r of the chunk, columns dy_c ..
+	const int dy_r = (tid % (P::TW / 4)) / (P::CW / 4), dy_c = 4 * ((tid % (P::TW / 4)) % (P::CW / 4));
+	const int dy_rel = (int)((tid / (P::TW / 4)) * plane_o) + dy_r * g.Wo + dy_c;  // + q * 16 rows of dy
 	int x_rel[P::P_PER_T], x_gy[P::P_PER_T], x_gx[P::P_PER_T];
 #pragma unroll
 	for (int q = 0; q < P::P_PER_T; q++) {
 		const int idx = tid + q * P::T;
 		const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
-		const int r = rowid % KH, ci = rowid / KH;
+		const int r = rowid % P::PROWS, ci = rowid / P::PROWS;
 		const bool exists = idx < P::PATCH_F4 && ci0 + ci < g.Cin;
 		x_gx[q] = 4 * f - 4;
 		x_gy[q] = exists ? r - g.ph : -(1 << 30);
@@ -242,7 +249,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 		if (VEC) {
 			const float* dyc = dy + (((int64_t)n_c * g.Cout + co0) * g.Ho + ho_c) * g.Wo + w0_c;
 			const float* xc = x + (((int64_t)n_c * g.Cin + ci0) * g.H + ho_c) * g.W + w0_c;
-			const bool dy_col = w0_c + 4 * (tid % (P::TW / 4)) < g.Wo;
+			const bool dy_col = w0_c + dy_c < g.Wo && ho_c + dy_r < g.Ho;
 #pragma unroll
 			for (int q = 0; q < P::DY_PER_T; q++) {
 				rdy[q] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -279,10 +286,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 		}
 	};
 	auto next_chunk = [&]() {
-		w0_c += P::TW;
+		w0_c += P::CW;
 		if (w0_c >= g.Wo) {
 			w0_c = 0;
-			if (++ho_c == g.Ho) { ho_c = 0; n_c++; }
+			ho_c += P::CR;
+			if (ho_c >= g.Ho) { ho_c = 0; n_c++; }
 		}
 	};
 	auto store_chunk = [&]() {
@@ -296,7 +304,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 		for (int q = 0; q < P::P_PER_T; q++) {
 			const int idx = tid + q * P::T;
 			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
-			float* d = s_patch + (rowid / KH) * P::CS + (rowid % KH) * P::PWS + 4 * f;
+			float* d = s_patch + (rowid / P::PROWS) * P::CS + (rowid % P::PROWS) * P::PWS + 4 * f;
 			if (idx < P::PATCH_F4) { d[0] = rp[q].x; d[1] = rp[q].y; d[2] = rp[q].z; d[3] = rp[q].w; }
 		}
 	};
@@ -308,7 +316,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 		for (int r = 0; r < 16; r++) acc[t][r] = 0.0f;
 
 	const float* pa = s_dy + (mt * 32 + lrow) * P::DYS + phalf * (P::TW / 2) + half;
-	const float* pb = s_patch + lrow * P::CS + phalf * (P::TW / 2) + half + 4 - g.pw;
+	// pixel half phalf of the chunk: the second 32 columns of the row, or (V2) the second row
+	const float* pb = s_patch + lrow * P::CS + (V2 ? phalf * P::PWS : phalf * (P::TW / 2)) + half + 4 - g.pw;
 
 	if (PIPE) {
 		// piece k of the 16 + 4 * P_PER_T four-byte stores that put this thread's share of a chunk into a buffer
@@ -324,7 +333,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(PIPE ? 1 : 
 		for (int q = 0; q < P::P_PER_T; q++) {
 			const int idx = tid + q * P::T;
 			const int f = idx % P::F4_ROW, rowid = idx / P::F4_ROW;
-			off_p[q] = idx < P::PATCH_F4 ? P::DY_FLOATS + (rowid / KH) * P::CS + (rowid % KH) * P::PWS + 4 * f : -1;
+			off_p[q] = idx < P::PATCH_F4 ? P::DY_FLOATS + (rowid / P::PROWS) * P::CS + (rowid % P::PROWS) * P::PWS + 4 * f : -1;
 		}
 		auto store_piece = [&](float* buf, int k) {
 			if (k < 4 * P::DY_PER_T) {
@@ -524,6 +533,21 @@ bool conv_patch_wgrad_takes(const ConvGeo& g)
 	       (uint64_t)g.H * g.W < (1u << 25) && (uint64_t)g.Ho * g.Wo < (1u << 25);  // 32-bit lane offsets over 32 channels
 }
 
+// Whether the weight gradient walks chunks of two rows x 32 columns instead of 64 columns of one row: when that wastes
+// clearly fewer pixels (a 28-column image: 7/8 of a chunk against 7/16) and the rows allow 16-byte loads.
+static bool wgrad_two_row_chunk(const ConvGeo& g, bool vec)
+{
+	if (!vec || get_option(OPT_CONV_VARIANT) != 0) return false;
+	const double wide = (double)g.Wo / (64.0 * (double)ceil_div((uint64_t)g.Wo, 64));
+	const double tall = (double)g.Wo / (32.0 * (double)ceil_div((uint64_t)g.Wo, 32)) * (double)g.Ho / (2.0 * (double)ceil_div((uint64_t)g.Ho, 2));
+	return tall > 1.15 * wide;
+}
+
+static uint64_t wgrad_chunks(const ConvGeo& g, bool two_row)
+{
+	return two_row ? (uint64_t)g.N * ceil_div((uint64_t)g.Ho, 2) * ceil_div((uint64_t)g.Wo, 32) : (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, 64);
+}
+
 // upper_bound: the largest count any kernel choice can give (for sizing the workspace, so that a change of the
 // tuning option between the size query and the call can never make the kernel write past it)
 int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound)
@@ -531,9 +555,9 @@ int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound)
 	typedef PatchWgrad<3, 3> P;
 	// two workgroups per CU over all (co block, ci block) pairs, at least four chunks per part
 	const uint64_t blocks = ceil_div((uint64_t)g.Cout, P::BM) * ceil_div((uint64_t)g.Cin, P::CIB);
-	const uint64_t chunks = (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, P::TW);
 	// one workgroup per CU; two with the unpipelined kernel (rows that do not allow 16-byte loads, or conv_variant 3)
 	const bool vec = g.W % 4 == 0 && g.Wo % 4 == 0;
+	const uint64_t chunks = upper_bound ? std::max(wgrad_chunks(g, false), wgrad_chunks(g, true)) : wgrad_chunks(g, wgrad_two_row_chunk(g, vec));
 	uint64_t parts = std::max<uint64_t>(1, (upper_bound || get_option(OPT_CONV_VARIANT) == 3 || !vec ? 512 : 256) / blocks);
 	parts = std::min<uint64_t>(parts, std::max<uint64_t>(1, chunks / 4));
 	const uint64_t per = ceil_div(chunks, parts);
@@ -543,10 +567,17 @@ int conv_patch_wgrad_parts(const ConvGeo& g, bool upper_bound)
 int conv_patch_wgrad(const ConvGeo& g, const float* x, const float* dy, float* partial, int parts)
 {
 	typedef PatchWgrad<3, 3> P;
-	const uint64_t chunks = (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, P::TW);
-	const int per = (int)ceil_div(chunks, (uint64_t)parts);
 	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
+	const bool two_row = wgrad_two_row_chunk(g, g.W % 4 == 0 && g.Wo % 4 == 0) && vec;
+	const uint64_t chunks = wgrad_chunks(g, two_row);
+	const int per = (int)ceil_div(chunks, (uint64_t)parts);
 	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, P::BM), (unsigned)ceil_div((uint64_t)g.Cin, P::CIB));
+	if (two_row) {
+		set_kernel_name("conv2d_patch_wgrad_3x3_64x32_2x32");
+		conv2d_patch_wgrad_kernel<3, 3, true, true, true><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	if (get_option(OPT_CONV_VARIANT) == 0 && conv_patch_fast_wgrad_takes(g, x, dy)) return conv_patch_fast_wgrad(g, x, dy, partial, parts);
 	set_kernel_name("conv2d_patch_wgrad_3x3_64x32");
 	if (get_option(OPT_CONV_VARIANT) == 3 || !vec) {

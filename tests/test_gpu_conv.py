@@ -172,6 +172,23 @@ def test_conv_narrow_images_on_16x32_tiles(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)
 
 
+@pytest.mark.parametrize("geo", [(3, 16, 27, 28, 64, 3, 3, 1, 1, 1, 1),      # MNIST-sized with an odd number of rows: the last chunk has one
+                                 (2, 40, 9, 96, 33, 3, 3, 0, 1, 1, 1),      # three chunk columns, no row padding, ragged channel blocks
+                                 (4, 9, 5, 20, 5, 3, 3, 1, 1, 1, 1),        # 20 of a chunk's 32 columns, the fewest input channels
+                                 (2, 70, 30, 32, 130, 3, 3, 2, 1, 1, 1)])   # exactly one chunk column, row pad 2, three channel blocks each way
+def test_conv_weight_gradient_on_two_row_chunks(gpu, ob, geo):
+    """Narrow images whose rows allow 16-byte loads: the weight gradient walks chunks of two rows x 32 columns."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    gpu_conv(gpu, geo, x, w, dy, None)
+    assert gpu.last_kernel() == "conv2d_patch_wgrad_3x3_64x32_2x32", gpu.last_kernel()
+    _conv_vs_oracle(gpu, ob, geo)
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
