@@ -46,21 +46,43 @@ struct Chunk {
 	int n, ho, w0;
 };
 
-__device__ __forceinline__ Chunk chunk_at(const ConvGeo& g, int chunk, int tiles_w)
+// How a chunk's 128 pixels lie in the image: 128 columns of one row (a wavefront takes 32 of them), or, for narrow
+// images, 32 columns of four rows (a wavefront takes a row): a 24-column image fills three quarters of such a chunk
+// instead of a fifth.
+struct Tiling {
+	int cw, ch;           // columns and rows of a chunk
+	int tiles_w, rows_c;  // chunks per image row and chunk rows per image
+	int wx, wy;           // this wavefront's first column and its row inside the chunk
+};
+
+__device__ __forceinline__ Tiling make_tiling(const ConvGeo& g, int vert, int wave)
+{
+	Tiling t;
+	t.cw = vert ? 32 : SK_TW;
+	t.ch = vert ? 4 : 1;
+	t.tiles_w = (g.Wo + t.cw - 1) / t.cw;
+	t.rows_c = (g.Ho + t.ch - 1) / t.ch;
+	t.wx = vert ? 0 : wave * 32;
+	t.wy = vert ? wave : 0;
+	return t;
+}
+
+__device__ __forceinline__ Chunk chunk_at(const Tiling& t, int chunk)
 {
 	Chunk c;
-	c.w0 = (chunk % tiles_w) * SK_TW;
-	c.ho = (chunk / tiles_w) % g.Ho;
-	c.n = chunk / (tiles_w * g.Ho);
+	c.w0 = (chunk % t.tiles_w) * t.cw;
+	c.ho = ((chunk / t.tiles_w) % t.rows_c) * t.ch;
+	c.n = chunk / (t.tiles_w * t.rows_c);
 	return c;
 }
 
-__device__ __forceinline__ Chunk next_chunk(const ConvGeo& g, Chunk c)
+__device__ __forceinline__ Chunk next_chunk(const ConvGeo& g, const Tiling& t, Chunk c)
 {
-	c.w0 += SK_TW;
+	c.w0 += t.cw;
 	if (c.w0 >= g.Wo) {
 		c.w0 = 0;
-		if (++c.ho == g.Ho) { c.ho = 0; c.n++; }
+		c.ho += t.ch;
+		if (c.ho >= g.Ho) { c.ho = 0; c.n++; }
 	}
 	return c;
 }
@@ -78,7 +100,7 @@ struct PatchLane {
 };
 
 template <int P_PER_T>
-__device__ __forceinline__ void init_patch_lane(const ConvGeo& g, int wave, int lane, PatchLane<P_PER_T>& p)
+__device__ __forceinline__ void init_patch_lane(const ConvGeo& g, const Tiling& t, int lane, PatchLane<P_PER_T>& p)
 {
 	const int rows = g.Cin * g.kh;
 #pragma unroll
@@ -86,9 +108,9 @@ __device__ __forceinline__ void init_patch_lane(const ConvGeo& g, int wave, int 
 		const int idx = lane + q * 64;
 		const int f = idx % SK_F4_ROW, r = idx / SK_F4_ROW;
 		const int ci = r / g.kh, i = r - ci * g.kh;
-		p.gx[q] = wave * 32 - 4 + 4 * f;
-		p.gy[q] = r < rows ? i - g.ph : -(1 << 30);
-		p.rel[q] = r < rows ? (ci * g.H + i - g.ph) * g.W + p.gx[q] : 0;
+		p.gx[q] = t.wx - 4 + 4 * f;
+		p.gy[q] = r < rows ? t.wy + i - g.ph : -(1 << 30);
+		p.rel[q] = r < rows ? (ci * g.H + t.wy + i - g.ph) * g.W + p.gx[q] : 0;
 	}
 }
 
@@ -131,14 +153,15 @@ __device__ __forceinline__ int tap_offset(const ConvGeo& g, int k)
 // take tap 2s, lanes 32-63 tap 2s + 1.  The weights stay in registers for the whole kernel.
 template <bool VEC, int RC>
 __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ w,
-                                                                    const float* __restrict__ bias, float* __restrict__ y, int chunks_per_group)
+                                                                    const float* __restrict__ bias, float* __restrict__ y, int chunks_per_group, int vert)
 {
 	using S = SkShape<RC>;
 	__shared__ __attribute__((aligned(16))) float s_mem[4 * 2 * S::PATCH];
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, half = lane >> 5;
 	const int K = g.Cin * g.kh * g.kw, steps = (K + 1) / 2;
 	const int co0 = blockIdx.y * 32;
-	const int tiles_w = (g.Wo + SK_TW - 1) / SK_TW, total = g.N * g.Ho * tiles_w;
+	const Tiling tl = make_tiling(g, vert, wave);
+	const int total = g.N * tl.rows_c * tl.tiles_w;
 	const int begin = blockIdx.x * chunks_per_group, end = min(total, begin + chunks_per_group);
 	if (begin >= end) return;
 
@@ -165,17 +188,17 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 
 	// stores: a row of y per register; the address is a part all lanes share plus this lane's offset
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
-	const unsigned y_lane = (unsigned)(half * 4 * plane) + wave * 32 + lrow;
+	const unsigned y_lane = (unsigned)(half * 4 * plane) + tl.wy * g.Wo + tl.wx + lrow;
 	const bool all_channels = co0 + 32 <= g.Cout;
 
 	PatchLane<S::P_PER_T> pr;
-	init_patch_lane(g, wave, lane, pr);
-	Chunk c = chunk_at(g, begin, tiles_w);
+	init_patch_lane(g, tl, lane, pr);
+	Chunk c = chunk_at(tl, begin);
 	fetch_patch<VEC>(g, x, c, pr);
 	store_patch(mine, lane, pr);
 	for (int chunk = begin; chunk < end; chunk++) {
 		const int cur = (chunk - begin) & 1;
-		const Chunk nc = next_chunk(g, c);
+		const Chunk nc = next_chunk(g, tl, c);
 		if (chunk + 1 < end) fetch_patch<VEC>(g, x, nc, pr);
 
 		v16f acc;
@@ -189,7 +212,7 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 		}
 
 		float* yc = y + (((int64_t)c.n * g.Cout + co0) * g.Ho + c.ho) * g.Wo + c.w0;  // same for the whole workgroup
-		if (c.w0 + wave * 32 + lrow < g.Wo) {
+		if (c.w0 + tl.wx + lrow < g.Wo && c.ho + tl.wy < g.Ho) {
 			if (all_channels) {
 #pragma unroll
 				for (int r = 0; r < 16; r++) (yc + ((r >> 2) * 8 + (r & 3)) * plane)[y_lane] = acc[r];
@@ -215,7 +238,7 @@ __global__ __launch_bounds__(256) void conv2d_smallk_forward_kernel(ConvGeo g, c
 // that twice as many loads are in flight per CU for the same number of partial sums.
 template <bool VEC, int RC, int WPG>
 __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g, const float* __restrict__ x, const float* __restrict__ dy,
-                                                                  float* __restrict__ partial, int chunks_per_part)
+                                                                  float* __restrict__ partial, int chunks_per_part, int vert)
 {
 	using S = SkShape<RC>;
 	constexpr int RED = (WPG - 1) * 16 * 64;  // the other wavefronts' accumulator tiles for the final sum
@@ -232,7 +255,8 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 	const int wave = wid & 3;  // which 32 pixels of a chunk
 	const int K = g.Cin * g.kh * g.kw;
 	const int co0 = blockIdx.y * 32, co = co0 + lrow;
-	const int tiles_w = (g.Wo + SK_TW - 1) / SK_TW, total = g.N * g.Ho * tiles_w;
+	const Tiling tl = make_tiling(g, vert, wave);
+	const int total = g.N * tl.rows_c * tl.tiles_w;
 	const int begin = blockIdx.x * chunks_per_part + (wid >> 2), end = min(total, (int)blockIdx.x * chunks_per_part + chunks_per_part);
 
 	float* const mine = s_mem + wid * 2 * S::PATCH;  // this wavefront's two buffers
@@ -243,13 +267,13 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 	// dy: the address is a part all lanes share plus this lane's offset; with VEC (Wo % 4 == 0) the four
 	// pixels of a load are inside or outside the row together
 	const int64_t plane = (int64_t)g.Ho * g.Wo;
-	const unsigned dy_lane = VEC ? (unsigned)(r8 * plane) + wave * 32 + c4 : (unsigned)(lrow * plane) + wave * 32 + 4 * half;
+	const unsigned dy_lane = (VEC ? (unsigned)(r8 * plane) + c4 : (unsigned)(lrow * plane) + 4 * half) + tl.wy * g.Wo + tl.wx;
 	const bool co_ok = co < g.Cout;
 	// VEC: a[i] = rows 8i + r8, pixels c4 .. c4+3 (to be staged); else a[u] = the operand itself
 	auto load_dy = [&](const Chunk& c, float4 (&a)[4]) {
 		const float* dc = dy + (((int64_t)c.n * g.Cout + co0) * g.Ho + c.ho) * g.Wo + c.w0;  // same for the whole workgroup
 		if (VEC) {
-			const bool col_ok = c.w0 + wave * 32 + c4 < g.Wo;
+			const bool col_ok = c.w0 + tl.wx + c4 < g.Wo && c.ho + tl.wy < g.Ho;
 #pragma unroll
 			for (int i = 0; i < 4; i++) {
 				a[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -257,11 +281,11 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 			}
 			return;
 		}
-		const int col = c.w0 + wave * 32 + 4 * half;
+		const int col = c.w0 + tl.wx + 4 * half;
 #pragma unroll
 		for (int u = 0; u < 4; u++) {
 			a[u] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-			if (co_ok) a[u] = load_row4<false>(dc + dy_lane - (wave * 32 + 4 * half) - c.w0, col + 8 * u, g.Wo);
+			if (co_ok && c.ho + tl.wy < g.Ho) a[u] = load_row4<false>(dc + dy_lane - (tl.wx + 4 * half) - c.w0, col + 8 * u, g.Wo);
 		}
 	};
 	// VEC: through the slab into the operand layout
@@ -284,8 +308,8 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 
 	float4 a_cur[4], a_next[4];
 	PatchLane<S::P_PER_T> pr;
-	init_patch_lane(g, wave, lane, pr);
-	Chunk c = chunk_at(g, begin, tiles_w);
+	init_patch_lane(g, tl, lane, pr);
+	Chunk c = chunk_at(tl, begin);
 	if (begin < end) {
 		fetch_patch<VEC>(g, x, c, pr);
 		load_dy(c, a_cur);
@@ -295,7 +319,7 @@ __global__ __launch_bounds__(WPG * 64) void conv2d_smallk_wgrad_kernel(ConvGeo g
 	for (int chunk = begin; chunk < end; chunk += STRIDE) {
 		const int cur = ((chunk - begin) / STRIDE) & 1;
 #pragma unroll
-		for (int q = 0; q < STRIDE; q++) c = next_chunk(g, c);
+		for (int q = 0; q < STRIDE; q++) c = next_chunk(g, tl, c);
 		if (chunk + STRIDE < end) {
 			fetch_patch<VEC>(g, x, c, pr);
 			load_dy(c, a_next);
@@ -380,7 +404,20 @@ bool conv_smallk_takes(const ConvGeo& g)
 // The small kernel size: patch rows fit 8 and the taps fit 8 MFMA steps.
 static bool smallk_small(const ConvGeo& g) { return g.Cin * g.kh <= 8 && g.Cin * g.kh * g.kw <= 16; }
 
-static uint64_t smallk_chunks(const ConvGeo& g) { return (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, SK_TW); }
+// Chunks of four rows x 32 columns instead of 128 columns of one row, when that wastes clearly fewer pixels (l-ten's
+// MNIST layer, 24 output columns: three quarters of a chunk are pixels instead of a fifth).
+static bool smallk_vertical(const ConvGeo& g)
+{
+	const double wide = (double)g.Wo / (128.0 * (double)ceil_div((uint64_t)g.Wo, 128));
+	const double tall = (double)g.Wo / (32.0 * (double)ceil_div((uint64_t)g.Wo, 32)) * (double)g.Ho / (4.0 * (double)ceil_div((uint64_t)g.Ho, 4));
+	return tall > 1.15 * wide;
+}
+
+static uint64_t smallk_chunks(const ConvGeo& g)
+{
+	if (smallk_vertical(g)) return (uint64_t)g.N * ceil_div((uint64_t)g.Ho, 4) * ceil_div((uint64_t)g.Wo, 32);
+	return (uint64_t)g.N * g.Ho * ceil_div((uint64_t)g.Wo, SK_TW);
+}
 
 // Workgroups along x: about `target` over all channel blocks, at least two chunks each (none empty).
 static int smallk_groups(const ConvGeo& g, int target)
@@ -398,14 +435,15 @@ int conv_smallk_forward(const ConvGeo& g, const float* x, const float* w, const 
 	const int per = (int)ceil_div(smallk_chunks(g), (uint64_t)groups);
 	const dim3 grid((unsigned)groups, (unsigned)ceil_div((uint64_t)g.Cout, 32));
 	const bool vec = g.W % 4 == 0 && aligned16(x);
+	const int vert = smallk_vertical(g) ? 1 : 0;
 	if (smallk_small(g)) {
-		set_kernel_name("conv2d_smallk_forward_32x128_r8");
-		if (vec) conv2d_smallk_forward_kernel<true, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
-		else conv2d_smallk_forward_kernel<false, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+		set_kernel_name(vert ? "conv2d_smallk_forward_32x4x32_r8" : "conv2d_smallk_forward_32x128_r8");
+		if (vec) conv2d_smallk_forward_kernel<true, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per, vert);
+		else conv2d_smallk_forward_kernel<false, 8><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per, vert);
 	} else {
-		set_kernel_name("conv2d_smallk_forward_32x128");
-		if (vec) conv2d_smallk_forward_kernel<true, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
-		else conv2d_smallk_forward_kernel<false, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per);
+		set_kernel_name(vert ? "conv2d_smallk_forward_32x4x32" : "conv2d_smallk_forward_32x128");
+		if (vec) conv2d_smallk_forward_kernel<true, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per, vert);
+		else conv2d_smallk_forward_kernel<false, SK_MAXK><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y, per, vert);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
@@ -419,14 +457,15 @@ int conv_smallk_wgrad(const ConvGeo& g, const float* x, const float* dy, float* 
 	const int per = (int)ceil_div(smallk_chunks(g), (uint64_t)parts);
 	const dim3 grid((unsigned)parts, (unsigned)ceil_div((uint64_t)g.Cout, 32));
 	const bool vec = g.W % 4 == 0 && aligned16(x) && g.Wo % 4 == 0 && aligned16(dy);
+	const int vert = smallk_vertical(g) ? 1 : 0;
 	if (smallk_small(g)) {
-		set_kernel_name("conv2d_smallk_wgrad_32x128_r8");
-		if (vec) conv2d_smallk_wgrad_kernel<true, 8, 8><<<grid, dim3(512), 0, stream()>>>(g, x, dy, partial, per);
-		else conv2d_smallk_wgrad_kernel<false, 8, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		set_kernel_name(vert ? "conv2d_smallk_wgrad_32x4x32_r8" : "conv2d_smallk_wgrad_32x128_r8");
+		if (vec) conv2d_smallk_wgrad_kernel<true, 8, 8><<<grid, dim3(512), 0, stream()>>>(g, x, dy, partial, per, vert);
+		else conv2d_smallk_wgrad_kernel<false, 8, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per, vert);
 	} else {
-		set_kernel_name("conv2d_smallk_wgrad_32x128");
-		if (vec) conv2d_smallk_wgrad_kernel<true, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
-		else conv2d_smallk_wgrad_kernel<false, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per);
+		set_kernel_name(vert ? "conv2d_smallk_wgrad_32x4x32" : "conv2d_smallk_wgrad_32x128");
+		if (vec) conv2d_smallk_wgrad_kernel<true, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per, vert);
+		else conv2d_smallk_wgrad_kernel<false, SK_MAXK, 4><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, per, vert);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;

@@ -189,6 +189,25 @@ def test_conv_weight_gradient_on_two_row_chunks(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)
 
 
+@pytest.mark.parametrize("geo", [(64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1),      # l-ten's MNIST conv layer at batch 64: 24 x 24 outputs
+                                 (3, 1, 28, 28, 32, 3, 3, 0, 0, 1, 1),      # 26 columns: no 16-byte loads of dy; 8-row patch variant
+                                 (5, 3, 33, 32, 40, 3, 3, 1, 1, 1, 1),      # three channels, a ragged last chunk row, two channel blocks
+                                 (2, 1, 9, 68, 16, 4, 3, 1, 1, 1, 1)])      # three chunk columns (68 of 96), 12 taps: the 16x16x4 weight gradient
+def test_conv_first_layers_of_narrow_images_on_four_row_chunks(gpu, ob, geo):
+    """Short reductions (Cin * kh * kw <= 32) on images where chunks of four rows x 32 columns waste fewer pixels than 128
+    columns of one row: forward and weight gradient against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    _, _, fk = gpu_conv(gpu, geo, x, w, dy, None)
+    assert fk.startswith("conv2d_smallk_forward_32x4x32"), fk
+    assert gpu.last_kernel().startswith("conv2d_smallk_wgrad_32x4x32"), gpu.last_kernel()
+    _conv_vs_oracle(gpu, ob, geo)
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
