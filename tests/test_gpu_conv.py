@@ -208,6 +208,29 @@ def test_conv_first_layers_of_narrow_images_on_four_row_chunks(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)
 
 
+@pytest.mark.parametrize("geo", [
+    (64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1),   # l-ten's MNIST layer: eight threads an element, 250 products padded to 256
+    (3, 1, 28, 28, 32, 3, 3, 0, 0, 1, 1),    # elements not a multiple of the 32 a workgroup holds
+    (2, 4, 19, 23, 7, 4, 2, 2, 1, 1, 1),     # four input channels, even window, padding on both sides
+    (32, 2, 64, 64, 24, 4, 4, 1, 1, 1, 1),   # 2^18 elements: one thread an element
+    (1, 3, 9, 300, 5, 1, 7, 0, 3, 1, 1),     # one-row window on a wide image
+])
+def test_conv_data_gradient_of_first_layers(gpu, ob, geo):
+    """Data gradient for at most four input channels and a short reduction, outside the 3 x 3 same-size case that the
+    few-output kernel takes: one kernel, products shared by the threads of an element, against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_dgrad_direct", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
