@@ -326,12 +326,14 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 			// Outputs that give 128 x 128 tiles to at most a quarter of the CUs, with a long K: several workgroups share a
 			// tile, each with a slice of K (option "qgemm_split": 0 automatic, 1 off, 2 / 4 / 8 forced).  The exchange of
 			// partial sums between workgroups is dear on this part, so the split pays only there: 1024 x 4096 weights
-			// at M = 256 27 -> 19 us, 2048 x 8192 at M = 128 51 -> 27 us, but 4096 x 4096 at M = 512 30 -> 35 us.
+			// at M = 256 16.5 -> 14.0 us, 8192 x 8192 at M = 128 30.4 -> 25.6 us, but 4096 x 4096 at M = 256 17.3 -> 19.0
+			// us and at M = 512 17.5 -> 26.5 us.
 			const int want = get_option(OPT_QGEMM_SPLIT);
 			const uint64_t tiles = ceil_div(p.M, 128) * ceil_div(p.N, 128);
 			int splits = 1;
 			if (want >= 2) splits = want;
-			else if (want == 0 && tiles <= 64 && p.K >= 4096) splits = tiles <= 32 ? 4 : 2;
+			else if (want == 0 && tiles <= 64 && p.K >= 8192) splits = tiles <= 32 ? 4 : 2;
+			else if (want == 0 && tiles <= 32 && p.K >= 4096) splits = 2;
 			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits, scratch) == 0) return 0;
 			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
 		}

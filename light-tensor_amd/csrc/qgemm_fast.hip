@@ -44,7 +44,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	constexpr int LOADS = STAGE / 1024;    // wave-wide loads per stage
 	constexpr int LPW = LOADS / W;         // per wavefront
 	constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
-	static_assert(LOADS % W == 0 && S == 2 && NS >= 2 && NS % 2 == 0, "pipeline shape");
+	static_assert(LOADS % W == 0 && S >= 2 && S <= 4 && (S - 1) * LPW < 64 && NS >= 2 && NS % 2 == 0, "pipeline shape");
 
 	constexpr int WP = TN + 16;  // row pitch of a wavefront's output strip in LDS (keeps rows 16-byte aligned)
 	static_assert(W * 32 * WP <= S * STAGE, "the output strips fit into the operand stages");
@@ -184,20 +184,40 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		constexpr int FLIP0 = NM - NFLIP;      // flips ride on the last NFLIP MFMAs
 		constexpr int HL = LPW / 2;            // refill loads per beat
 		constexpr int STEP = NM >= HL ? NM / HL : 1;
+		// A beat with as few MFMAs as operands (64 x 64 per wavefront: four and four) would flip each operand behind
+		// the very MFMA that its read rode on, and wait out the LDS latency four times a beat: there the reads go
+		// two at a time behind the first MFMAs (activations first) and all flips behind the last.
+		constexpr bool DENSE = NM <= NR;
 		const uint8_t* sbase = smem + stg * STAGE;
 #pragma unroll
 		for (int m = 0; m < NM; m++) {
 			const int i = m / FM, j = m % FM;
 			acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(cw[i], cx[j], acc[i][j], 0, 0, 0);
-			if (m < NR) {
-				if (m < FN) nw[m] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + m * 32 * BK);
-				else nx[m - FN] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + (m - FN) * 32 * BK);
-			}
-			if (m >= FLIP0) {
-				const int f = m - FLIP0;
-				if (WPRE) nx[f] = flip_sign_bits(nx[f]);
-				else if (f < FN) nw[f] = flip_sign_bits(nw[f]);
-				else nx[f - FN] = flip_sign_bits(nx[f - FN]);
+			if (DENSE) {
+#pragma unroll
+				for (int f = 2 * m; f < 2 * m + 2 && f < NR; f++) {
+					if (f < FM) nx[f] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + f * 32 * BK);
+					else nw[f - FM] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + (f - FM) * 32 * BK);
+				}
+				if (m == NM - 1) {
+#pragma unroll
+					for (int f = 0; f < FM; f++) nx[f] = flip_sign_bits(nx[f]);
+					if (!WPRE) {
+#pragma unroll
+						for (int f = 0; f < FN; f++) nw[f] = flip_sign_bits(nw[f]);
+					}
+				}
+			} else {
+				if (m < NR) {
+					if (m < FN) nw[m] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + m * 32 * BK);
+					else nx[m - FN] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + (m - FN) * 32 * BK);
+				}
+				if (m >= FLIP0) {
+					const int f = m - FLIP0;
+					if (WPRE) nx[f] = flip_sign_bits(nx[f]);
+					else if (f < FN) nw[f] = flip_sign_bits(nw[f]);
+					else nx[f - FN] = flip_sign_bits(nx[f - FN]);
+				}
 			}
 			if (refill) {
 #pragma unroll
@@ -208,10 +228,18 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		}
 	};
 
+	// Waits until at most n whole stages of this wavefront's loads (the youngest ones) are still in flight.  The count
+	// holds only while every stage issues all LPW loads: with a partial last k-step in flight the caller asks for 0.
+	auto wait_stages = [&](int n) {
+		if (S >= 4 && n >= 2) wait_vmcnt<2 * LPW>();
+		else if (S >= 3 && n == 1) wait_vmcnt<LPW>();
+		else wait_vmcnt<0>();
+	};
 	v4i fw0[FN], fx0[FM], fw1[FN], fx1[FM];
 	const int pre = min(S, KT);
 	for (int st = 0; st < pre; st++) issue(st, st);
-	if (pre == 2) wait_vmcnt<LPW>(); else wait_vmcnt<0>();
+	if (S == 2) { if (pre == 2) wait_vmcnt<LPW>(); else wait_vmcnt<0>(); }
+	else wait_stages(TAIL && KT <= S ? 0 : pre - 1);
 	__syncthreads();
 	read_frags(fw0, fx0, 0, 0);
 	flip_frags(fw0, fx0);
@@ -228,25 +256,30 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	};
 
 	int stage = 0, kt = 0;
-	// steady state (branch-free apart from the first k-step's missing half refill): stage kt+1 is in flight
-	// or has landed, stage kt is refilled with k-step kt+2 once everybody has left it
+	// steady state (branch-free apart from the first k-step's missing half refill): k-steps kt+1 .. kt+S-1 are in
+	// flight or have landed (the youngest still lacks the second half of its loads), stage kt is refilled with
+	// k-step kt+S once everybody has left it.  With S = 2 a load has one k-step of MFMAs to land, which covers the
+	// memory latency when a CU holds two 128 x 128 tiles or one of 256 x 256; a CU with a single 128 x 128 tile
+	// needs the deeper ring.
 	for (; kt + S < KT; kt++) {
-		inner_beats(stage, kt > 0 ? 2 : 0, stage ^ 1, kt + 1);
-		wait_vmcnt<0>();
+		const int next = stage + 1 == S ? 0 : stage + 1, prev = stage == 0 ? S - 1 : stage - 1;
+		inner_beats(stage, kt > 0 ? 2 : 0, prev, kt + S - 1);
+		wait_vmcnt<(S - 2) * LPW>();  // k-step kt+1 has landed
 		__syncthreads();
 		// NS is even: the last slice always sits in the second register set
-		beat(fw1, fx1, fw0, fx0, stage ^ 1, 0, 1, stage, kt + S);
-		stage ^= 1;
+		beat(fw1, fx1, fw0, fx0, next, 0, 1, stage, kt + S);
+		stage = next;
 	}
 	// the second half of the last refill: in the first beat of the next k-step as before when there is one
 	const bool half_open = kt > 0;
 	// drain: nothing left to issue
 	for (; kt < KT - 1; kt++) {
-		inner_beats(stage, (half_open && kt + S == KT) ? 2 : 0, stage ^ 1, kt + 1);
-		wait_vmcnt<0>();
+		const int next = stage + 1 == S ? 0 : stage + 1, prev = stage == 0 ? S - 1 : stage - 1;
+		inner_beats(stage, (half_open && kt + S == KT) ? 2 : 0, prev, kt + S - 1);
+		wait_stages(TAIL ? 0 : KT - kt - 2);
 		__syncthreads();
-		beat(fw1, fx1, fw0, fx0, stage ^ 1, 0, 0, 0, 0);
-		stage ^= 1;
+		beat(fw1, fx1, fw0, fx0, next, 0, 0, 0, 0);
+		stage = next;
 	}
 	inner_beats(stage, 0, 0, 0);
 	mma(fw1, fx1);
@@ -419,18 +452,43 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits, const Spli
 	const dim3 grid((unsigned)tiles, (unsigned)splits), block(256);
 	const bool terms = p.rterm != nullptr;
 	const bool wpre = p.b_flip == 0;
-	set_kernel_name(wpre ? "qgemm_fast_128x128x128_w2x2_s2_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s2_splitk");
-#define LTEN_LAUNCH2(OUTV, TERMSV)                                                                              \
-	if (wpre) qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, TERMSV, true, false, true><<<grid, block, 0, stream()>>>(p); \
-	else qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, TERMSV, true, false, false><<<grid, block, 0, stream()>>>(p);
+	// a ring of four stages where a CU holds one workgroup anyway and the share of K is long enough to repay the
+	// longer prologue (see launch_tile128)
+	const bool deep = p.K / splits >= 4096 && tiles * splits <= 256;
+	set_kernel_name(deep ? (wpre ? "qgemm_fast_128x128x128_w2x2_s4_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s4_splitk")
+	                     : (wpre ? "qgemm_fast_128x128x128_w2x2_s2_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s2_splitk"));
+#define LTEN_LAUNCH3(OUTV, TERMSV, WPREV)                                                                           \
+	if (deep) qgemm_fast_kernel<T, BK, 2, 2, 4, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p); \
+	else qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p);
+#define LTEN_LAUNCH2(OUTV, TERMSV) if (wpre) { LTEN_LAUNCH3(OUTV, TERMSV, true) } else { LTEN_LAUNCH3(OUTV, TERMSV, false) }
 #define LTEN_LAUNCH(OUTV) if (terms) { LTEN_LAUNCH2(OUTV, true) } else { LTEN_LAUNCH2(OUTV, false) }
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
 #undef LTEN_LAUNCH
 #undef LTEN_LAUNCH2
+#undef LTEN_LAUNCH3
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
+}
+
+// 128 x 128 tiles for outputs too small to give every CU a 256 x 256 tile.  Two stages let a CU hold two workgroups,
+// whose MFMAs cover each other's load latency; where there is at most one workgroup per CU anyway, a ring of four
+// stages does that, once K is long enough to repay the longer prologue (4096 x 4096 weights at M = 512: 21.6 -> 17.4
+// us, 8192 x 8192 at M = 256: 41.4 -> 30.8 us; 2048 x 2048 at M = 512: 10.0 -> 10.7 us, so not there).
+static int launch_tile128(const QProblem& p, int out, bool ktail, bool wpre)
+{
+	const bool deep = p.K >= 4096 && ceil_div(p.M, 128) * ceil_div(p.N, 128) <= 256;
+	if (deep) {
+		if (wpre) return ktail ? launch_fast<128, 128, 2, 2, 4, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail_wpre")
+		                       : launch_fast<128, 128, 2, 2, 4, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_wpre");
+		return ktail ? launch_fast<128, 128, 2, 2, 4, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail")
+		             : launch_fast<128, 128, 2, 2, 4>(p, out, "qgemm_fast_128x128x128_w2x2_s4");
+	}
+	if (wpre) return ktail ? launch_fast<128, 128, 2, 2, 2, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail_wpre")
+	                       : launch_fast<128, 128, 2, 2, 2, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_wpre");
+	return ktail ? launch_fast<128, 128, 2, 2, 2, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail")
+	             : launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
 }
 
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
@@ -455,11 +513,7 @@ int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 	// the same tile with the wavefronts laid out the other way round (raw weights only)
 	case 34: return wpre ? -1 : launch_fast<256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
 	// 128 x 128 tiles for outputs too small to give every CU a 256 x 256 tile
-	case 41:
-		if (wpre) return ktail ? launch_fast<128, 128, 2, 2, 2, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail_wpre")
-		                       : launch_fast<128, 128, 2, 2, 2, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_wpre");
-		return ktail ? launch_fast<128, 128, 2, 2, 2, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail")
-		             : launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
+	case 41: return launch_tile128(p, out, ktail, wpre);
 	default: return -1;
 	}
 }

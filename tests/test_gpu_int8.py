@@ -208,6 +208,34 @@ def test_batch_sizes_between_the_tile_sizes(gpu):
         assert np.array_equal(dC.numpy(np.uint8, (M, N)), requant_numpy(want, mult, zp[2]))
 
 
+@pytest.mark.parametrize("shape", [
+    (384, 1536, 4096, "qgemm_fast_128x128x128_w2x2_s4"),          # 36 tiles, one per CU: the ring of four stages
+    (300, 1540, 4112, "qgemm_fast_128x128x128_w2x2_s4_ktail"),    # the same with ragged edges and a partial last k-step
+    (384, 1536, 8192, "qgemm_fast_128x128x128_w2x2_s4_splitk"),   # 36 tiles, K in two shares of 4096
+    (130, 1024, 512 * 5, "qgemm_fast_128x128x128_w2x2_s2"),       # K below 4096: two stages
+    (1024, 4096, 640, "qgemm_fast_128x128x128_w2x2_s2"),          # five k-steps, one workgroup per CU
+])
+def test_128_tiles_ring_depth(gpu, shape):
+    """Where a CU holds a single 128 x 128 tile and K is at least 4096 the stages form a ring of four (three k-steps
+    in flight), otherwise of two: int32 sums against the closed form, bytes against the requantize of those sums."""
+    M, N, K, kernel = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    zp, sc = [11, 140, 120], [0.02, 0.02, 3.0]
+    bias = rng.integers(-9000, 9000, N).astype(np.int32)
+    dA, dB, dBias = gpu.DeviceBuffer.from_numpy(A), gpu.DeviceBuffer.from_numpy(B), gpu.DeviceBuffer.from_numpy(bias)
+    dC, dacc, ws = gpu.DeviceBuffer(M * N), gpu.DeviceBuffer(4 * M * N), gpu.DeviceBuffer(4 * (M + N))
+    qp = gpu.qparams3(sc, zp)
+    gpu.quantized_matmul_acc(False, True, M, N, K, dA, dB, dacc, qp, dBias, ws)
+    assert gpu.last_kernel() == kernel, gpu.last_kernel()
+    want = exact_acc(A, B, zp[0], zp[1]) + bias[None, :]
+    assert np.array_equal(dacc.numpy(np.int32, (M, N)), want)
+    gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, dBias, ws)
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    assert np.array_equal(dC.numpy(np.uint8, (M, N)), requant_numpy(want, mult, zp[2]))
+
+
 def test_medium_batch_picks_128_tiles(gpu, ob):
     """512 x 1024 x 1024: 8 tiles of 256x256 would occupy 8 CUs; the library takes 32 tiles of 128x128."""
     rng = np.random.default_rng(77)
@@ -239,7 +267,7 @@ def test_split_k_tiles_forced(gpu, ob, splits):
 
 
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
-    """256 x 1024 x 4096 (16 tiles): the library splits K in four; the closed form in int64 is the check.  With the
+    """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
     rng = np.random.default_rng(5)
     M, N, K = 256, 1024, 4096
