@@ -323,6 +323,9 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 		// workgroups, two per CU) below that.
 		if (p.K >= 512) {
 			if (ceil_div(p.M, 256) * ceil_div(p.N, 256) > 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+			// about one 256 x 128 tile per CU: less operand traffic per MFMA than two 128 x 128 tiles per CU
+			const uint64_t tiles_256x128 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
+			if (tiles_256x128 > 160 && tiles_256x128 <= 256 && p.K >= 2048 && qgemm_fast_dispatch(p, out, 51) == 0) return 0;
 			// Outputs that give 128 x 128 tiles to at most a quarter of the CUs, with a long K: several workgroups share a
 			// tile, each with a slice of K (option "qgemm_split": 0 automatic, 1 off, 2 / 4 / 8 forced).  The exchange of
 			// partial sums between workgroups is dear on this part, so the split pays only there: 1024 x 4096 weights

@@ -1,7 +1,7 @@
 // Tuned int8 GEMM tiles for large NT problems (both operands contiguous in K, K a multiple of 16 and at least
 // one k-step long, N a multiple of 4; M and N need not be multiples of the tile: a load that would start past
 // the last row of an operand fetches the last row instead, and what is computed from it is not stored):
-// T x T output tile (256 or 128), k-steps of BK bytes, a ring of S LDS stages filled by direct global->LDS loads
+// BM x BN output tile (256 x 256, 256 x 128 or 128 x 128), k-steps of BK bytes, a ring of S LDS stages filled by direct global->LDS loads
 // (no register staging), MFMA 32x32x32 int8.
 //
 // Data path per k-step: every wavefront issues its share of the stage's wave-wide 16-byte-per-lane
@@ -32,10 +32,9 @@
 
 namespace lten_hip {
 
-template <int T, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false, bool TAIL = false, bool WPRE = false>
+template <int BM, int BN, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false, bool TAIL = false, bool WPRE = false>
 __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 {
-	constexpr int BM = T, BN = T;  // square output tile, 256 or 128
 	constexpr int W = WM * WN;
 	constexpr int CPR = BK / 16;           // 16-byte chunks per tile row
 	constexpr int RPL = 64 / CPR;          // tile rows covered by one wave-wide load
@@ -76,8 +75,9 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 
 	// ---- global -> LDS: what this lane fetches for each of its wavefront's loads.  Load q covers rows
 	// q*RPL .. q*RPL+RPL-1 of the stacked [A tile; B tile]; wavefront w issues loads w, w+W, w+2W, ...,
-	// so its first LPW/2 loads are A rows and the rest B rows whatever w is.
-	static_assert((BM / RPL) % W == 0 && LPW % 4 == 0, "A and B loads split evenly over the wavefronts and the two refill beats");
+	// so its first BM / RPL / W loads are A rows and the rest B rows whatever w is.
+	static_assert((BM / RPL) % W == 0 && (BN / RPL) % W == 0 && LPW % 2 == 0, "A and B loads split evenly over the wavefronts and the two refill beats");
+	constexpr int NA = BM / RPL / W;  // a wavefront's loads of A rows; the rest are B rows
 	uint32_t voff[LPW];
 	uint32_t lds_slot[LPW];
 	bool in_tail[LPW];  // TAIL: this lane's chunk lies inside the last, partial k-step
@@ -87,7 +87,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		const int q = wave + i * W;
 		const int r = q * RPL + lane / CPR;
 		const int kc = (lane % CPR) ^ swz<CPR>(r);
-		voff[i] = (i < LPW / 2 ? (uint32_t)min(m0 + r, p.M - 1) : (uint32_t)min(n0 + r - BM, p.N - 1)) * (uint32_t)p.K + kc * 16;
+		voff[i] = (i < NA ? (uint32_t)min(m0 + r, p.M - 1) : (uint32_t)min(n0 + r - BM, p.N - 1)) * (uint32_t)p.K + kc * 16;
 		lds_slot[i] = smem_addr + q * 1024;
 		in_tail[i] = kc * 16 < p.K % BK;
 	}
@@ -100,14 +100,14 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	auto load_one = [&](int i, int stage, int kt) {
 		if (TAIL && kt == KT - 1 && p.K % BK != 0) {
 			if (in_tail[i]) {
-				async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
-			} else if (i < LPW / 2) {
+				async_load16(lds_slot[i] + stage * STAGE, (i < NA ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
+			} else if (i < NA) {
 				const v4i pad = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
 				*reinterpret_cast<v4i*>(smem + (lds_slot[i] - smem_addr) + stage * STAGE + lane * 16) = pad;
 			}
 			return;
 		}
-		async_load16(lds_slot[i] + stage * STAGE, (i < LPW / 2 ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
+		async_load16(lds_slot[i] + stage * STAGE, (i < NA ? a_base : b_base) + (int64_t)kt * BK, voff[i]);
 	};
 	auto issue = [&](int stage, int kt) {
 #pragma unroll
@@ -392,18 +392,18 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	}
 }
 
-template <int T, int BK, int WM, int WN, int S, bool TAIL = false, bool WPRE = false>
+template <int BM, int BN, int BK, int WM, int WN, int S, bool TAIL = false, bool WPRE = false>
 static int launch_fast(const QProblem& p, int out, const char* name)
 {
 	if (!TAIL && p.K % BK != 0) return -1;
-	const dim3 grid((unsigned)(ceil_div(p.M, T) * ceil_div(p.N, T))), block(WM * WN * 64);
+	const dim3 grid((unsigned)(ceil_div(p.M, BM) * ceil_div(p.N, BN))), block(WM * WN * 64);
 	const bool terms = p.rterm != nullptr;
 	set_kernel_name(name);
 #define LTEN_LAUNCH(OUTV)                                                                                            \
 	if (terms)                                                                                                   \
-		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, true, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);      \
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, true, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);      \
 	else                                                                                                         \
-		qgemm_fast_kernel<T, BK, WM, WN, S, OUTV, false, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, false, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
@@ -458,8 +458,8 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits, const Spli
 	set_kernel_name(deep ? (wpre ? "qgemm_fast_128x128x128_w2x2_s4_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s4_splitk")
 	                     : (wpre ? "qgemm_fast_128x128x128_w2x2_s2_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s2_splitk"));
 #define LTEN_LAUNCH3(OUTV, TERMSV, WPREV)                                                                           \
-	if (deep) qgemm_fast_kernel<T, BK, 2, 2, 4, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p); \
-	else qgemm_fast_kernel<T, BK, 2, 2, 2, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p);
+	if (deep) qgemm_fast_kernel<T, T, BK, 2, 2, 4, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p); \
+	else qgemm_fast_kernel<T, T, BK, 2, 2, 2, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p);
 #define LTEN_LAUNCH2(OUTV, TERMSV) if (wpre) { LTEN_LAUNCH3(OUTV, TERMSV, true) } else { LTEN_LAUNCH3(OUTV, TERMSV, false) }
 #define LTEN_LAUNCH(OUTV) if (terms) { LTEN_LAUNCH2(OUTV, true) } else { LTEN_LAUNCH2(OUTV, false) }
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
@@ -480,21 +480,21 @@ static int launch_tile128(const QProblem& p, int out, bool ktail, bool wpre)
 {
 	const bool deep = p.K >= 4096 && ceil_div(p.M, 128) * ceil_div(p.N, 128) <= 256;
 	if (deep) {
-		if (wpre) return ktail ? launch_fast<128, 128, 2, 2, 4, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail_wpre")
-		                       : launch_fast<128, 128, 2, 2, 4, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_wpre");
-		return ktail ? launch_fast<128, 128, 2, 2, 4, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail")
-		             : launch_fast<128, 128, 2, 2, 4>(p, out, "qgemm_fast_128x128x128_w2x2_s4");
+		if (wpre) return ktail ? launch_fast<128, 128, 128, 2, 2, 4, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail_wpre")
+		                       : launch_fast<128, 128, 128, 2, 2, 4, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_wpre");
+		return ktail ? launch_fast<128, 128, 128, 2, 2, 4, true>(p, out, "qgemm_fast_128x128x128_w2x2_s4_ktail")
+		             : launch_fast<128, 128, 128, 2, 2, 4>(p, out, "qgemm_fast_128x128x128_w2x2_s4");
 	}
-	if (wpre) return ktail ? launch_fast<128, 128, 2, 2, 2, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail_wpre")
-	                       : launch_fast<128, 128, 2, 2, 2, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_wpre");
-	return ktail ? launch_fast<128, 128, 2, 2, 2, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail")
-	             : launch_fast<128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
+	if (wpre) return ktail ? launch_fast<128, 128, 128, 2, 2, 2, true, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail_wpre")
+	                       : launch_fast<128, 128, 128, 2, 2, 2, false, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_wpre");
+	return ktail ? launch_fast<128, 128, 128, 2, 2, 2, true>(p, out, "qgemm_fast_128x128x128_w2x2_s2_ktail")
+	             : launch_fast<128, 128, 128, 2, 2, 2>(p, out, "qgemm_fast_128x128x128_w2x2_s2");
 }
 
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
-	// K: any multiple of 16 at least one k-step long (variants 33 and 41), or a multiple of the k-step
+	// K: any multiple of 16 at least one k-step long (variants 33, 41 and 51), or a multiple of the k-step
 	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % 16 == 0 && p.K >= 128 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
@@ -506,14 +506,22 @@ int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 	// 256 x 256 tiles: eight wavefronts of 64 x 128 (the activation operand is the one with fewer fragments
 	// per wavefront, so prepared weights leave two fragments per k-slice to flip)
 	case 33:
-		if (wpre) return ktail ? launch_fast<256, 128, 4, 2, 2, true, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_ktail_wpre")
-		                       : launch_fast<256, 128, 4, 2, 2, false, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_wpre");
-		return ktail ? launch_fast<256, 128, 4, 2, 2, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_ktail")
-		             : launch_fast<256, 128, 4, 2, 2>(p, out, "qgemm_fast_256x256x128_w4x2_s2");
+		if (wpre) return ktail ? launch_fast<256, 256, 128, 4, 2, 2, true, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_ktail_wpre")
+		                       : launch_fast<256, 256, 128, 4, 2, 2, false, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_wpre");
+		return ktail ? launch_fast<256, 256, 128, 4, 2, 2, true>(p, out, "qgemm_fast_256x256x128_w4x2_s2_ktail")
+		             : launch_fast<256, 256, 128, 4, 2, 2>(p, out, "qgemm_fast_256x256x128_w4x2_s2");
 	// the same tile with the wavefronts laid out the other way round (raw weights only)
-	case 34: return wpre ? -1 : launch_fast<256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
+	case 34: return wpre ? -1 : launch_fast<256, 256, 128, 2, 4, 2>(p, out, "qgemm_fast_256x256x128_w2x4_s2");
 	// 128 x 128 tiles for outputs too small to give every CU a 256 x 256 tile
 	case 41: return launch_tile128(p, out, ktail, wpre);
+	// 256 x 128 tiles, four wavefronts of 64 x 128, three stages (144 KB): for outputs that give every CU about one such
+	// tile and too few 256 x 256 ones; a k-step brings 48 KB through the CU's vector L1 for 1024 clocks of MFMAs where
+	// two 128 x 128 tiles bring 64 KB (2048 x 4096 x 4096: 36.1 -> 32.8 us)
+	case 51:
+		if (wpre) return ktail ? launch_fast<256, 128, 128, 4, 1, 3, true, true>(p, out, "qgemm_fast_256x128x128_w4x1_s3_ktail_wpre")
+		                       : launch_fast<256, 128, 128, 4, 1, 3, false, true>(p, out, "qgemm_fast_256x128x128_w4x1_s3_wpre");
+		return ktail ? launch_fast<256, 128, 128, 4, 1, 3, true>(p, out, "qgemm_fast_256x128x128_w4x1_s3_ktail")
+		             : launch_fast<256, 128, 128, 4, 1, 3>(p, out, "qgemm_fast_256x128x128_w4x1_s3");
 	default: return -1;
 	}
 }

@@ -176,6 +176,50 @@ def test_direct_to_lds_tiles_partial_last_k_step(gpu, ob, variant, shape):
     run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=variant)
 
 
+@pytest.mark.parametrize("shape", [(256, 128, 128), (512, 384, 640), (300, 272, 400), (520, 392, 2064), (1, 16, 256), (257, 132, 1152)])
+def test_direct_to_lds_256x128_tiles(gpu, ob, shape):
+    """The 256 x 128 form (four wavefronts of 64 x 128, three stages), forced by option on shapes the oracle finishes:
+    whole and ragged tiles, K with and without a partial last k-step, N a multiple of 16 or of 4 only; with and
+    without zero-point terms and bias, exact-convert epilogue; prepared weights give the same bytes."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8), tile=51)
+    assert gpu.last_kernel() == "qgemm_fast_256x128x128_w4x1_s3" + ("_ktail" if K % 128 else ""), gpu.last_kernel()
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8), bias=bias, tile=51)
+    run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 128, 9], np.uint8), tile=51)
+    l = gpu.lib()
+    gpu.set_option("qgemm_tile", 51)
+    try:
+        sc, zp = [0.02, 0.013, 0.9 * K / 512], [200, 17, 99]
+        want, k0 = fcq(gpu, l.lten_hip_fcq_forward, A, B, sc, zp, bias)
+        got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, A, B, sc, zp, bias, prepared=True)
+    finally:
+        gpu.set_option("qgemm_tile", 0)
+    assert k0.startswith("qgemm_fast_256x128") and k1 == k0 + "_wpre", (k0, k1)
+    assert np.array_equal(got, want)
+
+
+def test_256x128_tiles_are_picked_for_about_one_tile_per_cu(gpu):
+    """2048 x 2688 x 2048: 88 tiles of 256 x 256 would leave most CUs idle, 336 of 128 x 128 bring more operand bytes
+    per MFMA; the library takes 168 tiles of 256 x 128.  Closed form in fp64 (exact) as the check."""
+    M, N, K = 2048, 2688, 2048
+    rng = np.random.default_rng(51)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    zp, sc = [11, 140, 120], [0.02, 0.02, 3.0]
+    bias = rng.integers(-9000, 9000, N).astype(np.int32)
+    dA, dB, dBias = gpu.DeviceBuffer.from_numpy(A), gpu.DeviceBuffer.from_numpy(B), gpu.DeviceBuffer.from_numpy(bias)
+    dC, ws = gpu.DeviceBuffer(M * N), gpu.DeviceBuffer(4 * (M + N))
+    gpu.quantized_matmul(False, True, M, N, K, dA, dB, dC, gpu.qparams3(sc, zp), dBias, ws)
+    assert gpu.last_kernel() == "qgemm_fast_256x128x128_w4x1_s3", gpu.last_kernel()
+    want = exact_acc(A, B, zp[0], zp[1]) + bias[None, :]
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    assert np.array_equal(dC.numpy(np.uint8, (M, N)), requant_numpy(want, mult, zp[2]))
+
+
 @pytest.mark.parametrize("variant", [33, 34])
 def test_direct_to_lds_256_tiles_ragged(gpu, ob, variant):
     """300 x 272 x 640 on 256 x 256 tiles: two row tiles and two column tiles, all of them edge tiles."""
