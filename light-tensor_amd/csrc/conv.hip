@@ -50,12 +50,12 @@ __global__ __launch_bounds__(256) void col2im_kernel(const T* col, ConvGeo g, T*
 	}
 }
 
-// Per reduction index k = (ci, i, j): offset of the tap inside one image and the tap coordinates.
+// Per reduction index k = (ci, i, j): where the tap lies relative to the top left tap of channel 0, and which tap it is.
 struct KTap {
 	int off;  // (ci*H + i*dh)*W + j*dw
 	int ij;   // i*dh | (j*dw) << 16
 };
-constexpr int MAX_KTAB = 2304;  // Cin*kh*kw up to 2304 (e.g. 256 channels of 3x3) use the LDS table
+constexpr int MAX_KTAB = 4096;  // Cin*kh*kw up to 4096 (e.g. 448 channels of 3x3) use the LDS table
 
 __device__ __forceinline__ KTap make_tap(const ConvGeo& g, int k)
 {
@@ -66,79 +66,99 @@ __device__ __forceinline__ KTap make_tap(const ConvGeo& g, int k)
 	return t;
 }
 
-// Forward: y[n][co][hw] = sum_k w[co][k] * col_n[k][hw]  (+ bias[co]).  GEMM rows = co, columns = hw.
+// Forward: y[n][co][hw] = sum_k w[co][k] * col_n[k][hw]  (+ bias[co]).  GEMM rows = co, columns = the pixels of the
+// whole batch (n, hw) in one run, so that small images fill the column tiles together.  A thread stages the same
+// column in every k-step (the tile's columns divide the workgroup's threads), so its pixel is decomposed once; every
+// load is issued whatever the position, from an address that lies inside the operand (see GemmCore::run).
 template <int BM, int BN, int BK, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, const float* x, const float* w, const float* bias, float* y)
 {
 	typedef GemmCore<BM, BN, BK, WM, WN, false, true> Core;
+	static_assert(Core::T % BN == 0 && (BM * BK) % Core::T == 0 && (BN * BK) % Core::T == 0, "a thread's column is the same in every fetch");
 	__shared__ float lds[Core::LDS_FLOATS];
 	__shared__ KTap ktab[MAX_KTAB];
+	__shared__ int col_img[BN], col_hw[BN];  // for the stores: image and pixel of every column of the tile (-1: none)
 
 	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
-	const int tiles_n = (HW + BN - 1) / BN;
-	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
-	const float* xi = x + (int64_t)blockIdx.z * g.Cin * g.H * g.W;
-	float* yi = y + (int64_t)blockIdx.z * g.Cout * HW;
+	const int cols = g.N * HW;  // below 2^31 (checked by the host)
+	const int tiles_n = (int)(((int64_t)cols + BN - 1) / BN);
+	const int m0 = (blockIdx.x / tiles_n) * BM;
+	const int n0 = (blockIdx.x % tiles_n) * BN;
 	const bool use_tab = Kc <= MAX_KTAB;
 	if (use_tab) {
-		for (int k = threadIdx.x; k < Kc; k += WM * WN * 64) ktab[k] = make_tap(g, k);
-		__syncthreads();
+		for (int k = threadIdx.x; k < Kc; k += Core::T) ktab[k] = make_tap(g, k);
 	}
+	// this thread's column
+	const unsigned col = (unsigned)n0 + threadIdx.x % BN;
+	const bool col_ok = col < (unsigned)cols;
+	const int img = (int)(min(col, (unsigned)cols - 1) / (unsigned)HW), hw = (int)(min(col, (unsigned)cols - 1) - (unsigned)img * HW);
+	const int ho = hw / g.Wo, wo = hw - ho * g.Wo;
+	const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
+	const float* xi = x + (int64_t)img * g.Cin * g.H * g.W;
+	const int pix = yy * g.W + xx;  // the top left tap of channel 0 (may lie outside the image)
+	if (threadIdx.x < BN) {
+		col_img[threadIdx.x] = col_ok ? img : -1;
+		col_hw[threadIdx.x] = hw;
+	}
+	__syncthreads();
 
-	auto fetch_a = [&](int row, int k) -> float {
-		const int co = m0 + row;
-		return (co < g.Cout && k < Kc) ? w[(int64_t)co * Kc + k] : 0.0f;
+	auto fetch_a = [&](int row, int k, bool& inside) -> float {
+		inside = m0 + row < g.Cout && k < Kc;
+		return w[(int64_t)min(m0 + row, g.Cout - 1) * Kc + min(k, Kc - 1)];
 	};
-	auto fetch_b = [&](int row, int k) -> float {
-		const int n = n0 + row;
-		if (n >= HW || k >= Kc) return 0.0f;
-		const int ho = n / g.Wo, wo = n - ho * g.Wo;
-		const KTap t = use_tab ? ktab[k] : make_tap(g, k);
-		const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
+	auto fetch_b = [&](int, int k, bool& inside) -> float {
+		const KTap t = use_tab ? ktab[min(k, Kc - 1)] : make_tap(g, min(k, Kc - 1));
 		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
-		if ((unsigned)ty >= (unsigned)g.H || (unsigned)tx >= (unsigned)g.W) return 0.0f;
-		return xi[t.off + yy * g.W + xx];
+		inside = col_ok && k < Kc && (unsigned)ty < (unsigned)g.H && (unsigned)tx < (unsigned)g.W;
+		return xi[inside ? pix + t.off : 0];
 	};
 
 	v16f acc[Core::FM][Core::FN];
 	Core::run(lds, 0, Kc, fetch_a, fetch_b, acc);
-	Core::for_each(acc, [&](int row, int col, float v) {
-		const int co = m0 + row, n = n0 + col;
-		if (co < g.Cout && n < HW) yi[(int64_t)co * HW + n] = bias ? v + bias[co] : v;
+	Core::for_each(acc, [&](int row, int c, float v) {
+		const int co = m0 + row, im = col_img[c];
+		if (co < g.Cout && im >= 0) y[((int64_t)im * g.Cout + co) * HW + col_hw[c]] = bias ? v + bias[co] : v;
 	});
 }
 
-// Weight gradient: dw[co][k] = sum_n sum_hw dy[n][co][hw] * col_n[k][hw].  GEMM rows = co, columns = k,
-// reduction over hw.  Workgroup (tile, image, slice) reduces one slice of one image's hw range and writes
-// a partial [Cout x Kc] matrix; conv_reduce_partials adds the partials in a fixed order.
+// Weight gradient: dw[co][k] = sum_n sum_hw dy[n][co][hw] * col_n[k][hw].  GEMM rows = co, columns = k, reduction
+// over the pixels of the whole batch (n, hw) in one run.  Workgroup (tile, slice) reduces one slice of that run and
+// writes a partial [Cout x Kc] matrix; conv_reduce_partials adds the partials in a fixed order.  A thread stages the
+// same pixel offset of every k-step, so the pixel is decomposed once per step; loads are unconditional as in the
+// forward kernel.
 template <int BM, int BN, int BK, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, const float* x, const float* dy, float* partial, int slices, int slice_len)
+__global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, const float* x, const float* dy, float* partial, int64_t slice_len)
 {
 	typedef GemmCore<BM, BN, BK, WM, WN, false, false> Core;
+	static_assert(Core::T % BK == 0 && (BM * BK) % Core::T == 0 && (BN * BK) % Core::T == 0, "a thread's pixel offset is the same in every fetch of a step");
 	__shared__ float lds[Core::LDS_FLOATS];
+	__shared__ KTap ktab[BN];
 
 	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	const int R = g.N * HW;  // below 2^31 (checked by the host)
 	const int tiles_n = (Kc + BN - 1) / BN;
 	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
-	const int img = blockIdx.z / slices, slice = blockIdx.z % slices;
-	const int r0 = slice * slice_len, r1 = min(HW, r0 + slice_len);
-	const float* xi = x + (int64_t)img * g.Cin * g.H * g.W;
-	const float* dyi = dy + (int64_t)img * g.Cout * HW;
-	float* out = partial + (int64_t)blockIdx.z * g.Cout * Kc;
+	const int r0 = (int)(blockIdx.y * slice_len), r1 = (int)min((int64_t)R, r0 + slice_len);
+	float* out = partial + (int64_t)blockIdx.y * g.Cout * Kc;
+	if (threadIdx.x < BN) ktab[threadIdx.x] = make_tap(g, min(n0 + (int)threadIdx.x, Kc - 1));
+	__syncthreads();
+	const int64_t in_image = (int64_t)g.Cin * g.H * g.W;
 
-	auto fetch_a = [&](int row, int r) -> float {
-		const int co = m0 + row;
-		return (co < g.Cout && r < r1) ? dyi[(int64_t)co * HW + r] : 0.0f;
+	auto fetch_a = [&](int row, int rr, bool& inside) -> float {
+		const int r = min(rr, r1 - 1);
+		const int img = r / HW, hw = r - img * HW;
+		inside = m0 + row < g.Cout && rr < r1;
+		return dy[((int64_t)img * g.Cout + min(m0 + row, g.Cout - 1)) * HW + hw];
 	};
-	auto fetch_b = [&](int row, int r) -> float {
-		const int k = n0 + row;
-		if (k >= Kc || r >= r1) return 0.0f;
-		const KTap t = make_tap(g, k);
-		const int ho = r / g.Wo, wo = r - ho * g.Wo;
+	auto fetch_b = [&](int row, int rr, bool& inside) -> float {
+		const int r = min(rr, r1 - 1);
+		const int img = r / HW, hw = r - img * HW;
+		const int ho = hw / g.Wo, wo = hw - ho * g.Wo;
+		const KTap t = ktab[row];
 		const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
 		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
-		if ((unsigned)ty >= (unsigned)g.H || (unsigned)tx >= (unsigned)g.W) return 0.0f;
-		return xi[t.off + yy * g.W + xx];
+		inside = n0 + row < Kc && rr < r1 && (unsigned)ty < (unsigned)g.H && (unsigned)tx < (unsigned)g.W;
+		return x[img * in_image + (inside ? yy * g.W + xx + t.off : 0)];
 	};
 
 	v16f acc[Core::FM][Core::FN];
@@ -165,16 +185,16 @@ static int make_geo(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W
 	return 0;
 }
 
-static void wgrad_split(const ConvGeo& g, int& slices, int& slice_len)
+// The implicit-GEMM weight gradient cuts the batch's run of pixels into slices: enough (tile, slice) pairs to fill 256
+// CUs four times over, slices a multiple of the k-step and at least 256 pixels long.
+static void wgrad_split(const ConvGeo& g, int& slices, int64_t& slice_len)
 {
-	// enough (image, slice) pairs to fill 256 CUs a few times over, slices a multiple of the k-step
-	const int HW = g.Ho * g.Wo;
-	int want = (int)ceil_div(256, (uint64_t)g.N);
-	if (want < 1) want = 1;
-	slice_len = (int)ceil_div((uint64_t)HW, (uint64_t)want);
-	slice_len = (int)(ceil_div((uint64_t)slice_len, 64) * 64);
+	const uint64_t R = (uint64_t)g.N * g.Ho * g.Wo, Kc = (uint64_t)g.Cin * g.kh * g.kw;
+	const uint64_t tiles = g.Cout > 32 ? ceil_div((uint64_t)g.Cout, 64) * ceil_div(Kc, 64) : ceil_div((uint64_t)g.Cout, 32) * ceil_div(Kc, 32);
+	const uint64_t want = std::max<uint64_t>(1, 1024 / tiles);
+	slice_len = (int64_t)(ceil_div(ceil_div(R, want), 64) * 64);
 	if (slice_len < 256) slice_len = 256;
-	slices = (int)ceil_div((uint64_t)HW, (uint64_t)slice_len);
+	slices = (int)ceil_div(R, (uint64_t)slice_len);
 }
 
 // Picks the forward kernel for a geometry (x, w, y non-null, non-empty problem).
@@ -195,13 +215,14 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	// output channels to offer its 32 x 128 tile.
 	const bool narrow = variant == 0 && g.Wo < 32 && g.Cout > 32;
 	if (!narrow && variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
+	LTEN_HIP_REQUIRE(N * HW < (1ull << 31), "conv2d_forward: the batch's output pixels must number less than 2^31 on this route");
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(HW, 64)), 1, (unsigned)N);
+		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(N * HW, 64)));
 		conv2d_forward_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	} else {
 		set_kernel_name("conv2d_forward_32x128x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(HW, 128)), 1, (unsigned)N);
+		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(N * HW, 128)));
 		conv2d_forward_kernel<32, 128, 32, 1, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
@@ -411,10 +432,11 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
 {
 	ConvGeo g;
 	if (make_geo(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw, 1, 1)) return 0;
-	int slices, slice_len;
+	int slices;
+	int64_t slice_len;
 	wgrad_split(g, slices, slice_len);
 	// enough for whichever kernel the call picks
-	uint64_t parts = (uint64_t)N * slices;
+	uint64_t parts = (uint64_t)slices;
 	if (conv_smallk_takes(g)) parts = std::max<uint64_t>(parts, conv_smallk_wgrad_parts(g));
 	if (conv_patch_wgrad_takes(g)) parts = std::max<uint64_t>(parts, conv_patch_wgrad_parts(g, true));
 	return parts * Cout * Cin * kh * kw * sizeof(float);
@@ -442,19 +464,19 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
 		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
 	}
-	int slices, slice_len;
-	wgrad_split(g, slices, slice_len);
-	const int parts = (int)N * slices;
-	LTEN_HIP_REQUIRE(parts < 65536, "conv2d_wgrad: too many partial sums");
+	int parts;
+	int64_t slice_len;
+	wgrad_split(g, parts, slice_len);
+	LTEN_HIP_REQUIRE(parts < 65536 && (uint64_t)N * g.Ho * g.Wo < (1ull << 31), "conv2d_wgrad: the batch's output pixels must number less than 2^31 on this route");
 	float* partial = static_cast<float*>(workspace);
 	if (Cout > 32) {
 		set_kernel_name("conv2d_wgrad_64x64x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(Kc, 64)), 1, (unsigned)parts);
-		conv2d_wgrad_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, slices, slice_len);
+		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(Kc, 64)), (unsigned)parts);
+		conv2d_wgrad_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, dy, partial, slice_len);
 	} else {
 		set_kernel_name("conv2d_wgrad_32x32x32");
-		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(Kc, 32)), 1, (unsigned)parts);
-		conv2d_wgrad_kernel<32, 32, 32, 1, 1><<<grid, dim3(64), 0, stream()>>>(g, x, dy, partial, slices, slice_len);
+		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(Kc, 32)), (unsigned)parts);
+		conv2d_wgrad_kernel<32, 32, 32, 1, 1><<<grid, dim3(64), 0, stream()>>>(g, x, dy, partial, slice_len);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return conv_reduce_partials(partial, parts, count, dw);

@@ -28,15 +28,15 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
 	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
 	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
 
-	auto fetch_a = [&](int row, int k) -> float {
-		const int m = m0 + row;
-		if (m >= p.M || k >= p.K) return 0.0f;
-		return TA ? A[(int64_t)k * p.lda + m] : A[(int64_t)m * p.lda + k];
+	auto fetch_a = [&](int row, int k, bool& inside) -> float {
+		inside = m0 + row < p.M && k < p.K;
+		const int m = min(m0 + row, p.M - 1), kc = min(k, p.K - 1);
+		return TA ? A[(int64_t)kc * p.lda + m] : A[(int64_t)m * p.lda + kc];
 	};
-	auto fetch_b = [&](int row, int k) -> float {
-		const int n = n0 + row;
-		if (n >= p.N || k >= p.K) return 0.0f;
-		return TB ? B[(int64_t)n * p.ldb + k] : B[(int64_t)k * p.ldb + n];
+	auto fetch_b = [&](int row, int k, bool& inside) -> float {
+		inside = n0 + row < p.N && k < p.K;
+		const int n = min(n0 + row, p.N - 1), kc = min(k, p.K - 1);
+		return TB ? B[(int64_t)n * p.ldb + kc] : B[(int64_t)kc * p.ldb + n];
 	};
 
 	v16f acc[Core::FM][Core::FN];
