@@ -70,13 +70,13 @@ __device__ __forceinline__ KTap make_tap(const ConvGeo& g, int k)
 // whole batch (n, hw) in one run, so that small images fill the column tiles together.  A thread stages the same
 // column in every k-step (the tile's columns divide the workgroup's threads), so its pixel is decomposed once; every
 // load is issued whatever the position, from an address that lies inside the operand (see GemmCore::run).
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, bool TAB>
 __global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, const float* x, const float* w, const float* bias, float* y)
 {
 	typedef GemmCore<BM, BN, BK, WM, WN, false, true> Core;
 	static_assert(Core::T % BN == 0 && (BM * BK) % Core::T == 0 && (BN * BK) % Core::T == 0, "a thread's column is the same in every fetch");
 	__shared__ float lds[Core::LDS_FLOATS];
-	__shared__ KTap ktab[MAX_KTAB];
+	__shared__ KTap ktab[TAB ? MAX_KTAB : 1];  // TAB: Cin*kh*kw <= MAX_KTAB (the host picks the instantiation)
 	__shared__ int col_img[BN], col_hw[BN];  // for the stores: image and pixel of every column of the tile (-1: none)
 
 	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
@@ -84,8 +84,7 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, 
 	const int tiles_n = (int)(((int64_t)cols + BN - 1) / BN);
 	const int m0 = (blockIdx.x / tiles_n) * BM;
 	const int n0 = (blockIdx.x % tiles_n) * BN;
-	const bool use_tab = Kc <= MAX_KTAB;
-	if (use_tab) {
+	if (TAB) {
 		for (int k = threadIdx.x; k < Kc; k += Core::T) ktab[k] = make_tap(g, k);
 	}
 	// this thread's column
@@ -102,15 +101,16 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_forward_kernel(ConvGeo g, 
 	}
 	__syncthreads();
 
+	// (conditions joined with & rather than &&: no branches between the loads)
 	auto fetch_a = [&](int row, int k, bool& inside) -> float {
-		inside = m0 + row < g.Cout && k < Kc;
+		inside = (m0 + row < g.Cout) & (k < Kc);
 		return w[(int64_t)min(m0 + row, g.Cout - 1) * Kc + min(k, Kc - 1)];
 	};
 	auto fetch_b = [&](int, int k, bool& inside) -> float {
-		const KTap t = use_tab ? ktab[min(k, Kc - 1)] : make_tap(g, min(k, Kc - 1));
+		const KTap t = TAB ? ktab[min(k, Kc - 1)] : make_tap(g, min(k, Kc - 1));
 		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
-		inside = col_ok && k < Kc && (unsigned)ty < (unsigned)g.H && (unsigned)tx < (unsigned)g.W;
-		return xi[inside ? pix + t.off : 0];
+		inside = col_ok & (k < Kc) & ((unsigned)ty < (unsigned)g.H) & ((unsigned)tx < (unsigned)g.W);
+		return xi[(pix + t.off) & -(int)inside];  // offset 0 for what lies outside; a mask, not a choice: a choice becomes a branch around the table read
 	};
 
 	v16f acc[Core::FM][Core::FN];
@@ -147,7 +147,7 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, co
 	auto fetch_a = [&](int row, int rr, bool& inside) -> float {
 		const int r = min(rr, r1 - 1);
 		const int img = r / HW, hw = r - img * HW;
-		inside = m0 + row < g.Cout && rr < r1;
+		inside = (m0 + row < g.Cout) & (rr < r1);
 		return dy[((int64_t)img * g.Cout + min(m0 + row, g.Cout - 1)) * HW + hw];
 	};
 	auto fetch_b = [&](int row, int rr, bool& inside) -> float {
@@ -157,8 +157,8 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, co
 		const KTap t = ktab[row];
 		const int yy = ho * g.sh - g.ph, xx = wo * g.sw - g.pw;
 		const int ty = yy + (t.ij & 0xFFFF), tx = xx + (t.ij >> 16);
-		inside = n0 + row < Kc && rr < r1 && (unsigned)ty < (unsigned)g.H && (unsigned)tx < (unsigned)g.W;
-		return x[img * in_image + (inside ? yy * g.W + xx + t.off : 0)];
+		inside = (n0 + row < Kc) & (rr < r1) & ((unsigned)ty < (unsigned)g.H) & ((unsigned)tx < (unsigned)g.W);
+		return x[img * in_image + ((yy * g.W + xx + t.off) & -(int)inside)];
 	};
 
 	v16f acc[Core::FM][Core::FN];
@@ -219,11 +219,13 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	if (Cout > 32) {
 		set_kernel_name("conv2d_forward_64x64x32");
 		const dim3 grid((unsigned)(ceil_div(Cout, 64) * ceil_div(N * HW, 64)));
-		conv2d_forward_kernel<64, 64, 32, 2, 2><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		if (g.Cin * g.kh * g.kw <= MAX_KTAB) conv2d_forward_kernel<64, 64, 32, 2, 2, true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		else conv2d_forward_kernel<64, 64, 32, 2, 2, false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	} else {
 		set_kernel_name("conv2d_forward_32x128x32");
 		const dim3 grid((unsigned)(ceil_div(Cout, 32) * ceil_div(N * HW, 128)));
-		conv2d_forward_kernel<32, 128, 32, 1, 4><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		if (g.Cin * g.kh * g.kw <= MAX_KTAB) conv2d_forward_kernel<32, 128, 32, 1, 4, true><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
+		else conv2d_forward_kernel<32, 128, 32, 1, 4, false><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, y);
 	}
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;

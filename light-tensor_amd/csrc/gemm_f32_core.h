@@ -69,14 +69,14 @@ struct GemmCore {
 				const int e = min(tid + i * T, BM * BK - 1);
 				bool inside;
 				ra[i] = fetch_a(LA::row_of(e), k0 + LA::k_of(e), inside);
-				keep_a |= (unsigned)(inside && tid + i * T < BM * BK) << i;
+				keep_a |= (unsigned)(inside & (tid + i * T < BM * BK)) << i;
 			}
 #pragma unroll
 			for (int i = 0; i < B_PER_T; i++) {
 				const int e = min(tid + i * T, BN * BK - 1);
 				bool inside;
 				rb[i] = fetch_b(LB::row_of(e), k0 + LB::k_of(e), inside);
-				keep_b |= (unsigned)(inside && tid + i * T < BN * BK) << i;
+				keep_b |= (unsigned)(inside & (tid + i * T < BN * BK)) << i;
 			}
 		};
 		auto store_lds = [&](int buf) {

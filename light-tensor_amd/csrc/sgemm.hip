@@ -29,12 +29,12 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_kernel(SProblem p)
 	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
 
 	auto fetch_a = [&](int row, int k, bool& inside) -> float {
-		inside = m0 + row < p.M && k < p.K;
+		inside = (m0 + row < p.M) & (k < p.K);
 		const int m = min(m0 + row, p.M - 1), kc = min(k, p.K - 1);
 		return TA ? A[(int64_t)kc * p.lda + m] : A[(int64_t)m * p.lda + kc];
 	};
 	auto fetch_b = [&](int row, int k, bool& inside) -> float {
-		inside = n0 + row < p.N && k < p.K;
+		inside = (n0 + row < p.N) & (k < p.K);
 		const int n = min(n0 + row, p.N - 1), kc = min(k, p.K - 1);
 		return TB ? B[(int64_t)n * p.ldb + kc] : B[(int64_t)kc * p.ldb + n];
 	};
