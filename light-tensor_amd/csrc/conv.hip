@@ -210,10 +210,11 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	// one with its four-row tile also where the two-row tile would be picked
 	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
 	// The register-staged patch kernel's tiles are 128 columns wide (the direct-to-LDS one above has 16 x 32 tiles for
-	// narrow images): on images narrower than 32 columns three quarters of a tile are padding and the implicit GEMM over
-	// the flattened pixels is ahead (8 x 256 x 14 x 14 -> 512 channels: 158 against 325 us), unless it has at most 32
-	// output channels to offer its 32 x 128 tile.
-	const bool narrow = variant == 0 && g.Wo < 32 && g.Cout > 32;
+	// narrow images): on images of at most 56 columns more than half of a tile is padding, and with fewer than 256 tiles
+	// CUs stay idle; the implicit GEMM over the batch's flattened pixels is ahead there (32 x 48 x 50 x 50 -> 96
+	// channels: 154 against 178 us, 4 x 64 x 126 x 126 -> 64: 82 against 90 us, 64 x 16 x 30 x 30 -> 32: 18 against 27 us).
+	const uint64_t patch_tiles = ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 4) * ceil_div(Cout, 64) * N;
+	const bool narrow = variant == 0 && (g.Wo <= 56 || patch_tiles < 256);
 	if (!narrow && variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
 	LTEN_HIP_REQUIRE(N * HW < (1ull << 31), "conv2d_forward: the batch's output pixels must number less than 2^31 on this route");
 	if (Cout > 32) {
@@ -459,8 +460,10 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		if (int rc = conv_smallk_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
 		return conv_reduce_partials(static_cast<const float*>(workspace), parts, count, dw);
 	}
-	// images of at most 16 columns: an eighth of the patch kernel's 128-column tile (8 x 256 x 14 x 14 -> 512: 129 against 199 us)
-	const bool narrow = get_option(OPT_CONV_VARIANT) == 0 && g.Wo <= 16;
+	// images of at most 16 columns: an eighth of the patch kernel's 128-column tile (8 x 256 x 14 x 14 -> 512: 129 against 199 us);
+	// rows that do not allow 16-byte loads, of at most 56 columns (the kernel's chunks are 64 pixels of one row):
+	// 32 x 32 x 30 x 30 -> 64: 33 against 47 us, 32 x 48 x 50 x 50 -> 96: 151 against 177 us
+	const bool narrow = get_option(OPT_CONV_VARIANT) == 0 && (g.Wo <= 16 || ((g.W % 4 != 0 || g.Wo % 4 != 0) && g.Wo <= 56));
 	if (!narrow && get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
 		const int parts = conv_patch_wgrad_parts(g);
 		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;
