@@ -1004,7 +1004,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// NT products whose 128 x 128 tiles would not give every CU a workgroup while 64 x 64 tiles do (a FullyConnected forward
 	// at a batch of 256 to 768 against a 4096-wide layer: 512 x 4096 x 4096 in 132 us instead of 240, the time of batch 1024)
 	const bool nt64 = !tA && tB && tiles128 < 256 && tiles64 >= 256;
-	if (choice == 0 && (tiles128 >= 128 || nt64) && K >= 256) {
+	// (a K that is no multiple of 32 costs a second launch over all of C: only worth it from K = 512 on)
+	if (choice == 0 && (tiles128 >= 128 || nt64) && K >= 256 && (K % 32 == 0 || K >= 512)) {
 		// large problems: 256 x 256 tiles when they fill the chip, else 128 x 128 (or 64 x 64, above).  The tiles walk K in
 		// steps of 32: what is left over is added by a second, general launch (beta = 1, no bias).
 		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192;
@@ -1020,12 +1021,16 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	if (choice == 0) {
 		// Few output tiles and a long K: the LDS-tiled kernels would leave most CUs idle while a handful of
 		// workgroups walk K in sequence; the direct kernel cuts K across the wavefronts of a workgroup instead.
-		// With 16-byte loads the 32x32 kernels stay ahead of the LDS-tiled ones at every size measured (1280^3: 58 vs
-		// 40 TFLOP/s, 4000^3 with K a multiple of 4: 74 vs 63, 3000 x 3000 x 300: 65 vs 44); without them only while
-		// the tiles are few (4095^3: 25 vs 66).
+		// With 16-byte loads the 32x32 kernels stay ahead of the LDS-tiled ones at every size measured (1280^3: 74 vs
+		// 80 us, 200 x 5000 x 700: 45 vs 44 us); without them while the tiles are few, except for NT products,
+		// whose 4-byte loads along K they handle badly (1001 x 1003 x 1005: NN 55 vs 51 us, TN 40 vs 51, NT 83 vs 48).
+		// Of the LDS-tiled kernels the 64 x 64 tile is ahead until the problem is large (2047 x 2049 x 513: 79 vs 103 us,
+		// 6000 x 500 x 999: 89 vs 128 us; 4095^3: 1677 vs 1424 us).
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32) * batch;
-		if (tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20))) choice = 4;
-		else choice = tiles128 >= 128 ? 1 : 2;
+		const int lds_tiled = tiles128 >= 512 ? 1 : 2;
+		if (operands_vec(p) && tiles32 < (1u << 20)) choice = 4;
+		else if (!tA && tB) choice = tiles64 >= 64 ? lds_tiled : 4;
+		else choice = tiles32 <= 1024 ? 4 : lds_tiled;
 	}
 	if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
 	switch (choice) {
