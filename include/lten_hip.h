@@ -223,7 +223,9 @@ uint64_t lten_hip_conv2d_dgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
  * byte 0, as in l-ten's column buffer.  bias, when not null, holds Ho*Wo ints and is added per output position:
  * that is what l-ten's call computes (quantized_matmul indexes the bias by GEMM column, l-ten/math_fns.cpp:1470-1473,
  * and the columns of this product are output positions).  workspace: lten_hip_conv2dq_workspace_bytes device
- * bytes, 16-byte aligned (column buffer and zero-point terms of the fallback for windows above 64 taps). */
+ * bytes, 16-byte aligned.  Windows above 64 taps use it: the patches of all output positions of the batch as rows
+ * of a matrix, the padded weights, the int32 sums of one int8 GEMM over the whole batch and its zero-point terms;
+ * where that would exceed 2 GiB, the column buffer of one image (l-ten's decomposition, image by image). */
 uint64_t lten_hip_conv2dq_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                                           int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w);
 int lten_hip_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kernel_h,

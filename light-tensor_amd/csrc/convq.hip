@@ -9,8 +9,13 @@
 // launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
-// Longer windows follow l-ten's own decomposition per image: im2col_u8 into the caller's workspace, then the
-// int8 GEMM of qgemm.hip.
+// Longer windows run as three launches for the whole batch: the patches of all output positions as rows of a
+// [N * Ho * Wo][K] matrix (K padded to a multiple of 16 with the input zero point, the weights padded alike with
+// theirs, so the padding multiplies to nothing), one int8 GEMM of qgemm.hip with the positions as rows (NT: both
+// operands contiguous in K, the shape its MFMA tiles are built for) into int32 sums, and a pass that adds l-ten's
+// per-position bias, requantizes and stores in NCHW order.  When the workspace that needs would exceed 2 GiB the
+// call follows l-ten's own decomposition image by image: im2col_u8, then the GEMM with the weights on the left.
+#include <algorithm>
 #include "conv_common.h"
 #include "qgemm_common.h"
 
@@ -115,6 +120,76 @@ static void launch_conv2dq_direct(const dim3& grid, int K, const ConvGeo& g, con
 	else conv2dq_direct_kernel<OUT, 16><<<grid, dim3(256), 0, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
 }
 
+// Row r = n * Ho * Wo + p of the patch matrix: the window of output position p of image n in l-ten's column order
+// (ci, i, j).  Bytes outside the image are 0, as in l-ten's im2col (not the zero point); bytes from K on hold the input
+// zero point.  A thread builds four consecutive bytes of a row; the tap table (offset of the tap inside an image and
+// its (i, j)) is built once per workgroup in LDS.
+__global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint8_t* __restrict__ x, uint8_t* __restrict__ rows, int Kp, int zp_in)
+{
+	extern __shared__ int s_tap[];  // [Kp] offsets, then [Kp] i | j << 16
+	const int K = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	for (int k = threadIdx.x; k < Kp; k += 256) {
+		const int kc = min(k, K - 1);
+		const int j = kc % g.kw, i = (kc / g.kw) % g.kh, ci = kc / (g.kw * g.kh);
+		s_tap[k] = (ci * g.H + i) * g.W + j;
+		s_tap[Kp + k] = i | (j << 16);
+	}
+	__syncthreads();
+	const uint32_t kq_per_row = (uint32_t)Kp / 4;
+	const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+	const uint32_t r = (uint32_t)(idx / kq_per_row), kq = (uint32_t)(idx - (uint64_t)r * kq_per_row);
+	if (r >= (uint32_t)g.N * (uint32_t)HW) return;
+	const int n = (int)(r / (uint32_t)HW), pos = (int)(r - (uint32_t)n * (uint32_t)HW);
+	const int ho = pos / g.Wo, wo = pos - ho * g.Wo;
+	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
+	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+	uint32_t word = 0;
+#pragma unroll
+	for (int b = 0; b < 4; b++) {
+		const int k = 4 * (int)kq + b;
+		const int ij = s_tap[Kp + k];
+		const int yy = y0 + (ij & 0xFFFF), xx = x0 + (ij >> 16);
+		const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W);
+		const uint32_t byte = xn[(s_tap[k] + y0 * g.W + x0) & -(int)inside];  // offset 0 for taps outside: always a valid address
+		word |= (k < K ? (inside ? byte : 0u) : (uint32_t)zp_in) << (8 * b);
+	}
+	reinterpret_cast<uint32_t*>(rows)[idx] = word;
+}
+
+// wp[co][k] for co < Cp, k < Kp: the weights, with the weight zero point past K and in the rows past Cout.
+__global__ __launch_bounds__(256) void conv2dq_pad_weights_kernel(const uint8_t* __restrict__ w, uint8_t* __restrict__ wp, int Cout, int K, int Cp, int Kp, int zp_w)
+{
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	if (idx >= Cp * Kp) return;
+	const int co = idx / Kp, k = idx - co * Kp;
+	wp[idx] = (co < Cout && k < K) ? w[(int64_t)co * K + k] : (uint8_t)zp_w;
+}
+
+// y[n][co][p] = requantize(acc[n * HW + p][co] + bias[p]) (or the int32 sum itself): a workgroup takes 64 positions x 64
+// channels, reads the sums along the channels and stores along the positions, through LDS.
+template <int OUT>
+__global__ __launch_bounds__(256) void conv2dq_finish_kernel(const int32_t* __restrict__ acc, const int32_t* __restrict__ bias, void* __restrict__ y,
+                                                             int rows, int HW, int Cout, int Cp, float mult, float zp_out)
+{
+	__shared__ int s[64][65];
+	const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+	for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+		const int rr = e >> 6, cc = e & 63;
+		s[rr][cc] = acc[(int64_t)min(r0 + rr, rows - 1) * Cp + min(c0 + cc, Cp - 1)];
+	}
+	__syncthreads();
+	for (int e = threadIdx.x; e < 64 * 64; e += 256) {
+		const int cc = e >> 6, rr = e & 63;
+		const int r = r0 + rr, co = c0 + cc;
+		if (r >= rows || co >= Cout) continue;
+		const int n = r / HW, pos = r - n * HW;
+		const int v = s[rr][cc] + (bias ? bias[pos] : 0);
+		const int64_t o = ((int64_t)n * Cout + co) * HW + pos;
+		if (OUT == Q_OUT_ACC) static_cast<int*>(y)[o] = v;
+		else static_cast<uint8_t*>(y)[o] = (uint8_t)requant<OUT>(v, mult, zp_out);
+	}
+}
+
 static int make_geo_q(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh, int sw)
 {
 	LTEN_HIP_REQUIRE(kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0, "conv2dq: bad kernel geometry");
@@ -131,6 +206,28 @@ static int make_geo_q(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t
 }
 
 static uint64_t align16(uint64_t v) { return (v + 15) & ~15ull; }
+static uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
+
+// Workspace of the whole-batch route: patch rows, padded weights, int32 sums, the GEMM's zero-point terms.
+struct BatchedPlan {
+	bool ok;
+	uint64_t rows, Kp, Cp, off_wp, off_acc, off_terms, bytes;
+};
+
+static BatchedPlan batched_plan(const ConvGeo& g)
+{
+	BatchedPlan b;
+	const uint64_t K = (uint64_t)g.Cin * g.kh * g.kw;
+	b.rows = (uint64_t)g.N * g.Ho * g.Wo;
+	b.Kp = (K + 15) & ~15ull;
+	b.Cp = ((uint64_t)g.Cout + 3) & ~3ull;
+	b.off_wp = align256(b.rows * b.Kp);
+	b.off_acc = b.off_wp + align256(b.Cp * b.Kp);
+	b.off_terms = b.off_acc + align256(b.rows * b.Cp * 4);
+	b.bytes = b.off_terms + 4 * (b.rows + b.Cp) + 16;
+	b.ok = b.bytes <= (2ull << 30) && b.rows < (1ull << 31) && b.rows * b.Kp < (1ull << 32) && b.Kp * 8 <= 48 * 1024 && b.Cp * b.Kp < (1ull << 31);
+	return b;
+}
 
 static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh, int sw,
                        const uint8_t* x, const uint8_t* w, const int32_t* bias, const lten_hip_qparams* qp, void* y, bool out_acc,
@@ -158,8 +255,30 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		return 0;
 	}
 
-	// l-ten's own decomposition, image by image: column buffer, then C[Cout x HW] = W[Cout x K] * col[K x HW]
 	LTEN_HIP_REQUIRE(workspace != nullptr, "conv2dq: workspace is null");
+	const BatchedPlan bp = batched_plan(g);
+	if (bp.ok && get_option(OPT_CONV_VARIANT) != 1) {
+		uint8_t* base = static_cast<uint8_t*>(workspace);
+		uint8_t* rows = base;
+		uint8_t* wp = base + bp.off_wp;
+		int32_t* sums = reinterpret_cast<int32_t*>(base + bp.off_acc);
+		int32_t* terms = reinterpret_cast<int32_t*>(base + bp.off_terms);
+		conv2dq_rows_kernel<<<dim3((unsigned)ceil_div(bp.rows * (bp.Kp / 4), 256)), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in);
+		LTEN_HIP_LAUNCH_CHECK();
+		conv2dq_pad_weights_kernel<<<dim3((unsigned)ceil_div(bp.Cp * bp.Kp, 256)), dim3(256), 0, stream()>>>(w, wp, (int)Cout, (int)K, (int)bp.Cp, (int)bp.Kp, zp_w);
+		LTEN_HIP_LAUNCH_CHECK();
+		if (int rc = lten_hip_quantized_matmul_acc(0, 1, bp.rows, bp.Cp, bp.Kp, rows, wp, sums, qp, nullptr, terms)) return rc;
+		const dim3 grid((unsigned)ceil_div(bp.rows, 64), (unsigned)ceil_div(Cout, 64));
+		set_kernel_name("conv2dq_rows_gemm_finish");
+		if (out_acc) conv2dq_finish_kernel<Q_OUT_ACC><<<grid, dim3(256), 0, stream()>>>(sums, bias, y, (int)bp.rows, (int)HW, (int)Cout, (int)bp.Cp, mult, zp_out);
+		else if (mult == mult && (mult < 0 ? -mult : mult) <= 0.99f)
+			conv2dq_finish_kernel<Q_OUT_U8_FAST><<<grid, dim3(256), 0, stream()>>>(sums, bias, y, (int)bp.rows, (int)HW, (int)Cout, (int)bp.Cp, mult, zp_out);
+		else conv2dq_finish_kernel<Q_OUT_U8_EXACT><<<grid, dim3(256), 0, stream()>>>(sums, bias, y, (int)bp.rows, (int)HW, (int)Cout, (int)bp.Cp, mult, zp_out);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
+
+	// l-ten's own decomposition, image by image: column buffer, then C[Cout x HW] = W[Cout x K] * col[K x HW]
 	uint8_t* col = static_cast<uint8_t*>(workspace);
 	int32_t* terms = reinterpret_cast<int32_t*>(col + align16((uint64_t)K * HW));
 	const lten_hip_qparams q3[3] = { qp[1], qp[0], qp[2] };
@@ -185,7 +304,9 @@ uint64_t lten_hip_conv2dq_workspace_bytes(uint64_t N, uint64_t Cin, uint64_t H, 
 	ConvGeo g;
 	if (make_geo_q(g, N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)) return 0;
 	const uint64_t HW = (uint64_t)g.Ho * g.Wo, K = Cin * kh * kw;
-	return align16(K * HW) + 4 * (Cout + HW) + 16;
+	const uint64_t per_image = align16(K * HW) + 4 * (Cout + HW) + 16;
+	const BatchedPlan bp = batched_plan(g);
+	return bp.ok ? std::max(per_image, bp.bytes) : per_image;
 }
 
 int lten_hip_conv2dq_forward(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph, int pw, int sh,

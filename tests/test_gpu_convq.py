@@ -27,7 +27,13 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
 
 @pytest.mark.parametrize("geo", [(64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1),      # l-ten's quantized MNIST conv1 at batch 64
                                  (3, 7, 13, 17, 70, 3, 3, 1, 1, 1, 1),       # 63 taps, two channel blocks
-                                 (2, 16, 20, 22, 24, 3, 3, 1, 1, 2, 1),      # 144 taps: column buffer + GEMM
+                                 (2, 16, 20, 22, 24, 3, 3, 1, 1, 2, 1),      # 144 taps: patch rows + GEMM + finish
+                                 (5, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1),      # l-ten's quantized MNIST conv2: 250 taps (padded to 256)
+                                 (3, 8, 9, 7, 10, 3, 3, 1, 1, 1, 1),         # 72 taps, 10 channels (padded to 12), 63 positions an image
+                                 (2, 64, 6, 10, 70, 3, 3, 1, 1, 1, 1),       # 576 taps, two channel blocks of the finish pass
+                                 (4, 128, 5, 5, 33, 1, 1, 0, 0, 1, 1),       # 1x1 with 128 channels
+                                 (2, 6, 14, 14, 16, 5, 5, 2, 2, 1, 1),       # 150 taps, padding 2
+                                 (1, 20, 17, 9, 6, 3, 5, 0, 2, 2, 2),        # 300 taps, strides, oblong window
                                  (1, 3, 33, 300, 5, 7, 3, 3, 0, 2, 3),       # 63 taps, strides, ragged
                                  (2, 32, 9, 9, 40, 1, 1, 0, 0, 1, 1),        # 1x1
                                  (2, 5, 11, 13, 9, 3, 3, 1, 0, 1, 2),        # 45 taps: twelve packed dwords
@@ -47,6 +53,14 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         want_y, want_acc = ob.conv2dq_forward(geo, x, w, sc, zp, bias=bias)
         y, acc = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
         kern = gpu.last_kernel()
-        assert (kern == "conv2dq_direct") == (K <= 64), kern
+        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
         assert np.array_equal(y, want_y), kern
+    if K > 64:   # l-ten's decomposition image by image (what a workspace beyond 2 GiB falls back to) gives the same bytes
+        gpu.set_option("conv_variant", 1)
+        try:
+            y1, acc1 = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
+            assert gpu.last_kernel() != "conv2dq_rows_gemm_finish"
+        finally:
+            gpu.set_option("conv_variant", 0)
+        assert np.array_equal(acc1, want_acc) and np.array_equal(y1, want_y)
