@@ -169,6 +169,78 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, co
 	});
 }
 
+// Data gradient for any stride: dx[n][ci][y][x] = sum over (co, i, j) of dy[n][co][oy][ox] * w[co][ci][i][j] with
+// oy = (y + ph - i) / sh, ox = (x + pw - j) / sw where those divide and lie inside dy.  GEMM rows = ci, columns = the
+// input pixels of the whole batch, reduction over (co, i, j).  Which output row a tap row i reaches from input row y
+// (or none) is tabulated per column of the tile in LDS, likewise for the columns, so a gather costs three table reads
+// and no division.  With a stride above 1 most taps of a pixel reach nothing (three in four at stride 2): the MFMAs
+// run over those zeros, which still beats l-ten's decomposition (a GEMM and a col2im launch per image) many times over.
+constexpr int DG_MAXW = 16;  // window rows and columns the per-column tables hold
+template <int BM, int BN, int BK, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void conv2d_dgrad_kernel(ConvGeo g, const float* w, const float* dy, float* dx)
+{
+	typedef GemmCore<BM, BN, BK, WM, WN, false, true> Core;
+	static_assert(Core::T % BN == 0 && (BM * BK) % Core::T == 0 && (BN * BK) % Core::T == 0, "a thread's column is the same in every fetch");
+	__shared__ float lds[Core::LDS_FLOATS];
+	__shared__ KTap ktab[MAX_KTAB];            // per k = (co, i, j): co * Ho * Wo, and i | j << 16
+	__shared__ int col_img[BN], col_hw[BN];    // for the stores: image and pixel of every column of the tile (-1: none)
+	__shared__ int row_of[BN][DG_MAXW], column_of[BN][DG_MAXW];  // output row reached through tap row i (-1: none), likewise columns
+
+	const int taps = g.kh * g.kw, Kd = g.Cout * taps, HWi = g.H * g.W, HWo = g.Ho * g.Wo;
+	const int cols = g.N * HWi;  // below 2^31 (checked by the host)
+	const int tiles_n = (int)(((int64_t)cols + BN - 1) / BN);
+	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+	for (int k = threadIdx.x; k < Kd; k += Core::T) {
+		const int co = k / taps, t = k - co * taps, i = t / g.kw;
+		ktab[k].off = co * HWo;
+		ktab[k].ij = i | ((t - i * g.kw) << 16);
+	}
+	const unsigned col = (unsigned)n0 + threadIdx.x % BN;
+	const bool col_ok = col < (unsigned)cols;
+	const int img = (int)(min(col, (unsigned)cols - 1) / (unsigned)HWi), hw = (int)(min(col, (unsigned)cols - 1) - (unsigned)img * HWi);
+	const int yy = hw / g.W, xx = hw - yy * g.W;
+	const int c = threadIdx.x % BN;
+	if (threadIdx.x < BN) {
+		col_img[c] = col_ok ? img : -1;
+		col_hw[c] = hw;
+		for (int i = 0; i < g.kh; i++) {
+			const int num = yy + g.ph - i, q = num / g.sh;
+			row_of[c][i] = (num >= 0 && q * g.sh == num && q < g.Ho) ? q : -1;
+		}
+		for (int j = 0; j < g.kw; j++) {
+			const int num = xx + g.pw - j, q = num / g.sw;
+			column_of[c][j] = (num >= 0 && q * g.sw == num && q < g.Wo) ? q : -1;
+		}
+	}
+	__syncthreads();
+	const float* dyi = dy + (int64_t)img * g.Cout * HWo;
+
+	auto fetch_a = [&](int row, int k, bool& inside) -> float {
+		inside = (m0 + row < g.Cin) & (k < Kd);
+		const int kc = min(k, Kd - 1), co = kc / taps, t = kc - co * taps;
+		return w[((int64_t)co * g.Cin + min(m0 + row, g.Cin - 1)) * taps + t];
+	};
+	auto fetch_b = [&](int, int k, bool& inside) -> float {
+		const KTap t = ktab[min(k, Kd - 1)];
+		const int oy = row_of[c][t.ij & 0xFFFF], ox = column_of[c][t.ij >> 16];
+		inside = col_ok & (k < Kd) & ((oy | ox) >= 0);
+		return dyi[(t.off + oy * g.Wo + ox) & -(int)inside];
+	};
+
+	v16f acc[Core::FM][Core::FN];
+	Core::run(lds, 0, Kd, fetch_a, fetch_b, acc);
+	Core::for_each(acc, [&](int row, int cc, float v) {
+		const int ci = m0 + row, im = col_img[cc];
+		if (ci < g.Cin && im >= 0) dx[((int64_t)im * g.Cin + ci) * HWi + col_hw[cc]] = v;
+	});
+}
+
+static bool dgrad_gemm_takes(const ConvGeo& g)
+{
+	return g.dh == 1 && g.dw == 1 && g.kh <= DG_MAXW && g.kw <= DG_MAXW && (uint64_t)g.Cout * g.kh * g.kw <= MAX_KTAB &&
+	       (uint64_t)g.N * g.H * g.W < (1ull << 31) && (uint64_t)g.Cout * g.Ho * g.Wo < (1ull << 31);
+}
+
 static int make_geo(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
                     int pw, int sh, int sw, int dh, int dw)
 {
@@ -422,6 +494,13 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		if (int rc = make_geo(g2, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
 		LTEN_HIP_REQUIRE(g2.Ho == (int)H && g2.Wo == (int)W, "conv2d_dgrad: internal geometry mismatch");
 		return conv_forward_dispatch(g2, dy, work, nullptr, dx);
+	}
+	// any stride: one implicit-GEMM launch for the batch (64 x 64 x 28 x 28 <- 128 channels at stride 2: 722 us image by image)
+	if (get_option(OPT_CONV_VARIANT) == 0 && (!few_narrow || !dgrad_as_forward(g)) && dgrad_gemm_takes(g)) {
+		set_kernel_name("conv2d_dgrad_64x64x32");
+		conv2d_dgrad_kernel<64, 64, 32, 2, 2><<<dim3((unsigned)(ceil_div(Cin, 64) * ceil_div(N * H * W, 64))), dim3(256), 0, stream()>>>(g, w, dy, dx);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
 	}
 	// l-ten/backprop.cpp:2022-2028 per image: col = W^T dy_n (TN GEMM), then col2im
 	for (uint64_t n = 0; n < N; n++) {

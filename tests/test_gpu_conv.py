@@ -231,6 +231,29 @@ def test_conv_data_gradient_of_first_layers(gpu, ob, geo):
     assert rel_err(dx, want_dx) < TOL
 
 
+@pytest.mark.parametrize("geo", [
+    (2, 5, 9, 11, 7, 3, 3, 1, 1, 2, 2),       # stride 2, odd sizes
+    (3, 16, 12, 10, 40, 5, 3, 2, 1, 2, 3),    # strides 2 x 3, oblong window
+    (1, 70, 8, 8, 3, 1, 1, 0, 0, 2, 2),       # 1 x 1 at stride 2: three pixels in four get no gradient
+    (2, 8, 15, 15, 8, 4, 4, 1, 1, 3, 3),      # stride 3, even window
+    (5, 33, 7, 6, 65, 3, 3, 1, 1, 2, 1),      # two row tiles, columns that cross images
+])
+def test_conv_data_gradient_with_strides(gpu, ob, geo):
+    """Data gradient at strides above 1: one implicit-GEMM launch for the batch (rows = input channels, columns = input
+    pixels, per-column tables of the output rows and columns each tap reaches), against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_dgrad_64x64x32", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+
+
 def _conv_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
