@@ -6,7 +6,7 @@ zero-point correction and the requantize fused in) over one synthetic batch whos
 are already resident in HBM; the layer's weights were converted to int8 once, when the layer
 was set up, as the host-side FullyConnected_q does in to(GPU).  The same step on l-ten's raw
 uint8 weight bytes (lten_hip_quantized_matmul) is timed beside it.  Prints ONE JSON line.  The headline fields describe config 3;
-"configs" adds one record per other benchmark configuration (1, 2, 4, 5) and one for the Conv2d_q
+"configs" adds one record per other benchmark configuration (1, 2, 4, 5) and two for the Conv2d_q
 forward, each with its own roofline figure and the CPU path timed beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra] [--no-vendor] [--copy-calibration MiB]
@@ -405,6 +405,23 @@ def extra_configs(lt, wl, with_cpu):
         t = best_of(f, 3)
         rec.update(cpu_ms=round(t * 1e3, 3), cpu_cores=1, cpu_kind="reference" if ob.ref() is not None else "port",
                    speedup=round(t * 1e3 / ms, 1))
+    out.append(rec)
+
+    # ---- the second conv of that network, 10 -> 20 channels 5x5 on the pooled 12x12 maps: 250 taps, the whole-batch
+    # route (patch rows, one int8 GEMM, bias + requantize + NCHW store)
+    geo2 = (64, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1)
+    xq2 = rng.integers(0, 256, (64, 10, 12, 12), dtype=np.uint8)
+    wq2 = rng.integers(0, 256, (20, 10, 5, 5), dtype=np.uint8)
+    dxq2, dwq2, dyq2 = D.from_numpy(xq2), D.from_numpy(wq2), D(64 * 20 * 8 * 8)
+    wsq2 = D(max(int(l.lten_hip_conv2dq_workspace_bytes(*geo2)), 16))
+    ms2 = timed(lt, lambda: lt.check(l.lten_hip_conv2dq_forward(*geo2, dxq2.ptr, dwq2.ptr, None, qpq, dyq2.ptr, wsq2.ptr)), 100)
+    rec = {"config": "Conv2d_q forward 64x10x12x12 -> 20 ch 5x5 (l-ten's quantized MNIST conv2, batch 64)", "gpu_us": round(ms2 * 1e3, 2),
+           "kernel": lt.last_kernel(), "bound": "launch latency (three launches)", "algorithmic_bytes": xq2.nbytes + wq2.nbytes + 64 * 20 * 8 * 8}
+    if with_cpu:
+        f2 = (lambda: ob.ref_conv2dq_forward(geo2, xq2, wq2, sc, zp)) if ob.ref() is not None else (lambda: ob.conv2dq_forward(geo2, xq2, wq2, sc, zp, want_acc=False))
+        t2 = best_of(f2, 3)
+        rec.update(cpu_ms=round(t2 * 1e3, 3), cpu_cores=1, cpu_kind="reference" if ob.ref() is not None else "port",
+                   speedup=round(t2 * 1e3 / ms2, 1))
     out.append(rec)
 
     # ---- beyond the five configs: a large fp32 product in the three layouts l-ten's layers use (FullyConnected forward
