@@ -55,7 +55,7 @@ struct KTap {
 	int off;  // (ci*H + i*dh)*W + j*dw
 	int ij;   // i*dh | (j*dw) << 16
 };
-constexpr int MAX_KTAB = 4096;  // Cin*kh*kw up to 4096 (e.g. 448 channels of 3x3) use the LDS table
+constexpr int MAX_KTAB = 4608;  // Cin*kh*kw up to 4608 (e.g. 512 channels of 3x3) use the LDS table
 
 __device__ __forceinline__ KTap make_tap(const ConvGeo& g, int k)
 {
@@ -468,9 +468,10 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	if (Cout == 0 || HW == 0) return lten_hip_zero(dx, N * Cin * H * W * sizeof(float));
 	LTEN_HIP_REQUIRE(w && dy && workspace, "conv2d_dgrad: null pointer");
 	float* work = static_cast<float*>(workspace);
-	// Few images of at most 16 columns: l-ten's decomposition (GEMM + col2im per image) is ahead of a convolution on
-	// tiles an eighth full (8 x 256 x 14 x 14 <- 512 channels: 167 against 425 us)
-	const bool few_narrow = get_option(OPT_CONV_VARIANT) == 0 && W <= 16 && N <= 16 && Cin > 32;
+	// Few images of at most 16 columns: l-ten's decomposition (GEMM + col2im per image) is ahead of a convolution with so
+	// few columns that its workgroups walk a long reduction one after another (8 x 256 x 14 x 14 <- 512 channels: 166
+	// against 237 us; at 16 images the two launches per image cost more: 16 x 64 x 8 x 8 <- 64: 160 against 41 us)
+	const bool few_narrow = get_option(OPT_CONV_VARIANT) == 0 && W <= 16 && N <= 8 && Cin > 32;
 	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1 && !few_narrow) {
 		ConvGeo gt;  // the transposed problem: dy is the input, dx the output
 		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
