@@ -1001,17 +1001,18 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		if (sgemm_fast_dispatch(p, tA, tB, batch, choice) == 0) return 0;
 		choice = 0;
 	}
-	// NT products whose 128 x 128 tiles would not give every CU a workgroup while 64 x 64 tiles do (a FullyConnected forward
-	// at a batch of 256 to 768 against a 4096-wide layer: 512 x 4096 x 4096 in 132 us instead of 240, the time of batch 1024)
-	const bool nt64 = !tA && tB && tiles128 < 256 && tiles64 >= 256;
-	// (a K that is no multiple of 32 costs a second launch over all of C: only worth it from K = 512 on)
-	if (choice == 0 && (tiles128 >= 128 || nt64) && K >= 256 && (K % 32 == 0 || K >= 512)) {
+	// Products whose 128 x 128 tiles would not give every CU a workgroup while 64 x 64 tiles fill half of them or more (a
+	// FullyConnected layer at a batch of 256 to 768 against a 4096-wide layer: 512 x 4096 x 4096 forward in 132 us
+	// instead of 240, the time of batch 1024; its data and weight gradients 130 instead of 237 us; 1024^3 in any layout
+	// 22 instead of 37 us)
+	const bool t64 = tiles128 < 256 && tiles64 >= 128;
+	if (choice == 0 && (tiles128 >= 128 || t64) && K >= 256 && (K % 32 == 0 || K >= 512)) {
 		// large problems: 256 x 256 tiles when they fill the chip, else 128 x 128 (or 64 x 64, above).  The tiles walk K in
 		// steps of 32: what is left over is added by a second, general launch (beta = 1, no bias).
 		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192;
 		const uint64_t k_main = K & ~31ull;
 		p.K = (int)k_main;
-		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : (nt64 ? 31 : 21)) == 0) {
+		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : (t64 ? 31 : 21)) == 0) {
 			if (k_main == K) return 0;
 			return sgemm_run(tA, tB, M, N, K - k_main, alpha, A + (tA ? k_main * lda : k_main), lda, stride_a,
 			                 B + (tB ? k_main : k_main * ldb), ldb, stride_b, 1.0f, C, ldc, stride_c, batch, nullptr, nullptr, nullptr);

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 	constexpr int RA = A_KC ? FM : 4 * FM, RB = B_KC ? FN : 4 * FN;  // LDS reads per slice
 	constexpr int NR = RA + RB, NM = FM * FN * 4;
 	static_assert(LOADS % W == 0 && LPW % 2 == 0 && (T / 8) % W == 0, "A and B loads split evenly over the wavefronts");
-	static_assert(S >= 2 && S <= 4 && (S - 2) * LPW < 64 && NM >= NR && NM >= LPW, "pipeline shape");
+	static_assert(S >= 2 && S <= 4 && (S - 2) * LPW < 64 && 2 * NM >= NR && NM >= LPW, "pipeline shape");
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[S * STAGE];
 
 	const int tid = threadIdx.x, lane = tid & 63;
@@ -147,7 +147,10 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 		for (int m = 0; m < NM; m++) {
 			const int t = m / (FM * FN), blk = m % (FM * FN), i = blk / FN, j = blk % FN;  // neighbours use different accumulators
 			acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ca[i][t], cb[j][t], acc[i][j], 0, 0, 0);
-			if (read_next && m < NR) read_one(na, nb, sbase, s, m);
+			if (read_next) {  // one operand read behind each MFMA; two where a 32 x 32 wavefront tile has fewer MFMAs per slice than reads
+#pragma unroll
+				for (int e = m; e < NR; e += NM) read_one(na, nb, sbase, s, e);
+			}
 			if (refill) {
 #pragma unroll
 				for (int l = m; l < LPW; l += NM) load_one(l, refill_stage, refill_kt);
@@ -274,15 +277,9 @@ int sgemm_fast_dispatch(const SProblem& p, int tA, int tB, uint64_t batch, int v
 	case 21: return launch_fast<128, 2, 2, 2>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s2");
 	case 22: return launch_fast<128, 2, 2, 3>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s3");
 	case 23: return launch_fast<128, 2, 2, 4>(p, tA, tB, batch, "sgemm_fast_128x128x32_w2x2_s4");
-	case 31: {
-		// 64 x 64 tiles, NT only: with a row-contiguous operand a 32 x 32 wavefront tile has fewer MFMAs per slice than LDS reads
-		if (tA || !tB) return -1;
-		const dim3 grid((unsigned)(ceil_div(p.M, 64) * ceil_div(p.N, 64)), 1, (unsigned)batch), block(256);
-		set_kernel_name("sgemm_fast_64x64x32_w2x2_s2");
-		sgemm_fast_kernel<64, 2, 2, 2, true, true><<<grid, block, 0, stream()>>>(p);
-		LTEN_HIP_LAUNCH_CHECK();
-		return 0;
-	}
+	// 64 x 64 tiles (a 32 x 32 tile per wavefront): up to two operand reads ride behind an MFMA when an operand is
+	// row-contiguous
+	case 31: return launch_fast<64, 2, 2, 2>(p, tA, tB, batch, "sgemm_fast_64x64x32_w2x2_s2");
 	default: return -1;
 	}
 }

@@ -315,8 +315,6 @@ FAST_TILES = {11: "sgemm_fast_256x256x32_w2x4_s2", 12: "sgemm_fast_256x256x32_w4
 def test_direct_to_lds_tiles_exact_all_layouts(gpu, tile, tA, tB):
     """The direct-to-LDS tiles by number: integer-valued operands make every summation order exact, so the result
     must equal the int64 product bit for bit, with padded leading dimensions, alpha / beta and an untouched pad."""
-    if tile == 31 and (tA, tB) != (0, 1):
-        pytest.skip("the 64 x 64 tiles exist for NT products only")
     rng = np.random.default_rng(500 + 10 * tile + 2 * tA + tB)
     M, N, K = (512, 256, 160) if tile < 20 else (256, 384, 96)   # K / 32 = 5 or 3 k-steps: prologue, steady state, drain
     A = rng.integers(-8, 9, (M, K)).astype(np.float32)
@@ -360,13 +358,13 @@ def test_direct_to_lds_tiles_are_the_default_for_large_aligned_problems(gpu):
     gpu.check(l.lten_hip_fc_forward_f32(300, fin, 3400, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
     assert gpu.last_kernel() == FAST_TILES[31]
     assert np.array_equal(dY.numpy(np.float32, (300, 3400)), x[:300] @ w[:3400].T + b[:3400])
-    # strided batch of 4 (Tensor::matmul over a leading dimension), NN
-    a4 = rng.integers(-4, 5, (4, 512, 256)).astype(np.float32)   # 4 x (4 x 8) tiles of 128
+    # strided batch of 4 (Tensor::matmul over a leading dimension), NN: 128 tiles of 128 x 128 in all, so 64-tiles here too
+    a4 = rng.integers(-4, 5, (4, 512, 256)).astype(np.float32)
     b4 = rng.integers(-4, 5, (4, 256, 1024)).astype(np.float32)
     dA4, dB4, dC4 = D.from_numpy(a4), D.from_numpy(b4), D(4 * 4 * 512 * 1024)
     gpu.check(l.lten_hip_sgemm_strided_batched(0, 0, 512, 1024, 256, 1.0, dA4.ptr, 256, 512 * 256, dB4.ptr, 1024, 256 * 1024, 0.0,
                                                dC4.ptr, 1024, 512 * 1024, 4))
-    assert gpu.last_kernel() == FAST_TILES[21]
+    assert gpu.last_kernel() == FAST_TILES[31]
     assert np.array_equal(dC4.numpy(np.float32, (4, 512, 1024)), a4 @ b4)
     # an operand base that is not 16-byte aligned: general kernel
     dXo = D(x.nbytes + 16)
