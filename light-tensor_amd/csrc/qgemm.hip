@@ -321,8 +321,11 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 		// Problems that tile exactly go to the direct-to-LDS kernels when K is long enough to amortise their prologue
 		// and epilogue: 256x256 tiles once those occupy most of the 256 CUs, 128x128 tiles (up to four times as many
 		// workgroups, two per CU) below that.
-		if (p.K >= 512) {
-			if (ceil_div(p.M, 256) * ceil_div(p.N, 256) > 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
+		// (a shorter K only with many tiles: the positions x channels products of a quantized convolution, 16384 x 64 x
+		// 288: 5.6 against 7.8 us on the guarded kernel)
+		if (p.K >= 512 || (p.K >= 128 && ceil_div(p.M, 128) * ceil_div(p.N, 128) >= 64)) {
+			// 256 x 256 tiles only where both dimensions fill most of one (100352 x 64 x 576: 20.7 us on 128 x 128 tiles, 26.5 on these)
+			if (p.M >= 192 && p.N >= 192 && ceil_div(p.M, 256) * ceil_div(p.N, 256) > 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
 			// about one 256 x 128 tile per CU: less operand traffic per MFMA than two 128 x 128 tiles per CU
 			const uint64_t tiles_256x128 = ceil_div(p.M, 256) * ceil_div(p.N, 128);
 			if (tiles_256x128 > 160 && tiles_256x128 <= 256 && p.K >= 2048 && qgemm_fast_dispatch(p, out, 51) == 0) return 0;
