@@ -122,8 +122,8 @@ static void launch_conv2dq_direct(const dim3& grid, int K, const ConvGeo& g, con
 
 // Row r = n * Ho * Wo + p of the patch matrix: the window of output position p of image n in l-ten's column order
 // (ci, i, j).  Bytes outside the image are 0, as in l-ten's im2col (not the zero point); bytes from K on hold the input
-// zero point.  A thread builds four consecutive bytes of a row; the tap table (offset of the tap inside an image and
-// its (i, j)) is built once per workgroup in LDS.
+// zero point.  A thread builds sixteen consecutive bytes of a row; the tap table (offset of the tap inside an image and
+// its (i, j)) is built once per workgroup in LDS.  (Sixteen bytes and one 16-byte store per thread.)
 __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint8_t* __restrict__ x, uint8_t* __restrict__ rows, int Kp, int zp_in)
 {
 	extern __shared__ int s_tap[];  // [Kp] offsets, then [Kp] i | j << 16
@@ -135,25 +135,31 @@ __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint
 		s_tap[Kp + k] = i | (j << 16);
 	}
 	__syncthreads();
-	const uint32_t kq_per_row = (uint32_t)Kp / 4;
+	const uint32_t chunks_per_row = (uint32_t)Kp / 16;
 	const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-	const uint32_t r = (uint32_t)(idx / kq_per_row), kq = (uint32_t)(idx - (uint64_t)r * kq_per_row);
+	const uint32_t r = (uint32_t)(idx / chunks_per_row), kc = (uint32_t)(idx - (uint64_t)r * chunks_per_row);
 	if (r >= (uint32_t)g.N * (uint32_t)HW) return;
 	const int n = (int)(r / (uint32_t)HW), pos = (int)(r - (uint32_t)n * (uint32_t)HW);
 	const int ho = pos / g.Wo, wo = pos - ho * g.Wo;
 	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
 	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
-	uint32_t word = 0;
+	const int base = y0 * g.W + x0;
+	uint32_t bytes[16];
 #pragma unroll
-	for (int b = 0; b < 4; b++) {
-		const int k = 4 * (int)kq + b;
+	for (int b = 0; b < 16; b++) {  // all sixteen loads first
+		const int k = 16 * (int)kc + b;
 		const int ij = s_tap[Kp + k];
 		const int yy = y0 + (ij & 0xFFFF), xx = x0 + (ij >> 16);
 		const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W);
-		const uint32_t byte = xn[(s_tap[k] + y0 * g.W + x0) & -(int)inside];  // offset 0 for taps outside: always a valid address
-		word |= (k < K ? (inside ? byte : 0u) : (uint32_t)zp_in) << (8 * b);
+		const uint32_t byte = xn[(s_tap[k] + base) & -(int)inside];  // offset 0 for taps outside: always a valid address
+		bytes[b] = k < K ? (inside ? byte : 0u) : (uint32_t)zp_in;
 	}
-	reinterpret_cast<uint32_t*>(rows)[idx] = word;
+	uint4 out;
+	out.x = bytes[0] | bytes[1] << 8 | bytes[2] << 16 | bytes[3] << 24;
+	out.y = bytes[4] | bytes[5] << 8 | bytes[6] << 16 | bytes[7] << 24;
+	out.z = bytes[8] | bytes[9] << 8 | bytes[10] << 16 | bytes[11] << 24;
+	out.w = bytes[12] | bytes[13] << 8 | bytes[14] << 16 | bytes[15] << 24;
+	reinterpret_cast<uint4*>(rows)[idx] = out;
 }
 
 // wp[co][k] for co < Cp, k < Kp: the weights, with the weight zero point past K and in the rows past Cout.
@@ -263,7 +269,7 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		uint8_t* wp = base + bp.off_wp;
 		int32_t* sums = reinterpret_cast<int32_t*>(base + bp.off_acc);
 		int32_t* terms = reinterpret_cast<int32_t*>(base + bp.off_terms);
-		conv2dq_rows_kernel<<<dim3((unsigned)ceil_div(bp.rows * (bp.Kp / 4), 256)), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in);
+		conv2dq_rows_kernel<<<dim3((unsigned)ceil_div(bp.rows * (bp.Kp / 16), 256)), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in);
 		LTEN_HIP_LAUNCH_CHECK();
 		conv2dq_pad_weights_kernel<<<dim3((unsigned)ceil_div(bp.Cp * bp.Kp, 256)), dim3(256), 0, stream()>>>(w, wp, (int)Cout, (int)K, (int)bp.Cp, (int)bp.Kp, zp_w);
 		LTEN_HIP_LAUNCH_CHECK();
