@@ -9,7 +9,7 @@
 // launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
-// Longer windows run as three launches for the whole batch: the patches of all output positions as rows of a
+// Longer windows run as three launches for the whole batch (the first also pads the weights): the patches of all output positions as rows of a
 // [N * Ho * Wo][K] matrix (K padded to a multiple of 16 with the input zero point, the weights padded alike with
 // theirs, so the padding multiplies to nothing), one int8 GEMM of qgemm.hip with the positions as rows (NT: both
 // operands contiguous in K, the shape its MFMA tiles are built for) into int32 sums, and a pass that adds l-ten's
@@ -124,10 +124,21 @@ static void launch_conv2dq_direct(const dim3& grid, int K, const ConvGeo& g, con
 // (ci, i, j).  Bytes outside the image are 0, as in l-ten's im2col (not the zero point); bytes from K on hold the input
 // zero point.  A thread builds sixteen consecutive bytes of a row; the tap table (offset of the tap inside an image and
 // its (i, j)) is built once per workgroup in LDS.  (Sixteen bytes and one 16-byte store per thread.)
-__global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint8_t* __restrict__ x, uint8_t* __restrict__ rows, int Kp, int zp_in)
+__global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint8_t* __restrict__ x, uint8_t* __restrict__ rows, int Kp, int zp_in,
+                                                           unsigned row_blocks, const uint8_t* __restrict__ w, uint8_t* __restrict__ wp, int Cp, int zp_w)
 {
 	extern __shared__ int s_tap[];  // [Kp] offsets, then [Kp] i | j << 16
 	const int K = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	if (blockIdx.x >= row_blocks) {
+		// the workgroups behind the rows pad the weights: wp[co][k] for co < Cp, k < Kp, with the weight zero point past K
+		// and in the rows past Cout
+		const int idx = (int)(blockIdx.x - row_blocks) * 256 + (int)threadIdx.x;
+		if (idx < Cp * Kp) {
+			const int co = idx / Kp, k = idx - co * Kp;
+			wp[idx] = (co < g.Cout && k < K) ? w[(int64_t)co * K + k] : (uint8_t)zp_w;
+		}
+		return;
+	}
 	for (int k = threadIdx.x; k < Kp; k += 256) {
 		const int kc = min(k, K - 1);
 		const int j = kc % g.kw, i = (kc / g.kw) % g.kh, ci = kc / (g.kw * g.kh);
@@ -160,15 +171,6 @@ __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint
 	out.z = bytes[8] | bytes[9] << 8 | bytes[10] << 16 | bytes[11] << 24;
 	out.w = bytes[12] | bytes[13] << 8 | bytes[14] << 16 | bytes[15] << 24;
 	reinterpret_cast<uint4*>(rows)[idx] = out;
-}
-
-// wp[co][k] for co < Cp, k < Kp: the weights, with the weight zero point past K and in the rows past Cout.
-__global__ __launch_bounds__(256) void conv2dq_pad_weights_kernel(const uint8_t* __restrict__ w, uint8_t* __restrict__ wp, int Cout, int K, int Cp, int Kp, int zp_w)
-{
-	const int idx = blockIdx.x * 256 + threadIdx.x;
-	if (idx >= Cp * Kp) return;
-	const int co = idx / Kp, k = idx - co * Kp;
-	wp[idx] = (co < Cout && k < K) ? w[(int64_t)co * K + k] : (uint8_t)zp_w;
 }
 
 // y[n][co][p] = requantize(acc[n * HW + p][co] + bias[p]) (or the int32 sum itself): a workgroup takes 64 positions x 64
@@ -269,9 +271,9 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		uint8_t* wp = base + bp.off_wp;
 		int32_t* sums = reinterpret_cast<int32_t*>(base + bp.off_acc);
 		int32_t* terms = reinterpret_cast<int32_t*>(base + bp.off_terms);
-		conv2dq_rows_kernel<<<dim3((unsigned)ceil_div(bp.rows * (bp.Kp / 16), 256)), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in);
-		LTEN_HIP_LAUNCH_CHECK();
-		conv2dq_pad_weights_kernel<<<dim3((unsigned)ceil_div(bp.Cp * bp.Kp, 256)), dim3(256), 0, stream()>>>(w, wp, (int)Cout, (int)K, (int)bp.Cp, (int)bp.Kp, zp_w);
+		const unsigned row_blocks = (unsigned)ceil_div(bp.rows * (bp.Kp / 16), 256), weight_blocks = (unsigned)ceil_div(bp.Cp * bp.Kp, 256);
+		conv2dq_rows_kernel<<<dim3(row_blocks + weight_blocks), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in, row_blocks, w, wp,
+		                                                                                                (int)bp.Cp, zp_w);
 		LTEN_HIP_LAUNCH_CHECK();
 		if (int rc = lten_hip_quantized_matmul_acc(0, 1, bp.rows, bp.Cp, bp.Kp, rows, wp, sums, qp, nullptr, terms)) return rc;
 		const dim3 grid((unsigned)ceil_div(bp.rows, 64), (unsigned)ceil_div(Cout, 64));
