@@ -29,7 +29,8 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (3, 7, 13, 17, 70, 3, 3, 1, 1, 1, 1),       # 63 taps, two channel blocks
                                  (2, 16, 20, 22, 24, 3, 3, 1, 1, 2, 1),      # 144 taps: patch rows + GEMM + finish
                                  (5, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1),      # l-ten's quantized MNIST conv2: 250 taps (padded to 256)
-                                 (3, 8, 9, 7, 10, 3, 3, 1, 1, 1, 1),         # 72 taps, 10 channels (padded to 12), 63 positions an image
+                                 (3, 8, 9, 7, 10, 3, 3, 1, 1, 1, 1),         # 72 taps, 63 positions an image
+                                 (3, 15, 9, 7, 10, 3, 3, 1, 1, 1, 1),        # 135 taps, 10 channels (padded to 12), 63 positions an image
                                  (2, 64, 6, 10, 70, 3, 3, 1, 1, 1, 1),       # 576 taps, two channel blocks of the finish pass
                                  (4, 128, 5, 5, 33, 1, 1, 0, 0, 1, 1),       # 1x1 with 128 channels
                                  (2, 6, 14, 14, 16, 5, 5, 2, 2, 1, 1),       # 150 taps, padding 2
