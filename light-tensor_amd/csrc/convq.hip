@@ -181,18 +181,20 @@ __global__ __launch_bounds__(256) void conv2dq_finish_kernel(const int32_t* __re
 {
 	__shared__ int s[64][65];
 	const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-	for (int e = threadIdx.x; e < 64 * 64; e += 256) {
-		const int rr = e >> 6, cc = e & 63;
-		s[rr][cc] = acc[(int64_t)min(r0 + rr, rows - 1) * Cp + min(c0 + cc, Cp - 1)];
+	const int ncp = min(64, Cp - c0), nco = min(64, Cout - c0);  // columns of the sums to read, channels to store
+	for (int e = threadIdx.x; e < 64 * ncp; e += 256) {
+		const int rr = e / ncp, cc = e - rr * ncp;
+		s[rr][cc] = acc[(int64_t)min(r0 + rr, rows - 1) * Cp + c0 + cc];
 	}
 	__syncthreads();
-	for (int e = threadIdx.x; e < 64 * 64; e += 256) {
-		const int cc = e >> 6, rr = e & 63;
-		const int r = r0 + rr, co = c0 + cc;
-		if (r >= rows || co >= Cout) continue;
-		const int n = r / HW, pos = r - n * HW;
-		const int v = s[rr][cc] + (bias ? bias[pos] : 0);
-		const int64_t o = ((int64_t)n * Cout + co) * HW + pos;
+	// a thread keeps its position and walks the channels: the position is decomposed once
+	const int rr = threadIdx.x & 63, r = r0 + rr;
+	if (r >= rows) return;
+	const int n = r / HW, pos = r - n * HW;
+	const int b = bias ? bias[pos] : 0;
+	for (int cc = threadIdx.x >> 6; cc < nco; cc += 4) {
+		const int v = s[rr][cc] + b;
+		const int64_t o = ((int64_t)n * Cout + c0 + cc) * HW + pos;
 		if (OUT == Q_OUT_ACC) static_cast<int*>(y)[o] = v;
 		else static_cast<uint8_t*>(y)[o] = (uint8_t)requant<OUT>(v, mult, zp_out);
 	}
