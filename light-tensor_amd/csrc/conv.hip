@@ -280,7 +280,8 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
 	// one with its four-row tile also where the two-row tile would be picked
-	if ((variant == 0 || variant == 5) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
+	// (6: the direct-to-LDS one with its narrow-image tiles however few workgroups that gives)
+	if ((variant == 0 || variant == 5 || variant == 6) && conv_patch_forward_takes(g, x, y) && conv_patch_fast_forward_takes(g, x, w)) return conv_patch_fast_forward(g, x, w, bias, y);
 	// The register-staged patch kernel's tiles are 128 columns wide (the direct-to-LDS one above has 16 x 32 tiles for
 	// narrow images): on images of at most 56 columns more than half of a tile is padding, and with fewer than 256 tiles
 	// CUs stay idle; the implicit GEMM over the batch's flattened pixels is ahead there (32 x 48 x 50 x 50 -> 96

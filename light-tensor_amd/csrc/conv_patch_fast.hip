@@ -26,16 +26,21 @@ namespace {
 // VERT: the tile for narrow images, 16 rows x 32 columns: a wavefront owns four rows of 32 pixels (its four MFMA column
 // blocks lie below one another instead of side by side), the patch is [4 channels][18 rows][40 columns].  On a 28 x 28
 // image 77 % of such tiles are pixels that exist, against 22 % of the 128-column tiles.
-template <int BM_, int TH_, bool VERT_ = false>
+// ELEM (with VERT): the patch is fetched four bytes per lane instead of sixteen, for input rows that do not start on
+// 16-byte boundaries (a width that is no multiple of four): four times the load instructions, the same bytes.
+template <int BM_, int TH_, bool VERT_ = false, bool ELEM_ = false>
 struct FastFwd {
 	static_assert(TH_ == 4 || TH_ == 2, "a wavefront owns a whole row of the tile (TH = 4) or half a row (TH = 2)");
-	static constexpr bool VERT = VERT_;
+	static constexpr bool VERT = VERT_, ELEM = ELEM_;
+	static_assert(!ELEM || VERT, "the 4-byte patch loads exist for the narrow-image tile");
 	static constexpr int BM = BM_, MT = BM / 32, TH = TH_, NT = VERT ? 4 : TH, CB = 4;
 	static constexpr int TW = VERT ? 32 : 128, TROWS = VERT ? 16 : TH, PR = TROWS + 2, PWS = TW + 8, F4R = PWS / 4;
 	static constexpr int BLOCK_STEP = VERT ? PWS : 32;            // floats between a wavefront's MFMA column blocks in the patch
 	static constexpr int PATCH_F4 = CB * PR * F4R;                 // 816
-	static constexpr int PATCH_LOADS = (PATCH_F4 + 63) / 64;       // 13
-	static constexpr int PATCH_BYTES = PATCH_LOADS * 1024;
+	static constexpr int PATCH_UNITS = ELEM ? 4 * PATCH_F4 : PATCH_F4;  // what a lane fetches: a float or four
+	static constexpr int PATCH_LOAD_BYTES = ELEM ? 256 : 1024;          // bytes of one wave-wide patch load
+	static constexpr int PATCH_LOADS = (PATCH_UNITS + 63) / 64;    // 13 (45 with ELEM)
+	static constexpr int PATCH_BYTES = PATCH_LOADS * PATCH_LOAD_BYTES;
 	static constexpr int W_F4 = BM * 9;                            // 36 floats per channel
 	static constexpr int W_LOADS = (W_F4 + 63) / 64;
 	static constexpr int W_BYTES = W_LOADS * 1024;
@@ -48,11 +53,11 @@ struct FastFwd {
 
 }  // namespace
 
-template <int BM, int TH, bool VERT = false>
+template <int BM, int TH, bool VERT = false, bool ELEM = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 256 ? 2 : 4, BM * TH == 256 ? 2 : 4))) void conv2d_patch_fast_forward_kernel(
     ConvGeo g, const float* __restrict__ x, const float* __restrict__ w, const float* __restrict__ bias, float* __restrict__ y)
 {
-	typedef FastFwd<BM, TH, VERT> P;
+	typedef FastFwd<BM, TH, VERT, ELEM> P;
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[2 * P::STAGE];
 
 	const int tid = threadIdx.x, lane = tid & 63;
@@ -76,12 +81,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 		const int q = wave + 4 * i;
 		valid[i] = false;
 		voff[i] = 0;
-		slot[i] = smem_addr + q * 1024;
+		slot[i] = smem_addr + (q < P::PATCH_LOADS ? q * P::PATCH_LOAD_BYTES : P::PATCH_BYTES + (q - P::PATCH_LOADS) * 1024);
 		if (q < P::PATCH_LOADS) {
 			const int idx = q * 64 + lane;
-			const int f = idx % P::F4R, r = (idx / P::F4R) % P::PR, c = idx / (P::F4R * P::PR);
-			const int gy = h0 - g.ph + r, gx = w0 - 4 + 4 * f;
-			if (idx < P::PATCH_F4 && gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
+			constexpr int UPR = ELEM ? P::PWS : P::F4R;  // units per patch row
+			const int f = idx % UPR, r = (idx / UPR) % P::PR, c = idx / (UPR * P::PR);
+			const int gy = h0 - g.ph + r, gx = w0 - 4 + (ELEM ? f : 4 * f);
+			if (idx < P::PATCH_UNITS && gy >= 0 && gy < g.H && gx >= 0 && gx < g.W) {
 				valid[i] = true;
 				voff[i] = (uint32_t)(((c * g.H + gy) * g.W + gx) * 4);
 			}
@@ -98,7 +104,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	auto load_one = [&](int i, int stage, int kt) {
 		if (wave + 4 * i >= P::LOADS) return;  // the same for the whole wavefront
 		const float* base = wave + 4 * i < P::PATCH_LOADS ? xn + kt * x_step : wb + kt * (P::CB * 9);
-		if (valid[i]) async_load16(slot[i] + stage * P::STAGE, base, voff[i]);
+		if (valid[i]) {
+			if (ELEM && wave + 4 * i < P::PATCH_LOADS) async_load4(slot[i] + stage * P::STAGE, base, voff[i]);
+			else async_load16(slot[i] + stage * P::STAGE, base, voff[i]);
+		}
 	};
 
 	// ---- zeros everywhere once: what no load ever writes is the padding
@@ -169,6 +178,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 	case 4: wait_vmcnt_lgkm0<4>(); break;
 	case 5: wait_vmcnt_lgkm0<5>(); break;
 	case 6: wait_vmcnt_lgkm0<6>(); break;
+	case 7: wait_vmcnt_lgkm0<7>(); break;
+	case 8: wait_vmcnt_lgkm0<8>(); break;
+	case 9: wait_vmcnt_lgkm0<9>(); break;
+	case 10: wait_vmcnt_lgkm0<10>(); break;
+	case 11: wait_vmcnt_lgkm0<11>(); break;
+	case 12: wait_vmcnt_lgkm0<12>(); break;
+	case 13: wait_vmcnt_lgkm0<13>(); break;
+	case 14: wait_vmcnt_lgkm0<14>(); break;
 	default: wait_vmcnt_lgkm0<0>(); break;
 	}
 	__syncthreads();
@@ -241,10 +258,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(BM * TH == 
 		}
 }
 
+bool conv_patch_fast_forward_vertical(const ConvGeo& g);
+
 bool conv_patch_fast_forward_takes(const ConvGeo& g, const float* x, const float* w)
 {
+	// Rows off 16-byte boundaries: the narrow-image tile has a form with 4-byte patch loads, the 128-column tile has not.
+	// The narrow-image tiles need enough workgroups: with few, the implicit GEMM over the batch's flattened pixels is
+	// ahead (8 x 128 x 28 x 28 -> 128 channels, 64 workgroups: 55 against 72 us; 64 x 32 x 28 x 28 -> 64, 256 workgroups:
+	// 44 against 23 us), and the 4-byte form, whose loads are four times as many, needs more of them (32 x 32 x 30 x 30
+	// -> 64, 128 workgroups: 24 against 31 us; 32 x 48 x 50 x 50 -> 96, 768 workgroups: 154 against 95 us).
+	const bool rows16 = g.W % 4 == 0 && aligned16(x);
+	if (conv_patch_fast_forward_vertical(g)) {
+		const uint64_t tiles = ceil_div((uint64_t)g.Wo, 32) * ceil_div((uint64_t)g.Ho, 16), wgs = tiles * ceil_div((uint64_t)g.Cout, 32) * g.N;
+		// ... and images that fill at least half of their tiles (64 x 256 x 7 x 7 -> 256 fills a tenth: 118 against 307 us)
+		const bool half_full = 2 * (uint64_t)g.Ho * g.Wo >= tiles * 16 * 32;
+		if ((wgs < (rows16 ? 200u : 256u) || !half_full) && get_option(OPT_CONV_VARIANT) == 0) return false;
+	}
 	return g.sh == 1 && g.sw == 1 && g.dh == 1 && g.dw == 1 && g.kh == 3 && g.kw == 3 && g.pw <= 4 && g.Cin % 4 == 0 && g.Cin >= 8 &&
-	       g.W % 4 == 0 && aligned16(x) && aligned16(w) && (uint64_t)g.H * g.W < (1u << 26) && (uint64_t)g.Ho * g.Wo <= (1u << 26) &&
+	       (rows16 || (conv_patch_fast_forward_vertical(g) && get_option(OPT_CONV_VARIANT) != 5)) && aligned16(w) && (uint64_t)g.H * g.W < (1u << 26) && (uint64_t)g.Ho * g.Wo <= (1u << 26) &&
 	       (uint64_t)64 * g.Cin * 9 * 4 < (1ull << 31) && ceil_div((uint64_t)g.Cout, 32) < 65536 && g.N < 65536;
 }
 
@@ -258,12 +289,15 @@ int conv_patch_fast_forward(const ConvGeo& g, const float* x, const float* w, co
 	if (conv_patch_fast_forward_vertical(g) && get_option(OPT_CONV_VARIANT) != 5) {
 		const unsigned vtiles = (unsigned)(ceil_div((uint64_t)g.Wo, 32) * ceil_div((uint64_t)g.Ho, 16));
 		// 64 output channels per workgroup when that still gives every CU two workgroups, else 32
+		const bool elem = g.W % 4 != 0 || !aligned16(x);  // 4-byte patch loads
 		if (blocks32 % 2 == 0 && (uint64_t)vtiles * blocks64 * g.N >= 512) {
-			set_kernel_name("conv2d_patch_fast_forward_3x3_64x16x32");
-			conv2d_patch_fast_forward_kernel<64, 4, true><<<dim3(vtiles, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+			set_kernel_name(elem ? "conv2d_patch_fast_forward_3x3_64x16x32_e4" : "conv2d_patch_fast_forward_3x3_64x16x32");
+			if (elem) conv2d_patch_fast_forward_kernel<64, 4, true, true><<<dim3(vtiles, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+			else conv2d_patch_fast_forward_kernel<64, 4, true><<<dim3(vtiles, blocks64, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
 		} else {
-			set_kernel_name("conv2d_patch_fast_forward_3x3_32x16x32");
-			conv2d_patch_fast_forward_kernel<32, 4, true><<<dim3(vtiles, blocks32, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+			set_kernel_name(elem ? "conv2d_patch_fast_forward_3x3_32x16x32_e4" : "conv2d_patch_fast_forward_3x3_32x16x32");
+			if (elem) conv2d_patch_fast_forward_kernel<32, 4, true, true><<<dim3(vtiles, blocks32, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
+			else conv2d_patch_fast_forward_kernel<32, 4, true><<<dim3(vtiles, blocks32, (unsigned)g.N), dim3(256), 0, stream()>>>(g, x, w, bias, y);
 		}
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;

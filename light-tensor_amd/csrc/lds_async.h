@@ -16,6 +16,12 @@ __device__ __forceinline__ void async_load16(uint32_t lds_addr, const void* base
 	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
 }
 
+// The 4-byte form: lane L's dword goes to lds_addr + 4*L.  For operands whose rows do not start on 16-byte boundaries.
+__device__ __forceinline__ void async_load4(uint32_t lds_addr, const void* base, uint32_t voff)
+{
+	asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
 // The same for the lanes of `mask` only, without a branch: a taken branch costs a wavefront that is alone on its
 // SIMD far more than the load (its MFMA stream stops while instructions are fetched again).  The execution mask is
 // saved and put back inside the statement, so the compiler never sees it change; lanes that are inactive on entry

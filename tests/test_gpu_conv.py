@@ -167,9 +167,13 @@ def test_conv_narrow_images_on_16x32_tiles(gpu, ob, geo):
     bias = rng.standard_normal(Cout).astype(np.float32)
     Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
     dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
-    y, _, fk = gpu_conv(gpu, geo, x, w, dy, bias)
-    assert fk.startswith("conv2d_patch_fast_forward_3x3_") and fk.endswith("x16x32"), fk
-    _conv_vs_oracle(gpu, ob, geo)
+    gpu.set_option("conv_variant", 6)   # these tiles however few workgroups the small test shapes give
+    try:
+        y, _, fk = gpu_conv(gpu, geo, x, w, dy, bias)
+        assert fk.startswith("conv2d_patch_fast_forward_3x3_") and fk.endswith("x16x32"), fk
+        _conv_vs_oracle(gpu, ob, geo)
+    finally:
+        gpu.set_option("conv_variant", 0)
 
 
 @pytest.mark.parametrize("geo", [(3, 16, 27, 28, 64, 3, 3, 1, 1, 1, 1),      # MNIST-sized with an odd number of rows: the last chunk has one
@@ -252,6 +256,29 @@ def test_conv_data_gradient_with_strides(gpu, ob, geo):
     dx = gpu_dgrad(gpu, geo, w, dy)
     assert gpu.last_kernel() == "conv2d_dgrad_64x64x32", gpu.last_kernel()
     assert rel_err(dx, want_dx) < TOL
+
+
+@pytest.mark.parametrize("geo", [(3, 16, 20, 30, 64, 3, 3, 1, 1, 1, 1),      # 30 columns: rows start 8 bytes off 16-byte boundaries
+                                 (2, 8, 17, 26, 33, 3, 3, 0, 0, 1, 1),      # MNIST after one unpadded 3x3: 26 columns, no padding
+                                 (2, 12, 33, 50, 130, 3, 3, 1, 1, 1, 1),    # two column tiles, three tile rows, three channel blocks
+                                 (5, 64, 15, 15, 64, 3, 3, 1, 1, 1, 1),     # odd width: every row starts at another offset
+                                 (1, 8, 7, 95, 40, 3, 3, 2, 1, 1, 1)])      # three column tiles, the last 31 columns wide, row pad 2
+def test_conv_narrow_images_with_unaligned_rows(gpu, ob, geo):
+    """The 16 x 32 tiles with the patch fetched four bytes per lane: input widths that are no multiple of four, where
+    rows do not start on 16-byte boundaries; forward, and the stride-1 data gradient through it, against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    gpu.set_option("conv_variant", 6)   # these tiles however few workgroups the small test shapes give
+    try:
+        y, _, fk = gpu_conv(gpu, geo, x, w, dy, rng.standard_normal(Cout).astype(np.float32))
+        assert fk.startswith("conv2d_patch_fast_forward_3x3_") and fk.endswith("x16x32_e4"), fk
+        _conv_vs_oracle(gpu, ob, geo)
+    finally:
+        gpu.set_option("conv_variant", 0)
 
 
 def _conv_vs_oracle(gpu, ob, geo):
