@@ -170,39 +170,54 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_wgrad_kernel(ConvGeo g, co
 }
 
 // Data gradient for any stride: dx[n][ci][y][x] = sum over (co, i, j) of dy[n][co][oy][ox] * w[co][ci][i][j] with
-// oy = (y + ph - i) / sh, ox = (x + pw - j) / sw where those divide and lie inside dy.  GEMM rows = ci, columns = the
-// input pixels of the whole batch, reduction over (co, i, j).  Which output row a tap row i reaches from input row y
-// (or none) is tabulated per column of the tile in LDS, likewise for the columns, so a gather costs three table reads
-// and no division.  With a stride above 1 most taps of a pixel reach nothing (three in four at stride 2): the MFMAs
-// run over those zeros, which still beats l-ten's decomposition (a GEMM and a col2im launch per image) many times over.
-constexpr int DG_MAXW = 16;  // window rows and columns the per-column tables hold
+// oy = (y + ph - i) / sh, ox = (x + pw - j) / sw where those divide and lie inside dy.  GEMM rows = ci, columns = input
+// pixels, reduction over (co, i, j).  A pixel is reached only through the tap rows i = (y + ph) mod sh (+ sh, + 2 sh ...)
+// and the tap columns alike, so the pixels are taken class by class (blockIdx.y = (y mod sh, x mod sw)): the columns of
+// a tile are pixels of one class from the whole batch, and the reduction runs over that class's taps only, a quarter of
+// the window at stride 2.  Which output row a tap row reaches from input row y (or none) is tabulated per column of
+// the tile in LDS, likewise for the columns, so a gather costs three table reads and no division.  A class without
+// taps (a 1 x 1 window at stride 2 reaches one pixel in four) stores zeros.
+constexpr int DG_MAXW = 16;    // window rows and columns the per-column tables hold
+constexpr int DG_MAXK = 2304;  // reduction length of a class the LDS tables hold (Cout * taps of the class)
 template <int BM, int BN, int BK, int WM, int WN>
-__global__ __launch_bounds__(WM* WN * 64) void conv2d_dgrad_kernel(ConvGeo g, const float* w, const float* dy, float* dx)
+__global__ __launch_bounds__(WM* WN * 64) void conv2d_dgrad_kernel(ConvGeo g, const float* w, const float* dy, float* dx, int max_tiles_n)
 {
 	typedef GemmCore<BM, BN, BK, WM, WN, false, true> Core;
 	static_assert(Core::T % BN == 0 && (BM * BK) % Core::T == 0 && (BN * BK) % Core::T == 0, "a thread's column is the same in every fetch");
 	__shared__ float lds[Core::LDS_FLOATS];
-	__shared__ KTap ktab[MAX_KTAB];            // per k = (co, i, j): co * Ho * Wo, and i | j << 16
+	__shared__ KTap ktab[DG_MAXK];             // per k = (co, tap of the class): co * Ho * Wo, and i | j << 16
+	__shared__ int wtab[DG_MAXK];              // (co * Cin * kh + i) * kw + j: the weight of channel 0 for that k
 	__shared__ int col_img[BN], col_hw[BN];    // for the stores: image and pixel of every column of the tile (-1: none)
 	__shared__ int row_of[BN][DG_MAXW], column_of[BN][DG_MAXW];  // output row reached through tap row i (-1: none), likewise columns
 
-	const int taps = g.kh * g.kw, Kd = g.Cout * taps, HWi = g.H * g.W, HWo = g.Ho * g.Wo;
-	const int cols = g.N * HWi;  // below 2^31 (checked by the host)
+	const int taps = g.kh * g.kw, HWi = g.H * g.W, HWo = g.Ho * g.Wo;
+	// this workgroup's class of pixels and its taps
+	const int cy = blockIdx.y / g.sw, cx = blockIdx.y % g.sw;
+	const int Hc = cy < g.H ? (g.H - cy + g.sh - 1) / g.sh : 0, Wc = cx < g.W ? (g.W - cx + g.sw - 1) / g.sw : 0;
+	const int i0 = (cy + g.ph) % g.sh, j0 = (cx + g.pw) % g.sw;
+	const int Na = i0 < g.kh ? (g.kh - i0 + g.sh - 1) / g.sh : 0, Nb = j0 < g.kw ? (g.kw - j0 + g.sw - 1) / g.sw : 0;
+	const int Kd = g.Cout * Na * Nb;
+	const int cols = g.N * Hc * Wc;  // below 2^31 (checked by the host)
 	const int tiles_n = (int)(((int64_t)cols + BN - 1) / BN);
-	const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+	const int tn = blockIdx.x % max_tiles_n, m0 = (blockIdx.x / max_tiles_n) * BM, n0 = tn * BN;
+	if (tn >= tiles_n) return;  // the classes differ in size by a row or a column
 	for (int k = threadIdx.x; k < Kd; k += Core::T) {
-		const int co = k / taps, t = k - co * taps, i = t / g.kw;
+		const int co = k / (Na * Nb), t = k - co * (Na * Nb), a = t / Nb;
+		const int i = i0 + g.sh * a, j = j0 + g.sw * (t - a * Nb);
 		ktab[k].off = co * HWo;
-		ktab[k].ij = i | ((t - i * g.kw) << 16);
+		ktab[k].ij = i | (j << 16);
+		wtab[k] = (co * g.Cin * g.kh + i) * g.kw + j;
 	}
 	const unsigned col = (unsigned)n0 + threadIdx.x % BN;
 	const bool col_ok = col < (unsigned)cols;
-	const int img = (int)(min(col, (unsigned)cols - 1) / (unsigned)HWi), hw = (int)(min(col, (unsigned)cols - 1) - (unsigned)img * HWi);
-	const int yy = hw / g.W, xx = hw - yy * g.W;
+	const unsigned per_image = (unsigned)(Hc * Wc);
+	const unsigned colc = min(col, (unsigned)cols - 1);
+	const int img = (int)(colc / per_image), rem = (int)(colc - (unsigned)img * per_image);
+	const int yy = cy + g.sh * (rem / Wc), xx = cx + g.sw * (rem % Wc);
 	const int c = threadIdx.x % BN;
 	if (threadIdx.x < BN) {
 		col_img[c] = col_ok ? img : -1;
-		col_hw[c] = hw;
+		col_hw[c] = yy * g.W + xx;
 		for (int i = 0; i < g.kh; i++) {
 			const int num = yy + g.ph - i, q = num / g.sh;
 			row_of[c][i] = (num >= 0 && q * g.sh == num && q < g.Ho) ? q : -1;
@@ -217,11 +232,10 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_dgrad_kernel(ConvGeo g, co
 
 	auto fetch_a = [&](int row, int k, bool& inside) -> float {
 		inside = (m0 + row < g.Cin) & (k < Kd);
-		const int kc = min(k, Kd - 1), co = kc / taps, t = kc - co * taps;
-		return w[((int64_t)co * g.Cin + min(m0 + row, g.Cin - 1)) * taps + t];
+		return w[wtab[min(k, max(Kd - 1, 0))] + min(m0 + row, g.Cin - 1) * taps];
 	};
 	auto fetch_b = [&](int, int k, bool& inside) -> float {
-		const KTap t = ktab[min(k, Kd - 1)];
+		const KTap t = ktab[min(k, max(Kd - 1, 0))];
 		const int oy = row_of[c][t.ij & 0xFFFF], ox = column_of[c][t.ij >> 16];
 		inside = col_ok & (k < Kd) & ((oy | ox) >= 0);
 		return dyi[(t.off + oy * g.Wo + ox) & -(int)inside];
@@ -237,8 +251,10 @@ __global__ __launch_bounds__(WM* WN * 64) void conv2d_dgrad_kernel(ConvGeo g, co
 
 static bool dgrad_gemm_takes(const ConvGeo& g)
 {
-	return g.dh == 1 && g.dw == 1 && g.kh <= DG_MAXW && g.kw <= DG_MAXW && (uint64_t)g.Cout * g.kh * g.kw <= MAX_KTAB &&
-	       (uint64_t)g.N * g.H * g.W < (1ull << 31) && (uint64_t)g.Cout * g.Ho * g.Wo < (1ull << 31);
+	const uint64_t class_taps = ceil_div((uint64_t)g.kh, g.sh) * ceil_div((uint64_t)g.kw, g.sw);
+	return g.dh == 1 && g.dw == 1 && g.kh <= DG_MAXW && g.kw <= DG_MAXW && (uint64_t)g.Cout * class_taps <= DG_MAXK &&
+	       g.sh * g.sw <= 64 && (uint64_t)g.N * g.H * g.W < (1ull << 31) && (uint64_t)g.Cout * g.Ho * g.Wo < (1ull << 31) &&
+	       (uint64_t)g.Cout * g.Cin * g.kh * g.kw < (1ull << 31);
 }
 
 static int make_geo(ConvGeo& g, uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout, int kh, int kw, int ph,
@@ -500,7 +516,9 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	// any stride: one implicit-GEMM launch for the batch (64 x 64 x 28 x 28 <- 128 channels at stride 2: 722 us image by image)
 	if (get_option(OPT_CONV_VARIANT) == 0 && (!few_narrow || !dgrad_as_forward(g)) && dgrad_gemm_takes(g)) {
 		set_kernel_name("conv2d_dgrad_64x64x32");
-		conv2d_dgrad_kernel<64, 64, 32, 2, 2><<<dim3((unsigned)(ceil_div(Cin, 64) * ceil_div(N * H * W, 64))), dim3(256), 0, stream()>>>(g, w, dy, dx);
+		// one grid row per class of pixels (y mod sh, x mod sw); class (0, 0) has the most
+		const uint64_t max_tiles_n = ceil_div(N * ceil_div(H, (uint64_t)sh) * ceil_div(W, (uint64_t)sw), 64);
+		conv2d_dgrad_kernel<64, 64, 32, 2, 2><<<dim3((unsigned)(ceil_div(Cin, 64) * max_tiles_n), (unsigned)(sh * sw)), dim3(256), 0, stream()>>>(g, w, dy, dx, (int)max_tiles_n);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}
