@@ -241,10 +241,12 @@ def test_conv_data_gradient_of_first_layers(gpu, ob, geo):
     (1, 70, 8, 8, 3, 1, 1, 0, 0, 2, 2),       # 1 x 1 at stride 2: three pixels in four get no gradient
     (2, 8, 15, 15, 8, 4, 4, 1, 1, 3, 3),      # stride 3, even window
     (5, 33, 7, 6, 65, 3, 3, 1, 1, 2, 1),      # two row tiles, columns that cross images
+    (2, 4, 1, 9, 6, 1, 3, 0, 1, 3, 2),        # one image row at stride 3: two of the three row classes hold no pixel
 ])
 def test_conv_data_gradient_with_strides(gpu, ob, geo):
-    """Data gradient at strides above 1: one implicit-GEMM launch for the batch (rows = input channels, columns = input
-    pixels, per-column tables of the output rows and columns each tap reaches), against the oracle."""
+    """Data gradient at strides above 1: one implicit-GEMM launch for the batch (rows = input channels, columns = the input
+    pixels of one class (y mod sh, x mod sw) per grid row, reduction over the taps that reach that class, per-column
+    tables of the output rows and columns each tap reaches), against the oracle."""
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
     w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
