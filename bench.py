@@ -497,14 +497,14 @@ def main():
     X, W, sc, zp = wl.cfg3()
     l = lt.lib()
     dA, dB = lt.DeviceBuffer.from_numpy(X), lt.DeviceBuffer.from_numpy(W)
-    dBp = lt.DeviceBuffer(N * K)
-    lt.check(l.lten_hip_fcq_prepare_weights(dB.ptr, dBp.ptr, N * K))   # once per layer, as FullyConnected_q::to(GPU) does
+    dBp, dBs = lt.DeviceBuffer(N * K), lt.DeviceBuffer(4 * N)
+    lt.check(l.lten_hip_fcq_prepare_weights(dB.ptr, dBp.ptr, N, K, dBs.ptr))   # once per layer, as FullyConnected_q::to(GPU) does
     dC = lt.DeviceBuffer(M * N)
     ws = lt.DeviceBuffer(4 * (M + N))
     qp = lt.qparams3(sc, zp)
 
     def step():
-        lt.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dA.ptr, dBp.ptr, None, qp, dC.ptr, ws.ptr))
+        lt.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dA.ptr, dBp.ptr, dBs.ptr, None, qp, dC.ptr, ws.ptr))
 
     def step_raw():
         lt.quantized_matmul(False, True, M, N, K, dA, dB, dC, qp, None, ws)
@@ -530,6 +530,32 @@ def main():
     ops = 2.0 * M * N * K
     raw_ms = sustained(step_raw)
     raw_kernel = lt.last_kernel()
+
+    # The same product with zero points that need the correction terms: a post-relu activation tensor (zero point 0)
+    # against symmetric weights, and a general triple.  On prepared weights both stay one launch.
+    general_zp = []
+    for zps in ((0, 128, 128), (17, 250, 100)):
+        qpz = lt.qparams3(sc, zps)
+
+        def step_zp():
+            lt.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dA.ptr, dBp.ptr, dBs.ptr, None, qpz, dC.ptr, ws.ptr))
+
+        def step_zp_raw():
+            lt.quantized_matmul(False, True, M, N, K, dA, dB, dC, qpz, None, ws)
+        zms = sustained(step_zp)
+        zkern = lt.last_kernel()
+        ok = None
+        if not args.no_verify:
+            acc = ((X.astype(np.float64) - float(zps[0])) @ (W.astype(np.float64) - float(zps[1])).T)
+            mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+            sfl = (acc.astype(np.float32) * mult).astype(np.float32) + np.float32(zps[2])
+            ok = bool(np.array_equal(dC.numpy(np.uint8, (M, N)), (np.trunc(sfl).astype(np.int64) & 0xFF).astype(np.uint8)))
+        zraw_ms = sustained(step_zp_raw)
+        general_zp.append({"zero_points_in_wt_out": list(zps), "kernel": zkern, "launches": 1, "sustained_kernel_us": round(zms * 1e3, 2),
+                           "tops": round(ops / (zms * 1e-3) / 1e12, 1),
+                           "roofline": {"bound": "mfma", "achieved": round(ops / (zms * 1e-3) / 1e12, 1), "peak": INT8_MFMA_PEAK_TOPS,
+                                        "unit": "TOP/s", "frac": round(ops / (zms * 1e-3) / 1e12 / INT8_MFMA_PEAK_TOPS, 4)},
+                           "raw_uint8_weights_two_launches_us": round(zraw_ms * 1e3, 2), "verified_bit_exact": ok})
     sustained_ms = sustained(step)
     achieved = ops / (sustained_ms * 1e-3) / 1e12
 
@@ -623,6 +649,7 @@ def main():
                      "measured_mfma_only_data_operands_shader_mhz": {str(k): round(v) for k, v in data_mhz.items()},
                      "frac_of_measured_mfma_only_data_operands": round(achieved / measured_peak_data, 4),
                      "vendor_int8_gemm_same_shape": vendor,
+                     "same_shape_other_zero_points": general_zp,
                      "note": "int8 multiply-add counted as 2 ops; achieved = 2*4096^3 / sustained_kernel_us (300 back-to-back "
                              "launches after at least 60 ms of the same load, HIP events on the library's stream); "
                              "timed_region_kernel_us = the same over the --steps launches; measured_mfma_only = a kernel that "
@@ -638,7 +665,7 @@ def main():
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(X, W, sc, zp)
-    del dA, dB, dBp, dC, ws
+    del dA, dB, dBp, dBs, dC, ws
     if not args.no_extra:
         out["configs"] = extra_configs(lt, wl, not args.no_cpu)
     print(json.dumps(out), flush=True)

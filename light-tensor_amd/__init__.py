@@ -53,8 +53,8 @@ _SIGNATURES = {
     "lten_hip_quantized_matmul_acc": (C.c_int, [C.c_int, C.c_int, u64, u64, u64, vp, vp, vp, C.POINTER(QParams), vp,
                                                 vp]),
     "lten_hip_fcq_forward": (C.c_int, [u64, u64, u64, u64, vp, vp, vp, C.POINTER(QParams), vp, vp]),
-    "lten_hip_fcq_forward_prepared": (C.c_int, [u64, u64, u64, u64, vp, vp, vp, C.POINTER(QParams), vp, vp]),
-    "lten_hip_fcq_prepare_weights": (C.c_int, [vp, vp, u64]),
+    "lten_hip_fcq_forward_prepared": (C.c_int, [u64, u64, u64, u64, vp, vp, vp, vp, C.POINTER(QParams), vp, vp]),
+    "lten_hip_fcq_prepare_weights": (C.c_int, [vp, vp, u64, u64, vp]),
     "lten_hip_fcq_forward_static": (C.c_int, [u64, u64, u64, u64, vp, vp, vp, C.POINTER(QParams), vp]),
     "lten_hip_im2col_f32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),
     "lten_hip_im2col_i32": (C.c_int, [vp] + [C.c_int] * 11 + [vp]),

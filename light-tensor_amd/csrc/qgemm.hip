@@ -308,7 +308,9 @@ static int launch_tile(const QProblem& p, int out, const char* name)
 	return 0;
 }
 
-static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratch)
+// fast_only: try the direct-to-LDS tiles alone and return -1 when none of them takes the problem (the caller then
+// prepares the zero-point vectors the general kernels need and calls again).
+static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratch, bool fast_only = false)
 {
 	const bool kmajor = p.a_ks == 1 && p.b_ks == 1;
 	const bool c_ok = (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
@@ -343,6 +345,7 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits, scratch) == 0) return 0;
 			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
 		}
+		if (fast_only) return -1;
 		if (fits(256, 256, 64) && out_elems >= 256ull * 256 * 192)
 			choice = 1;
 		else if (fits(128, 128, 64) && out_elems >= 128ull * 128 * 128)
@@ -354,9 +357,11 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 	}
 	if (choice >= 20) {
 		const int rc = qgemm_fast_dispatch(p, out, choice);
+		if (fast_only) return rc;
 		LTEN_HIP_REQUIRE(rc >= 0, "qgemm: forced fast variant %d does not fit this problem", choice);
 		return rc;
 	}
+	if (fast_only) return -1;
 	switch (choice) {
 	case 1:
 		LTEN_HIP_REQUIRE(fits(256, 256, 64), "qgemm: forced 256x256x64 tile does not fit this problem");
@@ -381,7 +386,7 @@ struct RunScratch {
 
 static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A, const uint8_t* B, void* C,
                      int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace,
-                     bool weights_prepared = false, const RunScratch* scratch = nullptr)
+                     bool weights_prepared = false, const RunScratch* scratch = nullptr, const int32_t* weight_sums = nullptr)
 {
 	LTEN_HIP_REQUIRE(qp != nullptr, "quantized_matmul: qparams is null");
 	if (M == 0 || N == 0) return 0;
@@ -461,6 +466,16 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	}
 
 	const int coef_a = 128 - zpB, coef_b = 128 - zpA;
+	// Prepared weights come with their byte sums: the tiled kernels then work out every zero-point term themselves
+	// and this call is one launch.
+	if (weights_prepared && weight_sums != nullptr && (coef_a != 0 || coef_b != 0 || bias != nullptr)) {
+		QProblem f = p;
+		f.wsum = weight_sums;
+		f.bias = bias;
+		f.coef_a = coef_a;
+		f.coef_b = coef_b;
+		if (qgemm_dispatch(f, out, scratch ? &scratch->split : nullptr, true) == 0) return 0;
+	}
 	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {
 		if (scratch != nullptr) {
 			LTEN_HIP_REQUIRE(M + N <= scratch->terms_ints, "quantized_matmul: M + N = %llu exceeds the %llu rows and columns the static scratch holds",
@@ -482,6 +497,40 @@ __global__ __launch_bounds__(256) void fcq_prepare_weights_kernel(const v4i* __r
 {
 	for (uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256) dst[i] = flip_sign_bits(src[i]);
 	if (blockIdx.x == 0 && (int)threadIdx.x < tail) dst_tail[threadIdx.x] = src_tail[threadIdx.x] ^ 0x80;
+}
+
+// The same conversion row by row, with each weight row's byte sum (of the uint8 values, as l-ten/math_fns.cpp:1364-1369
+// adds them up on every call) kept in sums[row]: one wavefront per row.
+__global__ __launch_bounds__(256) void fcq_prepare_weights_sums_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int32_t* __restrict__ sums,
+                                                                       uint64_t rows, uint64_t cols, int vec_ok)
+{
+	const int lane = threadIdx.x & 63;
+	const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+	if (row >= rows) return;
+	const uint8_t* r = src + row * cols;
+	uint8_t* w = dst + row * cols;
+	unsigned sum = 0;
+	uint64_t k = 0;
+	if (vec_ok) {
+		for (k = (uint64_t)lane * 16; k + 16 <= cols; k += 64 * 16) {
+			const v4i v = *reinterpret_cast<const v4i*>(r + k);
+			const unsigned one = 0x01010101u;
+			sum = __builtin_amdgcn_udot4((unsigned)v.x, one, sum, false);
+			sum = __builtin_amdgcn_udot4((unsigned)v.y, one, sum, false);
+			sum = __builtin_amdgcn_udot4((unsigned)v.z, one, sum, false);
+			sum = __builtin_amdgcn_udot4((unsigned)v.w, one, sum, false);
+			*reinterpret_cast<v4i*>(w + k) = flip_sign_bits(v);
+		}
+		k = cols / 16 * 16;  // what is left of the row: fewer than 16 bytes
+	}
+	for (uint64_t kk = k + lane; kk < cols; kk += 64) {
+		const uint8_t b = r[kk];
+		sum += b;
+		w[kk] = b ^ 0x80;
+	}
+#pragma unroll
+	for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
+	if (lane == 0) sums[row] = (int32_t)sum;
 }
 
 // Scratch of lten_hip_fcq_forward_static: device memory that exists from the moment the library is loaded, so the
@@ -549,12 +598,22 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
 	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, workspace);
 }
 
-int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t count)
+int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t out_features, uint64_t in_features, int32_t* weight_sums)
 {
+	const uint64_t count = out_features * in_features;
 	if (count == 0) return 0;
 	LTEN_HIP_REQUIRE(W && W_prepared, "lten_hip_fcq_prepare_weights: null pointer");
 	LTEN_HIP_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(W_prepared)) & 15) == 0,
 	                 "lten_hip_fcq_prepare_weights: both buffers must be 16-byte aligned");
+	if (weight_sums != nullptr) {
+		LTEN_HIP_REQUIRE((reinterpret_cast<uintptr_t>(weight_sums) & 15) == 0, "lten_hip_fcq_prepare_weights: weight_sums must be 16-byte aligned");
+		LTEN_HIP_REQUIRE(out_features < (1ull << 31) && in_features * 255ull < (1ull << 31), "lten_hip_fcq_prepare_weights: dimension too large");
+		const unsigned blocks = (unsigned)ceil_div(out_features, 4);
+		fcq_prepare_weights_sums_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(W, W_prepared, weight_sums, out_features, in_features,
+		                                                                           in_features % 16 == 0 ? 1 : 0);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	const uint64_t n16 = count / 16;
 	const int tail = (int)(count % 16);
 	const unsigned blocks = (unsigned)std::min<uint64_t>(std::max<uint64_t>(ceil_div(n16, 256), 1), 4096);
@@ -565,10 +624,12 @@ int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t
 }
 
 int lten_hip_fcq_forward_prepared(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features, const uint8_t* X,
-                                  const uint8_t* W_prepared, const int32_t* bias, const lten_hip_qparams* qparams, uint8_t* Y,
-                                  int32_t* workspace)
+                                  const uint8_t* W_prepared, const int32_t* weight_sums, const int32_t* bias,
+                                  const lten_hip_qparams* qparams, uint8_t* Y, int32_t* workspace)
 {
-	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W_prepared, Y, 0, qparams, bias, workspace, true);
+	LTEN_HIP_REQUIRE(weight_sums != nullptr, "lten_hip_fcq_forward_prepared: weight_sums is null (lten_hip_fcq_prepare_weights fills it)");
+	LTEN_HIP_REQUIRE((reinterpret_cast<uintptr_t>(weight_sums) & 15) == 0, "lten_hip_fcq_forward_prepared: weight_sums must be 16-byte aligned");
+	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W_prepared, Y, 0, qparams, bias, workspace, true, nullptr, weight_sums);
 }
 
 int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features, uint64_t out_features, const uint8_t* X,
@@ -579,8 +640,9 @@ int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features
 	                 (unsigned long long)(batch * M + out_features), (unsigned long long)STATIC_TERMS_INTS);
 	RunScratch rs;
 	if (int rc = static_scratch(&rs)) return rc;
-	// the array keeps whatever the last call left: the arrival counters of a split-K launch must start at zero
-	if (int rc = lten_hip_zero(rs.split.counters, (size_t)rs.split.max_tiles * sizeof(unsigned))) return rc;
+	// The array keeps whatever the last call left.  The arrival counters of a split-K launch must start at zero, and
+	// they do without a fill launch: the array is zero when the code object is loaded, and the workgroup that arrives
+	// last at a tile stores zero into its counter again (qgemm_fast_kernel).
 	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, nullptr, false, &rs);
 }
 

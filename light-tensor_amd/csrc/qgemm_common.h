@@ -31,6 +31,14 @@ struct QProblem {
 	int32_t* split_partial;     // [tile][split][T*T] partial sums in register order
 	unsigned* split_counters;   // [tile] arrivals; zero between launches
 	int splits;
+	// Zero-point terms worked out by the tiled kernel itself (prepared weights only; rterm and cterm are null then):
+	// the column term is coef_b * wsum[n] + bias[n] with wsum the weight rows' byte sums kept since the weights were
+	// prepared, the row term coef_a * (byte sum of activation row m), which the kernel takes from the operand
+	// fragments it feeds to the matrix cores.  l-ten/math_fns.cpp:1362-1380 computes both on every call.
+	const int32_t* wsum = nullptr;  // [N] sum_k W[n][k] of the uint8 weight bytes, 16-byte aligned; null = not fused
+	const int32_t* bias = nullptr;  // [N] or null (fused form only)
+	int coef_a = 0;                 // 128 - zpB
+	int coef_b = 0;                 // 128 - zpA
 };
 
 // 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).

@@ -22,7 +22,14 @@
 // beat and the wavefronts, which issue in order, stop feeding the matrix pipe while they queue.
 //
 // The zero-point terms of a tile (per row, per column, constant) are what its accumulators start from, so the
-// epilogue is the requantize alone: a wavefront turns each of its 32-row blocks into bytes (the convert
+// epilogue is the requantize alone.  TERMS says where they come from: 0 = only the constant (both zero points 128, no
+// bias); 1 = the vectors a launch of qgemm_terms_kernel left in the caller's workspace; 2 = the column term is worked
+// out here from the weight sums kept since the weights were prepared (coef_b * wsum[n] + bias[n]) and there is no row
+// term; 3 = the same, and the row term comes from the activation fragments on their way into the matrix cores: before
+// the sign flip a fragment holds l-ten's uint8 bytes, and one instruction adds four of them to a sum.  The two wavefronts that multiply the same
+// activation rows share that work (each sums the row blocks j with j % WN == wn), the sums meet in LDS behind the
+// main loop and are added to the accumulators there.  No launch but this one runs in forms 2 and 3.
+// The epilogue: a wavefront turns each of its 32-row blocks into bytes (the convert
 // instruction drops its byte into the packed word itself), passes them through a strip of LDS of its own to
 // get whole row segments of TN bytes, and stores those with the non-temporal hint (the output is not read
 // again by this kernel, and lines that leave the L2 early do not have to be written back when the kernel ends).
@@ -32,7 +39,7 @@
 
 namespace lten_hip {
 
-template <int BM, int BN, int BK, int WM, int WN, int S, int OUT, bool TERMS, bool SPLIT = false, bool TAIL = false, bool WPRE = false>
+template <int BM, int BN, int BK, int WM, int WN, int S, int OUT, int TERMS, bool SPLIT = false, bool TAIL = false, bool WPRE = false>
 __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 {
 	constexpr int W = WM * WN;
@@ -48,6 +55,8 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	constexpr int WP = TN + 16;  // row pitch of a wavefront's output strip in LDS (keeps rows 16-byte aligned)
 	static_assert(W * 32 * WP <= S * STAGE, "the output strips fit into the operand stages");
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[S * STAGE];
+	constexpr bool ROWSUM = TERMS == 3;
+	__shared__ int row_sums[ROWSUM ? BM : 1];  // TERMS == 3: byte sum over this workgroup's share of K, per tile row
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -120,39 +129,102 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	const int chunk0 = lgrp ^ swz<CPR>(lrow);
 	const int off_w = BM * BK + (wn * TN + lrow) * BK + (chunk0 << 4);
 	const int off_x = (wm * TM + lrow) * BK + (chunk0 << 4);
+	// Which 32-row block of the wavefront's activation rows its fragment slot j holds: block j, except that with
+	// TERMS == 3 and two wavefronts per row of wavefronts the second one holds them in the other order, so that "the
+	// slot I sum" is slot 0 for both and the main loop needs no branch on the wavefront's number.
+	static_assert(!ROWSUM || WN == 1 || (WN == 2 && FM == 2), "sharing of the row sums");
+	const int jsw = (ROWSUM && WN == 2) ? wn : 0;
+	int xblk[FM];  // byte offset of slot j's row block inside the activation tile
+#pragma unroll
+	for (int j = 0; j < FM; j++) xblk[j] = (j ^ jsw) * 32 * BK;
 
 	// Accumulators start from the zero-point terms.  Lane (lrow, lgrp), register 4q + e of block (i, j) is the output at
-	//   m = m0 + wm*TM + j*32 + lrow,  n = n0 + wn*TN + i*32 + 8q + 4*lgrp + e.
-	// With SPLIT only the workgroup with the first share of K carries them.
+	//   m = m0 + wm*TM + (j ^ jsw)*32 + lrow,  n = n0 + wn*TN + i*32 + 8q + 4*lgrp + e.
+	// With SPLIT only the workgroup with the first share of K carries them.  The loads of the term vectors are issued
+	// behind the first stages' loads (init_acc is called there): ahead of them they cost the prologue a second round
+	// trip to memory, 2.5 us at 4096^3.
 	v16i acc[FN][FM];
-	{
+	auto init_acc = [&]() {
 		const bool carry = !SPLIT || blockIdx.y == 0;
 		int rt[FM];
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
 			rt[j] = carry ? p.konst : 0;
-			if (TERMS && carry) rt[j] += p.rterm[min(m0 + wm * TM + j * 32 + lrow, p.M - 1)];
+			if (TERMS == 1 && carry) rt[j] += p.rterm[min(m0 + wm * TM + (j ^ jsw) * 32 + lrow, p.M - 1)];
+		}
+		// Every load below is unconditional, from a column clamped into the matrix (N % 4 == 0: four columns exist
+		// together; what a clamped load brings is never stored), and the one choice, how the bias is fetched, is made
+		// outside the loops: a branch per vector would make each load wait for the one before it.
+		v4i ct[FN][4];
+		const int ncol = n0 + wn * TN + lgrp * 4;
+		const bool have = TERMS != 0 && carry;
+#pragma unroll
+		for (int i = 0; i < FN; i++)
+#pragma unroll
+			for (int q = 0; q < 4; q++) ct[i][q] = v4i{ 0, 0, 0, 0 };
+		if (TERMS == 1 && have) {
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int q = 0; q < 4; q++) ct[i][q] = *reinterpret_cast<const v4i*>(p.cterm + min(ncol + i * 32 + q * 8, p.N - 4));
+		}
+		if (TERMS >= 2 && have) {
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int q = 0; q < 4; q++) {
+					const v4i ws = *reinterpret_cast<const v4i*>(p.wsum + min(ncol + i * 32 + q * 8, p.N - 4));
+#pragma unroll
+					for (int e = 0; e < 4; e++) ct[i][q][e] = ws[e] * p.coef_b;
+				}
+			if (p.bias != nullptr && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) {
+#pragma unroll
+				for (int i = 0; i < FN; i++)
+#pragma unroll
+					for (int q = 0; q < 4; q++) ct[i][q] += *reinterpret_cast<const v4i*>(p.bias + min(ncol + i * 32 + q * 8, p.N - 4));
+			} else if (p.bias != nullptr) {  // a bias vector that only has the alignment of its ints
+#pragma unroll
+				for (int i = 0; i < FN; i++)
+#pragma unroll
+					for (int q = 0; q < 4; q++) {
+						const int32_t* b = p.bias + min(ncol + i * 32 + q * 8, p.N - 4);
+						ct[i][q] += v4i{ b[0], b[1], b[2], b[3] };
+					}
+			}
 		}
 #pragma unroll
 		for (int i = 0; i < FN; i++)
 #pragma unroll
-			for (int q = 0; q < 4; q++) {
-				v4i ct = { 0, 0, 0, 0 };
-				const int n = n0 + wn * TN + i * 32 + q * 8 + lgrp * 4;
-				if (TERMS && carry && n < p.N) ct = *reinterpret_cast<const v4i*>(p.cterm + n);  // N % 4 == 0: the four exist together
+			for (int q = 0; q < 4; q++)
 #pragma unroll
 				for (int j = 0; j < FM; j++)
 #pragma unroll
-					for (int e = 0; e < 4; e++) acc[i][j][q * 4 + e] = rt[j] + ct[e];
-			}
-	}
+					for (int e = 0; e < 4; e++) acc[i][j][q * 4 + e] = rt[j] + ct[i][q][e];
+	};
 
+	// TERMS == 3: this wavefront's share of the activation row sums, lane (lrow, lgrp) holding the bytes it has fed so
+	// far.  A fragment is added up right before its sign flip, while it still holds l-ten's uint8 bytes: one
+	// sum-of-absolute-differences against zero per dword (full rate; the 4 x int8 dot product that would take the
+	// flipped bytes issues at a quarter of that and cost 3.2 us at 4096^3 against 0.9), each dword into a sum of its own
+	// so that no instruction waits for the one before.
+	constexpr int NSUM = WN == 1 ? FM : 1;  // row blocks (fragment slots) this wavefront sums
+	unsigned rsum[NSUM][4];
+#pragma unroll
+	for (int j = 0; j < NSUM; j++)
+#pragma unroll
+		for (int d = 0; d < 4; d++) rsum[j][d] = 0;
+	auto add_rowsum = [&](int j, const v4i& raw) {
+		if (ROWSUM && j < NSUM) {
+#pragma unroll
+			for (int d = 0; d < 4; d++) rsum[j][d] = __builtin_amdgcn_sad_u8((unsigned)raw[d], 0u, rsum[j][d]);
+		}
+	};
 	auto read_frags = [&](v4i(&fw)[FN], v4i(&fx)[FM], int stg, int s) {
 		const uint8_t* sbase = smem + stg * STAGE;
 #pragma unroll
 		for (int i = 0; i < FN; i++) fw[i] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + i * 32 * BK);
 #pragma unroll
-		for (int j = 0; j < FM; j++) fx[j] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + j * 32 * BK);
+		for (int j = 0; j < FM; j++) fx[j] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + xblk[j]);
 	};
 	auto flip_frags = [&](v4i(&fw)[FN], v4i(&fx)[FM]) {
 		if (!WPRE) {
@@ -160,7 +232,10 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 			for (int i = 0; i < FN; i++) fw[i] = flip_sign_bits(fw[i]);
 		}
 #pragma unroll
-		for (int j = 0; j < FM; j++) fx[j] = flip_sign_bits(fx[j]);
+		for (int j = 0; j < FM; j++) {
+			add_rowsum(j, fx[j]);
+			fx[j] = flip_sign_bits(fx[j]);
+		}
 	};
 	auto mma = [&](const v4i(&fw)[FN], const v4i(&fx)[FM]) {
 #pragma unroll
@@ -196,12 +271,15 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 			if (DENSE) {
 #pragma unroll
 				for (int f = 2 * m; f < 2 * m + 2 && f < NR; f++) {
-					if (f < FM) nx[f] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + f * 32 * BK);
+					if (f < FM) nx[f] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + xblk[f]);
 					else nw[f - FM] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + (f - FM) * 32 * BK);
 				}
 				if (m == NM - 1) {
 #pragma unroll
-					for (int f = 0; f < FM; f++) nx[f] = flip_sign_bits(nx[f]);
+					for (int f = 0; f < FM; f++) {
+						add_rowsum(f, nx[f]);
+						nx[f] = flip_sign_bits(nx[f]);
+					}
 					if (!WPRE) {
 #pragma unroll
 						for (int f = 0; f < FN; f++) nw[f] = flip_sign_bits(nw[f]);
@@ -210,13 +288,19 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 			} else {
 				if (m < NR) {
 					if (m < FN) nw[m] = *reinterpret_cast<const v4i*>(sbase + (off_w ^ (s << 5)) + m * 32 * BK);
-					else nx[m - FN] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + (m - FN) * 32 * BK);
+					else nx[m - FN] = *reinterpret_cast<const v4i*>(sbase + (off_x ^ (s << 5)) + xblk[m - FN]);
 				}
 				if (m >= FLIP0) {
 					const int f = m - FLIP0;
-					if (WPRE) nx[f] = flip_sign_bits(nx[f]);
-					else if (f < FN) nw[f] = flip_sign_bits(nw[f]);
-					else nx[f - FN] = flip_sign_bits(nx[f - FN]);
+					if (WPRE) {
+						add_rowsum(f, nx[f]);
+						nx[f] = flip_sign_bits(nx[f]);
+					} else if (f < FN) {
+						nw[f] = flip_sign_bits(nw[f]);
+					} else {
+						add_rowsum(f - FN, nx[f - FN]);
+						nx[f - FN] = flip_sign_bits(nx[f - FN]);
+					}
 				}
 			}
 			if (refill) {
@@ -238,7 +322,10 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	v4i fw0[FN], fx0[FM], fw1[FN], fx1[FM];
 	const int pre = min(S, KT);
 	for (int st = 0; st < pre; st++) issue(st, st);
-	if (S == 2) { if (pre == 2) wait_vmcnt<LPW>(); else wait_vmcnt<0>(); }
+	init_acc();
+	// with term vectors this wavefront's youngest loads are theirs, not a stage's: wait for everything
+	if (TERMS != 0) wait_vmcnt<0>();
+	else if (S == 2) { if (pre == 2) wait_vmcnt<LPW>(); else wait_vmcnt<0>(); }
 	else wait_stages(TAIL && KT <= S ? 0 : pre - 1);
 	__syncthreads();
 	read_frags(fw0, fx0, 0, 0);
@@ -284,6 +371,29 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	inner_beats(stage, 0, 0, 0);
 	mma(fw1, fx1);
 
+	// TERMS == 3: the two k-halves of a row sit in lanes lrow and lrow + 32; the wavefront that summed row block j
+	// leaves the sums in LDS, every wavefront of that row of wavefronts picks them up and adds coef_a times the sum to
+	// the accumulators of the row (with SPLIT each workgroup adds its own share of K, which the exchange below sums).
+	// The bytes that pad a partial last k-step are 0x80 before the flip and count 128 each: taken off again here.
+	if (ROWSUM) {
+#pragma unroll
+		for (int j = 0; j < FM; j++)
+			if (WN == 1 || j == 0) {
+				const int mine = (int)(rsum[j < NSUM ? j : 0][0] + rsum[j < NSUM ? j : 0][1] + rsum[j < NSUM ? j : 0][2] + rsum[j < NSUM ? j : 0][3]);
+				const int both = mine + __shfl_xor(mine, 32, 64) - (TAIL ? 128 * (KT * BK - p.K) : 0);
+				if (lgrp == 0) row_sums[wm * TM + (j ^ jsw) * 32 + lrow] = both;
+			}
+		__syncthreads();
+#pragma unroll
+		for (int j = 0; j < FM; j++) {
+			const int rt = row_sums[wm * TM + (j ^ jsw) * 32 + lrow] * p.coef_a;
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int r = 0; r < 16; r++) acc[i][j][r] += rt;
+		}
+	}
+
 	// Split K: every workgroup of a tile publishes its partial sums (in register order, so a wavefront of any of them
 	// reads back exactly what the same wavefront of another wrote), then counts itself in; the one that arrives last
 	// adds the others' sums to its own and carries on to the epilogue.  int32 sums do not depend on the order.  The
@@ -326,7 +436,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	if (OUT == Q_OUT_ACC) {
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
-			const int m = m0 + wm * TM + j * 32 + lrow;
+			const int m = m0 + wm * TM + (j ^ jsw) * 32 + lrow;
 			if (m >= p.M) continue;
 #pragma unroll
 			for (int i = 0; i < FN; i++)
@@ -350,6 +460,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		uint8_t* const cbase = static_cast<uint8_t*>(p.C) + (int64_t)row0 * p.N + col0;
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
+			const int jrow = (j ^ jsw) * 32;  // the tile rows of this slot
 #pragma unroll
 			for (int i = 0; i < FN; i++)
 #pragma unroll
@@ -376,14 +487,14 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 				for (int t = 0; t < 32 / RPI; t++) {
 					const int r = t * RPI + lane / LPS, ch = lane % LPS;
 					const v4i val = *reinterpret_cast<const v4i*>(strip + r * WP + ch * 16);
-					if (row0 + j * 32 + r < p.M && col0 + ch * 16 < p.N)
-						__builtin_nontemporal_store(val, reinterpret_cast<v4i*>(cbase + (int64_t)(j * 32 + r) * p.N + ch * 16));
+					if (row0 + jrow + r < p.M && col0 + ch * 16 < p.N)
+						__builtin_nontemporal_store(val, reinterpret_cast<v4i*>(cbase + (int64_t)(jrow + r) * p.N + ch * 16));
 				}
 			} else {  // N is a multiple of 4: four bytes at a time
 				for (int c = lane; c < 32 * (TN / 4); c += 64) {
 					const int r = c / (TN / 4), dw = c % (TN / 4);
-					if (row0 + j * 32 + r < p.M && col0 + dw * 4 < p.N)
-						*reinterpret_cast<int*>(cbase + (int64_t)(j * 32 + r) * p.N + dw * 4) = *reinterpret_cast<const int*>(strip + r * WP + dw * 4);
+					if (row0 + jrow + r < p.M && col0 + dw * 4 < p.N)
+						*reinterpret_cast<int*>(cbase + (int64_t)(jrow + r) * p.N + dw * 4) = *reinterpret_cast<const int*>(strip + r * WP + dw * 4);
 				}
 			}
 			wait_vmcnt_lgkm0<63>();  // the strip is read before the next block overwrites it
@@ -392,18 +503,43 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	}
 }
 
+// Which TERMS form a launch takes; -1 = a combination these kernels are not built for (prepared weights with the
+// vectors of qgemm_terms_kernel, raw weights with kept sums): the caller falls back to the general kernels.
+static int fast_terms_mode(const QProblem& p)
+{
+	const bool wpre = p.b_flip == 0;
+	if (p.wsum != nullptr) return wpre && p.rterm == nullptr && p.cterm == nullptr ? (p.coef_a != 0 ? 3 : 2) : -1;
+	if (p.rterm != nullptr) return wpre ? -1 : 1;
+	return 0;
+}
+
+// The reported kernel name says which zero-point terms the launch worked out itself.
+static void set_fast_name(const char* name, int terms)
+{
+	char full[96];
+	snprintf(full, sizeof(full), "%s%s", name, terms == 3 ? "+zpcol+zprow" : terms == 2 ? "+zpcol" : "");
+	set_kernel_name(full);
+}
+
 template <int BM, int BN, int BK, int WM, int WN, int S, bool TAIL = false, bool WPRE = false>
 static int launch_fast(const QProblem& p, int out, const char* name)
 {
 	if (!TAIL && p.K % BK != 0) return -1;
 	const dim3 grid((unsigned)(ceil_div(p.M, BM) * ceil_div(p.N, BN))), block(WM * WN * 64);
-	const bool terms = p.rterm != nullptr;
-	set_kernel_name(name);
+	// prepared weights come with their sums (TERMS 2 or 3, or 0 when no term is needed), raw weights with the vectors of
+	// qgemm_terms_kernel (1 or 0): see fast_terms_mode
+	const int terms = fast_terms_mode(p);
+	if (terms < 0) return -1;
+	set_fast_name(name, terms);
 #define LTEN_LAUNCH(OUTV)                                                                                            \
-	if (terms)                                                                                                   \
-		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, true, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);      \
+	if (WPRE && terms == 3)                                                                                      \
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, WPRE ? 3 : 0, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p); \
+	else if (WPRE && terms == 2)                                                                                 \
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, WPRE ? 2 : 0, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p); \
+	else if (!WPRE && terms == 1)                                                                                \
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, WPRE ? 0 : 1, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p); \
 	else                                                                                                         \
-		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, false, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);
+		qgemm_fast_kernel<BM, BN, BK, WM, WN, S, OUTV, 0, false, TAIL, WPRE><<<grid, block, 0, stream()>>>(p);
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
@@ -444,29 +580,34 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits, const Spli
 	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
+	                  (reinterpret_cast<uintptr_t>(p.wsum) & 15) == 0 &&
 	                  tiles * T * T * 4 * splits <= scratch->partial_bytes && tiles <= (uint64_t)scratch->max_tiles;
 	if (!fits) return -1;
 	p.split_partial = scratch->partial;
 	p.split_counters = scratch->counters;
 	p.splits = splits;
 	const dim3 grid((unsigned)tiles, (unsigned)splits), block(256);
-	const bool terms = p.rterm != nullptr;
+	const int terms = fast_terms_mode(p);
+	if (terms < 0) return -1;
 	const bool wpre = p.b_flip == 0;
 	// a ring of four stages where a CU holds one workgroup anyway and the share of K is long enough to repay the
 	// longer prologue (see launch_tile128)
 	const bool deep = p.K / splits >= 4096 && tiles * splits <= 256;
-	set_kernel_name(deep ? (wpre ? "qgemm_fast_128x128x128_w2x2_s4_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s4_splitk")
-	                     : (wpre ? "qgemm_fast_128x128x128_w2x2_s2_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s2_splitk"));
+	set_fast_name(deep ? (wpre ? "qgemm_fast_128x128x128_w2x2_s4_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s4_splitk")
+	                   : (wpre ? "qgemm_fast_128x128x128_w2x2_s2_splitk_wpre" : "qgemm_fast_128x128x128_w2x2_s2_splitk"), terms);
 #define LTEN_LAUNCH3(OUTV, TERMSV, WPREV)                                                                           \
 	if (deep) qgemm_fast_kernel<T, T, BK, 2, 2, 4, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p); \
 	else qgemm_fast_kernel<T, T, BK, 2, 2, 2, OUTV, TERMSV, true, false, WPREV><<<grid, block, 0, stream()>>>(p);
-#define LTEN_LAUNCH2(OUTV, TERMSV) if (wpre) { LTEN_LAUNCH3(OUTV, TERMSV, true) } else { LTEN_LAUNCH3(OUTV, TERMSV, false) }
-#define LTEN_LAUNCH(OUTV) if (terms) { LTEN_LAUNCH2(OUTV, true) } else { LTEN_LAUNCH2(OUTV, false) }
+#define LTEN_LAUNCH(OUTV)                                                     \
+	if (terms == 3) { LTEN_LAUNCH3(OUTV, 3, true) }                           \
+	else if (terms == 2) { LTEN_LAUNCH3(OUTV, 2, true) }                      \
+	else if (terms == 1) { LTEN_LAUNCH3(OUTV, 1, false) }                     \
+	else if (wpre) { LTEN_LAUNCH3(OUTV, 0, true) }                            \
+	else { LTEN_LAUNCH3(OUTV, 0, false) }
 	if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_LAUNCH(Q_OUT_U8_EXACT) }
 	else { LTEN_LAUNCH(Q_OUT_ACC) }
 #undef LTEN_LAUNCH
-#undef LTEN_LAUNCH2
 #undef LTEN_LAUNCH3
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
@@ -498,7 +639,8 @@ int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % 16 == 0 && p.K >= 128 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
-	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0);
+	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
+	                  (reinterpret_cast<uintptr_t>(p.wsum) & 15) == 0;
 	if (!fits) return -1;
 	const bool wpre = p.b_flip == 0;
 	const bool ktail = p.K % 128 != 0;

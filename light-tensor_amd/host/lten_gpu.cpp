@@ -581,7 +581,8 @@ void FullyConnected_q::to(device target_device, int target_device_index)
 	if (use_bias_ && bias_.defined()) bias_ = bias_.to(target_device, target_device_index);
 	workspace_ = Tensor();
 	max_rows_ = 0;
-	prepared_ = Tensor();  // the int8 copy of the weights is made again by the next forward
+	prepared_ = Tensor();  // the int8 copy of the weights and their row sums are made again by the next forward
+	weight_sums_ = Tensor();
 	prepared_valid_ = false;
 }
 
@@ -593,6 +594,7 @@ void FullyConnected_q::clear_gradients()
 
 std::vector<Tensor*> FullyConnected_q::get_all_weights()
 {
+	prepared_valid_ = false;  // the caller may write new weights through these (l-ten/net.h:227-236 does)
 	std::vector<Tensor*> w{ &weight_ };
 	if (use_bias_) w.push_back(&bias_);
 	return w;
@@ -632,17 +634,21 @@ Tensor FullyConnected_q::forward(Tensor& input)
 	}
 	lten_hip_qparams qp[3] = { { qparams_in_.scale, qparams_in_.zero_point }, { qparams_wt_.scale, qparams_wt_.zero_point },
 		                   { qparams_out_.scale, qparams_out_.zero_point } };
-	// The weights are constant between forward calls: their int8 form (w - 128, what the matrix cores multiply) is
-	// made once per to() / weights_changed() and every forward runs on it.
+	// The weights are constant between forward calls: their int8 form (w - 128, what the matrix cores multiply) and the
+	// byte sum of every weight row (the zero-point correction's column term, l-ten/math_fns.cpp:1362-1369) are made
+	// once per to() / weights_changed() / hand-out of the weight tensor, and every forward runs on them.
 	if (!prepared_valid_) {
 		options.data_type = UINT8;
 		if (!prepared_.defined()) prepared_ = AllocateTensor({ 1, 1, output_features_, input_features_ }, &options);
+		options.data_type = INT32;
+		if (!weight_sums_.defined()) weight_sums_ = AllocateTensor({ output_features_ }, &options);
 		LTEN_HIP_CALL(lten_hip_fcq_prepare_weights(static_cast<const uint8_t*>(weight_.get_data_ptr()), static_cast<uint8_t*>(prepared_.get_data_ptr()),
-		                                           output_features_ * input_features_));
+		                                           output_features_, input_features_, static_cast<int32_t*>(weight_sums_.get_data_ptr())));
 		prepared_valid_ = true;
 	}
 	LTEN_HIP_CALL(lten_hip_fcq_forward_prepared(batch, M, input_features_, output_features_, static_cast<const uint8_t*>(input.get_data_ptr()),
 	                                            static_cast<const uint8_t*>(prepared_.get_data_ptr()),
+	                                            static_cast<const int32_t*>(weight_sums_.get_data_ptr()),
 	                                            use_bias_ ? static_cast<const int32_t*>(bias_.get_data_ptr()) : nullptr, qp,
 	                                            static_cast<uint8_t*>(result.get_data_ptr()), static_cast<int32_t*>(workspace_.get_data_ptr())));
 	return result;

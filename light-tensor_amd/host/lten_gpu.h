@@ -148,7 +148,11 @@ public:
 	    : input_features_(input_features), output_features_(output_features), use_bias_(use_bias) { (void)data_type; }
 	bool init() override;
 	Tensor forward(Tensor& input);
-	Tensor* get_weights() { return &weight_; }
+	// The accessors that hand out the weight tensor for writing (l-ten's load_checkpoint fills GPU-resident parameters
+	// through get_all_weights, l-ten/net.h:227-236) mark the layer's int8 copy of the weights stale: the next forward
+	// converts them again.  A caller that keeps the pointer and writes through it after a later forward must call
+	// weights_changed() itself.
+	Tensor* get_weights() { prepared_valid_ = false; return &weight_; }
 	Tensor* get_bias() { return use_bias_ ? &bias_ : nullptr; }
 	void clear_gradients() override;
 	std::vector<Tensor*> get_all_weights() override;
@@ -163,7 +167,8 @@ public:
 private:
 	uint64_t input_features_, output_features_;
 	Tensor weight_, bias_, workspace_;
-	Tensor prepared_;  // int8 form of weight_ for the GEMM (lten_hip_fcq_prepare_weights)
+	Tensor prepared_;     // int8 form of weight_ for the GEMM (lten_hip_fcq_prepare_weights)
+	Tensor weight_sums_;  // byte sum of every weight row, made by the same call
 	bool prepared_valid_ = false;
 	bool use_bias_;
 	uint64_t max_rows_ = 0;

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "lten_gpu.h"
+#include "../../include/lten_hip.h"
 
 template <typename Dtype>
 static int Compare(const Dtype* A, const Dtype* B, uint64_t len, double error = 0)
@@ -340,6 +341,54 @@ static int fcq_test()
 	return Compare((uint8_t*)Y.get_data_ptr(), want.data(), want.size());
 }
 
+// A layer whose weights are written again while it sits on the GPU (what l-ten's load_checkpoint does through
+// get_all_weights, l-ten/net.h:227-236): the forward that follows must run on the new weights, not on the int8 copy
+// and row sums made for the old ones.  Shape on the direct-to-LDS tiles, zero points that need every correction term.
+static int fcq_reload_test()
+{
+	const uint64_t M = 160, K = 512, N = 256;
+	std::vector<uint8_t> x(M * K), w0(N * K), w1(N * K);
+	unsigned s = 4321;
+	auto rnd = [&]() { s = s * 1664525u + 1013904223u; return (s >> 16) & 0xFF; };
+	for (auto& e : x) e = (uint8_t)rnd();
+	for (auto& e : w0) e = (uint8_t)rnd();
+	for (auto& e : w1) e = (uint8_t)rnd();
+	lten::TensorOps ops;
+	ops.data_type = lten::UINT8;
+	lten::Tensor X = lten::TensorFromBuffer({ 1, M, K }, x.data(), false, &ops).to(lten::GPU);
+	lten::FullyConnected_q fc(K, N, false);
+	fc.init();
+	fc.train(false);
+	memcpy(fc.get_weights()->get_data_ptr(), w0.data(), w0.size());
+	QuantizationParams qi{ 0.02f, 17 }, qw{ 0.013f, 250 }, qo{ 3.1f, 100 };
+	fc.set_qparams_in(qi);
+	fc.set_qparams_params(&qw, 1);
+	fc.set_qparams_out(qo);
+	fc.to(lten::GPU);
+	const float mult = qi.scale * qw.scale / qo.scale;
+	auto expect = [&](const std::vector<uint8_t>& w, std::vector<uint8_t>& want) {
+		want.resize(M * N);
+		for (uint64_t r = 0; r < M; r++)
+			for (uint64_t n = 0; n < N; n++) {
+				int acc = 0;
+				for (uint64_t k = 0; k < K; k++) acc += ((int)x[r * K + k] - qi.zero_point) * ((int)w[n * K + k] - qw.zero_point);
+				volatile float p = mult * (float)acc;
+				volatile float sum = p + (float)qo.zero_point;
+				want[r * N + n] = (uint8_t)((int)sum & 0xFF);
+			}
+	};
+	std::vector<uint8_t> want;
+	lten::Tensor Y = fc.forward(X).to(lten::CPU);
+	expect(w0, want);
+	if (Compare((uint8_t*)Y.get_data_ptr(), want.data(), want.size())) return -1;
+	// new weights straight into the GPU-resident tensor, as a checkpoint loader does
+	std::vector<lten::Tensor*> params = fc.get_all_weights();
+	if (lten_hip_copy_to_gpu(params[0]->get_data_ptr(), w1.data(), w1.size()) != 0) return -1;
+	Y = fc.forward(X).to(lten::CPU);
+	expect(w1, want);
+	return Compare((uint8_t*)Y.get_data_ptr(), want.data(), want.size());
+}
+
 // Conv2d_q (the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network, plus a padded strided one) against plain loops
 static int convq_test()
 {
@@ -513,7 +562,7 @@ int main(int argc, char** argv)
 		try { return api_bench(); } catch (std::exception& e) { printf("exception: %s\n", e.what()); return 1; }
 	}
 	struct { const char* name; int (*fn)(); } tests[] = { { "matmul_test", matmul_test }, { "fc_test", fc_test }, { "fc_chain_test", fc_chain_test }, { "mlp_step_test", mlp_step_test }, { "training_test", training_test }, { "conv_training_test", conv_training_test },
-		                                                  { "fcq_test", fcq_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
+		                                                  { "fcq_test", fcq_test }, { "fcq_reload_test", fcq_reload_test }, { "conv_test", conv_test }, { "convq_test", convq_test }, { "error_test", error_test } };
 	int failed = 0;
 	for (auto& t : tests) {
 		printf("running %s\n", t.name);

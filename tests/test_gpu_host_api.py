@@ -16,5 +16,5 @@ def test_host_layer_program():
     print(r.stdout)
     print(r.stderr[-2000:])
     assert r.returncode == 0
-    for name in ("matmul_test", "fc_test", "fc_chain_test", "mlp_step_test", "training_test", "conv_training_test", "fcq_test", "conv_test", "convq_test", "error_test"):
+    for name in ("matmul_test", "fc_test", "fc_chain_test", "mlp_step_test", "training_test", "conv_training_test", "fcq_test", "fcq_reload_test", "conv_test", "convq_test", "error_test"):
         assert f"{name} passed" in r.stdout

@@ -198,7 +198,8 @@ def test_direct_to_lds_256x128_tiles(gpu, ob, shape):
         got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, A, B, sc, zp, bias, prepared=True)
     finally:
         gpu.set_option("qgemm_tile", 0)
-    assert k0.startswith("qgemm_fast_256x128") and k1 == k0 + "_wpre", (k0, k1)
+    # prepared weights: the tiles work out the zero-point terms themselves (the name says which), no launch before them
+    assert k0.startswith("qgemm_fast_256x128") and k1 == k0 + "_wpre+zpcol+zprow", (k0, k1)
     assert np.array_equal(got, want)
 
 
@@ -508,11 +509,13 @@ def fcq(gpu, entry, X, W, sc, zp, bias=None, prepared=False):
     dX, dW, dY, ws = D.from_numpy(X), D.from_numpy(W), D(M * N), D(4 * (M + N))
     db = D.from_numpy(np.asarray(bias, np.int32)) if bias is not None else None
     if prepared:
-        dWp = D(W.size + 16)
-        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, W.size))
+        dWp, dS = D(W.size + 16), D(4 * N + 16)
+        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, N, K, dS.ptr))
         assert np.array_equal(dWp.numpy(np.uint8, W.shape), W ^ 0x80)
-        dW = dWp
-    gpu.check(entry(1, M, K, N, dX.ptr, dW.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
+        assert np.array_equal(dS.numpy(np.int32, (N,)), W.sum(axis=1, dtype=np.int64))
+        gpu.check(entry(1, M, K, N, dX.ptr, dWp.ptr, dS.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
+    else:
+        gpu.check(entry(1, M, K, N, dX.ptr, dW.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
     return dY.numpy(np.uint8, (M, N)), gpu.last_kernel()
 
 
@@ -534,6 +537,10 @@ def test_prepared_weights_match_unprepared(gpu, ob, shape):
         want, k0 = fcq(gpu, l.lten_hip_fcq_forward, X, W, sc, zp, bias)
         got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, X, W, sc, zp, bias, prepared=True)
         assert np.array_equal(got, want), (shape, zp, k0, k1)
+        # the direct-to-LDS tiles on prepared weights take the zero-point terms in the same launch
+        # (the name says which terms the launch took on; the unfused form is a launch of qgemm_terms_kernel before it)
+        if k1.startswith("qgemm_fast"):
+            assert k1.endswith("" if zp == [128, 128, 128] and not with_bias else "+zpcol" if zp[1] == 128 else "+zpcol+zprow"), k1
         Co, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias)
         assert np.array_equal(want, Co), (shape, zp, k0)
 
@@ -543,8 +550,15 @@ def test_prepare_weights_in_place_and_odd_count(gpu):
     for n in (1, 15, 16, 17, 4099, 1 << 20):
         w = rng.integers(0, 256, n, dtype=np.uint8)
         d = gpu.DeviceBuffer.from_numpy(w)
-        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, n))
+        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, 1, n, None))
         assert np.array_equal(d.numpy(np.uint8, (n,)), w ^ 0x80)
+    # with the row sums, on rows of any length (16-byte loads only where every row allows them)
+    for rows, cols in ((1, 1), (3, 15), (5, 16), (7, 100), (130, 784), (64, 4099), (33, 4096)):
+        w = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
+        d, sums = gpu.DeviceBuffer.from_numpy(w), gpu.DeviceBuffer(4 * rows + 16)
+        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, rows, cols, sums.ptr))
+        assert np.array_equal(d.numpy(np.uint8, (rows, cols)), w ^ 0x80)
+        assert np.array_equal(sums.numpy(np.int32, (rows,)), w.sum(axis=1, dtype=np.int64))
 
 
 def test_cfg3_prepared_weights_full_size(gpu, wl):
@@ -555,3 +569,59 @@ def test_cfg3_prepared_weights_full_size(gpu, wl):
     got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, X, W, sc, zp, prepared=True)
     assert k1.endswith("_wpre") and not k0.endswith("_wpre"), (k0, k1)
     assert np.array_equal(got, want)
+
+
+ZP_FUSED = ([0, 128, 128], [17, 250, 100])   # a post-relu activation tensor against symmetric weights; every term needed
+
+
+@pytest.mark.parametrize("tile", [33, 41, 51, 0])
+@pytest.mark.parametrize("shape", [(512, 512, 512), (300, 260, 400), (256, 384, 4096), (130, 1024, 8192)])
+def test_prepared_forward_takes_zero_point_terms_in_the_gemm_launch(gpu, ob, shape, tile):
+    """Prepared weights with their row sums: the direct-to-LDS tiles (256 x 256, 128 x 128, 256 x 128, forced by option,
+    and whatever the heuristic picks, split-K included) work out the column term from the kept sums and the row term
+    from the activation fragments, in the one launch, with and without a bias (16-byte aligned and not), whole and
+    ragged tiles and a partial last k-step.  Checked against the oracle."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 5 + N * 3 + K + tile)
+    X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    dX, dW, dWp, dS, dY, ws = D.from_numpy(X), D.from_numpy(W), D(W.size), D(4 * N), D(M * N), D(4 * (M + N))
+    gpu.check(l.lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, N, K, dS.ptr))
+    bias = rng.integers(-5000, 5000, N + 1).astype(np.int32)
+    dbias = D.from_numpy(bias)
+    gpu.set_option("qgemm_tile", tile)
+    seen_fast = False
+    try:
+        for zp in ZP_FUSED:
+            for bias_off in (None, 0, 1):
+                sc = [0.02, 0.013, 0.9 * K / 512]
+                b = None if bias_off is None else bias[bias_off:bias_off + N]
+                gpu.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dX.ptr, dWp.ptr, dS.ptr, None if b is None else dbias.ptr + 4 * bias_off,
+                                                          gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
+                kern = gpu.last_kernel()
+                assert tile == 0 or kern.startswith("qgemm_fast"), kern   # (small outputs go to the one-launch kernel by themselves)
+                if kern.startswith("qgemm_fast"):
+                    assert kern.endswith("+zpcol" if zp[1] == 128 else "+zpcol+zprow"), kern
+                    seen_fast = True
+                want, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=b)
+                assert np.array_equal(dY.numpy(np.uint8, (M, N)), want), (shape, tile, zp, bias_off, kern)
+    finally:
+        gpu.set_option("qgemm_tile", 0)
+    assert seen_fast or shape in ((300, 260, 400), (256, 384, 4096)), shape
+
+
+@pytest.mark.parametrize("zp", ZP_FUSED)
+def test_cfg3_shape_with_general_zero_points_full_size(gpu, wl, zp):
+    """4096^3 with zero points other than 128 on prepared weights: one launch (the name says so), every output equal to
+    the requantize rule applied to the exact closed form of the accumulator."""
+    X, W, sc, _ = wl.cfg3()
+    M = N = K = 4096
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    dX, dW, dWp, dS, dY = D.from_numpy(X), D.from_numpy(W), D(W.size), D(4 * N), D(M * N)
+    gpu.check(l.lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, N, K, dS.ptr))
+    gpu.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dX.ptr, dWp.ptr, dS.ptr, None, gpu.qparams3(sc, zp), dY.ptr, None))
+    assert gpu.last_kernel() == "qgemm_fast_256x256x128_w4x2_s2_wpre" + ("+zpcol" if zp[1] == 128 else "+zpcol+zprow"), gpu.last_kernel()
+    want = exact_acc(X, W, zp[0], zp[1])
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    assert np.array_equal(dY.numpy(np.uint8, (M, N)), requant_numpy(want, mult, zp[2]))
