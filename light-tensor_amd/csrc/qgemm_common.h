@@ -39,6 +39,7 @@ struct QProblem {
 	const int32_t* bias = nullptr;  // [N] or null (fused form only)
 	int coef_a = 0;                 // 128 - zpB
 	int coef_b = 0;                 // 128 - zpA
+	int32_t acc_offset = 0;         // set by the tiled kernels' launchers: see accumulator_offset (qgemm_fast.hip)
 };
 
 // 16-byte-chunk swizzle: chunk kc of tile row `row` lives at chunk kc ^ swz(row).

@@ -56,6 +56,12 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 	static_assert(W * 32 * WP <= S * STAGE, "the output strips fit into the operand stages");
 	__shared__ __attribute__((aligned(1024))) uint8_t smem[S * STAGE];
 	constexpr bool ROWSUM = TERMS == 3;
+	// The accumulators of a requantizing launch run at a distance from zero (QProblem::acc_offset, added to what they
+	// start from and taken off again before the convert; with wrapping int32 arithmetic the result is the same bit for
+	// bit): sums that hover around zero change sign all the time, and every sign change toggles all upper bits of a
+	// two's-complement accumulator in the matrix pipe, which costs clock under the part's power limit (4096^3 on
+	// uniform x N(0,40) bytes: 56.9 -> 55.3 us on one part, the subtraction in the epilogue included).
+	constexpr bool OFFSET = !SPLIT && OUT != Q_OUT_ACC;
 	__shared__ int row_sums[ROWSUM ? BM : 1];  // TERMS == 3: byte sum over this workgroup's share of K, per tile row
 
 	const int tid = threadIdx.x, lane = tid & 63;
@@ -150,6 +156,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
 			rt[j] = carry ? p.konst : 0;
+			if (OFFSET) rt[j] += p.acc_offset;
 			if (TERMS == 1 && carry) rt[j] += p.rterm[min(m0 + wm * TM + (j ^ jsw) * 32 + lrow, p.M - 1)];
 		}
 		// Every load below is unconditional, from a column clamped into the matrix (N % 4 == 0: four columns exist
@@ -386,7 +393,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		__syncthreads();
 #pragma unroll
 		for (int j = 0; j < FM; j++) {
-			const int rt = row_sums[wm * TM + (j ^ jsw) * 32 + lrow] * p.coef_a;
+			const int rt = row_sums[wm * TM + (j ^ jsw) * 32 + lrow] * p.coef_a - (OFFSET ? p.acc_offset : 0);
 #pragma unroll
 			for (int i = 0; i < FN; i++)
 #pragma unroll
@@ -456,6 +463,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		// arithmetic of the next.
 		__syncthreads();  // every wavefront is done reading operand stages (SPLIT: and the arrival word)
 		uint8_t* const strip = smem + wave * (32 * WP);
+		const int epi_off = (OFFSET && !ROWSUM) ? p.acc_offset : 0;  // with row sums the offset went out with the row term
 		const int row0 = m0 + wm * TM, col0 = n0 + wn * TN;
 		uint8_t* const cbase = static_cast<uint8_t*>(p.C) + (int64_t)row0 * p.N + col0;
 #pragma unroll
@@ -467,13 +475,13 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 				for (int q = 0; q < 4; q++) {
 					unsigned word = 0;
 					if (OUT == Q_OUT_U8_FAST) {
-						requant_into<0>(word, acc[i][j][q * 4 + 0], p.mult, p.zp_c);
-						requant_into<1>(word, acc[i][j][q * 4 + 1], p.mult, p.zp_c);
-						requant_into<2>(word, acc[i][j][q * 4 + 2], p.mult, p.zp_c);
-						requant_into<3>(word, acc[i][j][q * 4 + 3], p.mult, p.zp_c);
+						requant_into<0>(word, acc[i][j][q * 4 + 0] - epi_off, p.mult, p.zp_c);
+						requant_into<1>(word, acc[i][j][q * 4 + 1] - epi_off, p.mult, p.zp_c);
+						requant_into<2>(word, acc[i][j][q * 4 + 2] - epi_off, p.mult, p.zp_c);
+						requant_into<3>(word, acc[i][j][q * 4 + 3] - epi_off, p.mult, p.zp_c);
 					} else {
-						const unsigned b0 = requant<OUT>(acc[i][j][q * 4], p.mult, p.zp_c), b1 = requant<OUT>(acc[i][j][q * 4 + 1], p.mult, p.zp_c);
-						const unsigned b2 = requant<OUT>(acc[i][j][q * 4 + 2], p.mult, p.zp_c), b3 = requant<OUT>(acc[i][j][q * 4 + 3], p.mult, p.zp_c);
+						const unsigned b0 = requant<OUT>(acc[i][j][q * 4] - epi_off, p.mult, p.zp_c), b1 = requant<OUT>(acc[i][j][q * 4 + 1] - epi_off, p.mult, p.zp_c);
+						const unsigned b2 = requant<OUT>(acc[i][j][q * 4 + 2] - epi_off, p.mult, p.zp_c), b3 = requant<OUT>(acc[i][j][q * 4 + 3] - epi_off, p.mult, p.zp_c);
 						word = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
 					}
 					*reinterpret_cast<unsigned*>(strip + lrow * WP + i * 32 + q * 8 + lgrp * 4) = word;
@@ -513,6 +521,17 @@ static int fast_terms_mode(const QProblem& p)
 	return 0;
 }
 
+// How far from zero a requantizing launch keeps its accumulators (see OFFSET in the kernel): the smallest of
+// 0x2AAAAAAA, 0x0AAAAAAA, 0x02AAAAAA, ... that no sum of K products of two int8 values can bring below zero.  The
+// alternating bits keep the distance clear of a power of two, where a sum that passes it would toggle a run of bits
+// just as a change of sign does (4096^3: 0x800000 55.5 us, 0xAAAAAA 54.9, 0x2AAAAAAA 55.1, none 56.4).
+static int32_t accumulator_offset(int K)
+{
+	int32_t off = 0x2AAAAAAA;
+	while ((off >> 2) >= (int64_t)K * 16384) off >>= 2;
+	return off;
+}
+
 // The reported kernel name says which zero-point terms the launch worked out itself.
 static void set_fast_name(const char* name, int terms)
 {
@@ -522,9 +541,11 @@ static void set_fast_name(const char* name, int terms)
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int S, bool TAIL = false, bool WPRE = false>
-static int launch_fast(const QProblem& p, int out, const char* name)
+static int launch_fast(const QProblem& q, int out, const char* name)
 {
-	if (!TAIL && p.K % BK != 0) return -1;
+	if (!TAIL && q.K % BK != 0) return -1;
+	QProblem p = q;
+	p.acc_offset = accumulator_offset(p.K);
 	const dim3 grid((unsigned)(ceil_div(p.M, BM) * ceil_div(p.N, BN))), block(WM * WN * 64);
 	// prepared weights come with their sums (TERMS 2 or 3, or 0 when no term is needed), raw weights with the vectors of
 	// qgemm_terms_kernel (1 or 0): see fast_terms_mode
