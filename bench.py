@@ -78,6 +78,81 @@ def vendor_int8(timeout_s=240):
 SETTLE_S = 0.06
 
 
+def telemetry(lt, fn, seconds=2.0):
+    """Socket power, power cap and shader clock while `fn` is launched back to back for `seconds`: a side thread reads
+    the amdgpu hwmon files (power1_input, power1_cap, in microwatts) and the current level of pp_dpm_sclk every 20 ms,
+    and asks amd-smi once, a second into the run, for the socket power and the clock of each of the eight XCDs (a child
+    process; it never touches this process's GPU state).  The hwmon power figure is a filtered one that takes about
+    half a second to follow a load step, so the reported values are medians over the second half of the run.  Fields
+    the box does not offer are None."""
+    import glob
+    import re
+    import subprocess
+    import threading
+    power_f = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input") +
+               glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_average") + [None])[0]
+    cap_f = (glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap") + [None])[0]
+    sclk_f = (glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk") + [None])[0]
+    samples, smi, stop = [], {}, threading.Event()
+    t0 = time.perf_counter()
+
+    def sampler():
+        while not stop.is_set():
+            rec = [time.perf_counter() - t0, None, None]
+            try:
+                if power_f:
+                    rec[1] = int(open(power_f).read()) / 1e6
+                if sclk_f:
+                    cur = [ln for ln in open(sclk_f).read().splitlines() if "*" in ln]
+                    m = re.search(r"(\d+)\s*[Mm][Hh]z", cur[0]) if cur else None
+                    rec[2] = int(m.group(1)) if m else None
+            except (OSError, ValueError):
+                pass
+            samples.append(rec)
+            time.sleep(0.02)
+
+    def ask_smi():
+        time.sleep(min(1.0, seconds / 2))
+        try:
+            r = subprocess.run(["amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True, timeout=20)
+            d = json.loads(r.stdout)
+            g = (d["gpu_data"] if isinstance(d, dict) else d)[0]
+            smi["socket_power_w"] = g["power"]["socket_power"]["value"]
+            smi["xcd_clk_mhz"] = [g["clock"][k]["clk"]["value"] for k in sorted(g["clock"]) if k.startswith("gfx_")]
+        except Exception as e:  # noqa: BLE001  (no tool, another format: the fields stay absent)
+            smi["error"] = repr(e)[:120]
+
+    threads = [threading.Thread(target=sampler), threading.Thread(target=ask_smi)]
+    for t in threads:
+        t.start()
+    n = 0
+    timer = lt.Timer()
+    timer.start()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(200):
+            fn()
+        lt.sync()
+        n += 200
+    kernel_us = timer.stop_ms() / n * 1e3
+    stop.set()
+    for t in threads:
+        t.join()
+
+    def median_late(idx):
+        v = sorted(r[idx] for r in samples if r[idx] is not None and r[0] >= seconds / 2)
+        return v[len(v) // 2] if v else None
+    cap = None
+    try:
+        cap = int(open(cap_f).read()) / 1e6 if cap_f else None
+    except (OSError, ValueError):
+        pass
+    p = median_late(1)
+    return {"power_w": None if p is None else round(p), "power_cap_w": None if cap is None else round(cap),
+            "sclk_mhz": median_late(2), "sclk_max_mhz": 2400, "xcd_clk_mhz": smi.get("xcd_clk_mhz"),
+            "socket_power_w_amd_smi": smi.get("socket_power_w"), "kernel_us_during": round(kernel_us, 2),
+            "seconds": seconds, "launches": n}
+
+
 def timed(lt, fn, iters, warmup=3):
     """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on the library's stream), in the
     steady state: after an idle spell the part needs tens of milliseconds of load before its clocks settle (the first
@@ -466,6 +541,7 @@ def main():
     ap.add_argument("--no-verify", action="store_true", help="skip the post-run output check")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-config records for configs 1, 2, 4, 5")
     ap.add_argument("--no-vendor", action="store_true", help="skip the torch._int_mm (hipBLASLt) calibration leg")
+    ap.add_argument("--no-telemetry", action="store_true", help="skip the two-second power / clock reading")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="run only the plain copy kernel on buffers of this size (what FETCH_SIZE / WRITE_SIZE "
                          "counters are scaled against) and exit")
@@ -482,12 +558,12 @@ def main():
         src, dst = lt.DeviceBuffer(nbytes), lt.DeviceBuffer(nbytes)
         lt.check(lt.lib().lten_hip_zero(src.ptr, nbytes))
         for _ in range(max(args.warmup, 1)):
-            lt.check(lt.lib().lten_hip_copy_kernel(src.ptr, dst.ptr, nbytes))
+            lt.measure_copy(src, dst, nbytes)
         lt.sync()
         timer = lt.Timer()
         timer.start()
         for _ in range(args.steps):
-            lt.check(lt.lib().lten_hip_copy_kernel(src.ptr, dst.ptr, nbytes))
+            lt.measure_copy(src, dst, nbytes)
         ms = timer.stop_ms() / args.steps
         print(json.dumps({"copy_bytes_read": nbytes, "copy_bytes_written": nbytes, "us": round(ms * 1e3, 2),
                           "GB_per_s": round(2 * nbytes / ms / 1e6, 1)}))
@@ -530,6 +606,8 @@ def main():
     ops = 2.0 * M * N * K
     raw_ms = sustained(step_raw)
     raw_kernel = lt.last_kernel()
+    # what the part draws and clocks at while it runs the headline kernel (two seconds of it)
+    tele = None if args.no_telemetry else telemetry(lt, step)
 
     # The same product with zero points that need the correction terms: a post-relu activation tensor (zero point 0)
     # against symmetric weights, and a general triple.  On prepared weights both stay one launch.
@@ -620,6 +698,12 @@ def main():
         data_peaks[wps] = lt.measure_mfma_peak(2, wps)
         data_mhz[wps] = lt.measure_last_clocks()[1]
     measured_peak_data = max(data_peaks.values())
+    # and on operands taken from this very product's matrices (uniform bytes against N(0,40) bytes): its own ceiling
+    own_peaks, own_mhz = {}, {}
+    for wps in (1, 2, 4):
+        own_peaks[wps] = lt.measure_mfma_peak_operands(dA, dBp, M * K, wps)
+        own_mhz[wps] = lt.measure_last_clocks()[1]
+    measured_peak_own = max(own_peaks.values())
     vendor = None if args.no_vendor else vendor_int8()
 
     out = {
@@ -630,13 +714,16 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5),
+        "value_raw_uint8_weights": round(ops / (raw_ms * 1e-3) / 1e12, 2),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "cfg3 int8 FullyConnected_q forward M=N=K=4096: uint8 activations (zero point 128) x "
-                               "8-bit weights (N(0,40) clipped, zero point 128) -> int32 -> fused requantize to uint8",
+                               "8-bit weights (N(0,40) clipped, zero point 128) -> int32 -> fused requantize to uint8; the layer's "
+                               "weights were converted to int8 once outside the timed region (lten_hip_fcq_prepare_weights), "
+                               "value_raw_uint8_weights is the same product on l-ten's uint8 weight bytes",
                    "M": M, "N": N, "K": K, "input_digest": wl.digest(X, W)},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s",
                      "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic_bytes(kernel),
@@ -648,6 +735,12 @@ def main():
                      "measured_mfma_only_data_operands_tops": {str(k): round(v, 1) for k, v in data_peaks.items()},
                      "measured_mfma_only_data_operands_shader_mhz": {str(k): round(v) for k, v in data_mhz.items()},
                      "frac_of_measured_mfma_only_data_operands": round(achieved / measured_peak_data, 4),
+                     "measured_mfma_only_cfg3_operands_tops": {str(k): round(v, 1) for k, v in own_peaks.items()},
+                     "measured_mfma_only_cfg3_operands_shader_mhz": {str(k): round(v) for k, v in own_mhz.items()},
+                     "frac_of_measured_mfma_only_cfg3_operands": round(achieved / measured_peak_own, 4),
+                     "frac_driver_timed": round(value / INT8_MFMA_PEAK_TOPS, 4),
+                     "power_w": tele and tele["power_w"], "power_cap_w": tele and tele["power_cap_w"],
+                     "sclk_mhz": tele and tele["sclk_mhz"], "telemetry": tele,
                      "vendor_int8_gemm_same_shape": vendor,
                      "same_shape_other_zero_points": general_zp,
                      "note": "int8 multiply-add counted as 2 ops; achieved = 2*4096^3 / sustained_kernel_us (300 back-to-back "
@@ -655,7 +748,11 @@ def main():
                              "timed_region_kernel_us = the same over the --steps launches; measured_mfma_only = a kernel that "
                              "issues nothing but 32x32x32 int8 MFMAs on constant operands; _data_operands = the same with "
                              "pseudo-random operands that change with every MFMA, per wavefronts per SIMD (the part lowers its "
-                             "clock under that load although nothing but the matrix pipes is busy); vendor_int8_gemm_same_shape = "
+                             "clock under that load although nothing but the matrix pipes is busy); _cfg3_operands = the same loop on "
+                             "operands loaded from this product's own activation and weight matrices; frac = achieved / peak on the "
+                             "sustained figure, frac_driver_timed = value / peak on the --steps launches (wall clock); power_w / "
+                             "power_cap_w / sclk_mhz = socket power, its cap and the shader clock during two seconds of the headline "
+                             "kernel (amdgpu hwmon and pp_dpm_sclk; per-XCD clocks from amd-smi under telemetry); vendor_int8_gemm_same_shape = "
                              "torch._int_mm (hipBLASLt) at 4096^3 in a process of its own, a calibration only"},
         "verified_bit_exact": verified,
         "with_pcie_copies": {"ms_per_step": round(copies_ms, 3), "tops": round(ops / (copies_ms * 1e-3) / 1e12, 2),

@@ -335,14 +335,6 @@ int lten_hip_event_record(void* event);
 int lten_hip_event_elapsed_ms(void* start, void* stop, float* ms); /* synchronises on `stop` */
 int lten_hip_event_destroy(void* event);
 
-/* Calibration for roofline figures (no counterpart in l-ten): the MFMA issue rate sustained by a kernel
- * that does nothing else (kind 0: int8 32x32x32 in tera-ops/s, kind 1: fp32 32x32x2 in TFLOP/s, kinds 2 and 3:
- * the same two on pseudo-random operands that change with every MFMA, as a GEMM's do; 1..8 wavefronts per
- * SIMD), and a plain 16-byte-per-lane copy kernel whose HBM traffic is 2 * bytes. */
-int lten_hip_measure_mfma_peak(int kind, int waves_per_simd, float* tera_per_s);
-int lten_hip_measure_last_clocks(double* cycles_per_mfma, double* shader_mhz);
-int lten_hip_copy_kernel(const void* device_src, void* device_dst, uint64_t bytes);
-
 /* Kernel-selection override for tests and tuning sweeps; 0 restores the built-in heuristic.
  * Options: "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant", "qgemm_split".  No counterpart in l-ten. */
 int lten_hip_set_option(const char* name, int value);

@@ -99,10 +99,37 @@ _SIGNATURES = {
     "lten_hip_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "lten_hip_event_destroy": (C.c_int, [vp]),
     "lten_hip_set_option": (C.c_int, [C.c_char_p, C.c_int]),
-    "lten_hip_measure_mfma_peak": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_float)]),
-    "lten_hip_measure_last_clocks": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_double)]),
-    "lten_hip_copy_kernel": (C.c_int, [vp, vp, u64]),
 }
+
+# The calibration library (include/lten_hip_measure.h): not part of the drop-in surface, loaded on first use.
+MEASURE_LIB_PATH = os.path.join(HERE, "liblten_hip_measure.so")
+MEASURE_HEADER_PATH = os.path.join(os.path.dirname(HERE), "include", "lten_hip_measure.h")
+_MEASURE_SIGNATURES = {
+    "lten_measure_last_error": (C.c_char_p, []),
+    "lten_measure_mfma_peak": (C.c_int, [C.c_int, C.c_int, C.POINTER(C.c_float)]),
+    "lten_measure_mfma_peak_operands": (C.c_int, [vp, vp, u64, C.c_int, C.POINTER(C.c_float)]),
+    "lten_measure_last_clocks": (C.c_int, [C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "lten_measure_copy": (C.c_int, [vp, vp, u64]),
+}
+_measure_lib = None
+
+
+def measure_lib():
+    global _measure_lib
+    if _measure_lib is None:
+        if not os.path.exists(MEASURE_LIB_PATH):
+            raise LtenHipError(f"{MEASURE_LIB_PATH} is missing: build it with `python light-tensor_amd/build.py`")
+        m = C.CDLL(MEASURE_LIB_PATH)
+        for name, (res, args) in _MEASURE_SIGNATURES.items():
+            fn = getattr(m, name)
+            fn.restype, fn.argtypes = res, args
+        _measure_lib = m
+    return _measure_lib
+
+
+def _mcheck(rc):
+    if rc != 0:
+        raise LtenHipError(measure_lib().lten_measure_last_error().decode())
 
 _lib = None
 
@@ -155,14 +182,25 @@ def set_option(name, value):
 
 def measure_mfma_peak(kind=0, waves_per_simd=1):
     out = C.c_float()
-    check(lib().lten_hip_measure_mfma_peak(kind, waves_per_simd, C.byref(out)))
+    _mcheck(measure_lib().lten_measure_mfma_peak(kind, waves_per_simd, C.byref(out)))
+    return out.value
+
+
+def measure_mfma_peak_operands(a_u8, b_i8, nbytes, waves_per_simd=1):
+    """int8 MFMA-only rate on operands drawn from two device buffers (uint8 activations, prepared int8 weights)."""
+    out = C.c_float()
+    _mcheck(measure_lib().lten_measure_mfma_peak_operands(a_u8.ptr, b_i8.ptr, nbytes, waves_per_simd, C.byref(out)))
     return out.value
 
 
 def measure_last_clocks():
     a, b = C.c_double(), C.c_double()
-    check(lib().lten_hip_measure_last_clocks(C.byref(a), C.byref(b)))
+    _mcheck(measure_lib().lten_measure_last_clocks(C.byref(a), C.byref(b)))
     return a.value, b.value
+
+
+def measure_copy(src, dst, nbytes):
+    _mcheck(measure_lib().lten_measure_copy(src.ptr, dst.ptr, nbytes))
 
 
 def qparams3(scales, zps):

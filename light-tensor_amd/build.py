@@ -1,4 +1,5 @@
-"""Compiles the HIP sources under csrc/ into liblten_hip.so (gfx950 only), in-tree.
+"""Compiles the HIP sources under csrc/ into liblten_hip.so (gfx950 only), in-tree, and the calibration kernels
+under measure/ into a library of their own, liblten_hip_measure.so (used by bench.py and the profile commands only).
 
 Usage: python light-tensor_amd/build.py [--verbose]
 """
@@ -10,6 +11,8 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "liblten_hip.so")
+MEASURE_SRC = os.path.join(HERE, "measure", "measure.hip")
+MEASURE_LIB = os.path.join(HERE, "liblten_hip_measure.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
@@ -52,6 +55,13 @@ def build(verbose=False, extra_flags=()):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
+    cmd = [hipcc] + HIPCC_FLAGS + [MEASURE_SRC, "-o", MEASURE_LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if r.returncode != 0:
+        print(r.stdout, file=sys.stderr)
+        raise RuntimeError("hipcc failed")
     return LIB
 
 

@@ -21,6 +21,19 @@ def test_every_declared_symbol_is_exported(lt):
     assert sorted(lt._SIGNATURES) == declared
 
 
+def test_calibration_library_is_separate(lt):
+    """The calibration kernels live in a library of their own: it exports what include/lten_hip_measure.h declares,
+    and the product library exports none of it."""
+    import re
+    text = re.sub(r"/\*.*?\*/", "", open(lt.MEASURE_HEADER_PATH).read(), flags=re.S)
+    declared = sorted(set(re.findall(r"\b(lten_measure_[a-z0-9_]+)\s*\(", text)))
+    assert declared == sorted(lt._MEASURE_SIGNATURES)
+    m, raw = C.CDLL(lt.MEASURE_LIB_PATH), C.CDLL(lt.LIB_PATH)
+    assert all(hasattr(m, s) for s in declared)
+    assert not any(hasattr(raw, s) for s in declared)
+    assert not any("measure" in s or "copy_kernel" in s for s in lt.declared_symbols())
+
+
 def test_qparams_layout_matches_lten(lt):
     # l-ten/math_fns.h:12-16: float scale; uint8_t zero_point -> 8 bytes, zero_point at offset 4
     assert C.sizeof(lt.QParams) == 8 and lt.QParams.zero_point.offset == 4
