@@ -39,8 +39,9 @@ int lten_hip_init(int device);
 const char* lten_hip_last_error(void);
 /* Replaces GetDevice (l-ten/utils.h:41, l-ten/utils.cu:110-116). */
 int lten_hip_get_device(int* device);
-/* Routes all later work to `hip_stream` (a hipStream_t; NULL = the null stream).
- * No counterpart in l-ten, which only ever uses the default stream. */
+/* Routes all later work to `hip_stream` (a hipStream_t; NULL = the null stream), after waiting for the work
+ * already issued on the stream it leaves (blocks that lten_hip_free returned to the pool while that work was pending
+ * may be handed out again at once).  No counterpart in l-ten, which only ever uses the default stream. */
 int lten_hip_set_stream(void* hip_stream);
 /* Blocks until the stream is idle. l-ten's equivalent is the implicit sync of cudaMemcpy. */
 int lten_hip_sync(void);
@@ -50,11 +51,15 @@ int lten_hip_sync(void);
 /* Replaces AllocateMemoryOnGPU / gpu_alloc (l-ten/utils.h:29,33; l-ten/utils.cu:8-28,30-58), memory pool included
  * (l-ten's default build serves GPU buffers from its power-of-two MemoryPool, l-ten/utils.cu:33-37,
  * l-ten/memorypool.h:142-173): sizes are rounded up to a power of two (to a multiple of 64 MB above 64 MB), freed
- * blocks are kept and handed out again without a wait — correct for work issued in order on the library's stream.  Up
- * to 64 GB stay cached; they go back to the driver when an allocation would otherwise fail. */
+ * blocks are kept and handed out again without a wait — correct for work issued in order on the library's stream
+ * (a caller that uses a block on a stream of its own must finish that work before it frees the block).  Up to 16 GB
+ * stay cached; they go back to the driver when an allocation would otherwise fail or lten_hip_pool_release is called. */
 int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory);
 /* Replaces FreeMemoryOnGPU / gpu_free (l-ten/utils.h:30,35; l-ten/utils.cu:60-71).  Freeing a block twice fails. */
 int lten_hip_free(void* device_ptr);
+/* Gives every cached block back to the driver (l-ten's MemoryPool frees its blocks only in its destructor,
+ * l-ten/memorypool.h; a library has no such moment).  Blocks in use are not touched. */
+int lten_hip_pool_release(void);
 /* Replaces ZeroMemoryOnGPU (l-ten/utils.h:34; l-ten/utils.cu:49-52). */
 int lten_hip_zero(void* device_ptr, size_t size);
 /* Replace CopyDataToGPU / CopyDataFromGPU / GPUToGPUCopy (l-ten/utils.h:36-38; l-ten/utils.cu:73-108).
@@ -319,7 +324,9 @@ int lten_hip_get_min_max(const float* data, uint64_t len, float* min_val, float*
  * set_stream / get_min_max / event_elapsed_ms fail with a message (they allocate, copy or wait, which a recording
  * cannot hold), and lten_hip_last_kernel names
  * what was recorded, not what ran.  When the library is on the null stream the recording uses a stream of
- * the library's own; replays still go to the library's stream.  One capture at a time per process.
+ * the library's own; replays still go to the library's stream.  One capture at a time per process.  A buffer a
+ * recording names must not be handed to lten_hip_free while the handle lives (the pool would give it to the next
+ * lten_hip_alloc); lten_hip_graph_destroy waits for the stream before it lets go of the recording.
  * No counterpart in l-ten, whose GPU branches launch eagerly on the default stream. */
 int lten_hip_graph_begin(void);
 int lten_hip_graph_end(void** graph);

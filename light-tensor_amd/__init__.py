@@ -35,6 +35,7 @@ _SIGNATURES = {
     "lten_hip_set_stream": (C.c_int, [vp]),
     "lten_hip_sync": (C.c_int, []),
     "lten_hip_alloc": (C.c_int, [C.POINTER(vp), u64, C.c_int]),
+    "lten_hip_pool_release": (C.c_int, []),
     "lten_hip_free": (C.c_int, [vp]),
     "lten_hip_zero": (C.c_int, [vp, C.c_size_t]),
     "lten_hip_copy_to_gpu": (C.c_int, [vp, vp, C.c_size_t]),

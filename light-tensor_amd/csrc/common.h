@@ -22,6 +22,9 @@ bool capturing();  // a launch graph is being recorded: no allocation, no synchr
 enum Option { OPT_QGEMM_TILE = 0, OPT_SGEMM_TILE, OPT_QSKINNY, OPT_CONV_VARIANT, OPT_QGEMM_SPLIT, OPT_COUNT };
 int get_option(Option o);
 
+// Looks up the current device's copy of the static scratch of lten_hip_fcq_forward_static (qgemm.hip); 0 on success.
+int prepare_static_scratch();
+
 inline uint64_t ceil_div(uint64_t a, uint64_t b) { return (a + b - 1) / b; }
 
 }  // namespace lten_hip

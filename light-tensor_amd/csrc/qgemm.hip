@@ -566,6 +566,14 @@ static int static_scratch(RunScratch* rs)
 	return 0;
 }
 
+// Called by lten_hip_init for the device it selects, so that the first lten_hip_fcq_forward_static on it (which may
+// sit inside a recording) finds the address in place; the entry point still looks it up itself where init was skipped.
+int prepare_static_scratch()
+{
+	RunScratch rs;
+	return static_scratch(&rs);
+}
+
 }  // namespace lten_hip
 
 using namespace lten_hip;

@@ -20,6 +20,10 @@ static int g_device = -1;
 static hipStream_t g_capture_stream = nullptr;
 static hipStream_t g_stream_before_capture = nullptr;
 static bool g_capturing = false;
+struct RecordedGraph {  // what a handle of lten_hip_graph_end points to
+	hipGraph_t graph;
+	hipGraphExec_t exec;
+};
 
 void set_error(const char* fmt, ...)
 {
@@ -46,9 +50,11 @@ int get_option(Option o) { return g_options[o]; }
 // (l-ten/utils.cu:30-47 with USE_MEMORYPOOL, l-ten/memorypool.h:142-173): sizes are rounded up to a power of two (to a
 // multiple of 64 MB above that), freed blocks are kept per size and handed out again, so that a layer's forward pass,
 // which allocates its result tensor on every call, does not pay a hipMalloc each time.  Blocks are reused without any
-// wait: safe for work issued in order on the library's stream, which is the only order this library creates.  At most
-// POOL_CACHE_LIMIT bytes stay cached; beyond that a freed block goes back to the driver.
-constexpr uint64_t POOL_CACHE_LIMIT = 64ull << 30;
+// wait: safe for work issued in order on the library's stream, which is the only order this library creates, and
+// lten_hip_set_stream waits for the stream it leaves, so that a block freed while work was pending there cannot be
+// handed to work on the next stream before that work is done.  At most POOL_CACHE_LIMIT bytes stay cached; beyond
+// that a freed block goes back to the driver, and lten_hip_pool_release returns everything cached.
+constexpr uint64_t POOL_CACHE_LIMIT = 16ull << 30;
 static std::mutex g_pool_mutex;
 static std::map<uint64_t, std::vector<void*>> g_pool_free;  // rounded size -> cached blocks
 static std::unordered_map<void*, uint64_t> g_pool_size;     // every block handed out or cached -> its rounded size, bit 0 set while cached
@@ -61,6 +67,22 @@ static uint64_t pool_round(uint64_t size)
 	uint64_t r = 256;
 	while (r < size) r <<= 1;
 	return r;
+}
+
+// Everything the pool holds (cached or handed out) comes from hipMalloc; this gives the cached part back.
+static int pool_drop_cached()
+{
+	std::vector<void*> drop;
+	{
+		std::lock_guard<std::mutex> lock(g_pool_mutex);
+		for (auto& kv : g_pool_free) {
+			for (void* q : kv.second) { drop.push_back(q); g_pool_size.erase(q); }
+			kv.second.clear();
+		}
+		g_pool_cached = 0;
+	}
+	for (void* q : drop) (void)hipFree(q);  // hipFree waits for the device: no pending work loses its memory
+	return 0;
 }
 
 template <typename T>
@@ -100,7 +122,7 @@ int lten_hip_init(int device)
 	LTEN_HIP_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
 	                 "lten_hip_init: device %d is %s; this library is built for gfx950 only", device, prop.gcnArchName);
 	g_device = device;
-	return 0;
+	return prepare_static_scratch();
 }
 
 const char* lten_hip_last_error(void) { return g_error; }
@@ -121,7 +143,13 @@ int lten_hip_get_device(int* device)
 int lten_hip_set_stream(void* hip_stream)
 {
 	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_set_stream");
-	g_stream = static_cast<hipStream_t>(hip_stream);
+	hipStream_t next = static_cast<hipStream_t>(hip_stream);
+	if (next == g_stream) return 0;
+	// Work still pending on the stream being left may use blocks that lten_hip_free has put back into the pool; the
+	// next lten_hip_alloc could hand them to work on the new stream, which is not ordered behind it.  Waiting here
+	// once keeps the pool free of per-block events.
+	LTEN_HIP_CHECK(hipStreamSynchronize(g_stream));
+	g_stream = next;
 	return 0;
 }
 
@@ -153,16 +181,7 @@ int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
 		if (e != hipSuccess) {
 			// out of memory with blocks cached: give them back and try once more
 			(void)hipGetLastError();
-			std::vector<void*> drop;
-			{
-				std::lock_guard<std::mutex> lock(g_pool_mutex);
-				for (auto& kv : g_pool_free) {
-					for (void* q : kv.second) { drop.push_back(q); g_pool_size.erase(q); }
-					kv.second.clear();
-				}
-				g_pool_cached = 0;
-			}
-			for (void* q : drop) (void)hipFree(q);
+			pool_drop_cached();
 			LTEN_HIP_CHECK(hipMalloc(device_ptr, rounded));
 		}
 		std::lock_guard<std::mutex> lock(g_pool_mutex);
@@ -170,6 +189,12 @@ int lten_hip_alloc(void** device_ptr, uint64_t size, int zero_memory)
 	}
 	if (zero_memory && size) return lten_hip_zero(*device_ptr, size);  // a fill kernel, stream ordered
 	return 0;
+}
+
+int lten_hip_pool_release(void)
+{
+	LTEN_HIP_NOT_WHILE_RECORDING("lten_hip_pool_release");
+	return pool_drop_cached();
 }
 
 int lten_hip_free(void* device_ptr)
@@ -281,12 +306,14 @@ int lten_hip_graph_end(void** graph)
 	}
 	hipGraphExec_t exec = nullptr;
 	const hipError_t ei = hipGraphInstantiate(&exec, captured, nullptr, nullptr, 0);
-	(void)hipGraphDestroy(captured);
 	if (ei != hipSuccess) {
+		(void)hipGraphDestroy(captured);
 		set_error("lten_hip_graph_end: hipGraphInstantiate: %s", hipGetErrorString(ei));
 		return 1;
 	}
-	*graph = exec;
+	// The handle owns both objects until lten_hip_graph_destroy: the executable graph is specified to be independent
+	// of the graph it was instantiated from, but nothing is gained by destroying that one early.
+	*graph = new RecordedGraph{ captured, exec };
 	return 0;
 }
 
@@ -294,13 +321,20 @@ int lten_hip_graph_launch(void* graph)
 {
 	LTEN_HIP_REQUIRE(graph != nullptr, "lten_hip_graph_launch: null graph");
 	LTEN_HIP_REQUIRE(!g_capturing, "lten_hip_graph_launch: a capture is open");
-	LTEN_HIP_CHECK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), stream()));
+	LTEN_HIP_CHECK(hipGraphLaunch(static_cast<RecordedGraph*>(graph)->exec, stream()));
 	return 0;
 }
 
 int lten_hip_graph_destroy(void* graph)
 {
-	if (graph) LTEN_HIP_CHECK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+	if (graph == nullptr) return 0;
+	RecordedGraph* g = static_cast<RecordedGraph*>(graph);
+	// replays may still be running: the objects go only once the stream they were launched on is idle
+	LTEN_HIP_CHECK(hipStreamSynchronize(stream()));
+	const hipError_t e0 = hipGraphExecDestroy(g->exec), e1 = hipGraphDestroy(g->graph);
+	delete g;
+	LTEN_HIP_CHECK(e0);
+	LTEN_HIP_CHECK(e1);
 	return 0;
 }
 

@@ -51,6 +51,52 @@ def test_fill_zero_copy_and_get_device(gpu):
     assert l.lten_hip_free(p2) != 0 and b"freed already" in l.lten_hip_last_error()
 
 
+def test_pool_release_and_stream_change(gpu):
+    """lten_hip_pool_release gives the cached blocks back (free device memory grows by at least their size, a later
+    allocation of that size works and is usable); lten_hip_set_stream waits for the work pending on the stream it
+    leaves, so a block freed behind pending work there is safe to reuse on the next stream."""
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    hip = C.CDLL("libamdhip64.so")
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    size = 96 << 20                      # rounds to 128 MiB (a multiple of 64 MiB)
+    p = C.c_void_p()
+    gpu.check(l.lten_hip_alloc(C.byref(p), size, 0))
+    gpu.check(l.lten_hip_free(p))        # cached now
+    gpu.sync()
+    assert hip.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+    gpu.check(l.lten_hip_pool_release())
+    assert hip.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+    assert free1.value >= free0.value + (128 << 20), (free0.value, free1.value)
+    z = D(size, zero=True)               # a fresh block after the release
+    assert not z.numpy(np.uint8, (4096,)).any()
+    z.free()
+    # a long fill on a caller's stream, the block freed behind it, the stream changed: the fill must have finished
+    # by the time lten_hip_set_stream returns (the next user of the block may run on the other stream)
+    st = C.c_void_p()
+    assert hip.hipStreamCreate(C.byref(st)) == 0
+    try:
+        gpu.check(l.lten_hip_set_stream(st))
+        n = 64 << 20
+        q = C.c_void_p()
+        gpu.check(l.lten_hip_alloc(C.byref(q), 4 * n, 0))
+        for v in range(8):
+            gpu.check(l.lten_hip_fill_i32(q, n, v))
+        gpu.check(l.lten_hip_free(q))
+        gpu.check(l.lten_hip_set_stream(None))
+        assert hip.hipStreamQuery(st) == 0   # hipSuccess: nothing pending on the stream that was left
+        r = C.c_void_p()
+        gpu.check(l.lten_hip_alloc(C.byref(r), 4 * n, 0))
+        assert r.value == q.value            # the same block, now used on the null stream
+        gpu.check(l.lten_hip_fill_i32(r, n, -1))
+        out = np.empty(n, np.int32)
+        gpu.check(l.lten_hip_copy_from_gpu(out.ctypes.data, r, 4 * n))
+        assert (out == -1).all()
+        gpu.check(l.lten_hip_free(r))
+    finally:
+        gpu.check(l.lten_hip_set_stream(None))
+        hip.hipStreamDestroy(st)
+
+
 def test_calls_that_cannot_be_recorded_fail_with_a_message(gpu):
     """Between graph_begin and graph_end, allocation, freeing, copies, waits and the range search return an error
     that names the call; the recording survives and replays."""

@@ -23,6 +23,45 @@ def both(gpu, X, W, sc, zp, bias):
     return y_ref.numpy(np.uint8, (M, N)), y_new.numpy(np.uint8, (M, N)), k_ref, k_new
 
 
+def test_static_entry_point_inside_a_recording_and_without_allocation(gpu):
+    """The call recorded into a launch graph, where lten_hip_alloc is refused (first use of the entry point in this
+    process when the file runs alone): every replay, with eager work and waits between them, returns the eager
+    result; and a call leaves the device's free memory as it found it."""
+    import ctypes as C
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    rng = np.random.default_rng(7)
+    M, N, K = 256, 1024, 4096   # split-K: zero-point terms, partial sums and counters all in the static array
+    X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    sc, zp = [0.02, 0.013, 3.0], [3, 250, 77]
+    dX, dW, db, ws = D.from_numpy(X), D.from_numpy(W), D.from_numpy(bias), D(4 * (M + N))
+    y_ref, y_new = D(M * N, zero=True), D(M * N, zero=True)
+    qp = gpu.qparams3(sc, zp)
+    with gpu.Graph() as g:
+        p = C.c_void_p()
+        assert l.lten_hip_alloc(C.byref(p), 1024, 0) != 0        # a recording cannot allocate ...
+        gpu.check(l.lten_hip_fcq_forward_static(1, M, K, N, dX.ptr, dW.ptr, db.ptr, qp, y_new.ptr))   # ... this call need not
+    assert "splitk" in gpu.last_kernel()
+    gpu.check(l.lten_hip_fcq_forward(1, M, K, N, dX.ptr, dW.ptr, db.ptr, qp, y_ref.ptr, ws.ptr))
+    want = y_ref.numpy(np.uint8, (M, N))
+    for rep in range(3):
+        gpu.check(l.lten_hip_zero(y_new.ptr, M * N))
+        g.launch()
+        assert np.array_equal(y_new.numpy(np.uint8, (M, N)), want), rep
+        gpu.check(l.lten_hip_fcq_forward(1, M, K, N, dX.ptr, dW.ptr, db.ptr, qp, y_ref.ptr, ws.ptr))   # eager work between replays
+        gpu.sync()
+    hip = C.CDLL("libamdhip64.so")
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    gpu.sync()
+    assert hip.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+    gpu.check(l.lten_hip_fcq_forward_static(1, M, K, N, dX.ptr, dW.ptr, db.ptr, qp, y_new.ptr))
+    gpu.sync()
+    assert hip.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+    assert free1.value == free0.value
+    assert np.array_equal(y_new.numpy(np.uint8, (M, N)), want)
+
+
 def test_static_entry_point_matches_twice_in_a_row(gpu, ob):
     rng = np.random.default_rng(2024)
     sc, zp = [0.02, 0.013, 3.0], [3, 250, 77]
