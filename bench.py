@@ -529,6 +529,16 @@ def extra_configs(lt, wl, with_cpu):
                 "algorithmic_bytes": nbytes,
                 "roofline": {"bound": "hbm", "achieved": round(nbytes / ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                              "frac": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}})
+    # both products of the time step (x U and h W, l-ten/gru.cpp:358-361) as one strided batch of two: one launch
+    gxh = D.from_numpy(np.random.default_rng(15).standard_normal((2, hid)).astype(np.float32))
+    guw = D.from_numpy(np.random.default_rng(16).standard_normal((2, hid, 3 * hid)).astype(np.float32))
+    gy2 = D(4 * 2 * 3 * hid)
+    ms = timed(lt, lambda: lt.check(l.lten_hip_sgemm_strided_batched(0, 0, 1, 3 * hid, hid, 1.0, gxh.ptr, hid, hid, guw.ptr, 3 * hid, hid * 3 * hid,
+                                                                     0.0, gy2.ptr, 3 * hid, 3 * hid, 2)), 100)
+    out.append({"config": "GRU time step, both products (x U and h W, 1 x 1024 times 1024 x 3072 each) in one batched launch", "gpu_us": round(ms * 1e3, 2),
+                "kernel": lt.last_kernel(), "algorithmic_bytes": 2 * nbytes,
+                "roofline": {"bound": "hbm", "achieved": round(2 * nbytes / ms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                             "frac": round(2 * nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}})
     return out
 
 

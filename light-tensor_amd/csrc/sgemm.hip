@@ -869,13 +869,18 @@ __global__ __launch_bounds__(256) void sgemm_rank1_kernel(SProblem p, int tA, in
 // (column, slice) with eight loads in flight; the slices are combined in slice order.  A null A stands for a
 // vector of ones, so the bias_multiplier tensor of l-ten's FullyConnected is never needed on the device.
 // Two shapes: 64 columns x 4 slices when the columns alone give every CU a workgroup, else 16 x 64 (rows
-// are then read in 64-byte pieces, but four times as many workgroups share a long K).
+// are then read in 64-byte pieces, but four times as many workgroups share a long K).  blockIdx.z counts the problems
+// of a strided batch (the x U and h W products of one GRU time step, l-ten/gru.cpp:358-361, are a batch of two when
+// the input and hidden sizes agree): one launch for all of them.
 template <int COLS, int SLICES>
 __global__ __launch_bounds__(COLS* SLICES) void sgemm_rowvec_kernel(SProblem p, int tA)
 {
 	__shared__ float part[SLICES][COLS];
 	const int tx = threadIdx.x % COLS, ty = threadIdx.x / COLS;
 	const int n = blockIdx.x * COLS + tx;
+	if (p.A != nullptr) p.A += (int64_t)blockIdx.z * p.stride_a;
+	p.B += (int64_t)blockIdx.z * p.stride_b;
+	p.C += (int64_t)blockIdx.z * p.stride_c;
 	float s = 0.0f;
 	if (n < p.N) {
 		auto a_at = [&](int k) { return p.A == nullptr ? 1.0f : (tA ? p.A[(int64_t)k * p.lda] : p.A[k]); };
@@ -905,11 +910,13 @@ __global__ __launch_bounds__(COLS* SLICES) void sgemm_rowvec_kernel(SProblem p, 
 	}
 }
 
-static void launch_rowvec(const SProblem& p, int tA)
+static void launch_rowvec(const SProblem& p, int tA, uint64_t batch)
 {
-	set_kernel_name("sgemm_rowvec");
-	if (ceil_div(p.N, 64) >= 256 || p.K < 128) sgemm_rowvec_kernel<64, 4><<<dim3((unsigned)ceil_div(p.N, 64)), dim3(256), 0, stream()>>>(p, tA);
-	else sgemm_rowvec_kernel<16, 64><<<dim3((unsigned)ceil_div(p.N, 16)), dim3(1024), 0, stream()>>>(p, tA);
+	set_kernel_name(batch > 1 ? "sgemm_rowvec_batched" : "sgemm_rowvec");
+	if (ceil_div(p.N, 64) * batch >= 256 || p.K < 128)
+		sgemm_rowvec_kernel<64, 4><<<dim3((unsigned)ceil_div(p.N, 64), 1, (unsigned)batch), dim3(256), 0, stream()>>>(p, tA);
+	else
+		sgemm_rowvec_kernel<16, 64><<<dim3((unsigned)ceil_div(p.N, 16), 1, (unsigned)batch), dim3(1024), 0, stream()>>>(p, tA);
 }
 
 template <int BM, int BN, int BK, int WM, int WN>
@@ -963,8 +970,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}
-	if (force == 0 && batch == 1 && bias == nullptr && M == 1 && !tB) {
-		launch_rowvec(p, tA);
+	if (force == 0 && bias == nullptr && M == 1 && !tB) {
+		launch_rowvec(p, tA, batch);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}
@@ -1153,7 +1160,7 @@ static int fc_backward(uint64_t M, uint64_t in, uint64_t out, const float* X, co
 		p.ldb = (int64_t)out; p.ldc = (int64_t)out;
 		p.M = 1; p.N = (int)out; p.K = (int)M;
 		p.alpha = 1.0f; p.beta = 1.0f;
-		launch_rowvec(p, 0);
+		launch_rowvec(p, 0, 1);
 		LTEN_HIP_LAUNCH_CHECK();
 	}
 	return rc;

@@ -171,6 +171,34 @@ def test_gru_step_products(gpu, ob):
     assert np.array_equal(got, x @ u)
 
 
+def test_gru_step_both_products_in_one_launch(gpu, ob):
+    """x U and h W of one GRU time step (l-ten/gru.cpp:358-361) as one strided batch of two M = 1 products: one launch
+    of the row-vector kernel; each product equal to the single call (same kernel, same order) and to the oracle.
+    The two operand pairs sit in separate allocations: the strides are the distances between them."""
+    rng = np.random.default_rng(22)
+    H = 1024
+    K, N = H, 3 * H
+    D = gpu.DeviceBuffer
+    xh = rng.standard_normal((2, K)).astype(np.float32)                  # x_t and h_{t-1}
+    uw = (rng.standard_normal((2, K, N)) * 0.05).astype(np.float32)      # weights_u and weights_w
+    dX, dU, dOut = D.from_numpy(xh), D.from_numpy(uw), D(2 * N * 4, zero=True)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(0, 0, 1, N, K, 1.0, dX.ptr, K, K, dU.ptr, N, K * N, 0.0, dOut.ptr, N, N, 2))
+    assert gpu.last_kernel() == "sgemm_rowvec_batched", gpu.last_kernel()
+    got = dOut.numpy(np.float32, (2, N))
+    for i in range(2):
+        want = np.zeros((1, N), np.float32)
+        ob.sgemm(0, 0, 1, N, K, 1.0, xh[i:i + 1], K, uw[i], N, 0.0, want, N)
+        assert rel_err(got[i:i + 1], want) < TOL, i
+        single = gpu_sgemm(gpu, 0, 0, 1, N, K, 1.0, xh[i:i + 1], K, uw[i], N, 0.0, np.zeros((1, N), np.float32), N)
+        assert np.array_equal(got[i:i + 1], single), i
+    # beta = 1 accumulates per product, a broadcast input row (stride 0) is allowed
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(0, 0, 1, N, K, 2.0, dX.ptr, K, 0, dU.ptr, N, K * N, 1.0, dOut.ptr, N, N, 2))
+    again = dOut.numpy(np.float32, (2, N))
+    for i in range(2):
+        want = got[i].astype(np.float64) + 2.0 * (xh[0].astype(np.float64) @ uw[i].astype(np.float64))
+        assert rel_err(again[i], want) < TOL, i
+
+
 def test_strided_batched_and_broadcast(gpu, ob):
     g = np.load(golden_path("layer_cases.npz"))
     # case 0: a{2,1,4,8} x b{1,1,8,15}: b broadcast over the leading index (stride 0)
