@@ -770,8 +770,15 @@ __global__ __launch_bounds__(512) void sgemm_fc_backward_pair_wide_kernel(SProbl
 	static_assert(8 * SLAB >= 4 * 16 * 64 + 4 * 32, "the exchange of the halves fits the slabs");
 	__shared__ __attribute__((aligned(16))) float lds[FLOATS];
 	if ((int)blockIdx.x >= blocks_w) {
+		// Consecutive workgroups go round-robin to the eight XCDs, each with an L2 of its own.  XCD x takes a contiguous
+		// run of the (column block, row block) pairs in column-major order, i.e. a range of column blocks with all their
+		// row blocks: a column block reads 64-byte pieces of the weight rows, so neighbours share every cache line, and
+		// with neighbours on different XCDs each line crossed the L2 boundary twice.
 		const int b = (int)blockIdx.x - blocks_w;
-		sgemm_skinny_body<2, false>(px, b % cols_x, b / cols_x, lds);
+		const int rows_x = (px.M + 31) / 32, total = cols_x * rows_x;
+		const int x = b & 7, q = total >> 3, r = total & 7;
+		const int idx = x * q + min(x, r) + (b >> 3);
+		sgemm_skinny_body<2, false>(px, idx / rows_x, idx % rows_x, lds);
 		return;
 	}
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, lrow = lane & 31, g = lane >> 5;
