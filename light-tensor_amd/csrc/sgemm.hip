@@ -884,14 +884,19 @@ __global__ __launch_bounds__(COLS* SLICES) void sgemm_rowvec_kernel(SProblem p, 
 {
 	__shared__ float part[SLICES][COLS];
 	const int tx = threadIdx.x % COLS, ty = threadIdx.x / COLS;
-	const int n = blockIdx.x * COLS + tx;
-	if (p.A != nullptr) p.A += (int64_t)blockIdx.z * p.stride_a;
-	p.B += (int64_t)blockIdx.z * p.stride_b;
-	p.C += (int64_t)blockIdx.z * p.stride_c;
+	// Consecutive workgroups go round-robin to the eight XCDs; XCD x takes a contiguous run of column blocks, so that
+	// neighbours, which share the cache lines of every row of B (a block reads 64-byte pieces), meet in one L2: with
+	// neighbours on different XCDs the matrix occupies the L2s twice and a step's two weight matrices no longer fit.
+	const int nblk = gridDim.x, bx = blockIdx.x & 7, bq = nblk >> 3, br = nblk & 7;
+	const int blk = bx * bq + min(bx, br) + ((int)blockIdx.x >> 3);
+	const int n = blk * COLS + tx;
+	const float* const A = p.A == nullptr ? nullptr : p.A + (int64_t)blockIdx.z * p.stride_a;
+	const float* const B = p.B + (int64_t)blockIdx.z * p.stride_b;
+	float* const C = p.C + (int64_t)blockIdx.z * p.stride_c;
 	float s = 0.0f;
 	if (n < p.N) {
-		auto a_at = [&](int k) { return p.A == nullptr ? 1.0f : (tA ? p.A[(int64_t)k * p.lda] : p.A[k]); };
-		const float* bcol = p.B + n;
+		auto a_at = [&](int k) { return A == nullptr ? 1.0f : (tA ? A[(int64_t)k * p.lda] : A[k]); };
+		const float* bcol = B + n;
 		int k = ty;
 		for (; k + 7 * SLICES < p.K; k += 8 * SLICES) {
 			float bv[8], av[8];
@@ -912,8 +917,8 @@ __global__ __launch_bounds__(COLS* SLICES) void sgemm_rowvec_kernel(SProblem p, 
 #pragma unroll
 		for (int q = 1; q < SLICES; q++) v += part[q][tx];
 		v *= p.alpha;
-		if (p.beta != 0.0f) v += p.beta * p.C[n];
-		p.C[n] = v;
+		if (p.beta != 0.0f) v += p.beta * C[n];
+		C[n] = v;
 	}
 }
 
