@@ -112,6 +112,10 @@ def telemetry(lt, fn, seconds=2.0):
             time.sleep(0.02)
 
     def ask_smi():
+        # not under a profiler: its preloaded tool library would come up inside the child as well
+        if "ROCP_TOOL_LIBRARIES" in os.environ or "rocprofiler" in os.environ.get("LD_PRELOAD", ""):
+            smi["error"] = "skipped under a profiler"
+            return
         time.sleep(min(1.0, seconds / 2))
         try:
             r = subprocess.run(["amd-smi", "metric", "-p", "-c", "--json"], capture_output=True, text=True, timeout=20)

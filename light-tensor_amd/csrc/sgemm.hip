@@ -708,7 +708,11 @@ template <int MB>
 __global__ __launch_bounds__(512) void sgemm_skinny_nn_kernel(SProblem p)
 {
 	__shared__ __attribute__((aligned(16))) float lds[SkinnyShape<MB, false>::LDS_FLOATS];
-	sgemm_skinny_body<MB, false>(p, blockIdx.x, blockIdx.y, lds);
+	// XCD x (consecutive workgroups go round-robin to the eight of them) takes a contiguous run of column blocks: a block
+	// reads 64-byte pieces of B's rows, and neighbours that share those cache lines should share an L2 as well
+	const int nblk = gridDim.x, bx = blockIdx.x & 7;
+	const int blk = bx * (nblk >> 3) + min(bx, nblk & 7) + ((int)blockIdx.x >> 3);
+	sgemm_skinny_body<MB, false>(p, blk, blockIdx.y, lds);
 }
 
 // sgemm_tn_wave_tile_lines over k in [k_begin, k_end) only, the sums left in `acc` and `asum` (this lane's share of the
