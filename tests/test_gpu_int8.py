@@ -479,7 +479,7 @@ def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
     multiple of 4 or not, K a multiple of 16 / 128 or not, short and long K), each with random zero points, with and
     without bias, u8 and int32 outputs against the oracle; the kernel names show that every family took part."""
     rng = np.random.default_rng(20240607)
-    seen = set()
+    seen, seen_prepared = set(), set()
     Ms = [1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 100, 127, 128, 129, 200, 255, 257, 300]
     Ns = [1, 10, 16, 36, 100, 128, 130, 132, 256, 500, 512, 1000, 1024, 2048, 2052]
     Ks = [1, 7, 16, 48, 100, 128, 144, 512, 528, 784, 1000, 1024, 2048, 2064, 4096]
@@ -496,9 +496,14 @@ def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
         zp = np.array([rng.choice([0, 128, int(rng.integers(0, 256))]) for _ in range(3)], np.uint8)
         sc = [0.02, 0.013, float(rng.choice([0.9, 0.05, 7.0]))]
         bias = rng.integers(-20000, 20000, N).astype(np.int32) if rng.integers(0, 2) else None
-        run_case(gpu, ob, A, B, sc, zp, bias=bias)
+        Cg = run_case(gpu, ob, A, B, sc, zp, bias=bias)
         seen.add(gpu.last_kernel().split("_")[0] + "_" + gpu.last_kernel().split("_")[1])
+        # the same layer on prepared weights with their kept sums: the same bytes, whatever kernel the shape selects
+        Cp, kp = fcq(gpu, gpu.lib().lten_hip_fcq_forward_prepared, A, B, sc, zp, bias, prepared=True)
+        assert np.array_equal(Cp, Cg), (M, N, K, zp, kp)
+        seen_prepared.add(kp.split("_")[0] + "_" + kp.split("_")[1] + ("+zp" if "+zp" in kp else ""))
     assert {"qskinny_mfma", "qdirect_16x16", "qgemm_fast", "qgemm_guard"} <= seen, seen
+    assert {"qgemm_fast+zp", "qgemm_guard"} <= seen_prepared, seen_prepared
 
 
 def fcq(gpu, entry, X, W, sc, zp, bias=None, prepared=False):
