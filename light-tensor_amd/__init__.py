@@ -267,6 +267,13 @@ class Timer:
 
     def stop_ms(self):
         check(lib().lten_hip_event_record(self.e1))
+        return self.elapsed_ms()
+
+    def record_stop(self):
+        check(lib().lten_hip_event_record(self.e1))
+
+    def elapsed_ms(self):
+        """Milliseconds between the two recorded events (waits for the second one)."""
         ms = C.c_float()
         check(lib().lten_hip_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
         return ms.value
