@@ -9,7 +9,8 @@
 // launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
-// Longer windows run as three launches for the whole batch (the first also pads the weights): the patches of all output positions as rows of a
+// Longer windows on small images (at most 32 KB an image, at most 64 output channels, at most 1024 taps) also run in
+// one launch: convq_image.hip.  Other longer windows run as three launches for the whole batch (the first also pads the weights): the patches of all output positions as rows of a
 // [N * Ho * Wo][K] matrix (K padded to a multiple of 16 with the input zero point, the weights padded alike with
 // theirs, so the padding multiplies to nothing), one int8 GEMM of qgemm.hip with the positions as rows (NT: both
 // operands contiguous in K, the shape its MFMA tiles are built for) into int32 sums, and a pass that adds l-ten's
@@ -22,6 +23,10 @@
 namespace lten_hip {
 
 constexpr int CQ_MAXK = 64, CQ_CO = 64;
+
+// one launch for small images with windows above 64 taps (convq_image.hip); -1 = not a shape for it
+int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
+                           float zp_out, void* y, bool out_acc);
 
 // ND = dwords of packed taps a thread holds (4 taps each): 4, 8, 12 or 16, the smallest that covers K.
 template <int OUT, int ND>
@@ -263,6 +268,13 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		else launch_conv2dq_direct<Q_OUT_U8_EXACT>(grid, (int)K, g, x, w, bias, zp_in, zp_w, mult, zp_out, y);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
+	}
+
+	// small images with a longer window (l-ten's quantized MNIST conv2): still one launch, no workspace (convq_image.hip;
+	// option "conv_variant" 2 keeps such shapes on the three launches below)
+	if (get_option(OPT_CONV_VARIANT) == 0) {
+		const int rc = conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
+		if (rc >= 0) return rc;
 	}
 
 	LTEN_HIP_REQUIRE(workspace != nullptr, "conv2dq: workspace is null");

@@ -40,7 +40,14 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (2, 5, 11, 13, 9, 3, 3, 1, 0, 1, 2),        # 45 taps: twelve packed dwords
                                  (1, 4, 8, 8, 3, 2, 2, 1, 1, 1, 1),          # 16 taps: four dwords, all full
                                  (2, 11, 7, 9, 5, 1, 3, 0, 1, 1, 1),         # 33 taps: one tap in the ninth dword
-                                 (1, 3, 12, 10, 7, 4, 4, 1, 2, 1, 1)])       # 48 taps
+                                 (1, 3, 12, 10, 7, 4, 4, 1, 2, 1, 1),        # 48 taps
+                                 (64, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1),     # l-ten's quantized MNIST conv2 at batch 64
+                                 (3, 9, 15, 11, 64, 3, 3, 1, 1, 1, 1),       # 81 taps, four blocks of 16 channels, 165 positions
+                                 (2, 16, 28, 32, 17, 3, 3, 2, 2, 1, 1),      # 144 taps, 1020 positions an image: 64 workgroups each
+                                 (2, 40, 5, 5, 30, 5, 5, 2, 2, 1, 1),        # 1000 taps, most of them outside the image
+                                 (2, 40, 5, 5, 50, 5, 5, 2, 2, 1, 1),        # the same with 50 channels: weights beyond the 64 KB of LDS the route allows
+                                 (1, 33, 31, 31, 3, 2, 2, 0, 0, 3, 3),       # 132 taps, image of 31.7 KB, stride 3
+                                 (1, 65, 9, 9, 70, 1, 1, 0, 0, 1, 1)])       # 65 taps but 70 channels: not for the one-launch route
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -54,9 +61,23 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         want_y, want_acc = ob.conv2dq_forward(geo, x, w, sc, zp, bias=bias)
         y, acc = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
         kern = gpu.last_kernel()
-        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_rows_gemm_finish"), kern
+        # up to 64 taps: one launch from registers; longer windows on small images: one launch from the image in LDS;
+        # else patch rows + GEMM + finish
+        Kp, ncb = (K + 63) // 64 * 64, (Cout + 15) // 16
+        lds = (Cin * H * W + 15) // 16 * 16 + ncb * 16 * (Kp + 16) + 4 * Kp
+        small = (Cin * H * W <= 32768 and Cout <= 64 and K <= 1024 and Ho * Wo <= 1024 and lds <= 65536 and
+                 N * ((Ho * Wo + 15) // 16) <= 4096)
+        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
         assert np.array_equal(y, want_y), kern
+        if kern == "conv2dq_image":   # the three-launch route on the same shape gives the same bytes
+            gpu.set_option("conv_variant", 2)
+            try:
+                y2, acc2 = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
+                assert gpu.last_kernel() == "conv2dq_rows_gemm_finish"
+            finally:
+                gpu.set_option("conv_variant", 0)
+            assert np.array_equal(acc2, want_acc) and np.array_equal(y2, want_y)
     if K > 64:   # l-ten's decomposition image by image (what a workspace beyond 2 GiB falls back to) gives the same bytes
         gpu.set_option("conv_variant", 1)
         try:
