@@ -27,6 +27,9 @@ constexpr int CQ_MAXK = 64, CQ_CO = 64;
 // one launch for small images with windows above 64 taps (convq_image.hip); -1 = not a shape for it
 int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
                            float zp_out, void* y, bool out_acc);
+// one launch for larger images, a band of output rows per workgroup (convq_image.hip); -1 = not a shape for it
+int conv2dq_band_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
+                          float zp_out, void* y, bool out_acc);
 
 // ND = dwords of packed taps a thread holds (4 taps each): 4, 8, 12 or 16, the smallest that covers K.
 template <int OUT, int ND>
@@ -272,8 +275,11 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 
 	// small images with a longer window (l-ten's quantized MNIST conv2): still one launch, no workspace (convq_image.hip;
 	// option "conv_variant" 2 keeps such shapes on the three launches below)
-	if (get_option(OPT_CONV_VARIANT) == 0) {
-		const int rc = conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
+	if (get_option(OPT_CONV_VARIANT) == 0 || get_option(OPT_CONV_VARIANT) == 3) {
+		int rc = get_option(OPT_CONV_VARIANT) == 3 ? -1 : conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
+		if (rc >= 0) return rc;
+		// larger images: a band of output rows per workgroup, the input rows it needs in LDS (at most 64 output channels)
+		rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
 	}
 

@@ -199,6 +199,263 @@ __global__ __launch_bounds__(256) void conv2dq_image_kernel(ConvGeo g, const uin
 	}
 }
 
+// The same idea for images of any size: a workgroup takes a band of TB output rows of one image and stages the input rows
+// the band's windows reach, pixel-major with the channels innermost: [RH rows][RW columns][PP bytes], byte ci of a
+// pixel its channel ci, channels padded with zeros to a multiple of CP (4, 8 or 16 by the channel count), the padding
+// written out as zero pixels (PL zero columns on the left, rows above and below the image as zero rows).  The
+// reduction runs in the order (tap, channel) instead of l-ten's (channel, tap), the weights being staged in the same
+// order, so that the 16 bytes a lane feeds to a 16x16x64 MFMA are 16 / CP aligned pieces of CP consecutive channels of
+// a pixel: one to four LDS reads and no arithmetic per fragment, no bounds checks (the byte-wise gather of the
+// small-image kernel above, an addition, a byte read and a shift-or per byte, made this kernel take 73.7 us on 32 x 64 x
+// 56 x 56 -> 64 channels 3 x 3; the patch-row route with its workspace 157 us).  A wavefront owns up to four blocks of
+// 16 positions at a time and walks the k-steps once for all of them.
+struct BandPlan {
+	int CP, CPtot, PP, UC, Kp, ncb, wpitch, TB, RH, RW, PL;
+	unsigned off_w, off_unit, off_kmap, bytes;
+};
+
+template <int OUT, int CP>
+__global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
+                                                           const int32_t* __restrict__ bias, int zp_in, int zp_w, float mult, float zp_out,
+                                                           void* __restrict__ y, BandPlan pl, int bands_per_image)
+{
+	extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+	uint8_t* const s_rgn = smem;
+	uint8_t* const s_w = smem + pl.off_w;
+	uint32_t* const s_unit = reinterpret_cast<uint32_t*>(smem + pl.off_unit);
+
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+	const int lrow = lane & 15, lgrp = lane >> 4;
+	const int T = g.kh * g.kw, K = g.Cin * T, HW = g.Ho * g.Wo, Kp = pl.Kp, RH = pl.RH, RW = pl.RW, PP = pl.PP, CPtot = pl.CPtot;
+	const int n = (int)blockIdx.x / bands_per_image, hb = ((int)blockIdx.x % bands_per_image) * pl.TB;
+	const int rows_here = min(pl.TB, g.Ho - hb);
+	const int rgn_y0 = hb * g.sh - g.ph;  // image row of region row 0
+	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+
+	// ---- the region: four columns of four channels at a time (four dword loads where the image's rows keep dword
+	// alignment, W % 4 == 0 and an aligned image: such a dword lies inside the image or outside as a whole), transposed
+	// in registers into four dwords of four channels each
+	const int rw4 = RW / 4, cg_n = CPtot / 4, items = cg_n * RH * rw4;
+	const bool fast = (g.W & 3) == 0 && (reinterpret_cast<uintptr_t>(xn) & 3) == 0;
+	for (int idx = tid; idx < items; idx += 256) {
+		const int c4 = idx % rw4, r = (idx / rw4) % RH, cg = idx / (rw4 * RH);
+		const int yy = rgn_y0 + r, col0 = c4 * 4 - pl.PL;
+		uint32_t d[4] = { 0, 0, 0, 0 };
+		if (yy >= 0 && yy < g.H) {
+#pragma unroll
+			for (int c = 0; c < 4; c++) {
+				const int ci = cg * 4 + c;
+				if (ci >= g.Cin) continue;
+				const uint8_t* row = xn + ((int64_t)ci * g.H + yy) * g.W;
+				if (fast) {
+					if (col0 >= 0 && col0 + 4 <= g.W) d[c] = *reinterpret_cast<const uint32_t*>(row + col0);
+				} else {
+#pragma unroll
+					for (int b = 0; b < 4; b++)
+						if (col0 + b >= 0 && col0 + b < g.W) d[c] |= (uint32_t)row[col0 + b] << (8 * b);
+				}
+			}
+		}
+		// byte b of d[c] is (column b, channel c): out[b] = the four channels of column b
+		const uint32_t lo01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+		const uint32_t lo23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+		uint32_t out[4];
+		out[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+		out[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+		out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+		out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+		uint8_t* dst = s_rgn + (r * RW + c4 * 4) * PP + cg * 4;
+#pragma unroll
+		for (int b = 0; b < 4; b++) *reinterpret_cast<uint32_t*>(dst + b * PP) = out[b];
+	}
+	// ---- unit table: a unit is CP consecutive channels of one tap; entry = its byte offset inside the region for the
+	// position (hb, 0), bit 30 for units past the last tap
+	for (int u = tid; u < Kp / CP; u += 256) {
+		const int t = u / pl.UC, cc = u - t * pl.UC;
+		const int tc = min(t, T - 1), i = tc / g.kw, j = tc - i * g.kw;
+		s_unit[u] = (uint32_t)((i * RW + j + pl.PL - g.pw) * PP + cc * CP) | (t < T ? 0u : TAP_PAST_K);
+	}
+	// ---- weights in the order (tap, channel), into the signed domain; rows past Cout, channels past Cin and units past
+	// the last tap hold signed zeros.  Where the weight rows keep dword alignment they are read along memory, a dword of
+	// four consecutive (channel, tap) bytes per thread, and scattered byte by byte into the new order (a quarter of
+	// the load instructions of the other way round, and whole cache lines per wave-wide load: on 4 x 64 x 56 x 56 -> 64
+	// channels 3 x 3 staging the weights by gathered bytes was 10.8 of the kernel's 22.8 us); else a thread builds a
+	// dword of the new order from four bytes it gathers.
+	const bool w_fast = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
+	if (w_fast) {
+		// where byte k of a weight row (l-ten's order: channel k / T, tap k % T) goes in the new order: worked out once, the
+		// divisions by T for every byte had been most of the staging time
+		uint16_t* const s_kmap = reinterpret_cast<uint16_t*>(smem + pl.off_kmap);
+		for (int k = tid; k < K; k += 256) {
+			const int ci = k / T;
+			s_kmap[k] = (uint16_t)((k - ci * T) * CPtot + ci);
+		}
+		for (int idx = tid; idx < pl.ncb * pl.wpitch; idx += 256) reinterpret_cast<v4i*>(s_w)[idx] = v4i{ 0, 0, 0, 0 };
+		__syncthreads();
+		// (eight loads in flight per thread: one load, then its four byte writes, made a chain of round trips to the L2)
+		const int total = g.Cout * (K / 4);   // the weights are one run of Cout * K bytes: dword number idx holds bytes 4 idx .. + 3
+		constexpr int U = 8;
+		// this thread's dwords are 256 apart: (row, byte in the row) advance by (1024 / K, 1024 % K), no division per dword
+		const int step_co = 1024 / K, step_k = 1024 - step_co * K;
+		int co = (4 * tid) / K, k = 4 * tid - co * K;
+		for (int idx0 = tid; idx0 < total; idx0 += 256 * U) {
+			uint32_t v[U];
+#pragma unroll
+			for (int u = 0; u < U; u++) v[u] = reinterpret_cast<const uint32_t*>(w)[min(idx0 + u * 256, total - 1)] ^ 0x80808080u;
+#pragma unroll
+			for (int u = 0; u < U; u++) {
+				if (idx0 + u * 256 < total) {
+					uint8_t* row = s_w + co * pl.wpitch;
+#pragma unroll
+					for (int b = 0; b < 4; b++) row[s_kmap[k + b]] = (uint8_t)(v[u] >> (8 * b));  // K % 4 == 0: the four bytes lie in one row
+				}
+				co += step_co;
+				k += step_k;
+				if (k >= K) {
+					k -= K;
+					co++;
+				}
+			}
+		}
+	} else {
+		const int kd = Kp / 4;
+		for (int idx = tid; idx < pl.ncb * 16 * kd; idx += 256) {
+			const int co = idx / kd, k0 = (idx - co * kd) * 4;
+			const int t = k0 / CPtot, c0 = k0 - t * CPtot;
+			uint32_t v = 0;
+			if (co < g.Cout && t < T) {
+				const uint8_t* wr = w + (int64_t)co * K + t;
+#pragma unroll
+				for (int b = 0; b < 4; b++) {
+					const uint32_t raw = wr[min(c0 + b, g.Cin - 1) * T];
+					v |= ((c0 + b < g.Cin ? raw : 0x80u) ^ 0x80u) << (8 * b);
+				}
+			}
+			*reinterpret_cast<uint32_t*>(s_w + co * pl.wpitch + k0) = v;
+		}
+	}
+	__syncthreads();
+
+	const int coef_a = 128 - zp_w, coef_b = 128 - zp_in;
+	const int konst = K * (zp_in * zp_w - 16384);
+	const int band_pos = rows_here * g.Wo;            // positions of this band
+	const int nblocks = (band_pos + 15) / 16;
+	constexpr int BW = 4;                             // blocks a wavefront holds at a time
+	constexpr int UPG = 16 / CP;                      // units per k-group of 16 bytes
+	for (int pass0 = 0; pass0 < nblocks; pass0 += 4 * BW) {
+		// this wavefront's blocks of the pass: pass0 + wave + 4 u
+		int base[BW];
+#pragma unroll
+		for (int u = 0; u < BW; u++) {
+			const int p = min((pass0 + wave + 4 * u) * 16 + lrow, band_pos - 1);  // positions past the band repeat its last one and are not stored
+			const int dh = p / g.Wo, wo = p - dh * g.Wo;
+			base[u] = (dh * g.sh * RW + wo * g.sw) * PP;
+		}
+		v4i acc[BW][4];
+		uint32_t sa[BW], sw[4];
+#pragma unroll
+		for (int u = 0; u < BW; u++) {
+			sa[u] = 0;
+#pragma unroll
+			for (int cb = 0; cb < 4; cb++) acc[u][cb] = v4i{ 0, 0, 0, 0 };
+		}
+#pragma unroll
+		for (int cb = 0; cb < 4; cb++) sw[cb] = 0;
+		for (int ks = 0; ks < Kp; ks += 64) {
+			uint32_t uoff[UPG];
+#pragma unroll
+			for (int q = 0; q < UPG; q++) uoff[q] = s_unit[(ks + lgrp * 16) / CP + q];
+			v4i bf[4];
+#pragma unroll
+			for (int cb = 0; cb < 4; cb++) {
+				bf[cb] = v4i{ 0, 0, 0, 0 };
+				if (cb < pl.ncb) {
+					bf[cb] = *reinterpret_cast<const v4i*>(s_w + (cb * 16 + lrow) * pl.wpitch + ks + lgrp * 16);
+					const v4i braw = flip_sign_bits(bf[cb]);  // back to l-ten's bytes for the sum (padding then holds 0x80)
+#pragma unroll
+					for (int q = 0; q < 4; q++) sw[cb] = __builtin_amdgcn_sad_u8((unsigned)braw[q], 0u, sw[cb]);
+				}
+			}
+#pragma unroll
+			for (int u = 0; u < BW; u++) {
+				if (pass0 + wave + 4 * u >= nblocks) break;  // the same for the whole wavefront
+				uint32_t d[4];
+#pragma unroll
+				for (int q = 0; q < UPG; q++) {
+					// a unit past the last tap reads the region's first bytes and counts as nothing
+					const bool real = (uoff[q] & TAP_PAST_K) == 0;
+					const uint8_t* src = s_rgn + (real ? uoff[q] + (uint32_t)base[u] : 0u);
+					if (CP == 16) {
+						const v4i v = *reinterpret_cast<const v4i*>(src);
+						d[0] = real ? (uint32_t)v.x : 0u; d[1] = real ? (uint32_t)v.y : 0u; d[2] = real ? (uint32_t)v.z : 0u; d[3] = real ? (uint32_t)v.w : 0u;
+					} else if (CP == 8) {
+						const uint2 v = *reinterpret_cast<const uint2*>(src);
+						d[2 * q] = real ? v.x : 0u; d[2 * q + 1] = real ? v.y : 0u;
+					} else {
+						const uint32_t v = *reinterpret_cast<const uint32_t*>(src);
+						d[q] = real ? v : 0u;
+					}
+				}
+#pragma unroll
+				for (int q = 0; q < 4; q++) sa[u] = __builtin_amdgcn_sad_u8(d[q], 0u, sa[u]);
+				const v4i a = flip_sign_bits(v4i{ (int)d[0], (int)d[1], (int)d[2], (int)d[3] });
+#pragma unroll
+				for (int cb = 0; cb < 4; cb++)
+					if (cb < pl.ncb) acc[u][cb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bf[cb], acc[u][cb], 0, 0, 0);
+			}
+		}
+		// channel sums: the four k-groups of channel 16 cb + lrow sit in lanes lrow, + 16, + 32, + 48; every byte of
+		// padding in a weight row held 0x80
+		int ct[4];
+#pragma unroll
+		for (int cb = 0; cb < 4; cb++) {
+			uint32_t s4 = sw[cb];
+			s4 += __shfl_xor(s4, 16, 64);
+			s4 += __shfl_xor(s4, 32, 64);
+			ct[cb] = coef_b * ((int)s4 - 128 * (Kp - K));
+		}
+#pragma unroll
+		for (int u = 0; u < BW; u++) {
+			const int blk = pass0 + wave + 4 * u;
+			if (blk >= nblocks) break;
+			uint32_t rs = sa[u];
+			rs += __shfl_xor(rs, 16, 64);
+			rs += __shfl_xor(rs, 32, 64);
+			const int p0 = blk * 16 + lgrp * 4;  // first of this lane's four positions in the band
+			int rt[4];
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				const int row_sum = __shfl((int)rs, lgrp * 4 + e, 64);
+				const int pos = min(hb * g.Wo + p0 + e, HW - 1);
+				rt[e] = coef_a * row_sum + konst + (bias != nullptr ? bias[pos] : 0);
+			}
+			// the four positions are four consecutive bytes of y: one dword store where they all exist and the dword is aligned
+			const bool whole = OUT != Q_OUT_ACC && p0 + 4 <= band_pos && ((HW | (hb * g.Wo)) & 3) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
+#pragma unroll
+			for (int cb = 0; cb < 4; cb++) {
+				const int co = cb * 16 + lrow;
+				if (cb >= pl.ncb || co >= g.Cout) continue;
+				const int64_t o = ((int64_t)n * g.Cout + co) * HW + hb * g.Wo + p0;
+				if (OUT == Q_OUT_ACC) {
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (p0 + e < band_pos) static_cast<int*>(y)[o + e] = acc[u][cb][e] + rt[e] + ct[cb];
+				} else {
+					uint32_t word = 0;
+#pragma unroll
+					for (int e = 0; e < 4; e++) word |= (requant<OUT>(acc[u][cb][e] + rt[e] + ct[cb], mult, zp_out) & 0xFFu) << (8 * e);
+					if (whole) *reinterpret_cast<uint32_t*>(static_cast<uint8_t*>(y) + o) = word;
+					else {
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							if (p0 + e < band_pos) static_cast<uint8_t*>(y)[o + e] = (uint8_t)(word >> (8 * e));
+					}
+				}
+			}
+		}
+	}
+}
+
 // Whether the one-launch route takes the call, and its LDS layout.  Few workgroups per image and few in all: every
 // workgroup stages the whole image and all weights, which pays while the call is bound by launch latency (three
 // launches otherwise) and not beyond.
@@ -219,12 +476,79 @@ static bool image_plan(const ConvGeo& g, ImagePlan& pl)
 	return pl.bytes <= 64 * 1024;
 }
 
+// The band kernel's plan: the tallest band whose region, the weights and the unit table fit 64 KB of LDS, shortened
+// while that leaves the chip with fewer than two workgroups per CU.
+static bool band_plan(const ConvGeo& g, BandPlan& pl)
+{
+	const int64_t T = (int64_t)g.kh * g.kw, K = (int64_t)g.Cin * T;
+	if (K <= 64 || g.Cout > 64 || g.pw > 64 || g.Cin > 1024) return false;
+	pl.CP = g.Cin <= 4 ? 4 : g.Cin <= 8 ? 8 : 16;
+	pl.CPtot = (g.Cin + pl.CP - 1) / pl.CP * pl.CP;
+	pl.PP = pl.CPtot + (pl.CPtot % 32 == 0 ? 16 : 0);  // pixels 32 or 64 bytes apart would meet on the same LDS banks
+	pl.UC = pl.CPtot / pl.CP;
+	const int64_t kprime = T * pl.CPtot;
+	if (kprime > 4096) return false;
+	pl.Kp = (int)((kprime + 63) & ~63ll);
+	pl.ncb = (g.Cout + 15) / 16;
+	pl.wpitch = pl.Kp + CQI_PAD;
+	pl.PL = (g.pw + 3) & ~3;
+	// the rightmost byte a window reaches is column (Wo - 1) sw + kw - 1 - pw of the image
+	const int reach = (g.Wo - 1) * g.sw + g.kw - g.pw;   // image columns 0 .. reach - 1 (beyond W: padding)
+	pl.RW = (pl.PL + (reach > g.W ? reach : g.W) + 3) & ~3;
+	const int64_t fixed = (int64_t)pl.ncb * 16 * pl.wpitch + (int64_t)(pl.Kp / pl.CP) * 4 + 2 * K + 32;
+	int tb = 0;
+	for (int t = 1; t <= g.Ho && t <= 64; t++) {
+		const int64_t rh = (int64_t)(t - 1) * g.sh + g.kh;
+		if (rh * pl.RW * pl.PP + fixed > 64 * 1024) break;
+		tb = t;
+	}
+	if (tb == 0) return false;
+	while (tb > 1 && (int64_t)g.N * ((g.Ho + tb - 1) / tb) < 512) tb--;
+	pl.TB = tb;
+	pl.RH = (tb - 1) * g.sh + g.kh;
+	pl.off_w = (unsigned)((pl.RH * pl.RW * pl.PP + 15) & ~15);
+	pl.off_unit = pl.off_w + (unsigned)(pl.ncb * 16 * pl.wpitch);
+	pl.off_kmap = pl.off_unit + (unsigned)(pl.Kp / pl.CP) * 4;
+	pl.bytes = pl.off_kmap + (unsigned)((2 * K + 15) & ~15ll);
+	return (int64_t)g.N * ((g.Ho + tb - 1) / tb) < (1ll << 31);
+}
+
+// 0 = launched; -1 = not a shape for this route
+int conv2dq_band_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
+                          float zp_out, void* y, bool out_acc)
+{
+	BandPlan pl;
+	if (!band_plan(g, pl)) return -1;
+	const int per_image = (g.Ho + pl.TB - 1) / pl.TB;
+	const dim3 grid((unsigned)(g.N * per_image));
+	set_kernel_name("conv2dq_band");
+	const int out = out_acc ? Q_OUT_ACC : (mult == mult && (mult < 0 ? -mult : mult) <= 0.99f) ? Q_OUT_U8_FAST : Q_OUT_U8_EXACT;
+#define LTEN_LAUNCH(OUTV, CPV) conv2dq_band_kernel<OUTV, CPV><<<grid, dim3(256), pl.bytes, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, pl, per_image)
+#define LTEN_LAUNCH_CP(OUTV)                                  \
+	if (pl.CP == 16) LTEN_LAUNCH(OUTV, 16);                   \
+	else if (pl.CP == 8) LTEN_LAUNCH(OUTV, 8);                \
+	else LTEN_LAUNCH(OUTV, 4);
+	if (out == Q_OUT_ACC) { LTEN_LAUNCH_CP(Q_OUT_ACC) }
+	else if (out == Q_OUT_U8_FAST) { LTEN_LAUNCH_CP(Q_OUT_U8_FAST) }
+	else { LTEN_LAUNCH_CP(Q_OUT_U8_EXACT) }
+#undef LTEN_LAUNCH_CP
+#undef LTEN_LAUNCH
+	LTEN_HIP_LAUNCH_CHECK();
+	return 0;
+}
+
 // 0 = launched; -1 = not a shape for this route
 int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
                            float zp_out, void* y, bool out_acc)
 {
 	ImagePlan pl;
 	if (!image_plan(g, pl)) return -1;
+	// Every workgroup stages the image and all weights again: beyond 16 MB of that in all, the band kernel is ahead where
+	// it applies (16 x 32 x 28 x 28 -> 64 channels 3 x 3, 784 workgroups staging 43 KB each: 26.9 us here, 16.7 us there;
+	// 64 x 32 x 14 x 14 -> 32, 832 workgroups staging 15.5 KB: 15.0 us here, 22.1 us there)
+	const int64_t staged = (int64_t)g.N * ((g.Ho * g.Wo + CQI_POS - 1) / CQI_POS) * ((int64_t)pl.img16 + (int64_t)pl.ncb * 16 * pl.Kp);
+	BandPlan other;
+	if (staged > (16ll << 20) && band_plan(g, other)) return -1;
 	const int per_image = (g.Ho * g.Wo + CQI_POS - 1) / CQI_POS;
 	const dim3 grid((unsigned)(g.N * per_image));
 	// windows that cannot reach outside the image need no bounds checks on the way

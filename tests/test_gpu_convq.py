@@ -47,7 +47,12 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (2, 40, 5, 5, 30, 5, 5, 2, 2, 1, 1),        # 1000 taps, most of them outside the image
                                  (2, 40, 5, 5, 50, 5, 5, 2, 2, 1, 1),        # the same with 50 channels: weights beyond the 64 KB of LDS the route allows
                                  (1, 33, 31, 31, 3, 2, 2, 0, 0, 3, 3),       # 132 taps, image of 31.7 KB, stride 3
-                                 (1, 65, 9, 9, 70, 1, 1, 0, 0, 1, 1)])       # 65 taps but 70 channels: not for the one-launch route
+                                 (1, 65, 9, 9, 70, 1, 1, 0, 0, 1, 1),        # 65 taps but 70 channels: not for the one-launch route
+                                 (2, 16, 40, 40, 24, 3, 3, 1, 1, 1, 1),      # 1600 positions an image: bands of output rows
+                                 (1, 8, 50, 70, 64, 5, 3, 2, 1, 2, 1),       # bands with a row stride of 2, 64 channels, 120 taps
+                                 (1, 3, 100, 37, 9, 5, 5, 0, 0, 1, 1),       # rows of 37 bytes: the region is filled byte by byte
+                                 (3, 12, 33, 41, 20, 3, 3, 0, 2, 1, 3),      # column stride 3, padding 2 on the columns only
+                                 (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1)])     # 576 taps, 64 channels: several passes of blocks per band
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -67,10 +72,22 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         lds = (Cin * H * W + 15) // 16 * 16 + ncb * 16 * (Kp + 16) + 4 * Kp
         small = (Cin * H * W <= 32768 and Cout <= 64 and K <= 1024 and Ho * Wo <= 1024 and lds <= 65536 and
                  N * ((Ho * Wo + 15) // 16) <= 4096)
-        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_rows_gemm_finish"), kern
+        # larger images with at most 64 channels: a band of output rows per workgroup, as long as one row's region fits LDS
+        PL = (pw + 3) // 4 * 4
+        RW = (PL + max((Wo - 1) * sw + kw - pw, W) + 3) // 4 * 4
+        CP = 4 if Cin <= 4 else 8 if Cin <= 8 else 16
+        CPtot = (Cin + CP - 1) // CP * CP
+        PP = CPtot + (16 if CPtot % 32 == 0 else 0)
+        Kb = (kh * kw * CPtot + 63) // 64 * 64      # the band kernel reduces over (tap, channel padded to a multiple of CP)
+        band = (Cout <= 64 and pw <= 64 and kh * kw * CPtot <= 4096 and
+                kh * RW * PP + ncb * 16 * (Kb + 16) + 4 * (Kb // CP) + 2 * K + 32 <= 65536)
+        # (the small-image kernel only while its workgroups stage at most 16 MB in all, where the band kernel applies)
+        staged = N * ((Ho * Wo + 15) // 16) * ((Cin * H * W + 15) // 16 * 16 + ncb * 16 * Kp)
+        small = small and not (band and staged > 16 << 20)
+        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_band" if band else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
         assert np.array_equal(y, want_y), kern
-        if kern == "conv2dq_image":   # the three-launch route on the same shape gives the same bytes
+        if kern in ("conv2dq_image", "conv2dq_band"):   # the three-launch route on the same shape gives the same bytes
             gpu.set_option("conv_variant", 2)
             try:
                 y2, acc2 = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
