@@ -207,15 +207,53 @@ __global__ __launch_bounds__(256) void conv2dq_image_kernel(ConvGeo g, const uin
 // order, so that the 16 bytes a lane feeds to a 16x16x64 MFMA are 16 / CP aligned pieces of CP consecutive channels of
 // a pixel: one to four LDS reads and no arithmetic per fragment, no bounds checks (the byte-wise gather of the
 // small-image kernel above, an addition, a byte read and a shift-or per byte, made this kernel take 73.7 us on 32 x 64 x
-// 56 x 56 -> 64 channels 3 x 3; the patch-row route with its workspace 157 us).  A wavefront owns up to four blocks of
-// 16 positions at a time and walks the k-steps once for all of them.
+// 56 x 56 -> 64 channels 3 x 3; the patch-row route with its workspace 157 us; this kernel 28.9 us, of which about 7 are
+// the loads of the region, 3.7 the weights, 9.5 the k-steps and 3.8 the stores: all 448 workgroups are resident at
+// once and pass through these phases together).  A wavefront owns up to four blocks of 16 positions at a time and
+// walks the k-steps once for all of them.
 struct BandPlan {
 	int CP, CPtot, PP, UC, Kp, ncb, wpitch, TB, RH, RW, PL;
 	unsigned off_w, off_unit, off_kmap, bytes;
+	unsigned inv_rw4, inv_rh, inv_cq;  // reciprocals for small_div: RW / 4, RH, Cin / 4
 };
 
+// n / d for n d < 2^32 by one multiplication, inv = small_div_inverse(d): a thread of the band kernel's staging loops
+// splits its item number three ways per item, 30-odd instructions per 32-bit division otherwise.
+static inline unsigned small_div_inverse(unsigned d) { return d <= 1 ? 0u : (unsigned)((0x100000000ull + d - 1) / d); }
+__device__ __forceinline__ int small_div(int n, unsigned inv) { return inv == 0 ? n : (int)__umulhi((unsigned)n, inv); }
+
+// Weights of a window of T taps into the band kernel's order, for rows that keep dword alignment and channel counts
+// that are multiples of four: four channels of a row are 4 T consecutive bytes, T dwords, and become T dwords of the
+// new order (one per tap, its four bytes the four channels), permuted in registers: T dword loads along memory and T
+// dword writes to LDS per thread, where scattering the bytes of every loaded dword took four byte writes that met on a
+// few LDS banks (8 of 20 us on 4 x 64 x 56 x 56 -> 64 channels 3 x 3).
+template <int T>
+__device__ __forceinline__ void band_stage_weights(const uint8_t* __restrict__ w, uint8_t* s_w, int Cout, int Cin, int CPtot, int wpitch, int tid,
+                                                   unsigned inv_cq)
+{
+	const int cq = Cin / 4, K = Cin * T;
+	for (int u = tid; u < Cout * cq; u += 256) {
+		const int co = small_div(u, inv_cq), q = u - co * cq;
+		const uint32_t* src = reinterpret_cast<const uint32_t*>(w + (int64_t)co * K) + q * T;
+		uint32_t in[T];
+#pragma unroll
+		for (int i = 0; i < T; i++) in[i] = src[i];
+		uint8_t* dst = s_w + co * wpitch + 4 * q;
+#pragma unroll
+		for (int t = 0; t < T; t++) {
+			uint32_t v = 0;
+#pragma unroll
+			for (int b = 0; b < 4; b++) {
+				const int pos = b * T + t;  // byte of the 4 T that holds (channel b, tap t)
+				v |= ((in[pos >> 2] >> (8 * (pos & 3))) & 0xFFu) << (8 * b);
+			}
+			*reinterpret_cast<uint32_t*>(dst + t * CPtot) = v ^ 0x80808080u;
+		}
+	}
+}
+
 template <int OUT, int CP>
-__global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
+__global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
                                                            const int32_t* __restrict__ bias, int zp_in, int zp_w, float mult, float zp_out,
                                                            void* __restrict__ y, BandPlan pl, int bands_per_image)
 {
@@ -227,7 +265,12 @@ __global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int lrow = lane & 15, lgrp = lane >> 4;
 	const int T = g.kh * g.kw, K = g.Cin * T, HW = g.Ho * g.Wo, Kp = pl.Kp, RH = pl.RH, RW = pl.RW, PP = pl.PP, CPtot = pl.CPtot;
-	const int n = (int)blockIdx.x / bands_per_image, hb = ((int)blockIdx.x % bands_per_image) * pl.TB;
+	// workgroups go to the eight XCDs in turn: number b works on band (b % 8) * (bands / 8) + b / 8 (the first bands % 8
+	// XCDs one more), so that neighbouring bands of an image, which share the input rows under their windows, find
+	// them in the same L2
+	const int nb = (int)gridDim.x, xcd = (int)blockIdx.x & 7;
+	const int bid = xcd * (nb >> 3) + min(xcd, nb & 7) + ((int)blockIdx.x >> 3);
+	const int n = bid / bands_per_image, hb = (bid % bands_per_image) * pl.TB;
 	const int rows_here = min(pl.TB, g.Ho - hb);
 	const int rgn_y0 = hb * g.sh - g.ph;  // image row of region row 0
 	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
@@ -237,22 +280,36 @@ __global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint
 	// in registers into four dwords of four channels each
 	const int rw4 = RW / 4, cg_n = CPtot / 4, items = cg_n * RH * rw4;
 	const bool fast = (g.W & 3) == 0 && (reinterpret_cast<uintptr_t>(xn) & 3) == 0;
+	// Every load comes from an address clamped into the image and its value is dropped afterwards where the dword lies
+	// outside: no branch stands between the four loads of an item.  The split of the item number is by multiplication.
+	// (Several items in flight per thread are no faster, 32.9 us with three and 33.7 with six against 31.3 with one on
+	// 32 x 64 x 56 x 56 -> 64 channels 3 x 3: the loads of all workgroups start together on caches that hold nothing
+	// yet, and what they wait for is the memory behind them, 7 us in all, not one another.)
 	for (int idx = tid; idx < items; idx += 256) {
-		const int c4 = idx % rw4, r = (idx / rw4) % RH, cg = idx / (rw4 * RH);
+		const int q1 = small_div(idx, pl.inv_rw4), c4 = idx - q1 * rw4, cg = small_div(q1, pl.inv_rh), r = q1 - cg * RH;
 		const int yy = rgn_y0 + r, col0 = c4 * 4 - pl.PL;
-		uint32_t d[4] = { 0, 0, 0, 0 };
-		if (yy >= 0 && yy < g.H) {
+		const int yc = min(max(yy, 0), g.H - 1);
+		uint32_t d[4];
+		if (fast) {
+			const bool inside = yy == yc && col0 >= 0 && col0 + 4 <= g.W;
+			const int cc = min(max(col0, 0), g.W - 4);
 #pragma unroll
 			for (int c = 0; c < 4; c++) {
 				const int ci = cg * 4 + c;
-				if (ci >= g.Cin) continue;
-				const uint8_t* row = xn + ((int64_t)ci * g.H + yy) * g.W;
-				if (fast) {
-					if (col0 >= 0 && col0 + 4 <= g.W) d[c] = *reinterpret_cast<const uint32_t*>(row + col0);
-				} else {
+				const uint32_t v = *reinterpret_cast<const uint32_t*>(xn + ((int64_t)min(ci, g.Cin - 1) * g.H + yc) * g.W + cc);
+				d[c] = inside && ci < g.Cin ? v : 0u;
+			}
+		} else {
 #pragma unroll
-					for (int b = 0; b < 4; b++)
-						if (col0 + b >= 0 && col0 + b < g.W) d[c] |= (uint32_t)row[col0 + b] << (8 * b);
+			for (int c = 0; c < 4; c++) {
+				const int ci = cg * 4 + c;
+				const uint8_t* row = xn + ((int64_t)min(ci, g.Cin - 1) * g.H + yc) * g.W;
+				d[c] = 0;
+#pragma unroll
+				for (int b = 0; b < 4; b++) {
+					const int col = col0 + b;
+					const uint32_t v = row[min(max(col, 0), g.W - 1)];
+					d[c] |= (yy == yc && col >= 0 && col < g.W && ci < g.Cin ? v : 0u) << (8 * b);
 				}
 			}
 		}
@@ -276,13 +333,20 @@ __global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint
 		s_unit[u] = (uint32_t)((i * RW + j + pl.PL - g.pw) * PP + cc * CP) | (t < T ? 0u : TAP_PAST_K);
 	}
 	// ---- weights in the order (tap, channel), into the signed domain; rows past Cout, channels past Cin and units past
-	// the last tap hold signed zeros.  Where the weight rows keep dword alignment they are read along memory, a dword of
-	// four consecutive (channel, tap) bytes per thread, and scattered byte by byte into the new order (a quarter of
-	// the load instructions of the other way round, and whole cache lines per wave-wide load: on 4 x 64 x 56 x 56 -> 64
-	// channels 3 x 3 staging the weights by gathered bytes was 10.8 of the kernel's 22.8 us); else a thread builds a
-	// dword of the new order from four bytes it gathers.
+	// the last tap hold signed zeros.  Three ways, by what the shape allows: permuted in registers (band_stage_weights:
+	// 3 x 3, 5 x 5 and 7 x 7 windows of a multiple of four channels); else, where the weight rows keep dword alignment,
+	// read along memory, a dword of four consecutive (channel, tap) bytes per thread, and scattered byte by byte into
+	// the new order; else a thread builds a dword of the new order from four bytes it gathers.  On 4 x 64 x 56 x 56 ->
+	// 64 channels 3 x 3 the three take 3.7, 8 and 10.8 us of the kernel's time.
 	const bool w_fast = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
-	if (w_fast) {
+	const bool w_taps = w_fast && (g.Cin & 3) == 0 && (T == 9 || T == 25 || T == 49);
+	if (w_taps) {
+		for (int idx = tid; idx < pl.ncb * pl.wpitch; idx += 256) reinterpret_cast<v4i*>(s_w)[idx] = v4i{ 0, 0, 0, 0 };
+		__syncthreads();
+		if (T == 9) band_stage_weights<9>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		else if (T == 25) band_stage_weights<25>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		else band_stage_weights<49>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+	} else if (w_fast) {
 		// where byte k of a weight row (l-ten's order: channel k / T, tap k % T) goes in the new order: worked out once, the
 		// divisions by T for every byte had been most of the staging time
 		uint16_t* const s_kmap = reinterpret_cast<uint16_t*>(smem + pl.off_kmap);
@@ -361,25 +425,24 @@ __global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint
 		}
 #pragma unroll
 		for (int cb = 0; cb < 4; cb++) sw[cb] = 0;
-		for (int ks = 0; ks < Kp; ks += 64) {
+		// operands of a k-step: the weights' fragments and, per block, the 16 bytes of this lane's position and k-group.
+		// The next step's are read from LDS while this step's MFMAs run (two sets of registers in turn): with two
+		// wavefronts per SIMD, reading and then multiplying left the matrix pipe idle for the length of the reads.
+		struct Operands {
+			v4i bf[4];
+			uint32_t d[BW][4];
+		};
+		auto read_step = [&](int ks, Operands& f) {
 			uint32_t uoff[UPG];
 #pragma unroll
 			for (int q = 0; q < UPG; q++) uoff[q] = s_unit[(ks + lgrp * 16) / CP + q];
-			v4i bf[4];
 #pragma unroll
 			for (int cb = 0; cb < 4; cb++) {
-				bf[cb] = v4i{ 0, 0, 0, 0 };
-				if (cb < pl.ncb) {
-					bf[cb] = *reinterpret_cast<const v4i*>(s_w + (cb * 16 + lrow) * pl.wpitch + ks + lgrp * 16);
-					const v4i braw = flip_sign_bits(bf[cb]);  // back to l-ten's bytes for the sum (padding then holds 0x80)
-#pragma unroll
-					for (int q = 0; q < 4; q++) sw[cb] = __builtin_amdgcn_sad_u8((unsigned)braw[q], 0u, sw[cb]);
-				}
+				f.bf[cb] = v4i{ 0, 0, 0, 0 };
+				if (cb < pl.ncb) f.bf[cb] = *reinterpret_cast<const v4i*>(s_w + (cb * 16 + lrow) * pl.wpitch + ks + lgrp * 16);
 			}
 #pragma unroll
 			for (int u = 0; u < BW; u++) {
-				if (pass0 + wave + 4 * u >= nblocks) break;  // the same for the whole wavefront
-				uint32_t d[4];
 #pragma unroll
 				for (int q = 0; q < UPG; q++) {
 					// a unit past the last tap reads the region's first bytes and counts as nothing
@@ -387,21 +450,48 @@ __global__ __launch_bounds__(256) void conv2dq_band_kernel(ConvGeo g, const uint
 					const uint8_t* src = s_rgn + (real ? uoff[q] + (uint32_t)base[u] : 0u);
 					if (CP == 16) {
 						const v4i v = *reinterpret_cast<const v4i*>(src);
-						d[0] = real ? (uint32_t)v.x : 0u; d[1] = real ? (uint32_t)v.y : 0u; d[2] = real ? (uint32_t)v.z : 0u; d[3] = real ? (uint32_t)v.w : 0u;
+						f.d[u][0] = real ? (uint32_t)v.x : 0u; f.d[u][1] = real ? (uint32_t)v.y : 0u;
+						f.d[u][2] = real ? (uint32_t)v.z : 0u; f.d[u][3] = real ? (uint32_t)v.w : 0u;
 					} else if (CP == 8) {
 						const uint2 v = *reinterpret_cast<const uint2*>(src);
-						d[2 * q] = real ? v.x : 0u; d[2 * q + 1] = real ? v.y : 0u;
+						f.d[u][2 * q] = real ? v.x : 0u; f.d[u][2 * q + 1] = real ? v.y : 0u;
 					} else {
 						const uint32_t v = *reinterpret_cast<const uint32_t*>(src);
-						d[q] = real ? v : 0u;
+						f.d[u][q] = real ? v : 0u;
 					}
 				}
+			}
+		};
+		auto multiply = [&](const Operands& f) {
 #pragma unroll
-				for (int q = 0; q < 4; q++) sa[u] = __builtin_amdgcn_sad_u8(d[q], 0u, sa[u]);
-				const v4i a = flip_sign_bits(v4i{ (int)d[0], (int)d[1], (int)d[2], (int)d[3] });
+			for (int cb = 0; cb < 4; cb++) {
+				if (cb < pl.ncb) {
+					const v4i braw = flip_sign_bits(f.bf[cb]);  // back to l-ten's bytes for the sum (padding then holds 0x80)
+#pragma unroll
+					for (int q = 0; q < 4; q++) sw[cb] = __builtin_amdgcn_sad_u8((unsigned)braw[q], 0u, sw[cb]);
+				}
+			}
+#pragma unroll
+			for (int u = 0; u < BW; u++) {
+				if (pass0 + wave + 4 * u >= nblocks) break;  // the same for the whole wavefront
+#pragma unroll
+				for (int q = 0; q < 4; q++) sa[u] = __builtin_amdgcn_sad_u8(f.d[u][q], 0u, sa[u]);
+				const v4i a = flip_sign_bits(v4i{ (int)f.d[u][0], (int)f.d[u][1], (int)f.d[u][2], (int)f.d[u][3] });
 #pragma unroll
 				for (int cb = 0; cb < 4; cb++)
-					if (cb < pl.ncb) acc[u][cb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bf[cb], acc[u][cb], 0, 0, 0);
+					if (cb < pl.ncb) acc[u][cb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, f.bf[cb], acc[u][cb], 0, 0, 0);
+			}
+		};
+		Operands f0, f1;
+		{
+			read_step(0, f0);
+			for (int ks = 0; ks < Kp; ks += 128) {
+				if (ks + 64 < Kp) read_step(ks + 64, f1);
+				multiply(f0);
+				if (ks + 64 < Kp) {
+					if (ks + 128 < Kp) read_step(ks + 128, f0);
+					multiply(f1);
+				}
 			}
 		}
 		// channel sums: the four k-groups of channel 16 cb + lrow sit in lanes lrow, + 16, + 32, + 48; every byte of
@@ -506,6 +596,9 @@ static bool band_plan(const ConvGeo& g, BandPlan& pl)
 	while (tb > 1 && (int64_t)g.N * ((g.Ho + tb - 1) / tb) < 512) tb--;
 	pl.TB = tb;
 	pl.RH = (tb - 1) * g.sh + g.kh;
+	pl.inv_rw4 = small_div_inverse((unsigned)pl.RW / 4);
+	pl.inv_rh = small_div_inverse((unsigned)pl.RH);
+	pl.inv_cq = small_div_inverse((unsigned)g.Cin / 4);
 	pl.off_w = (unsigned)((pl.RH * pl.RW * pl.PP + 15) & ~15);
 	pl.off_unit = pl.off_w + (unsigned)(pl.ncb * 16 * pl.wpitch);
 	pl.off_kmap = pl.off_unit + (unsigned)(pl.Kp / pl.CP) * 4;
@@ -543,12 +636,16 @@ int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w,
 {
 	ImagePlan pl;
 	if (!image_plan(g, pl)) return -1;
-	// Every workgroup stages the image and all weights again: beyond 16 MB of that in all, the band kernel is ahead where
-	// it applies (16 x 32 x 28 x 28 -> 64 channels 3 x 3, 784 workgroups staging 43 KB each: 26.9 us here, 16.7 us there;
-	// 64 x 32 x 14 x 14 -> 32, 832 workgroups staging 15.5 KB: 15.0 us here, 22.1 us there)
+	// The band kernel, where it applies, is ahead whenever it can permute the weights in registers (3 x 3, 5 x 5 or 7 x 7
+	// windows of a multiple of four channels: 16 x 64 x 14 x 14 -> 64 channels 3 x 3 takes 19.4 us here and 10.0 there,
+	// 1 x 16 x 32 x 32 -> 32 7.0 and 5.4) and otherwise once the workgroups of this kernel, each of which stages the
+	// image and all weights again, would stage more than 16 MB in all (l-ten's quantized MNIST conv2, 10 channels and
+	// 5 x 5: 5.5 us here and 9.7 there for one image, 9.5 and 11.7 for 256, 9.4 MB staged; 512 images go there, 11.6 us)
 	const int64_t staged = (int64_t)g.N * ((g.Ho * g.Wo + CQI_POS - 1) / CQI_POS) * ((int64_t)pl.img16 + (int64_t)pl.ncb * 16 * pl.Kp);
+	const int taps = g.kh * g.kw;
+	const bool permuted = (g.Cin & 3) == 0 && (taps == 9 || taps == 25 || taps == 49) && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
 	BandPlan other;
-	if (staged > (16ll << 20) && band_plan(g, other)) return -1;
+	if ((permuted || staged > (16ll << 20)) && band_plan(g, other)) return -1;
 	const int per_image = (g.Ho * g.Wo + CQI_POS - 1) / CQI_POS;
 	const dim3 grid((unsigned)(g.N * per_image));
 	// windows that cannot reach outside the image need no bounds checks on the way

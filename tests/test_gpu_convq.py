@@ -52,7 +52,10 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (1, 8, 50, 70, 64, 5, 3, 2, 1, 2, 1),       # bands with a row stride of 2, 64 channels, 120 taps
                                  (1, 3, 100, 37, 9, 5, 5, 0, 0, 1, 1),       # rows of 37 bytes: the region is filled byte by byte
                                  (3, 12, 33, 41, 20, 3, 3, 0, 2, 1, 3),      # column stride 3, padding 2 on the columns only
-                                 (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1)])     # 576 taps, 64 channels: several passes of blocks per band
+                                 (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1),      # 576 taps, 64 channels: several passes of blocks per band
+                                 (3, 8, 44, 36, 16, 5, 5, 2, 2, 1, 1),       # bands, 5 x 5 windows of 8 channels (weights permuted in registers, 25 taps)
+                                 (2, 4, 67, 70, 12, 7, 7, 3, 3, 2, 2),       # bands, 7 x 7 windows of 4 channels, stride 2 (49 taps)
+                                 (19, 12, 36, 36, 40, 3, 3, 1, 1, 1, 1)])    # 19 images x 9 bands = 171 workgroups: not a multiple of the 8 XCDs
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -81,9 +84,11 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         Kb = (kh * kw * CPtot + 63) // 64 * 64      # the band kernel reduces over (tap, channel padded to a multiple of CP)
         band = (Cout <= 64 and pw <= 64 and kh * kw * CPtot <= 4096 and
                 kh * RW * PP + ncb * 16 * (Kb + 16) + 4 * (Kb // CP) + 2 * K + 32 <= 65536)
-        # (the small-image kernel only while its workgroups stage at most 16 MB in all, where the band kernel applies)
+        # (where the band kernel applies, the small-image kernel only while its workgroups stage at most 16 MB in all and
+        # the window is none of those whose weights the band kernel permutes in registers)
         staged = N * ((Ho * Wo + 15) // 16) * ((Cin * H * W + 15) // 16 * 16 + ncb * 16 * Kp)
-        small = small and not (band and staged > 16 << 20)
+        permuted = Cin % 4 == 0 and kh * kw in (9, 25, 49)
+        small = small and not (band and (permuted or staged > 16 << 20))
         assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_band" if band else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
         assert np.array_equal(y, want_y), kern
@@ -95,6 +100,14 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
             finally:
                 gpu.set_option("conv_variant", 0)
             assert np.array_equal(acc2, want_acc) and np.array_equal(y2, want_y)
+        if kern == "conv2dq_image" and band:   # and so does the band kernel where both one-launch kernels apply
+            gpu.set_option("conv_variant", 3)
+            try:
+                y3, acc3 = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
+                assert gpu.last_kernel() == "conv2dq_band"
+            finally:
+                gpu.set_option("conv_variant", 0)
+            assert np.array_equal(acc3, want_acc) and np.array_equal(y3, want_y)
     if K > 64:   # l-ten's decomposition image by image (what a workspace beyond 2 GiB falls back to) gives the same bytes
         gpu.set_option("conv_variant", 1)
         try:
