@@ -6,7 +6,7 @@ zero-point correction and the requantize fused in) over one synthetic batch whos
 are already resident in HBM; the layer's weights were converted to int8 once, when the layer
 was set up, as the host-side FullyConnected_q does in to(GPU).  The same step on l-ten's raw
 uint8 weight bytes (lten_hip_quantized_matmul) is timed beside it.  Prints ONE JSON line.  The headline fields describe config 3;
-"configs" adds one record per other benchmark configuration (1, 2, 4, 5) and two for the Conv2d_q
+"configs" adds one record per other benchmark configuration (1, 2, 4, 5) and three for the Conv2d_q
 forward, each with its own roofline figure and the CPU path timed beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-verify] [--no-extra] [--no-vendor] [--copy-calibration MiB]
@@ -486,8 +486,8 @@ def extra_configs(lt, wl, with_cpu):
                    speedup=round(t * 1e3 / ms, 1))
     out.append(rec)
 
-    # ---- the second conv of that network, 10 -> 20 channels 5x5 on the pooled 12x12 maps: 250 taps, the whole-batch
-    # route (patch rows, one int8 GEMM, bias + requantize + NCHW store)
+    # ---- the second conv of that network, 10 -> 20 channels 5x5 on the pooled 12x12 maps: 250 taps, one launch from the
+    # image in LDS
     geo2 = (64, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1)
     xq2 = rng.integers(0, 256, (64, 10, 12, 12), dtype=np.uint8)
     wq2 = rng.integers(0, 256, (20, 10, 5, 5), dtype=np.uint8)
@@ -495,13 +495,37 @@ def extra_configs(lt, wl, with_cpu):
     wsq2 = D(max(int(l.lten_hip_conv2dq_workspace_bytes(*geo2)), 16))
     ms2 = timed(lt, lambda: lt.check(l.lten_hip_conv2dq_forward(*geo2, dxq2.ptr, dwq2.ptr, None, qpq, dyq2.ptr, wsq2.ptr)), 100)
     rec = {"config": "Conv2d_q forward 64x10x12x12 -> 20 ch 5x5 (l-ten's quantized MNIST conv2, batch 64)", "gpu_us": round(ms2 * 1e3, 2),
-           "kernel": lt.last_kernel(), "bound": "launch latency (three launches)", "algorithmic_bytes": xq2.nbytes + wq2.nbytes + 64 * 20 * 8 * 8}
+           "kernel": lt.last_kernel(), "bound": "launch latency", "algorithmic_bytes": xq2.nbytes + wq2.nbytes + 64 * 20 * 8 * 8}
     if with_cpu:
         f2 = (lambda: ob.ref_conv2dq_forward(geo2, xq2, wq2, sc, zp)) if ob.ref() is not None else (lambda: ob.conv2dq_forward(geo2, xq2, wq2, sc, zp, want_acc=False))
         t2 = best_of(f2, 3)
         rec.update(cpu_ms=round(t2 * 1e3, 3), cpu_cores=1, cpu_kind="reference" if ob.ref() is not None else "port",
                    speedup=round(t2 * 1e3 / ms2, 1))
     out.append(rec)
+
+    # ---- a quantized layer of the size of a ResNet block, 64 -> 64 channels 3x3 on 56x56 maps, batch 32: one launch, a band
+    # of output rows per workgroup (checked against the three-launch route of the same library, option conv_variant 2)
+    geo3 = (32, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1)
+    xq3 = rng.integers(0, 256, (32, 64, 56, 56), dtype=np.uint8)
+    wq3 = rng.integers(0, 256, (64, 64, 3, 3), dtype=np.uint8)
+    qpq3 = lt.qparams3([0.02, 0.013, 0.9], [17, 250, 100])
+    dxq3, dwq3, dyq3, dyq3b = D.from_numpy(xq3), D.from_numpy(wq3), D(xq3.size), D(xq3.size)
+    wsq3 = D(max(int(l.lten_hip_conv2dq_workspace_bytes(*geo3)), 16))
+    run3 = lambda dy: lt.check(l.lten_hip_conv2dq_forward(*geo3, dxq3.ptr, dwq3.ptr, None, qpq3, dy.ptr, wsq3.ptr))
+    ms3 = timed(lt, lambda: run3(dyq3), 100)
+    k3 = lt.last_kernel()
+    lt.set_option("conv_variant", 2)
+    try:
+        ms3b = timed(lt, lambda: run3(dyq3b), 20)
+    finally:
+        lt.set_option("conv_variant", 0)
+    same3 = bool(np.array_equal(dyq3.numpy(np.uint8, (xq3.size,)), dyq3b.numpy(np.uint8, (xq3.size,))))
+    ops3 = 2.0 * 32 * 64 * 56 * 56 * 64 * 9
+    out.append({"config": "Conv2d_q forward 32x64x56x56 -> 64 ch 3x3, pad 1 (beyond l-ten's networks)", "gpu_us": round(ms3 * 1e3, 2), "kernel": k3,
+                "three_launch_route_us": round(ms3b * 1e3, 2), "same_bytes_as_three_launch_route": same3,
+                "achieved_TOPs": round(ops3 / ms3 / 1e9, 1), "bound": "LDS reads; memory latency at the start",
+                "algorithmic_bytes": xq3.nbytes + wq3.nbytes + xq3.size})
+    del dxq3, dwq3, dyq3, dyq3b, wsq3
 
     # ---- beyond the five configs: a large fp32 product in the three layouts l-ten's layers use (FullyConnected forward
     # NT, data gradient NN, weight gradient TN), synthetic N(0,1) operands

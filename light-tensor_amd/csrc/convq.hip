@@ -9,8 +9,10 @@
 // launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
-// Longer windows on small images (at most 32 KB an image, at most 64 output channels, at most 1024 taps) also run in
-// one launch: convq_image.hip.  Other longer windows run as three launches for the whole batch (the first also pads the weights): the patches of all output positions as rows of a
+// Longer windows for at most 64 output channels also run in one launch where the weights fit LDS beside the image
+// (small images) or beside the input rows of a band of output rows (any image): convq_image.hip.  Other longer
+// windows run as three launches for the whole batch (the first also pads the weights): the patches of all output
+// positions as rows of a
 // [N * Ho * Wo][K] matrix (K padded to a multiple of 16 with the input zero point, the weights padded alike with
 // theirs, so the padding multiplies to nothing), one int8 GEMM of qgemm.hip with the positions as rows (NT: both
 // operands contiguous in K, the shape its MFMA tiles are built for) into int32 sums, and a pass that adds l-ten's
@@ -274,7 +276,7 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 	}
 
 	// small images with a longer window (l-ten's quantized MNIST conv2): still one launch, no workspace (convq_image.hip;
-	// option "conv_variant" 2 keeps such shapes on the three launches below)
+	// option "conv_variant" 2 keeps such shapes on the three launches below, 3 skips the small-image kernel)
 	if (get_option(OPT_CONV_VARIANT) == 0 || get_option(OPT_CONV_VARIANT) == 3) {
 		int rc = get_option(OPT_CONV_VARIANT) == 3 ? -1 : conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
