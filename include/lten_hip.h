@@ -235,8 +235,8 @@ uint64_t lten_hip_conv2d_dgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
  * byte 0, as in l-ten's column buffer.  bias, when not null, holds Ho*Wo ints and is added per output position:
  * that is what l-ten's call computes (quantized_matmul indexes the bias by GEMM column, l-ten/math_fns.cpp:1470-1473,
  * and the columns of this product are output positions).  workspace: lten_hip_conv2dq_workspace_bytes device
- * bytes, 16-byte aligned.  Windows of at most 64 taps, and longer windows for at most 64 output channels whose
- * weights and a few input rows fit 64 KB of LDS, run in one launch and leave it untouched.  Other windows use it: the
+ * bytes, 16-byte aligned.  Windows of at most 64 taps, and longer windows whose weights (of 32 output channels at
+ * least) and a few input rows fit 64 KB of LDS, run in one launch and leave it untouched.  Other windows use it: the
  * patches of all output positions of the batch as rows
  * of a matrix, the padded weights, the int32 sums of one int8 GEMM over the whole batch and its zero-point terms;
  * where that would exceed 2 GiB, the column buffer of one image (l-ten's decomposition, image by image). */

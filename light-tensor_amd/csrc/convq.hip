@@ -9,8 +9,9 @@
 // launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
-// Longer windows for at most 64 output channels also run in one launch where the weights fit LDS beside the image
-// (small images) or beside the input rows of a band of output rows (any image): convq_image.hip.  Other longer
+// Longer windows also run in one launch where the weights fit LDS beside the image (small images, at most 64 output
+// channels) or, a block of output channels at a time, beside the input rows of a band of output rows (any image):
+// convq_image.hip.  Other longer
 // windows run as three launches for the whole batch (the first also pads the weights): the patches of all output
 // positions as rows of a
 // [N * Ho * Wo][K] matrix (K padded to a multiple of 16 with the input zero point, the weights padded alike with
@@ -280,7 +281,7 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 	if (get_option(OPT_CONV_VARIANT) == 0 || get_option(OPT_CONV_VARIANT) == 3) {
 		int rc = get_option(OPT_CONV_VARIANT) == 3 ? -1 : conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
-		// larger images: a band of output rows per workgroup, the input rows it needs in LDS (at most 64 output channels)
+		// larger images or more channels: a band of output rows and a block of output channels per workgroup, the input rows it needs in LDS
 		rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
 	}

@@ -199,8 +199,9 @@ __global__ __launch_bounds__(256) void conv2dq_image_kernel(ConvGeo g, const uin
 	}
 }
 
-// The same idea for images of any size: a workgroup takes a band of TB output rows of one image and stages the input rows
-// the band's windows reach, pixel-major with the channels innermost: [RH rows][RW columns][PP bytes], byte ci of a
+// The same idea for images of any size and any number of output channels: a workgroup takes a band of TB output rows of
+// one image and a block of up to 64 output channels (the grid's second axis) and stages the input rows the band's
+// windows reach, pixel-major with the channels innermost: [RH rows][RW columns][PP bytes], byte ci of a
 // pixel its channel ci, channels padded with zeros to a multiple of CP (4, 8 or 16 by the channel count), the padding
 // written out as zero pixels (PL zero columns on the left, rows above and below the image as zero rows).  The
 // reduction runs in the order (tap, channel) instead of l-ten's (channel, tap), the weights being staged in the same
@@ -272,6 +273,9 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 	const int bid = xcd * (nb >> 3) + min(xcd, nb & 7) + ((int)blockIdx.x >> 3);
 	const int n = bid / bands_per_image, hb = (bid % bands_per_image) * pl.TB;
 	const int rows_here = min(pl.TB, g.Ho - hb);
+	// grid row: this workgroup's block of 16 ncb output channels
+	const int co0 = (int)blockIdx.y * pl.ncb * 16, cout_here = min(g.Cout - co0, pl.ncb * 16);
+	w += (int64_t)co0 * (g.Cin * g.kh * g.kw);
 	const int rgn_y0 = hb * g.sh - g.ph;  // image row of region row 0
 	const uint8_t* xn = x + (int64_t)n * g.Cin * g.H * g.W;
 
@@ -343,9 +347,9 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 	if (w_taps) {
 		for (int idx = tid; idx < pl.ncb * pl.wpitch; idx += 256) reinterpret_cast<v4i*>(s_w)[idx] = v4i{ 0, 0, 0, 0 };
 		__syncthreads();
-		if (T == 9) band_stage_weights<9>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
-		else if (T == 25) band_stage_weights<25>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
-		else band_stage_weights<49>(w, s_w, g.Cout, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		if (T == 9) band_stage_weights<9>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		else if (T == 25) band_stage_weights<25>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		else band_stage_weights<49>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
 	} else if (w_fast) {
 		// where byte k of a weight row (l-ten's order: channel k / T, tap k % T) goes in the new order: worked out once, the
 		// divisions by T for every byte had been most of the staging time
@@ -357,7 +361,7 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 		for (int idx = tid; idx < pl.ncb * pl.wpitch; idx += 256) reinterpret_cast<v4i*>(s_w)[idx] = v4i{ 0, 0, 0, 0 };
 		__syncthreads();
 		// (eight loads in flight per thread: one load, then its four byte writes, made a chain of round trips to the L2)
-		const int total = g.Cout * (K / 4);   // the weights are one run of Cout * K bytes: dword number idx holds bytes 4 idx .. + 3
+		const int total = cout_here * (K / 4);   // the block's weights are one run of cout_here * K bytes: dword number idx holds bytes 4 idx .. + 3
 		constexpr int U = 8;
 		// this thread's dwords are 256 apart: (row, byte in the row) advance by (1024 / K, 1024 % K), no division per dword
 		const int step_co = 1024 / K, step_k = 1024 - step_co * K;
@@ -387,7 +391,7 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 			const int co = idx / kd, k0 = (idx - co * kd) * 4;
 			const int t = k0 / CPtot, c0 = k0 - t * CPtot;
 			uint32_t v = 0;
-			if (co < g.Cout && t < T) {
+			if (co < cout_here && t < T) {
 				const uint8_t* wr = w + (int64_t)co * K + t;
 #pragma unroll
 				for (int b = 0; b < 4; b++) {
@@ -524,8 +528,8 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 #pragma unroll
 			for (int cb = 0; cb < 4; cb++) {
 				const int co = cb * 16 + lrow;
-				if (cb >= pl.ncb || co >= g.Cout) continue;
-				const int64_t o = ((int64_t)n * g.Cout + co) * HW + hb * g.Wo + p0;
+				if (cb >= pl.ncb || co >= cout_here) continue;
+				const int64_t o = ((int64_t)n * g.Cout + co0 + co) * HW + hb * g.Wo + p0;
 				if (OUT == Q_OUT_ACC) {
 #pragma unroll
 					for (int e = 0; e < 4; e++)
@@ -566,12 +570,13 @@ static bool image_plan(const ConvGeo& g, ImagePlan& pl)
 	return pl.bytes <= 64 * 1024;
 }
 
-// The band kernel's plan: the tallest band whose region, the weights and the unit table fit 64 KB of LDS, shortened
-// while that leaves the chip with fewer than two workgroups per CU.
+// The band kernel's plan: blocks of 64 output channels per workgroup (32 or 16 where the weights of 64 would not leave
+// room for one window's height of input rows), the tallest band whose region fits 64 KB of LDS beside the weights
+// and the tables, shortened while that leaves the chip with fewer than two workgroups per CU.
 static bool band_plan(const ConvGeo& g, BandPlan& pl)
 {
 	const int64_t T = (int64_t)g.kh * g.kw, K = (int64_t)g.Cin * T;
-	if (K <= 64 || g.Cout > 64 || g.pw > 64 || g.Cin > 1024) return false;
+	if (K <= 64 || g.pw > 64 || g.Cin > 1024 || g.Cout > 16 * 65535) return false;
 	pl.CP = g.Cin <= 4 ? 4 : g.Cin <= 8 ? 8 : 16;
 	pl.CPtot = (g.Cin + pl.CP - 1) / pl.CP * pl.CP;
 	pl.PP = pl.CPtot + (pl.CPtot % 32 == 0 ? 16 : 0);  // pixels 32 or 64 bytes apart would meet on the same LDS banks
@@ -579,21 +584,30 @@ static bool band_plan(const ConvGeo& g, BandPlan& pl)
 	const int64_t kprime = T * pl.CPtot;
 	if (kprime > 4096) return false;
 	pl.Kp = (int)((kprime + 63) & ~63ll);
-	pl.ncb = (g.Cout + 15) / 16;
 	pl.wpitch = pl.Kp + CQI_PAD;
 	pl.PL = (g.pw + 3) & ~3;
 	// the rightmost byte a window reaches is column (Wo - 1) sw + kw - 1 - pw of the image
 	const int reach = (g.Wo - 1) * g.sw + g.kw - g.pw;   // image columns 0 .. reach - 1 (beyond W: padding)
 	pl.RW = (pl.PL + (reach > g.W ? reach : g.W) + 3) & ~3;
-	const int64_t fixed = (int64_t)pl.ncb * 16 * pl.wpitch + (int64_t)(pl.Kp / pl.CP) * 4 + 2 * K + 32;
+	const int all_cb = (g.Cout + 15) / 16;
 	int tb = 0;
-	for (int t = 1; t <= g.Ho && t <= 64; t++) {
-		const int64_t rh = (int64_t)(t - 1) * g.sh + g.kh;
-		if (rh * pl.RW * pl.PP + fixed > 64 * 1024) break;
-		tb = t;
+	int64_t fixed = 0;
+	for (int ncb = all_cb < 4 ? all_cb : 4; ncb >= 1 && tb == 0; ncb = ncb == 3 ? 2 : ncb / 2) {
+		pl.ncb = ncb;
+		fixed = (int64_t)ncb * 16 * pl.wpitch + (int64_t)(pl.Kp / pl.CP) * 4 + 2 * K + 32;
+		for (int t = 1; t <= g.Ho && t <= 64; t++) {
+			const int64_t rh = (int64_t)(t - 1) * g.sh + g.kh;
+			if (rh * pl.RW * pl.PP + fixed > 64 * 1024) break;
+			tb = t;
+		}
 	}
 	if (tb == 0) return false;
-	while (tb > 1 && (int64_t)g.N * ((g.Ho + tb - 1) / tb) < 512) tb--;
+	// 16 channels per workgroup against many blocks of them: every block stages the region again and an operand read
+	// from it feeds one MFMA; the patch-row route with its GEMM is level there (8 x 256 x 14 x 14 -> 256 channels: 42 us
+	// both ways) and ahead beyond
+	if (pl.ncb == 1 && all_cb > 2) return false;
+	const int64_t cblocks = (all_cb + pl.ncb - 1) / pl.ncb;
+	while (tb > 1 && (int64_t)g.N * ((g.Ho + tb - 1) / tb) * cblocks < 512) tb--;
 	pl.TB = tb;
 	pl.RH = (tb - 1) * g.sh + g.kh;
 	pl.inv_rw4 = small_div_inverse((unsigned)pl.RW / 4);
@@ -613,7 +627,8 @@ int conv2dq_band_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, 
 	BandPlan pl;
 	if (!band_plan(g, pl)) return -1;
 	const int per_image = (g.Ho + pl.TB - 1) / pl.TB;
-	const dim3 grid((unsigned)(g.N * per_image));
+	const int all_cb = (g.Cout + 15) / 16;
+	const dim3 grid((unsigned)(g.N * per_image), (unsigned)((all_cb + pl.ncb - 1) / pl.ncb));
 	set_kernel_name("conv2dq_band");
 	const int out = out_acc ? Q_OUT_ACC : (mult == mult && (mult < 0 ? -mult : mult) <= 0.99f) ? Q_OUT_U8_FAST : Q_OUT_U8_EXACT;
 #define LTEN_LAUNCH(OUTV, CPV) conv2dq_band_kernel<OUTV, CPV><<<grid, dim3(256), pl.bytes, stream()>>>(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, pl, per_image)

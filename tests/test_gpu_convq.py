@@ -55,7 +55,11 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (1, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1),      # 576 taps, 64 channels: several passes of blocks per band
                                  (3, 8, 44, 36, 16, 5, 5, 2, 2, 1, 1),       # bands, 5 x 5 windows of 8 channels (weights permuted in registers, 25 taps)
                                  (2, 4, 67, 70, 12, 7, 7, 3, 3, 2, 2),       # bands, 7 x 7 windows of 4 channels, stride 2 (49 taps)
-                                 (19, 12, 36, 36, 40, 3, 3, 1, 1, 1, 1)])    # 19 images x 9 bands = 171 workgroups: not a multiple of the 8 XCDs
+                                 (19, 12, 36, 36, 40, 3, 3, 1, 1, 1, 1),     # 19 images x 9 bands = 171 workgroups: not a multiple of the 8 XCDs
+                                 (2, 16, 20, 24, 80, 3, 3, 1, 1, 1, 1),      # 80 channels: a block of 64 and one of 16 per band
+                                 (1, 128, 14, 14, 136, 3, 3, 1, 1, 1, 1),    # 1152 taps: weights of 32 channels at a time fit LDS, 5 blocks
+                                 (1, 400, 9, 9, 40, 3, 3, 0, 0, 1, 1),       # 3600 taps: the weights of 32 channels do not fit, three launches
+                                 (1, 200, 9, 9, 30, 3, 3, 0, 0, 1, 1)])      # 1800 taps, 30 channels: two blocks of 16 channels
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -82,8 +86,10 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         CPtot = (Cin + CP - 1) // CP * CP
         PP = CPtot + (16 if CPtot % 32 == 0 else 0)
         Kb = (kh * kw * CPtot + 63) // 64 * 64      # the band kernel reduces over (tap, channel padded to a multiple of CP)
-        band = (Cout <= 64 and pw <= 64 and kh * kw * CPtot <= 4096 and
-                kh * RW * PP + ncb * 16 * (Kb + 16) + 4 * (Kb // CP) + 2 * K + 32 <= 65536)
+        # (blocks of 64 output channels per workgroup, or 32 where the weights of 64 leave no room for one window's rows; 16
+        # only for layers of at most 32 channels)
+        band = (pw <= 64 and kh * kw * CPtot <= 4096 and
+                kh * RW * PP + (1 if ncb <= 2 else 2) * 16 * (Kb + 16) + 4 * (Kb // CP) + 2 * K + 32 <= 65536)
         # (where the band kernel applies, the small-image kernel only while its workgroups stage at most 16 MB in all and
         # the window is none of those whose weights the band kernel permutes in registers)
         staged = N * ((Ho * Wo + 15) // 16) * ((Cin * H * W + 15) // 16 * 16 + ncb * 16 * Kp)
