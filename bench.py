@@ -295,7 +295,7 @@ def extra_configs(lt, wl, with_cpu):
                                                 tmpg[i].ptr, gWs[i].ptr, gbs_[i].ptr))
             if i > 0:
                 lt.check(l.lten_hip_relu_backward_f32(grads[i].ptr, tmpg[i].ptr, pre[i].ptr, B_ * sizes[i]))
-    def mlp_step_fused():
+    def mlp_step_fused(input_gradient=True):
         for i in range(3):
             if i < 2:
                 lt.check(l.lten_hip_fc_forward_relu_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, dbs[i].ptr, pre[i + 1].ptr, acts[i + 1].ptr))
@@ -308,9 +308,15 @@ def extra_configs(lt, wl, with_cpu):
                 lt.check(l.lten_hip_fc_backward_relu_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, grads[i + 1].ptr, pre[i].ptr,
                                                          grads[i].ptr, gWs[i].ptr, gbs_[i].ptr))
             else:
-                lt.check(l.lten_hip_fc_backward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, grads[i + 1].ptr, tmpg[i].ptr, gWs[i].ptr, gbs_[i].ptr))
+                lt.check(l.lten_hip_fc_backward_f32(B_, sizes[i], sizes[i + 1], acts[i].ptr, dWs[i].ptr, grads[i + 1].ptr,
+                                                    tmpg[i].ptr if input_gradient else None, gWs[i].ptr, gbs_[i].ptr))
     unfused_ms = timed(lt, mlp_step, 100)
     ms = timed(lt, mlp_step_fused, 100)
+    # l-ten's backward pass also works out the gradient with respect to the network's input (its traversal calls
+    # fc_backward for every child, l-ten/backprop.cpp:312-349) and drops it when the input tensor takes no gradient;
+    # the step without that product is timed beside the one above
+    no_dx_ms = timed(lt, lambda: mlp_step_fused(False), 100)
+    no_dx_kernel = lt.last_kernel()
     # The same launches recorded once and replayed with one submit.  Not under a profiler: rocprofv3's interception of
     # graph launches segfaulted in its own code in about half of the runs of this loop on this image.
     graph_ms = None
@@ -325,6 +331,7 @@ def extra_configs(lt, wl, with_cpu):
                      "dX and dW of a layer in one, log_softmax, the loss and its gradient inside the last layer's backward launch)",
            "gpu_us": round(ms * 1e3, 2), "unfused_entry_points_us": round(unfused_ms * 1e3, 2), "unfused_graph_replay_us": None if graph_ms is None else round(graph_ms * 1e3, 2),
            "gflop_per_step": round(flops / 1e9, 3),
+           "without_the_gradient_of_the_input_us": round(no_dx_ms * 1e3, 2), "without_the_gradient_of_the_input_last_kernel": no_dx_kernel,
            "roofline": {"bound": "mfma", "achieved": round(tf, 2), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                         "frac": round(tf / FP32_MFMA_PEAK_TFLOPS, 4)},
            "note": "six dependent launches; the launch-to-launch latency (3 to 4.4 us from box to box for a kernel that does nothing), not the MFMA rate, sets this time (GEMM flops "
