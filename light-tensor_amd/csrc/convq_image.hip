@@ -338,16 +338,17 @@ __global__ __launch_bounds__(256, 2) void conv2dq_band_kernel(ConvGeo g, const u
 	}
 	// ---- weights in the order (tap, channel), into the signed domain; rows past Cout, channels past Cin and units past
 	// the last tap hold signed zeros.  Three ways, by what the shape allows: permuted in registers (band_stage_weights:
-	// 3 x 3, 5 x 5 and 7 x 7 windows of a multiple of four channels); else, where the weight rows keep dword alignment,
+	// 1 x 1, 3 x 3, 5 x 5 and 7 x 7 windows of a multiple of four channels); else, where the weight rows keep dword alignment,
 	// read along memory, a dword of four consecutive (channel, tap) bytes per thread, and scattered byte by byte into
 	// the new order; else a thread builds a dword of the new order from four bytes it gathers.  On 4 x 64 x 56 x 56 ->
 	// 64 channels 3 x 3 the three take 3.7, 8 and 10.8 us of the kernel's time.
 	const bool w_fast = (K & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
-	const bool w_taps = w_fast && (g.Cin & 3) == 0 && (T == 9 || T == 25 || T == 49);
+	const bool w_taps = w_fast && (g.Cin & 3) == 0 && (T == 1 || T == 9 || T == 25 || T == 49);
 	if (w_taps) {
 		for (int idx = tid; idx < pl.ncb * pl.wpitch; idx += 256) reinterpret_cast<v4i*>(s_w)[idx] = v4i{ 0, 0, 0, 0 };
 		__syncthreads();
-		if (T == 9) band_stage_weights<9>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
+		if (T == 1) band_stage_weights<1>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);  // a plain copy: one tap, the orders agree
+		else if (T == 9) band_stage_weights<9>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
 		else if (T == 25) band_stage_weights<25>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
 		else band_stage_weights<49>(w, s_w, cout_here, g.Cin, CPtot, pl.wpitch, tid, pl.inv_cq);
 	} else if (w_fast) {
@@ -651,14 +652,14 @@ int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w,
 {
 	ImagePlan pl;
 	if (!image_plan(g, pl)) return -1;
-	// The band kernel, where it applies, is ahead whenever it can permute the weights in registers (3 x 3, 5 x 5 or 7 x 7
-	// windows of a multiple of four channels: 16 x 64 x 14 x 14 -> 64 channels 3 x 3 takes 19.4 us here and 10.0 there,
+	// The band kernel, where it applies, is ahead whenever it can permute the weights in registers (1 x 1, 3 x 3, 5 x 5 or
+	// 7 x 7 windows of a multiple of four channels: 16 x 64 x 14 x 14 -> 64 channels 3 x 3 takes 19.4 us here and 10.0 there,
 	// 1 x 16 x 32 x 32 -> 32 7.0 and 5.4) and otherwise once the workgroups of this kernel, each of which stages the
 	// image and all weights again, would stage more than 16 MB in all (l-ten's quantized MNIST conv2, 10 channels and
 	// 5 x 5: 5.5 us here and 9.7 there for one image, 9.5 and 11.7 for 256, 9.4 MB staged; 512 images go there, 11.6 us)
 	const int64_t staged = (int64_t)g.N * ((g.Ho * g.Wo + CQI_POS - 1) / CQI_POS) * ((int64_t)pl.img16 + (int64_t)pl.ncb * 16 * pl.Kp);
 	const int taps = g.kh * g.kw;
-	const bool permuted = (g.Cin & 3) == 0 && (taps == 9 || taps == 25 || taps == 49) && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
+	const bool permuted = (g.Cin & 3) == 0 && (taps == 1 || taps == 9 || taps == 25 || taps == 49) && (reinterpret_cast<uintptr_t>(w) & 3) == 0;
 	BandPlan other;
 	if ((permuted || staged > (16ll << 20)) && band_plan(g, other)) return -1;
 	const int per_image = (g.Ho * g.Wo + CQI_POS - 1) / CQI_POS;

@@ -59,7 +59,9 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (2, 16, 20, 24, 80, 3, 3, 1, 1, 1, 1),      # 80 channels: a block of 64 and one of 16 per band
                                  (1, 128, 14, 14, 136, 3, 3, 1, 1, 1, 1),    # 1152 taps: weights of 32 channels at a time fit LDS, 5 blocks
                                  (1, 400, 9, 9, 40, 3, 3, 0, 0, 1, 1),       # 3600 taps: the weights of 32 channels do not fit, three launches
-                                 (1, 200, 9, 9, 30, 3, 3, 0, 0, 1, 1)])      # 1800 taps, 30 channels: two blocks of 16 channels
+                                 (1, 200, 9, 9, 30, 3, 3, 0, 0, 1, 1),       # 1800 taps, 30 channels: two blocks of 16 channels
+                                 (3, 96, 20, 20, 72, 1, 1, 0, 0, 1, 1),      # a 1 x 1 layer of 96 channels: the weights are copied as they lie
+                                 (2, 68, 21, 22, 40, 1, 1, 1, 0, 2, 1)])     # 1 x 1 with a row stride of 2 and padded rows
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -93,7 +95,7 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         # (where the band kernel applies, the small-image kernel only while its workgroups stage at most 16 MB in all and
         # the window is none of those whose weights the band kernel permutes in registers)
         staged = N * ((Ho * Wo + 15) // 16) * ((Cin * H * W + 15) // 16 * 16 + ncb * 16 * Kp)
-        permuted = Cin % 4 == 0 and kh * kw in (9, 25, 49)
+        permuted = Cin % 4 == 0 and kh * kw in (1, 9, 25, 49)
         small = small and not (band and (permuted or staged > 16 << 20))
         assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_band" if band else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
