@@ -147,14 +147,20 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
 /* Weights of a FullyConnected_q layer never change between forward calls (l-ten keeps them in the layer,
  * l-ten/fully_connected.cpp:301-303, and fills them once from a checkpoint).  lten_hip_fcq_prepare_weights, to be
  * called once when the layer moves to the GPU, turns the layer's uint8 weight bytes W[out_features][in_features]
- * into the int8 values w - 128 the matrix cores multiply (both buffers 16-byte aligned; in place when W_prepared ==
- * W) and, when weight_sums is not NULL, leaves each weight row's byte sum in weight_sums[out_features] (16-byte
+ * into the int8 values w - 128 the matrix cores multiply, with every row on a 16-byte boundary: W_prepared holds
+ * out_features rows of (in_features + 15) / 16 * 16 bytes, the bytes past in_features zero (both buffers 16-byte
+ * aligned; in place when W_prepared == W and in_features is a multiple of 16, else the buffers may not overlap)
+ * and, when weight_sums is not NULL, leaves each weight row's byte sum in weight_sums[out_features] (16-byte
  * aligned): the sums of the zero-point correction that quantized_matmul recomputes on every call
  * (l-ten/math_fns.cpp:1362-1369).  lten_hip_fcq_forward_prepared is lten_hip_fcq_forward on such weights and
  * returns bit-identical outputs.  For every shape the direct-to-LDS tiles take (in_features % 16 == 0 and >= 128,
  * out_features % 4 == 0, more than 32 rows) it is a single launch whatever the zero points and the bias: the
  * column term comes from weight_sums, the activation rows' byte sums (needed when the weight zero point is not 128)
- * are added up from the operand fragments inside the GEMM.  qparams are the layer's unchanged (the weight zero
+ * are added up from the operand fragments inside the GEMM.  When in_features is no multiple of 16 the activations
+ * are first copied into rows of that length in memory the library owns (one more launch; the memory is allocated by
+ * the first such call and grows with later ones, which cannot happen while a launch graph is being recorded), and
+ * lten_hip_fcq_forward and lten_hip_quantized_matmul(0, 1, ...) copy both operands that way on every call.
+ * qparams are the layer's unchanged (the weight zero
  * point still refers to the uint8 representation).  workspace as for lten_hip_fcq_forward; only shapes that fall to
  * the general kernels use it.  No counterpart in l-ten, whose quantized layers are CPU-only. */
 int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t out_features, uint64_t in_features,

@@ -82,7 +82,7 @@ __global__ __launch_bounds__(WAVES * 64) void qdirect_kernel(QProblem p, const i
 	if (n >= p.N) return;
 	// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 	//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-	const int base = coef_b * tsb + p.K * coef_a * coef_b + (bias ? bias[n] : 0);
+	const int base = coef_b * tsb + (p.K - p.k_pad) * coef_a * coef_b + (bias ? bias[n] : 0);
 #pragma unroll
 	for (int e = 0; e < 4; e++) {
 		const int m = m0 + lgrp * 4 + e;

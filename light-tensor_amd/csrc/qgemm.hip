@@ -384,9 +384,84 @@ struct RunScratch {
 	SplitScratch split;
 };
 
+// Rows of any length and alignment to rows of Kp bytes (a multiple of 16, so 16-byte aligned where dst is): one thread
+// per 16 bytes of dst; bytes K .. Kp - 1 of a row become 128, the byte that reads as zero once the operands are
+// taken as a - 128.  Rows 0 .. rows_a - 1 come from src_a, the others from src_b (the two operands of one product in
+// one launch).  A dword of a row is put together from the two aligned dwords that hold it, whatever the row's
+// alignment; only the dword that straddles the row's end is read byte by byte.
+__global__ __launch_bounds__(256) void qgemm_pad_rows_kernel(const uint8_t* __restrict__ src_a, uint8_t* __restrict__ dst_a, uint64_t rows_a,
+                                                             const uint8_t* __restrict__ src_b, uint8_t* __restrict__ dst_b, uint64_t rows_b, int K, int Kp)
+{
+	const uint64_t cpr = (uint64_t)Kp / 16, total = (rows_a + rows_b) * cpr;
+	for (uint64_t c = (uint64_t)blockIdx.x * 256 + threadIdx.x; c < total; c += (uint64_t)gridDim.x * 256) {
+		uint64_t row = c / cpr;
+		const int k0 = (int)(c - row * cpr) * 16;
+		const uint8_t* src = src_a;
+		uint8_t* dst = dst_a;
+		if (row >= rows_a) {
+			row -= rows_a;
+			src = src_b;
+			dst = dst_b;
+		}
+		const uint8_t* r = src + row * (uint64_t)K;
+		uint32_t v[4];
+#pragma unroll
+		for (int j = 0; j < 4; j++) {
+			const int k = k0 + 4 * j;
+			v[j] = 0x80808080u;
+			if (k + 4 <= K) {
+				const uintptr_t a = reinterpret_cast<uintptr_t>(r + k);
+				const uint32_t* al = reinterpret_cast<const uint32_t*>(a & ~(uintptr_t)3);
+				const unsigned sh = (unsigned)(a & 3);
+				const uint32_t lo = al[0], hi = al[sh ? 1 : 0];  // all four bytes lie inside the row, so both dwords hold some of them
+				v[j] = __builtin_amdgcn_alignbyte(hi, lo, sh);
+			} else if (k < K) {
+#pragma unroll
+				for (int b = 0; b < 3; b++)
+					if (k + b < K) v[j] = (v[j] & ~(0xFFu << (8 * b))) | ((uint32_t)r[k + b] << (8 * b));
+			}
+		}
+		*reinterpret_cast<v4i*>(dst + row * (uint64_t)Kp + k0) = v4i{ (int)v[0], (int)v[1], (int)v[2], (int)v[3] };
+	}
+}
+
+// Where the padded copies live: owned by the library, one block per device, grown when a call needs more (never while
+// a launch graph is being recorded), kept until the process ends.  One stream uses it at a time, as everything else
+// in this library; work queued on that stream may still read the old block when it has to grow, hence the wait.
+struct PadScratch {
+	uint8_t* base;
+	uint64_t bytes;
+};
+static PadScratch g_pad[8] = {};
+
+static uint8_t* pad_scratch(uint64_t bytes)
+{
+	int dev = -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
+	PadScratch& ps = g_pad[dev];
+	if (ps.bytes >= bytes) return ps.base;
+	if (capturing()) return nullptr;
+	if (ps.base != nullptr) {
+		if (hipStreamSynchronize(stream()) != hipSuccess) return nullptr;
+		(void)hipFree(ps.base);
+		ps.base = nullptr;
+		ps.bytes = 0;
+	}
+	const uint64_t want = (bytes + (bytes >> 2) + (2u << 20)) & ~((2ull << 20) - 1);  // a quarter more, whole 2 MB pages
+	void* ptr = nullptr;
+	if (hipMalloc(&ptr, want) != hipSuccess) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	ps.base = static_cast<uint8_t*>(ptr);
+	ps.bytes = want;
+	return ps.base;
+}
+
+// k_pad: the last k_pad bytes of every row of A and B are padding (QProblem::k_pad); the call that pads passes it
 static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A, const uint8_t* B, void* C,
                      int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace,
-                     bool weights_prepared = false, const RunScratch* scratch = nullptr, const int32_t* weight_sums = nullptr)
+                     bool weights_prepared = false, const RunScratch* scratch = nullptr, const int32_t* weight_sums = nullptr, int k_pad = 0)
 {
 	LTEN_HIP_REQUIRE(qp != nullptr, "quantized_matmul: qparams is null");
 	if (M == 0 || N == 0) return 0;
@@ -396,6 +471,30 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	// it overflows and there is nothing defined to match.
 	LTEN_HIP_REQUIRE(K * 65025ull < (1ull << 31), "quantized_matmul: K=%llu overflows the reference's int accumulator",
 	                 (unsigned long long)K);
+
+	// Rows that are no multiple of 16 bytes long (a layer of 1000 or 50 inputs) fit none of the kernels that load 16
+	// bytes at a time, which is all but the guarded one: 4096 x 4096 x 4100 took 2.4 ms there where K = 4096 takes 56 us,
+	// one row against 4096 x 4100 weights 197 us against 5.  Such products in the layout the layers use (both operands
+	// contiguous in K) run on copies with padded rows instead: one more launch, then the kernels of the padded
+	// shape.  Prepared weights are padded already (lten_hip_fcq_prepare_weights), so only the activations are copied.
+	// The entry point that may not allocate keeps the guarded kernel, and so do products too small to care.
+	if (k_pad == 0 && !tA && tB && (K & 15) != 0 && scratch == nullptr && (weights_prepared || M * N * K >= (1ull << 20))) {
+		const uint64_t Kp = (K + 15) & ~15ull;
+		const uint64_t bytes_a = M * Kp, bytes_b = weights_prepared ? 0 : N * Kp;
+		uint8_t* buf = pad_scratch(bytes_a + bytes_b);
+		LTEN_HIP_REQUIRE(buf != nullptr || !weights_prepared,
+		                 "quantized_matmul: no memory for the padded copy of the activations (in_features = %llu is no multiple of 16; while a "
+		                 "launch graph is being recorded the copy's memory cannot be allocated: run the call once before recording)",
+		                 (unsigned long long)K);
+		if (buf != nullptr) {
+			const uint64_t chunks = (M + (weights_prepared ? 0 : N)) * (Kp / 16);
+			const unsigned blocks = (unsigned)std::min<uint64_t>(ceil_div(chunks, 256), 16384);
+			qgemm_pad_rows_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(A, buf, M, B, buf + bytes_a, weights_prepared ? 0 : N, (int)K, (int)Kp);
+			LTEN_HIP_LAUNCH_CHECK();
+			return qgemm_run(0, 1, M, N, Kp, buf, weights_prepared ? B : buf + bytes_a, C, out_acc, qp, bias, workspace, weights_prepared, nullptr,
+			                 weight_sums, (int)(Kp - K));
+		}
+	}
 
 	const int zpA = qp[0].zero_point, zpB = qp[1].zero_point;
 	QProblem p;
@@ -410,7 +509,10 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	p.M = (int)M;
 	p.N = (int)N;
 	p.K = (int)K;
-	p.konst = (int32_t)((uint32_t)K * (uint32_t)(zpA * zpB - 16384));
+	// With k_pad padding bytes of 128 in every row, byte sums over whole rows hold 128 k_pad too much each: taken off
+	// here once for both sum terms (wrapping arithmetic, as the accumulators)
+	p.k_pad = k_pad;
+	p.konst = (int32_t)((uint32_t)(K - k_pad) * (uint32_t)(zpA * zpB - 16384) - (uint32_t)(128 * k_pad) * (uint32_t)((128 - zpB) + (128 - zpA)));
 	// l-ten/math_fns.cpp:1436, left to right in fp32
 	volatile float ab = qp[0].scale * qp[1].scale;
 	p.mult = ab / qp[2].scale;
@@ -474,6 +576,7 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		f.bias = bias;
 		f.coef_a = coef_a;
 		f.coef_b = coef_b;
+		f.konst = (int32_t)((uint32_t)p.konst + (uint32_t)(128 * k_pad) * (uint32_t)coef_b);  // the kept weight sums count no padding
 		if (qgemm_dispatch(f, out, scratch ? &scratch->split : nullptr, true) == 0) return 0;
 	}
 	if (coef_a != 0 || coef_b != 0 || bias != nullptr) {
@@ -500,15 +603,16 @@ __global__ __launch_bounds__(256) void fcq_prepare_weights_kernel(const v4i* __r
 }
 
 // The same conversion row by row, with each weight row's byte sum (of the uint8 values, as l-ten/math_fns.cpp:1364-1369
-// adds them up on every call) kept in sums[row]: one wavefront per row.
+// adds them up on every call) kept in sums[row] (when not null): one wavefront per row.  Rows of dst are dst_cols
+// bytes apart (cols rounded up to a multiple of 16); the bytes past cols become 0, the int8 form of the byte 128.
 __global__ __launch_bounds__(256) void fcq_prepare_weights_sums_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int32_t* __restrict__ sums,
-                                                                       uint64_t rows, uint64_t cols, int vec_ok)
+                                                                       uint64_t rows, uint64_t cols, uint64_t dst_cols, int vec_ok)
 {
 	const int lane = threadIdx.x & 63;
 	const uint64_t row = (uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
 	if (row >= rows) return;
 	const uint8_t* r = src + row * cols;
-	uint8_t* w = dst + row * cols;
+	uint8_t* w = dst + row * dst_cols;
 	unsigned sum = 0;
 	uint64_t k = 0;
 	if (vec_ok) {
@@ -528,9 +632,10 @@ __global__ __launch_bounds__(256) void fcq_prepare_weights_sums_kernel(const uin
 		sum += b;
 		w[kk] = b ^ 0x80;
 	}
+	if (cols + lane < dst_cols) w[cols + lane] = 0;  // fewer than 16 bytes of padding
 #pragma unroll
 	for (int off = 32; off > 0; off >>= 1) sum += __shfl_down(sum, off, 64);
-	if (lane == 0) sums[row] = (int32_t)sum;
+	if (lane == 0 && sums != nullptr) sums[row] = (int32_t)sum;
 }
 
 // Scratch of lten_hip_fcq_forward_static: device memory that exists from the moment the library is loaded, so the
@@ -613,11 +718,20 @@ int lten_hip_fcq_prepare_weights(const uint8_t* W, uint8_t* W_prepared, uint64_t
 	LTEN_HIP_REQUIRE(W && W_prepared, "lten_hip_fcq_prepare_weights: null pointer");
 	LTEN_HIP_REQUIRE(((reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(W_prepared)) & 15) == 0,
 	                 "lten_hip_fcq_prepare_weights: both buffers must be 16-byte aligned");
-	if (weight_sums != nullptr) {
+	// rows of the prepared form start on 16-byte boundaries: in_features rounded up to a multiple of 16 bytes apart
+	const uint64_t padded = (in_features + 15) & ~15ull;
+	if (padded != in_features) {
+		const uint8_t* w_end = W + count;
+		const uint8_t* p_end = W_prepared + out_features * padded;
+		LTEN_HIP_REQUIRE(w_end <= W_prepared || p_end <= W,
+		                 "lten_hip_fcq_prepare_weights: in_features = %llu is no multiple of 16, so the prepared rows are padded to %llu bytes and "
+		                 "the two buffers must not overlap", (unsigned long long)in_features, (unsigned long long)padded);
+	}
+	if (weight_sums != nullptr || padded != in_features) {
 		LTEN_HIP_REQUIRE((reinterpret_cast<uintptr_t>(weight_sums) & 15) == 0, "lten_hip_fcq_prepare_weights: weight_sums must be 16-byte aligned");
 		LTEN_HIP_REQUIRE(out_features < (1ull << 31) && in_features * 255ull < (1ull << 31), "lten_hip_fcq_prepare_weights: dimension too large");
 		const unsigned blocks = (unsigned)ceil_div(out_features, 4);
-		fcq_prepare_weights_sums_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(W, W_prepared, weight_sums, out_features, in_features,
+		fcq_prepare_weights_sums_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(W, W_prepared, weight_sums, out_features, in_features, padded,
 		                                                                           in_features % 16 == 0 ? 1 : 0);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;

@@ -18,9 +18,13 @@ struct QProblem {
 	void* C;           // uint8 [M x N] or int32 [M x N], row-major, ld = N
 	int64_t a_rs, a_ks, b_rs, b_ks;
 	int M, N, K;
+	// Rows padded to a multiple of 16 bytes: the last k_pad of the K bytes of every row of A and B are padding that holds
+	// the byte 128 (0 in a prepared B), which multiplies to nothing; konst already allows for what the padding adds to
+	// byte sums taken over all K bytes of a row, and kernels that need the number of real bytes use K - k_pad
+	int k_pad = 0;
 	const int32_t* rterm;  // [M] (128 - zpB) * SA_m, or null
 	const int32_t* cterm;  // [N] (128 - zpA) * SB_n + bias_n, or null
-	int32_t konst;         // K (zpA zpB - 16384)
+	int32_t konst;         // K (zpA zpB - 16384) over the real bytes, less what padding bytes add to the two sum terms
 	float mult;            // real_multiplier
 	float zp_c;            // (float) output zero point
 	int vec_ok;            // operand bases and row strides are multiples of 16 bytes

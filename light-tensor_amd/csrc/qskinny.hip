@@ -180,7 +180,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 		const int n = group * 16 + lrow;
 		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-		const int base = coef_b * tsb + p.K * coef_a * coef_b + bias_n;
+		const int base = coef_b * tsb + (p.K - p.k_pad) * coef_a * coef_b + bias_n;
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) {
 			v4i tot = { 0, 0, 0, 0 };

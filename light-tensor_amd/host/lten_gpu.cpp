@@ -639,7 +639,8 @@ Tensor FullyConnected_q::forward(Tensor& input)
 	// once per to() / weights_changed() / hand-out of the weight tensor, and every forward runs on them.
 	if (!prepared_valid_) {
 		options.data_type = UINT8;
-		if (!prepared_.defined()) prepared_ = AllocateTensor({ 1, 1, output_features_, input_features_ }, &options);
+		// (rows of the int8 form start on 16-byte boundaries: input_features_ rounded up to a multiple of 16 bytes apart)
+		if (!prepared_.defined()) prepared_ = AllocateTensor({ 1, 1, output_features_, (input_features_ + 15) / 16 * 16 }, &options);
 		options.data_type = INT32;
 		if (!weight_sums_.defined()) weight_sums_ = AllocateTensor({ output_features_ }, &options);
 		LTEN_HIP_CALL(lten_hip_fcq_prepare_weights(static_cast<const uint8_t*>(weight_.get_data_ptr()), static_cast<uint8_t*>(prepared_.get_data_ptr()),

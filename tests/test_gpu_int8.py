@@ -514,9 +514,11 @@ def fcq(gpu, entry, X, W, sc, zp, bias=None, prepared=False):
     dX, dW, dY, ws = D.from_numpy(X), D.from_numpy(W), D(M * N), D(4 * (M + N))
     db = D.from_numpy(np.asarray(bias, np.int32)) if bias is not None else None
     if prepared:
-        dWp, dS = D(W.size + 16), D(4 * N + 16)
+        Kp = (K + 15) // 16 * 16   # rows of the prepared form start on 16-byte boundaries, zeros behind the weights
+        dWp, dS = D(N * Kp + 16), D(4 * N + 16)
         gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, N, K, dS.ptr))
-        assert np.array_equal(dWp.numpy(np.uint8, W.shape), W ^ 0x80)
+        Wp = dWp.numpy(np.uint8, (N, Kp))
+        assert np.array_equal(Wp[:, :K], W ^ 0x80) and not Wp[:, K:].any()
         assert np.array_equal(dS.numpy(np.int32, (N,)), W.sum(axis=1, dtype=np.int64))
         gpu.check(entry(1, M, K, N, dX.ptr, dWp.ptr, dS.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr, ws.ptr))
     else:
@@ -550,20 +552,61 @@ def test_prepared_weights_match_unprepared(gpu, ob, shape):
         assert np.array_equal(want, Co), (shape, zp, k0)
 
 
+@pytest.mark.parametrize("shape", [(1, 4096, 4100), (16, 512, 1000), (64, 512, 1000), (128, 1000, 1000), (300, 260, 401), (1024, 1024, 1000),
+                                   (512, 10, 50), (700, 520, 2050), (33, 65, 100), (40, 4096, 1937)])
+def test_rows_that_are_no_multiple_of_16_bytes(gpu, ob, shape):
+    """A layer whose in_features is no multiple of 16 (l-ten's own quantized MNIST network has one of 50): the product runs on
+    copies with padded rows, through the kernels of the padded shape instead of the guarded general kernel, and returns
+    the oracle's bytes and int32 sums through every entry point, with every zero-point pattern and a bias."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 11 + N * 5 + K)
+    X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    l = gpu.lib()
+    for zp, with_bias in (([128, 128, 128], False), ([0, 128, 3], True), ([200, 17, 99], True), ([255, 0, 255], False)):
+        bias = rng.integers(-5000, 5000, N).astype(np.int32) if with_bias else None
+        sc = [0.02, 0.013, 0.9 * K / 512]
+        Co, acco = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias)
+        raw, k0 = fcq(gpu, l.lten_hip_fcq_forward, X, W, sc, zp, bias)
+        got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, X, W, sc, zp, bias, prepared=True)
+        _, accg = gpu.qgemm_host(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias, want_acc=True)
+        assert np.array_equal(raw, Co), (shape, zp, k0)
+        assert np.array_equal(got, Co), (shape, zp, k1)
+        assert np.array_equal(accg, acco), (shape, zp)
+        if N % 4 == 0 and M * N * K >= 1 << 20:
+            assert "guard" not in k0 and "guard" not in k1, (k0, k1)
+    # the entry point that allocates nothing has no memory for such copies and keeps the guarded kernel: same bytes
+    D = gpu.DeviceBuffer
+    dX, dW, dY = D.from_numpy(X), D.from_numpy(W), D(M * N)
+    db = D.from_numpy(bias) if bias is not None else None
+    gpu.check(l.lten_hip_fcq_forward_static(1, M, K, N, dX.ptr, dW.ptr, db.ptr if db else None, gpu.qparams3(sc, zp), dY.ptr))
+    assert np.array_equal(dY.numpy(np.uint8, (M, N)), Co)
+
+
 def test_prepare_weights_in_place_and_odd_count(gpu):
     rng = np.random.default_rng(5)
-    for n in (1, 15, 16, 17, 4099, 1 << 20):
+    for n in (16, 4096, 1 << 20):   # rows that are multiples of 16 bytes: in place
         w = rng.integers(0, 256, n, dtype=np.uint8)
         d = gpu.DeviceBuffer.from_numpy(w)
         gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, 1, n, None))
         assert np.array_equal(d.numpy(np.uint8, (n,)), w ^ 0x80)
-    # with the row sums, on rows of any length (16-byte loads only where every row allows them)
-    for rows, cols in ((1, 1), (3, 15), (5, 16), (7, 100), (130, 784), (64, 4099), (33, 4096)):
+    # with and without the row sums, on rows of any length (16-byte loads only where every row allows them); rows that are
+    # no multiple of 16 bytes are padded with zeros to the next one, which cannot happen in place
+    for rows, cols in ((1, 1), (1, 15), (1, 17), (1, 4099), (3, 15), (5, 16), (7, 100), (130, 784), (64, 4099), (33, 4096)):
         w = rng.integers(0, 256, (rows, cols), dtype=np.uint8)
-        d, sums = gpu.DeviceBuffer.from_numpy(w), gpu.DeviceBuffer(4 * rows + 16)
-        gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, rows, cols, sums.ptr))
-        assert np.array_equal(d.numpy(np.uint8, (rows, cols)), w ^ 0x80)
-        assert np.array_equal(sums.numpy(np.int32, (rows,)), w.sum(axis=1, dtype=np.int64))
+        cp = (cols + 15) // 16 * 16
+        for with_sums in (True, False):
+            d, sums = gpu.DeviceBuffer.from_numpy(w), gpu.DeviceBuffer(4 * rows + 16)
+            out = d if cp == cols else gpu.DeviceBuffer(rows * cp, zero=False)
+            gpu.check(gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, out.ptr, rows, cols, sums.ptr if with_sums else None))
+            got = out.numpy(np.uint8, (rows, cp))
+            assert np.array_equal(got[:, :cols], w ^ 0x80) and not got[:, cols:].any()
+            if with_sums:
+                assert np.array_equal(sums.numpy(np.int32, (rows,)), w.sum(axis=1, dtype=np.int64))
+        if cp != cols:
+            d = gpu.DeviceBuffer.from_numpy(np.concatenate([w.ravel(), np.zeros(rows * (cp - cols), np.uint8)]))
+            assert gpu.lib().lten_hip_fcq_prepare_weights(d.ptr, d.ptr, rows, cols, None) != 0
+            assert b"must not overlap" in gpu.lib().lten_hip_last_error()
 
 
 def test_cfg3_prepared_weights_full_size(gpu, wl):
