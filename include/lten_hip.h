@@ -154,7 +154,7 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
  * aligned): the sums of the zero-point correction that quantized_matmul recomputes on every call
  * (l-ten/math_fns.cpp:1362-1369).  lten_hip_fcq_forward_prepared is lten_hip_fcq_forward on such weights and
  * returns bit-identical outputs.  For every shape the direct-to-LDS tiles take (in_features % 16 == 0 and >= 128,
- * out_features % 4 == 0, more than 32 rows) it is a single launch whatever the zero points and the bias: the
+ * more than 32 rows) it is a single launch whatever the zero points and the bias: the
  * column term comes from weight_sums, the activation rows' byte sums (needed when the weight zero point is not 128)
  * are added up from the operand fragments inside the GEMM.  When in_features is no multiple of 16 the activations
  * are first copied into rows of that length in memory the library owns (one more launch; the memory is allocated by

@@ -98,9 +98,25 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 {
 	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.M >= 1 && p.N >= 1 && p.K >= 1)) return -1;
 	const int64_t tiles = (int64_t)ceil_div((uint64_t)p.M, 16) * ceil_div((uint64_t)p.N, 16);
-	// up to 512 tiles; with an N the direct-to-LDS tiles do not take (no multiple of 4) up to 8192, where the alternative
-	// is the guarded kernel (4096 x 50 x 5760: 83 us there)
-	if (tiles > (p.N % 4 != 0 ? 8192 : 512) || p.K > 16384) return -1;
+	// Up to 8192 tiles, as long as this kernel is ahead of the 128 x 128 direct-to-LDS tiles where those apply (at least
+	// 128 output columns, K >= 512 or at least 64 such tiles: qgemm_dispatch).  It takes about 2.3 us + 4.1 us per million
+	// (tiles x K), they about 5.4 us + 0.33 us per k-step of 128 bytes of a workgroup's share of K while they run in one
+	// round, 4 us more when workgroups share tiles (split K, as qgemm_dispatch picks it) or N is no multiple of 4 (byte
+	// stores), 2.5 us more with a partial last k-step.  300 x 1000 x 512: 4.8 us here, 6.9 there; 400 x 400 x 2048: 7.7
+	// and 10.8; 256 x 512 x 4096: 9.4 and 13.8; 200 x 2000 x 256: 4.3 (13.8 on the guarded kernel, which took it before);
+	// 1024 x 1000 x 1024: 16.8 and 8.6; 128 x 4096 x 1024: 9.6 and 7.4; 128 x 1024 x 16384: 30.3 and 23.3.  A few output
+	// columns make poor use of 128-column tiles and stay here (4096 x 50 x 5760, l-ten's quantized MNIST layer at a large
+	// batch: 22.5 us).
+	if (tiles > 8192 || p.K > 16384) return -1;
+	const uint64_t tiles128 = ceil_div((uint64_t)p.M, 128) * ceil_div((uint64_t)p.N, 128);
+	const bool tiles_apply = p.N >= 128 && (p.K >= 512 || (p.K >= 128 && tiles128 >= 64)) && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
+	                         (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32);
+	if (tiles_apply) {
+		const int splits = (tiles128 <= 64 && p.K >= 8192) ? (tiles128 <= 32 ? 4 : 2) : (tiles128 <= 32 && p.K >= 4096) ? 2 : 1;
+		const double here = 2.3 + 4.1e-6 * (double)tiles * p.K;
+		const double there = 5.4 + 0.0026 * p.K / splits + (splits > 1 ? 4.0 : 0.0) + (p.N % 4 != 0 ? 4.0 : 0.0) + (p.K % 128 != 0 ? 2.5 : 0.0);
+		if (here >= there) return -1;
+	}
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
 	const dim3 grid((unsigned)tiles);
 	if (p.K <= 1024) {

@@ -535,7 +535,7 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 	// skinny activations: one streaming pass over the weights (option "qskinny": 0 = auto, 2 = off)
 	p.cterm = nullptr;
 	p.rterm = nullptr;
-	const bool may_stream = get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0;
+	const bool may_stream = get_option(OPT_QSKINNY) != 2 && get_option(OPT_QGEMM_TILE) == 0 && get_option(OPT_QGEMM_SPLIT) < 2;  // (a forced tile or split goes to the tiles)
 	// below a megabyte of weights the one-launch kernel's many small workgroups win (option "qskinny" 1: stream anyway)
 	const bool large_weights = N * K >= (1ull << 20) || get_option(OPT_QSKINNY) == 1;
 	if (M <= 32 && large_weights && may_stream) {

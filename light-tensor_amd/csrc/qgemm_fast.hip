@@ -159,7 +159,7 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 			if (OFFSET) rt[j] += p.acc_offset;
 			if (TERMS == 1 && carry) rt[j] += p.rterm[min(m0 + wm * TM + (j ^ jsw) * 32 + lrow, p.M - 1)];
 		}
-		// Every load below is unconditional, from a column clamped into the matrix (N % 4 == 0: four columns exist
+		// Every load below is unconditional, from a column clamped into the matrix (with N % 4 == 0 four columns exist
 		// together; what a clamped load brings is never stored), and the one choice, how the bias is fetched, is made
 		// outside the loops: a branch per vector would make each load wait for the one before it.
 		v4i ct[FN][4];
@@ -169,35 +169,49 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		for (int i = 0; i < FN; i++)
 #pragma unroll
 			for (int q = 0; q < 4; q++) ct[i][q] = v4i{ 0, 0, 0, 0 };
-		if (TERMS == 1 && have) {
-#pragma unroll
-			for (int i = 0; i < FN; i++)
-#pragma unroll
-				for (int q = 0; q < 4; q++) ct[i][q] = *reinterpret_cast<const v4i*>(p.cterm + min(ncol + i * 32 + q * 8, p.N - 4));
-		}
-		if (TERMS >= 2 && have) {
-#pragma unroll
-			for (int i = 0; i < FN; i++)
-#pragma unroll
-				for (int q = 0; q < 4; q++) {
-					const v4i ws = *reinterpret_cast<const v4i*>(p.wsum + min(ncol + i * 32 + q * 8, p.N - 4));
-#pragma unroll
-					for (int e = 0; e < 4; e++) ct[i][q][e] = ws[e] * p.coef_b;
-				}
-			if (p.bias != nullptr && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) {
+		if ((p.N & 3) == 0) {
+			if (TERMS == 1 && have) {
 #pragma unroll
 				for (int i = 0; i < FN; i++)
 #pragma unroll
-					for (int q = 0; q < 4; q++) ct[i][q] += *reinterpret_cast<const v4i*>(p.bias + min(ncol + i * 32 + q * 8, p.N - 4));
-			} else if (p.bias != nullptr) {  // a bias vector that only has the alignment of its ints
+					for (int q = 0; q < 4; q++) ct[i][q] = *reinterpret_cast<const v4i*>(p.cterm + min(ncol + i * 32 + q * 8, p.N - 4));
+			}
+			if (TERMS >= 2 && have) {
 #pragma unroll
 				for (int i = 0; i < FN; i++)
 #pragma unroll
 					for (int q = 0; q < 4; q++) {
-						const int32_t* b = p.bias + min(ncol + i * 32 + q * 8, p.N - 4);
-						ct[i][q] += v4i{ b[0], b[1], b[2], b[3] };
+						const v4i ws = *reinterpret_cast<const v4i*>(p.wsum + min(ncol + i * 32 + q * 8, p.N - 4));
+#pragma unroll
+						for (int e = 0; e < 4; e++) ct[i][q][e] = ws[e] * p.coef_b;
 					}
+				if (p.bias != nullptr && (reinterpret_cast<uintptr_t>(p.bias) & 15) == 0) {
+#pragma unroll
+					for (int i = 0; i < FN; i++)
+#pragma unroll
+						for (int q = 0; q < 4; q++) ct[i][q] += *reinterpret_cast<const v4i*>(p.bias + min(ncol + i * 32 + q * 8, p.N - 4));
+				} else if (p.bias != nullptr) {  // a bias vector that only has the alignment of its ints
+#pragma unroll
+					for (int i = 0; i < FN; i++)
+#pragma unroll
+						for (int q = 0; q < 4; q++) {
+							const int32_t* b = p.bias + min(ncol + i * 32 + q * 8, p.N - 4);
+							ct[i][q] += v4i{ b[0], b[1], b[2], b[3] };
+						}
+				}
 			}
+		} else if (have) {
+			// N is no multiple of 4: the last columns do not come in fours, so every column is clamped and loaded by itself
+#pragma unroll
+			for (int i = 0; i < FN; i++)
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						const int col = min(ncol + i * 32 + q * 8 + e, p.N - 1);
+						if (TERMS == 1) ct[i][q][e] = p.cterm[col];
+						if (TERMS >= 2) ct[i][q][e] = p.wsum[col] * p.coef_b + (p.bias != nullptr ? p.bias[col] : 0);
+					}
 		}
 #pragma unroll
 		for (int i = 0; i < FN; i++)
@@ -450,9 +464,15 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 #pragma unroll
 				for (int q = 0; q < 4; q++) {
 					const int n = n0 + wn * TN + i * 32 + q * 8 + lgrp * 4;
-					if (n >= p.N) continue;  // N is a multiple of 4: the four columns exist together
-					const v4i v = { acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3] };
-					*reinterpret_cast<v4i*>(static_cast<int*>(p.C) + (int64_t)m * p.N + n) = v;
+					if (n >= p.N) continue;
+					if ((p.N & 3) == 0) {  // the four columns exist together, on a 16-byte boundary
+						const v4i v = { acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3] };
+						*reinterpret_cast<v4i*>(static_cast<int*>(p.C) + (int64_t)m * p.N + n) = v;
+					} else {
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							if (n + e < p.N) static_cast<int*>(p.C)[(int64_t)m * p.N + n + e] = acc[i][j][q * 4 + e];
+					}
 				}
 		}
 	} else {
@@ -498,11 +518,16 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 					if (row0 + jrow + r < p.M && col0 + ch * 16 < p.N)
 						__builtin_nontemporal_store(val, reinterpret_cast<v4i*>(cbase + (int64_t)(jrow + r) * p.N + ch * 16));
 				}
-			} else {  // N is a multiple of 4: four bytes at a time
+			} else if ((p.N & 3) == 0) {  // four bytes at a time
 				for (int c = lane; c < 32 * (TN / 4); c += 64) {
 					const int r = c / (TN / 4), dw = c % (TN / 4);
 					if (row0 + jrow + r < p.M && col0 + dw * 4 < p.N)
 						*reinterpret_cast<int*>(cbase + (int64_t)(jrow + r) * p.N + dw * 4) = *reinterpret_cast<const int*>(strip + r * WP + dw * 4);
+				}
+			} else {  // rows of C start anywhere: byte by byte, a lane per column so that a wavefront's stores run along a row
+				for (int c = lane; c < 32 * TN; c += 64) {
+					const int r = c / TN, b = c % TN;
+					if (row0 + jrow + r < p.M && col0 + b < p.N) cbase[(int64_t)(jrow + r) * p.N + b] = strip[r * WP + b];
 				}
 			}
 			wait_vmcnt_lgkm0<63>();  // the strip is read before the next block overwrites it
@@ -597,7 +622,7 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits, const Spli
 		scratch = &g_split;
 	}
 	const uint64_t tiles = ceil_div(p.M, T) * ceil_div(p.N, T);
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % (BK * splits) == 0 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % (BK * splits) == 0 &&
 	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
@@ -657,7 +682,7 @@ int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
 	// K: any multiple of 16 at least one k-step long (variants 33, 41 and 51), or a multiple of the k-step
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.N % 4 == 0 && p.K % 16 == 0 && p.K >= 128 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.K >= 128 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&

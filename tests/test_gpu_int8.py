@@ -84,6 +84,32 @@ def test_direct_to_lds_tiles(gpu, ob, variant, shape):
              bias=rng.integers(-5000, 5000, N).astype(np.int32), tile=variant)
 
 
+@pytest.mark.parametrize("variant", [33, 41, 51])
+@pytest.mark.parametrize("shape", [(300, 1001, 512), (256, 258, 640), (130, 4099, 256), (257, 129, 400), (512, 50257 // 16, 768)])
+def test_direct_to_lds_tiles_with_any_number_of_columns(gpu, ob, variant, shape):
+    """out_features that are no multiple of 4 (1001 classes, a vocabulary of 50257): rows of the output then start on any
+    byte, and the zero-point vectors end inside a group of four.  Raw and prepared weights, int32 and uint8 outputs,
+    with every term and a bias, on each tile family."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K + variant)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    l = gpu.lib()
+    for zp, with_bias in (([128, 128, 128], False), ([0, 128, 3], True), ([3, 250, 77], True)):
+        bias = rng.integers(-5000, 5000, N).astype(np.int32) if with_bias else None
+        sc = [0.02, 0.013, 0.9]
+        run_case(gpu, ob, A, B, sc, np.array(zp, np.uint8), bias=bias, tile=variant)
+        assert gpu.last_kernel().startswith("qgemm_fast"), gpu.last_kernel()
+        gpu.set_option("qgemm_tile", variant)
+        try:
+            got, k1 = fcq(gpu, l.lten_hip_fcq_forward_prepared, A, B, sc, zp, bias, prepared=True)
+        finally:
+            gpu.set_option("qgemm_tile", 0)
+        assert k1.startswith("qgemm_fast") and "wpre" in k1, k1
+        Co, _ = ob.quantized_matmul(A, B, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias)
+        assert np.array_equal(got, Co), (shape, zp, k1)
+
+
 def test_requantize_exact_epilogue_in_tiled_kernels(gpu, ob):
     """Multipliers above 1 select the epilogue that spells out the x86 conversion (out-of-range -> 0x80000000)."""
     rng = np.random.default_rng(4)
@@ -257,7 +283,7 @@ def test_batch_sizes_between_the_tile_sizes(gpu):
     (384, 1536, 4096, "qgemm_fast_128x128x128_w2x2_s4"),          # 36 tiles, one per CU: the ring of four stages
     (300, 1540, 4112, "qgemm_fast_128x128x128_w2x2_s4_ktail"),    # the same with ragged edges and a partial last k-step
     (384, 1536, 8192, "qgemm_fast_128x128x128_w2x2_s4_splitk"),   # 36 tiles, K in two shares of 4096
-    (130, 1024, 512 * 5, "qgemm_fast_128x128x128_w2x2_s2"),       # K below 4096: two stages
+    (130, 2048, 512 * 5, "qgemm_fast_128x128x128_w2x2_s2"),       # K below 4096: two stages
     (1024, 4096, 640, "qgemm_fast_128x128x128_w2x2_s2"),          # five k-steps, one workgroup per CU
 ])
 def test_128_tiles_ring_depth(gpu, shape):
@@ -483,7 +509,7 @@ def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
     Ms = [1, 2, 15, 16, 17, 31, 32, 33, 47, 63, 64, 65, 100, 127, 128, 129, 200, 255, 257, 300]
     Ns = [1, 10, 16, 36, 100, 128, 130, 132, 256, 500, 512, 1000, 1024, 2048, 2052]
     Ks = [1, 7, 16, 48, 100, 128, 144, 512, 528, 784, 1000, 1024, 2048, 2064, 4096]
-    larger = [(300, 1000, 1024), (129, 2052, 784), (257, 516, 2064), (200, 1024, 144)]   # past the one-launch kernel's 512 tiles
+    larger = [(1024, 1000, 1024), (520, 2052, 784), (1025, 516, 2064), (2100, 2048, 144)]   # where the 128 x 128 tiles are ahead of the one-launch kernel
     for case in range(60 + len(larger)):
         if case < 60:
             M, N, K = int(rng.choice(Ms)), int(rng.choice(Ns)), int(rng.choice(Ks))
@@ -503,7 +529,8 @@ def test_seeded_sweep_over_dispatch_boundaries(gpu, ob):
         assert np.array_equal(Cp, Cg), (M, N, K, zp, kp)
         seen_prepared.add(kp.split("_")[0] + "_" + kp.split("_")[1] + ("+zp" if "+zp" in kp else ""))
     assert {"qskinny_mfma", "qdirect_16x16", "qgemm_fast", "qgemm_guard"} <= seen, seen
-    assert {"qgemm_fast+zp", "qgemm_guard"} <= seen_prepared, seen_prepared
+    # (prepared weights keep their rows on 16-byte boundaries, so the guarded kernel no longer sees them)
+    assert {"qgemm_fast+zp", "qdirect_16x16", "qskinny_mfma"} <= seen_prepared, seen_prepared
 
 
 def fcq(gpu, entry, X, W, sc, zp, bias=None, prepared=False):
@@ -656,7 +683,7 @@ def test_prepared_forward_takes_zero_point_terms_in_the_gemm_launch(gpu, ob, sha
                 assert np.array_equal(dY.numpy(np.uint8, (M, N)), want), (shape, tile, zp, bias_off, kern)
     finally:
         gpu.set_option("qgemm_tile", 0)
-    assert seen_fast or shape in ((300, 260, 400), (256, 384, 4096)), shape
+    assert seen_fast or shape in ((300, 260, 400), (256, 384, 4096), (512, 512, 512)), shape
 
 
 @pytest.mark.parametrize("zp", ZP_FUSED)
