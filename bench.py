@@ -534,6 +534,30 @@ def extra_configs(lt, wl, with_cpu):
                 "algorithmic_bytes": xq3.nbytes + wq3.nbytes + xq3.size})
     del dxq3, dwq3, dyq3, dyq3b, wsq3
 
+    # ---- int8 layers whose sizes are no multiples of the kernels' vector widths: in_features no multiple of 16 (the rows
+    # are copied into padded ones first; prepared weights are padded once), out_features no multiple of 4 (byte stores).
+    # Prepared weights, zero points (17, 250, 100); the first rows (2^30 multiply-adds' worth) against the oracle.
+    for (Mo, No, Ko, what) in ((4096, 4096, 4100, "in_features = 4100, no multiple of 16"), (4096, 1001, 4096, "out_features = 1001, no multiple of 4"),
+                               (64, 500, 1000, "a 1000 -> 500 layer at batch 64")):
+        rngo = np.random.default_rng(Mo + No + Ko)
+        Xo = rngo.integers(0, 256, (Mo, Ko), dtype=np.uint8)
+        Wo_ = (np.clip(np.round(rngo.normal(0, 40, (No, Ko))), -127, 127).astype(np.int16) + 128).astype(np.uint8)
+        Kp = (Ko + 15) // 16 * 16
+        dXo, dWo, dWp, dSo, dYo, wso = D.from_numpy(Xo), D.from_numpy(Wo_), D(No * Kp), D(4 * No), D(Mo * No), D(4 * (Mo + No))
+        lt.check(l.lten_hip_fcq_prepare_weights(dWo.ptr, dWp.ptr, No, Ko, dSo.ptr))
+        sco, zpo = [0.02, 0.01, 3.0 * Ko / 4096], [17, 250, 100]
+        qpo = lt.qparams3(sco, zpo)
+        fo = lambda: lt.check(l.lten_hip_fcq_forward_prepared(1, Mo, Ko, No, dXo.ptr, dWp.ptr, dSo.ptr, None, qpo, dYo.ptr, wso.ptr))
+        mso = timed(lt, fo, 100)
+        rec = {"config": f"int8 FC {Mo}x{No}x{Ko} ({what}), prepared weights, zero points (17, 250, 100)", "gpu_us": round(mso * 1e3, 2),
+               "kernel": lt.last_kernel(), "achieved_TOPs": round(2.0 * Mo * No * Ko / mso / 1e9, 1)}
+        if with_cpu:
+            rows = max(1, min(Mo, (1 << 30) // (No * Ko)))
+            want_o, _ = ob.quantized_matmul(Xo[:rows], Wo_, np.array(sco, np.float32), np.array(zpo, np.uint8))
+            rec["verified_bit_exact_rows"] = rows if np.array_equal(dYo.numpy(np.uint8, (Mo, No))[:rows], want_o) else 0
+        out.append(rec)
+        del dXo, dWo, dWp, dSo, dYo, wso
+
     # ---- beyond the five configs: a large fp32 product in the three layouts l-ten's layers use (FullyConnected forward
     # NT, data gradient NN, weight gradient TN), synthetic N(0,1) operands
     n = 4096
