@@ -5,8 +5,8 @@
 //   - zpW * sum_k col[k][p] - zpIn * sum_k w[co][k] + K * zpW * zpIn (+ bias[p]), then the requantize of
 // l-ten/math_fns.cpp:1474.  Positions outside the image hold the byte 0 in the column buffer (not the zero point).
 //
-// Windows of at most 64 taps (the 1 -> 10 channel 5x5 layer of l-ten's quantized MNIST network has 25) run in one
-// launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
+// Windows of at most 64 taps for fewer than 48 output channels (the 1 -> 10 channel 5x5 layer of l-ten's quantized
+// MNIST network has 25 taps) run in one launch without a column buffer: a thread owns one output position, gathers its window into 16 packed dwords,
 // and takes the products with unsigned dot4 instructions against the weights of up to 64 output channels held in
 // LDS; consecutive lanes are consecutive positions of a row, so loads and the byte stores of y run along rows.
 // Longer windows also run in one launch where the weights fit LDS beside the image (small images, at most 64 output
@@ -265,6 +265,15 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 	volatile float ab = qp[1].scale * qp[0].scale;
 	const float mult = ab / qp[2].scale, zp_out = (float)qp[2].zero_point;
 
+	// Windows of at most 64 taps for 48 output channels and more: the band kernel's matrix cores are ahead of the dot
+	// products below, which issue at a quarter of the vector rate (8 x 16 x 56 x 56 -> 64 channels 2 x 2, stride 2: 26.5
+	// -> 6.9 us; 8 x 64 x 56 x 56 -> 256 channels 1 x 1: 30.0 -> 16.6 us; 64 x 3 x 224 x 224 -> 64 channels 3 x 3: 181 ->
+	// 130 us), not for fewer (256 x 3 x 32 x 32 -> 32: 14.5 us below, 19.0 there; l-ten's MNIST conv1, 10 channels: 6.6
+	// and 7.3).  Option "conv_variant" 2 keeps the kernel below.
+	if (K <= CQ_MAXK && Cout >= 48 && (get_option(OPT_CONV_VARIANT) == 0 || get_option(OPT_CONV_VARIANT) == 3)) {
+		const int rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
+		if (rc >= 0) return rc;
+	}
 	if (K <= CQ_MAXK && (uint64_t)N * HW < (1ull << 31) && get_option(OPT_CONV_VARIANT) != 1) {
 		const dim3 grid((unsigned)ceil_div((uint64_t)N * HW, 256), (unsigned)ceil_div(Cout, CQ_CO));
 		set_kernel_name("conv2dq_direct");

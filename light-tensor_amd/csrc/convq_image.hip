@@ -577,7 +577,7 @@ static bool image_plan(const ConvGeo& g, ImagePlan& pl)
 static bool band_plan(const ConvGeo& g, BandPlan& pl)
 {
 	const int64_t T = (int64_t)g.kh * g.kw, K = (int64_t)g.Cin * T;
-	if (K <= 64 || g.pw > 64 || g.Cin > 1024 || g.Cout > 16 * 65535) return false;
+	if (g.pw > 64 || g.Cin > 1024 || g.Cout > 16 * 65535) return false;
 	pl.CP = g.Cin <= 4 ? 4 : g.Cin <= 8 ? 8 : 16;
 	pl.CPtot = (g.Cin + pl.CP - 1) / pl.CP * pl.CP;
 	pl.PP = pl.CPtot + (pl.CPtot % 32 == 0 ? 16 : 0);  // pixels 32 or 64 bytes apart would meet on the same LDS banks

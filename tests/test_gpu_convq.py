@@ -61,7 +61,11 @@ def test_conv2dq_golden_from_compiled_layer(gpu):
                                  (1, 400, 9, 9, 40, 3, 3, 0, 0, 1, 1),       # 3600 taps: the weights of 32 channels do not fit, three launches
                                  (1, 200, 9, 9, 30, 3, 3, 0, 0, 1, 1),       # 1800 taps, 30 channels: two blocks of 16 channels
                                  (3, 96, 20, 20, 72, 1, 1, 0, 0, 1, 1),      # a 1 x 1 layer of 96 channels: the weights are copied as they lie
-                                 (2, 68, 21, 22, 40, 1, 1, 1, 0, 2, 1)])     # 1 x 1 with a row stride of 2 and padded rows
+                                 (2, 68, 21, 22, 40, 1, 1, 1, 0, 2, 1),      # 1 x 1 with a row stride of 2 and padded rows
+                                 (8, 16, 20, 24, 64, 2, 2, 0, 0, 2, 2),      # 64 taps, 64 channels: short windows on the band kernel
+                                 (2, 3, 40, 44, 64, 3, 3, 1, 1, 1, 1),       # 27 taps of 3 channels (padded to 4), one k-step
+                                 (2, 64, 12, 12, 80, 1, 1, 0, 0, 1, 1),      # 1 x 1 with 64 channels in, 80 out
+                                 (3, 5, 17, 19, 50, 3, 3, 2, 2, 1, 2)])      # 45 taps, 50 channels, ragged everything
 def test_conv2dq_vs_oracle(gpu, ob, geo):
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -97,14 +101,16 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         staged = N * ((Ho * Wo + 15) // 16) * ((Cin * H * W + 15) // 16 * 16 + ncb * 16 * Kp)
         permuted = Cin % 4 == 0 and kh * kw in (1, 9, 25, 49)
         small = small and not (band and (permuted or staged > 16 << 20))
-        assert kern == ("conv2dq_direct" if K <= 64 else "conv2dq_image" if small else "conv2dq_band" if band else "conv2dq_rows_gemm_finish"), kern
+        # (windows of at most 64 taps: the band kernel from 48 output channels on, else one launch from registers)
+        assert kern == (("conv2dq_band" if Cout >= 48 and band else "conv2dq_direct") if K <= 64 else
+                        "conv2dq_image" if small else "conv2dq_band" if band else "conv2dq_rows_gemm_finish"), kern
         assert np.array_equal(acc, want_acc), kern
         assert np.array_equal(y, want_y), kern
         if kern in ("conv2dq_image", "conv2dq_band"):   # the three-launch route on the same shape gives the same bytes
             gpu.set_option("conv_variant", 2)
             try:
                 y2, acc2 = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
-                assert gpu.last_kernel() == "conv2dq_rows_gemm_finish"
+                assert gpu.last_kernel() == ("conv2dq_direct" if K <= 64 else "conv2dq_rows_gemm_finish")
             finally:
                 gpu.set_option("conv_variant", 0)
             assert np.array_equal(acc2, want_acc) and np.array_equal(y2, want_y)
