@@ -513,8 +513,16 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		LTEN_HIP_REQUIRE(g2.Ho == (int)H && g2.Wo == (int)W, "conv2d_dgrad: internal geometry mismatch");
 		return conv_forward_dispatch(g2, dy, work, nullptr, dx);
 	}
+	// A strided first layer: the rows of the implicit GEMM below are the input channels, a handful in a tile of 64, and
+	// with a large window the padding costs more than l-ten's decomposition image by image does (32 x 3 x 224 x 224 <- 64
+	// channels 7 x 7 stride 2: 3.8 ms below, 1.0 ms image by image; 3 x 3 and 5 x 5 windows stay below: 32 x 4 x 56 x 56
+	// <- 64 channels 3 x 3 stride 2 64 against 332 us).  Estimates: the tile loop at 45 TFLOP/s of padded work; 16 us +
+	// 9 us per million elements of the column buffer per image.
+	const double padded_us = 2.0 * 64 * ceil_div(Cin, 64) * (double)(N * H * W) * Cout * kh * kw / ((double)sh * sw) / 45e6;
+	const double by_image_us = (double)N * (16.0 + 9e-6 * (double)Kc * HW);
+	const bool padded_rows = get_option(OPT_CONV_VARIANT) == 0 && Cin <= 8 && padded_us > 1.5 * by_image_us;
 	// any stride: one implicit-GEMM launch for the batch (64 x 64 x 28 x 28 <- 128 channels at stride 2: 722 us image by image)
-	if (get_option(OPT_CONV_VARIANT) == 0 && (!few_narrow || !dgrad_as_forward(g)) && dgrad_gemm_takes(g)) {
+	if (get_option(OPT_CONV_VARIANT) == 0 && (!few_narrow || !dgrad_as_forward(g)) && !padded_rows && dgrad_gemm_takes(g)) {
 		set_kernel_name("conv2d_dgrad_64x64x32");
 		// one grid row per class of pixels (y mod sh, x mod sw); class (0, 0) has the most
 		const uint64_t max_tiles_n = ceil_div(N * ceil_div(H, (uint64_t)sh) * ceil_div(W, (uint64_t)sw), 64);

@@ -260,6 +260,23 @@ def test_conv_data_gradient_with_strides(gpu, ob, geo):
     assert rel_err(dx, want_dx) < TOL
 
 
+def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
+    """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
+    padding costs more than l-ten's own decomposition (GEMM + col2im image by image), which the library then takes."""
+    geo = (2, 3, 128, 128, 64, 7, 7, 3, 3, 2, 2)
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_dgrad_sgemm_col2im", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+
+
 @pytest.mark.parametrize("geo", [(3, 16, 20, 30, 64, 3, 3, 1, 1, 1, 1),      # 30 columns: rows start 8 bytes off 16-byte boundaries
                                  (2, 8, 17, 26, 33, 3, 3, 0, 0, 1, 1),      # MNIST after one unpadded 3x3: 26 columns, no padding
                                  (2, 12, 33, 50, 130, 3, 3, 1, 1, 1, 1),    # two column tiles, three tile rows, three channel blocks
