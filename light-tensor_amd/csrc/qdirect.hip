@@ -101,8 +101,8 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 	// Up to 8192 tiles, as long as this kernel is ahead of the 128 x 128 direct-to-LDS tiles where those apply (at least
 	// 128 output columns, K >= 512 or at least 64 such tiles: qgemm_dispatch).  It takes about 2.3 us + 4.1 us per million
 	// (tiles x K), they about 5.4 us + 0.33 us per k-step of 128 bytes of a workgroup's share of K while they run in one
-	// round, 4 us more when workgroups share tiles (split K, as qgemm_dispatch picks it) or N is no multiple of 4 (byte
-	// stores), 2.5 us more with a partial last k-step.  300 x 1000 x 512: 4.8 us here, 6.9 there; 400 x 400 x 2048: 7.7
+	// round, 4 us more when workgroups share tiles (split K, as qgemm_dispatch picks it), 2 us more when N is no multiple
+	// of 4 (rows of the output that start on any byte), 2.5 us more with a partial last k-step.  300 x 1000 x 512: 4.8 us here, 6.9 there; 400 x 400 x 2048: 7.7
 	// and 10.8; 256 x 512 x 4096: 9.4 and 13.8; 200 x 2000 x 256: 4.3 (13.8 on the guarded kernel, which took it before);
 	// 1024 x 1000 x 1024: 16.8 and 8.6; 128 x 4096 x 1024: 9.6 and 7.4; 128 x 1024 x 16384: 30.3 and 23.3.  A few output
 	// columns make poor use of 128-column tiles and stay here (4096 x 50 x 5760, l-ten's quantized MNIST layer at a large
@@ -114,7 +114,7 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 	if (tiles_apply) {
 		const int splits = (tiles128 <= 64 && p.K >= 8192) ? (tiles128 <= 32 ? 4 : 2) : (tiles128 <= 32 && p.K >= 4096) ? 2 : 1;
 		const double here = 2.3 + 4.1e-6 * (double)tiles * p.K;
-		const double there = 5.4 + 0.0026 * p.K / splits + (splits > 1 ? 4.0 : 0.0) + (p.N % 4 != 0 ? 4.0 : 0.0) + (p.K % 128 != 0 ? 2.5 : 0.0);
+		const double there = 5.4 + 0.0026 * p.K / splits + (splits > 1 ? 4.0 : 0.0) + (p.N % 4 != 0 ? 2.0 : 0.0) + (p.K % 128 != 0 ? 2.5 : 0.0);
 		if (here >= there) return -1;
 	}
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;

@@ -524,10 +524,36 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 					if (row0 + jrow + r < p.M && col0 + dw * 4 < p.N)
 						*reinterpret_cast<int*>(cbase + (int64_t)(jrow + r) * p.N + dw * 4) = *reinterpret_cast<const int*>(strip + r * WP + dw * 4);
 				}
-			} else {  // rows of C start anywhere: byte by byte, a lane per column so that a wavefront's stores run along a row
-				for (int c = lane; c < 32 * TN; c += 64) {
-					const int r = c / TN, b = c % TN;
-					if (row0 + jrow + r < p.M && col0 + b < p.N) cbase[(int64_t)(jrow + r) * p.N + b] = strip[r * WP + b];
+			} else {
+				// Rows of C start on any byte.  A row's piece of the strip is stored as the aligned dwords of C that lie inside
+				// it (each put together from the two strip dwords that hold its bytes), then the up to three bytes before the
+				// first and after the last of them, two lanes a row.  (Byte by byte it is 64 store instructions a block
+				// instead of 21, and every one of them costs the memory pipeline the same: 4 us more at 300 x 1001 x 512.)
+				const int cols = min(TN, p.N - col0);  // bytes of a row's piece that exist
+				constexpr int SLOTS = TN / 4 + 1;
+				for (int c = lane; c < 32 * SLOTS; c += 64) {
+					const int r = c / SLOTS, d = c - r * SLOTS;
+					uint8_t* const rowp = cbase + (int64_t)(jrow + r) * p.N;
+					const int s = 4 * d - (int)(reinterpret_cast<uintptr_t>(rowp) & 3);  // first byte of the slot within the piece
+					if (row0 + jrow + r < p.M && s >= 0 && s + 4 <= cols) {
+						const int at = r * WP + s;
+						const uint32_t* al = reinterpret_cast<const uint32_t*>(strip + (at & ~3));
+						const uint32_t lo = al[0], hi = al[(at & 3) ? 1 : 0];
+						*reinterpret_cast<uint32_t*>(rowp + s) = __builtin_amdgcn_alignbyte(hi, lo, (unsigned)(at & 3));
+					}
+				}
+				{
+					const int r = lane >> 1;
+					uint8_t* const rowp = cbase + (int64_t)(jrow + r) * p.N;
+					const int a = (int)(reinterpret_cast<uintptr_t>(rowp) & 3);
+					const int head = min((4 - a) & 3, cols);             // bytes before the first aligned dword
+					const int full = (cols - head) & ~3;                 // bytes stored as dwords above
+					const int from = (lane & 1) ? head + full : 0, to = (lane & 1) ? cols : head;
+					if (row0 + jrow + r < p.M) {
+#pragma unroll
+						for (int e = 0; e < 3; e++)
+							if (from + e < to) rowp[from + e] = strip[r * WP + from + e];
+					}
 				}
 			}
 			wait_vmcnt_lgkm0<63>();  // the strip is read before the next block overwrites it
