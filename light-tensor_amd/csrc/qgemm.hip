@@ -425,6 +425,38 @@ __global__ __launch_bounds__(256) void qgemm_pad_rows_kernel(const uint8_t* __re
 	}
 }
 
+// An operand that lies with K as its outer index (src[k * R + r]: a transposed A, or B as quantized_matmul(.., false, ..)
+// takes it) to rows of Kp bytes contiguous in K, padded with 128 as above: tiles of 64 x 64 bytes through LDS, read
+// along r, written along k.
+__global__ __launch_bounds__(256) void qgemm_transpose_rows_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, int R, int K, int Kp)
+{
+	__shared__ __attribute__((aligned(16))) uint8_t tile[64][68];  // [r][k]
+	const int tid = threadIdx.x, r0 = (int)blockIdx.x * 64, k0 = (int)blockIdx.y * 64;
+	const bool dwords = (R & 3) == 0 && (reinterpret_cast<uintptr_t>(src) & 3) == 0;  // four r of a k in one aligned load
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int k = tid / 16 + 16 * i, r = 4 * (tid % 16);
+		uint32_t v = 0x80808080u;
+		if (k0 + k < K) {
+			const uint8_t* p = src + (int64_t)(k0 + k) * R + r0 + r;
+			if (dwords && r0 + r + 4 <= R) v = *reinterpret_cast<const uint32_t*>(p);
+			else {
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					if (r0 + r + e < R) v = (v & ~(0xFFu << (8 * e))) | ((uint32_t)p[e] << (8 * e));
+			}
+		}
+#pragma unroll
+		for (int e = 0; e < 4; e++) tile[r + e][k] = (uint8_t)(v >> (8 * e));
+	}
+	__syncthreads();
+#pragma unroll
+	for (int i = 0; i < 4; i++) {
+		const int r = tid / 16 + 16 * i, k = 4 * (tid % 16);
+		if (r0 + r < R && k0 + k < Kp) *reinterpret_cast<uint32_t*>(dst + (int64_t)(r0 + r) * Kp + k0 + k) = *reinterpret_cast<const uint32_t*>(&tile[r][k]);
+	}
+}
+
 // Where the padded copies live: owned by the library, one block per device, grown when a call needs more (never while
 // a launch graph is being recorded), kept until the process ends.  One stream uses it at a time, as everything else
 // in this library; work queued on that stream may still read the old block when it has to grow, hence the wait.
@@ -474,25 +506,44 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 
 	// Rows that are no multiple of 16 bytes long (a layer of 1000 or 50 inputs) fit none of the kernels that load 16
 	// bytes at a time, which is all but the guarded one: 4096 x 4096 x 4100 took 2.4 ms there where K = 4096 takes 56 us,
-	// one row against 4096 x 4100 weights 197 us against 5.  Such products in the layout the layers use (both operands
-	// contiguous in K) run on copies with padded rows instead: one more launch, then the kernels of the padded
-	// shape.  Prepared weights are padded already (lten_hip_fcq_prepare_weights), so only the activations are copied.
-	// The entry point that may not allocate keeps the guarded kernel, and so do products too small to care.
-	if (k_pad == 0 && !tA && tB && (K & 15) != 0 && scratch == nullptr && (weights_prepared || M * N * K >= (1ull << 20))) {
+	// one row against 4096 x 4100 weights 197 us against 5.  The same holds for operands that lie with K as the outer
+	// index (a transposed A; B as quantized_matmul(.., false, ..) takes it, which is how l-ten's Conv2d_q calls it).
+	// Such products run on copies in the layout the layers use (both operands contiguous in K, rows padded to a
+	// multiple of 16 bytes): one more launch per operand that needs it, then the kernels of the padded shape.  Prepared
+	// weights are padded already (lten_hip_fcq_prepare_weights), so only the activations are copied.  The entry point
+	// that may not allocate keeps the guarded kernel, and so do products too small to care (20 x 64 x 250, one image of
+	// l-ten's quantized MNIST conv2 as l-ten multiplies it: 24 us on the guarded kernel, 8 us this way).
+	const bool layer_layout = !tA && tB;
+	if (k_pad == 0 && (!layer_layout || (K & 15) != 0) && scratch == nullptr && (weights_prepared || M * N * K >= (1ull << 16))) {
 		const uint64_t Kp = (K + 15) & ~15ull;
-		const uint64_t bytes_a = M * Kp, bytes_b = weights_prepared ? 0 : N * Kp;
+		const bool copy_a = tA || Kp != K, copy_b = !weights_prepared && (!tB || Kp != K);
+		const uint64_t bytes_a = copy_a ? M * Kp : 0, bytes_b = copy_b ? N * Kp : 0;
 		uint8_t* buf = pad_scratch(bytes_a + bytes_b);
 		LTEN_HIP_REQUIRE(buf != nullptr || !weights_prepared,
 		                 "quantized_matmul: no memory for the padded copy of the activations (in_features = %llu is no multiple of 16; while a "
 		                 "launch graph is being recorded the copy's memory cannot be allocated: run the call once before recording)",
 		                 (unsigned long long)K);
 		if (buf != nullptr) {
-			const uint64_t chunks = (M + (weights_prepared ? 0 : N)) * (Kp / 16);
-			const unsigned blocks = (unsigned)std::min<uint64_t>(ceil_div(chunks, 256), 16384);
-			qgemm_pad_rows_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(A, buf, M, B, buf + bytes_a, weights_prepared ? 0 : N, (int)K, (int)Kp);
-			LTEN_HIP_LAUNCH_CHECK();
-			return qgemm_run(0, 1, M, N, Kp, buf, weights_prepared ? B : buf + bytes_a, C, out_acc, qp, bias, workspace, weights_prepared, nullptr,
-			                 weight_sums, (int)(Kp - K));
+			uint8_t* const a2 = buf;
+			uint8_t* const b2 = buf + bytes_a;
+			// operands contiguous in K: both in one launch
+			const uint64_t rows_a = copy_a && !tA ? M : 0, rows_b = copy_b && tB ? N : 0;
+			if (rows_a + rows_b > 0) {
+				const uint64_t chunks = (rows_a + rows_b) * (Kp / 16);
+				const unsigned blocks = (unsigned)std::min<uint64_t>(ceil_div(chunks, 256), 16384);
+				qgemm_pad_rows_kernel<<<dim3(blocks), dim3(256), 0, stream()>>>(A, a2, rows_a, B, b2, rows_b, (int)K, (int)Kp);
+				LTEN_HIP_LAUNCH_CHECK();
+			}
+			if (tA) {
+				qgemm_transpose_rows_kernel<<<dim3((unsigned)ceil_div(M, 64), (unsigned)(Kp / 64 + (Kp % 64 != 0))), dim3(256), 0, stream()>>>(A, a2, (int)M, (int)K, (int)Kp);
+				LTEN_HIP_LAUNCH_CHECK();
+			}
+			if (copy_b && !tB) {
+				qgemm_transpose_rows_kernel<<<dim3((unsigned)ceil_div(N, 64), (unsigned)(Kp / 64 + (Kp % 64 != 0))), dim3(256), 0, stream()>>>(B, b2, (int)N, (int)K, (int)Kp);
+				LTEN_HIP_LAUNCH_CHECK();
+			}
+			return qgemm_run(0, 1, M, N, Kp, copy_a ? a2 : A, copy_b ? b2 : B, C, out_acc, qp, bias, workspace, weights_prepared, nullptr, weight_sums,
+			                 (int)(Kp - K));
 		}
 	}
 

@@ -610,6 +610,22 @@ def test_rows_that_are_no_multiple_of_16_bytes(gpu, ob, shape):
     assert np.array_equal(dY.numpy(np.uint8, (M, N)), Co)
 
 
+@pytest.mark.parametrize("tA,tB", [(False, False), (True, False), (True, True)])
+@pytest.mark.parametrize("shape", [(300, 260, 400), (200, 130, 1000), (65, 1030, 333), (1024, 512, 512)])
+def test_operands_that_lie_with_k_outermost(gpu, ob, shape, tA, tB):
+    """quantized_matmul with a transposed A ([K x M] in memory) or an untransposed B ([K x N], how l-ten's Conv2d_q calls
+    it): the operands are copied into the layers' layout (rows contiguous in K, padded to a multiple of 16 bytes) and the
+    product runs on the kernels of that layout; int32 sums and bytes against the oracle."""
+    M, N, K = shape
+    rng = np.random.default_rng(M + 3 * N + 7 * K + 2 * tA + tB)
+    A = rng.integers(0, 256, (K, M) if tA else (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K) if tB else (K, N), dtype=np.uint8)
+    for zp, with_bias in (([128, 128, 128], False), ([7, 201, 99], True)):
+        bias = rng.integers(-5000, 5000, N).astype(np.int32) if with_bias else None
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9 * K / 512], np.array(zp, np.uint8), tA=tA, tB=tB, bias=bias, M=M, N=N, K=K)
+        assert "guard" not in gpu.last_kernel(), gpu.last_kernel()
+
+
 def test_prepare_weights_in_place_and_odd_count(gpu):
     rng = np.random.default_rng(5)
     for n in (16, 4096, 1 << 20):   # rows that are multiples of 16 bytes: in place
