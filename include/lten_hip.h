@@ -126,6 +126,10 @@ int lten_hip_fc_backward_relu_f32(uint64_t M, uint64_t in_features, uint64_t out
  * same argument list: C_u8[M x N] from A_u8, B_u8 (all four transpose modes), qparams[3] =
  * {A, B, C} (host memory), optional int32 bias[N] (device), int32 workspace[M + N]
  * (device scratch for the zero-point row/column terms; contents unspecified on return).
+ * Operands outside the layout FullyConnected_q uses (transpose_a = 0, transpose_b = 1: both contiguous in K) or
+ * with a K that is no multiple of 16 are first copied into that layout, rows padded, in memory the library owns
+ * (allocated by the first such call, grown by later ones; not while a launch graph is being recorded, where such
+ * calls run on a slower general kernel).
  * alpha != 1 or beta != 0 fail, as in l-ten (:1331-1334).  Outputs are bit-exact with the
  * CPU function wherever that function does not overflow int32 (K * 255^2 < 2^31) and
  * |real_multiplier * acc + zero_point| stays representable as a float. */
