@@ -1028,11 +1028,17 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// FullyConnected layer at a batch of 256 to 768 against a 4096-wide layer: 512 x 4096 x 4096 forward in 132 us
 	// instead of 240, the time of batch 1024; its data and weight gradients 130 instead of 237 us; 1024^3 in any layout
 	// 22 instead of 37 us)
-	const bool t64 = tiles128 < 256 && tiles64 >= 128;
-	if (choice == 0 && (tiles128 >= 128 || t64) && K >= 256 && (K % 32 == 0 || K >= 512)) {
+	// (and products with a side of at most 64, which would leave half or more of every larger tile empty: a batch of 96
+	// products 512 x 64 x 512 took 125 us on 256 x 256 tiles)
+	const bool t64 = (tiles128 < 256 || M <= 64 || N <= 64) && tiles64 >= 128;
+	// (a short K, 64 to 255 in whole steps of 32, only with many tiles: the products of a batch of attention heads, or an
+	// outer-product-like update; 96 x (512 x 512 x 64): 78-91 us on the 32 x 32 kernel, 45 us here; 4096 x 4096 x 64:
+	// 52-58 and 28 us; with 96 tiles of 128 x 128 the two are level)
+	const bool short_k = K >= 64 && K < 256 && K % 32 == 0 && tiles128 >= 512;
+	if (choice == 0 && (tiles128 >= 128 || t64) && ((K >= 256 && (K % 32 == 0 || K >= 512)) || short_k)) {
 		// large problems: 256 x 256 tiles when they fill the chip, else 128 x 128 (or 64 x 64, above).  The tiles walk K in
 		// steps of 32: what is left over is added by a second, general launch (beta = 1, no bias).
-		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192;
+		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192 && M >= 192 && N >= 192 && !short_k;
 		const uint64_t k_main = K & ~31ull;
 		p.K = (int)k_main;
 		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : (t64 ? 31 : 21)) == 0) {
