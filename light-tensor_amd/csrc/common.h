@@ -22,6 +22,12 @@ bool capturing();  // a launch graph is being recorded: no allocation, no synchr
 enum Option { OPT_QGEMM_TILE = 0, OPT_SGEMM_TILE, OPT_QSKINNY, OPT_CONV_VARIANT, OPT_QGEMM_SPLIT, OPT_COUNT };
 int get_option(Option o);
 
+// Device memory the library owns for what does not fit its entry points' workspaces (padded copies of int8 operands,
+// partial sums of a reduction split over workgroups): one block per device, grown when a call needs more (never while
+// a launch graph is being recorded: nullptr then, and when there is no memory), kept until the process ends.  One
+// stream uses it at a time, as everything else in this library.
+void* library_scratch(uint64_t bytes);
+
 // Looks up the current device's copy of the static scratch of lten_hip_fcq_forward_static (qgemm.hip); 0 on success.
 int prepare_static_scratch();
 

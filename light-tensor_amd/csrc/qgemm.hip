@@ -457,39 +457,6 @@ __global__ __launch_bounds__(256) void qgemm_transpose_rows_kernel(const uint8_t
 	}
 }
 
-// Where the padded copies live: owned by the library, one block per device, grown when a call needs more (never while
-// a launch graph is being recorded), kept until the process ends.  One stream uses it at a time, as everything else
-// in this library; work queued on that stream may still read the old block when it has to grow, hence the wait.
-struct PadScratch {
-	uint8_t* base;
-	uint64_t bytes;
-};
-static PadScratch g_pad[8] = {};
-
-static uint8_t* pad_scratch(uint64_t bytes)
-{
-	int dev = -1;
-	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
-	PadScratch& ps = g_pad[dev];
-	if (ps.bytes >= bytes) return ps.base;
-	if (capturing()) return nullptr;
-	if (ps.base != nullptr) {
-		if (hipStreamSynchronize(stream()) != hipSuccess) return nullptr;
-		(void)hipFree(ps.base);
-		ps.base = nullptr;
-		ps.bytes = 0;
-	}
-	const uint64_t want = (bytes + (bytes >> 2) + (2u << 20)) & ~((2ull << 20) - 1);  // a quarter more, whole 2 MB pages
-	void* ptr = nullptr;
-	if (hipMalloc(&ptr, want) != hipSuccess) {
-		(void)hipGetLastError();
-		return nullptr;
-	}
-	ps.base = static_cast<uint8_t*>(ptr);
-	ps.bytes = want;
-	return ps.base;
-}
-
 // k_pad: the last k_pad bytes of every row of A and B are padding (QProblem::k_pad); the call that pads passes it
 static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const uint8_t* A, const uint8_t* B, void* C,
                      int out_acc, const lten_hip_qparams* qp, const int32_t* bias, int32_t* workspace,
@@ -518,7 +485,7 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		const uint64_t Kp = (K + 15) & ~15ull;
 		const bool copy_a = tA || Kp != K, copy_b = !weights_prepared && (!tB || Kp != K);
 		const uint64_t bytes_a = copy_a ? M * Kp : 0, bytes_b = copy_b ? N * Kp : 0;
-		uint8_t* buf = pad_scratch(bytes_a + bytes_b);
+		uint8_t* buf = static_cast<uint8_t*>(library_scratch(bytes_a + bytes_b));
 		LTEN_HIP_REQUIRE(buf != nullptr || !weights_prepared,
 		                 "quantized_matmul: no memory for the padded copy of the activations (in_features = %llu is no multiple of 16; while a "
 		                 "launch graph is being recorded the copy's memory cannot be allocated: run the call once before recording)",

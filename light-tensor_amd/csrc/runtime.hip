@@ -42,6 +42,37 @@ void set_kernel_name(const char* name)
 hipStream_t stream() { return g_stream; }
 bool capturing() { return g_capturing; }
 
+// (work queued on the stream may still read the old block when it has to grow, hence the wait)
+struct LibraryScratch {
+	void* base;
+	uint64_t bytes;
+};
+static LibraryScratch g_scratch[8] = {};
+
+void* library_scratch(uint64_t bytes)
+{
+	int dev = -1;
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
+	LibraryScratch& ls = g_scratch[dev];
+	if (ls.bytes >= bytes) return ls.base;
+	if (capturing()) return nullptr;
+	if (ls.base != nullptr) {
+		if (hipStreamSynchronize(stream()) != hipSuccess) return nullptr;
+		(void)hipFree(ls.base);
+		ls.base = nullptr;
+		ls.bytes = 0;
+	}
+	const uint64_t want = (bytes + (bytes >> 2) + (2u << 20)) & ~((2ull << 20) - 1);  // a quarter more, whole 2 MB pages
+	void* ptr = nullptr;
+	if (hipMalloc(&ptr, want) != hipSuccess) {
+		(void)hipGetLastError();
+		return nullptr;
+	}
+	ls.base = ptr;
+	ls.bytes = want;
+	return ls.base;
+}
+
 static int g_options[OPT_COUNT] = { 0 };
 static const char* const g_option_names[OPT_COUNT] = { "qgemm_tile", "sgemm_tile", "qskinny", "conv_variant", "qgemm_split" };
 int get_option(Option o) { return g_options[o]; }

@@ -949,6 +949,18 @@ static int launch_sgemm(const SProblem& p, int tA, int tB, uint64_t batch, const
 	return 0;
 }
 
+// C = alpha * (partial[0] + partial[1] + ...) + beta * C, the partial matrices [parts][M][N] added in index order
+__global__ __launch_bounds__(256) void sgemm_add_partials_kernel(const float* __restrict__ partial, int parts, int M, int N, float alpha, float beta,
+                                                                 float* __restrict__ C, int64_t ldc)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, count = (int64_t)M * N;
+	if (idx >= count) return;
+	float sum = 0.0f;
+	for (int s = 0; s < parts; s++) sum += partial[(int64_t)s * count + idx];
+	float* c = C + (idx / N) * ldc + idx % N;
+	*c = beta == 0.0f ? alpha * sum : alpha * sum + beta * *c;
+}
+
 int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
               int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
               int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done, float* relu_out = nullptr,
@@ -969,6 +981,34 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 			if (rc) return rc;
 		}
 		return 0;
+	}
+	// A long reduction into a small output (the weight gradient of a small layer over a large batch: 128 x 128 x 16384)
+	// gives the kernels below a handful of workgroups that each walk all of K: 114 us where the operands' 17 MB take 5.
+	// K is cut into up to 64 slices (of 512 or more) that run as one strided batch into partial matrices (in memory the library owns),
+	// which a second launch adds up in the order of the slices, so the result does not depend on timing.
+	// (Not where the weight-streaming kernels below take the product: few rows against a long or wide weight matrix,
+	// l-ten's 5760 -> 50 layer at batch 64, is their shape and cuts K over a workgroup's wavefronts already.)
+	const bool streams = (!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512);
+	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && bias == nullptr && !streams && K >= 4096 && ceil_div(M, 32) * ceil_div(N, 32) <= 256) {
+		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);
+		uint64_t slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
+		while (slices > 2 && K / slices < 512) slices /= 2;
+		const uint64_t kc = (K / slices) & ~31ull, rest = K - slices * kc, parts = slices + (rest != 0 ? 1 : 0);
+		float* partial = kc >= 256 ? static_cast<float*>(library_scratch(parts * M * N * sizeof(float))) : nullptr;
+		if (partial != nullptr) {
+			int rc = sgemm_run(tA, tB, M, N, kc, 1.0f, A, lda, (int64_t)(tA ? kc * lda : kc), B, ldb, (int64_t)(tB ? kc : kc * ldb), 0.0f, partial, N,
+			                   (int64_t)(M * N), slices, nullptr, nullptr, nullptr);
+			if (rc) return rc;
+			if (rest != 0) {
+				rc = sgemm_run(tA, tB, M, N, rest, 1.0f, A + (tA ? slices * kc * lda : slices * kc), lda, 0, B + (tB ? slices * kc : slices * kc * ldb), ldb, 0,
+				               0.0f, partial + slices * M * N, N, 0, 1, nullptr, nullptr, nullptr);
+				if (rc) return rc;
+			}
+			set_kernel_name("sgemm_split_k");
+			sgemm_add_partials_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(partial, (int)parts, (int)M, (int)N, alpha, beta, C, (int64_t)ldc);
+			LTEN_HIP_LAUNCH_CHECK();
+			return 0;
+		}
 	}
 	SProblem p;
 	p.A = A; p.B = B; p.C = C; p.bias = bias; p.rowsum = nullptr; p.relu_out = nullptr; p.relu_in = nullptr;

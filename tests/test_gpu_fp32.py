@@ -54,6 +54,39 @@ def test_integer_valued_exact_with_leading_dims(gpu, tile, tA, tB):
     assert np.array_equal(got2[:, :N], want)
 
 
+@pytest.mark.parametrize("tA,tB,M,N,K", [(1, 0, 128, 128, 16384), (1, 0, 10, 32, 20011), (0, 0, 64, 200, 8200), (0, 1, 100, 37, 4099 + 2),
+                                          (1, 1, 256, 256, 4096), (1, 0, 64, 64, 65536)])
+def test_long_reduction_into_a_small_output_is_split(gpu, tA, tB, M, N, K):
+    """The weight gradient of a small layer over a large batch: K is cut into slices that run as a batch into partial
+    matrices, added in slice order by a second launch.  Integer-valued operands come out exactly whatever the order;
+    alpha, beta and padded leading dimensions as in every other route; two runs give the same bits."""
+    rng = np.random.default_rng(M + N + K + 2 * tA + tB)
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    want = (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32)
+    lda, ldb, ldc = (M if tA else K) + 4, (K if tB else N) + 8, N + 3
+    As = np.zeros(((K if tA else M), lda), np.float32)
+    As[:, :(M if tA else K)] = A.T if tA else A
+    Bs = np.zeros(((N if tB else K), ldb), np.float32)
+    Bs[:, :(K if tB else N)] = B.T if tB else B
+    C0 = np.full((M, ldc), 7.0, np.float32)
+    got = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, C0, ldc)
+    assert gpu.last_kernel() == "sgemm_split_k", gpu.last_kernel()
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, tA, tB, M, N, K, 2.0, As, lda, Bs, ldb, -1.0, got, ldc)
+    assert np.array_equal(got2[:, :N], want)
+    # real-valued operands: within the tolerance of every other route, and the same bits on a second run
+    Ar = rng.standard_normal(As.shape).astype(np.float32)
+    Br = rng.standard_normal(Bs.shape).astype(np.float32)
+    a64 = (Ar[:, :M].T if tA else Ar[:, :K]).astype(np.float64)
+    b64 = (Br[:, :K].T if tB else Br[:, :N]).astype(np.float64)
+    r1 = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, Ar, lda, Br, ldb, 0.0, C0, ldc)
+    r2 = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, Ar, lda, Br, ldb, 0.0, C0, ldc)
+    assert np.array_equal(r1, r2)
+    assert rel_err(r1[:, :N], (a64 @ b64).astype(np.float32)) < TOL
+
+
 def test_beta_zero_overwrites_nan(gpu):
     A = np.ones((5, 3), np.float32)
     B = np.ones((3, 6), np.float32)
