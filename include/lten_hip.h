@@ -82,7 +82,9 @@ int lten_hip_fill_u8(uint8_t* device_ptr, uint64_t count, uint8_t value);
  * l-ten/backprop.cpp:562,580,2003,2024,2228,2252,2267).  beta == 0 overwrites C
  * (NaN/Inf in C are not propagated); A and B are never modified.  The K == 1
  * (bias rank-1 update) and M == 1 (bias-gradient column sum) shapes those sites use
- * are served by dedicated kernels. */
+ * are served by dedicated kernels.  A reduction of 4096 or more into a small output
+ * (a weight gradient over a large batch) is cut into slices whose partial sums live in
+ * memory the library owns and are added in a fixed order. */
 int lten_hip_sgemm(int trans_a, int trans_b, uint64_t M, uint64_t N, uint64_t K, float alpha,
                    const float* A, uint64_t lda, const float* B, uint64_t ldb, float beta,
                    float* C, uint64_t ldc);
