@@ -260,6 +260,29 @@ def test_conv_data_gradient_with_strides(gpu, ob, geo):
     assert rel_err(dx, want_dx) < TOL
 
 
+@pytest.mark.parametrize("geo", [(3, 64, 20, 20, 48, 1, 1, 0, 0, 1, 1), (2, 100, 13, 17, 70, 1, 1, 0, 0, 1, 1), (5, 40, 56, 56, 256, 1, 1, 0, 0, 1, 1)])
+def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
+    """A 1 x 1 layer without bias, and its data gradient, run as a strided batch of plain products on the images as they
+    lie in memory; with a bias the layer stays on the convolution kernels.  Both against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, 1, 1)) * 0.2).astype(np.float32)
+    dy = rng.standard_normal((N, Cout, H, W)).astype(np.float32)
+    col = np.empty(Cin * H * W, np.float32)
+    want_y = np.empty((N, Cout, H, W), np.float32)
+    ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
+    y, _, fk = gpu_conv(gpu, geo, x, w)
+    assert fk == "conv2d_1x1_batched_gemm", fk
+    assert rel_err(y, want_y) < TOL
+    want_dx = np.empty_like(x)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_1x1_batched_gemm", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+    _conv_vs_oracle(gpu, ob, geo)   # with a bias: the convolution kernels
+
+
 def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
     """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
     padding costs more than l-ten's own decomposition (GEMM + col2im image by image), which the library then takes."""
