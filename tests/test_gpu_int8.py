@@ -626,6 +626,32 @@ def test_operands_that_lie_with_k_outermost(gpu, ob, shape, tA, tB):
         assert "guard" not in gpu.last_kernel(), gpu.last_kernel()
 
 
+def test_padded_rows_inside_a_recorded_launch_graph(gpu, ob):
+    """A prepared layer of 1000 inputs run once eagerly (which allocates the memory of the padded copy) and then
+    recorded: the copy and the product both land in the graph, and every replay on new activations matches the oracle."""
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    rng = np.random.default_rng(1000)
+    M, N, K = 96, 512, 1000
+    Kp = (K + 15) // 16 * 16
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    sc, zp = [0.02, 0.013, 0.9], [5, 200, 90]
+    dX, dW, dWp, dS, dY, ws = D(M * K), D.from_numpy(W), D(N * Kp), D(4 * N), D(M * N), D(4 * (M + N))
+    gpu.check(l.lten_hip_fcq_prepare_weights(dW.ptr, dWp.ptr, N, K, dS.ptr))
+    qp = gpu.qparams3(sc, zp)
+    call = lambda: gpu.check(l.lten_hip_fcq_forward_prepared(1, M, K, N, dX.ptr, dWp.ptr, dS.ptr, None, qp, dY.ptr, ws.ptr))
+    dX.upload(rng.integers(0, 256, (M, K), dtype=np.uint8))
+    call()
+    with gpu.Graph() as g:
+        call()
+    for rep in range(3):
+        X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+        dX.upload(X)
+        gpu.check(l.lten_hip_zero(dY.ptr, M * N))
+        g.launch()
+        want, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8))
+        assert np.array_equal(dY.numpy(np.uint8, (M, N)), want), rep
+
+
 def test_prepare_weights_in_place_and_odd_count(gpu):
     rng = np.random.default_rng(5)
     for n in (16, 4096, 1 << 20):   # rows that are multiples of 16 bytes: in place
