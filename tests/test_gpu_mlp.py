@@ -213,6 +213,38 @@ def test_fused_fc_relu_entry_points_match_the_unfused_calls(gpu, shape):
     assert np.array_equal(b0.numpy(np.float32, b.shape), b1.numpy(np.float32, b.shape))
 
 
+@pytest.mark.parametrize("rows,cols", [(2000, 16), (5000, 10), (3000, 32), (4001, 20), (1024, 1), (64, 50257), (7, 1024), (300, 2048), (9, 8192),
+                                       (3, 70000), (2, 8193), (33, 1500), (1023, 16), (100, 1023), (500, 256), (40, 255), (2000, 1000)])
+def test_log_softmax_on_narrow_and_wide_rows(gpu, rows, cols):
+    """Rows of at most 32 values share a wavefront, rows of 256 and more take a workgroup each: forward and backward
+    against float64 within the fp32 tolerance, the same bits on a second run, and rows that hold large and equal values."""
+    rng = np.random.default_rng(rows * 3 + cols)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    x = (rng.standard_normal((rows, cols)) * 4).astype(np.float32)
+    x[0, :] = 80.0                       # equal values: log(1 / cols)
+    if cols > 1:
+        x[-1, 0] = 300.0                 # one dominant value: exp of the others underflows
+    dy = rng.standard_normal((rows, cols)).astype(np.float32)
+    dx_, dg = D.from_numpy(x), D.from_numpy(dy)
+    y0, y1, g0 = D(x.nbytes), D(x.nbytes), D(x.nbytes)
+    gpu.check(l.lten_hip_log_softmax_f32(rows, cols, dx_.ptr, y0.ptr))
+    gpu.check(l.lten_hip_log_softmax_f32(rows, cols, dx_.ptr, y1.ptr))
+    y = y0.numpy(np.float32, x.shape)
+    assert np.array_equal(y, y1.numpy(np.float32, x.shape))
+    x64 = x.astype(np.float64)
+    m = x64.max(axis=1, keepdims=True)
+    e = np.exp(x64 - m)
+    with np.errstate(divide="ignore"):
+        want = np.log(e.astype(np.float32).astype(np.float64) / e.sum(axis=1, keepdims=True))   # l-ten's chain: log(exp(x - max) / sum)
+    finite = np.isfinite(want)
+    assert np.array_equal(np.isfinite(y), finite)
+    assert np.abs(y[finite] - want[finite]).max() < 1e-4 * max(1.0, np.abs(want[finite]).max())
+    gpu.check(l.lten_hip_log_softmax_backward_f32(rows, cols, y0.ptr, dg.ptr, g0.ptr))
+    g = g0.numpy(np.float32, x.shape)
+    want_g = dy.astype(np.float64) - np.exp(y.astype(np.float64)) * dy.astype(np.float64).sum(axis=1, keepdims=True)
+    assert np.abs(g - want_g).max() < 1e-4 * max(1.0, np.abs(want_g).max())
+
+
 def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
     rng = np.random.default_rng(11)
     D, l = gpu.DeviceBuffer, gpu.lib()
