@@ -102,14 +102,15 @@ __global__ __launch_bounds__(256) void log_softmax_narrow_kernel(uint64_t rows, 
 	if (live) y[row * cols + sub] = logf(e / t);
 }
 
-template <int LPR>
+// (SCALED: the incoming gradient is alpha times dy, as nll_log_softmax_backward_kernel takes it)
+template <int LPR, bool SCALED = false>
 __global__ __launch_bounds__(256) void log_softmax_backward_narrow_kernel(uint64_t rows, int cols, const float* __restrict__ y, const float* __restrict__ dy,
-                                                                          float* __restrict__ dx)
+                                                                          float* __restrict__ dx, float alpha = 1.0f)
 {
 	const int lane = threadIdx.x & 63, sub = lane % LPR;
 	const uint64_t row = ((uint64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * (64 / LPR) + lane / LPR;
 	const bool live = row < rows && sub < cols;
-	const float g = live ? dy[row * cols + sub] : 0.0f;
+	const float g = live ? (SCALED ? alpha * dy[row * cols + sub] : dy[row * cols + sub]) : 0.0f;
 	float t = g;
 #pragma unroll
 	for (int o = 32; o >= LPR; o >>= 1) t += 0.0f;
@@ -175,9 +176,9 @@ __global__ __launch_bounds__(T) void log_softmax_wide_kernel(uint64_t cols, cons
 	}
 }
 
-template <int T, int R, bool FITS>
+template <int T, int R, bool FITS, bool SCALED = false>
 __global__ __launch_bounds__(T) void log_softmax_backward_wide_kernel(uint64_t cols, const float* __restrict__ y, const float* __restrict__ dy,
-                                                                      float* __restrict__ dx)
+                                                                      float* __restrict__ dx, float alpha = 1.0f)
 {
 	__shared__ float part[T / 64];
 	const int tid = threadIdx.x;
@@ -190,11 +191,11 @@ __global__ __launch_bounds__(T) void log_softmax_backward_wide_kernel(uint64_t c
 #pragma unroll
 		for (int i = 0; i < R; i++) {
 			const uint64_t c = (uint64_t)tid + (uint64_t)i * T;
-			g[i] = c < cols ? gr[c] : 0.0f;
+			g[i] = c < cols ? (SCALED ? alpha * gr[c] : gr[c]) : 0.0f;
 			s += g[i];
 		}
 	} else {
-		for (uint64_t c = tid; c < cols; c += T) s += gr[c];
+		for (uint64_t c = tid; c < cols; c += T) s += SCALED ? alpha * gr[c] : gr[c];
 	}
 	s = wave_sum(s);
 	if ((tid & 63) == 0) part[tid >> 6] = s;
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(T) void log_softmax_backward_wide_kernel(uint64_t c
 			if (c < cols) dr[c] = g[i] - expf(yr[c]) * s;
 		}
 	} else {
-		for (uint64_t c = tid; c < cols; c += T) dr[c] = gr[c] - expf(yr[c]) * s;
+		for (uint64_t c = tid; c < cols; c += T) dr[c] = (SCALED ? alpha * gr[c] : gr[c]) - expf(yr[c]) * s;
 	}
 }
 
@@ -229,6 +230,35 @@ __global__ __launch_bounds__(1024) void nll_loss_kernel(const float* __restrict_
 		for (int w = 0; w < 16; w++) tot += part[w];
 		*loss = tot * scale;
 	}
+}
+
+// The same sum for long arrays (the log-probabilities of a large batch over a large vocabulary: one workgroup took 9.6
+// ms over 32768 x 1000 values): workgroup b sums a contiguous share the way the kernel above sums the whole array and
+// leaves it in partial[b]; a second launch of the kernel below adds the shares in index order and scales.
+__global__ __launch_bounds__(1024) void nll_loss_partial_kernel(const float* __restrict__ input, const float* __restrict__ target, float* __restrict__ partial,
+                                                                uint64_t len, uint64_t share)
+{
+	__shared__ float part[16];
+	const uint64_t begin = (uint64_t)blockIdx.x * share, end = begin + share < len ? begin + share : len;
+	float s = 0.0f;
+	for (uint64_t i = begin + threadIdx.x; i < end; i += 1024) s += input[i] * target[i];
+	s = wave_sum(s);
+	if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		float tot = 0.0f;
+#pragma unroll
+		for (int w = 0; w < 16; w++) tot += part[w];
+		partial[blockIdx.x] = tot;
+	}
+}
+
+__global__ __launch_bounds__(64) void nll_loss_finish_kernel(const float* __restrict__ partial, int count, float* __restrict__ loss, float scale)
+{
+	if (threadIdx.x != 0) return;
+	float tot = 0.0f;
+	for (int b = 0; b < count; b++) tot += partial[b];
+	*loss = tot * scale;
 }
 
 // log_softmax, nll_loss and (GRAD) the gradient of the loss with respect to the logits for a small batch of narrow
@@ -497,6 +527,18 @@ int lten_hip_nll_loss_f32(const float* input, const float* target, float* loss, 
 {
 	LTEN_HIP_REQUIRE(loss != nullptr && batches > 0, "nll_loss: null loss pointer or zero batch");
 	LTEN_HIP_REQUIRE(len == 0 || (input && target), "nll_loss: null pointer");
+	// (up to 65536 values one workgroup: the order of that sum is the one the one-launch loss kernels reproduce)
+	constexpr uint64_t SHARE = 32768;
+	float* partial = len > 65536 ? static_cast<float*>(library_scratch(4096 * sizeof(float))) : nullptr;
+	if (partial != nullptr) {
+		const uint64_t share = std::max<uint64_t>(SHARE, (ceil_div(len, 2048) + 1023) / 1024 * 1024);  // at most 2048 shares, whole rounds of the workgroup
+		const unsigned count = (unsigned)ceil_div(len, share);
+		nll_loss_partial_kernel<<<dim3(count), dim3(1024), 0, stream()>>>(input, target, partial, len, share);
+		LTEN_HIP_LAUNCH_CHECK();
+		nll_loss_finish_kernel<<<dim3(1), dim3(64), 0, stream()>>>(partial, (int)count, loss, -1.0f / (float)batches);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	nll_loss_kernel<<<dim3(1), dim3(1024), 0, stream()>>>(input, target, loss, len, -1.0f / (float)batches);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
@@ -537,7 +579,14 @@ int lten_hip_nll_log_softmax_backward_f32(uint64_t rows, uint64_t cols, const fl
 {
 	if (rows == 0 || cols == 0) return 0;
 	LTEN_HIP_REQUIRE(y && target && dx, "nll_log_softmax_backward: null pointer");
-	nll_log_softmax_backward_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, y, target, alpha, dx);
+	// the forms of lten_hip_log_softmax_backward_f32 for narrow and wide rows, fed alpha * target
+	if (cols <= 16 && rows >= 1024) log_softmax_backward_narrow_kernel<16, true><<<dim3((unsigned)ceil_div(rows, 16)), dim3(256), 0, stream()>>>(rows, (int)cols, y, target, dx, alpha);
+	else if (cols <= 32 && rows >= 1024) log_softmax_backward_narrow_kernel<32, true><<<dim3((unsigned)ceil_div(rows, 8)), dim3(256), 0, stream()>>>(rows, (int)cols, y, target, dx, alpha);
+	else if (cols >= 256 && cols <= 2048) log_softmax_backward_wide_kernel<256, 8, true, true><<<dim3((unsigned)rows), dim3(256), 0, stream()>>>(cols, y, target, dx, alpha);
+	else if (cols > 2048 && cols <= 8192) log_softmax_backward_wide_kernel<256, 32, true, true><<<dim3((unsigned)rows), dim3(256), 0, stream()>>>(cols, y, target, dx, alpha);
+	else if (cols > 8192 && cols <= 65536) log_softmax_backward_wide_kernel<1024, 64, true, true><<<dim3((unsigned)rows), dim3(1024), 0, stream()>>>(cols, y, target, dx, alpha);
+	else if (cols > 65536) log_softmax_backward_wide_kernel<1024, 1, false, true><<<dim3((unsigned)rows), dim3(1024), 0, stream()>>>(cols, y, target, dx, alpha);
+	else nll_log_softmax_backward_kernel<<<dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream()>>>(rows, cols, y, target, alpha, dx);
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
 }

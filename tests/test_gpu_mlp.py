@@ -245,6 +245,29 @@ def test_log_softmax_on_narrow_and_wide_rows(gpu, rows, cols):
     assert np.abs(g - want_g).max() < 1e-4 * max(1.0, np.abs(want_g).max())
 
 
+@pytest.mark.parametrize("rows,cols", [(4096, 1000), (64, 50257), (1 << 18, 16), (700, 100), (65537, 1)])
+def test_nll_loss_over_long_arrays(gpu, rows, cols):
+    """Beyond 65536 values the loss is summed share by share on many workgroups and the shares in index order: against
+    float64, twice the same bits, and through the entry points that stand for several launches."""
+    rng = np.random.default_rng(rows + cols)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    x = (rng.standard_normal((rows, cols)) * 3).astype(np.float32)
+    labels = rng.integers(0, cols, rows)
+    t = np.zeros((rows, cols), np.float32)
+    t[np.arange(rows), labels] = 1.0
+    dx_, dt, y, l0, l1, l2, g = D.from_numpy(x), D.from_numpy(t), D(x.nbytes), D(4), D(4), D(4), D(x.nbytes)
+    gpu.check(l.lten_hip_log_softmax_f32(rows, cols, dx_.ptr, y.ptr))
+    gpu.check(l.lten_hip_nll_loss_f32(y.ptr, dt.ptr, l0.ptr, rows * cols, rows))
+    gpu.check(l.lten_hip_nll_loss_f32(y.ptr, dt.ptr, l1.ptr, rows * cols, rows))
+    logp = y.numpy(np.float32, x.shape)
+    want = -logp[np.arange(rows), labels].astype(np.float64).sum() / rows
+    got = float(l0.numpy(np.float32, (1,))[0])
+    assert got == float(l1.numpy(np.float32, (1,))[0])
+    assert abs(got - want) < 1e-4 * max(1.0, abs(want)), (got, want)
+    gpu.check(l.lten_hip_log_softmax_nll_loss_grad_f32(rows, cols, dx_.ptr, dt.ptr, -1.0 / rows, y.ptr, l2.ptr, g.ptr))
+    assert float(l2.numpy(np.float32, (1,))[0]) == got
+
+
 def test_fused_loss_entry_points_match_the_unfused_calls(gpu):
     rng = np.random.default_rng(11)
     D, l = gpu.DeviceBuffer, gpu.lib()
