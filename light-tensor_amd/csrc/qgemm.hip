@@ -560,20 +560,9 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 		const int rc = qskinny_dispatch(p, out, bias, zpA, zpB);
 		if (rc >= 0) return rc;
 	}
-	// 33 to 64 rows: two streaming passes (32 rows, then the rest) still beat one pass of 128-row tiles, three would not;
-	// with a short K the tiles win (4096 x 1024 weights: 8.2 us against 9.7-11.3 us)
-	if (M > 32 && M <= 64 && N >= 2048 && K >= 2048 && K <= 8192 && may_stream) {
-		QProblem top = p, rest = p;
-		top.M = 32;
-		rest.M = (int)M - 32;
-		rest.A = p.A + 32 * p.a_rs;
-		rest.C = static_cast<uint8_t*>(p.C) + (uint64_t)32 * N * (out == Q_OUT_ACC ? 4 : 1);
-		if (qskinny_dispatch(top, out, bias, zpA, zpB) == 0) {
-			const int rc = qskinny_dispatch(rest, out, bias, zpA, zpB);
-			LTEN_HIP_REQUIRE(rc == 0, "quantized_matmul: the second streaming pass did not launch");
-			return 0;
-		}
-	}
+	// (33 to 64 rows used to take two streaming passes, 32 rows and the rest; the 128 x 128 tiles with their split K have
+	// since overtaken that: 64 x 4096 x 4096 15.3 against 18.0 us, 64 x 8192 x 8192 25.4 against 32.3 us, 40 x 11008 x
+	// 4096 17.5 against 24.2 us)
 	// small outputs: one launch that also takes the zero-point sums (same option switches it off)
 	if (may_stream) {
 		int rc = qdirect_dispatch(p, out, bias, zpA, zpB);
