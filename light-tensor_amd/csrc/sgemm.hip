@@ -973,6 +973,13 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	LTEN_HIP_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "sgemm: null operand");
 	LTEN_HIP_REQUIRE(M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) && batch < 65536, "sgemm: dimension too large");
 	LTEN_HIP_REQUIRE(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N, "sgemm: leading dimension smaller than the row");
+	if (batch > 1 && stride_c == 0 && tA && !tB && bias == nullptr && stride_a == (int64_t)(K * lda) && stride_b == (int64_t)(K * ldb) &&
+	    batch * K < (1ull << 31)) {
+		// The problems' operands lie one behind the other along the reduction (the gradient of a matrix that a stack of
+		// matrices was multiplied by: dB = sum over the stack of A_i^T dC_i, l-ten/backprop.cpp:533-585): one product with
+		// batch * K rows to reduce over, instead of batch launches that each add to C.
+		return sgemm_run(1, 0, M, N, batch * K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, nullptr, nullptr, nullptr);
+	}
 	if (batch > 1 && stride_c == 0) {
 		// every problem writes the same C: run them one after another so the sum has one fixed order
 		for (uint64_t b = 0; b < batch; b++) {

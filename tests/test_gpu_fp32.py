@@ -248,6 +248,21 @@ def test_strided_batched_and_broadcast(gpu, ob):
     assert rel_err(dDB.numpy(np.float32, db.shape), db) < TOL
 
 
+@pytest.mark.parametrize("batch,M,K,N", [(64, 100, 96, 80), (7, 33, 50, 20), (512, 64, 32, 48)])
+def test_gradient_of_a_broadcast_matrix_over_a_stack(gpu, batch, M, K, N):
+    """dB = sum_i A_i^T dC_i for a[batch, M, K] x b[K, N] (b shared by the stack): the stack lies along the reduction, so the
+    batch that all writes one C runs as a single product over batch * M rows; with beta = 1 on top of what dB held."""
+    rng = np.random.default_rng(batch + M + K + N)
+    a = rng.standard_normal((batch, M, K)).astype(np.float32)
+    dc = rng.standard_normal((batch, M, N)).astype(np.float32)
+    db0 = rng.standard_normal((K, N)).astype(np.float32)
+    D = gpu.DeviceBuffer
+    dA, dDC, dDB = D.from_numpy(a), D.from_numpy(dc), D.from_numpy(db0)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(1, 0, K, N, M, 1.0, dA.ptr, K, M * K, dDC.ptr, N, M * N, 1.0, dDB.ptr, N, 0, batch))
+    want = db0.astype(np.float64) + np.einsum("bmk,bmn->kn", a.astype(np.float64), dc.astype(np.float64))
+    assert rel_err(dDB.numpy(np.float32, (K, N)), want.astype(np.float32)) < TOL, gpu.last_kernel()
+
+
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     cases = []
