@@ -973,6 +973,12 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	LTEN_HIP_REQUIRE(K == 0 || (A != nullptr && B != nullptr), "sgemm: null operand");
 	LTEN_HIP_REQUIRE(M < (1ull << 31) && N < (1ull << 31) && K < (1ull << 31) && batch < 65536, "sgemm: dimension too large");
 	LTEN_HIP_REQUIRE(lda >= (tA ? M : K) && ldb >= (tB ? K : N) && ldc >= N, "sgemm: leading dimension smaller than the row");
+	if (batch > 1 && !tA && stride_b == 0 && stride_a == (int64_t)(M * lda) && stride_c == (int64_t)(M * ldc) && batch * M < (1ull << 31) && rowsum == nullptr &&
+	    relu_done == nullptr) {
+		// A stack of matrices against one shared matrix, the stack's rows one behind the other in A and in C: one product
+		// with batch * M rows (1024 x (16 x 128) against 128 x 128 is 16384 x 128 x 128, not 1024 products of 16 rows).
+		return sgemm_run(0, tB, batch * M, N, K, alpha, A, lda, 0, B, ldb, 0, beta, C, ldc, 0, 1, bias, nullptr, nullptr);
+	}
 	if (batch > 1 && stride_c == 0 && tA && !tB && bias == nullptr && stride_a == (int64_t)(K * lda) && stride_b == (int64_t)(K * ldb) &&
 	    batch * K < (1ull << 31)) {
 		// The problems' operands lie one behind the other along the reduction (the gradient of a matrix that a stack of

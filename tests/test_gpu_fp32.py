@@ -263,6 +263,23 @@ def test_gradient_of_a_broadcast_matrix_over_a_stack(gpu, batch, M, K, N):
     assert rel_err(dDB.numpy(np.float32, (K, N)), want.astype(np.float32)) < TOL, gpu.last_kernel()
 
 
+@pytest.mark.parametrize("tB", [0, 1])
+@pytest.mark.parametrize("batch,M,K,N", [(64, 10, 96, 80), (7, 33, 50, 20), (300, 16, 128, 128)])
+def test_stack_against_one_shared_matrix(gpu, batch, M, K, N, tB):
+    """a[batch, M, K] x b[K, N] (or b^T given as [N, K]) with b shared by the stack (stride 0) and the stack's matrices one
+    behind the other in a and c: runs as one product with batch * M rows; alpha, beta as in every route."""
+    rng = np.random.default_rng(batch + M + K + N + tB)
+    a = rng.standard_normal((batch, M, K)).astype(np.float32)
+    b = rng.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    c0 = rng.standard_normal((batch, M, N)).astype(np.float32)
+    D = gpu.DeviceBuffer
+    dA, dB, dC = D.from_numpy(a), D.from_numpy(b), D.from_numpy(c0)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(0, tB, M, N, K, 0.5, dA.ptr, K, M * K, dB.ptr, K if tB else N, 0, 2.0, dC.ptr, N, M * N, batch))
+    b64 = (b.T if tB else b).astype(np.float64)
+    want = 0.5 * a.astype(np.float64) @ b64 + 2.0 * c0
+    assert rel_err(dC.numpy(np.float32, c0.shape), want.astype(np.float32)) < TOL, gpu.last_kernel()
+
+
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     cases = []
