@@ -46,6 +46,7 @@ bool capturing() { return g_capturing; }
 struct LibraryScratch {
 	void* base;
 	uint64_t bytes;
+	bool recorded;  // a launch graph holds this block's address: it is never freed
 };
 static LibraryScratch g_scratch[8] = {};
 
@@ -54,13 +55,18 @@ void* library_scratch(uint64_t bytes)
 	int dev = -1;
 	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
 	LibraryScratch& ls = g_scratch[dev];
-	if (ls.bytes >= bytes) return ls.base;
+	if (ls.bytes >= bytes) {
+		if (capturing()) ls.recorded = true;
+		return ls.base;
+	}
 	if (capturing()) return nullptr;
 	if (ls.base != nullptr) {
 		if (hipStreamSynchronize(stream()) != hipSuccess) return nullptr;
-		(void)hipFree(ls.base);
+		// a block whose address a recorded graph replays stays allocated for the rest of the process; any other is freed
+		if (!ls.recorded) (void)hipFree(ls.base);
 		ls.base = nullptr;
 		ls.bytes = 0;
+		ls.recorded = false;
 	}
 	const uint64_t want = (bytes + (bytes >> 2) + (2u << 20)) & ~((2ull << 20) - 1);  // a quarter more, whole 2 MB pages
 	void* ptr = nullptr;

@@ -651,6 +651,16 @@ def test_padded_rows_inside_a_recorded_launch_graph(gpu, ob):
         g.launch()
         want, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8))
         assert np.array_equal(dY.numpy(np.uint8, (M, N)), want), rep
+        if rep == 1:
+            # an eager call that needs far more of that memory than anything before it: the library takes a new block,
+            # and the one whose address the recording holds must stay where it is for the replay that follows
+            Mb, Nb = 60000, 16
+            Xb = rng.integers(0, 256, (Mb, K), dtype=np.uint8)
+            Wb = rng.integers(0, 256, (Nb, K), dtype=np.uint8)
+            dXb, dWb, dYb, wsb = D.from_numpy(Xb), D.from_numpy(Wb), D(Mb * Nb), D(4 * (Mb + Nb))
+            gpu.check(l.lten_hip_fcq_forward(1, Mb, K, Nb, dXb.ptr, dWb.ptr, None, qp, dYb.ptr, wsb.ptr))
+            wb, _ = ob.quantized_matmul(Xb[:500], Wb, np.array(sc, np.float32), np.array(zp, np.uint8))
+            assert np.array_equal(dYb.numpy(np.uint8, (Mb, Nb))[:500], wb)
 
 
 def test_prepare_weights_in_place_and_odd_count(gpu):
