@@ -1130,11 +1130,16 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 }
 
 // Whether sgemm_run sends a product without bias and batch (M x N x K, neither M, N nor K equal to 1) to the 32x32
-// kernels: not large enough for the direct-to-LDS tiles, and few tiles or operands that allow 16-byte loads.
+// kernels: not large enough for the direct-to-LDS tiles (nor a short reduction over many of them), and few tiles or
+// operands that allow 16-byte loads.
 static bool takes_32x32(const SProblem& p, uint64_t M, uint64_t N, uint64_t K)
 {
 	if (K <= 1 || M <= 1) return false;
-	if (ceil_div(M, 128) * ceil_div(N, 128) >= 128 && K >= 256) return false;
+	const uint64_t tiles128 = ceil_div(M, 128) * ceil_div(N, 128);
+	if (tiles128 >= 128 && K >= 256) return false;
+	// the short reductions sgemm_run gives to the 128 x 128 tiles, where those are clearly ahead (the weight gradient of a
+	// 4096-wide layer at a batch of 64: level; 128 x 8192 -> 8192, both gradients: 326 us with it there, 530 us without)
+	if (K >= 64 && K < 256 && K % 32 == 0 && tiles128 >= 512 && (tiles128 >= 1024 || K >= 128)) return false;
 	const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);
 	return tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20));
 }

@@ -328,6 +328,7 @@ def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     (128, 1024, 10, ("sgemm_fc_backward_pair_32x32_w8",)),           # config 2, last layer
     (1024, 2048, 2048, ("sgemm_rowvec",)),                           # direct-to-LDS tiles, then the column-sum kernel
     (640, 1101, 999, ("sgemm_rowvec",)),                             # unaligned rows, many tiles: LDS-tiled GEMM, then the column sum
+    (128, 2048, 8192, ("sgemm_rowvec",)),                            # a wide layer at a small batch: dW on the 128 x 128 tiles, no paired launch
 ])
 def test_fc_backward_bias_gradient_accumulates_on_every_route(gpu, M, fin, fout, kernels):
     """db += column sums of dY (l-ten/backprop.cpp:2267, beta = 1) whichever kernel computes dW: integer-valued
