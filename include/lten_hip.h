@@ -82,7 +82,7 @@ int lten_hip_fill_u8(uint8_t* device_ptr, uint64_t count, uint8_t value);
  * l-ten/backprop.cpp:562,580,2003,2024,2228,2252,2267).  beta == 0 overwrites C
  * (NaN/Inf in C are not propagated); A and B are never modified.  The K == 1
  * (bias rank-1 update) and M == 1 (bias-gradient column sum) shapes those sites use
- * are served by dedicated kernels.  A reduction of 4096 or more into a small output
+ * are served by dedicated kernels.  A reduction of 1536 or more into a small output
  * (a weight gradient over a large batch) is cut into slices whose partial sums live in
  * memory the library owns and are added in a fixed order. */
 int lten_hip_sgemm(int trans_a, int trans_b, uint64_t M, uint64_t N, uint64_t K, float alpha,
@@ -213,7 +213,13 @@ int lten_hip_col2im_u8(const uint8_t* col, int channels, int height, int width, 
                        uint8_t* im);
 
 /* Conv2d::forward's per-image im2col + cublasSgemm loop (l-ten/conv2d.cpp:164-171) as one
- * implicit-GEMM launch over the whole batch; no col buffer is materialised.
+ * implicit-GEMM launch over the whole batch; no col buffer is materialised, except for layers
+ * of many channels on small images (96 or more output channels, Cin*kh*kw >= 256, 64 or more
+ * output pixels in a multiple of 4, no patch kernel for the shape), which follow l-ten's scheme
+ * with the batch's column matrices (at most 512 MB) in memory the library owns: one im2col
+ * launch, one strided batch of GEMMs, one pass for the bias.  Inside a graph recording that
+ * route needs the memory to exist already (run the call once before recording it); otherwise
+ * the implicit GEMM runs.
  * x[N,Cin,H,W], w[Cout,Cin*kh*kw], y[N,Cout,Hout,Wout]; bias[Cout] may be NULL
  * (l-ten adds it afterwards as a broadcast tensor add, l-ten/conv2d.cpp:189-192). */
 int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,

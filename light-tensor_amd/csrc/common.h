@@ -27,6 +27,12 @@ int get_option(Option o);
 // a launch graph is being recorded: nullptr then, and when there is no memory), kept until the process ends.  One
 // stream uses it at a time, as everything else in this library.
 void* library_scratch(uint64_t bytes);
+// While one of these lives, library_scratch hands out nothing: for a caller that keeps data in the block across a call
+// into another entry point of the library.
+struct LibraryScratchHold {
+	LibraryScratchHold();
+	~LibraryScratchHold();
+};
 
 // Looks up the current device's copy of the static scratch of lten_hip_fcq_forward_static (qgemm.hip); 0 on success.
 int prepare_static_scratch();

@@ -2,9 +2,10 @@
 //
 // l-ten lowers Conv2d to one im2col + one GEMM per image (l-ten/conv2d.cpp:164-171 forward,
 // l-ten/backprop.cpp:1949-1953 weight gradient), writing and re-reading a [Cin*kh*kw, Hout*Wout] column
-// buffer each time.  Here the column matrix is never stored: the GEMM operand fetch computes the im2col
+// buffer each time.  Here the column matrix is not stored as a rule: the GEMM operand fetch computes the im2col
 // address on the fly (col[k][hw] = x[ci][ho*sh - ph + i][wo*sw - pw + j], zero outside the image), and one
-// launch covers the whole batch.  The standalone im2col / col2im kernels keep the semantics of l-ten's
+// launch covers the whole batch (deep layers on small images are the exception: conv_forward_by_columns).
+// The standalone im2col / col2im kernels keep the semantics of l-ten's
 // CUDA ones (l-ten/im_col.cu:65-96, 123-162) for callers that still want the buffer.
 #include "conv_common.h"
 #include "gemm_f32_core.h"
@@ -285,6 +286,94 @@ static void wgrad_split(const ConvGeo& g, int& slices, int64_t& slice_len)
 	slices = (int)ceil_div(R, (uint64_t)slice_len);
 }
 
+// The column matrices of the whole batch, col[n][k][hw] with k = (ci, i, j): a thread writes four consecutive pixels of
+// one row (n, k) per step, the threads of a row side by side, several short rows to a workgroup.  The pixel count of an
+// image is a multiple of 4 here, so every store is one of 16 bytes.
+__global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows)
+{
+	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
+	const int r = threadIdx.x / row_threads, q = threadIdx.x - r * row_threads;
+	const int64_t row = (int64_t)blockIdx.x * block_rows + r;
+	if (r >= block_rows || row >= (int64_t)g.N * Kc) return;
+	const int n = (int)(row / Kc), k = (int)(row - (int64_t)n * Kc);
+	const int ci = k / (g.kh * g.kw), ij = k - ci * (g.kh * g.kw), i = ij / g.kw, j = ij - i * g.kw;
+	const float* xc = x + ((int64_t)n * g.Cin + ci) * g.H * g.W;
+	float* out = col + row * HW;
+	for (int hw = q * 4; hw < HW; hw += row_threads * 4) {
+		int ho = hw / g.Wo, wo = hw - ho * g.Wo;
+		float v[4];
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			const int yy = ho * g.sh - g.ph + i * g.dh, xx = wo * g.sw - g.pw + j * g.dw;
+			const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W);
+			const float t = xc[(yy * g.W + xx) & -(int)inside];
+			v[e] = inside ? t : 0.0f;
+			if (++wo == g.Wo) { wo = 0; ho++; }
+		}
+		*reinterpret_cast<float4*>(out + hw) = make_float4(v[0], v[1], v[2], v[3]);
+	}
+}
+
+// y[n][co][hw] += bias[co], four pixels per thread
+__global__ __launch_bounds__(256) void conv_add_bias_kernel(float* __restrict__ y, const float* __restrict__ bias, int Cout, int hw4, int64_t total4)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= total4) return;
+	const float b = bias[(int)((idx / hw4) % Cout)];
+	float4 v = reinterpret_cast<float4*>(y)[idx];
+	v.x += b; v.y += b; v.z += b; v.w += b;
+	reinterpret_cast<float4*>(y)[idx] = v;
+}
+
+// Deep layers on small images that the patch kernels do not take (a stride, a window other than 3 x 3, images that fill
+// less than half of a patch tile): the implicit GEMM below gathers its operand element by element and runs at 45
+// TFLOP/s, the direct-to-LDS GEMM tiles at 85-90 on a column matrix that is already laid out.  With enough output
+// channels to pay for writing and reading that matrix (4 bytes per 2 x Cout flops), l-ten's own scheme is ahead: the
+// column matrices of the batch into library memory in one launch, one strided batch of products W x col_n straight into
+// y, the bias in a pass over y (32 x 256 x 14 x 14 -> 256 channels 3 x 3: 156 us on the implicit GEMM).
+// Returns -1 when the layer does not qualify or the library memory cannot be had.
+static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
+{
+	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
+	const uint64_t elems = N * Kc * HW;
+	if (!(g.Cout >= 96 && HW >= 64 && HW % 4 == 0 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) && aligned16(y) &&
+	      elems <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30))) return -1;
+	// Measured rates, on the work of whole tiles.  The implicit GEMM: 46 TFLOP/s once its 64 x 64 tiles give every CU a
+	// workgroup.  The batch of products: 110 TFLOP/s on the 64 x 64 direct-to-LDS tiles and 92 on the 128 x 128 ones, which
+	// sgemm_run picks when they fill the chip (a K that is no multiple of their k-step costs a second pass); 45 on the
+	// 32 x 32 tiles that take a batch too small for those, again in proportion to the CUs they fill.  The column matrix
+	// is written and read at 2.5 TB/s, and the two extra launches cost 8 us.
+	auto whole = [](uint64_t n, uint64_t t) { return (double)(ceil_div(n, t) * t); };
+	const double implicit_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(N * HW, 64) * (double)Kc /
+	                           (46e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 64) * ceil_div(N * HW, 64)) / 256.0));
+	const uint64_t tiles128 = ceil_div((uint64_t)g.Cout, 128) * ceil_div(HW, 128) * N, tiles64 = ceil_div((uint64_t)g.Cout, 64) * ceil_div(HW, 64) * N;
+	double gemm_us;
+	if (tiles128 >= 256) gemm_us = 2.0 * whole((uint64_t)g.Cout, 128) * whole(HW, 128) * (double)(N * Kc) / 92e6;
+	else if (tiles64 >= 128) gemm_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(HW, 64) * (double)(N * Kc) / 110e6;
+	else gemm_us = 2.0 * (double)g.Cout * (double)elems / (45e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 32) * ceil_div(HW, 32) * N) / 256.0));
+	if (Kc % 32 != 0) gemm_us *= 1.15;
+	if (implicit_us < 1.05 * (gemm_us + 4.0 * (double)elems / 2.5e6 + 8.0)) return -1;
+	float* col = static_cast<float*>(library_scratch(elems * sizeof(float)));
+	if (col == nullptr) return -1;
+	const int row_threads = (int)std::min<uint64_t>(256, HW / 4), block_rows = 256 / row_threads;
+	im2col_batch_kernel<<<dim3((unsigned)ceil_div(N * Kc, (uint64_t)block_rows)), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows);
+	LTEN_HIP_LAUNCH_CHECK();
+	int rc;
+	{
+		LibraryScratchHold hold;  // the GEMM entry must not hand the same memory to a split reduction
+		rc = lten_hip_sgemm_strided_batched(0, 0, (uint64_t)g.Cout, HW, Kc, 1.0f, w, Kc, 0, col, HW, (int64_t)(Kc * HW), 0.0f, y, HW,
+		                                    (int64_t)((uint64_t)g.Cout * HW), N);
+	}
+	if (rc != 0) return rc;
+	if (bias != nullptr) {
+		const int64_t total4 = (int64_t)(N * g.Cout * HW / 4);
+		conv_add_bias_kernel<<<dim3((unsigned)ceil_div((uint64_t)total4, 256)), dim3(256), 0, stream()>>>(y, bias, g.Cout, (int)(HW / 4), total4);
+		LTEN_HIP_LAUNCH_CHECK();
+	}
+	set_kernel_name("conv2d_im2col_batched_gemm");
+	return 0;
+}
+
 // Picks the forward kernel for a geometry (x, w, y non-null, non-empty problem).
 static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
@@ -317,6 +406,10 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	const uint64_t patch_tiles = ceil_div((uint64_t)g.Wo, 128) * ceil_div((uint64_t)g.Ho, 4) * ceil_div(Cout, 64) * N;
 	const bool narrow = variant == 0 && (g.Wo <= 56 || patch_tiles < 256);
 	if (!narrow && variant != 1 && conv_patch_forward_takes(g, x, y)) return conv_patch_forward(g, x, w, bias, y);
+	if (variant == 0) {
+		const int rc = conv_forward_by_columns(g, x, w, bias, y);
+		if (rc >= 0) return rc;
+	}
 	LTEN_HIP_REQUIRE(N * HW < (1ull << 31), "conv2d_forward: the batch's output pixels must number less than 2^31 on this route");
 	// at most 32 output channels: 32 x 128 tiles, unless those are fewer than the CUs (then half-empty 64 x 64 tiles,
 	// twice as many: 64 x 10 x 12 x 12 -> 20 channels 5 x 5: 14.7 against 18.7 us)
@@ -499,8 +592,20 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	float* work = static_cast<float*>(workspace);
 	// Few images of at most 16 columns: l-ten's decomposition (GEMM + col2im per image) is ahead of a convolution with so
 	// few columns that its workgroups walk a long reduction one after another (8 x 256 x 14 x 14 <- 512 channels: 166
-	// against 237 us; at 16 images the two launches per image cost more: 16 x 64 x 8 x 8 <- 64: 160 against 41 us)
-	const bool few_narrow = get_option(OPT_CONV_VARIANT) == 0 && W <= 16 && N <= 8 && Cin > 32;
+	// against 237 us; at 16 images the two launches per image cost more: 16 x 64 x 8 x 8 <- 64: 160 against 41 us, and
+	// so they do when the reduction is short: 8 x 64 x 8 x 8 <- 64 channels 89 us)
+	const bool few_narrow = get_option(OPT_CONV_VARIANT) == 0 && W <= 16 && N <= 8 && Cin > 32 && Cout * kh * kw >= 2048;
+	if (dgrad_as_forward(g) && few_narrow) {
+		// ... unless the transposed problem is one for the column matrices of the whole batch (8 x 256 x 14 x 14 <- 256: 60 us)
+		ConvGeo g2;
+		if (int rc = make_geo(g2, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
+		if (g2.Ho == (int)H && g2.Wo == (int)W) {
+			flip_weights_kernel<<<dim3((unsigned)std::min<uint64_t>(ceil_div(Cout * Kc, 256), 1024)), dim3(256), 0, stream()>>>(w, work, (int)Cout, (int)Cin, kh, kw);
+			LTEN_HIP_LAUNCH_CHECK();
+			const int rc = conv_forward_by_columns(g2, dy, work, nullptr, dx);
+			if (rc >= 0) return rc;
+		}
+	}
 	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1 && !few_narrow) {
 		ConvGeo gt;  // the transposed problem: dy is the input, dx the output
 		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;

@@ -50,8 +50,13 @@ struct LibraryScratch {
 };
 static LibraryScratch g_scratch[8] = {};
 
+static int g_scratch_held = 0;
+LibraryScratchHold::LibraryScratchHold() { g_scratch_held++; }
+LibraryScratchHold::~LibraryScratchHold() { g_scratch_held--; }
+
 void* library_scratch(uint64_t bytes)
 {
+	if (g_scratch_held > 0) return nullptr;
 	int dev = -1;
 	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
 	LibraryScratch& ls = g_scratch[dev];

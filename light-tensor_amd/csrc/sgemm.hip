@@ -1002,7 +1002,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// (Not where the weight-streaming kernels below take the product: few rows against a long or wide weight matrix,
 	// l-ten's 5760 -> 50 layer at batch 64, is their shape and cuts K over a workgroup's wavefronts already.)
 	const bool streams = (!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512);
-	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && bias == nullptr && !streams && K >= 4096 && ceil_div(M, 32) * ceil_div(N, 32) <= 256) {
+	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && bias == nullptr && !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256) {
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);
 		uint64_t slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
 		while (slices > 2 && K / slices < 512) slices /= 2;

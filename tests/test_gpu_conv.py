@@ -283,6 +283,36 @@ def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)   # with a bias: the convolution kernels
 
 
+@pytest.mark.parametrize("geo", [(1, 96, 12, 12, 96, 3, 3, 1, 1, 1, 1),       # one image: a single product on the 32 x 32 tiles; its data gradient the same way
+                                 (3, 64, 16, 12, 130, 3, 3, 1, 1, 2, 1),     # strides (2, 1), ragged channel blocks
+                                 (2, 60, 12, 12, 100, 3, 3, 1, 1, 1, 1),     # K = 540: whole k-steps, then the rest in a second pass
+                                 (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1)])   # enough tiles for the 64 x 64 direct-to-LDS kernel
+def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
+    """Many channels on images too small for the patch tiles: the batch's column matrices go to memory of the library in one
+    launch, a strided batch of products writes y, a pass adds the bias.  Forward (with and without bias), and the gradients
+    on their own routes, against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_y = np.empty((N, Cout, Ho, Wo), np.float32)
+    ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
+    y, _, fk = gpu_conv(gpu, geo, x, w)
+    assert fk == "conv2d_im2col_batched_gemm", fk
+    assert rel_err(y, want_y) < TOL
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    yb, _, fk = gpu_conv(gpu, geo, x, w, None, bias)
+    assert fk == "conv2d_im2col_batched_gemm", fk
+    assert rel_err(yb, want_y + bias[None, :, None, None]) < TOL
+    if geo[0] == 1:
+        dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+        gpu_dgrad(gpu, geo, w, dy)
+        assert gpu.last_kernel() == "conv2d_im2col_batched_gemm", gpu.last_kernel()
+    _conv_vs_oracle(gpu, ob, geo)
+
+
 def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
     """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
     padding costs more than l-ten's own decomposition (GEMM + col2im image by image), which the library then takes."""
