@@ -27,10 +27,10 @@ int get_option(Option o);
 // a launch graph is being recorded: nullptr then, and when there is no memory), kept until the process ends.  One
 // stream uses it at a time, as everything else in this library.
 void* library_scratch(uint64_t bytes);
-// While one of these lives, library_scratch hands out nothing: for a caller that keeps data in the block across a call
-// into another entry point of the library.
+// For a caller that keeps data in the first `bytes` of the block across a call into another entry point of the library:
+// while one of these lives, library_scratch hands out only what the block has behind those bytes and never moves it.
 struct LibraryScratchHold {
-	LibraryScratchHold();
+	explicit LibraryScratchHold(uint64_t bytes);
 	~LibraryScratchHold();
 };
 

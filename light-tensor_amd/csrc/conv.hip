@@ -291,16 +291,16 @@ static void wgrad_split(const ConvGeo& g, int& slices, int64_t& slice_len)
 // image is a multiple of 4 here, so every store is one of 16 bytes.
 __global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows)
 {
-	const int Kc = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
-	const int r = threadIdx.x / row_threads, q = threadIdx.x - r * row_threads;
-	const int64_t row = (int64_t)blockIdx.x * block_rows + r;
-	if (r >= block_rows || row >= (int64_t)g.N * Kc) return;
-	const int n = (int)(row / Kc), k = (int)(row - (int64_t)n * Kc);
-	const int ci = k / (g.kh * g.kw), ij = k - ci * (g.kh * g.kw), i = ij / g.kw, j = ij - i * g.kw;
+	const unsigned Kc = (unsigned)(g.Cin * g.kh * g.kw), HW = (unsigned)(g.Ho * g.Wo), taps = (unsigned)(g.kh * g.kw);
+	const unsigned r = threadIdx.x / (unsigned)row_threads, q = threadIdx.x - r * row_threads;
+	const unsigned n = blockIdx.y, k = blockIdx.x * block_rows + r;
+	if (r >= (unsigned)block_rows || k >= Kc) return;
+	const unsigned ci = k / taps, ij = k - ci * taps;
+	const int i = (int)(ij / (unsigned)g.kw), j = (int)ij - i * g.kw;
 	const float* xc = x + ((int64_t)n * g.Cin + ci) * g.H * g.W;
-	float* out = col + row * HW;
-	for (int hw = q * 4; hw < HW; hw += row_threads * 4) {
-		int ho = hw / g.Wo, wo = hw - ho * g.Wo;
+	float* out = col + ((int64_t)n * Kc + k) * HW;
+	for (unsigned hw = q * 4; hw < HW; hw += row_threads * 4) {
+		int ho = (int)(hw / (unsigned)g.Wo), wo = (int)hw - ho * g.Wo;
 		float v[4];
 #pragma unroll
 		for (int e = 0; e < 4; e++) {
@@ -353,14 +353,16 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	else gemm_us = 2.0 * (double)g.Cout * (double)elems / (45e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 32) * ceil_div(HW, 32) * N) / 256.0));
 	if (Kc % 32 != 0) gemm_us *= 1.15;
 	if (implicit_us < 1.05 * (gemm_us + 4.0 * (double)elems / 2.5e6 + 8.0)) return -1;
-	float* col = static_cast<float*>(library_scratch(elems * sizeof(float)));
+	// (behind the columns: room for the partial sums of a reduction that the GEMM entry splits, one image on a long K)
+	const uint64_t behind = g.N == 1 ? 65 * (uint64_t)g.Cout * HW * sizeof(float) + 4096 : 0;
+	float* col = static_cast<float*>(library_scratch(elems * sizeof(float) + behind));
 	if (col == nullptr) return -1;
 	const int row_threads = (int)std::min<uint64_t>(256, HW / 4), block_rows = 256 / row_threads;
-	im2col_batch_kernel<<<dim3((unsigned)ceil_div(N * Kc, (uint64_t)block_rows)), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows);
+	im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows);
 	LTEN_HIP_LAUNCH_CHECK();
 	int rc;
 	{
-		LibraryScratchHold hold;  // the GEMM entry must not hand the same memory to a split reduction
+		LibraryScratchHold hold(elems * sizeof(float));  // the GEMM entry must not hand the columns' memory to a split reduction
 		rc = lten_hip_sgemm_strided_batched(0, 0, (uint64_t)g.Cout, HW, Kc, 1.0f, w, Kc, 0, col, HW, (int64_t)(Kc * HW), 0.0f, y, HW,
 		                                    (int64_t)((uint64_t)g.Cout * HW), N);
 	}

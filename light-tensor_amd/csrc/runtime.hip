@@ -50,16 +50,22 @@ struct LibraryScratch {
 };
 static LibraryScratch g_scratch[8] = {};
 
-static int g_scratch_held = 0;
-LibraryScratchHold::LibraryScratchHold() { g_scratch_held++; }
-LibraryScratchHold::~LibraryScratchHold() { g_scratch_held--; }
+static bool g_scratch_held = false;
+static uint64_t g_scratch_held_bytes = 0;
+LibraryScratchHold::LibraryScratchHold(uint64_t bytes)
+{
+	g_scratch_held = true;
+	g_scratch_held_bytes = (bytes + 255) & ~255ull;
+}
+LibraryScratchHold::~LibraryScratchHold() { g_scratch_held = false; }
 
 void* library_scratch(uint64_t bytes)
 {
-	if (g_scratch_held > 0) return nullptr;
 	int dev = -1;
 	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 8) return nullptr;
 	LibraryScratch& ls = g_scratch[dev];
+	// held: only what the block has left behind the holder's part, and the block stays where it is
+	if (g_scratch_held) return (ls.base != nullptr && g_scratch_held_bytes + bytes <= ls.bytes) ? static_cast<char*>(ls.base) + g_scratch_held_bytes : nullptr;
 	if (ls.bytes >= bytes) {
 		if (capturing()) ls.recorded = true;
 		return ls.base;

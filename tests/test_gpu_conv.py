@@ -284,6 +284,7 @@ def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
 
 
 @pytest.mark.parametrize("geo", [(1, 96, 12, 12, 96, 3, 3, 1, 1, 1, 1),       # one image: a single product on the 32 x 32 tiles; its data gradient the same way
+                                 (1, 192, 10, 10, 96, 3, 3, 1, 1, 1, 1),     # one image, K = 1728: the product splits its reduction, partial sums behind the columns
                                  (3, 64, 16, 12, 130, 3, 3, 1, 1, 2, 1),     # strides (2, 1), ragged channel blocks
                                  (2, 60, 12, 12, 100, 3, 3, 1, 1, 1, 1),     # K = 540: whole k-steps, then the rest in a second pass
                                  (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1)])   # enough tiles for the 64 x 64 direct-to-LDS kernel
