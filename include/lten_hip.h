@@ -237,8 +237,11 @@ uint64_t lten_hip_conv2d_wgrad_workspace_bytes(uint64_t N, uint64_t Cin, uint64_
                                                int stride_h, int stride_w);
 /* conv2_backward's data branch (l-ten/backprop.cpp:1955-1968 CPU, :2007-2028 CUDA: per image col = W^T dy_n, then
  * col2im) for the whole batch: dx[N,Cin,H,W] is overwritten.  With stride 1 it runs as a convolution of dy with
- * the flipped, channel-transposed weights on the forward kernels (no column buffer); other strides follow l-ten's
- * GEMM + col2im per image.  workspace: lten_hip_conv2d_dgrad_workspace_bytes(...) device bytes. */
+ * the flipped, channel-transposed weights on the forward kernels; other strides run as one implicit GEMM over the
+ * stride classes of the input pixels or, from a megabyte of columns on, as l-ten's GEMM + col2im done once for the
+ * batch with the columns (at most 512 MB) in memory the library owns (inside a graph recording only if that memory
+ * exists already: run the call once before recording it).  workspace: lten_hip_conv2d_dgrad_workspace_bytes(...)
+ * device bytes. */
 int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                               int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
                               const float* w, const float* dy, float* dx, void* workspace);

@@ -376,6 +376,68 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	return 0;
 }
 
+// dx[n][c][y][x] = sum over the taps (i, j) that reach the pixel of col[n][(c, i, j)][(y + ph - i) / sh][(x + pw - j) / sw],
+// taps in increasing (i, j) order as in col2im_kernel; one thread per pixel, the taps of its stride class only.
+__global__ __launch_bounds__(256) void col2im_batch_kernel(const float* __restrict__ col, ConvGeo g, float* __restrict__ dx)
+{
+	const unsigned pix = blockIdx.x * 256 + threadIdx.x, HWi = (unsigned)(g.H * g.W), HW = (unsigned)(g.Ho * g.Wo);
+	if (pix >= HWi) return;
+	const unsigned c = blockIdx.y, n = blockIdx.z;
+	const int y = (int)(pix / (unsigned)g.W), x = (int)pix - y * g.W;
+	const int qy = (y + g.ph) / g.sh, ry = (y + g.ph) - qy * g.sh, qx = (x + g.pw) / g.sw, rx = (x + g.pw) - qx * g.sw;
+	const float* cc = col + ((int64_t)n * g.Cin + c) * (g.kh * g.kw) * HW;
+	float s = 0.0f;
+	for (int i = ry, yy = qy; i < g.kh && yy >= 0; i += g.sh, yy--) {
+		if (yy >= g.Ho) continue;
+		for (int j = rx, xx = qx; j < g.kw && xx >= 0; j += g.sw, xx--) {
+			if (xx >= g.Wo) continue;
+			s += cc[(unsigned)(i * g.kw + j) * HW + (unsigned)(yy * g.Wo + xx)];
+		}
+	}
+	dx[((int64_t)n * g.Cin + c) * HWi + pix] = s;
+}
+
+// rows of `cols` floats copied into rows of `pitch` floats, the tail of every row zero
+__global__ __launch_bounds__(256) void pad_rows_f32_kernel(const float* __restrict__ src, float* __restrict__ dst, int rows, int cols, int pitch)
+{
+	const int idx = blockIdx.x * 256 + threadIdx.x;
+	if (idx >= rows * pitch) return;
+	const int r = idx / pitch, c = idx - r * pitch;
+	dst[idx] = c < cols ? src[r * cols + c] : 0.0f;
+}
+
+// The data gradient with a stride, l-ten's decomposition (l-ten/backprop.cpp:2022-2028: col = W^T dy_n, then col2im) done
+// once for the batch: one strided batch of TN products into column matrices in library memory, one col2im launch.
+// Returns -1 when the layer does not qualify or the memory cannot be had.
+static int conv_dgrad_by_columns(const ConvGeo& g, const float* w, const float* dy, float* dx)
+{
+	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
+	const uint64_t elems = N * Kc * HW, pitch = (Kc + 3) & ~3ull;
+	if (!(HW % 4 == 0 && g.Cout >= 32 && g.Cout % 4 == 0 && aligned16(w) && aligned16(dy) && elems <= (1ull << 27) && (uint64_t)g.H * g.W < (1ull << 30) && g.Cin < 65536 &&
+	      (uint64_t)g.Cout * pitch < (1ull << 30))) return -1;
+	const uint64_t w_bytes = pitch != Kc ? (uint64_t)g.Cout * pitch * sizeof(float) : 0;
+	float* col = static_cast<float*>(library_scratch(elems * sizeof(float) + w_bytes));
+	if (col == nullptr) return -1;
+	const float* wp = w;
+	if (pitch != Kc) {  // rows of the weights that start on 16-byte boundaries, for the GEMM's loads
+		float* padded = col + elems;
+		pad_rows_f32_kernel<<<dim3((unsigned)ceil_div((uint64_t)g.Cout * pitch, 256)), dim3(256), 0, stream()>>>(w, padded, g.Cout, (int)Kc, (int)pitch);
+		LTEN_HIP_LAUNCH_CHECK();
+		wp = padded;
+	}
+	int rc;
+	{
+		LibraryScratchHold hold(elems * sizeof(float) + w_bytes);
+		rc = lten_hip_sgemm_strided_batched(1, 0, Kc, HW, (uint64_t)g.Cout, 1.0f, wp, pitch, 0, dy, HW, (int64_t)((uint64_t)g.Cout * HW), 0.0f, col, HW,
+		                                    (int64_t)(Kc * HW), N);
+	}
+	if (rc != 0) return rc;
+	col2im_batch_kernel<<<dim3((unsigned)ceil_div((uint64_t)g.H * g.W, 256), (unsigned)g.Cin, (unsigned)N), dim3(256), 0, stream()>>>(col, g, dx);
+	LTEN_HIP_LAUNCH_CHECK();
+	set_kernel_name("conv2d_dgrad_batched_gemm_col2im");
+	return 0;
+}
+
 // Picks the forward kernel for a geometry (x, w, y non-null, non-empty problem).
 static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
@@ -640,6 +702,14 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	const double padded_us = 2.0 * 64 * ceil_div(Cin, 64) * (double)(N * H * W) * Cout * kh * kw / ((double)sh * sw) / 45e6;
 	const double by_image_us = (double)N * (16.0 + 9e-6 * (double)Kc * HW);
 	const bool padded_rows = get_option(OPT_CONV_VARIANT) == 0 && Cin <= 8 && padded_us > 1.5 * by_image_us;
+	// With a stride, l-ten's decomposition done once for the batch is ahead of the implicit GEMM below from about a
+	// megabyte of columns on (32 x 64 x 56 x 56 <- 128 channels 3 x 3 stride 2: 130 -> 101 us; 32 x 128 x 28 x 28 <- 256:
+	// 174 -> 86 us; 32 x 4 x 56 x 56 <- 64: 65 -> 15 us; the first layer above: 333 us), except for 1 x 1 windows, whose
+	// columns are dy itself (32 x 64 x 56 x 56 <- 128 at stride 2: 24 against 36 us).
+	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows) && N * Kc * HW >= (1u << 18)) {
+		const int rc = conv_dgrad_by_columns(g, w, dy, dx);
+		if (rc >= 0) return rc;
+	}
 	// any stride: one implicit-GEMM launch for the batch (64 x 64 x 28 x 28 <- 128 channels at stride 2: 722 us image by image)
 	if (get_option(OPT_CONV_VARIANT) == 0 && (!few_narrow || !dgrad_as_forward(g)) && !padded_rows && dgrad_gemm_takes(g)) {
 		set_kernel_name("conv2d_dgrad_64x64x32");

@@ -316,7 +316,8 @@ def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
 
 def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
     """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
-    padding costs more than l-ten's own decomposition (GEMM + col2im image by image), which the library then takes."""
+    padding costs more than l-ten's own decomposition (GEMM + col2im), which the library then takes: once for the batch,
+    with the columns in memory of its own; image by image in the caller's workspace when that memory cannot be had."""
     geo = (2, 3, 128, 128, 64, 7, 7, 3, 3, 2, 2)
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
@@ -327,8 +328,36 @@ def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob
     want_dx = np.empty((N, Cin, H, W), np.float32)
     ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
     dx = gpu_dgrad(gpu, geo, w, dy)
-    assert gpu.last_kernel() == "conv2d_dgrad_sgemm_col2im", gpu.last_kernel()
+    assert gpu.last_kernel() == "conv2d_dgrad_batched_gemm_col2im", gpu.last_kernel()
     assert rel_err(dx, want_dx) < TOL
+
+
+@pytest.mark.parametrize("geo", [(8, 32, 40, 48, 48, 3, 3, 1, 1, 2, 2),       # 3 x 3 at stride 2
+                                 (4, 24, 34, 30, 36, 5, 4, 2, 1, 3, 2),       # strides 3 x 2, oblong window
+                                 (3, 5, 40, 40, 32, 7, 7, 3, 3, 2, 2),        # K = 245: the weights' rows are padded to a multiple of four floats
+                                 (8, 40, 32, 32, 64, 2, 2, 0, 0, 2, 2)])      # windows that do not overlap
+def test_conv_strided_data_gradient_by_column_matrices(gpu, ob, geo):
+    """With a stride and a megabyte or more of columns, l-ten's GEMM + col2im runs once for the batch: a strided batch of
+    TN products into memory of the library, one col2im launch; against the oracle, and against the implicit GEMM."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    assert N * Cin * kh * kw * Ho * Wo >= 1 << 18 and (Ho * Wo) % 4 == 0
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_dgrad_batched_gemm_col2im", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+    gpu.set_option("conv_variant", 1)
+    try:
+        dx1 = gpu_dgrad(gpu, geo, w, dy)
+        assert gpu.last_kernel() != "conv2d_dgrad_batched_gemm_col2im"
+    finally:
+        gpu.set_option("conv_variant", 0)
+    assert rel_err(dx, dx1) < TOL
 
 
 @pytest.mark.parametrize("geo", [(3, 16, 20, 30, 64, 3, 3, 1, 1, 1, 1),      # 30 columns: rows start 8 bytes off 16-byte boundaries
