@@ -534,6 +534,45 @@ def extra_configs(lt, wl, with_cpu):
                 "algorithmic_bytes": xq3.nbytes + wq3.nbytes + xq3.size})
     del dxq3, dwq3, dyq3, dyq3b, wsq3
 
+    # ---- fp32 Conv2d layers of many channels on small maps (the late stages of a ResNet-like network), where no patch
+    # kernel applies: the batch's column matrices in library memory and the direct-to-LDS GEMM tiles, against the implicit
+    # GEMM (forward) and l-ten's GEMM + col2im image by image (data gradient) of the same library (option conv_variant 1)
+    # on the same operands
+    for geo4, what in (((32, 256, 14, 14, 256, 3, 3, 1, 1, 1, 1), "256 -> 256 ch 3x3 on 32x256x14x14"),
+                       ((32, 128, 28, 28, 256, 3, 3, 1, 1, 2, 2), "128 -> 256 ch 3x3 stride 2 on 32x128x28x28")):
+        N4, Ci4, H4, W4, Co4, kh4, kw4, ph4, pw4, sh4, sw4 = geo4
+        Ho4, Wo4 = (H4 + 2 * ph4 - kh4) // sh4 + 1, (W4 + 2 * pw4 - kw4) // sw4 + 1
+        rng4 = np.random.default_rng(sum(geo4))
+        x4 = D.from_numpy(rng4.standard_normal((N4, Ci4, H4, W4)).astype(np.float32))
+        w4 = D.from_numpy((rng4.standard_normal((Co4, Ci4 * kh4 * kw4)) * 0.05).astype(np.float32))
+        b4 = D.from_numpy(rng4.standard_normal(Co4).astype(np.float32))
+        dy4 = D.from_numpy(rng4.standard_normal((N4, Co4, Ho4, Wo4)).astype(np.float32))
+        ny, nx = N4 * Co4 * Ho4 * Wo4, N4 * Ci4 * H4 * W4
+        y4, y4b, dx4, dx4b = D(4 * ny), D(4 * ny), D(4 * nx), D(4 * nx)
+        ws4 = D(max(int(l.lten_hip_conv2d_dgrad_workspace_bytes(*geo4)), 16))
+        fwd = lambda y: lt.check(l.lten_hip_conv2d_forward_f32(*geo4, x4.ptr, w4.ptr, b4.ptr, y.ptr))
+        bwd = lambda dx: lt.check(l.lten_hip_conv2d_dgrad_f32(*geo4, w4.ptr, dy4.ptr, dx.ptr, ws4.ptr))
+        ms_f = timed(lt, lambda: fwd(y4), 50)
+        kf4 = lt.last_kernel()
+        ms_d = timed(lt, lambda: bwd(dx4), 50)
+        kd4 = lt.last_kernel()
+        lt.set_option("conv_variant", 1)
+        try:
+            ms_f1 = timed(lt, lambda: fwd(y4b), 20)
+            ms_d1 = timed(lt, lambda: bwd(dx4b), 20)
+        finally:
+            lt.set_option("conv_variant", 0)
+        ya, yb = y4.numpy(np.float32, (ny,)), y4b.numpy(np.float32, (ny,))
+        da, db_ = dx4.numpy(np.float32, (nx,)), dx4b.numpy(np.float32, (nx,))
+        fl4 = 2.0 * ny * Ci4 * kh4 * kw4
+        out.append({"config": f"Conv2d fp32 {what} (beyond l-ten's networks), forward with bias + data gradient",
+                    "forward_us": round(ms_f * 1e3, 1), "forward_kernel": kf4, "dgrad_us": round(ms_d * 1e3, 1), "dgrad_kernel": kd4,
+                    "implicit_gemm_forward_us": round(ms_f1 * 1e3, 1), "dgrad_image_by_image_gemm_col2im_us": round(ms_d1 * 1e3, 1),
+                    "max_rel_diff_to_those": float(max(np.abs(ya - yb).max() / np.abs(yb).max(), np.abs(da - db_).max() / np.abs(db_).max())),
+                    "roofline": {"bound": "mfma", "achieved": round(fl4 / ms_f / 1e9, 1), "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                 "frac": round(fl4 / ms_f / 1e9 / FP32_MFMA_PEAK_TFLOPS, 4)}})
+        del x4, w4, dy4, y4, y4b, dx4, dx4b, ws4
+
     # ---- int8 layers whose sizes are no multiples of the kernels' vector widths: in_features no multiple of 16 (the rows
     # are copied into padded ones first; prepared weights are padded once), out_features no multiple of 4 (byte stores).
     # Prepared weights, zero points (17, 250, 100); the first rows (2^30 multiply-adds' worth) against the oracle.
