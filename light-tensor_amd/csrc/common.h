@@ -27,6 +27,14 @@ int get_option(Option o);
 // a launch graph is being recorded: nullptr then, and when there is no memory), kept until the process ends.  One
 // stream uses it at a time, as everything else in this library.
 void* library_scratch(uint64_t bytes);
+// While one of these lives, the caller promises that every row of the operands it passes to the GEMM entry points can be
+// read up to its leading dimension, the last row included (BLAS only guarantees the row itself): the direct-to-LDS
+// tiles then take row-contiguous operands whose row count is no multiple of 4.
+struct RowsReadableToPitch {
+	RowsReadableToPitch();
+	~RowsReadableToPitch();
+};
+bool rows_readable_to_pitch();
 // For a caller that keeps data in the first `bytes` of the block across a call into another entry point of the library:
 // while one of these lives, library_scratch hands out only what the block has behind those bytes and never moves it.
 struct LibraryScratchHold {

@@ -288,8 +288,8 @@ static void wgrad_split(const ConvGeo& g, int& slices, int64_t& slice_len)
 
 // The column matrices of the whole batch, col[n][k][hw] with k = (ci, i, j): a thread writes four consecutive pixels of
 // one row (n, k) per step, the threads of a row side by side, several short rows to a workgroup.  The pixel count of an
-// image is a multiple of 4 here, so every store is one of 16 bytes.
-__global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows)
+// image is rounded up to a multiple of 4 in the rows of col (`pitch`, the tail zero), so every store is one of 16 bytes.
+__global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows, unsigned pitch)
 {
 	const unsigned Kc = (unsigned)(g.Cin * g.kh * g.kw), HW = (unsigned)(g.Ho * g.Wo), taps = (unsigned)(g.kh * g.kw);
 	const unsigned r = threadIdx.x / (unsigned)row_threads, q = threadIdx.x - r * row_threads;
@@ -298,14 +298,14 @@ __global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restri
 	const unsigned ci = k / taps, ij = k - ci * taps;
 	const int i = (int)(ij / (unsigned)g.kw), j = (int)ij - i * g.kw;
 	const float* xc = x + ((int64_t)n * g.Cin + ci) * g.H * g.W;
-	float* out = col + ((int64_t)n * Kc + k) * HW;
-	for (unsigned hw = q * 4; hw < HW; hw += row_threads * 4) {
+	float* out = col + ((int64_t)n * Kc + k) * pitch;
+	for (unsigned hw = q * 4; hw < pitch; hw += row_threads * 4) {
 		int ho = (int)(hw / (unsigned)g.Wo), wo = (int)hw - ho * g.Wo;
 		float v[4];
 #pragma unroll
 		for (int e = 0; e < 4; e++) {
 			const int yy = ho * g.sh - g.ph + i * g.dh, xx = wo * g.sw - g.pw + j * g.dw;
-			const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W);
+			const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W) & (hw + e < HW);
 			const float t = xc[(yy * g.W + xx) & -(int)inside];
 			v[e] = inside ? t : 0.0f;
 			if (++wo == g.Wo) { wo = 0; ho++; }
@@ -325,6 +325,25 @@ __global__ __launch_bounds__(256) void conv_add_bias_kernel(float* __restrict__ 
 	reinterpret_cast<float4*>(y)[idx] = v;
 }
 
+// the same, one pixel per thread (pixel counts that are no multiple of 4)
+__global__ __launch_bounds__(256) void conv_add_bias_each_kernel(float* __restrict__ y, const float* __restrict__ bias, int Cout, int hw, int64_t total)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= total) return;
+	y[idx] += bias[(int)((idx / hw) % Cout)];
+}
+
+static void conv_add_bias(float* y, const float* bias, uint64_t N, uint64_t Cout, uint64_t HW)
+{
+	if (HW % 4 == 0 && aligned16(y)) {
+		const int64_t total4 = (int64_t)(N * Cout * HW / 4);
+		conv_add_bias_kernel<<<dim3((unsigned)ceil_div((uint64_t)total4, 256)), dim3(256), 0, stream()>>>(y, bias, (int)Cout, (int)(HW / 4), total4);
+	} else {
+		const int64_t total = (int64_t)(N * Cout * HW);
+		conv_add_bias_each_kernel<<<dim3((unsigned)ceil_div((uint64_t)total, 256)), dim3(256), 0, stream()>>>(y, bias, (int)Cout, (int)HW, total);
+	}
+}
+
 // Deep layers on small images that the patch kernels do not take (a stride, a window other than 3 x 3, images that fill
 // less than half of a patch tile): the implicit GEMM below gathers its operand element by element and runs at 45
 // TFLOP/s, the direct-to-LDS GEMM tiles at 85-90 on a column matrix that is already laid out.  With enough output
@@ -335,14 +354,14 @@ __global__ __launch_bounds__(256) void conv_add_bias_kernel(float* __restrict__ 
 static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
 	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
-	const uint64_t elems = N * Kc * HW;
-	if (!(g.Cout >= 96 && HW >= 64 && HW % 4 == 0 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) && aligned16(y) &&
-	      elems <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30))) return -1;
+	const uint64_t pitch = (HW + 3) & ~3ull;  // rows of the column matrices start on 16-byte boundaries
+	const uint64_t elems = N * Kc * pitch;
+	if (!(g.Cout >= 96 && HW >= 32 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) &&
+	      elems <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30) && N * g.Cout * HW < (1ull << 40))) return -1;
 	// Measured rates, on the work of whole tiles.  The implicit GEMM: 46 TFLOP/s once its 64 x 64 tiles give every CU a
 	// workgroup.  The batch of products: 110 TFLOP/s on the 64 x 64 direct-to-LDS tiles and 92 on the 128 x 128 ones, which
 	// sgemm_run picks when they fill the chip (a K that is no multiple of their k-step costs a second pass); 45 on the
-	// 32 x 32 tiles that take a batch too small for those, again in proportion to the CUs they fill.  The column matrix
-	// is written and read at 2.5 TB/s, and the two extra launches cost 8 us.
+	// 32 x 32 tiles that take a batch too small for those, again in proportion to the CUs they fill.  The column matrix is written and read at 2.5 TB/s, and the two extra launches cost 8 us.
 	auto whole = [](uint64_t n, uint64_t t) { return (double)(ceil_div(n, t) * t); };
 	const double implicit_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(N * HW, 64) * (double)Kc /
 	                           (46e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 64) * ceil_div(N * HW, 64)) / 256.0));
@@ -350,26 +369,26 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	double gemm_us;
 	if (tiles128 >= 256) gemm_us = 2.0 * whole((uint64_t)g.Cout, 128) * whole(HW, 128) * (double)(N * Kc) / 92e6;
 	else if (tiles64 >= 128) gemm_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(HW, 64) * (double)(N * Kc) / 110e6;
-	else gemm_us = 2.0 * (double)g.Cout * (double)elems / (45e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 32) * ceil_div(HW, 32) * N) / 256.0));
+	else gemm_us = 2.0 * whole((uint64_t)g.Cout, 32) * whole(HW, 32) * (double)(N * Kc) / (45e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 32) * ceil_div(HW, 32) * N) / 256.0));
 	if (Kc % 32 != 0) gemm_us *= 1.15;
 	if (implicit_us < 1.05 * (gemm_us + 4.0 * (double)elems / 2.5e6 + 8.0)) return -1;
 	// (behind the columns: room for the partial sums of a reduction that the GEMM entry splits, one image on a long K)
 	const uint64_t behind = g.N == 1 ? 65 * (uint64_t)g.Cout * HW * sizeof(float) + 4096 : 0;
 	float* col = static_cast<float*>(library_scratch(elems * sizeof(float) + behind));
 	if (col == nullptr) return -1;
-	const int row_threads = (int)std::min<uint64_t>(256, HW / 4), block_rows = 256 / row_threads;
-	im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows);
+	const int row_threads = (int)std::min<uint64_t>(256, pitch / 4), block_rows = 256 / row_threads;
+	im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows, (unsigned)pitch);
 	LTEN_HIP_LAUNCH_CHECK();
 	int rc;
 	{
 		LibraryScratchHold hold(elems * sizeof(float));  // the GEMM entry must not hand the columns' memory to a split reduction
-		rc = lten_hip_sgemm_strided_batched(0, 0, (uint64_t)g.Cout, HW, Kc, 1.0f, w, Kc, 0, col, HW, (int64_t)(Kc * HW), 0.0f, y, HW,
+		RowsReadableToPitch promise;                     // (the columns' rows are `pitch` long, the weights' rows whole)
+		rc = lten_hip_sgemm_strided_batched(0, 0, (uint64_t)g.Cout, HW, Kc, 1.0f, w, Kc, 0, col, pitch, (int64_t)(Kc * pitch), 0.0f, y, HW,
 		                                    (int64_t)((uint64_t)g.Cout * HW), N);
 	}
 	if (rc != 0) return rc;
 	if (bias != nullptr) {
-		const int64_t total4 = (int64_t)(N * g.Cout * HW / 4);
-		conv_add_bias_kernel<<<dim3((unsigned)ceil_div((uint64_t)total4, 256)), dim3(256), 0, stream()>>>(y, bias, g.Cout, (int)(HW / 4), total4);
+		conv_add_bias(y, bias, N, (uint64_t)g.Cout, HW);
 		LTEN_HIP_LAUNCH_CHECK();
 	}
 	set_kernel_name("conv2d_im2col_batched_gemm");
@@ -447,17 +466,26 @@ static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* 
 	if (variant == 0 && conv_fewin_takes(g, x, y)) return conv_fewin_forward(g, x, w, bias, y);
 	if (variant != 1 && conv_smallk_takes(g)) return conv_smallk_forward(g, x, w, bias, y);
 	if (variant == 0 && conv_fewout_takes(g, x, y)) return conv_fewout_forward(g, x, w, bias, y, false);
-	// A 1 x 1 layer (stride 1, no padding) without bias is a product per image of the weights with the image as it lies
-	// in memory, y[n] = W[Cout x Cin] x[n][Cin x HW]: a strided batch of plain GEMMs with the weights as the operand all
-	// share (32 x 256 x 56 x 56 -> 64 channels: 44 us there, 70 us on the implicit GEMM below; 32 x 512 x 14 x 14 -> 512:
-	// 38 against 73 us; the stride-1 data gradient of such a layer comes the same way).  The GEMM has no per-row
-	// bias, and adding one afterwards would cost a pass over y: layers with a bias stay below.
-	if (variant == 0 && bias == nullptr && g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.dh == 1 && g.dw == 1 &&
-	    g.Cin >= 16 && N < 65536) {
-		const int rc = lten_hip_sgemm_strided_batched(0, 0, Cout, (uint64_t)HW, (uint64_t)g.Cin, 1.0f, w, (uint64_t)g.Cin, 0, x, (uint64_t)HW,
-		                                              (int64_t)g.Cin * HW, 0.0f, y, (uint64_t)HW, (int64_t)Cout * HW, N);
-		if (rc == 0) set_kernel_name("conv2d_1x1_batched_gemm");
-		return rc;
+	// A 1 x 1 layer (stride 1, no padding) is a product per image of the weights with the image as it lies in memory,
+	// y[n] = W[Cout x Cin] x[n][Cin x HW]: a strided batch of plain GEMMs with the weights as the operand all share
+	// (32 x 256 x 56 x 56 -> 64 channels: 44 us there, 70 us on the implicit GEMM below; 32 x 512 x 14 x 14 -> 512: 38
+	// against 73 us; the stride-1 data gradient of such a layer comes the same way).  The GEMM has no per-row bias: a
+	// bias is added in a pass over y, which pays while y is small beside the work (estimates: 75 TFLOP/s here, 48 on the
+	// implicit GEMM, the pass at 4 TB/s + 3 us; 256 -> 64 channels yes, 64 -> 256 no).
+	if (variant == 0 && g.kh == 1 && g.kw == 1 && g.sh == 1 && g.sw == 1 && g.ph == 0 && g.pw == 0 && g.dh == 1 && g.dw == 1 &&
+	    g.Cin >= 16 && N < 65536 && (HW % 4 == 0 || g.Cin < 256)) {  // (channel images off 16-byte boundaries: by columns, below)
+		const double flops = 2.0 * (double)N * (double)Cout * HW * g.Cin, y_bytes = 4.0 * (double)N * (double)Cout * HW;
+		const bool pass_pays = HW % 4 == 0 && aligned16(y) && flops / 48e6 > flops / 75e6 + 2.0 * y_bytes / 4e6 + 3.0;
+		if (bias == nullptr || pass_pays) {
+			int rc = lten_hip_sgemm_strided_batched(0, 0, Cout, (uint64_t)HW, (uint64_t)g.Cin, 1.0f, w, (uint64_t)g.Cin, 0, x, (uint64_t)HW,
+			                                        (int64_t)g.Cin * HW, 0.0f, y, (uint64_t)HW, (int64_t)Cout * HW, N);
+			if (rc == 0 && bias != nullptr) {
+				conv_add_bias(y, bias, N, Cout, (uint64_t)HW);
+				LTEN_HIP_LAUNCH_CHECK();
+			}
+			if (rc == 0) set_kernel_name("conv2d_1x1_batched_gemm");
+			return rc;
+		}
 	}
 	// variant 2: the register-staged patch kernel even where the direct-to-LDS one would run; 5: the direct-to-LDS
 	// one with its four-row tile also where the two-row tile would be picked

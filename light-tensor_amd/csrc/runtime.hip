@@ -50,6 +50,11 @@ struct LibraryScratch {
 };
 static LibraryScratch g_scratch[8] = {};
 
+static int g_rows_readable = 0;
+RowsReadableToPitch::RowsReadableToPitch() { g_rows_readable++; }
+RowsReadableToPitch::~RowsReadableToPitch() { g_rows_readable--; }
+bool rows_readable_to_pitch() { return g_rows_readable > 0; }
+
 static bool g_scratch_held = false;
 static uint64_t g_scratch_held_bytes = 0;
 LibraryScratchHold::LibraryScratchHold(uint64_t bytes)

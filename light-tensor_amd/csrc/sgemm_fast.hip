@@ -89,7 +89,8 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 		} else {
 			constexpr int KPL = 256 / T, LPR = T / 4;  // k rows per load, lanes per k row
 			const int k = q * KPL + lane / LPR, r4 = (lane % LPR) * 4;
-			voff[i] = (k * ld + (uint32_t)min(row0 + r4, rows - 4)) * 4;  // rows is a multiple of 4 here
+			// (rows is a multiple of 4, or the caller has promised that the array's rows can be read up to the next one)
+			voff[i] = (k * ld + (uint32_t)min(row0 + r4, ((rows + 3) & ~3) - 4)) * 4;
 		}
 		lds_slot[i] = smem_addr + (is_a ? 0 : TILE) + q * 1024;
 	}
@@ -264,7 +265,9 @@ int sgemm_fast_dispatch(const SProblem& p, int tA, int tB, uint64_t batch, int v
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
 	const uint64_t a_rows = tA ? p.K : p.M, b_rows = tB ? p.N : p.K;  // rows of the arrays as stored
 	// an operand that is contiguous along its tile rows is fetched four rows at a time: whole groups of four only
-	const bool fits = (!tA || p.M % 4 == 0) && (tB || p.N % 4 == 0) && p.M >= 4 && p.N >= 4 &&
+	const bool slack = rows_readable_to_pitch();
+	const bool fits = (!tA || p.M % 4 == 0 || (slack && (uint64_t)p.lda >= (((uint64_t)p.M + 3) & ~3ull))) &&
+	                  (tB || p.N % 4 == 0 || (slack && (uint64_t)p.ldb >= (((uint64_t)p.N + 3) & ~3ull))) && p.M >= 4 && p.N >= 4 &&
 	                  p.K % 32 == 0 && p.K >= 64 && (p.lda & 3) == 0 && (p.ldb & 3) == 0 &&
 	                  (p.stride_a & 3) == 0 && (p.stride_b & 3) == 0 &&
 	                  ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) & 15) == 0 &&

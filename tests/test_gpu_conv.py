@@ -263,7 +263,8 @@ def test_conv_data_gradient_with_strides(gpu, ob, geo):
 @pytest.mark.parametrize("geo", [(3, 64, 20, 20, 48, 1, 1, 0, 0, 1, 1), (2, 100, 13, 17, 70, 1, 1, 0, 0, 1, 1), (5, 40, 56, 56, 256, 1, 1, 0, 0, 1, 1)])
 def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
     """A 1 x 1 layer without bias, and its data gradient, run as a strided batch of plain products on the images as they
-    lie in memory; with a bias the layer stays on the convolution kernels.  Both against the oracle."""
+    lie in memory; with a bias only where a pass over y that adds it pays (not at these sizes: the convolution kernels).
+    Both against the oracle."""
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
     x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
@@ -287,7 +288,9 @@ def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
                                  (1, 192, 10, 10, 96, 3, 3, 1, 1, 1, 1),     # one image, K = 1728: the product splits its reduction, partial sums behind the columns
                                  (3, 64, 16, 12, 130, 3, 3, 1, 1, 2, 1),     # strides (2, 1), ragged channel blocks
                                  (2, 60, 12, 12, 100, 3, 3, 1, 1, 1, 1),     # K = 540: whole k-steps, then the rest in a second pass
-                                 (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1)])   # enough tiles for the 64 x 64 direct-to-LDS kernel
+                                 (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1),    # enough tiles for the 64 x 64 direct-to-LDS kernel
+                                 (4, 512, 7, 7, 256, 1, 1, 0, 0, 1, 1),      # 1 x 1 on 7 x 7 maps: 49 pixels, rows of the columns padded to 52
+                                 (3, 64, 9, 9, 100, 3, 3, 1, 1, 1, 1)])      # 81 pixels
 def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
     """Many channels on images too small for the patch tiles: the batch's column matrices go to memory of the library in one
     launch, a strided batch of products writes y, a pass adds the bias.  Forward (with and without bias), and the gradients
