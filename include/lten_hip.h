@@ -214,7 +214,7 @@ int lten_hip_col2im_u8(const uint8_t* col, int channels, int height, int width, 
 
 /* Conv2d::forward's per-image im2col + cublasSgemm loop (l-ten/conv2d.cpp:164-171) as one
  * implicit-GEMM launch over the whole batch; no col buffer is materialised, except for layers
- * of many channels on small images (96 or more output channels, Cin*kh*kw >= 256, 32 or more
+ * of many channels on small images (32 or more output channels, Cin*kh*kw >= 256, 32 or more
  * output pixels, no patch kernel for the shape, a cost estimate in favour), which follow l-ten's scheme
  * with the batch's column matrices (at most 512 MB) in memory the library owns: one im2col
  * launch, one strided batch of GEMMs, one pass for the bias.  Inside a graph recording that

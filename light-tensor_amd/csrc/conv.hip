@@ -356,7 +356,7 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
 	const uint64_t pitch = (HW + 3) & ~3ull;  // rows of the column matrices start on 16-byte boundaries
 	const uint64_t elems = N * Kc * pitch;
-	if (!(g.Cout >= 96 && HW >= 32 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) &&
+	if (!(g.Cout >= 32 && HW >= 32 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) &&
 	      elems <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30) && N * g.Cout * HW < (1ull << 40))) return -1;
 	// Measured rates, on the work of whole tiles.  The implicit GEMM: 46 TFLOP/s once its 64 x 64 tiles give every CU a
 	// workgroup.  The batch of products: 110 TFLOP/s on the 64 x 64 direct-to-LDS tiles and 92 on the 128 x 128 ones, which
@@ -397,9 +397,10 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 
 // dx[n][c][y][x] = sum over the taps (i, j) that reach the pixel of col[n][(c, i, j)][(y + ph - i) / sh][(x + pw - j) / sw],
 // taps in increasing (i, j) order as in col2im_kernel; one thread per pixel, the taps of its stride class only.
-__global__ __launch_bounds__(256) void col2im_batch_kernel(const float* __restrict__ col, ConvGeo g, float* __restrict__ dx)
+__global__ __launch_bounds__(256) void col2im_batch_kernel(const float* __restrict__ col, ConvGeo g, float* __restrict__ dx, unsigned HW)
 {
-	const unsigned pix = blockIdx.x * 256 + threadIdx.x, HWi = (unsigned)(g.H * g.W), HW = (unsigned)(g.Ho * g.Wo);
+	// (HW: the length of a row of col, the output pixels rounded up to a multiple of 4)
+	const unsigned pix = blockIdx.x * 256 + threadIdx.x, HWi = (unsigned)(g.H * g.W);
 	if (pix >= HWi) return;
 	const unsigned c = blockIdx.y, n = blockIdx.z;
 	const int y = (int)(pix / (unsigned)g.W), x = (int)pix - y * g.W;
@@ -419,10 +420,10 @@ __global__ __launch_bounds__(256) void col2im_batch_kernel(const float* __restri
 // rows of `cols` floats copied into rows of `pitch` floats, the tail of every row zero
 __global__ __launch_bounds__(256) void pad_rows_f32_kernel(const float* __restrict__ src, float* __restrict__ dst, int rows, int cols, int pitch)
 {
-	const int idx = blockIdx.x * 256 + threadIdx.x;
-	if (idx >= rows * pitch) return;
-	const int r = idx / pitch, c = idx - r * pitch;
-	dst[idx] = c < cols ? src[r * cols + c] : 0.0f;
+	const unsigned idx = blockIdx.x * 256 + threadIdx.x;  // (rows * pitch below 2^30: checked by the host)
+	if (idx >= (unsigned)rows * (unsigned)pitch) return;
+	const unsigned r = idx / (unsigned)pitch, c = idx - r * pitch;
+	dst[idx] = c < (unsigned)cols ? src[r * (unsigned)cols + c] : 0.0f;
 }
 
 // The data gradient with a stride, l-ten's decomposition (l-ten/backprop.cpp:2022-2028: col = W^T dy_n, then col2im) done
@@ -431,27 +432,37 @@ __global__ __launch_bounds__(256) void pad_rows_f32_kernel(const float* __restri
 static int conv_dgrad_by_columns(const ConvGeo& g, const float* w, const float* dy, float* dx)
 {
 	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
-	const uint64_t elems = N * Kc * HW, pitch = (Kc + 3) & ~3ull;
-	if (!(HW % 4 == 0 && g.Cout >= 32 && g.Cout % 4 == 0 && aligned16(w) && aligned16(dy) && elems <= (1ull << 27) && (uint64_t)g.H * g.W < (1ull << 30) && g.Cin < 65536 &&
-	      (uint64_t)g.Cout * pitch < (1ull << 30))) return -1;
-	const uint64_t w_bytes = pitch != Kc ? (uint64_t)g.Cout * pitch * sizeof(float) : 0;
-	float* col = static_cast<float*>(library_scratch(elems * sizeof(float) + w_bytes));
+	// rows of both operands and of the columns on 16-byte boundaries: what is not so already is copied into padded rows
+	const uint64_t kpitch = (Kc + 3) & ~3ull, hpitch = (HW + 3) & ~3ull;
+	const uint64_t elems = N * Kc * hpitch;
+	if (!(g.Cout >= 32 && g.Cout % 4 == 0 && aligned16(w) && aligned16(dy) && elems <= (1ull << 27) && (uint64_t)g.H * g.W < (1ull << 30) && g.Cin < 65536 &&
+	      (uint64_t)g.Cout * kpitch < (1ull << 30) && N * g.Cout * hpitch < (1ull << 30))) return -1;
+	const uint64_t w_elems = kpitch != Kc ? (uint64_t)g.Cout * kpitch : 0, dy_elems = hpitch != HW ? N * g.Cout * hpitch : 0;
+	float* col = static_cast<float*>(library_scratch((elems + w_elems + dy_elems) * sizeof(float)));
 	if (col == nullptr) return -1;
 	const float* wp = w;
-	if (pitch != Kc) {  // rows of the weights that start on 16-byte boundaries, for the GEMM's loads
+	const float* dyp = dy;
+	if (w_elems != 0) {
 		float* padded = col + elems;
-		pad_rows_f32_kernel<<<dim3((unsigned)ceil_div((uint64_t)g.Cout * pitch, 256)), dim3(256), 0, stream()>>>(w, padded, g.Cout, (int)Kc, (int)pitch);
+		pad_rows_f32_kernel<<<dim3((unsigned)ceil_div(w_elems, 256)), dim3(256), 0, stream()>>>(w, padded, g.Cout, (int)Kc, (int)kpitch);
 		LTEN_HIP_LAUNCH_CHECK();
 		wp = padded;
 	}
+	if (dy_elems != 0) {
+		float* padded = col + elems + w_elems;
+		pad_rows_f32_kernel<<<dim3((unsigned)ceil_div(dy_elems, 256)), dim3(256), 0, stream()>>>(dy, padded, (int)(N * g.Cout), (int)HW, (int)hpitch);
+		LTEN_HIP_LAUNCH_CHECK();
+		dyp = padded;
+	}
 	int rc;
 	{
-		LibraryScratchHold hold(elems * sizeof(float) + w_bytes);
-		rc = lten_hip_sgemm_strided_batched(1, 0, Kc, HW, (uint64_t)g.Cout, 1.0f, wp, pitch, 0, dy, HW, (int64_t)((uint64_t)g.Cout * HW), 0.0f, col, HW,
-		                                    (int64_t)(Kc * HW), N);
+		LibraryScratchHold hold((elems + w_elems + dy_elems) * sizeof(float));
+		RowsReadableToPitch promise;  // (padded copies, or rows that are whole multiples of four floats as they are)
+		rc = lten_hip_sgemm_strided_batched(1, 0, Kc, HW, (uint64_t)g.Cout, 1.0f, wp, kpitch, 0, dyp, hpitch, (int64_t)((uint64_t)g.Cout * hpitch), 0.0f, col,
+		                                    hpitch, (int64_t)(Kc * hpitch), N);
 	}
 	if (rc != 0) return rc;
-	col2im_batch_kernel<<<dim3((unsigned)ceil_div((uint64_t)g.H * g.W, 256), (unsigned)g.Cin, (unsigned)N), dim3(256), 0, stream()>>>(col, g, dx);
+	col2im_batch_kernel<<<dim3((unsigned)ceil_div((uint64_t)g.H * g.W, 256), (unsigned)g.Cin, (unsigned)N), dim3(256), 0, stream()>>>(col, g, dx, (unsigned)hpitch);
 	LTEN_HIP_LAUNCH_CHECK();
 	set_kernel_name("conv2d_dgrad_batched_gemm_col2im");
 	return 0;
