@@ -228,7 +228,9 @@ int lten_hip_conv2d_forward_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W
 /* conv2_backward's weight branch (l-ten/backprop.cpp:1941-1954, the CPU semantics: the sum
  * over all images; the CUDA branch at :1989-2005 keeps only the last image and is not
  * followed).  dw[Cout, Cin*kh*kw] is overwritten.  workspace: device scratch of at least
- * lten_hip_conv2d_wgrad_workspace_bytes(...) bytes. */
+ * lten_hip_conv2d_wgrad_workspace_bytes(...) bytes.  With at most 8192 output pixels in the
+ * whole batch and many channels the gradient may instead be computed as one GEMM on copies of
+ * the columns and of dy in memory the library owns (as for the forward pass). */
 int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_t Cout,
                               int kernel_h, int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
                               const float* x, const float* dy, float* dw, void* workspace);

@@ -468,6 +468,94 @@ static int conv_dgrad_by_columns(const ConvGeo& g, const float* w, const float* 
 	return 0;
 }
 
+// The column matrix of the whole batch with a row per output pixel, colT[(n, hw)][k], k = (ci, i, j), rows `pitch` floats
+// long (a multiple of 4, the tail zero): a thread writes four consecutive k of one pixel.
+__global__ __launch_bounds__(256) void im2col_rows_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ colT, unsigned pitch, unsigned total4)
+{
+	const unsigned t = blockIdx.x * 256 + threadIdx.x;
+	if (t >= total4) return;
+	const unsigned kq = pitch / 4, p = t / kq, k0 = (t - p * kq) * 4;
+	const unsigned HW = (unsigned)(g.Ho * g.Wo), taps = (unsigned)(g.kh * g.kw), Kc = (unsigned)g.Cin * taps;
+	const unsigned n = p / HW, hw = p - n * HW, ho = hw / (unsigned)g.Wo, wo = hw - ho * g.Wo;
+	int ci = (int)(k0 / taps), r = (int)(k0 - ci * taps), i = r / g.kw, j = r - i * g.kw;
+	const int y0 = (int)ho * g.sh - g.ph, x0 = (int)wo * g.sw - g.pw;
+	const float* xn = x + (int64_t)n * g.Cin * g.H * g.W;
+	float v[4];
+#pragma unroll
+	for (int e = 0; e < 4; e++) {
+		const bool inside = (k0 + e < Kc) & ((unsigned)(y0 + i) < (unsigned)g.H) & ((unsigned)(x0 + j) < (unsigned)g.W);
+		const float f = xn[((ci * g.H + y0 + i) * g.W + x0 + j) & -(int)inside];
+		v[e] = inside ? f : 0.0f;
+		if (++j == g.kw) {
+			j = 0;
+			if (++i == g.kh) { i = 0; ci++; }
+		}
+	}
+	*reinterpret_cast<float4*>(colT + (int64_t)p * pitch + k0) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// out[(n * HW + hw) * pitch + co] = in[(n * Cout + co) * HW + hw] (0 for co >= Cout): 32 x 32 tiles through LDS
+__global__ __launch_bounds__(256) void pixels_major_kernel(const float* __restrict__ in, float* __restrict__ out, int Cout, int HW, int pitch)
+{
+	__shared__ float tile[32][33];
+	const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5, n = blockIdx.z;
+#pragma unroll
+	for (int r = 0; r < 4; r++) {
+		const int co = blockIdx.y * 32 + ty + 8 * r, hw = blockIdx.x * 32 + tx;
+		tile[ty + 8 * r][tx] = (co < Cout && hw < HW) ? in[((int64_t)n * Cout + co) * HW + hw] : 0.0f;
+	}
+	__syncthreads();
+#pragma unroll
+	for (int r = 0; r < 4; r++) {
+		const int hw = blockIdx.x * 32 + ty + 8 * r, co = blockIdx.y * 32 + tx;
+		if (hw < HW && co < pitch) out[((int64_t)n * HW + hw) * pitch + co] = tile[tx][ty + 8 * r];
+	}
+}
+
+// The weight gradient over few output pixels in all (small maps, small batches): the implicit GEMM's tiles each walk a
+// reduction of a few k-steps, most of their time is prologue and epilogue (32 x 512 x 7 x 7 -> 512 channels 3 x 3: 36
+// TFLOP/s; one image: 4).  With the batch's columns and dy both laid out with a row per pixel, dw = dyT^T colT is one
+// plain TN product over all pixels, which the GEMM entry places as it does any other (the direct-to-LDS tiles, a split
+// reduction when the output is small).  `current_us`: the estimate for the kernel that would run otherwise.
+// Returns -1 when the layer does not qualify or the library memory cannot be had.
+static int conv_wgrad_by_columns(const ConvGeo& g, const float* x, const float* dy, float* dw, double current_us)
+{
+	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N, Cout = g.Cout;
+	const uint64_t P = N * HW, kp = (Kc + 3) & ~3ull, cp = (Cout + 3) & ~3ull;
+	if (!(P <= 8192 && Cout >= 32 && Kc >= 64 && P * kp <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30) && aligned16(dw))) return -1;
+	auto whole = [](uint64_t n, uint64_t t) { return (double)(ceil_div(n, t) * t); };
+	const double flops = 2.0 * (double)(Cout * Kc) * (double)P;
+	if (flops < 1e8) return -1;  // (a handful of launches either way)
+	const uint64_t tiles128 = ceil_div(Cout, 128) * ceil_div(Kc, 128), tiles64 = ceil_div(Cout, 64) * ceil_div(Kc, 64), tiles32 = ceil_div(Cout, 32) * ceil_div(Kc, 32);
+	const bool splits = tiles32 <= 256 && P >= 1536;
+	double gemm_us;
+	// (sgemm_run: the direct-to-LDS tiles from K = 256 in whole k-steps of 32, or from 512 with a second pass for the rest)
+	if ((tiles128 >= 128 || tiles64 >= 128) && P >= 256 && (P % 32 == 0 || P >= 512))
+		gemm_us = 2.0 * whole(Cout, tiles128 >= 128 ? 128 : 64) * whole(Kc, tiles128 >= 128 ? 128 : 64) * (double)P / 85e6 * (P % 32 == 0 ? 1.0 : 1.15) + 8.0;
+	else
+		gemm_us = flops / (45e6 * (splits ? 1.0 : std::min(1.0, (double)tiles32 / 256.0))) + (splits ? 8.0 : 4.0);
+	// (the two copies: 4 bytes per column element at 2.5 TB/s and 12 us for the launches; a margin of 15 %)
+	if (current_us < 1.15 * (gemm_us + 4.0 * (double)(P * kp) / 2.5e6 + 12.0)) return -1;
+	const uint64_t behind = splits ? 65 * Cout * Kc * sizeof(float) + 4096 : 0;
+	const uint64_t held = (P * kp + P * cp) * sizeof(float);
+	float* colT = static_cast<float*>(library_scratch(held + behind));
+	if (colT == nullptr) return -1;
+	float* dyT = colT + P * kp;
+	const unsigned total4 = (unsigned)(P * (kp / 4));
+	im2col_rows_kernel<<<dim3((unsigned)ceil_div((uint64_t)total4, 256)), dim3(256), 0, stream()>>>(x, g, colT, (unsigned)kp, total4);
+	LTEN_HIP_LAUNCH_CHECK();
+	pixels_major_kernel<<<dim3((unsigned)ceil_div(HW, 32), (unsigned)ceil_div(cp, 32), (unsigned)N), dim3(256), 0, stream()>>>(dy, dyT, (int)Cout, (int)HW, (int)cp);
+	LTEN_HIP_LAUNCH_CHECK();
+	int rc;
+	{
+		LibraryScratchHold hold(held);
+		RowsReadableToPitch promise;  // (both copies have rows of whole multiples of four floats)
+		rc = lten_hip_sgemm(1, 0, Cout, Kc, P, 1.0f, dyT, cp, colT, kp, 0.0f, dw, Kc);
+	}
+	if (rc == 0) set_kernel_name("conv2d_wgrad_columns_gemm");
+	return rc;
+}
+
 // Picks the forward kernel for a geometry (x, w, y non-null, non-empty problem).
 static int conv_forward_dispatch(const ConvGeo& g, const float* x, const float* w, const float* bias, float* y)
 {
@@ -801,6 +889,15 @@ int lten_hip_conv2d_wgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	// rows that do not allow 16-byte loads, of at most 56 columns (the kernel's chunks are 64 pixels of one row):
 	// 32 x 32 x 30 x 30 -> 64: 33 against 47 us, 32 x 48 x 50 x 50 -> 96: 151 against 177 us
 	const bool narrow = get_option(OPT_CONV_VARIANT) == 0 && (g.Wo <= 16 || ((g.W % 4 != 0 || g.Wo % 4 != 0) && g.Wo <= 56));
+	if (get_option(OPT_CONV_VARIANT) == 0) {
+		// few output pixels in all: one plain product on pixel-major copies, when the estimate favours it.  What would run
+		// otherwise, measured up to the 8192 output pixels P of a batch that this route takes: the patch kernel 28 us + the
+		// work at 80 TFLOP/s; the implicit GEMM at 60 TFLOP/s x P / (P + 1100), 17 us or more (two launches).
+		const double P = (double)N * g.Ho * g.Wo, flops = 2.0 * (double)count * P;
+		const double current_us = (!narrow && conv_patch_wgrad_takes(g)) ? 28.0 + flops / 80e6 : std::max(17.0, flops / (60e6 * P / (P + 1100.0)));
+		const int rc = conv_wgrad_by_columns(g, x, dy, dw, current_us);
+		if (rc >= 0) return rc;
+	}
 	if (!narrow && get_option(OPT_CONV_VARIANT) != 1 && conv_patch_wgrad_takes(g)) {
 		const int parts = conv_patch_wgrad_parts(g);
 		if (int rc = conv_patch_wgrad(g, x, dy, static_cast<float*>(workspace), parts)) return rc;

@@ -317,6 +317,26 @@ def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
     _conv_vs_oracle(gpu, ob, geo)
 
 
+@pytest.mark.parametrize("geo", [(1, 512, 7, 7, 512, 3, 3, 1, 1, 1, 1),       # one image of 49 pixels: the product on the 32 x 32 tiles
+                                 (2, 2048, 7, 7, 510, 1, 1, 0, 0, 1, 1),      # a 1 x 1 layer; 510 channels: dy's pixel-major rows padded to 512
+                                 (16, 512, 7, 7, 256, 3, 3, 1, 1, 1, 1)])     # 784 pixels: the 64 x 64 direct-to-LDS tiles, K = 784 in two passes
+def test_conv_weight_gradient_over_few_pixels_by_column_matrices(gpu, ob, geo):
+    """Few output pixels in the whole batch and many channels: the columns and dy are copied with a row per pixel into memory
+    of the library and the weight gradient is one plain TN product over the pixels; against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = np.zeros((Cout, Cin, kh, kw), np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dw = np.empty_like(w)
+    ob.oracle().oracle_conv2d_wgrad(*geo, x.reshape(-1), dy.reshape(-1), want_dw.reshape(-1), col)
+    _, dw, _ = gpu_conv(gpu, geo, x, w, dy)
+    assert gpu.last_kernel() == "conv2d_wgrad_columns_gemm", gpu.last_kernel()
+    assert rel_err(dw, want_dw) < TOL
+
+
 def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
     """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
     padding costs more than l-ten's own decomposition (GEMM + col2im), which the library then takes: once for the batch,
