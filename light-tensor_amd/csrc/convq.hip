@@ -34,6 +34,8 @@ int conv2dq_image_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w,
 int conv2dq_band_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
                           float zp_out, void* y, bool out_acc);
 
+double conv2dq_band_estimate_us(const ConvGeo& g);
+
 // ND = dwords of packed taps a thread holds (4 taps each): 4, 8, 12 or 16, the smallest that covers K.
 template <int OUT, int ND>
 __global__ __launch_bounds__(256) void conv2dq_direct_kernel(ConvGeo g, const uint8_t* __restrict__ x, const uint8_t* __restrict__ w,
@@ -287,16 +289,21 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 
 	// small images with a longer window (l-ten's quantized MNIST conv2): still one launch, no workspace (convq_image.hip;
 	// option "conv_variant" 2 keeps such shapes on the three launches below, 3 skips the small-image kernel)
+	const BatchedPlan bp = batched_plan(g);
 	if (get_option(OPT_CONV_VARIANT) == 0 || get_option(OPT_CONV_VARIANT) == 3) {
 		int rc = get_option(OPT_CONV_VARIANT) == 3 ? -1 : conv2dq_image_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
-		// larger images or more channels: a band of output rows and a block of output channels per workgroup, the input rows it needs in LDS
-		rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
+		// larger images or more channels: a band of output rows and a block of output channels per workgroup, the input rows
+		// it needs in LDS -- unless long windows leave a workgroup so few pixels and channels that it stages more than it
+		// computes and the three launches below are ahead, which take 35 us + 2.1 us per MB of patch rows (32 x 1024 x 14
+		// x 14 -> 256 channels 1 x 1: 132 us on bands, 43 below; 32 x 128 x 28 x 28 -> 256 channels 3 x 3 stride 2: 55 and 44)
+		const bool rows_ahead = get_option(OPT_CONV_VARIANT) == 0 && bp.ok && workspace != nullptr &&
+		                        conv2dq_band_estimate_us(g) > 35.0 + 2.1e-6 * (double)bp.rows * (double)bp.Kp;
+		if (!rows_ahead) rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
 	}
 
 	LTEN_HIP_REQUIRE(workspace != nullptr, "conv2dq: workspace is null");
-	const BatchedPlan bp = batched_plan(g);
 	if (bp.ok && get_option(OPT_CONV_VARIANT) != 1) {
 		uint8_t* base = static_cast<uint8_t*>(workspace);
 		uint8_t* rows = base;

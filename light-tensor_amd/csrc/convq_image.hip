@@ -621,6 +621,18 @@ static bool band_plan(const ConvGeo& g, BandPlan& pl)
 	return (int64_t)g.N * ((g.Ho + tb - 1) / tb) < (1ll << 31);
 }
 
+// What the band kernel is expected to take, in us (negative: no plan for the shape).  Its workgroups stage their rows of
+// the input and their block of the weights before every band, and that staging is where the time goes: the bytes all
+// workgroups stage, at the 1.3 TB/s measured over shapes from 30 to 190 MB of it (32 x 64 x 56 x 56 -> 64 channels 3 x 3:
+// 38 MB, 29 us; 32 x 1024 x 14 x 14 -> 256 channels 1 x 1, one output row and 32 channels per workgroup: 186 MB, 132 us).
+double conv2dq_band_estimate_us(const ConvGeo& g)
+{
+	BandPlan pl;
+	if (!band_plan(g, pl)) return -1.0;
+	const double wgs = (double)g.N * ((g.Ho + pl.TB - 1) / pl.TB) * ((((g.Cout + 15) / 16) + pl.ncb - 1) / pl.ncb);
+	return wgs * ((double)pl.RH * pl.RW * pl.PP + (double)pl.ncb * 16 * pl.wpitch) / 1.3e6;
+}
+
 // 0 = launched; -1 = not a shape for this route
 int conv2dq_band_dispatch(const ConvGeo& g, const uint8_t* x, const uint8_t* w, const int32_t* bias, int zp_in, int zp_w, float mult,
                           float zp_out, void* y, bool out_acc)

@@ -130,3 +130,26 @@ def test_conv2dq_vs_oracle(gpu, ob, geo):
         finally:
             gpu.set_option("conv_variant", 0)
         assert np.array_equal(acc1, want_acc) and np.array_equal(y1, want_y)
+
+
+def test_conv2dq_long_windows_on_small_maps_take_the_three_launches(gpu, ob):
+    """A 1 x 1 layer of 1024 channels on 14 x 14 maps: the band kernel has a plan (one output row and 32 channels per
+    workgroup), but its workgroups would stage more than they compute, and the library's estimate sends the layer to patch
+    rows + GEMM + finish.  Both routes give the oracle's bytes."""
+    geo = (16, 1024, 14, 14, 256, 1, 1, 0, 0, 1, 1)
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.integers(0, 256, (N, Cin, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (Cout, Cin, kh, kw), dtype=np.uint8)
+    sc, zp = [0.02, 0.013, 0.9], [17, 250, 100]
+    want_y, want_acc = ob.conv2dq_forward(geo, x, w, sc, zp)
+    y, acc = gpu.conv2dq_host(geo, x, w, sc, zp, want_acc=True)
+    assert gpu.last_kernel() == "conv2dq_rows_gemm_finish", gpu.last_kernel()
+    assert np.array_equal(acc, want_acc) and np.array_equal(y, want_y)
+    gpu.set_option("conv_variant", 3)   # the band kernel whatever the estimate says
+    try:
+        y3, acc3 = gpu.conv2dq_host(geo, x, w, sc, zp, want_acc=True)
+        assert gpu.last_kernel() == "conv2dq_band", gpu.last_kernel()
+    finally:
+        gpu.set_option("conv_variant", 0)
+    assert np.array_equal(acc3, want_acc) and np.array_equal(y3, want_y)
