@@ -342,6 +342,8 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 			if (want >= 2) splits = want;
 			else if (want == 0 && tiles <= 64 && p.K >= 8192) splits = tiles <= 32 ? 4 : 2;
 			else if (want == 0 && tiles <= 32 && p.K >= 4096) splits = 2;
+			// (slices are whole k-steps of 128, the first ones a step longer when the slices do not divide them: 128 x 4096 x
+			// 11008, 86 k-steps, 38 us unsplit, 27 in four slices)
 			if (splits >= 2 && qgemm_fast_split_dispatch(p, out, splits, scratch) == 0) return 0;
 			if (qgemm_fast_dispatch(p, out, 41) == 0) return 0;
 		}

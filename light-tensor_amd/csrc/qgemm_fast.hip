@@ -106,10 +106,13 @@ __global__ __launch_bounds__(WM* WN * 64) void qgemm_fast_kernel(QProblem p)
 		lds_slot[i] = smem_addr + q * 1024;
 		in_tail[i] = kc * 16 < p.K % BK;
 	}
-	// with SPLIT, blockIdx.y picks this workgroup's share of K; with TAIL the last k-step is partial (K % 16 == 0)
-	const int KT = SPLIT ? p.K / BK / p.splits : (TAIL ? (p.K + BK - 1) / BK : p.K / BK);
-	const uint8_t* const a_base = p.A + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
-	const uint8_t* const b_base = p.B + (SPLIT ? (int64_t)blockIdx.y * KT * BK : 0);
+	// with SPLIT, blockIdx.y picks this workgroup's share of K (whole k-steps; the first K / BK % splits shares are one step
+	// longer than the rest); with TAIL the last k-step is partial (K % 16 == 0)
+	const int share = SPLIT ? p.K / BK / p.splits : 0, longer = SPLIT ? p.K / BK - share * p.splits : 0;
+	const int KT = SPLIT ? share + ((int)blockIdx.y < longer ? 1 : 0) : (TAIL ? (p.K + BK - 1) / BK : p.K / BK);
+	const int64_t k_first = SPLIT ? ((int64_t)blockIdx.y * share + min((int)blockIdx.y, longer)) * BK : 0;
+	const uint8_t* const a_base = p.A + k_first;
+	const uint8_t* const b_base = p.B + k_first;
 	// In the partial k-step a lane whose chunk lies past K loads nothing.  For the A tile it stores bytes of 0x80
 	// instead, which the sign flip turns into zeros, so whatever the B tile still holds there is multiplied by 0.
 	auto load_one = [&](int i, int stage, int kt) {
@@ -648,8 +651,8 @@ int qgemm_fast_split_dispatch(const QProblem& q, int out, int splits, const Spli
 		scratch = &g_split;
 	}
 	const uint64_t tiles = ceil_div(p.M, T) * ceil_div(p.N, T);
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % (BK * splits) == 0 &&
-	                  p.K / splits >= 2 * BK && splits >= 2 && splits <= 16 &&
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % BK == 0 &&
+	                  p.K / BK / splits >= 2 && splits >= 2 && splits <= 16 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 && (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&
 	                  (reinterpret_cast<uintptr_t>(p.wsum) & 15) == 0 &&

@@ -337,6 +337,24 @@ def test_split_k_tiles_forced(gpu, ob, splits):
         gpu.set_option("qgemm_split", 0)
 
 
+@pytest.mark.parametrize("splits,K", [(4, 128 * 13), (8, 128 * 21), (2, 128 * 5)])
+def test_split_k_shares_of_unequal_length(gpu, ob, splits, K):
+    """A number of k-steps that the shares do not divide (13 steps over 4 workgroups: 4, 3, 3, 3): the first shares are a
+    step longer.  Zero-point terms, bias, int32 and u8 outputs against the oracle."""
+    rng = np.random.default_rng(splits + K)
+    M, N = 200, 384
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    gpu.set_option("qgemm_split", splits)
+    try:
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([128, 128, 128], np.uint8))
+        assert gpu.last_kernel().endswith("splitk")
+        run_case(gpu, ob, A, B, [0.02, 0.013, 0.9], np.array([3, 250, 77], np.uint8), bias=rng.integers(-5000, 5000, N).astype(np.int32))
+        assert gpu.last_kernel().endswith("splitk")
+    finally:
+        gpu.set_option("qgemm_split", 0)
+
+
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
     """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
