@@ -22,6 +22,8 @@ struct SProblem {
 	int64_t stride_a, stride_b, stride_c;  // per blockIdx.z
 	int M, N, K;
 	float alpha, beta;
+	// direct-to-LDS tiles only (set by their launcher): all tiles of a problem of the batch go to one XCD
+	int problems_by_xcd = 0;
 };
 
 // The last step of every epilogue that supports the relu pieces: c points into p.C (batch index 0).

@@ -49,12 +49,19 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 
 	// Workgroup -> tile.  Consecutive workgroup ids go round-robin to the 8 XCDs, each with its own L2; every
 	// XCD gets compact 4 x 8 blocks of tiles so that its CUs stream the same rows of A and B.
+	// A batch of small problems (problems_by_xcd): XCD x takes problems x, x + 8, ... whole, so that a problem's operands
+	// cross one L2 only (the workgroups of the grid go round-robin to the XCDs in the order z * gridDim.x + x).
 	const int tiles_m = (p.M + T - 1) / T, tiles_n = (p.N + T - 1) / T;
-	int tm, tn;
+	int tm, tn, bz = blockIdx.z;
 	{
 		const int nb = tiles_m * tiles_n, bid = blockIdx.x;
 		int lid = bid;
-		if ((nb & 7) == 0) lid = (bid & 7) * (nb >> 3) + (bid >> 3);
+		if (p.problems_by_xcd) {
+			const unsigned linear = blockIdx.z * (unsigned)nb + bid, j = linear >> 3;
+			const unsigned prob = j / (unsigned)nb;  // (the division runs on the vector ALU: back to scalar registers)
+			bz = __builtin_amdgcn_readfirstlane((int)prob * 8 + (int)(linear & 7));
+			lid = __builtin_amdgcn_readfirstlane((int)(j - prob * (unsigned)nb));
+		} else if ((nb & 7) == 0) lid = (bid & 7) * (nb >> 3) + (bid >> 3);
 		constexpr int GM = 4, GN = 8;
 		if (tiles_m % GM == 0 && tiles_n % GN == 0) {
 			const int group = lid / (GM * GN), within = lid % (GM * GN), groups_n = tiles_n / GN;
@@ -66,9 +73,9 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 		}
 	}
 	const int m0 = tm * T, n0 = tn * T;
-	const float* A = p.A + (int64_t)blockIdx.z * p.stride_a;
-	const float* B = p.B + (int64_t)blockIdx.z * p.stride_b;
-	float* C = p.C + (int64_t)blockIdx.z * p.stride_c;
+	const float* A = p.A + (int64_t)bz * p.stride_a;
+	const float* B = p.B + (int64_t)bz * p.stride_b;
+	float* C = p.C + (int64_t)bz * p.stride_c;
 
 	// ---- global -> LDS.  Load q (1 KB) of a tile: k-contiguous: rows 8q .. 8q+7, lane -> (row 8q + L/8, chunk
 	// (L%8) ^ swz(row)); row-contiguous: k rows (1024 / (4T)) q .., lane -> 4 consecutive tile rows of one k.
@@ -248,9 +255,13 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 }
 
 template <int T, int WM, int WN, int S>
-static int launch_fast(const SProblem& p, int tA, int tB, uint64_t batch, const char* name)
+static int launch_fast(const SProblem& q, int tA, int tB, uint64_t batch, const char* name)
 {
-	const dim3 grid((unsigned)(ceil_div(p.M, T) * ceil_div(p.N, T)), 1, (unsigned)batch), block(WM * WN * 64);
+	SProblem p = q;
+	const uint64_t nb = ceil_div(p.M, T) * ceil_div(p.N, T);
+	// (problems of at most 64 tiles, a whole number of them per XCD; larger ones spread over the XCDs in compact blocks)
+	p.problems_by_xcd = batch >= 8 && batch % 8 == 0 && nb <= 64 && nb * batch < (1ull << 31) ? 1 : 0;
+	const dim3 grid((unsigned)nb, 1, (unsigned)batch), block(WM * WN * 64);
 	set_kernel_name(name);
 	if (!tA && !tB) sgemm_fast_kernel<T, WM, WN, S, true, false><<<grid, block, 0, stream()>>>(p);
 	if (!tA && tB) sgemm_fast_kernel<T, WM, WN, S, true, true><<<grid, block, 0, stream()>>>(p);
