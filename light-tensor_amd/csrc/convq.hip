@@ -136,11 +136,12 @@ static void launch_conv2dq_direct(const dim3& grid, int K, const ConvGeo& g, con
 // Row r = n * Ho * Wo + p of the patch matrix: the window of output position p of image n in l-ten's column order
 // (ci, i, j).  Bytes outside the image are 0, as in l-ten's im2col (not the zero point); bytes from K on hold the input
 // zero point.  A thread builds sixteen consecutive bytes of a row; the tap table (offset of the tap inside an image and
-// its (i, j)) is built once per workgroup in LDS.  (Sixteen bytes and one 16-byte store per thread.)
+// its (i, j)) of the workgroup's 64 bytes of a row is built once per workgroup in LDS.  (Sixteen bytes and one 16-byte
+// store per thread.)
 __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint8_t* __restrict__ x, uint8_t* __restrict__ rows, int Kp, int zp_in,
                                                            unsigned row_blocks, const uint8_t* __restrict__ w, uint8_t* __restrict__ wp, int Cp, int zp_w)
 {
-	extern __shared__ int s_tap[];  // [Kp] offsets, then [Kp] i | j << 16
+	__shared__ int s_tap[128];  // [64] offsets, then [64] i | j << 16
 	const int K = g.Cin * g.kh * g.kw, HW = g.Ho * g.Wo;
 	if (blockIdx.x >= row_blocks) {
 		// the workgroups behind the rows pad the weights: wp[co][k] for co < Cp, k < Kp, with the weight zero point past K
@@ -152,17 +153,20 @@ __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint
 		}
 		return;
 	}
-	for (int k = threadIdx.x; k < Kp; k += 256) {
-		const int kc = min(k, K - 1);
-		const int j = kc % g.kw, i = (kc / g.kw) % g.kh, ci = kc / (g.kw * g.kh);
-		s_tap[k] = (ci * g.H + i) * g.W + j;
-		s_tap[Kp + k] = i | (j << 16);
+	// A workgroup builds 64 consecutive rows x 64 bytes: a wavefront's lanes are 64 consecutive positions at one chunk, so
+	// that each of its loads reads neighbouring bytes of the image (consecutive chunks of one row would read 64 channel
+	// planes at once); the four wavefronts write the four chunks of the same 64 bytes of every row.
+	const uint32_t chunks_per_row = (uint32_t)Kp / 16, groups = (chunks_per_row + 3) / 4;
+	const uint32_t tile = blockIdx.x / groups, grp = blockIdx.x - tile * groups;
+	const uint32_t r = tile * 64 + (threadIdx.x & 63), kc = grp * 4 + (threadIdx.x >> 6);
+	if (threadIdx.x < 64) {  // the taps of this workgroup's 64 bytes of a row
+		const int kt = min((int)grp * 64 + (int)threadIdx.x, K - 1);
+		const int j = kt % g.kw, i = (kt / g.kw) % g.kh, ci = kt / (g.kw * g.kh);
+		s_tap[threadIdx.x] = (ci * g.H + i) * g.W + j;
+		s_tap[64 + threadIdx.x] = i | (j << 16);
 	}
 	__syncthreads();
-	const uint32_t chunks_per_row = (uint32_t)Kp / 16;
-	const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
-	const uint32_t r = (uint32_t)(idx / chunks_per_row), kc = (uint32_t)(idx - (uint64_t)r * chunks_per_row);
-	if (r >= (uint32_t)g.N * (uint32_t)HW) return;
+	if (r >= (uint32_t)g.N * (uint32_t)HW || kc >= chunks_per_row) return;
 	const int n = (int)(r / (uint32_t)HW), pos = (int)(r - (uint32_t)n * (uint32_t)HW);
 	const int ho = pos / g.Wo, wo = pos - ho * g.Wo;
 	const int y0 = ho * g.sh - g.ph, x0 = wo * g.sw - g.pw;
@@ -171,11 +175,11 @@ __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint
 	uint32_t bytes[16];
 #pragma unroll
 	for (int b = 0; b < 16; b++) {  // all sixteen loads first
-		const int k = 16 * (int)kc + b;
-		const int ij = s_tap[Kp + k];
+		const int k = 16 * (int)kc + b, kl = 16 * (int)(threadIdx.x >> 6) + b;
+		const int ij = s_tap[64 + kl];
 		const int yy = y0 + (ij & 0xFFFF), xx = x0 + (ij >> 16);
 		const bool inside = ((unsigned)yy < (unsigned)g.H) & ((unsigned)xx < (unsigned)g.W);
-		const uint32_t byte = xn[(s_tap[k] + base) & -(int)inside];  // offset 0 for taps outside: always a valid address
+		const uint32_t byte = xn[(s_tap[kl] + base) & -(int)inside];  // offset 0 for taps outside: always a valid address
 		bytes[b] = k < K ? (inside ? byte : 0u) : (uint32_t)zp_in;
 	}
 	uint4 out;
@@ -183,7 +187,7 @@ __global__ __launch_bounds__(256) void conv2dq_rows_kernel(ConvGeo g, const uint
 	out.y = bytes[4] | bytes[5] << 8 | bytes[6] << 16 | bytes[7] << 24;
 	out.z = bytes[8] | bytes[9] << 8 | bytes[10] << 16 | bytes[11] << 24;
 	out.w = bytes[12] | bytes[13] << 8 | bytes[14] << 16 | bytes[15] << 24;
-	reinterpret_cast<uint4*>(rows)[idx] = out;
+	reinterpret_cast<uint4*>(rows)[(uint64_t)r * chunks_per_row + kc] = out;
 }
 
 // y[n][co][p] = requantize(acc[n * HW + p][co] + bias[p]) (or the int32 sum itself): a workgroup takes 64 positions x 64
@@ -248,7 +252,7 @@ static BatchedPlan batched_plan(const ConvGeo& g)
 	b.off_acc = b.off_wp + align256(b.Cp * b.Kp);
 	b.off_terms = b.off_acc + align256(b.rows * b.Cp * 4);
 	b.bytes = b.off_terms + 4 * (b.rows + b.Cp) + 16;
-	b.ok = b.bytes <= (2ull << 30) && b.rows < (1ull << 31) && b.rows * b.Kp < (1ull << 32) && b.Kp * 8 <= 48 * 1024 && b.Cp * b.Kp < (1ull << 31);
+	b.ok = b.bytes <= (2ull << 30) && b.rows < (1ull << 31) && b.rows * b.Kp < (1ull << 32) && b.Cp * b.Kp < (1ull << 31);
 	return b;
 }
 
@@ -295,10 +299,10 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		if (rc >= 0) return rc;
 		// larger images or more channels: a band of output rows and a block of output channels per workgroup, the input rows
 		// it needs in LDS -- unless long windows leave a workgroup so few pixels and channels that it stages more than it
-		// computes and the three launches below are ahead, which take 35 us + 2.1 us per MB of patch rows (32 x 1024 x 14
+		// computes and the three launches below are ahead, which take 30 us + 1.3 us per MB of patch rows (32 x 1024 x 14
 		// x 14 -> 256 channels 1 x 1: 132 us on bands, 43 below; 32 x 128 x 28 x 28 -> 256 channels 3 x 3 stride 2: 55 and 44)
 		const bool rows_ahead = get_option(OPT_CONV_VARIANT) == 0 && bp.ok && workspace != nullptr &&
-		                        conv2dq_band_estimate_us(g) > 35.0 + 2.1e-6 * (double)bp.rows * (double)bp.Kp;
+		                        conv2dq_band_estimate_us(g) > 30.0 + 1.3e-6 * (double)bp.rows * (double)bp.Kp;
 		if (!rows_ahead) rc = conv2dq_band_dispatch(g, x, w, bias, zp_in, zp_w, mult, zp_out, y, out_acc);
 		if (rc >= 0) return rc;
 	}
@@ -310,8 +314,8 @@ static int conv2dq_run(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, uint64_
 		uint8_t* wp = base + bp.off_wp;
 		int32_t* sums = reinterpret_cast<int32_t*>(base + bp.off_acc);
 		int32_t* terms = reinterpret_cast<int32_t*>(base + bp.off_terms);
-		const unsigned row_blocks = (unsigned)ceil_div(bp.rows * (bp.Kp / 16), 256), weight_blocks = (unsigned)ceil_div(bp.Cp * bp.Kp, 256);
-		conv2dq_rows_kernel<<<dim3(row_blocks + weight_blocks), dim3(256), (size_t)(bp.Kp * 8), stream()>>>(g, x, rows, (int)bp.Kp, zp_in, row_blocks, w, wp,
+		const unsigned row_blocks = (unsigned)(ceil_div(bp.rows, 64) * ceil_div(bp.Kp / 16, 4)), weight_blocks = (unsigned)ceil_div(bp.Cp * bp.Kp, 256);
+		conv2dq_rows_kernel<<<dim3(row_blocks + weight_blocks), dim3(256), 0, stream()>>>(g, x, rows, (int)bp.Kp, zp_in, row_blocks, w, wp,
 		                                                                                                (int)bp.Cp, zp_w);
 		LTEN_HIP_LAUNCH_CHECK();
 		if (int rc = lten_hip_quantized_matmul_acc(0, 1, bp.rows, bp.Cp, bp.Kp, rows, wp, sums, qp, nullptr, terms)) return rc;
