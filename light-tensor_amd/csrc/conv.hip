@@ -9,6 +9,7 @@
 // CUDA ones (l-ten/im_col.cu:65-96, 123-162) for callers that still want the buffer.
 #include "conv_common.h"
 #include "gemm_f32_core.h"
+#include "sgemm_common.h"
 
 #include <algorithm>
 
@@ -289,7 +290,11 @@ static void wgrad_split(const ConvGeo& g, int& slices, int64_t& slice_len)
 // The column matrices of the whole batch, col[n][k][hw] with k = (ci, i, j): a thread writes four consecutive pixels of
 // one row (n, k) per step, the threads of a row side by side, several short rows to a workgroup.  The pixel count of an
 // image is rounded up to a multiple of 4 in the rows of col (`pitch`, the tail zero), so every store is one of 16 bytes.
-__global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows, unsigned pitch)
+// Row (n, k) starts at col + n * image_stride + k * k_stride: [n][k][pitch] for a batch of products, or [k][all pixels of
+// the batch] (image_stride = HW, pitch = HW: no padding between images) for one product over the whole batch; `vec`: the
+// rows start on 16-byte boundaries.
+__global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restrict__ x, ConvGeo g, float* __restrict__ col, int row_threads, int block_rows, unsigned pitch,
+                                                           int64_t image_stride, int64_t k_stride, bool vec)
 {
 	const unsigned Kc = (unsigned)(g.Cin * g.kh * g.kw), HW = (unsigned)(g.Ho * g.Wo), taps = (unsigned)(g.kh * g.kw);
 	const unsigned r = threadIdx.x / (unsigned)row_threads, q = threadIdx.x - r * row_threads;
@@ -298,7 +303,7 @@ __global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restri
 	const unsigned ci = k / taps, ij = k - ci * taps;
 	const int i = (int)(ij / (unsigned)g.kw), j = (int)ij - i * g.kw;
 	const float* xc = x + ((int64_t)n * g.Cin + ci) * g.H * g.W;
-	float* out = col + ((int64_t)n * Kc + k) * pitch;
+	float* out = col + (int64_t)n * image_stride + (int64_t)k * k_stride;
 	for (unsigned hw = q * 4; hw < pitch; hw += row_threads * 4) {
 		int ho = (int)(hw / (unsigned)g.Wo), wo = (int)hw - ho * g.Wo;
 		float v[4];
@@ -310,7 +315,12 @@ __global__ __launch_bounds__(256) void im2col_batch_kernel(const float* __restri
 			v[e] = inside ? t : 0.0f;
 			if (++wo == g.Wo) { wo = 0; ho++; }
 		}
-		*reinterpret_cast<float4*>(out + hw) = make_float4(v[0], v[1], v[2], v[3]);
+		if (vec) *reinterpret_cast<float4*>(out + hw) = make_float4(v[0], v[1], v[2], v[3]);
+		else {
+#pragma unroll
+			for (int e = 0; e < 4; e++)
+				if (hw + e < pitch) out[hw + e] = v[e];
+		}
 	}
 }
 
@@ -368,16 +378,49 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	const uint64_t tiles128 = ceil_div((uint64_t)g.Cout, 128) * ceil_div(HW, 128) * N, tiles64 = ceil_div((uint64_t)g.Cout, 64) * ceil_div(HW, 64) * N;
 	double gemm_us;
 	if (tiles128 >= 256) gemm_us = 2.0 * whole((uint64_t)g.Cout, 128) * whole(HW, 128) * (double)(N * Kc) / 92e6;
-	else if (tiles64 >= 128) gemm_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(HW, 64) * (double)(N * Kc) / 110e6;
+	else if (tiles64 >= 128) gemm_us = 2.0 * whole((uint64_t)g.Cout, 64) * whole(HW, 64) * (double)(N * Kc) / (110e6 * std::min(1.0, (double)tiles64 / 256.0));
 	else gemm_us = 2.0 * whole((uint64_t)g.Cout, 32) * whole(HW, 32) * (double)(N * Kc) / (45e6 * std::min(1.0, (double)(ceil_div((uint64_t)g.Cout, 32) * ceil_div(HW, 32) * N) / 256.0));
 	if (Kc % 32 != 0) gemm_us *= 1.15;
+	// Several images and a K in whole k-steps: one product over the pixels of the whole batch, col[k][(n, hw)], whose tiles
+	// the GEMM stores image by image into y.  No tile is padded per image (196 pixels fill 3.06 tiles of 64 columns, 49
+	// pixels 0.77 of one), and the images need no padding between them.
+	const uint64_t P = N * HW, ppitch = (P + 3) & ~3ull;
+	bool whole_batch = N >= 2 && Kc % 32 == 0 && N * g.Cout * HW < (1ull << 31) && Kc * ppitch <= (1ull << 27) && Kc * ppitch < (1ull << 30);
+	if (whole_batch) {
+		const double whole_us = sgemm_grouped_columns_estimate((uint64_t)g.Cout, P, Kc, nullptr);
+		if (whole_us < gemm_us) gemm_us = whole_us;
+		else whole_batch = false;  // (few images: a product per image on the 32 x 32 tiles fills more CUs)
+	}
 	if (implicit_us < 1.05 * (gemm_us + 4.0 * (double)elems / 2.5e6 + 8.0)) return -1;
+	if (whole_batch) {
+		float* col = static_cast<float*>(library_scratch(Kc * ppitch * sizeof(float)));
+		if (col == nullptr) return -1;
+		const int row_threads = (int)std::min<uint64_t>(256, pitch / 4), block_rows = 256 / row_threads;
+		im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows, (unsigned)HW,
+		                                                                                                             (int64_t)HW, (int64_t)ppitch, HW % 4 == 0);
+		LTEN_HIP_LAUNCH_CHECK();
+		int rc;
+		{
+			RowsReadableToPitch promise;  // (the rows of the columns are ppitch long)
+			rc = sgemm_grouped_columns((uint64_t)g.Cout, P, Kc, w, Kc, col, ppitch, y, HW, (int64_t)((uint64_t)g.Cout * HW));
+		}
+		if (rc == 0) {
+			if (bias != nullptr) {
+				conv_add_bias(y, bias, N, (uint64_t)g.Cout, HW);
+				LTEN_HIP_LAUNCH_CHECK();
+			}
+			set_kernel_name("conv2d_im2col_gemm");
+			return 0;
+		}
+		// (the tiles did not take the shape: the batch of products below)
+	}
 	// (behind the columns: room for the partial sums of a reduction that the GEMM entry splits, one image on a long K)
 	const uint64_t behind = g.N == 1 ? 65 * (uint64_t)g.Cout * HW * sizeof(float) + 4096 : 0;
 	float* col = static_cast<float*>(library_scratch(elems * sizeof(float) + behind));
 	if (col == nullptr) return -1;
 	const int row_threads = (int)std::min<uint64_t>(256, pitch / 4), block_rows = 256 / row_threads;
-	im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows, (unsigned)pitch);
+	im2col_batch_kernel<<<dim3((unsigned)ceil_div(Kc, (uint64_t)block_rows), (unsigned)N), dim3(256), 0, stream()>>>(x, g, col, row_threads, block_rows, (unsigned)pitch,
+	                                                                                                             (int64_t)(Kc * pitch), (int64_t)pitch, true);
 	LTEN_HIP_LAUNCH_CHECK();
 	int rc;
 	{

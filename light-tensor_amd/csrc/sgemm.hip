@@ -1144,6 +1144,41 @@ static bool takes_32x32(const SProblem& p, uint64_t M, uint64_t N, uint64_t K)
 	return tiles32 <= 1024 || (operands_vec(p) && tiles32 < (1u << 20));
 }
 
+// The tile for a product with grouped columns and what it is expected to take, in us: the work of whole tiles at the rate
+// measured for each size (256 x 256: 120 TFLOP/s, 128 x 128: 92, 64 x 64: 110), in proportion to the CUs the tiles fill.
+double sgemm_grouped_columns_estimate(uint64_t M, uint64_t N, uint64_t K, int* variant)
+{
+	const int sizes[3] = { 256, 128, 64 }, variants[3] = { 12, 21, 31 };
+	const double rates[3] = { 120e6, 92e6, 110e6 };
+	double best = 0.0;
+	for (int i = 0; i < 3; i++) {
+		const uint64_t t = (uint64_t)sizes[i], tiles = ceil_div(M, t) * ceil_div(N, t);
+		if (i == 0 && (M < 192 || N < 192)) continue;
+		const double us = 2.0 * (double)(ceil_div(M, t) * t) * (double)(ceil_div(N, t) * t) * (double)K / (rates[i] * std::min(1.0, (double)tiles / 256.0));
+		if (best == 0.0 || us < best) {
+			best = us;
+			if (variant) *variant = variants[i];
+		}
+	}
+	return best;
+}
+
+int sgemm_grouped_columns(uint64_t M, uint64_t N, uint64_t K, const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t group,
+                          int64_t group_stride)
+{
+	if (M == 0 || N == 0 || K < 64 || K % 32 != 0 || group == 0 || M >= (1ull << 31) || N >= (1ull << 31) || K >= (1ull << 31) || group >= (1ull << 31)) return -1;
+	SProblem p = {};
+	p.A = A; p.B = B; p.C = C;
+	p.lda = (int64_t)lda; p.ldb = (int64_t)ldb; p.ldc = (int64_t)group;
+	p.M = (int)M; p.N = (int)N; p.K = (int)K;
+	p.alpha = 1.0f; p.beta = 0.0f;
+	p.col_group = (int)group;
+	p.col_group_stride = group_stride;
+	int variant = 31;
+	(void)sgemm_grouped_columns_estimate(M, N, K, &variant);
+	return sgemm_fast_dispatch(p, 0, 0, 1, variant);
+}
+
 }  // namespace lten_hip
 
 using namespace lten_hip;

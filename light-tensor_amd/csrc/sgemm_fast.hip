@@ -221,6 +221,26 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 		const int n = n0 + wn * TN + j * 32 + lrow;
 		bv[j] = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
 	}
+	if (p.col_group != 0) {  // grouped columns (alpha = 1, beta = 0, no bias): the lane's columns are placed one by one
+		int64_t coff[FN];
+#pragma unroll
+		for (int j = 0; j < FN; j++) {
+			const unsigned n = (unsigned)(n0 + wn * TN + j * 32 + lrow), grp = n / (unsigned)p.col_group;
+			coff[j] = n < (unsigned)p.N ? (int64_t)grp * p.col_group_stride + (n - grp * (unsigned)p.col_group) : -1;
+		}
+#pragma unroll
+		for (int i = 0; i < FM; i++)
+#pragma unroll
+			for (int r = 0; r < 16; r++) {
+				const int m = m0 + wm * TM + i * 32 + (r >> 2) * 8 + 4 * lk + (r & 3);
+				if (m >= p.M) continue;
+				float* cr = C + (int64_t)m * p.ldc;
+#pragma unroll
+				for (int j = 0; j < FN; j++)
+					if (coff[j] >= 0) cr[coff[j]] = acc[i][j][r];
+			}
+		return;
+	}
 	float* cw = C + (int64_t)(m0 + wm * TM) * p.ldc + n0 + wn * TN;
 	const unsigned c_lane = (unsigned)(4 * lk * p.ldc) + lrow;
 	if (m0 + T <= p.M && n0 + T <= p.N) {
