@@ -402,13 +402,9 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 		int rc;
 		{
 			RowsReadableToPitch promise;  // (the rows of the columns are ppitch long)
-			rc = sgemm_grouped_columns((uint64_t)g.Cout, P, Kc, w, Kc, col, ppitch, y, HW, (int64_t)((uint64_t)g.Cout * HW));
+			rc = sgemm_grouped_columns((uint64_t)g.Cout, P, Kc, w, Kc, col, ppitch, y, HW, (int64_t)((uint64_t)g.Cout * HW), bias);
 		}
 		if (rc == 0) {
-			if (bias != nullptr) {
-				conv_add_bias(y, bias, N, (uint64_t)g.Cout, HW);
-				LTEN_HIP_LAUNCH_CHECK();
-			}
 			set_kernel_name("conv2d_im2col_gemm");
 			return 0;
 		}

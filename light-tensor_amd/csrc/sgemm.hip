@@ -1164,7 +1164,7 @@ double sgemm_grouped_columns_estimate(uint64_t M, uint64_t N, uint64_t K, int* v
 }
 
 int sgemm_grouped_columns(uint64_t M, uint64_t N, uint64_t K, const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t group,
-                          int64_t group_stride)
+                          int64_t group_stride, const float* row_bias)
 {
 	if (M == 0 || N == 0 || K < 64 || K % 32 != 0 || group == 0 || M >= (1ull << 31) || N >= (1ull << 31) || K >= (1ull << 31) || group >= (1ull << 31)) return -1;
 	SProblem p = {};
@@ -1174,6 +1174,7 @@ int sgemm_grouped_columns(uint64_t M, uint64_t N, uint64_t K, const float* A, ui
 	p.alpha = 1.0f; p.beta = 0.0f;
 	p.col_group = (int)group;
 	p.col_group_stride = group_stride;
+	p.row_bias = row_bias;
 	int variant = 31;
 	(void)sgemm_grouped_columns_estimate(M, N, K, &variant);
 	return sgemm_fast_dispatch(p, 0, 0, 1, variant);

@@ -28,6 +28,7 @@ struct SProblem {
 	// ldc apart inside it (the output maps of a batch of images, [image][channel][pixel], as one matrix [channel][all pixels])
 	int col_group = 0;
 	int64_t col_group_stride = 0;
+	const float* row_bias = nullptr;  // with col_group: added per row m (a convolution's bias per output channel), or null
 };
 
 // The last step of every epilogue that supports the relu pieces: c points into p.C (batch index 0).
@@ -41,10 +42,10 @@ __device__ __forceinline__ void sgemm_store(const SProblem& p, float* c, float o
 // Direct-to-LDS tiles for large aligned problems; returns -1 when the problem does not fit them.
 int sgemm_fast_dispatch(const SProblem& p, int tA, int tB, uint64_t batch, int variant);
 // C[m][(g, j)] = sum_k A[m][k] B[k][g * group + j] on the direct-to-LDS tiles (A row-major with K contiguous, B row-major
-// with all N columns contiguous), column (g, j) stored at C + g * group_stride + m * group + j; -1 when the tiles do not
-// take the shapes.
+// with all N columns contiguous), column (g, j) stored at C + g * group_stride + m * group + j, plus row_bias[m] when that
+// is not null; -1 when the tiles do not take the shapes.
 double sgemm_grouped_columns_estimate(uint64_t M, uint64_t N, uint64_t K, int* variant);
 int sgemm_grouped_columns(uint64_t M, uint64_t N, uint64_t K, const float* A, uint64_t lda, const float* B, uint64_t ldb, float* C, uint64_t group,
-                          int64_t group_stride);
+                          int64_t group_stride, const float* row_bias);
 
 }  // namespace lten_hip

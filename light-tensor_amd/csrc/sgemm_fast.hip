@@ -221,7 +221,7 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 		const int n = n0 + wn * TN + j * 32 + lrow;
 		bv[j] = (p.bias && n < p.N) ? p.bias[n] : 0.0f;
 	}
-	if (p.col_group != 0) {  // grouped columns (alpha = 1, beta = 0, no bias): the lane's columns are placed one by one
+	if (p.col_group != 0) {  // grouped columns (alpha = 1, beta = 0, a bias per row): the lane's columns are placed one by one
 		int64_t coff[FN];
 #pragma unroll
 		for (int j = 0; j < FN; j++) {
@@ -235,9 +235,10 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 				const int m = m0 + wm * TM + i * 32 + (r >> 2) * 8 + 4 * lk + (r & 3);
 				if (m >= p.M) continue;
 				float* cr = C + (int64_t)m * p.ldc;
+				const float rb = p.row_bias ? p.row_bias[m] : 0.0f;
 #pragma unroll
 				for (int j = 0; j < FN; j++)
-					if (coff[j] >= 0) cr[coff[j]] = acc[i][j][r];
+					if (coff[j] >= 0) cr[coff[j]] = acc[i][j][r] + rb;
 			}
 		return;
 	}
