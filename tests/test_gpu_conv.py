@@ -343,6 +343,56 @@ def test_conv_weight_gradient_over_few_pixels_by_column_matrices(gpu, ob, geo):
     assert rel_err(dw, want_dw) < TOL
 
 
+def test_conv_by_column_matrices_inside_a_recorded_launch_graph(gpu):
+    """The column routes keep their matrices in memory of the library, which is only allocated outside a recording: a layer
+    that ran once before is recorded with that route and replays to the same values (also after a larger eager call has made
+    the library take a new block); forward, strided data gradient and few-pixel weight gradient."""
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    rng = np.random.default_rng(11)
+    fgeo = (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1)      # forward by columns
+    dgeo = (8, 32, 40, 48, 48, 3, 3, 1, 1, 2, 2)        # strided data gradient by columns
+    wgeo = (2, 2048, 7, 7, 512, 1, 1, 0, 0, 1, 1)       # weight gradient over 98 pixels
+    def operands(geo):
+        N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+        Ho, Wo = (H + 2 * ph - kh) // sh + 1, (W + 2 * pw - kw) // sw + 1
+        x = D.from_numpy(rng.standard_normal((N, Cin, H, W)).astype(np.float32))
+        w = D.from_numpy((rng.standard_normal((Cout, Cin * kh * kw)) * 0.1).astype(np.float32))
+        dy = D.from_numpy(rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32))
+        return x, w, dy, N * Cout * Ho * Wo, N * Cin * H * W, Cout * Cin * kh * kw
+    fx, fw, _, fny, _, _ = operands(fgeo)
+    _, dw_, ddy, _, dnx, _ = operands(dgeo)
+    wx, _, wdy, _, _, wnw = operands(wgeo)
+    fb = D.from_numpy(rng.standard_normal(fgeo[4]).astype(np.float32))
+    y, dx, dwt = D(4 * fny), D(4 * dnx), D(4 * wnw)
+    dws = D(max(int(l.lten_hip_conv2d_dgrad_workspace_bytes(*dgeo)), 16))
+    wws = D(max(int(l.lten_hip_conv2d_wgrad_workspace_bytes(*wgeo)), 16))
+    names = []
+    def step():
+        gpu.check(l.lten_hip_conv2d_forward_f32(*fgeo, fx.ptr, fw.ptr, fb.ptr, y.ptr)); names.append(gpu.last_kernel())
+        gpu.check(l.lten_hip_conv2d_dgrad_f32(*dgeo, dw_.ptr, ddy.ptr, dx.ptr, dws.ptr)); names.append(gpu.last_kernel())
+        gpu.check(l.lten_hip_conv2d_wgrad_f32(*wgeo, wx.ptr, wdy.ptr, dwt.ptr, wws.ptr)); names.append(gpu.last_kernel())
+    step()
+    assert names == ["conv2d_im2col_batched_gemm", "conv2d_dgrad_batched_gemm_col2im", "conv2d_wgrad_columns_gemm"], names
+    want = [y.numpy(np.float32, (fny,)).copy(), dx.numpy(np.float32, (dnx,)).copy(), dwt.numpy(np.float32, (wnw,)).copy()]
+    del names[:]
+    with gpu.Graph() as graph:
+        step()
+    assert names == ["conv2d_im2col_batched_gemm", "conv2d_dgrad_batched_gemm_col2im", "conv2d_wgrad_columns_gemm"], names
+    for rep in range(3):
+        for buf, n in ((y, fny), (dx, dnx), (dwt, wnw)):
+            gpu.check(l.lten_hip_zero(buf.ptr, 4 * n))
+        graph.launch()
+        got = [y.numpy(np.float32, (fny,)), dx.numpy(np.float32, (dnx,)), dwt.numpy(np.float32, (wnw,))]
+        for g_, w_ in zip(got, want):
+            assert np.array_equal(g_, w_)
+        if rep == 0:   # a larger layer, eagerly: the library needs a bigger block and must leave the recorded one alone
+            big = (32, 128, 16, 16, 128, 3, 3, 1, 1, 1, 1)
+            bx, bw, _, bny, _, _ = operands(big)
+            by = D(4 * bny)
+            gpu.check(l.lten_hip_conv2d_forward_f32(*big, bx.ptr, bw.ptr, None, by.ptr))
+            assert gpu.last_kernel().startswith("conv2d_im2col_"), gpu.last_kernel()
+
+
 def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob):
     """Three input channels fill three of the 64 rows of the implicit GEMM's tiles; with a 7 x 7 window on a large image that
     padding costs more than l-ten's own decomposition (GEMM + col2im), which the library then takes: once for the batch,
