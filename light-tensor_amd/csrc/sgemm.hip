@@ -961,6 +961,18 @@ __global__ __launch_bounds__(256) void sgemm_add_partials_kernel(const float* __
 	*c = beta == 0.0f ? alpha * sum : alpha * sum + beta * *c;
 }
 
+// dst[64][cols]: the first `rows` rows of src (leading dimension ld), zeros below
+__global__ __launch_bounds__(256) void sgemm_pad_k_rows_kernel(const float* __restrict__ src, int64_t ld, int rows, int cols, float* __restrict__ dst)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one float4
+	const int c4 = cols / 4;
+	if (idx >= (int64_t)64 * c4) return;
+	const int r = (int)(idx / c4), c = (int)(idx - (int64_t)r * c4) * 4;
+	float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	if (r < rows) v = *reinterpret_cast<const float4*>(src + r * ld + c);
+	reinterpret_cast<float4*>(dst)[idx] = v;
+}
+
 int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
               int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
               int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done, float* relu_out = nullptr,
@@ -994,6 +1006,21 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 			if (rc) return rc;
 		}
 		return 0;
+	}
+	// A^T B over a reduction of fewer than 64 rows into a large output (the weight gradient of a wide layer at a batch of
+	// 32: 4096 x 25088 x 32) is bound by writing C, which the 32 x 32 kernels below do at 1.5 TB/s (100 000 workgroups of
+	// eight wavefronts for one k-step each); the direct-to-LDS tiles want 64 rows at least, so the operands are copied into
+	// 64 rows, the rest zero, in memory the library owns (7 MB against the 411 MB of C: 279 us before).
+	if (get_option(OPT_SGEMM_TILE) == 0 && tA && !tB && batch == 1 && bias == nullptr && relu_done == nullptr && K >= 8 && K < 64 && M % 4 == 0 && N % 4 == 0 &&
+	    lda % 4 == 0 && ldb % 4 == 0 && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
+	    ceil_div(M, 128) * ceil_div(N, 128) >= 512) {
+		float* rows64 = static_cast<float*>(library_scratch(64 * (M + N) * sizeof(float)));
+		if (rows64 != nullptr) {
+			sgemm_pad_k_rows_kernel<<<dim3((unsigned)ceil_div(16 * M, 256)), dim3(256), 0, stream()>>>(A, (int64_t)lda, (int)K, (int)M, rows64);
+			sgemm_pad_k_rows_kernel<<<dim3((unsigned)ceil_div(16 * N, 256)), dim3(256), 0, stream()>>>(B, (int64_t)ldb, (int)K, (int)N, rows64 + 64 * M);
+			LTEN_HIP_LAUNCH_CHECK();
+			return sgemm_run(1, 0, M, N, 64, alpha, rows64, M, 0, rows64 + 64 * M, N, 0, beta, C, ldc, 0, 1, nullptr, nullptr, nullptr);
+		}
 	}
 	// A long reduction into a small output (the weight gradient of a small layer over a large batch: 128 x 128 x 16384)
 	// gives the kernels below a handful of workgroups that each walk all of K: 114 us where the operands' 17 MB take 5.

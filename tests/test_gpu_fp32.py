@@ -87,6 +87,25 @@ def test_long_reduction_into_a_small_output_is_split(gpu, tA, tB, M, N, K):
     assert rel_err(r1[:, :N], (a64 @ b64).astype(np.float32)) < TOL
 
 
+@pytest.mark.parametrize("K", [8, 24, 32, 52])
+def test_short_reduction_into_a_large_output_on_the_large_tiles(gpu, K):
+    """The weight gradient of a wide layer at a small batch, dW = dY^T X with fewer than 64 rows to reduce over and 512 or more
+    tiles of 128 x 128 to write: the operands are copied into 64 rows (the rest zero) for the direct-to-LDS tiles.
+    Integer-valued operands come out exactly; alpha, beta and padded leading dimensions as in every other route."""
+    M, N = 2048, 4096
+    rng = np.random.default_rng(K)
+    A = rng.integers(-4, 5, (K, M + 4)).astype(np.float32)   # stored [K][M], leading dimension M + 4
+    B = rng.integers(-4, 5, (K, N + 8)).astype(np.float32)
+    want = (A[:, :M].astype(np.int64).T @ B[:, :N].astype(np.int64)).astype(np.float32)
+    C0 = np.full((M, N + 4), 7.0, np.float32)
+    got = gpu_sgemm(gpu, 1, 0, M, N, K, 1.0, A, M + 4, B, N + 8, 0.0, C0, N + 4)
+    assert gpu.last_kernel().startswith("sgemm_fast_128x128x32"), gpu.last_kernel()
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, 1, 0, M, N, K, 2.0, A, M + 4, B, N + 8, -1.0, got, N + 4)
+    assert np.array_equal(got2[:, :N], want)
+
+
 def test_beta_zero_overwrites_nan(gpu):
     A = np.ones((5, 3), np.float32)
     B = np.ones((3, 6), np.float32)
