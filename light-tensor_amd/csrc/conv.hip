@@ -474,7 +474,7 @@ static int conv_dgrad_by_columns(const ConvGeo& g, const float* w, const float* 
 	// rows of both operands and of the columns on 16-byte boundaries: what is not so already is copied into padded rows
 	const uint64_t kpitch = (Kc + 3) & ~3ull, hpitch = (HW + 3) & ~3ull;
 	const uint64_t elems = N * Kc * hpitch;
-	if (!(g.Cout >= 32 && g.Cout % 4 == 0 && aligned16(w) && aligned16(dy) && elems <= (1ull << 27) && (uint64_t)g.H * g.W < (1ull << 30) && g.Cin < 65536 &&
+	if (!(g.Cout >= 4 && aligned16(w) && aligned16(dy) && elems <= (1ull << 27) && (uint64_t)g.H * g.W < (1ull << 30) && g.Cin < 65536 &&
 	      (uint64_t)g.Cout * kpitch < (1ull << 30) && N * g.Cout * hpitch < (1ull << 30))) return -1;
 	const uint64_t w_elems = kpitch != Kc ? (uint64_t)g.Cout * kpitch : 0, dy_elems = hpitch != HW ? N * g.Cout * hpitch : 0;
 	float* col = static_cast<float*>(library_scratch((elems + w_elems + dy_elems) * sizeof(float)));
@@ -841,6 +841,16 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
 		if (get_option(OPT_CONV_VARIANT) == 0 && gt.Ho == (int)H && gt.Wo == (int)W && !conv_smallk_takes(gt) && conv_fewout_takes(gt, dy, dx))
 			return conv_fewout_forward(gt, dy, w, nullptr, dx, true);  // reads w transposed and flipped in place
+		// Few input channels, or few tiles of the transposed problem under a long reduction: as a convolution of dy the
+		// gradient fills a fraction of its tiles' rows (10 channels of 32) or leaves most CUs idle, and l-ten's decomposition
+		// done once for the batch is ahead while its columns stay below 100 MB (l-ten's own MNIST network, 1024 x 10 x 12 x 12
+		// <- 20 channels 5 x 5: 115 -> 93 us; its first layer 1024 x 1 x 28 x 28 <- 10: 105 -> 77 us on the element-wise
+		// kernel below, which keeps the small batches; 64 x 20 x 8 x 8 <- 50 channels 5 x 5: 61 -> 17 us).
+		if (get_option(OPT_CONV_VARIANT) == 0 && kh * kw > 1 && Kc * HW * N * sizeof(float) <= (100ull << 20) && N * Cin * H * W >= (1u << 18) / 4 &&
+		    ((Cin <= 16 && N * Cin * H * W >= (1u << 16)) || (ceil_div(Cin, 64) * ceil_div(N * H * W, 64) < 128 && Cout * kh * kw >= 1024))) {
+			const int rc = conv_dgrad_by_columns(g, w, dy, dx);
+			if (rc >= 0) return rc;
+		}
 		if (get_option(OPT_CONV_VARIANT) == 0 && dgrad_direct_takes(g)) {
 			const uint64_t total = N * Cin * H * W;
 			set_kernel_name("conv2d_dgrad_direct");

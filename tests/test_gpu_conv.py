@@ -216,7 +216,7 @@ def test_conv_first_layers_of_narrow_images_on_four_row_chunks(gpu, ob, geo):
     (64, 1, 28, 28, 10, 5, 5, 0, 0, 1, 1),   # l-ten's MNIST layer: eight threads an element, 250 products padded to 256
     (3, 1, 28, 28, 32, 3, 3, 0, 0, 1, 1),    # elements not a multiple of the 32 a workgroup holds
     (2, 4, 19, 23, 7, 4, 2, 2, 1, 1, 1),     # four input channels, even window, padding on both sides
-    (32, 2, 64, 64, 24, 4, 4, 1, 1, 1, 1),   # 2^18 elements: one thread an element
+    (32, 2, 64, 64, 3, 4, 4, 1, 1, 1, 1),    # 2^18 elements: one thread an element (three output channels: too few for the GEMM + col2im route that takes larger batches)
     (1, 3, 9, 300, 5, 1, 7, 0, 3, 1, 1),     # one-row window on a wide image
 ])
 def test_conv_data_gradient_of_first_layers(gpu, ob, geo):
@@ -398,6 +398,26 @@ def test_conv_data_gradient_of_a_strided_first_layer_with_a_large_window(gpu, ob
     padding costs more than l-ten's own decomposition (GEMM + col2im), which the library then takes: once for the batch,
     with the columns in memory of its own; image by image in the caller's workspace when that memory cannot be had."""
     geo = (2, 3, 128, 128, 64, 7, 7, 3, 3, 2, 2)
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel() == "conv2d_dgrad_batched_gemm_col2im", gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+
+
+@pytest.mark.parametrize("geo", [(256, 10, 12, 12, 20, 5, 5, 0, 0, 1, 1),     # l-ten's MNIST conv2 at batch 256: 10 input channels
+                                 (32, 2, 64, 64, 24, 4, 4, 1, 1, 1, 1),       # a first layer with 2^18 input elements
+                                 (64, 20, 8, 8, 50, 5, 5, 0, 0, 1, 1),        # 50 output channels (dy's rows as they lie), 64 tiles under K = 1250
+                                 (64, 6, 14, 14, 16, 5, 5, 0, 0, 1, 1)])      # LeNet's second layer
+def test_conv_data_gradient_of_few_channels_by_column_matrices(gpu, ob, geo):
+    """Stride 1 with few input channels (or few tiles under a long reduction): as a convolution of dy the gradient would fill a
+    fraction of its tiles, and the GEMM + col2im decomposition done once for the batch runs instead; against the oracle."""
     N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
     rng = np.random.default_rng(sum(geo))
     w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
