@@ -67,6 +67,12 @@ __global__ __launch_bounds__(WM* WN * 64) void sgemm_fast_kernel(SProblem p)
 			const int group = lid / (GM * GN), within = lid % (GM * GN), groups_n = tiles_n / GN;
 			tm = (group / groups_n) * GM + within / GN;
 			tn = (group % groups_n) * GN + within % GN;
+		} else if (tiles_m < tiles_n && (nb & 7) == 0 && !p.problems_by_xcd) {
+			// a wide product (few rows of tiles; tiles in a multiple of 8, so an XCD has a run of them): the run walks down the
+			// columns of tiles, so that the XCD reads a narrow range of B and all of the smaller A (256 x 6272 x 2304, 4 x 98
+			// tiles: B crossed the L2s 3.4 times with the run along a row of tiles)
+			tn = lid / tiles_m;
+			tm = lid % tiles_m;
 		} else {
 			tm = lid / tiles_n;
 			tn = lid % tiles_n;
