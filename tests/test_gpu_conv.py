@@ -291,6 +291,7 @@ def test_conv_1x1_layers_as_batched_products(gpu, ob, geo):
                                  (16, 64, 16, 16, 128, 3, 3, 1, 1, 1, 1),    # enough tiles for the 64 x 64 direct-to-LDS kernel
                                  (4, 512, 7, 7, 256, 1, 1, 0, 0, 1, 1),      # 1 x 1 on 7 x 7 maps: 49 pixels, rows of the columns padded to 52
                                  (3, 64, 9, 9, 100, 3, 3, 1, 1, 1, 1),       # 81 pixels
+                                 (63, 96, 7, 7, 128, 3, 3, 1, 1, 1, 1),      # 63 images of 49 pixels: one product with 3087 columns (images start off 16-byte boundaries)
                                  (64, 96, 14, 14, 128, 3, 3, 1, 1, 1, 1)])   # 64 images of 196 pixels: one product with 12544 columns, no tile padded per image
 def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
     """Many channels on images too small for the patch tiles: the batch's column matrices go to memory of the library in one
@@ -306,8 +307,8 @@ def test_conv_deep_layers_on_small_images_by_column_matrices(gpu, ob, geo):
     want_y = np.empty((N, Cout, Ho, Wo), np.float32)
     ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
     # one product over the pixels of the whole batch, stored image by image, where its tiles fill more of the chip than a
-    # product per image does (the last geometry here)
-    route = "conv2d_im2col_gemm" if N == 64 else "conv2d_im2col_batched_gemm"
+    # product per image does (the last two geometries here)
+    route = "conv2d_im2col_gemm" if N >= 63 else "conv2d_im2col_batched_gemm"
     y, _, fk = gpu_conv(gpu, geo, x, w)
     assert fk == route, fk
     assert rel_err(y, want_y) < TOL
