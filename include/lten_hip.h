@@ -83,8 +83,9 @@ int lten_hip_fill_u8(uint8_t* device_ptr, uint64_t count, uint8_t value);
  * (NaN/Inf in C are not propagated); A and B are never modified.  The K == 1
  * (bias rank-1 update) and M == 1 (bias-gradient column sum) shapes those sites use
  * are served by dedicated kernels.  A reduction of 1536 or more into a small output
- * (a weight gradient over a large batch) is cut into slices whose partial sums live in
- * memory the library owns and are added in a fixed order. */
+ * (a weight gradient over a large batch), or of 4096 or more into one of up to 255 tiles
+ * of 64 x 64, is cut into slices whose partial sums live in memory the library owns and
+ * are added in a fixed order. */
 int lten_hip_sgemm(int trans_a, int trans_b, uint64_t M, uint64_t N, uint64_t K, float alpha,
                    const float* A, uint64_t lda, const float* B, uint64_t ldb, float beta,
                    float* C, uint64_t ldc);

@@ -949,16 +949,19 @@ static int launch_sgemm(const SProblem& p, int tA, int tB, uint64_t batch, const
 	return 0;
 }
 
-// C = alpha * (partial[0] + partial[1] + ...) + beta * C, the partial matrices [parts][M][N] added in index order
+// C = alpha * (partial[0] + partial[1] + ...) + beta * C (+ bias per column), the partial matrices [parts][M][N] added in
+// index order
 __global__ __launch_bounds__(256) void sgemm_add_partials_kernel(const float* __restrict__ partial, int parts, int M, int N, float alpha, float beta,
-                                                                 float* __restrict__ C, int64_t ldc)
+                                                                 float* __restrict__ C, int64_t ldc, const float* __restrict__ bias)
 {
 	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, count = (int64_t)M * N;
 	if (idx >= count) return;
 	float sum = 0.0f;
 	for (int s = 0; s < parts; s++) sum += partial[(int64_t)s * count + idx];
-	float* c = C + (idx / N) * ldc + idx % N;
-	*c = beta == 0.0f ? alpha * sum : alpha * sum + beta * *c;
+	const int64_t n = idx % N;
+	float* c = C + (idx / N) * ldc + n;
+	const float v = beta == 0.0f ? alpha * sum : alpha * sum + beta * *c;
+	*c = bias ? v + bias[n] : v;
 }
 
 // dst[64][cols]: the first `rows` rows of src (leading dimension ld), zeros below
@@ -1027,12 +1030,28 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// K is cut into up to 64 slices (of 512 or more) that run as one strided batch into partial matrices (in memory the library owns),
 	// which a second launch adds up in the order of the slices, so the result does not depend on timing.
 	// (Not where the weight-streaming kernels below take the product: few rows against a long or wide weight matrix,
-	// l-ten's 5760 -> 50 layer at batch 64, is their shape and cuts K over a workgroup's wavefronts already.)
-	const bool streams = (!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512);
-	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && bias == nullptr && !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256) {
+	// l-ten's 5760 -> 50 layer at batch 64, is their shape and cuts K over a workgroup's wavefronts already; from 128 rows
+	// and a K of 8192 on the split is ahead of them: 384 x 384 x 16384 NT 97 -> 55 us, 128 x 256 x 8192 31 -> 20 us.)
+	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512));
+	const bool small_out = !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256;
+	// The same for outputs of 65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: the direct-to-LDS tiles run at
+	// their rate from about 512 workgroups on, so K is cut until the slices give that many (256 x 2304 x 6272, 144 tiles:
+	// 104 us whole, 98 in two slices, 75 + 4 in four; 768 x 768 x 8192: 134 -> 96 + 4 us; 512 x 1024 x 8192, which the
+	// weight-streaming kernels took at 104-133 us: 69 + 4 us).
+	const uint64_t tiles64_all = ceil_div(M, 64) * ceil_div(N, 64);
+	const bool mid_out = M >= 128 && N >= 128 && tiles64_all > 64 && tiles64_all < 256 && K >= 4096 && lda % 4 == 0 && ldb % 4 == 0 &&
+	                     ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (tA ? M % 4 == 0 : true) && (tB ? true : N % 4 == 0);
+	// (a bias per column, FullyConnected's, rides on the launch that adds the slices)
+	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && (small_out || mid_out)) {
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);
-		uint64_t slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
-		while (slices > 2 && K / slices < 512) slices /= 2;
+		uint64_t slices;
+		if (small_out) {
+			slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
+			while (slices > 2 && K / slices < 512) slices /= 2;
+		} else {
+			slices = 2;
+			while (tiles64_all * slices < 512 && slices < 16 && K / (slices * 2) >= 1024) slices *= 2;
+		}
 		const uint64_t kc = (K / slices) & ~31ull, rest = K - slices * kc, parts = slices + (rest != 0 ? 1 : 0);
 		float* partial = kc >= 256 ? static_cast<float*>(library_scratch(parts * M * N * sizeof(float))) : nullptr;
 		if (partial != nullptr) {
@@ -1045,7 +1064,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 				if (rc) return rc;
 			}
 			set_kernel_name("sgemm_split_k");
-			sgemm_add_partials_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(partial, (int)parts, (int)M, (int)N, alpha, beta, C, (int64_t)ldc);
+			sgemm_add_partials_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(partial, (int)parts, (int)M, (int)N, alpha, beta, C, (int64_t)ldc, bias);
 			LTEN_HIP_LAUNCH_CHECK();
 			return 0;
 		}

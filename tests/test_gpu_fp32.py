@@ -106,6 +106,38 @@ def test_short_reduction_into_a_large_output_on_the_large_tiles(gpu, K):
     assert np.array_equal(got2[:, :N], want)
 
 
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+def test_long_reduction_into_a_mid_size_output_is_split(gpu, tA, tB):
+    """65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: K is cut until the slices give the direct-to-LDS tiles
+    about 512 workgroups, the partial matrices are added in slice order.  Integer-valued operands come out exactly; alpha,
+    beta and padded leading dimensions as in every other route; FullyConnected's bias rides on the adding launch."""
+    M, N, K = 320, 1280, 4096 + 64
+    rng = np.random.default_rng(7 + 2 * tA + tB)
+    A = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    want = (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32)
+    lda, ldb, ldc = (M if tA else K) + 4, (K if tB else N) + 8, N + 4
+    As = np.zeros(((K if tA else M), lda), np.float32)
+    As[:, :(M if tA else K)] = A.T if tA else A
+    Bs = np.zeros(((N if tB else K), ldb), np.float32)
+    Bs[:, :(K if tB else N)] = B.T if tB else B
+    C0 = np.full((M, ldc), 7.0, np.float32)
+    got = gpu_sgemm(gpu, tA, tB, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, C0, ldc)
+    assert gpu.last_kernel() == "sgemm_split_k", gpu.last_kernel()
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, tA, tB, M, N, K, 2.0, As, lda, Bs, ldb, -1.0, got, ldc)
+    assert np.array_equal(got2[:, :N], want)
+    if not tA and tB:   # the same product as a FullyConnected forward pass with a bias
+        D = gpu.DeviceBuffer
+        X, W = np.ascontiguousarray(A), np.ascontiguousarray(B.T)
+        b = rng.integers(-9, 10, N).astype(np.float32)
+        dX, dW, dB, dY = D.from_numpy(X), D.from_numpy(W), D.from_numpy(b), D(4 * M * N)
+        gpu.check(gpu.lib().lten_hip_fc_forward_f32(M, K, N, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+        assert gpu.last_kernel() == "sgemm_split_k", gpu.last_kernel()
+        assert np.array_equal(dY.numpy(np.float32, (M, N)), want + b[None, :])
+
+
 def test_beta_zero_overwrites_nan(gpu):
     A = np.ones((5, 3), np.float32)
     B = np.ones((3, 6), np.float32)
