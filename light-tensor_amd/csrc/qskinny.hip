@@ -1,5 +1,5 @@
 // Weight-streaming int8 FC for skinny activations (M <= 32 rows against W[N x K], both contiguous in K, K any multiple
-// of 16 up to 8192 — up to 16384 for M <= 16 — and any N).
+// of 16 up to 8192 — up to 16384 for M <= 16, beyond that in chunks of K with a launch that adds them — and any N).
 //
 // The work is one pass over W (N*K bytes, read once from HBM); everything else is noise, so the kernel is
 // organised around that stream.  A workgroup takes 16 consecutive rows of W at a time (then the next such
@@ -23,9 +23,20 @@
 
 namespace lten_hip {
 
-template <int WAVES, int SMAX, int MB, int OUT, bool SUM_A, bool SUM_B>
-__global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const int32_t* bias, int coef_a, int coef_b, int kw)
+template <int WAVES, int SMAX, int MB, int OUT, bool SUM_A, bool SUM_B, bool CHUNKS = false>
+__global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const int32_t* bias, int coef_a, int coef_b, int kw, int chunk_k)
 {
+	// CHUNKS (int32 sums only): K in chunks over blockIdx.y, chunk y takes k from y * chunk_k on and writes its sums to the
+	// y-th [M x N] matrix behind C; the bias goes with the first chunk, the padding bytes are in the last
+	const int k0 = CHUNKS ? (int)blockIdx.y * chunk_k : 0;
+	const int Kc = CHUNKS ? min(chunk_k, p.K - k0) : p.K;
+	const int pad_here = (!CHUNKS || k0 + chunk_k >= p.K) ? p.k_pad : 0;
+	if (CHUNKS) {
+		p.A += k0;
+		p.B += k0;
+		p.C = static_cast<int*>(p.C) + (int64_t)blockIdx.y * p.M * p.N;
+		if (k0 != 0) bias = nullptr;
+	}
 	// kw = bytes of K per wavefront, a multiple of 64, at most SMAX * 64; wavefront w owns k in [w * kw, w * kw + kw) as
 	// far as it lies inside K (any multiple of 16).  A slab holds 1 KB of 16 weight rows: SMAX / 16 passes per row group.
 	constexpr int ROW = 1024 + 16;       // padded LDS row pitch
@@ -41,7 +52,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int kbeg = wave * kw;
-	const int klen = max(0, min(kw, p.K - kbeg));   // this wavefront's share of K (0 for wavefronts past a short K)
+	const int klen = max(0, min(kw, Kc - kbeg));    // this wavefront's share of K (0 for wavefronts past a short K)
 	const int steps = (klen + 63) / 64;              // MFMA steps of 64 k; the last may be partial (K % 64 != 0)
 	const uint32_t slab_addr = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t*)smem + wave * SLAB;
 	const int groups = (p.N + 15) / 16;
@@ -180,7 +191,7 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 		const int n = group * 16 + lrow;
 		// sum a'b' -> l-ten's element: + coef_a * sum_k a' + coef_b * sum_k b' + K * coef_a * coef_b (+ bias)
 		//   with a' = a - 128, coef_a = 128 - zpB, coef_b = 128 - zpA
-		const int base = coef_b * tsb + (p.K - p.k_pad) * coef_a * coef_b + bias_n;
+		const int base = coef_b * tsb + (Kc - pad_here) * coef_a * coef_b + bias_n;
 #pragma unroll
 		for (int mb = 0; mb < MB; mb++) {
 			v4i tot = { 0, 0, 0, 0 };
@@ -207,29 +218,50 @@ __global__ __launch_bounds__(WAVES * 64) void qskinny_kernel(QProblem p, const i
 }
 
 template <int WAVES, int SMAX, int MB>
-static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, int kw, const char* name)
+static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int coef_a, int coef_b, int kw, const char* name, int chunk_k = 0, int chunks = 1)
 {
 	// as many workgroups as fit the CUs' LDS at once (one per CU with eight wavefronts); each walks row groups blockIdx.x, blockIdx.x + grid, ...
 	constexpr int PAR = MB == 1 ? 2 : 1;
 	constexpr int LDS_BYTES = WAVES * 16 * (1024 + 16) + PAR * WAVES * MB * 1024 + (PAR + MB) * WAVES * 64;
 	static_assert(LDS_BYTES <= 160 * 1024, "slabs and partial tiles must fit the CU's LDS");
 	constexpr int PER_CU = (160 * 1024) / LDS_BYTES;
-	const dim3 grid((unsigned)std::min<int64_t>((p.N + 15) / 16, 256 * PER_CU)), block(WAVES * 64);
+	const dim3 grid((unsigned)std::min<int64_t>((p.N + 15) / 16, std::max(1, 256 * PER_CU / chunks)), (unsigned)chunks), block(WAVES * 64);
 	set_kernel_name(name);
 	const bool sum_a = coef_a != 0, sum_b = coef_b != 0;
-#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, SMAX, MB, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b, kw)
+#define LTEN_SK(OUTV, SA, SB) qskinny_kernel<WAVES, SMAX, MB, OUTV, SA, SB><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b, kw, chunk_k)
 #define LTEN_SK_OUT(OUTV)                                     \
 	if (sum_a && sum_b) LTEN_SK(OUTV, true, true);        \
 	else if (sum_a) LTEN_SK(OUTV, true, false);           \
 	else if (sum_b) LTEN_SK(OUTV, false, true);           \
 	else LTEN_SK(OUTV, false, false);
-	if (out == Q_OUT_U8_FAST) { LTEN_SK_OUT(Q_OUT_U8_FAST) }
+#define LTEN_SK_CHUNKS(SA, SB) qskinny_kernel<WAVES, SMAX, MB, Q_OUT_ACC, SA, SB, true><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b, kw, chunk_k)
+	if (chunk_k != 0) {  // (only with int32 sums, and one block of activation rows)
+		if (out != Q_OUT_ACC || MB != 1) return -1;
+		if (sum_a && sum_b) LTEN_SK_CHUNKS(true, true);
+		else if (sum_a) LTEN_SK_CHUNKS(true, false);
+		else if (sum_b) LTEN_SK_CHUNKS(false, true);
+		else LTEN_SK_CHUNKS(false, false);
+	}
+	else if (out == Q_OUT_U8_FAST) { LTEN_SK_OUT(Q_OUT_U8_FAST) }
 	else if (out == Q_OUT_U8_EXACT) { LTEN_SK_OUT(Q_OUT_U8_EXACT) }
 	else { LTEN_SK_OUT(Q_OUT_ACC) }
+#undef LTEN_SK_CHUNKS
 #undef LTEN_SK_OUT
 #undef LTEN_SK
 	LTEN_HIP_LAUNCH_CHECK();
 	return 0;
+}
+
+// out[i] = requantize(acc[0][i] + acc[1][i] + ...) (or the int32 sum itself): the K-chunks of a long reduction meet here
+template <int OUT>
+__global__ __launch_bounds__(256) void qskinny_sum_chunks_kernel(const int32_t* __restrict__ acc, int chunks, int64_t count, float mult, float zp_c, void* __restrict__ out)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	if (idx >= count) return;
+	int v = 0;
+	for (int c = 0; c < chunks; c++) v += acc[(int64_t)c * count + idx];
+	if (OUT == Q_OUT_ACC) static_cast<int*>(out)[idx] = v;
+	else static_cast<uint8_t*>(out)[idx] = (uint8_t)requant<OUT>(v, mult, zp_c);
 }
 
 // Returns -1 when the problem does not fit the streaming kernel (the caller then uses the other kernels): up to 32
@@ -237,10 +269,42 @@ static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int co
 // most 16 rows (the activations of a wavefront's share of K stay in registers).  N is arbitrary.
 int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b)
 {
-	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N >= 1 && p.K >= 64 && p.K <= 16384)) return -1;
+	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N >= 1 && p.K >= 64)) return -1;
 	if (p.K > 8192 && p.M > 16) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
-	// fewest wavefronts whose share of K fits one slab pass (1 KB): more workgroups per CU for a short K
+	if (p.K > 16384) {
+		// A reduction longer than the registers of eight wavefronts hold the activations of (a 25088 -> 4096 layer at batch
+		// 1): K in chunks, all in one launch (grid rows), each into int32 sums of its own in memory the library owns (the
+		// identity's terms are sums over k, so the chunks' l-ten accumulators add up; the bias goes with the first), and a
+		// second launch adds the chunks and requantizes.  As many chunks as give the chip about 512 workgroups with the
+		// groups of 16 weight rows there are (a 1000-row layer has 63), of 2048 or more k each.
+		const uint64_t groups = ceil_div((uint64_t)p.N, 16);
+		int chunks = (int)std::max<uint64_t>(ceil_div((uint64_t)p.K, 16384), std::min<uint64_t>(16, ceil_div(512, groups)));
+		while (chunks > 2 && p.K / chunks < 2048) chunks--;
+		if ((uint64_t)p.K * 255 * 255 >= (1ull << 31)) return -1;
+		const int ck = (int)ceil_div(ceil_div((uint64_t)p.K, (uint64_t)chunks), 64) * 64;
+		chunks = (int)ceil_div((uint64_t)p.K, (uint64_t)ck);
+		const int64_t count = (int64_t)p.M * p.N;
+		int32_t* acc = static_cast<int32_t*>(library_scratch((uint64_t)chunks * count * sizeof(int32_t)));
+		if (acc == nullptr) return -1;
+		QProblem pc = p;
+		pc.C = acc;
+		const int wv = ck <= 2048 ? 2 : (ck <= 4096 ? 4 : 8);
+		const int kwc = (int)ceil_div(ceil_div((uint64_t)ck, (uint64_t)wv), 64) * 64;
+		int rc;
+		if (ck > 8192) rc = launch_skinny<8, 32, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		else if (wv == 8) rc = launch_skinny<8, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		else if (wv == 4) rc = launch_skinny<4, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		else rc = launch_skinny<2, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		if (rc) return rc;
+		const dim3 grid((unsigned)ceil_div((uint64_t)count, 256));
+		if (out == Q_OUT_U8_FAST) qskinny_sum_chunks_kernel<Q_OUT_U8_FAST><<<grid, dim3(256), 0, stream()>>>(acc, chunks, count, p.mult, p.zp_c, p.C);
+		else if (out == Q_OUT_U8_EXACT) qskinny_sum_chunks_kernel<Q_OUT_U8_EXACT><<<grid, dim3(256), 0, stream()>>>(acc, chunks, count, p.mult, p.zp_c, p.C);
+		else qskinny_sum_chunks_kernel<Q_OUT_ACC><<<grid, dim3(256), 0, stream()>>>(acc, chunks, count, p.mult, p.zp_c, p.C);
+		LTEN_HIP_LAUNCH_CHECK();
+		set_kernel_name("qskinny_mfma_kchunks");
+		return 0;
+	}
 	const int waves = p.K <= 2048 ? 2 : (p.K <= 4096 ? 4 : 8);
 	const int kw = (int)ceil_div(ceil_div((uint64_t)p.K, (uint64_t)waves), 64) * 64;
 	if (p.K > 8192) return launch_skinny<8, 32, 1>(p, out, bias, coef_a, coef_b, kw, "qskinny_mfma_w8_2pass");

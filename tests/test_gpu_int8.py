@@ -355,6 +355,21 @@ def test_split_k_shares_of_unequal_length(gpu, ob, splits, K):
         gpu.set_option("qgemm_split", 0)
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 25088), (4, 300, 33024), (16, 130, 20000), (7, 64, 16400)])
+def test_few_rows_against_a_reduction_beyond_16384(gpu, ob, M, N, K):
+    """The weight-streaming kernel holds the activations of at most 16384 k in the registers of its wavefronts: a longer K
+    (a 25088 -> 1000 layer at batch 1) runs in chunks of K, a launch each into int32 sums, and a last launch adds them and
+    requantizes.  Zero points, bias, int32 and u8 outputs against the oracle; the chunks are not equal (K = 16400)."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    run_case(gpu, ob, A, B, [0.02, 0.013, 3.0], np.array([128, 128, 128], np.uint8))
+    assert gpu.last_kernel() == "qskinny_mfma_kchunks", gpu.last_kernel()
+    run_case(gpu, ob, A, B, [0.02, 0.013, 3.0], np.array([3, 250, 77], np.uint8), bias=rng.integers(-5000, 5000, N).astype(np.int32))
+    assert gpu.last_kernel() == "qskinny_mfma_kchunks", gpu.last_kernel()
+    run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 0, 9], np.uint8))
+
+
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
     """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
