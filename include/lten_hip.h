@@ -167,6 +167,9 @@ int lten_hip_fcq_forward(uint64_t batch, uint64_t M, uint64_t in_features, uint6
  * are first copied into rows of that length in memory the library owns (one more launch; the memory is allocated by
  * the first such call and grows with later ones, which cannot happen while a launch graph is being recorded), and
  * lten_hip_fcq_forward and lten_hip_quantized_matmul(0, 1, ...) copy both operands that way on every call.
+ * The same memory holds the int32 sums of the chunks of K that at most 16 rows against an in_features above 16384
+ * are computed in (one launch for the chunks, one that adds them; the tiled kernels take the call when the memory
+ * cannot be had).
  * qparams are the layer's unchanged (the weight zero
  * point still refers to the uint8 representation).  workspace as for lten_hip_fcq_forward; only shapes that fall to
  * the general kernels use it.  No counterpart in l-ten, whose quantized layers are CPU-only. */

@@ -774,6 +774,7 @@ int lten_hip_fcq_forward_static(uint64_t batch, uint64_t M, uint64_t in_features
 	// The array keeps whatever the last call left.  The arrival counters of a split-K launch must start at zero, and
 	// they do without a fill launch: the array is zero when the code object is loaded, and the workgroup that arrives
 	// last at a tile stores zero into its counter again (qgemm_fast_kernel).
+	LibraryScratchHold nothing_else(1ull << 60);  // no kernel choice below may reach for the library's growing block
 	return qgemm_run(0, 1, batch * M, out_features, in_features, X, W, Y, 0, qparams, bias, nullptr, false, &rs);
 }
 

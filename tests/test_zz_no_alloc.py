@@ -88,3 +88,34 @@ def test_static_entry_point_rejects_sizes_beyond_its_scratch(gpu):
     dX, dW, dY = D(M * K, zero=True), D(N * K, zero=True), D(M * N)
     rc = l.lten_hip_fcq_forward_static(1, M, K, N, dX.ptr, dW.ptr, None, gpu.qparams3([1, 1, 1], [0, 0, 0]), dY.ptr)
     assert rc != 0 and b"exceeds the limit" in l.lten_hip_last_error()
+
+
+def test_static_entry_point_on_a_long_reduction_stays_off_library_memory(gpu, ob):
+    """Four rows against K = 20000: lten_hip_fcq_forward runs the weight-streaming kernel in chunks of K with their sums in
+    memory the library allocates; the static entry point must not, takes another kernel, and returns the same bytes."""
+    import ctypes as C
+    rng = np.random.default_rng(99)
+    M, N, K = 4, 256, 20000
+    X = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    W = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    sc, zp = [0.02, 0.013, 3.0], [3, 250, 77]
+    hip = C.CDLL("libamdhip64.so")
+    free0, free1, total = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    l, D = gpu.lib(), gpu.DeviceBuffer
+    dX, dW, db, y = D.from_numpy(X), D.from_numpy(W), D.from_numpy(bias), D(M * N, zero=True)
+    qp = gpu.qparams3(sc, zp)
+    gpu.sync()
+    assert hip.hipMemGetInfo(C.byref(free0), C.byref(total)) == 0
+    gpu.check(l.lten_hip_fcq_forward_static(1, M, K, N, dX.ptr, dW.ptr, db.ptr, qp, y.ptr))
+    k_new = gpu.last_kernel()
+    gpu.sync()
+    assert hip.hipMemGetInfo(C.byref(free1), C.byref(total)) == 0
+    assert free1.value == free0.value
+    assert k_new != "qskinny_mfma_kchunks", k_new
+    got = y.numpy(np.uint8, (M, N)).copy()
+    want, _, k_ref, _ = both(gpu, X, W, sc, zp, bias)
+    assert k_ref == "qskinny_mfma_kchunks", k_ref
+    assert np.array_equal(got, want)
+    Co, _ = ob.quantized_matmul(X, W, np.array(sc, np.float32), np.array(zp, np.uint8), bias=bias)
+    assert np.array_equal(want, Co)
