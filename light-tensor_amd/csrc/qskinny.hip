@@ -235,8 +235,8 @@ static int launch_skinny(const QProblem& p, int out, const int32_t* bias, int co
 	else if (sum_b) LTEN_SK(OUTV, false, true);           \
 	else LTEN_SK(OUTV, false, false);
 #define LTEN_SK_CHUNKS(SA, SB) qskinny_kernel<WAVES, SMAX, MB, Q_OUT_ACC, SA, SB, true><<<grid, block, 0, stream()>>>(p, bias, coef_a, coef_b, kw, chunk_k)
-	if (chunk_k != 0) {  // (only with int32 sums, and one block of activation rows)
-		if (out != Q_OUT_ACC || MB != 1) return -1;
+	if (chunk_k != 0) {  // (only with int32 sums)
+		if (out != Q_OUT_ACC) return -1;
 		if (sum_a && sum_b) LTEN_SK_CHUNKS(true, true);
 		else if (sum_a) LTEN_SK_CHUNKS(true, false);
 		else if (sum_b) LTEN_SK_CHUNKS(false, true);
@@ -270,16 +270,16 @@ __global__ __launch_bounds__(256) void qskinny_sum_chunks_kernel(const int32_t* 
 int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, int zp_b)
 {
 	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N >= 1 && p.K >= 64)) return -1;
-	if (p.K > 8192 && p.M > 16) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
-	if (p.K > 16384) {
+	const int k_whole = p.M > 16 ? 8192 : 16384;  // what one launch takes whole: the activations of a wavefront's share sit in registers
+	if (p.K > k_whole) {
 		// A reduction longer than the registers of eight wavefronts hold the activations of (a 25088 -> 4096 layer at batch
-		// 1): K in chunks, all in one launch (grid rows), each into int32 sums of its own in memory the library owns (the
+		// 1; from 17 rows on, K above 8192): K in chunks, all in one launch (grid rows), each into int32 sums of its own in memory the library owns (the
 		// identity's terms are sums over k, so the chunks' l-ten accumulators add up; the bias goes with the first), and a
 		// second launch adds the chunks and requantizes.  As many chunks as give the chip about 512 workgroups with the
 		// groups of 16 weight rows there are (a 1000-row layer has 63), of 2048 or more k each.
 		const uint64_t groups = ceil_div((uint64_t)p.N, 16);
-		int chunks = (int)std::max<uint64_t>(ceil_div((uint64_t)p.K, 16384), std::min<uint64_t>(16, ceil_div(512, groups)));
+		int chunks = (int)std::max<uint64_t>(ceil_div((uint64_t)p.K, (uint64_t)k_whole), std::min<uint64_t>(16, ceil_div(512, groups)));
 		while (chunks > 2 && p.K / chunks < 2048) chunks--;
 		if ((uint64_t)p.K * 255 * 255 >= (1ull << 31)) return -1;
 		const int ck = (int)ceil_div(ceil_div((uint64_t)p.K, (uint64_t)chunks), 64) * 64;
@@ -292,7 +292,12 @@ int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 		const int wv = ck <= 2048 ? 2 : (ck <= 4096 ? 4 : 8);
 		const int kwc = (int)ceil_div(ceil_div((uint64_t)ck, (uint64_t)wv), 64) * 64;
 		int rc;
-		if (ck > 8192) rc = launch_skinny<8, 32, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		if (p.M > 16) {  // two blocks of 16 activation rows, chunks of at most 8192
+			if (wv == 8) rc = launch_skinny<8, 16, 2>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+			else if (wv == 4) rc = launch_skinny<4, 16, 2>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+			else rc = launch_skinny<2, 16, 2>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
+		}
+		else if (ck > 8192) rc = launch_skinny<8, 32, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
 		else if (wv == 8) rc = launch_skinny<8, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
 		else if (wv == 4) rc = launch_skinny<4, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);
 		else rc = launch_skinny<2, 16, 1>(pc, Q_OUT_ACC, bias, coef_a, coef_b, kwc, "qskinny", ck, chunks);

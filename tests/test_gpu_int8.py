@@ -355,10 +355,10 @@ def test_split_k_shares_of_unequal_length(gpu, ob, splits, K):
         gpu.set_option("qgemm_split", 0)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 1000, 25088), (4, 300, 33024), (16, 130, 20000), (7, 64, 16400)])
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 25088), (4, 300, 33024), (16, 130, 20000), (7, 64, 16400), (20, 200, 12000), (32, 100, 30000)])
 def test_few_rows_against_a_reduction_beyond_16384(gpu, ob, M, N, K):
-    """The weight-streaming kernel holds the activations of at most 16384 k in the registers of its wavefronts: a longer K
-    (a 25088 -> 1000 layer at batch 1) runs in chunks of K, a launch each into int32 sums, and a last launch adds them and
+    """The weight-streaming kernel holds the activations of at most 16384 k (8192 from 17 rows on) in the registers of its
+    wavefronts: a longer K (a 25088 -> 1000 layer at batch 1) runs in chunks of K, a launch each into int32 sums, and a last launch adds them and
     requantizes.  Zero points, bias, int32 and u8 outputs against the oracle; the chunks are not equal (K = 16400)."""
     rng = np.random.default_rng(M + N + K)
     A = rng.integers(0, 256, (M, K), dtype=np.uint8)
