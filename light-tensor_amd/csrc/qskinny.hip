@@ -272,7 +272,9 @@ int qskinny_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.M >= 1 && p.M <= 32 && p.N >= 1 && p.K >= 64)) return -1;
 	const int coef_a = 128 - zp_b, coef_b = 128 - zp_a;
 	const int k_whole = p.M > 16 ? 8192 : 16384;  // what one launch takes whole: the activations of a wavefront's share sit in registers
-	if (p.K > k_whole) {
+	// (also a K of 16384 against fewer than 128 groups of 16 weight rows, which would leave half of the CUs idle through two
+	// slab passes: 1 x 1000 x 16384 12 us whole)
+	if (p.K > k_whole || (p.K >= 16384 && p.N < 128 * 16)) {
 		// A reduction longer than the registers of eight wavefronts hold the activations of (a 25088 -> 4096 layer at batch
 		// 1; from 17 rows on, K above 8192): K in chunks, all in one launch (grid rows), each into int32 sums of its own in memory the library owns (the
 		// identity's terms are sums over k, so the chunks' l-ten accumulators add up; the bias goes with the first), and a
