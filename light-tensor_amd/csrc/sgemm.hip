@@ -874,6 +874,24 @@ __global__ __launch_bounds__(256) void sgemm_rank1_kernel(SProblem p, int tA, in
 	*c = v;
 }
 
+// The same, four columns per thread: N and ldc multiples of 4, C on a 16-byte boundary, b contiguous (tB == 0).
+__global__ __launch_bounds__(256) void sgemm_rank1_vec4_kernel(SProblem p, int tA)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	const int n4 = p.N / 4;
+	if (idx >= (int64_t)p.M * n4) return;
+	const int m = (int)(idx / n4), n = (int)(idx - (int64_t)m * n4) * 4;
+	const float a = tA ? p.A[m] : p.A[(int64_t)m * p.lda];
+	const float4 b = *reinterpret_cast<const float4*>(p.B + n);
+	float4* c = reinterpret_cast<float4*>(p.C + (int64_t)m * p.ldc + n);
+	float4 v = make_float4(p.alpha * (a * b.x), p.alpha * (a * b.y), p.alpha * (a * b.z), p.alpha * (a * b.w));
+	if (p.beta != 0.0f) {
+		const float4 o = *c;
+		v.x += p.beta * o.x; v.y += p.beta * o.y; v.z += p.beta * o.z; v.w += p.beta * o.w;
+	}
+	*c = v;
+}
+
 // M == 1 with B not transposed: c[n] = alpha * sum_k a[k] B[k][n] + beta * c[n] — the column sum that
 // l-ten uses for the bias gradient with a = ones (l-ten/backprop.cpp:2267) and the two products of a GRU time
 // step (l-ten/gru.cpp:267-268).  A workgroup takes COLS columns and cuts K into SLICES slices, one thread per
@@ -1014,7 +1032,7 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// 32: 4096 x 25088 x 32) is bound by writing C, which the 32 x 32 kernels below do at 1.5 TB/s (100 000 workgroups of
 	// eight wavefronts for one k-step each); the direct-to-LDS tiles want 64 rows at least, so the operands are copied into
 	// 64 rows, the rest zero, in memory the library owns (7 MB against the 411 MB of C: 279 us before).
-	if (get_option(OPT_SGEMM_TILE) == 0 && tA && !tB && batch == 1 && bias == nullptr && relu_done == nullptr && K >= 8 && K < 64 && M % 4 == 0 && N % 4 == 0 &&
+	if (get_option(OPT_SGEMM_TILE) == 0 && tA && !tB && batch == 1 && bias == nullptr && relu_done == nullptr && K >= 2 && K < 64 && M % 4 == 0 && N % 4 == 0 &&
 	    lda % 4 == 0 && ldb % 4 == 0 && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
 	    ceil_div(M, 128) * ceil_div(N, 128) >= 512) {
 		float* rows64 = static_cast<float*>(library_scratch(64 * (M + N) * sizeof(float)));
@@ -1032,7 +1050,9 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// (Not where the weight-streaming kernels below take the product: few rows against a long or wide weight matrix,
 	// l-ten's 5760 -> 50 layer at batch 64, is their shape and cuts K over a workgroup's wavefronts already; from 128 rows
 	// and a K of 8192 on the split is ahead of them: 384 x 384 x 16384 NT 97 -> 55 us, 128 x 256 x 8192 31 -> 20 us.)
-	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512));
+	// (the NN streaming kernel wants more than 16 rows, a single row has the row-vector kernel: 2 to 16 rows against a long K
+	// had neither and walked K on 32 workgroups, 4 x 1024 x 32000 in 202 us)
+	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0) || (!tA && !tB && N >= 512 && (M == 1 || M > 16)));
 	const bool small_out = !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256;
 	// The same for outputs of 65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: the direct-to-LDS tiles run at
 	// their rate from about 512 workgroups on, so K is cut until the slices give that many (256 x 2304 x 6272, 144 tiles:
@@ -1081,7 +1101,9 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	const int force = get_option(OPT_SGEMM_TILE);
 	if (force == 0 && batch == 1 && bias == nullptr && K == 1) {
 		set_kernel_name("sgemm_rank1");
-		sgemm_rank1_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(p, tA, tB);
+		if (!tB && N % 4 == 0 && ldc % 4 == 0 && ((reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && M * N >= (1u << 16))
+			sgemm_rank1_vec4_kernel<<<dim3((unsigned)ceil_div(M * (N / 4), 256)), dim3(256), 0, stream()>>>(p, tA);
+		else sgemm_rank1_kernel<<<dim3((unsigned)ceil_div(M * N, 256)), dim3(256), 0, stream()>>>(p, tA, tB);
 		LTEN_HIP_LAUNCH_CHECK();
 		return 0;
 	}

@@ -228,6 +228,15 @@ def test_rank1_and_rowvec_shapes(gpu, ob):
     got = gpu_sgemm(gpu, 0, 0, M, N, 1, 1.0, ones, 1, bias, N, 1.0, Y0, N)
     assert gpu.last_kernel() == "sgemm_rank1"
     assert np.array_equal(got, Y0 + bias)
+    # the weight gradient of a layer at batch 1, dW = dy^T x (A stored [1][M]), alpha and beta at work: the four-column form
+    # (M * N >= 2^16, N a multiple of 4) and the one-column form (N = 1023) give the same rounding, alpha * (a * b) + beta * c
+    dyv = rng.standard_normal((1, M)).astype(np.float32)
+    for n in (N, N - 1):
+        xv = rng.standard_normal((1, n)).astype(np.float32)
+        C0 = rng.standard_normal((M, n)).astype(np.float32)
+        got = gpu_sgemm(gpu, 1, 0, M, n, 1, 0.5, dyv, M, xv, n, -2.0, C0, n)
+        assert gpu.last_kernel() == "sgemm_rank1"
+        assert np.array_equal(got, np.float32(0.5) * (dyv.T * xv) + np.float32(-2.0) * C0)
     # l-ten/backprop.cpp:2267: db[1 x N] += ones[1 x M] dY[M x N]
     db0 = rng.standard_normal((1, N)).astype(np.float32)
     got = gpu_sgemm(gpu, 0, 0, 1, N, M, 1.0, np.ones((1, M), np.float32), M, Y0, N, 1.0, db0, N)
