@@ -138,6 +138,24 @@ def test_long_reduction_into_a_mid_size_output_is_split(gpu, tA, tB):
         assert np.array_equal(dY.numpy(np.float32, (M, N)), want + b[None, :])
 
 
+@pytest.mark.parametrize("rows", [1, 8])
+def test_fc_forward_of_few_rows_onto_few_outputs_over_a_long_reduction_is_split(gpu, rows):
+    """A classifier behind a flattened feature map (1 x 25088 -> 1000): one workgroup per 16 outputs of the streaming NT
+    kernel would leave most CUs idle, so the reduction of 8192 or more is cut into slices instead.  Integer-valued operands
+    come out exactly, bias included; one more column group (1040 outputs at 8 rows is still under 128 groups) too."""
+    K, N = 8192 + 64, 1000
+    rng = np.random.default_rng(31 + rows)
+    X = rng.integers(-4, 5, (rows, K)).astype(np.float32)
+    W = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    b = rng.integers(-9, 10, N).astype(np.float32)
+    want = (X.astype(np.float64) @ W.astype(np.float64).T).astype(np.float32) + b[None, :]
+    D = gpu.DeviceBuffer
+    dX, dW, dB, dY = D.from_numpy(X), D.from_numpy(W), D.from_numpy(b), D(4 * rows * N)
+    gpu.check(gpu.lib().lten_hip_fc_forward_f32(rows, K, N, dX.ptr, dW.ptr, dB.ptr, dY.ptr))
+    assert gpu.last_kernel() == "sgemm_split_k", gpu.last_kernel()
+    assert np.array_equal(dY.numpy(np.float32, (rows, N)), want)
+
+
 def test_beta_zero_overwrites_nan(gpu):
     A = np.ones((5, 3), np.float32)
     B = np.ones((3, 6), np.float32)
