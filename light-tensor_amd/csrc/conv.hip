@@ -881,8 +881,20 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	// With a stride, l-ten's decomposition done once for the batch is ahead of the implicit GEMM below from about a
 	// megabyte of columns on (32 x 64 x 56 x 56 <- 128 channels 3 x 3 stride 2: 130 -> 101 us; 32 x 128 x 28 x 28 <- 256:
 	// 174 -> 86 us; 32 x 4 x 56 x 56 <- 64: 65 -> 15 us; the first layer above: 333 us), except for 1 x 1 windows, whose
-	// columns are dy itself (32 x 64 x 56 x 56 <- 128 at stride 2: 24 against 36 us).
-	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows) && N * Kc * HW >= (1u << 18)) {
+	// columns are dy itself (32 x 64 x 56 x 56 <- 128 at stride 2: 24 against 36 us), while the layers are small: the
+	// implicit GEMM runs them at 29 TFLOP/s (only the pixels that a 1 x 1 window reaches do any work, and with few of
+	// them few of its tiles), the GEMM of the decomposition at 88, and the pass that spreads its result over dx takes
+	// the rest (32 x 256 x 56 x 56 <- 512 at stride 2: 222 -> 148 us; 32 x 1024 x 14 x 14 <- 2048: 231 -> 97 us;
+	// 4 x 512 x 28 x 28 <- 1024: 84 -> 32 us; 32 x 128 x 56 x 56 <- 256 level at 65 us and left below).
+	bool one_by_one_pays = false;
+	if (kh * kw == 1) {
+		const double flops = 2.0 * (double)N * HW * Cout * Cin;
+		const double tiles = (double)(ceil_div(Cin, 64) * ceil_div(N * HW, 64));
+		const double implicit_us = std::max(20.0, flops / (29e6 * std::min(1.0, tiles / 256.0)));
+		const double columns_us = 10.0 + flops / 88e6 + 4.0 * (double)(N * Cin * H * W + 2 * N * Cin * HW) / 2.5e6;
+		one_by_one_pays = columns_us * 1.1 < implicit_us;
+	}
+	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows || one_by_one_pays) && N * Kc * HW >= (1u << 18)) {
 		const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 		if (rc >= 0) return rc;
 	}

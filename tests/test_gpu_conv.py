@@ -437,7 +437,8 @@ def test_conv_data_gradient_of_few_channels_by_column_matrices(gpu, ob, geo):
                                  (3, 5, 40, 40, 32, 7, 7, 3, 3, 2, 2),        # K = 245: the weights' rows are padded to a multiple of four floats
                                  (8, 40, 32, 32, 64, 2, 2, 0, 0, 2, 2),       # windows that do not overlap
                                  (6, 32, 25, 29, 64, 3, 3, 1, 1, 2, 2),       # 13 x 15 = 195 output pixels: dy is copied into rows of 196 floats
-                                 (32, 5, 29, 29, 36, 3, 3, 1, 1, 2, 2)])      # K = 45 and 225 output pixels: both operands copied into padded rows
+                                 (32, 5, 29, 29, 36, 3, 3, 1, 1, 2, 2),       # K = 45 and 225 output pixels: both operands copied into padded rows
+                                 (6, 256, 28, 29, 512, 1, 1, 0, 0, 2, 2)])    # 1 x 1 at stride 2 between wide layers (a residual network's shortcut): the columns are dy
 def test_conv_strided_data_gradient_by_column_matrices(gpu, ob, geo):
     """With a stride and a megabyte or more of columns, l-ten's GEMM + col2im runs once for the batch: a strided batch of
     TN products into memory of the library, one col2im launch; against the oracle, and against the implicit GEMM."""
