@@ -846,8 +846,22 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		// done once for the batch is ahead while its columns stay below 100 MB (l-ten's own MNIST network, 1024 x 10 x 12 x 12
 		// <- 20 channels 5 x 5: 115 -> 93 us; its first layer 1024 x 1 x 28 x 28 <- 10: 105 -> 77 us on the element-wise
 		// kernel below, which keeps the small batches; 64 x 20 x 8 x 8 <- 50 channels 5 x 5: 61 -> 17 us).
+		// With few input channels an estimate of both decides: the columns are written and read at about 1.2 TB/s; as a
+		// convolution of dy the gradient runs on the 3 x 3 patch kernels at about 20 TFLOP/s where they take it, else on
+		// the implicit GEMM at 45 TFLOP/s of tile rows, 32 or 64 of them for the few channels (16 x 16 x 64 x 64 <- 16
+		// channels 3 x 3: columns 44, patch kernel 18 us; 64 x 16 x 32 x 32 <- 32: 46 against 30 us, <- 64: 44 against 55 us;
+		// 128 x 3 x 32 x 32 <- 64 channels 5 x 5: 48 against 272 us).
+		bool few_channels = false;
+		if (Cin <= 16 && N * Cin * H * W >= (1u << 16) && gt.Ho == (int)H && gt.Wo == (int)W) {
+			const double macs = 2.0 * (double)(N * H * W) * Cout * kh * kw;  // per output channel of the convolution of dy
+			const uint64_t patch_tiles = ceil_div(W, 128) * ceil_div(H, 4) * ceil_div(Cin, 64) * N;
+			const bool on_patches = conv_patch_forward_takes(gt, dy, dx) && (conv_patch_fast_forward_takes(gt, dy, work) || (W > 56 && patch_tiles >= 256));
+			const double tile_rows = ceil_div(N * H * W, 128) >= 256 ? 32.0 : 64.0;
+			const double as_convolution_us = on_patches ? 10.0 + macs * Cin / 20e6 : 14.0 + macs * tile_rows / 45e6;
+			few_channels = 15.0 + 4.0 * (double)(Kc * HW * N) / 1.2e6 < as_convolution_us;
+		}
 		if (get_option(OPT_CONV_VARIANT) == 0 && kh * kw > 1 && Kc * HW * N * sizeof(float) <= (100ull << 20) && N * Cin * H * W >= (1u << 18) / 4 &&
-		    ((Cin <= 16 && N * Cin * H * W >= (1u << 16)) || (ceil_div(Cin, 64) * ceil_div(N * H * W, 64) < 128 && Cout * kh * kw >= 1024))) {
+		    (few_channels || (ceil_div(Cin, 64) * ceil_div(N * H * W, 64) < 128 && Cout * kh * kw >= 1024))) {
 			const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 			if (rc >= 0) return rc;
 		}

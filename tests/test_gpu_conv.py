@@ -432,6 +432,25 @@ def test_conv_data_gradient_of_few_channels_by_column_matrices(gpu, ob, geo):
     assert rel_err(dx, want_dx) < TOL
 
 
+@pytest.mark.parametrize("geo,route", [((16, 16, 64, 64, 16, 3, 3, 1, 1, 1, 1), "conv2d_patch"),     # 3 x 3 on wide rows: the patch kernels
+                                       ((64, 8, 32, 32, 8, 3, 3, 1, 1, 1, 1), "conv2d_forward"),     # a short reduction: the implicit GEMM
+                                       ((64, 16, 16, 16, 128, 3, 3, 1, 1, 1, 1), "conv2d_dgrad_batched_gemm_col2im")])   # a long one: the columns
+def test_conv_data_gradient_of_few_channels_takes_the_cheaper_route(gpu, ob, geo, route):
+    """Few input channels at stride 1: an estimate decides between the column matrices and the convolution of dy with the
+    flipped weights (which runs 3 x 3 windows on the patch kernels); whichever it picks, against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.2).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    dy = rng.standard_normal((N, Cout, Ho, Wo)).astype(np.float32)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_dx = np.empty((N, Cin, H, W), np.float32)
+    ob.oracle().oracle_conv2d_dgrad(*geo, w.reshape(-1), dy.reshape(-1), want_dx.reshape(-1), col)
+    dx = gpu_dgrad(gpu, geo, w, dy)
+    assert gpu.last_kernel().startswith(route), gpu.last_kernel()
+    assert rel_err(dx, want_dx) < TOL
+
+
 @pytest.mark.parametrize("geo", [(8, 32, 40, 48, 48, 3, 3, 1, 1, 2, 2),       # 3 x 3 at stride 2
                                  (4, 24, 34, 30, 36, 5, 4, 2, 1, 3, 2),       # strides 3 x 2, oblong window
                                  (3, 5, 40, 40, 32, 7, 7, 3, 3, 2, 2),        # K = 245: the weights' rows are padded to a multiple of four floats
