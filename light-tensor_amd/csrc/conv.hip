@@ -569,7 +569,9 @@ static int conv_wgrad_by_columns(const ConvGeo& g, const float* x, const float* 
 	const bool splits = tiles32 <= 256 && P >= 1536;
 	double gemm_us;
 	// (sgemm_run: the direct-to-LDS tiles from K = 256 in whole k-steps of 32, or from 512 with a second pass for the rest)
-	if ((tiles128 >= 128 || tiles64 >= 128) && P >= 256 && (P % 32 == 0 || P >= 512))
+	if (tiles64 >= 65 && tiles64 < 256 && P >= 4096 && Cout >= 128 && Kc >= 128)  // (a long reduction into a mid-size output: slices of K on the same tiles)
+		gemm_us = flops / 95e6 + 8.0;
+	else if ((tiles128 >= 128 || tiles64 >= 128) && P >= 256 && (P % 32 == 0 || P >= 512))
 		gemm_us = 2.0 * whole(Cout, tiles128 >= 128 ? 128 : 64) * whole(Kc, tiles128 >= 128 ? 128 : 64) * (double)P / 85e6 * (P % 32 == 0 ? 1.0 : 1.15) + 8.0;
 	else
 		gemm_us = flops / (45e6 * (splits ? 1.0 : std::min(1.0, (double)tiles32 / 256.0))) + (splits ? 8.0 : 4.0);
