@@ -1156,14 +1156,19 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// (a short K, 64 to 255 in whole steps of 32, only with many tiles: the products of a batch of attention heads, or an
 	// outer-product-like update; 96 x (512 x 512 x 64): 78-91 us on the 32 x 32 kernel, 45 us here; 4096 x 4096 x 64:
 	// 52-58 and 28 us; with 96 tiles of 128 x 128 the two are level)
-	const bool short_k = K >= 64 && K < 256 && K % 32 == 0 && tiles128 >= 512;
+	// (measured again over batches of small products: at K = 64 the 128 x 128 tiles are ahead from 192 of them on, 16 x (512 x
+	// 512 x 64) 17 -> 9 us, 96 x (256 x 256 x 64) 24 -> 13 us, 2048 x 2048 x 64 17 -> 9 us, and behind with 64, where the 32 x
+	// 32 kernel stays; from K = 96 on the 64 x 64 tiles from 256 of them on: 8 x (512 x 512 x 128) 13 -> 10 us, 384 x (128 x 64 x
+	// 128) 22 -> 16 us, 2048 x 1024 x 96 11 -> 9 us)
+	const bool many128 = tiles128 >= 192 && M > 64 && N > 64;
+	const bool short_k = K >= 64 && K < 256 && K % 32 == 0 && (tiles128 >= 512 || many128 || (K >= 96 && tiles64 >= 256));
 	if (choice == 0 && (tiles128 >= 128 || t64) && ((K >= 256 && (K % 32 == 0 || K >= 512)) || short_k)) {
 		// large problems: 256 x 256 tiles when they fill the chip, else 128 x 128 (or 64 x 64, above).  The tiles walk K in
 		// steps of 32: what is left over is added by a second, general launch (beta = 1, no bias).
 		const bool big = ceil_div(M, 256) * ceil_div(N, 256) * batch >= 192 && M >= 192 && N >= 192 && !short_k;
 		const uint64_t k_main = K & ~31ull;
 		p.K = (int)k_main;
-		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : (t64 ? 31 : 21)) == 0) {
+		if (sgemm_fast_dispatch(p, tA, tB, batch, big ? 12 : (t64 && !(K < 96 && many128) ? 31 : 21)) == 0) {
 			if (k_main == K) return 0;
 			return sgemm_run(tA, tB, M, N, K - k_main, alpha, A + (tA ? k_main * lda : k_main), lda, stride_a,
 			                 B + (tB ? k_main : k_main * ldb), ldb, stride_b, 1.0f, C, ldc, stride_c, batch, nullptr, nullptr, nullptr);

@@ -358,6 +358,30 @@ def test_stack_against_one_shared_matrix(gpu, batch, M, K, N, tB):
     assert rel_err(dC.numpy(np.float32, c0.shape), want.astype(np.float32)) < TOL, gpu.last_kernel()
 
 
+@pytest.mark.parametrize("layout", [(0, 0), (0, 1), (1, 0)])
+@pytest.mark.parametrize("batch,M,N,K,tile", [(24, 256, 512, 64, "sgemm_fast_128x128"),    # 8 tiles of 128 x 128 a product: 192
+                                              (13, 256, 320, 128, "sgemm_fast_64x64"),     # 20 tiles of 64 x 64 a product: 260
+                                              (6, 260, 516, 96, "sgemm_fast_64x64")])      # ragged last tiles, K = 96: three k-steps
+def test_stack_of_products_over_a_short_reduction(gpu, batch, M, N, K, tile, layout):
+    """A batch of attention-head-sized products (K of 64 to 255 in whole steps of 32): on the direct-to-LDS tiles from 192 tiles
+    of 128 x 128 (K = 64) or 256 tiles of 64 x 64 (K >= 96) on.  Integer-valued operands come out exactly in every layout;
+    alpha and beta as everywhere."""
+    tA, tB = layout
+    rng = np.random.default_rng(batch + M + N + K + 2 * tA + tB)
+    a = rng.integers(-4, 5, (batch, M, K)).astype(np.float32)
+    b = rng.integers(-4, 5, (batch, K, N)).astype(np.float32)
+    c0 = rng.integers(-9, 10, (batch, M, N)).astype(np.float32)
+    want = 2.0 * (a.astype(np.float64) @ b.astype(np.float64)) - c0
+    D = gpu.DeviceBuffer
+    dA = D.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1)) if tA else a)
+    dB = D.from_numpy(np.ascontiguousarray(b.transpose(0, 2, 1)) if tB else b)
+    dC = D.from_numpy(c0)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(tA, tB, M, N, K, 2.0, dA.ptr, M if tA else K, M * K, dB.ptr, K if tB else N, K * N,
+                                                       -1.0, dC.ptr, N, M * N, batch))
+    assert gpu.last_kernel().startswith(tile), gpu.last_kernel()
+    assert np.array_equal(dC.numpy(np.float32, c0.shape), want.astype(np.float32))
+
+
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     cases = []
