@@ -163,3 +163,49 @@ def test_conv2d_random_geometries_exact(gpu, ob, seed):
         wsd, dDX = D(max(int(l.lten_hip_conv2d_dgrad_workspace_bytes(*geo)), 4)), D(x.nbytes)
         gpu.check(l.lten_hip_conv2d_dgrad_f32(*geo, dW.ptr, dDY.ptr, dDX.ptr, wsd.ptr))
         assert np.array_equal(dDX.numpy(np.float32, x.shape), want_dx), (seed, it, geo, "dgrad", gpu.last_kernel())
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_conv2dq_random_geometries_bit_exact(gpu, ob, seed):
+    """Conv2d_q forward on random geometries, zero points and (l-ten's per-pixel) bias: accumulators and requantized outputs
+    bit for bit against the oracle; even seeds draw network-like layers, odd seeds anything."""
+    rng = np.random.default_rng(seed)
+    for it in range(60):
+        while True:
+            N = int(rng.choice([1, 1, 2, 3, 4, 8, 16, 32]))
+            Cin = int(rng.choice([1, 2, 3, 4, 5, 8, 10, 16, 20, 24, 32, 48, 64, 96, 128, 256]))
+            Cout = int(rng.choice([1, 2, 3, 4, 6, 8, 10, 16, 20, 32, 33, 48, 64, 96, 128, 256]))
+            H = int(rng.choice([4, 5, 7, 8, 12, 13, 14, 16, 24, 28, 29, 32, 48, 56, 64]))
+            W = H if rng.random() < 0.6 else int(rng.choice([4, 6, 7, 8, 12, 14, 16, 20, 28, 30, 32, 50, 56, 64, 100]))
+            kh = int(rng.choice([1, 1, 2, 3, 3, 3, 4, 5, 5, 7]))
+            kw = kh if rng.random() < 0.8 else int(rng.choice([1, 2, 3, 4, 5]))
+            ph = int(rng.integers(0, kh)) if rng.random() < 0.7 else 0
+            pw = int(rng.integers(0, kw)) if rng.random() < 0.7 else 0
+            sh = int(rng.choice([1, 1, 1, 2, 2, 3]))
+            sw = sh if rng.random() < 0.85 else int(rng.choice([1, 2]))
+            if seed % 2 == 0:
+                Cin, Cout = int(rng.choice([3, 8, 16, 32, 64, 128, 256, 512, 1024])), int(rng.choice([16, 32, 64, 128, 256, 512]))
+                H = W = int(rng.choice([7, 8, 14, 16, 28, 32, 56]))
+                kh = kw = int(rng.choice([1, 3, 3, 3, 5]))
+                ph = pw = kh // 2 if rng.random() < 0.85 else 0
+                sh = sw = int(rng.choice([1, 1, 1, 2]))
+            if H + 2 * ph < kh or W + 2 * pw < kw:
+                continue
+            Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+            if 1.0 * N * Cout * Ho * Wo * Cin * kh * kw <= 1e9 and N * Cin * H * W <= 4e6 and N * Cout * Ho * Wo <= 4e6:
+                break
+        geo = (N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw)
+        x = rng.integers(0, 256, (N, Cin, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (Cout, Cin, kh, kw), dtype=np.uint8)
+        zp = rng.integers(0, 256, 3).astype(np.uint8)
+        if rng.random() < 0.3:
+            zp[:] = 128
+        if rng.random() < 0.2:
+            zp[0] = 0
+        sc = [0.02, 0.01, 0.02 * 0.01 * float(np.sqrt(Cin * kh * kw)) * 40]
+        bias = rng.integers(-9999, 9999, Ho * Wo).astype(np.int32) if rng.random() < 0.5 else None
+        want_y, want_acc = ob.conv2dq_forward(geo, x, w, sc, zp, bias=bias)
+        y, acc = gpu.conv2dq_host(geo, x, w, sc, zp, bias=bias, want_acc=True)
+        case = (seed, it, geo, zp.tolist(), bias is not None, gpu.last_kernel())
+        assert np.array_equal(acc, want_acc), case
+        assert np.array_equal(y, want_y), case
