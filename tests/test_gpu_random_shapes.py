@@ -209,3 +209,46 @@ def test_conv2dq_random_geometries_bit_exact(gpu, ob, seed):
         case = (seed, it, geo, zp.tolist(), bias is not None, gpu.last_kernel())
         assert np.array_equal(acc, want_acc), case
         assert np.array_equal(y, want_y), case
+
+
+@pytest.mark.parametrize("seed", [51, 52])
+def test_fc_backward_random_shapes_exact(gpu, seed):
+    """FullyConnected backward (dX = dY W, dW = dY^T X, db += column sums of dY), plain and with the relu's backward pass folded
+    in, over random batch sizes and layer widths (the paired launch, the weight-streaming kernels, split reductions, rank-1
+    updates at batch 1); any of the three outputs may be left out."""
+    rng = np.random.default_rng(seed)
+    D, l = gpu.DeviceBuffer, gpu.lib()
+    Ms = [1, 2, 3, 4, 8, 15, 16, 17, 32, 33, 64, 100, 128, 256, 257, 512, 1000, 2048, 4096, 16384]
+    widths = [1, 2, 5, 10, 16, 50, 64, 100, 128, 250, 256, 500, 512, 784, 1000, 1024, 2048, 4096, 5760, 8192, 25088, 32000]
+    if seed % 2 == 0:
+        widths = [w for w in widths if w % 4 == 0]
+    for it in range(70):
+        while True:
+            M, n_in, n_out = int(rng.choice(Ms)), int(rng.choice(widths)), int(rng.choice(widths))
+            if max(M * n_in, M * n_out, n_in * n_out) <= 2e7 and M * n_in * n_out <= 1.5e9:
+                break
+        X = rng.integers(-3, 4, (M, n_in)).astype(np.float32)
+        W = rng.integers(-3, 4, (n_out, n_in)).astype(np.float32)
+        dY = rng.integers(-3, 4, (M, n_out)).astype(np.float32)
+        db0 = rng.integers(-9, 10, n_out).astype(np.float32)
+        relu_in = rng.integers(-2, 3, (M, n_in)).astype(np.float32) if rng.random() < 0.4 else None
+        want_dx = (dY.astype(np.float64) @ W.astype(np.float64)).astype(np.float32)
+        if relu_in is not None:
+            want_dx = np.where(relu_in > 0, want_dx, np.float32(0.0))
+        want_dw = (dY.astype(np.float64).T @ X.astype(np.float64)).astype(np.float32)
+        want_db = (db0 + dY.astype(np.float64).sum(axis=0)).astype(np.float32)
+        wants = [rng.random() < 0.85 for _ in range(3)]
+        dXb, dWb, dDY, dR = D.from_numpy(X), D.from_numpy(W), D.from_numpy(dY), D.from_numpy(relu_in) if relu_in is not None else None
+        dDX, dDW, dDB = D(X.nbytes) if wants[0] else None, D(W.nbytes) if wants[1] else None, D.from_numpy(db0) if wants[2] else None
+        args = (dDX.ptr if dDX else None, dDW.ptr if dDW else None, dDB.ptr if dDB else None)
+        if relu_in is None:
+            gpu.check(l.lten_hip_fc_backward_f32(M, n_in, n_out, dXb.ptr, dWb.ptr, dDY.ptr, *args))
+        else:
+            gpu.check(l.lten_hip_fc_backward_relu_f32(M, n_in, n_out, dXb.ptr, dWb.ptr, dDY.ptr, dR.ptr, *args))
+        case = (seed, it, M, n_in, n_out, relu_in is not None, wants, gpu.last_kernel())
+        if dDX:
+            assert np.array_equal(dDX.numpy(np.float32, X.shape), want_dx), ("dX", case)
+        if dDW:
+            assert np.array_equal(dDW.numpy(np.float32, W.shape), want_dw), ("dW", case)
+        if dDB:
+            assert np.array_equal(dDB.numpy(np.float32, (n_out,)), want_db), ("db", case)
