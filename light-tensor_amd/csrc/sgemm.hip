@@ -701,6 +701,10 @@ template <int MB>
 __global__ __launch_bounds__(512) void sgemm_skinny_nt_kernel(SProblem p)
 {
 	__shared__ __attribute__((aligned(16))) float lds[SkinnyShape<MB, true>::LDS_FLOATS];
+	// (grid plane z: problem z of a strided batch)
+	p.A += (int64_t)blockIdx.z * p.stride_a;
+	p.B += (int64_t)blockIdx.z * p.stride_b;
+	p.C += (int64_t)blockIdx.z * p.stride_c;
 	sgemm_skinny_body<MB, true>(p, blockIdx.x, blockIdx.y, lds);
 }
 
@@ -974,8 +978,26 @@ __global__ __launch_bounds__(256) void sgemm_add_partials_kernel(const float* __
 {
 	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x, count = (int64_t)M * N;
 	if (idx >= count) return;
+	// (the loads of 16 slices in flight at a time: one load per addition took 64 memory latencies for 64 slices, 15 us for a
+	// 16 x 128 output)
 	float sum = 0.0f;
-	for (int s = 0; s < parts; s++) sum += partial[(int64_t)s * count + idx];
+	int s = 0;
+	for (; s + 16 <= parts; s += 16) {
+		float v[16];
+#pragma unroll
+		for (int j = 0; j < 16; j++) v[j] = partial[(int64_t)(s + j) * count + idx];
+#pragma unroll
+		for (int j = 0; j < 16; j++) sum += v[j];
+	}
+	if (s + 8 <= parts) {
+		float v[8];
+#pragma unroll
+		for (int j = 0; j < 8; j++) v[j] = partial[(int64_t)(s + j) * count + idx];
+#pragma unroll
+		for (int j = 0; j < 8; j++) sum += v[j];
+		s += 8;
+	}
+	for (; s < parts; s++) sum += partial[(int64_t)s * count + idx];
 	const int64_t n = idx % N;
 	float* c = C + (idx / N) * ldc + n;
 	const float v = beta == 0.0f ? alpha * sum : alpha * sum + beta * *c;
@@ -1052,7 +1074,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// and a K of 8192 on the split is ahead of them: 384 x 384 x 16384 NT 97 -> 55 us, 128 x 256 x 8192 31 -> 20 us.)
 	// (the NN streaming kernel wants more than 16 rows, a single row has the row-vector kernel: 2 to 16 rows against a long K
 	// had neither and walked K on 32 workgroups, 4 x 1024 x 32000 in 202 us)
-	const bool few_columns = K >= 8192 && ceil_div(N, 16) * ceil_div(M, 32) < 128;  // (their workgroups, one per 16 columns, leave half of the CUs idle)
+	// (up to 16 rows from K = 3072 on: the slices then run as a batch on the same streaming kernel, 1 x 4096 -> 1000 10.2 -> 6.6 us)
+	const bool few_columns = K >= (M <= 16 ? 3072 : 8192) && ceil_div(N, 16) * ceil_div(M, 32) < 128;  // (their workgroups, one per 16 columns, leave half of the CUs idle)
 	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0 && !few_columns) || (!tA && !tB && N >= 512 && (M == 1 || M > 16)));
 	const bool small_out = !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256;
 	// The same for outputs of 65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: the direct-to-LDS tiles run at
@@ -1068,7 +1091,14 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		uint64_t slices;
 		if (small_out) {
 			slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
-			while (slices > 2 && K / slices < 512) slices /= 2;
+			slices = std::max<uint64_t>(2, std::min<uint64_t>(slices, K / 512));  // (slices of 512 or more)
+			// (a count that divides K's steps of 32, if one is near: what the slices leave over costs a launch of its own,
+			// 7 of the 26 us of 384 x 48 x 8192 in ten slices of 800)
+			for (uint64_t s = slices; s > slices / 2 + 1 && s > 2; s--)
+				if ((K / 32) % s == 0) {
+					slices = s;
+					break;
+				}
 		} else {
 			slices = 2;
 			while (tiles64_all * slices < 512 && slices < 16 && K / (slices * 2) >= 1024) slices *= 2;
@@ -1118,13 +1148,16 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// that gives at most a few workgroups per CU: 128 rows against a 1024-wide layer are 256 tiles of 32 x 16 where the
 	// 32 x 32 tiles of the general small-GEMM kernels would occupy half of the CUs.
 	// A classifier head (a few output columns) takes the same kernel: one column block, K cut over eight wavefronts.
-	if (force == 0 && !tA && tB && K >= 256 && K % 4 == 0 && batch == 1 && operands_vec(p) &&
+	// (a strided batch of such products with at most 16 rows each, the slices of a split reduction among them, runs on
+	// the grid's planes)
+	const bool skinny_batch = batch > 1 && batch < 65536 && M <= 16 && bias == nullptr && stride_c != 0 && stride_a % 4 == 0 && stride_b % 4 == 0;
+	if (force == 0 && !tA && tB && K >= 256 && K % 4 == 0 && (batch == 1 || skinny_batch) && operands_vec(p) &&
 	    (M <= 32 || ceil_div(M, 32) * ceil_div(N, 16) <= 1024)) {
 		// few column blocks (a classifier head): blocks of 16 rows, twice the workgroups
 		const bool rows16 = M <= 16 || ceil_div(N, 16) * ceil_div(M, 32) < 64;
 		set_kernel_name(rows16 ? "sgemm_skinny_nt_16x16" : "sgemm_skinny_nt_32x16");
 		if (want_relu) { p.relu_out = relu_out; p.relu_in = relu_in; *relu_done = true; }
-		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(rows16 ? ceil_div(M, 16) : ceil_div(M, 32)));
+		const dim3 grid((unsigned)ceil_div(N, 16), (unsigned)(rows16 ? ceil_div(M, 16) : ceil_div(M, 32)), (unsigned)batch);
 		if (rows16) sgemm_skinny_nt_kernel<1><<<grid, dim3(512), 0, stream()>>>(p);
 		else sgemm_skinny_nt_kernel<2><<<grid, dim3(512), 0, stream()>>>(p);
 		LTEN_HIP_LAUNCH_CHECK();

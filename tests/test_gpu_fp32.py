@@ -382,6 +382,22 @@ def test_stack_of_products_over_a_short_reduction(gpu, batch, M, N, K, tile, lay
     assert np.array_equal(dC.numpy(np.float32, c0.shape), want.astype(np.float32))
 
 
+@pytest.mark.parametrize("batch,M,N,K", [(5, 7, 100, 1028), (64, 16, 128, 512), (300, 1, 33, 260)])
+def test_stack_of_few_row_products_against_transposed_matrices(gpu, batch, M, N, K):
+    """A strided batch of NT products with at most 16 rows each (the slices of a split reduction are one): the weight-streaming
+    kernel with one grid plane per problem.  Integer-valued operands, exact; alpha and beta as everywhere."""
+    rng = np.random.default_rng(batch + M + N + K)
+    a = rng.integers(-4, 5, (batch, M, K)).astype(np.float32)
+    b = rng.integers(-4, 5, (batch, N, K)).astype(np.float32)
+    c0 = rng.integers(-9, 10, (batch, M, N)).astype(np.float32)
+    want = (0.5 * (a.astype(np.float64) @ b.astype(np.float64).transpose(0, 2, 1)) + 2.0 * c0).astype(np.float32)
+    D = gpu.DeviceBuffer
+    dA, dB, dC = D.from_numpy(a), D.from_numpy(b), D.from_numpy(c0)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(0, 1, M, N, K, 0.5, dA.ptr, K, M * K, dB.ptr, K, N * K, 2.0, dC.ptr, N, M * N, batch))
+    assert gpu.last_kernel() == "sgemm_skinny_nt_16x16", gpu.last_kernel()
+    assert np.array_equal(dC.numpy(np.float32, c0.shape), want)
+
+
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     cases = []
