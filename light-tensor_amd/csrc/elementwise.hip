@@ -421,8 +421,17 @@ __global__ __launch_bounds__(256) void channel_sum_final_kernel(const float* __r
 {
 	const int c = blockIdx.x * 256 + threadIdx.x;
 	if (c >= C) return;
+	// (eight loads in flight at a time, the additions in slice order)
 	float sum = 0.0f;
-	for (int s = 0; s < slices; s++) sum += partial[c * slices + s];
+	int s = 0;
+	for (; s + 8 <= slices; s += 8) {
+		float v[8];
+#pragma unroll
+		for (int j = 0; j < 8; j++) v[j] = partial[c * slices + s + j];
+#pragma unroll
+		for (int j = 0; j < 8; j++) sum += v[j];
+	}
+	for (; s < slices; s++) sum += partial[c * slices + s];
 	db[c] = accumulate ? db[c] + sum : sum;
 }
 

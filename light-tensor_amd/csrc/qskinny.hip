@@ -258,8 +258,15 @@ __global__ __launch_bounds__(256) void qskinny_sum_chunks_kernel(const int32_t* 
 {
 	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
 	if (idx >= count) return;
-	int v = 0;
-	for (int c = 0; c < chunks; c++) v += acc[(int64_t)c * count + idx];
+	// (four loads in flight at a time)
+	int v = 0, c = 0;
+	for (; c + 4 <= chunks; c += 4) {
+		int t[4];
+#pragma unroll
+		for (int j = 0; j < 4; j++) t[j] = acc[(int64_t)(c + j) * count + idx];
+		v += (t[0] + t[1]) + (t[2] + t[3]);
+	}
+	for (; c < chunks; c++) v += acc[(int64_t)c * count + idx];
 	if (OUT == Q_OUT_ACC) static_cast<int*>(out)[idx] = v;
 	else static_cast<uint8_t*>(out)[idx] = (uint8_t)requant<OUT>(v, mult, zp_c);
 }
