@@ -1085,6 +1085,17 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	const uint64_t tiles64_all = ceil_div(M, 64) * ceil_div(N, 64);
 	const bool mid_out = M >= 128 && N >= 128 && tiles64_all > 64 && tiles64_all < 256 && K >= 4096 && lda % 4 == 0 && ldb % 4 == 0 &&
 	                     ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 && (tA ? M % 4 == 0 : true) && (tB ? true : N % 4 == 0);
+	// A small stack of such products (matmul's gradient for a stack of tall matrices: 2 x (32 x 512 x 25088) TN took 174 us as
+	// one batch of K-walking workgroups): one after the other, each split, 46 us; 8 x (16 x 16 x 65536) 442 -> 102 us.  With
+	// more than 64 tiles of 32 x 32 in the stack, or a shorter K, the one batch is ahead (8 x (128 x 128 x 8192): 64 against 89 us).
+	if (get_option(OPT_SGEMM_TILE) == 0 && batch > 1 && batch <= 8 && stride_c != 0 && bias == nullptr && K >= 8192 && small_out &&
+	    ceil_div(M, 32) * ceil_div(N, 32) * batch <= 64) {
+		for (uint64_t b = 0; b < batch; b++)
+			if (int rc = sgemm_run(tA, tB, M, N, K, alpha, A + (int64_t)b * stride_a, lda, 0, B + (int64_t)b * stride_b, ldb, 0, beta, C + (int64_t)b * stride_c, ldc, 0, 1,
+			                       nullptr, nullptr, nullptr))
+				return rc;
+		return 0;
+	}
 	// (a bias per column, FullyConnected's, rides on the launch that adds the slices)
 	if (get_option(OPT_SGEMM_TILE) == 0 && batch == 1 && (small_out || mid_out)) {
 		const uint64_t tiles32 = ceil_div(M, 32) * ceil_div(N, 32);

@@ -398,6 +398,26 @@ def test_stack_of_few_row_products_against_transposed_matrices(gpu, batch, M, N,
     assert np.array_equal(dC.numpy(np.float32, c0.shape), want)
 
 
+@pytest.mark.parametrize("tA,tB", [(1, 0), (0, 0)])
+def test_small_stack_of_long_reductions_is_split_one_by_one(gpu, tA, tB):
+    """matmul's gradient for a stack of tall matrices: a few products with a small output each under a reduction of 8192 or more
+    run one after the other, each cut into slices; integer-valued operands, exact, C's padding untouched."""
+    batch, M, N, K = 3, 40, 72, 8192 + 96
+    rng = np.random.default_rng(5 + tA)
+    a = rng.integers(-3, 4, (batch, M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, (batch, K, N)).astype(np.float32)
+    c0 = rng.integers(-9, 10, (batch, M, N + 4)).astype(np.float32)
+    want = (2.0 * (a.astype(np.float64) @ b.astype(np.float64)) - c0[:, :, :N]).astype(np.float32)
+    D = gpu.DeviceBuffer
+    dA, dB, dC = D.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1)) if tA else a), D.from_numpy(b), D.from_numpy(c0)
+    gpu.check(gpu.lib().lten_hip_sgemm_strided_batched(tA, tB, M, N, K, 2.0, dA.ptr, M if tA else K, M * K, dB.ptr, N, K * N, -1.0, dC.ptr, N + 4,
+                                                       M * (N + 4), batch))
+    assert gpu.last_kernel() == "sgemm_split_k", gpu.last_kernel()
+    got = dC.numpy(np.float32, c0.shape)
+    assert np.array_equal(got[:, :, :N], want)
+    assert np.array_equal(got[:, :, N:], c0[:, :, N:])
+
+
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
     g = np.load(golden_path("layer_cases.npz"))
     cases = []
