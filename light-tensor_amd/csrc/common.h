@@ -35,11 +35,18 @@ struct RowsReadableToPitch {
 	~RowsReadableToPitch();
 };
 bool rows_readable_to_pitch();
-// For a caller that keeps data in the first `bytes` of the block across a call into another entry point of the library:
-// while one of these lives, library_scratch hands out only what the block has behind those bytes and never moves it.
+// For a caller that keeps data in the first `bytes` of what library_scratch handed it across a call into another entry
+// point of the library: while one of these lives, library_scratch hands out only what the block has behind those bytes
+// and never moves it.  They nest: a callee that was itself handed the part behind a holder's bytes holds from there on.
 struct LibraryScratchHold {
 	explicit LibraryScratchHold(uint64_t bytes);
 	~LibraryScratchHold();
+	LibraryScratchHold(const LibraryScratchHold&) = delete;
+	LibraryScratchHold& operator=(const LibraryScratchHold&) = delete;
+
+private:
+	bool outer_held_;
+	uint64_t outer_bytes_;
 };
 
 // Looks up the current device's copy of the static scratch of lten_hip_fcq_forward_static (qgemm.hip); 0 on success.

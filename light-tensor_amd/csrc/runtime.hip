@@ -57,12 +57,16 @@ bool rows_readable_to_pitch() { return g_rows_readable > 0; }
 
 static bool g_scratch_held = false;
 static uint64_t g_scratch_held_bytes = 0;
-LibraryScratchHold::LibraryScratchHold(uint64_t bytes)
+LibraryScratchHold::LibraryScratchHold(uint64_t bytes) : outer_held_(g_scratch_held), outer_bytes_(g_scratch_held_bytes)
 {
+	g_scratch_held_bytes = (outer_held_ ? outer_bytes_ : 0) + ((bytes + 255) & ~255ull);
 	g_scratch_held = true;
-	g_scratch_held_bytes = (bytes + 255) & ~255ull;
 }
-LibraryScratchHold::~LibraryScratchHold() { g_scratch_held = false; }
+LibraryScratchHold::~LibraryScratchHold()
+{
+	g_scratch_held = outer_held_;
+	g_scratch_held_bytes = outer_bytes_;
+}
 
 void* library_scratch(uint64_t bytes)
 {

@@ -1102,7 +1102,9 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		uint64_t slices;
 		if (small_out) {
 			slices = std::min<uint64_t>(64, std::max<uint64_t>(2, 1024 / tiles32));  // (more slices were no faster: 64 x 64 x 65536 36 us with 64, 51 us with 128)
-			slices = std::max<uint64_t>(2, std::min<uint64_t>(slices, K / 512));  // (slices of 512 or more)
+			// (slices of 512 or more; of 256 or more from K = 4096 on, where the slices then fill the direct-to-LDS 64 x 64 tiles:
+			// 192 x 192 x 6144 in 12 slices 18.4 us, in 24 12.5; 128 x 128 x 16384 in 32 15.8, in 64 13.4; 1000 x 48 x 4096 14.4 -> 11.2)
+			slices = std::max<uint64_t>(2, std::min<uint64_t>(slices, K / (K >= 4096 ? 256 : 512)));
 			// (a count that divides K's steps of 32, if one is near: what the slices leave over costs a launch of its own,
 			// 7 of the 26 us of 384 x 48 x 8192 in ten slices of 800)
 			for (uint64_t s = slices; s > slices / 2 + 1 && s > 2; s--)
@@ -1117,6 +1119,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 		const uint64_t kc = (K / slices) & ~31ull, rest = K - slices * kc, parts = slices + (rest != 0 ? 1 : 0);
 		float* partial = kc >= 256 ? static_cast<float*>(library_scratch(parts * M * N * sizeof(float))) : nullptr;
 		if (partial != nullptr) {
+			// (what the slices leave over can be long enough to be split itself: its partial matrices go behind these)
+			LibraryScratchHold hold(parts * M * N * sizeof(float));
 			int rc = sgemm_run(tA, tB, M, N, kc, 1.0f, A, lda, (int64_t)(tA ? kc * lda : kc), B, ldb, (int64_t)(tB ? kc : kc * ldb), 0.0f, partial, N,
 			                   (int64_t)(M * N), slices, nullptr, nullptr, nullptr);
 			if (rc) return rc;

@@ -55,7 +55,8 @@ def test_integer_valued_exact_with_leading_dims(gpu, tile, tA, tB):
 
 
 @pytest.mark.parametrize("tA,tB,M,N,K", [(1, 0, 128, 128, 16384), (1, 0, 10, 32, 20011), (0, 0, 64, 200, 8200), (0, 1, 100, 37, 4099 + 2),
-                                          (1, 1, 256, 256, 4096), (1, 0, 64, 64, 65536)])
+                                          (1, 1, 256, 256, 4096), (1, 0, 64, 64, 65536),
+                                          (1, 0, 16, 16, 34815), (1, 0, 10, 32, 100000)])   # 64 slices of 512 leave 2047, which is split itself: its partial sums must not land on the first split's
 def test_long_reduction_into_a_small_output_is_split(gpu, tA, tB, M, N, K):
     """The weight gradient of a small layer over a large batch: K is cut into slices that run as a batch into partial
     matrices, added in slice order by a second launch.  Integer-valued operands come out exactly whatever the order;
