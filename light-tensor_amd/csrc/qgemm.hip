@@ -511,6 +511,8 @@ static int qgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, const u
 				qgemm_transpose_rows_kernel<<<dim3((unsigned)ceil_div(N, 64), (unsigned)(Kp / 64 + (Kp % 64 != 0))), dim3(256), 0, stream()>>>(B, b2, (int)N, (int)K, (int)Kp);
 				LTEN_HIP_LAUNCH_CHECK();
 			}
+			// (a kernel choice that takes library memory of its own, the K-chunks of the streaming kernel, gets it behind the copies)
+			LibraryScratchHold copies(bytes_a + bytes_b);
 			return qgemm_run(0, 1, M, N, Kp, copy_a ? a2 : A, copy_b ? b2 : B, C, out_acc, qp, bias, workspace, weights_prepared, nullptr, weight_sums,
 			                 (int)(Kp - K));
 		}

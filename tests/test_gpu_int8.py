@@ -370,6 +370,27 @@ def test_few_rows_against_a_reduction_beyond_16384(gpu, ob, M, N, K):
     run_case(gpu, ob, A, B, [0.5, 0.5, 0.2], np.array([128, 0, 9], np.uint8))
 
 
+@pytest.mark.parametrize("M,N,K", [(16, 8192, 16392), (3, 600, 20003)])
+def test_long_reduction_that_is_no_multiple_of_16_keeps_its_padded_copies(gpu, ob, M, N, K):
+    """in_features beyond 16384 and no multiple of 16: the operands are first copied into padded rows in memory the library
+    owns, and the K-chunks of the streaming kernel then take their int32 sums from the same block: behind the copies, not
+    on top of them.  Also with both operands transposed (copies of both).  Bit-exact against the closed form."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    zp, sc = np.array([3, 250, 77], np.uint8), [0.02, 0.013, 3.0]
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    want = requant_numpy(exact_acc(A, B, zp[0], zp[1]) + bias[None, :], mult, zp[2])
+    got, k0 = fcq(gpu, gpu.lib().lten_hip_fcq_forward, A, B, sc, zp, bias)
+    assert k0 == "qskinny_mfma_kchunks", k0
+    assert np.array_equal(got, want)
+    if N <= 1024:
+        got_t, _ = gpu.qgemm_host(np.ascontiguousarray(A.T), np.ascontiguousarray(B.T), sc, zp, tA=True, tB=False, bias=bias, M=M, N=N, K=K)
+        assert gpu.last_kernel() == "qskinny_mfma_kchunks", gpu.last_kernel()
+        assert np.array_equal(got_t, want)
+
+
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
     """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
