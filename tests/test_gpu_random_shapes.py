@@ -9,8 +9,8 @@ from conftest import exact_acc, requant_numpy
 pytestmark = pytest.mark.gpu
 
 DIMS = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 96, 100, 127, 128, 129, 192, 196, 200, 255, 256, 257, 320, 384, 500, 512, 513,
-        640, 768, 1000, 1024, 1025, 1536, 2048, 2304, 3000, 4096, 4100, 6272, 8192, 8200, 12288, 16384, 20000, 25088, 32000]
-DIMS_ALIGNED = [d for d in DIMS if d % 4 == 0] + [12, 20, 160, 1280, 3072]
+        640, 768, 1000, 1024, 1025, 1536, 2048, 2304, 3000, 4096, 4100, 6272, 8192, 8200, 12288, 16384, 20000, 20011, 25088, 32000, 34815, 100000]
+DIMS_ALIGNED = [d for d in DIMS if d % 4 == 0] + [12, 20, 160, 1280, 3072, 34812, 65536 + 2044]
 
 
 @pytest.mark.parametrize("seed", [11, 12, 13, 14])
@@ -69,7 +69,7 @@ def test_fcq_random_shapes_bit_exact(gpu, seed):
     rng = np.random.default_rng(seed)
     Ms = [1, 2, 3, 4, 7, 8, 15, 16, 17, 24, 31, 32, 33, 48, 63, 64, 65, 100, 127, 128, 129, 192, 255, 256, 257, 384, 500, 512, 1000, 1024, 2048]
     Ns = [1, 2, 5, 10, 16, 17, 50, 64, 100, 128, 250, 256, 500, 512, 1000, 1001, 1024, 2000, 2048, 4096]
-    Ks = [1, 3, 16, 33, 64, 100, 127, 128, 256, 300, 512, 784, 1000, 1024, 2048, 4000, 4096, 5760, 8192, 9216, 12288, 16384, 16400, 25088, 32768]
+    Ks = [1, 3, 16, 33, 64, 100, 127, 128, 256, 300, 512, 784, 1000, 1024, 2048, 4000, 4096, 5760, 8192, 9216, 12288, 16384, 16392, 16400, 20003, 25088, 32768]
     D, l = gpu.DeviceBuffer, gpu.lib()
     for it in range(120):
         while True:
