@@ -325,7 +325,9 @@ static int qgemm_dispatch(const QProblem& p, int out, const SplitScratch* scratc
 		// workgroups, two per CU) below that.
 		// (a shorter K only with many tiles: the positions x channels products of a quantized convolution, 16384 x 64 x
 		// 288: 5.6 against 7.8 us on the guarded kernel)
-		if (p.K >= 512 || (p.K >= 128 && ceil_div(p.M, 128) * ceil_div(p.N, 128) >= 64)) {
+		// (down to K = 32, one partial k-step: 2048 x 8192 x 64 took 42 us on the register-staged 256 x 256 tiles, 10 us here;
+		// 4096 x 4096 x 96 53 -> 9.5 us)
+		if (p.K >= 512 || (p.K >= 32 && ceil_div(p.M, 128) * ceil_div(p.N, 128) >= 64)) {
 			// 256 x 256 tiles only where both dimensions fill most of one (100352 x 64 x 576: 20.7 us on 128 x 128 tiles, 26.5 on these)
 			if (p.M >= 192 && p.N >= 192 && ceil_div(p.M, 256) * ceil_div(p.N, 256) > 160 && qgemm_fast_dispatch(p, out, 33) == 0) return 0;
 			// about one 256 x 128 tile per CU: less operand traffic per MFMA than two 128 x 128 tiles per CU

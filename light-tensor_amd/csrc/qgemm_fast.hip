@@ -710,8 +710,8 @@ static int launch_tile128(const QProblem& p, int out, bool ktail, bool wpre)
 int qgemm_fast_dispatch(const QProblem& p, int out, int variant)
 {
 	// preconditions of the direct-to-LDS tiles; the caller falls back to the general kernels otherwise
-	// K: any multiple of 16 at least one k-step long (variants 33, 41 and 51), or a multiple of the k-step
-	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.K >= 128 &&
+	// K: any multiple of 16 from 32 on (variants 33, 41 and 51; a K below the k-step is one partial step), or a multiple of the k-step
+	const bool fits = p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.K >= 32 &&
 	                  (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32) &&
 	                  (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                  (p.cterm == nullptr || (reinterpret_cast<uintptr_t>(p.cterm) & 15) == 0) &&

@@ -391,6 +391,30 @@ def test_long_reduction_that_is_no_multiple_of_16_keeps_its_padded_copies(gpu, o
         assert np.array_equal(got_t, want)
 
 
+@pytest.mark.parametrize("M,N,K", [(2048, 8192, 64), (2048, 2048, 32), (2048, 4096, 48), (1000, 8190, 80), (2048, 4096, 112)])
+def test_reduction_shorter_than_a_k_step_on_the_direct_to_lds_tiles(gpu, ob, M, N, K):
+    """in_features of 32 to 112 against an output of 64 tiles or more: one partial k-step of the direct-to-LDS tiles (the
+    activation tile padded with the zero point's image, whatever the weight tile holds there multiplied by zero).  l-ten's
+    uint8 weights and prepared weights, with and without zero-point terms and bias, int32 accumulators and uint8 outputs."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    for zp, b in (([128, 128, 128], None), ([0, 128, 3], bias), ([17, 250, 100], bias)):
+        zp, sc = np.array(zp, np.uint8), [0.02, 0.013, 0.9]
+        acc = exact_acc(A, B, zp[0], zp[1]) + (b[None, :] if b is not None else 0)
+        mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+        want = requant_numpy(acc, mult, zp[2])
+        got, k0 = fcq(gpu, gpu.lib().lten_hip_fcq_forward, A, B, sc, zp, b)
+        assert k0.startswith("qgemm_fast_") and "ktail" in k0, k0
+        assert np.array_equal(got, want), (zp.tolist(), k0)
+        got, k1 = fcq(gpu, gpu.lib().lten_hip_fcq_forward_prepared, A, B, sc, zp, b, prepared=True)
+        assert k1.startswith("qgemm_fast_") and "ktail" in k1, k1
+        assert np.array_equal(got, want), (zp.tolist(), k1)
+        _, accg = gpu.qgemm_host(A, B, sc, zp, bias=b, want_acc=True)
+        assert np.array_equal(accg, acc)
+
+
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
     """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
