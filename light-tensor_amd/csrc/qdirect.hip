@@ -99,7 +99,7 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 	if (!(p.a_ks == 1 && p.b_ks == 1 && p.vec_ok && p.K % 16 == 0 && p.M >= 1 && p.N >= 1 && p.K >= 1)) return -1;
 	const int64_t tiles = (int64_t)ceil_div((uint64_t)p.M, 16) * ceil_div((uint64_t)p.N, 16);
 	// Up to 8192 tiles, as long as this kernel is ahead of the 128 x 128 direct-to-LDS tiles where those apply (at least
-	// 128 output columns, K >= 512 or at least 64 such tiles: qgemm_dispatch).  It takes about 2.3 us + 4.1 us per million
+	// 64 output columns, K >= 512 or at least 64 such tiles: qgemm_dispatch).  It takes about 2.3 us + 4.1 us per million
 	// (tiles x K), they about 5.4 us + 0.33 us per k-step of 128 bytes of a workgroup's share of K while they run in one
 	// round, 4 us more when workgroups share tiles (split K, as qgemm_dispatch picks it), 2 us more when N is no multiple
 	// of 4 (rows of the output that start on any byte), 2.5 us more with a partial last k-step.  300 x 1000 x 512: 4.8 us here, 6.9 there; 400 x 400 x 2048: 7.7
@@ -109,7 +109,9 @@ int qdirect_dispatch(const QProblem& p, int out, const int32_t* bias, int zp_a, 
 	// batch: 22.5 us).
 	if (tiles > 8192 || p.K > 16384) return -1;
 	const uint64_t tiles128 = ceil_div((uint64_t)p.M, 128) * ceil_div((uint64_t)p.N, 128);
-	const bool tiles_apply = p.N >= 128 && (p.K >= 512 || (p.K >= 128 && tiles128 >= 64)) && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
+	// (from 64 output columns on: half-empty 128-column tiles still beat this kernel on long or many rows, 4096 x 100 x 9216 58 -> 25
+	// us, 16384 x 64 x 1024 17 -> 7.5 us; at 50 columns, l-ten's layer above, they are level)
+	const bool tiles_apply = p.N >= 64 && (p.K >= 512 || (p.K >= 32 && tiles128 >= 64)) && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0 &&
 	                         (uint64_t)p.M * p.K < (1ull << 32) && (uint64_t)p.N * p.K < (1ull << 32);
 	if (tiles_apply) {
 		const int splits = (tiles128 <= 64 && p.K >= 8192) ? (tiles128 <= 32 ? 4 : 2) : (tiles128 <= 32 && p.K >= 4096) ? 2 : 1;

@@ -415,6 +415,25 @@ def test_reduction_shorter_than_a_k_step_on_the_direct_to_lds_tiles(gpu, ob, M, 
         assert np.array_equal(accg, acc)
 
 
+@pytest.mark.parametrize("M,N,K", [(4096, 100, 9216), (8192, 66, 1024)])
+def test_many_rows_onto_64_to_127_outputs_take_the_128_column_tiles(gpu, ob, M, N, K):
+    """A layer of 64 to 127 outputs at a large batch: half-empty 128-column tiles (split over K where the tiles are few) are
+    ahead of the 16 x 16 kernel; bit-exact on raw and prepared weights with zero points and bias."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(0, 256, (M, K), dtype=np.uint8)
+    B = rng.integers(0, 256, (N, K), dtype=np.uint8)
+    bias = rng.integers(-5000, 5000, N).astype(np.int32)
+    zp, sc = np.array([17, 250, 100], np.uint8), [0.02, 0.013, 2.0]
+    mult = np.float32(np.float32(sc[0]) * np.float32(sc[1])) / np.float32(sc[2])
+    want = requant_numpy(exact_acc(A, B, zp[0], zp[1]) + bias[None, :], mult, zp[2])
+    got, k0 = fcq(gpu, gpu.lib().lten_hip_fcq_forward, A, B, sc, zp, bias)
+    assert k0.startswith("qgemm_fast_128x128"), k0
+    assert np.array_equal(got, want)
+    got, k1 = fcq(gpu, gpu.lib().lten_hip_fcq_forward_prepared, A, B, sc, zp, bias, prepared=True)
+    assert k1.startswith("qgemm_fast_128x128"), k1
+    assert np.array_equal(got, want)
+
+
 def test_split_k_is_the_default_for_few_tiles_and_long_k(gpu):
     """256 x 1024 x 4096 (16 tiles): the library splits K in two; the closed form in int64 is the check.  With the
     option at 1 the unsplit tiles run and give the same bytes; a launch recorded into a graph also matches."""
