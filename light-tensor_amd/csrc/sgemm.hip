@@ -1075,8 +1075,8 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// (the NN streaming kernel wants more than 16 rows, a single row has the row-vector kernel: 2 to 16 rows against a long K
 	// had neither and walked K on 32 workgroups, 4 x 1024 x 32000 in 202 us)
 	// (up to 16 rows from K = 3072 on: the slices then run as a batch on the same streaming kernel, 1 x 4096 -> 1000 10.2 -> 6.6 us)
-	const bool few_columns = K >= (M <= 16 ? 3072 : 8192) && ceil_div(N, 16) * ceil_div(M, 32) < 128;  // (their workgroups, one per 16 columns, leave half of the CUs idle)
-	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0 && !few_columns) || (!tA && !tB && N >= 512 && (M == 1 || M > 16)));
+	const bool few_columns = K >= (M <= 16 ? 3072 : 8192) && ceil_div(N, 16) * ceil_div(M, 32) < (M <= 16 ? 128 : 256);  // (their workgroups, one per 16 columns, leave half of the CUs idle)
+	const bool streams = (M < 128 || K < 8192) && ((!tA && tB && K % 4 == 0 && !few_columns) || (!tA && !tB && N >= 512 && (M == 1 || (M > 16 && !few_columns))));
 	const bool small_out = !streams && K >= 1536 && ceil_div(M, 32) * ceil_div(N, 32) <= 256;
 	// The same for outputs of 65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: the direct-to-LDS tiles run at
 	// their rate from about 512 workgroups on, so K is cut until the slices give that many (256 x 2304 x 6272, 144 tiles:
