@@ -896,6 +896,40 @@ __global__ __launch_bounds__(256) void sgemm_rank1_vec4_kernel(SProblem p, int t
 	*c = v;
 }
 
+// C = alpha * A^T B + beta * C over a reduction of 2 to 8 rows (the weight gradient of a layer at a batch that small): a
+// stream over C.  A thread takes four rows by four columns, so B's rows are read once per four rows of C; the products are
+// added in the order of k.  N, ldb and ldc multiples of 4, B and C on 16-byte boundaries.
+__global__ __launch_bounds__(256) void sgemm_tn_few_rows_kernel(SProblem p)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+	const int n4 = p.N / 4, m4 = (p.M + 3) / 4;
+	if (idx >= (int64_t)m4 * n4) return;
+	const int m = (int)(idx / n4) * 4, n = (int)(idx % n4) * 4;
+	float4 s[4];
+#pragma unroll
+	for (int r = 0; r < 4; r++) s[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+	for (int k = 0; k < p.K; k++) {
+		const float4 b = *reinterpret_cast<const float4*>(p.B + (int64_t)k * p.ldb + n);
+		const float* a = p.A + (int64_t)k * p.lda + m;
+#pragma unroll
+		for (int r = 0; r < 4; r++) {
+			const float ar = m + r < p.M ? a[r] : 0.0f;
+			s[r].x += ar * b.x; s[r].y += ar * b.y; s[r].z += ar * b.z; s[r].w += ar * b.w;
+		}
+	}
+#pragma unroll
+	for (int r = 0; r < 4; r++) {
+		if (m + r >= p.M) break;
+		float4* c = reinterpret_cast<float4*>(p.C + (int64_t)(m + r) * p.ldc + n);
+		float4 v = make_float4(p.alpha * s[r].x, p.alpha * s[r].y, p.alpha * s[r].z, p.alpha * s[r].w);
+		if (p.beta != 0.0f) {
+			const float4 o = *c;
+			v.x += p.beta * o.x; v.y += p.beta * o.y; v.z += p.beta * o.z; v.w += p.beta * o.w;
+		}
+		*c = v;
+	}
+}
+
 // M == 1 with B not transposed: c[n] = alpha * sum_k a[k] B[k][n] + beta * c[n] — the column sum that
 // l-ten uses for the bias gradient with a = ones (l-ten/backprop.cpp:2267) and the two products of a GRU time
 // step (l-ten/gru.cpp:267-268).  A workgroup takes COLS columns and cuts K into SLICES slices, one thread per
@@ -1054,6 +1088,19 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 	// 32: 4096 x 25088 x 32) is bound by writing C, which the 32 x 32 kernels below do at 1.5 TB/s (100 000 workgroups of
 	// eight wavefronts for one k-step each); the direct-to-LDS tiles want 64 rows at least, so the operands are copied into
 	// 64 rows, the rest zero, in memory the library owns (7 MB against the 411 MB of C: 279 us before).
+	// (2 to 8 rows: the stream over C below, 4096 x 25088 x 4 at the rate a fill reaches)
+	if (get_option(OPT_SGEMM_TILE) == 0 && tA && !tB && batch == 1 && bias == nullptr && relu_done == nullptr && K >= 2 && K <= 8 && N % 4 == 0 && ldb % 4 == 0 &&
+	    ldc % 4 == 0 && ((reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) & 15) == 0 && M * N >= (1u << 18) && M < (1ull << 31) && N < (1ull << 31)) {
+		SProblem pf = {};
+		pf.A = A; pf.B = B; pf.C = C;
+		pf.lda = (int64_t)lda; pf.ldb = (int64_t)ldb; pf.ldc = (int64_t)ldc;
+		pf.M = (int)M; pf.N = (int)N; pf.K = (int)K;
+		pf.alpha = alpha; pf.beta = beta;
+		set_kernel_name("sgemm_tn_few_rows");
+		sgemm_tn_few_rows_kernel<<<dim3((unsigned)ceil_div(ceil_div(M, 4) * (N / 4), 256)), dim3(256), 0, stream()>>>(pf);
+		LTEN_HIP_LAUNCH_CHECK();
+		return 0;
+	}
 	if (get_option(OPT_SGEMM_TILE) == 0 && tA && !tB && batch == 1 && bias == nullptr && relu_done == nullptr && K >= 2 && K < 64 && M % 4 == 0 && N % 4 == 0 &&
 	    lda % 4 == 0 && ldb % 4 == 0 && ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B)) & 15) == 0 &&
 	    ceil_div(M, 128) * ceil_div(N, 128) >= 512) {

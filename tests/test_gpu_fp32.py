@@ -88,7 +88,7 @@ def test_long_reduction_into_a_small_output_is_split(gpu, tA, tB, M, N, K):
     assert rel_err(r1[:, :N], (a64 @ b64).astype(np.float32)) < TOL
 
 
-@pytest.mark.parametrize("K", [8, 24, 32, 52])
+@pytest.mark.parametrize("K", [12, 24, 32, 52])   # (up to 8 rows: the stream over C, tested below)
 def test_short_reduction_into_a_large_output_on_the_large_tiles(gpu, K):
     """The weight gradient of a wide layer at a small batch, dW = dY^T X with fewer than 64 rows to reduce over and 512 or more
     tiles of 128 x 128 to write: the operands are copied into 64 rows (the rest zero) for the direct-to-LDS tiles.
@@ -417,6 +417,32 @@ def test_small_stack_of_long_reductions_is_split_one_by_one(gpu, tA, tB):
     got = dC.numpy(np.float32, c0.shape)
     assert np.array_equal(got[:, :, :N], want)
     assert np.array_equal(got[:, :, N:], c0[:, :, N:])
+
+
+@pytest.mark.parametrize("M,N,K", [(1027, 512, 2), (640, 1000, 5), (513, 2052, 8)])
+def test_weight_gradient_over_a_batch_of_2_to_8_is_a_stream_over_c(gpu, M, N, K):
+    """A^T B over 2 to 8 rows into a large output (dW of a wide layer at a batch that small): four rows by four columns per
+    thread, the products added in the order of k.  Row counts that are no multiple of four, padded leading dimensions, alpha
+    and beta; integer-valued operands, exact, C's padding untouched."""
+    rng = np.random.default_rng(M + N + K)
+    A = rng.integers(-4, 5, (K, M)).astype(np.float32)
+    B = rng.integers(-4, 5, (K, N)).astype(np.float32)
+    want = (A.astype(np.float64).T @ B.astype(np.float64)).astype(np.float32)
+    lda, ldb, ldc = M + 3, N + 4, N + 8
+    As = np.zeros((K, lda), np.float32)
+    As[:, :M] = A
+    Bs = np.zeros((K, ldb), np.float32)
+    Bs[:, :N] = B
+    C0 = np.full((M, ldc), 7.0, np.float32)
+    got = gpu_sgemm(gpu, 1, 0, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, C0, ldc)
+    assert gpu.last_kernel() == "sgemm_tn_few_rows", gpu.last_kernel()
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, 1, 0, M, N, K, 2.0, As, lda, Bs, ldb, -1.0, got, ldc)
+    assert np.array_equal(got2[:, :N], want)
+    assert (got2[:, N:] == 7.0).all()
+    nan0 = np.full((M, ldc), np.nan, np.float32)
+    assert np.array_equal(gpu_sgemm(gpu, 1, 0, M, N, K, 1.0, As, lda, Bs, ldb, 0.0, nan0, ldc)[:, :N], want)
 
 
 def test_fc_forward_backward_golden_and_lten_vectors(gpu):
