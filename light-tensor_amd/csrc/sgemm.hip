@@ -1050,6 +1050,16 @@ __global__ __launch_bounds__(256) void sgemm_pad_k_rows_kernel(const float* __re
 	reinterpret_cast<float4*>(dst)[idx] = v;
 }
 
+// dst[rows][64]: the first `cols` columns of src's rows (leading dimension ld), zeros behind them
+__global__ __launch_bounds__(256) void sgemm_pad_k_cols_kernel(const float* __restrict__ src, int64_t ld, int64_t rows, int cols, float* __restrict__ dst)
+{
+	const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one element
+	if (idx >= rows * 64) return;
+	const int64_t r = idx >> 6;
+	const int c = (int)(idx & 63);
+	dst[idx] = c < cols ? src[r * ld + c] : 0.0f;
+}
+
 int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, const float* A, uint64_t lda,
               int64_t stride_a, const float* B, uint64_t ldb, int64_t stride_b, float beta, float* C, uint64_t ldc,
               int64_t stride_c, uint64_t batch, const float* bias, float* rowsum, bool* rowsum_done, float* relu_out = nullptr,
@@ -1110,6 +1120,20 @@ int sgemm_run(int tA, int tB, uint64_t M, uint64_t N, uint64_t K, float alpha, c
 			sgemm_pad_k_rows_kernel<<<dim3((unsigned)ceil_div(16 * N, 256)), dim3(256), 0, stream()>>>(B, (int64_t)ldb, (int)K, (int)N, rows64 + 64 * M);
 			LTEN_HIP_LAUNCH_CHECK();
 			return sgemm_run(1, 0, M, N, 64, alpha, rows64, M, 0, rows64 + 64 * M, N, 0, beta, C, ldc, 0, 1, nullptr, nullptr, nullptr);
+		}
+	}
+	// The same for A B and A B^T over 9 to 63 columns of A (a layer of that many inputs or outputs against a large batch: 12288
+	// x 3072 x 48 ran 109 us on the 32 x 32 kernel): operands that are contiguous along K are copied into rows of 64.
+	if (get_option(OPT_SGEMM_TILE) == 0 && !tA && batch == 1 && bias == nullptr && relu_done == nullptr && K > 8 && K < 64 && M > 64 && N > 64 &&
+	    (tB || (N % 4 == 0 && ldb % 4 == 0 && (reinterpret_cast<uintptr_t>(B) & 15) == 0)) && ceil_div(M, 128) * ceil_div(N, 128) >= 512 && M < (1ull << 25) && N < (1ull << 25)) {  // (below 512 tiles the two copies cost what the tiles gain)
+		float* a64 = static_cast<float*>(library_scratch(64 * (M + N) * sizeof(float)));
+		if (a64 != nullptr) {
+			float* b64 = a64 + 64 * M;
+			sgemm_pad_k_cols_kernel<<<dim3((unsigned)ceil_div(64 * M, 256)), dim3(256), 0, stream()>>>(A, (int64_t)lda, (int64_t)M, (int)K, a64);
+			if (tB) sgemm_pad_k_cols_kernel<<<dim3((unsigned)ceil_div(64 * N, 256)), dim3(256), 0, stream()>>>(B, (int64_t)ldb, (int64_t)N, (int)K, b64);
+			else sgemm_pad_k_rows_kernel<<<dim3((unsigned)ceil_div(16 * N, 256)), dim3(256), 0, stream()>>>(B, (int64_t)ldb, (int)K, (int)N, b64);
+			LTEN_HIP_LAUNCH_CHECK();
+			return sgemm_run(0, tB, M, N, 64, alpha, a64, 64, 0, b64, tB ? 64 : N, 0, beta, C, ldc, 0, 1, nullptr, nullptr, nullptr);
 		}
 	}
 	// A long reduction into a small output (the weight gradient of a small layer over a large batch: 128 x 128 x 16384)

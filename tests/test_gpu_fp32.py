@@ -107,6 +107,26 @@ def test_short_reduction_into_a_large_output_on_the_large_tiles(gpu, K):
     assert np.array_equal(got2[:, :N], want)
 
 
+@pytest.mark.parametrize("tB,K", [(0, 12), (0, 50), (1, 9), (1, 33)])
+def test_short_reduction_of_row_major_operands_into_a_large_output(gpu, tB, K):
+    """A B and A B^T over 9 to 63 columns of A into 512 or more tiles of 128 x 128: the operands that are contiguous along K are
+    copied into rows of 64 (zeros behind) for the direct-to-LDS tiles.  Odd row counts and padded leading dimensions;
+    integer-valued operands, exact; alpha and beta."""
+    M, N = 2051, 4100
+    rng = np.random.default_rng(K + tB)
+    A = rng.integers(-4, 5, (M, K + 3)).astype(np.float32)            # leading dimension K + 3
+    B = rng.integers(-4, 5, (N, K + 5) if tB else (K, N + 8)).astype(np.float32)
+    b = B[:, :K].T if tB else B[:, :N]
+    want = (A[:, :K].astype(np.int64) @ b.astype(np.int64)).astype(np.float32)
+    C0 = np.full((M, N + 4), 7.0, np.float32)
+    got = gpu_sgemm(gpu, 0, tB, M, N, K, 1.0, A, K + 3, B, K + 5 if tB else N + 8, 0.0, C0, N + 4)
+    assert gpu.last_kernel().startswith("sgemm_fast_128x128x32"), gpu.last_kernel()
+    assert np.array_equal(got[:, :N], want)
+    assert (got[:, N:] == 7.0).all()
+    got2 = gpu_sgemm(gpu, 0, tB, M, N, K, 2.0, A, K + 3, B, K + 5 if tB else N + 8, -1.0, got, N + 4)
+    assert np.array_equal(got2[:, :N], want)
+
+
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
 def test_long_reduction_into_a_mid_size_output_is_split(gpu, tA, tB):
     """65 to 255 tiles of 64 x 64 under a reduction of 4096 or more: K is cut until the slices give the direct-to-LDS tiles
