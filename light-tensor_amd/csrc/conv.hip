@@ -366,7 +366,10 @@ static int conv_forward_by_columns(const ConvGeo& g, const float* x, const float
 	const uint64_t Kc = (uint64_t)g.Cin * g.kh * g.kw, HW = (uint64_t)g.Ho * g.Wo, N = g.N;
 	const uint64_t pitch = (HW + 3) & ~3ull;  // rows of the column matrices start on 16-byte boundaries
 	const uint64_t elems = N * Kc * pitch;
-	if (!(g.Cout >= 32 && HW >= 32 && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) &&
+	// (few output channels or pixels only under a long reduction, where the implicit GEMM's handful of tiles walk it one after
+	// another: 4 x 256 x 8 x 8 -> 512 channels 5 x 5 at stride 2, 16 pixels an image, took 519 us)
+	const bool long_k = Kc >= 2048 && g.Cout >= 8 && HW >= 4;
+	if (!(((g.Cout >= 32 && HW >= 32) || long_k) && Kc >= 256 && (Kc % 32 == 0 || (Kc % 4 == 0 && Kc >= 512)) && aligned16(w) &&
 	      elems <= (1ull << 27) && (uint64_t)g.Cin * g.H * g.W < (1ull << 30) && N * g.Cout * HW < (1ull << 40))) return -1;
 	// Measured rates, on the work of whole tiles.  The implicit GEMM: 46 TFLOP/s once its 64 x 64 tiles give every CU a
 	// workgroup.  The batch of products: 110 TFLOP/s on the 64 x 64 direct-to-LDS tiles and 92 on the 128 x 128 ones, which
@@ -854,7 +857,7 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		// channels 3 x 3: columns 44, patch kernel 18 us; 64 x 16 x 32 x 32 <- 32: 46 against 30 us, <- 64: 44 against 55 us;
 		// 128 x 3 x 32 x 32 <- 64 channels 5 x 5: 48 against 272 us).
 		bool few_channels = false;
-		if (Cin <= 16 && N * Cin * H * W >= (1u << 16) && gt.Ho == (int)H && gt.Wo == (int)W) {
+		if (Cin <= 16 && (N * Cin * H * W >= (1u << 16) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8) && gt.Ho == (int)H && gt.Wo == (int)W) {
 			const double macs = 2.0 * (double)(N * H * W) * Cout * kh * kw;  // per output channel of the convolution of dy
 			const uint64_t patch_tiles = ceil_div(W, 128) * ceil_div(H, 4) * ceil_div(Cin, 64) * N;
 			const bool on_patches = conv_patch_forward_takes(gt, dy, dx) && (conv_patch_fast_forward_takes(gt, dy, work) || (W > 56 && patch_tiles >= 256));
@@ -862,7 +865,9 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 			const double as_convolution_us = on_patches ? 10.0 + macs * Cin / 20e6 : 14.0 + macs * tile_rows / 45e6;
 			few_channels = 15.0 + 4.0 * (double)(Kc * HW * N) / 1.2e6 < as_convolution_us;
 		}
-		if (get_option(OPT_CONV_VARIANT) == 0 && kh * kw > 1 && Kc * HW * N * sizeof(float) <= (100ull << 20) && N * Cin * H * W >= (1u << 18) / 4 &&
+		// (small inputs only where the work is large all the same: 4 x 3 x 14 x 14 <- 1024 channels 7 x 7 took 3.8 ms as a convolution of dy)
+		if (get_option(OPT_CONV_VARIANT) == 0 && kh * kw > 1 && Kc * HW * N * sizeof(float) <= (100ull << 20) &&
+		    (N * Cin * H * W >= (1u << 18) / 4 || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8) &&
 		    (few_channels || (ceil_div(Cin, 64) * ceil_div(N * H * W, 64) < 128 && Cout * kh * kw >= 1024))) {
 			const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 			if (rc >= 0) return rc;
@@ -910,7 +915,8 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		const double columns_us = 10.0 + flops / 88e6 + 4.0 * (double)(N * Cin * H * W + 2 * N * Cin * HW) / 2.5e6;
 		one_by_one_pays = columns_us * 1.1 < implicit_us;
 	}
-	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows || one_by_one_pays) && N * Kc * HW >= (1u << 18)) {
+	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows || one_by_one_pays) &&
+	    (N * Kc * HW >= (1u << 18) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8)) {  // (or few columns under many channels: 64 x 8 x 8 x 8 <- 1024 at stride 2 ran image by image, 1.3 ms)
 		const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 		if (rc >= 0) return rc;
 	}

@@ -432,9 +432,30 @@ def test_conv_data_gradient_of_few_channels_by_column_matrices(gpu, ob, geo):
     assert rel_err(dx, want_dx) < TOL
 
 
+@pytest.mark.parametrize("geo,route", [((4, 256, 8, 8, 64, 5, 5, 2, 2, 2, 2), "conv2d_im2col"),           # 16 output pixels an image under K = 6400
+                                       ((8, 128, 7, 7, 8, 7, 7, 3, 3, 2, 2), "conv2d_im2col")])            # 8 output channels under K = 6272
+def test_conv_forward_of_tiny_outputs_under_a_long_reduction_by_column_matrices(gpu, ob, geo, route):
+    """Few output channels or pixels under a reduction of 2048 or more: the implicit GEMM's handful of tiles would walk it one
+    after another, the column matrices hand it to the GEMM entry (which splits it); forward with bias against the oracle."""
+    N, Cin, H, W, Cout, kh, kw, ph, pw, sh, sw = geo
+    rng = np.random.default_rng(sum(geo))
+    x = rng.standard_normal((N, Cin, H, W)).astype(np.float32)
+    w = (rng.standard_normal((Cout, Cin, kh, kw)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(Cout).astype(np.float32)
+    Ho, Wo = ob.conv_out_hw(H, W, kh, kw, ph, pw, sh, sw)
+    col = np.empty(Cin * kh * kw * Ho * Wo, np.float32)
+    want_y = np.empty((N, Cout, Ho, Wo), np.float32)
+    ob.oracle().oracle_conv2d_forward(*geo, x.reshape(-1), w.reshape(-1), want_y.reshape(-1), col)
+    want_y += bias[None, :, None, None]
+    y, _, fk = gpu_conv(gpu, geo, x, w, None, bias)
+    assert fk.startswith(route), fk
+    assert rel_err(y, want_y) < TOL
+
+
 @pytest.mark.parametrize("geo,route", [((16, 16, 64, 64, 16, 3, 3, 1, 1, 1, 1), "conv2d_patch"),     # 3 x 3 on wide rows: the patch kernels
                                        ((64, 8, 32, 32, 8, 3, 3, 1, 1, 1, 1), "conv2d_forward"),     # a short reduction: the implicit GEMM
-                                       ((64, 16, 16, 16, 128, 3, 3, 1, 1, 1, 1), "conv2d_dgrad_batched_gemm_col2im")])   # a long one: the columns
+                                       ((64, 16, 16, 16, 128, 3, 3, 1, 1, 1, 1), "conv2d_dgrad_batched_gemm_col2im"),    # a long one: the columns
+                                       ((4, 3, 14, 14, 512, 7, 7, 3, 3, 1, 1), "conv2d_dgrad_batched_gemm_col2im")])     # a small input under many channels: 13 tiles would walk K = 25088
 def test_conv_data_gradient_of_few_channels_takes_the_cheaper_route(gpu, ob, geo, route):
     """Few input channels at stride 1: an estimate decides between the column matrices and the convolution of dy with the
     flipped weights (which runs 3 x 3 windows on the patch kernels); whichever it picks, against the oracle."""
