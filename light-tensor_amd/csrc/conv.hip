@@ -916,7 +916,7 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		one_by_one_pays = columns_us * 1.1 < implicit_us;
 	}
 	if (get_option(OPT_CONV_VARIANT) == 0 && !dgrad_as_forward(g) && (kh * kw > 1 || padded_rows || one_by_one_pays) &&
-	    (N * Kc * HW >= (1u << 18) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8)) {  // (or few columns under many channels: 64 x 8 x 8 x 8 <- 1024 at stride 2 ran image by image, 1.3 ms)
+	    (N * Kc * HW >= (1u << 18) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 2e7)) {  // (or few columns under many channels: 64 x 8 x 8 x 8 <- 1024 at stride 2 ran image by image, 1.3 ms)
 		const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 		if (rc >= 0) return rc;
 	}
