@@ -844,7 +844,9 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 	if (dgrad_as_forward(g) && get_option(OPT_CONV_VARIANT) != 1 && !few_narrow) {
 		ConvGeo gt;  // the transposed problem: dy is the input, dx the output
 		if (int rc = make_geo(gt, N, Cout, g.Ho, g.Wo, Cin, kh, kw, kh - 1 - ph, kw - 1 - pw, 1, 1, 1, 1)) return rc;
-		if (get_option(OPT_CONV_VARIANT) == 0 && gt.Ho == (int)H && gt.Wo == (int)W && !conv_smallk_takes(gt) && conv_fewout_takes(gt, dy, dx))
+		// (the vector-ALU stream wants pixels to spread over the chip: one image of 56 x 56 <- 384 channels took 239 us on it)
+		if (get_option(OPT_CONV_VARIANT) == 0 && gt.Ho == (int)H && gt.Wo == (int)W && !conv_smallk_takes(gt) && conv_fewout_takes(gt, dy, dx) &&
+		    (N * H * W >= 32768 || Cout <= 64))
 			return conv_fewout_forward(gt, dy, w, nullptr, dx, true);  // reads w transposed and flipped in place
 		// Few input channels, or few tiles of the transposed problem under a long reduction: as a convolution of dy the
 		// gradient fills a fraction of its tiles' rows (10 channels of 32) or leaves most CUs idle, and l-ten's decomposition
@@ -857,7 +859,7 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		// channels 3 x 3: columns 44, patch kernel 18 us; 64 x 16 x 32 x 32 <- 32: 46 against 30 us, <- 64: 44 against 55 us;
 		// 128 x 3 x 32 x 32 <- 64 channels 5 x 5: 48 against 272 us).
 		bool few_channels = false;
-		if (Cin <= 16 && (N * Cin * H * W >= (1u << 16) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8) && gt.Ho == (int)H && gt.Wo == (int)W) {
+		if (Cin <= 16 && (N * Cin * H * W >= (1u << 16) || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 2e7) && gt.Ho == (int)H && gt.Wo == (int)W) {
 			const double macs = 2.0 * (double)(N * H * W) * Cout * kh * kw;  // per output channel of the convolution of dy
 			const uint64_t patch_tiles = ceil_div(W, 128) * ceil_div(H, 4) * ceil_div(Cin, 64) * N;
 			const bool on_patches = conv_patch_forward_takes(gt, dy, dx) && (conv_patch_fast_forward_takes(gt, dy, work) || (W > 56 && patch_tiles >= 256));
@@ -867,7 +869,7 @@ int lten_hip_conv2d_dgrad_f32(uint64_t N, uint64_t Cin, uint64_t H, uint64_t W, 
 		}
 		// (small inputs only where the work is large all the same: 4 x 3 x 14 x 14 <- 1024 channels 7 x 7 took 3.8 ms as a convolution of dy)
 		if (get_option(OPT_CONV_VARIANT) == 0 && kh * kw > 1 && Kc * HW * N * sizeof(float) <= (100ull << 20) &&
-		    (N * Cin * H * W >= (1u << 18) / 4 || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 1e8) &&
+		    (N * Cin * H * W >= (1u << 18) / 4 || 2.0 * (double)(N * HW) * (double)(Cout * Kc) >= 2e7) &&
 		    (few_channels || (ceil_div(Cin, 64) * ceil_div(N * H * W, 64) < 128 && Cout * kh * kw >= 1024))) {
 			const int rc = conv_dgrad_by_columns(g, w, dy, dx);
 			if (rc >= 0) return rc;
